@@ -1,0 +1,161 @@
+/*
+ * rocmlir_amd.h -- C ABI of librocmlir_amd.so: MI355X (gfx950) kernels for the
+ * Rock-dialect contraction ops (GEMM, forward convolution, fused attention,
+ * quantised-GEMM epilogue), handed back as launchable HIP code objects.
+ *
+ * The first block is a drop-in for the reference's kernel-generator library
+ * (mlir/tools/rocmlir-lib/Miir.h:16-101): same names, same argument meaning,
+ * same NULL / status error behaviour, same two-call buffer protocol.  The
+ * second block carries what MIGraphX reads through the MLIR C API
+ * (mlir/include/mlir-c/Dialect/MIGraphX.h:27-78, mlir-c/Dialect/Rock.h:22-167)
+ * for the same kernels: name, block/grid, argument list, perf-config string,
+ * tuning problem key.  The third block is a convenience launcher so that a
+ * host without its own hipModule plumbing (tests, benchmarks, a ctypes or
+ * cgo binding) can run what it was handed.
+ *
+ * All entry points are plain C, take only pointers, sizes and scalars, never
+ * throw, and may be called from several threads; a handle must not be used
+ * from two threads at once.
+ */
+#ifndef ROCMLIR_AMD_H
+#define ROCMLIR_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#if defined(__GNUC__)
+#define ROCMLIR_AMD_API __attribute__((visibility("default")))
+#else
+#define ROCMLIR_AMD_API
+#endif
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Miir.h:18 -- kernel ABI generation: bare pointers, one per tensor. */
+#define MIIR_VERSION_FLAT 6
+/* This library's own revision of the extension block below. */
+#define ROCMLIR_AMD_API_VERSION 1
+
+/* Miir.h:20-26 */
+enum MiirStatus {
+  MIIR_SUCCESS = 0,
+  MIIR_INVALID_PARAM,
+  MIIR_INVALID_MODULE,
+  MIIR_BUILD_FAILURE
+};
+typedef enum MiirStatus MiirStatus;
+
+/* Miir.h:30 */
+typedef void *MiirHandle;
+
+/* ---------------------------------------------------------------------------
+ * 1. Miir drop-in
+ * ------------------------------------------------------------------------- */
+
+/* Miir.h:50 (impl rocmlir-lib.cpp:117-154).  `options` is a whitespace
+ * separated "--key value" list.  Convolution keys are the reference's
+ * (ConvGenerator.cpp:492-661): operation, arch, num_cu, kernel_id,
+ * kernel_name, perf_config, in_type/fil_type/out_type, in_layout/fil_layout/
+ * out_layout, batchsize, groupsize, in_channels, out_channels, in_h, in_w,
+ * out_h, out_w, fil_h, fil_w, dilation_{h,w}, conv_stride_{h,w},
+ * padding_{h,w}.  `--operation gemm` and `--operation attention` take the
+ * reference's rocmlir-gen flag names (rocmlir-gen.cpp:90-561): t,
+ * out_datatype, g, m, k, n, transA, transB, transC; g, seq_len_q, seq_len_k,
+ * head_dim_qk, head_dim_v, transQ, transK, transV, transO, with-attn-bias.
+ * Epilogue keys (all optional): scale, zero_point, quant_scale,
+ * out_zero_point, bias, relu.  A single leading dash and "key=value" are
+ * accepted as well.  Returns NULL on any parse, validation or support
+ * failure, as the reference does. */
+ROCMLIR_AMD_API MiirHandle miirCreateHandle(const char *options);
+
+/* Miir.h:56 -- number of kernels the operation needs; -1 for a NULL handle. */
+ROCMLIR_AMD_API int miirGetKernelCount(MiirHandle handle);
+
+/* Miir.h:65 -- workspace bytes (always 0 for the forward ops built here). */
+ROCMLIR_AMD_API int miirGetWorkspaceSize(MiirHandle handle);
+
+/* Miir.h:70 -- resolves the perf config (table lookup); needed before
+ * miirGetExecutionDims, as in the reference flow. */
+ROCMLIR_AMD_API MiirStatus miirLowerTuningParams(MiirHandle handle);
+
+/* Miir.h:75 -- binds the code object for the selected kernel. */
+ROCMLIR_AMD_API MiirStatus miirLowerBin(MiirHandle handle);
+
+/* Miir.h:88 -- two-call protocol: buffer == NULL writes the size, otherwise
+ * copies the gfx950 ELF code object into caller memory. */
+ROCMLIR_AMD_API MiirStatus miirBufferGet(MiirHandle handle, char *buffer, size_t *size);
+
+/* Miir.h:96 -- 1-D launch: global = grid * block work-items, local = block. */
+ROCMLIR_AMD_API MiirStatus miirGetExecutionDims(MiirHandle handle, size_t *global_size,
+                                size_t *local_size);
+
+/* Miir.h:101 */
+ROCMLIR_AMD_API MiirStatus miirDestroyHandle(MiirHandle handle);
+
+/* ---------------------------------------------------------------------------
+ * 2. Kernel description (what mlirGetKernelInfo / mlirGetKernelAttrs /
+ *    mlirRockTuning* return in the reference)
+ * ------------------------------------------------------------------------- */
+
+/* Kernel symbol inside the code object (mlirGetKernelInfo's name,
+ * MIGraphX.cpp:54-90).  Two-call protocol on `size` (includes the NUL). */
+ROCMLIR_AMD_API MiirStatus rockamdGetKernelName(MiirHandle handle, char *buffer, size_t *size);
+
+/* {block_size, grid_size} as mlirGetKernelAttrs returns them
+ * (MIGraphX.cpp:93-110). */
+ROCMLIR_AMD_API MiirStatus rockamdGetKernelAttrs(MiirHandle handle, uint32_t attrs[2]);
+
+/* Kernel argument list: `num_pointers` bare device pointers in op order
+ * (GEMM: A, B, C, aux; conv: filter, input, output, aux; attention: Q, K, V,
+ * aux, O -- aux is the bias vector / pre-softmax bias tensor, NULL when
+ * unused), followed by ONE by-value parameter block of `*params_size` bytes.
+ * Two-call protocol: params == NULL writes the size only.  The reference
+ * bakes shapes into the kernel and passes pointers only (Pipelines.cpp:
+ * 246-248); this block is the documented extension that replaces that. */
+ROCMLIR_AMD_API MiirStatus rockamdGetKernelArgs(MiirHandle handle, int *num_pointers,
+                                void *params, size_t *params_size);
+
+/* perf-config string of the selected kernel in the reference's grammar
+ * ("v2:MPB,NPB,KpackPB,MPW,MnPerXdl,Kpack,splitK,forceUnroll,1" or
+ * "attn:v1:...", RockAttrDefs.td:241-329).  strncpy semantics, returns the
+ * full length like mlirRockTuningParamToString (Rock.h:60-75). */
+ROCMLIR_AMD_API size_t rockamdGetPerfConfig(MiirHandle handle, char *buffer, size_t buffer_size);
+
+/* Tuning problem key, "<arch>\t<numCU>\t<problem>" in the reference's format
+ * (RockTuningImpl.cpp:550-871; mlirRockTuningGetKey, Rock.h:120-130).
+ * Returns the full length, or (size_t)-1 on failure. */
+ROCMLIR_AMD_API size_t rockamdGetProblemKey(MiirHandle handle, char *buffer, size_t buffer_size);
+
+/* Epilogue scalars can be changed after creation (they live in the by-value
+ * parameter block; fetch it again after a change).  Formulas:
+ * MIGraphXToTosa.cpp:874-982.  No counterpart entry point in the reference,
+ * where these are IR constants. */
+ROCMLIR_AMD_API MiirStatus rockamdSetScale(MiirHandle handle, float scale);
+ROCMLIR_AMD_API MiirStatus rockamdSetZeroPoint(MiirHandle handle, int32_t zero_point);
+
+/* ---------------------------------------------------------------------------
+ * 3. Launch helpers (the client side of rocmlir-tuning-driver.cpp:131-185)
+ * ------------------------------------------------------------------------- */
+
+/* Loads the handle's code object on the current device (cached) and enqueues
+ * one launch on `stream` (a hipStream_t, NULL = default stream).  `pointers`
+ * holds exactly the pointer arguments described above.  Returns 0 or a
+ * hipError_t value; never synchronises. */
+ROCMLIR_AMD_API int rockamdLaunch(MiirHandle handle, void *const *pointers, int num_pointers,
+                  void *stream);
+
+/* Timed loop with HIP events on `stream`: `warmup` untimed launches, then
+ * `iters` launches between one start/stop event pair; writes the average
+ * milliseconds per launch.  Synchronises the stream. */
+ROCMLIR_AMD_API int rockamdBenchmark(MiirHandle handle, void *const *pointers, int num_pointers,
+                     void *stream, int warmup, int iters, float *avg_ms);
+
+/* Text of the last failure on the calling thread ("" if none). */
+ROCMLIR_AMD_API const char *rockamdGetLastError(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ROCMLIR_AMD_H */

@@ -1,0 +1,274 @@
+"""numpy front end of the CPU oracle (librock_oracle.so).
+
+Test infrastructure only: imported by tests/, the smoke check and the
+benchmark's CPU-baseline leg.  The shipped package never imports it.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "librock_oracle.so")
+
+F32, F16, BF16, I8, FP8, BF8, I32 = range(7)
+TYPE_CODES = {"f32": F32, "f16": F16, "bf16": BF16, "i8": I8, "fp8": FP8,
+              "bf8": BF8, "i32": I32}
+_NP_STORAGE = {F32: np.float32, F16: np.uint16, BF16: np.uint16, I8: np.int8,
+               FP8: np.uint8, BF8: np.uint8, I32: np.int32}
+
+
+def build():
+    """Compile the oracle with the Makefile next to it."""
+    subprocess.run(["make", "-C", _HERE, "-s", "librock_oracle.so"], check=True)
+
+
+class ConvDims(C.Structure):
+    _fields_ = [(n, C.c_int64) for n in (
+        "n", "g", "c", "k", "hi", "wi", "y", "x", "ho", "wo",
+        "stride_h", "stride_w", "pad_h", "pad_w", "dil_h", "dil_w")]
+
+
+class VerifyResult(C.Structure):
+    _fields_ = [("rms", C.c_double), ("max_abs_diff", C.c_double),
+                ("max_rel_diff", C.c_double), ("ave_abs_diff", C.c_double),
+                ("max_mag", C.c_double), ("pass_rms", C.c_int32),
+                ("pass_abs", C.c_int32), ("pass_rel", C.c_int32)]
+
+    def passed(self):
+        return bool(self.pass_rms and self.pass_abs and self.pass_rel)
+
+    def __repr__(self):
+        return ("VerifyResult(rms=%.3e, max_abs=%.3e, max_rel=%.3e, [%d %d %d])"
+                % (self.rms, self.max_abs_diff, self.max_rel_diff,
+                   self.pass_rms, self.pass_abs, self.pass_rel))
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = C.CDLL(_LIB_PATH)
+        i64, i32, f32, vp = C.c_int64, C.c_int32, C.c_float, C.c_void_p
+        L.orc_max_threads.restype = C.c_int
+        L.orc_f32_to_f16.restype = C.c_uint16
+        L.orc_f32_to_f16.argtypes = [f32]
+        L.orc_f16_to_f32.restype = f32
+        L.orc_f16_to_f32.argtypes = [C.c_uint16]
+        L.orc_f32_to_bf16.restype = C.c_uint16
+        L.orc_f32_to_bf16.argtypes = [f32]
+        for nm in ("orc_f32_to_e4m3fn_sat", "orc_f32_to_e4m3fn_nosat",
+                   "orc_f32_to_e5m2_sat", "orc_f32_to_e5m2_nosat"):
+            getattr(L, nm).restype = C.c_uint8
+            getattr(L, nm).argtypes = [f32]
+        for nm in ("orc_e4m3fn_to_f32", "orc_e5m2_to_f32"):
+            getattr(L, nm).restype = f32
+            getattr(L, nm).argtypes = [C.c_uint8]
+        L.orc_widen.argtypes = [vp, C.c_int, i64, vp]
+        L.orc_narrow.argtypes = [vp, C.c_int, i64, vp]
+        L.orc_round_through.argtypes = [vp, C.c_int, i64]
+        gemm_args = [vp, vp, vp, i64, i64, i64, i64, C.c_int, C.c_int, C.c_int,
+                     i64, i64, C.c_int]
+        L.orc_gemm_f32.argtypes = gemm_args
+        L.orc_gemm_i8.argtypes = gemm_args
+        conv_args = [vp, vp, vp, C.c_char_p, C.c_char_p, C.c_char_p,
+                     C.POINTER(ConvDims), i64, i64, C.c_int]
+        L.orc_conv_fwd_f32.argtypes = conv_args
+        L.orc_conv_fwd_f32.restype = C.c_int
+        L.orc_conv_fwd_i8.argtypes = conv_args
+        L.orc_conv_fwd_i8.restype = C.c_int
+        L.orc_attention_f32.argtypes = [vp, vp, vp, vp, vp, f32, vp, i64, i64,
+                                        i64, i64, i64, C.c_int, C.c_int,
+                                        C.c_int, C.c_int, i64, i64, C.c_int]
+        L.orc_softmax_f32.argtypes = [vp, vp, i64, i64]
+        L.orc_dequantize_i64.argtypes = [vp, i64, f32, i32, vp]
+        L.orc_quantize_i8.argtypes = [vp, i64, f32, i32, vp]
+        L.orc_scale_bias_f32.argtypes = [vp, i64, i64, f32, vp]
+        L.orc_verify_float.argtypes = [vp, vp, i64, f32, f32, f32,
+                                       C.POINTER(VerifyResult)]
+        L.orc_verify_int32_int64.argtypes = [vp, vp, i64, C.POINTER(i64),
+                                             C.POINTER(i64)]
+        L.orc_verify_int32_int64.restype = i64
+        L.orc_fill_fixed.argtypes = [vp, i64, C.c_int]
+        L.orc_seed.argtypes = [C.c_uint32]
+        L.orc_fill_rand.argtypes = [vp, i64, C.c_int, C.c_int, C.c_int]
+        _lib = L
+    return _lib
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+def _c(a, dt):
+    return np.ascontiguousarray(a, dtype=dt)
+
+
+def max_threads():
+    return lib().orc_max_threads()
+
+
+# ---- codecs -----------------------------------------------------------
+def widen(raw, type_code):
+    """Raw storage array (uint16 / uint8 / int8 / float32) -> float32."""
+    raw = _c(raw, _NP_STORAGE[type_code])
+    out = np.empty(raw.shape, np.float32)
+    lib().orc_widen(_p(raw), type_code, raw.size, _p(out))
+    return out
+
+
+def narrow(x, type_code):
+    """float32 -> raw storage array of the given type (RNE; fp8 saturates)."""
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, _NP_STORAGE[type_code])
+    lib().orc_narrow(_p(x), type_code, x.size, _p(out))
+    return out
+
+
+def round_through(x, type_code):
+    x = np.array(x, dtype=np.float32, order="C", copy=True)
+    lib().orc_round_through(_p(x), type_code, x.size)
+    return x
+
+
+# ---- GEMM -------------------------------------------------------------
+def gemm(A, B, G, M, N, K, transA=False, transB=False, transC=False,
+         rows=None, threads=0):
+    """A, B: flat (or any-shape) arrays in the reference's storage order.
+    float32 inputs -> float32 C; int8 inputs -> int64 C.  Returns a flat C of
+    G*M*N elements (rows outside `rows` are zero)."""
+    r0, r1 = rows if rows is not None else (0, M)
+    if A.dtype == np.int8:
+        A, B = _c(A, np.int8), _c(B, np.int8)
+        Cm = np.zeros(G * M * N, np.int64)
+        fn = lib().orc_gemm_i8
+    else:
+        A, B = _c(A, np.float32), _c(B, np.float32)
+        Cm = np.zeros(G * M * N, np.float32)
+        fn = lib().orc_gemm_f32
+    assert A.size == G * M * K and B.size == G * K * N
+    fn(_p(A), _p(B), _p(Cm), G, M, N, K, int(transA), int(transB), int(transC),
+       r0, r1, threads)
+    return Cm
+
+
+# ---- convolution --------------------------------------------------------
+def conv_out_dim(in_len, fil_len, pad_l, pad_r, stride, dil):
+    """Output extent, ConvGenerator.h:101-108."""
+    return (in_len + pad_l + pad_r - (fil_len - 1) * dil - 1) // stride + 1
+
+
+def conv_fwd(fil, inp, fil_layout, in_layout, out_layout, n, g, c, k, hi, wi,
+             y, x, stride=(1, 1), pad=(0, 0), dil=(1, 1), out_range=None,
+             threads=0):
+    """c and k are PER-GROUP channel counts.  Layout strings: permutations of
+    'gkcyx' / 'ngchw' / 'ngkhw'.  Returns (flat output, ho, wo)."""
+    ho = conv_out_dim(hi, y, pad[0], pad[0], stride[0], dil[0])
+    wo = conv_out_dim(wi, x, pad[1], pad[1], stride[1], dil[1])
+    d = ConvDims(n, g, c, k, hi, wi, y, x, ho, wo, stride[0], stride[1],
+                 pad[0], pad[1], dil[0], dil[1])
+    total = n * g * k * ho * wo
+    b, e = out_range if out_range is not None else (0, total)
+    if fil.dtype == np.int8:
+        fil, inp = _c(fil, np.int8), _c(inp, np.int8)
+        out = np.zeros(total, np.int64)
+        fn = lib().orc_conv_fwd_i8
+    else:
+        fil, inp = _c(fil, np.float32), _c(inp, np.float32)
+        out = np.zeros(total, np.float32)
+        fn = lib().orc_conv_fwd_f32
+    assert fil.size == g * k * c * y * x and inp.size == n * g * c * hi * wi
+    rc = fn(_p(fil), _p(inp), _p(out), fil_layout.encode(), in_layout.encode(),
+            out_layout.encode(), C.byref(d), b, e, threads)
+    if rc != 0:
+        raise ValueError("bad layout string")
+    return out, ho, wo
+
+
+# ---- attention ------------------------------------------------------------
+def attention(Q, K, V, G, sq, sk, dqk, dv, scale=1.0, scale_t=None,
+              bias_t=None, transQ=False, transK=False, transV=False,
+              transO=False, q_rows=None, threads=0):
+    Q, K, V = _c(Q, np.float32), _c(K, np.float32), _c(V, np.float32)
+    assert Q.size == G * sq * dqk and K.size == G * sk * dqk
+    assert V.size == G * sk * dv
+    st = _c(scale_t, np.float32) if scale_t is not None else None
+    bt = _c(bias_t, np.float32) if bias_t is not None else None
+    O = np.zeros(G * sq * dv, np.float32)
+    q0, q1 = q_rows if q_rows is not None else (0, sq)
+    lib().orc_attention_f32(_p(Q), _p(K), _p(V), _p(st), _p(bt),
+                            np.float32(scale), _p(O), G, sq, sk, dqk, dv,
+                            int(transQ), int(transK), int(transV), int(transO),
+                            q0, q1, threads)
+    return O
+
+
+def softmax(x):
+    x = _c(x, np.float32)
+    y = np.empty_like(x)
+    lib().orc_softmax_f32(_p(x), _p(y), x.size // x.shape[-1], x.shape[-1])
+    return y
+
+
+# ---- quantisation epilogue ----------------------------------------------------
+def dequantize(acc_i64, scale, zero_point=0):
+    acc = _c(acc_i64, np.int64)
+    y = np.empty(acc.shape, np.float32)
+    lib().orc_dequantize_i64(_p(acc), acc.size, np.float32(scale), zero_point,
+                             _p(y))
+    return y
+
+
+def quantize_i8(x, scale, zero_point=0):
+    x = _c(x, np.float32)
+    q = np.empty(x.shape, np.int8)
+    lib().orc_quantize_i8(_p(x), x.size, np.float32(scale), zero_point, _p(q))
+    return q
+
+
+def scale_bias(x, rows, cols, scale, bias=None):
+    x = np.array(x, dtype=np.float32, order="C", copy=True)
+    b = _c(bias, np.float32) if bias is not None else None
+    lib().orc_scale_bias_f32(_p(x), rows, cols, np.float32(scale), _p(b))
+    return x
+
+
+# ---- verifier -------------------------------------------------------------------
+def verify_float(gpu, val, thr_rms=3e-5, thr_abs=100.0, thr_rel=100.0):
+    gpu, val = _c(gpu, np.float32).ravel(), _c(val, np.float32).ravel()
+    assert gpu.size == val.size
+    res = VerifyResult()
+    lib().orc_verify_float(_p(gpu), _p(val), gpu.size, thr_rms, thr_abs,
+                           thr_rel, C.byref(res))
+    return res
+
+
+def verify_int(gpu_i32, val_i64):
+    gpu, val = _c(gpu_i32, np.int32).ravel(), _c(val_i64, np.int64).ravel()
+    assert gpu.size == val.size
+    ovf, mad = C.c_int64(0), C.c_int64(0)
+    fails = lib().orc_verify_int32_int64(_p(gpu), _p(val), gpu.size,
+                                         C.byref(ovf), C.byref(mad))
+    return fails, ovf.value, mad.value
+
+
+# ---- data fill ----------------------------------------------------------------------
+def fill_fixed(n, is_int=False):
+    x = np.empty(n, np.float32)
+    lib().orc_fill_fixed(_p(x), n, int(is_int))
+    return x
+
+
+def seed(s):
+    lib().orc_seed(s)
+
+
+def fill_rand(n, lo, hi, as_float):
+    x = np.empty(n, np.float32)
+    lib().orc_fill_rand(_p(x), n, lo, hi, int(as_float))
+    return x

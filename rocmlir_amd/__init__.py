@@ -1,0 +1,14 @@
+"""rocmlir_amd: MI355X (gfx950) kernels for the Rock-dialect contraction ops
+behind a Miir-shaped C ABI (include/rocmlir_amd.h).
+
+The compute path is librocmlir_amd.so (hand-written HIP, built by
+rocmlir_amd._build).  This package is the thin Python host side: a ctypes
+binding plus helpers that take torch tensors as device memory.  There is no
+CPU or eager fallback: if the library is missing, importing the binding
+raises.
+"""
+from .api import (RockError, RockKernel, attention, conv2d, gemm,  # noqa: F401
+                  library_path, load_library)
+
+__all__ = ["RockError", "RockKernel", "gemm", "conv2d", "attention",
+           "library_path", "load_library"]

@@ -1,0 +1,366 @@
+"""ctypes binding of librocmlir_amd.so and torch-tensor front ends.
+
+The option strings built here use the reference's own flag names
+(rocmlir-gen.cpp:90-561 for gemm / attention, ConvGenerator.cpp:492-661 for
+convolution), so a problem reads the same as on a rocmlir-gen command line.
+"""
+import ctypes as C
+import os
+import threading
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_PKG, "librocmlir_amd.so")
+_lib = None
+_lock = threading.Lock()
+
+MIIR_SUCCESS = 0
+MIIR_INVALID_PARAM = 1
+MIIR_INVALID_MODULE = 2
+MIIR_BUILD_FAILURE = 3
+
+
+class RockError(RuntimeError):
+    pass
+
+
+def library_path():
+    return _LIB_PATH
+
+
+def load_library():
+    """Loads librocmlir_amd.so; raises RockError when it has not been built."""
+    global _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(_LIB_PATH):
+            raise RockError(
+                "librocmlir_amd.so is missing (%s): run "
+                "`python -c 'import __graft_entry__ as g; g.build()'` "
+                "or `python -m rocmlir_amd._build`" % _LIB_PATH)
+        L = C.CDLL(_LIB_PATH)
+        vp, sz = C.c_void_p, C.c_size_t
+        L.miirCreateHandle.restype = vp
+        L.miirCreateHandle.argtypes = [C.c_char_p]
+        for name in ("miirGetKernelCount", "miirGetWorkspaceSize",
+                     "miirLowerTuningParams", "miirLowerBin",
+                     "miirDestroyHandle"):
+            getattr(L, name).restype = C.c_int
+            getattr(L, name).argtypes = [vp]
+        L.miirBufferGet.restype = C.c_int
+        L.miirBufferGet.argtypes = [vp, C.c_char_p, C.POINTER(sz)]
+        L.miirGetExecutionDims.restype = C.c_int
+        L.miirGetExecutionDims.argtypes = [vp, C.POINTER(sz), C.POINTER(sz)]
+        L.rockamdGetKernelName.restype = C.c_int
+        L.rockamdGetKernelName.argtypes = [vp, C.c_char_p, C.POINTER(sz)]
+        L.rockamdGetKernelAttrs.restype = C.c_int
+        L.rockamdGetKernelAttrs.argtypes = [vp, C.POINTER(C.c_uint32)]
+        L.rockamdGetKernelArgs.restype = C.c_int
+        L.rockamdGetKernelArgs.argtypes = [vp, C.POINTER(C.c_int), vp,
+                                           C.POINTER(sz)]
+        L.rockamdGetPerfConfig.restype = sz
+        L.rockamdGetPerfConfig.argtypes = [vp, C.c_char_p, sz]
+        L.rockamdGetProblemKey.restype = sz
+        L.rockamdGetProblemKey.argtypes = [vp, C.c_char_p, sz]
+        L.rockamdSetScale.restype = C.c_int
+        L.rockamdSetScale.argtypes = [vp, C.c_float]
+        L.rockamdSetZeroPoint.restype = C.c_int
+        L.rockamdSetZeroPoint.argtypes = [vp, C.c_int32]
+        L.rockamdLaunch.restype = C.c_int
+        L.rockamdLaunch.argtypes = [vp, C.POINTER(vp), C.c_int, vp]
+        L.rockamdBenchmark.restype = C.c_int
+        L.rockamdBenchmark.argtypes = [vp, C.POINTER(vp), C.c_int, vp, C.c_int,
+                                       C.c_int, C.POINTER(C.c_float)]
+        L.rockamdGetLastError.restype = C.c_char_p
+        L.rockamdGetLastError.argtypes = []
+        _lib = L
+        return _lib
+
+
+def last_error():
+    return load_library().rockamdGetLastError().decode()
+
+
+class RockKernel:
+    """One problem -> one launchable kernel (a MiirHandle).
+
+    Follows the reference client's call order (rocmlir-lib-test.cpp:31-96):
+    create, lower tuning params, lower bin, read the binary and the launch
+    dimensions."""
+
+    def __init__(self, options):
+        L = load_library()
+        self.options = options
+        self._h = L.miirCreateHandle(options.encode())
+        if not self._h:
+            raise RockError("miirCreateHandle failed: %s [%s]"
+                            % (last_error(), options))
+        if L.miirLowerTuningParams(self._h) != MIIR_SUCCESS:
+            raise RockError("miirLowerTuningParams failed")
+        if L.miirLowerBin(self._h) != MIIR_SUCCESS:
+            raise RockError("miirLowerBin failed")
+        attrs = (C.c_uint32 * 2)()
+        L.rockamdGetKernelAttrs(self._h, attrs)
+        self.block_size, self.grid_size = int(attrs[0]), int(attrs[1])
+        n = C.c_size_t(0)
+        L.rockamdGetKernelName(self._h, None, C.byref(n))
+        buf = C.create_string_buffer(n.value)
+        L.rockamdGetKernelName(self._h, buf, C.byref(n))
+        self.kernel_name = buf.value.decode()
+        npt, psz = C.c_int(0), C.c_size_t(0)
+        L.rockamdGetKernelArgs(self._h, C.byref(npt), None, C.byref(psz))
+        self.num_pointers = npt.value
+        self.params_size = psz.value
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h and _lib is not None:
+            _lib.miirDestroyHandle(h)
+
+    # ---- description ------------------------------------------------------
+    def _string(self, fn):
+        buf = C.create_string_buffer(2048)
+        n = fn(self._h, buf, 2048)
+        if n == C.c_size_t(-1).value:
+            raise RockError("string query failed")
+        return buf.value.decode()
+
+    @property
+    def perf_config(self):
+        return self._string(load_library().rockamdGetPerfConfig)
+
+    @property
+    def problem_key(self):
+        return self._string(load_library().rockamdGetProblemKey)
+
+    def code_object(self):
+        L = load_library()
+        n = C.c_size_t(0)
+        if L.miirBufferGet(self._h, None, C.byref(n)) != MIIR_SUCCESS:
+            raise RockError("miirBufferGet(size) failed")
+        buf = C.create_string_buffer(n.value)
+        if L.miirBufferGet(self._h, buf, C.byref(n)) != MIIR_SUCCESS:
+            raise RockError("miirBufferGet failed")
+        return buf.raw[:n.value]
+
+    def params(self):
+        L = load_library()
+        n = C.c_size_t(self.params_size)
+        buf = C.create_string_buffer(n.value)
+        npt = C.c_int(0)
+        L.rockamdGetKernelArgs(self._h, C.byref(npt), buf, C.byref(n))
+        return buf.raw
+
+    def execution_dims(self):
+        g, l = C.c_size_t(0), C.c_size_t(0)
+        rc = load_library().miirGetExecutionDims(self._h, C.byref(g),
+                                                 C.byref(l))
+        if rc != MIIR_SUCCESS:
+            raise RockError("miirGetExecutionDims failed (%d)" % rc)
+        return g.value, l.value
+
+    def set_scale(self, scale):
+        load_library().rockamdSetScale(self._h, float(scale))
+
+    def set_zero_point(self, zp):
+        load_library().rockamdSetZeroPoint(self._h, int(zp))
+
+    # ---- launch --------------------------------------------------------------
+    def _pointer_array(self, args):
+        if len(args) != self.num_pointers:
+            raise RockError("kernel %s takes %d pointer arguments, got %d"
+                            % (self.kernel_name, self.num_pointers, len(args)))
+        arr = (C.c_void_p * len(args))()
+        for i, a in enumerate(args):
+            if a is None:
+                arr[i] = None
+            elif isinstance(a, int):
+                arr[i] = a
+            else:  # torch tensor
+                if not a.is_cuda:
+                    raise RockError("tensor arguments must live on the GPU")
+                arr[i] = a.data_ptr()
+        return arr
+
+    @staticmethod
+    def _stream(stream):
+        if stream is None:
+            import torch
+            return torch.cuda.current_stream().cuda_stream
+        return getattr(stream, "cuda_stream", stream)
+
+    def launch(self, *args, stream=None):
+        arr = self._pointer_array(args)
+        rc = load_library().rockamdLaunch(self._h, arr, len(args),
+                                          self._stream(stream))
+        if rc != 0:
+            raise RockError("launch of %s failed (hip error %d): %s"
+                            % (self.kernel_name, rc, last_error()))
+
+    def benchmark(self, *args, warmup=3, iters=20, stream=None):
+        """Average milliseconds per launch (HIP events on the launch stream)."""
+        arr = self._pointer_array(args)
+        ms = C.c_float(0)
+        rc = load_library().rockamdBenchmark(self._h, arr, len(args),
+                                             self._stream(stream), warmup,
+                                             iters, C.byref(ms))
+        if rc != 0:
+            raise RockError("benchmark of %s failed (hip error %d): %s"
+                            % (self.kernel_name, rc, last_error()))
+        return ms.value
+
+
+# ---------------------------------------------------------------------------
+# torch front ends
+# ---------------------------------------------------------------------------
+_kernel_cache = {}
+
+
+def _kernel(options):
+    k = _kernel_cache.get(options)
+    if k is None:
+        k = _kernel_cache[options] = RockKernel(options)
+    return k
+
+
+def _dtype_name(dt):
+    import torch
+    names = {torch.float32: "f32", torch.float16: "f16", torch.bfloat16: "bf16",
+             torch.int8: "i8", torch.int32: "i32"}
+    if hasattr(torch, "float8_e4m3fn"):
+        names[torch.float8_e4m3fn] = "fp8"
+        names[torch.float8_e5m2] = "bf8"
+    try:
+        return names[dt]
+    except KeyError:
+        raise RockError("unsupported tensor dtype %s" % dt)
+
+
+def _torch_dtype(name):
+    import torch
+    return {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16,
+            "i8": torch.int8, "i32": torch.int32,
+            "fp8": torch.float8_e4m3fn, "bf8": torch.float8_e5m2}[name]
+
+
+def _epilogue_flags(scale, zero_point, bias, relu, quant_scale, out_zero_point):
+    s = ""
+    if scale is not None:
+        s += " -scale %.9g" % scale
+    if zero_point:
+        s += " -zero_point %d" % zero_point
+    if quant_scale is not None:
+        s += " -quant_scale %.9g" % quant_scale
+    if out_zero_point:
+        s += " -out_zero_point %d" % out_zero_point
+    if bias is not None:
+        s += " -bias true"
+    if relu:
+        s += " -relu true"
+    return s
+
+
+def gemm(a, b, *, transA=False, transB=False, transC=False, out_dtype=None,
+         scale=None, zero_point=0, bias=None, relu=False, quant_scale=None,
+         out_zero_point=0, out=None, perf_config=None, stream=None):
+    """C = epilogue(A x B) with the reference's storage conventions
+    (rocmlir-gen.cpp:2058-2080): a is [G,M,K] ([G,K,M] if transA), b is
+    [G,K,N] ([G,N,K] if transB), result [G,M,N] ([G,N,M] if transC).
+    2-D inputs mean G = 1."""
+    import torch
+    a3 = a if a.dim() == 3 else a.unsqueeze(0)
+    b3 = b if b.dim() == 3 else b.unsqueeze(0)
+    a3, b3 = a3.contiguous(), b3.contiguous()
+    G = a3.shape[0]
+    M, K = (a3.shape[2], a3.shape[1]) if transA else (a3.shape[1], a3.shape[2])
+    Kb, N = (b3.shape[2], b3.shape[1]) if transB else (b3.shape[1], b3.shape[2])
+    if Kb != K or b3.shape[0] != G:
+        raise RockError("gemm: operand shapes do not match")
+    ta, tb = _dtype_name(a3.dtype), _dtype_name(b3.dtype)
+    t = ta if ta == tb else "%s_%s" % (ta, tb)
+    opts = ("-operation gemm -arch gfx950 -t %s -g %d -m %d -n %d -k %d"
+            " -transA %s -transB %s -transC %s"
+            % (t, G, M, N, K, str(bool(transA)).lower(),
+               str(bool(transB)).lower(), str(bool(transC)).lower()))
+    if out_dtype is not None:
+        opts += " -out_datatype %s" % out_dtype
+    if perf_config:
+        opts += " -perf_config %s" % perf_config
+    opts += _epilogue_flags(scale, zero_point, bias, relu, quant_scale,
+                            out_zero_point)
+    k = _kernel(opts)
+    if out_dtype is None:
+        out_dtype = {"i8": "i32", "fp8": "f32", "bf8": "f32"}.get(ta, ta)
+    shape = (G, N, M) if transC else (G, M, N)
+    if out is None:
+        out = torch.empty(shape, dtype=_torch_dtype(out_dtype), device=a.device)
+    k.launch(a3, b3, out, bias, stream=stream)
+    return out if a.dim() == 3 else out.squeeze(0)
+
+
+def conv2d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize,
+           in_channels, out_channels, in_h, in_w, fil_h, fil_w, groupsize=1,
+           stride=(1, 1), padding=(0, 0), dilation=(1, 1), out_dtype=None,
+           scale=None, zero_point=0, bias=None, relu=False, quant_scale=None,
+           out_zero_point=0, out=None, perf_config=None, stream=None):
+    """Forward convolution; tensors are flat device buffers laid out as the
+    layout strings say (Miir / rocmlir-gen spelling, e.g. 'gkyxc', 'nhwgc',
+    'NGCHW').  Returns the flat output tensor."""
+    import torch
+    t = _dtype_name(inp.dtype)
+    ho = (in_h + 2 * padding[0] - (fil_h - 1) * dilation[0] - 1) // stride[0] + 1
+    wo = (in_w + 2 * padding[1] - (fil_w - 1) * dilation[1] - 1) // stride[1] + 1
+    opts = ("--operation conv --arch gfx950 --in_type %s --fil_type %s"
+            " --fil_layout %s --in_layout %s --out_layout %s --batchsize %d"
+            " --groupsize %d --in_channels %d --out_channels %d --in_h %d"
+            " --in_w %d --out_h %d --out_w %d --fil_h %d --fil_w %d"
+            " --dilation_h %d --dilation_w %d --conv_stride_h %d"
+            " --conv_stride_w %d --padding_h %d --padding_w %d"
+            % (t, _dtype_name(fil.dtype), fil_layout, in_layout, out_layout,
+               batchsize, groupsize, in_channels, out_channels, in_h, in_w, ho,
+               wo, fil_h, fil_w, dilation[0], dilation[1], stride[0], stride[1],
+               padding[0], padding[1]))
+    if out_dtype is not None:
+        opts += " --out_type %s" % out_dtype
+    if perf_config:
+        opts += " --perf_config %s" % perf_config
+    opts += _epilogue_flags(scale, zero_point, bias, relu, quant_scale,
+                            out_zero_point)
+    k = _kernel(opts)
+    if out_dtype is None:
+        out_dtype = {"i8": "i32", "fp8": "f32", "bf8": "f32"}.get(t, t)
+    if out is None:
+        out = torch.empty(batchsize * out_channels * ho * wo,
+                          dtype=_torch_dtype(out_dtype), device=inp.device)
+    k.launch(fil.contiguous(), inp.contiguous(), out, bias, stream=stream)
+    return out
+
+
+def attention(q, k, v, *, scale=1.0, bias=None, transQ=False, transK=False,
+              transV=False, transO=False, out=None, stream=None):
+    """O = softmax(scale * Q K + bias) V with the reference's storage
+    conventions (rocmlir-gen.cpp:2149-2200): q [G,seq_q,d] ([G,d,seq_q] if
+    transQ); k [G,d,seq_k] ([G,seq_k,d] if transK -- the usual row-major keys);
+    v [G,seq_k,dv] ([G,dv,seq_k] if transV); result [G,seq_q,dv]
+    ([G,dv,seq_q] if transO)."""
+    import torch
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    G = q.shape[0]
+    sq, dqk = (q.shape[2], q.shape[1]) if transQ else (q.shape[1], q.shape[2])
+    sk = k.shape[1] if transK else k.shape[2]
+    dv = v.shape[1] if transV else v.shape[2]
+    t = _dtype_name(q.dtype)
+    tf = lambda b: str(bool(b)).lower()  # noqa: E731
+    opts = ("-operation attention -arch gfx950 -t %s -g %d -seq_len_q %d"
+            " -seq_len_k %d -head_dim_qk %d -head_dim_v %d -transQ %s"
+            " -transK %s -transV %s -transO %s -scale %.9g"
+            % (t, G, sq, sk, dqk, dv, tf(transQ), tf(transK), tf(transV),
+               tf(transO), scale))
+    if bias is not None:
+        opts += " -with-attn-bias true"
+    kern = _kernel(opts)
+    shape = (G, dv, sq) if transO else (G, sq, dv)
+    if out is None:
+        out = torch.empty(shape, dtype=q.dtype, device=q.device)
+    kern.launch(q, k, v, bias, out, stream=stream)
+    return out

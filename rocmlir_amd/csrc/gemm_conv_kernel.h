@@ -1,0 +1,632 @@
+// Tiled MFMA contraction kernel for gfx950: GEMM and implicit-GEMM forward
+// convolution share one main loop and differ only in how a tile row is
+// addressed in global memory.
+//
+// Behaviour replaced: the reference's gridwise GEMM schedule
+// (mlir/lib/Dialect/Rock/Transforms/GridwiseGemmToBlockwise.cpp:2409-2811)
+// and its conv->GEMM views (mlir/lib/Dialect/Rock/Transforms/ConvToGemm.cpp:
+// 1190-1393).  Nothing of that code is reused; the design is:
+//
+//   * block tile BM x BN, K advanced 128 BYTES per iteration for every
+//     element type (128 int8/fp8, 64 f16/bf16, 32 f32 elements);
+//   * global -> registers -> LDS, two LDS stages, one barrier per iteration;
+//   * LDS tile = rows of 8 sixteen-byte chunks, chunk index XOR-swizzled with
+//     the row so that the 16 lanes of an MFMA row group hit 16 distinct
+//     16-byte bank groups;
+//   * the problem's B rows feed the MFMA row operand and its A rows the
+//     column operand, so every lane ends up with 4 CONSECUTIVE n of one m and
+//     the C tile is written with 8/16-byte stores;
+//   * out-of-range rows and the K tail are zero-filled on load, never read
+//     past the tensor; the epilogue (scale, zero point, bias, cast) runs on
+//     the accumulators in registers.
+#pragma once
+#include "mfma_gfx950.h"
+
+namespace rk {
+
+enum LoaderKind : int {
+  LD_ROWS_FAST = 0,     // K-contiguous rows, 16-byte aligned chunks
+  LD_ROWS_GENERIC = 1,  // arbitrary element strides, element-wise
+  LD_CONV_IN_FAST = 2,  // convolution input, channel-contiguous, C*ES % 16 == 0
+  LD_CONV_IN_GENERIC = 3,
+  LD_CONV_FIL_GENERIC = 4
+};
+
+constexpr int kChunk = 16;       // bytes
+constexpr int kRowBytes = 128;   // K bytes per tile row
+constexpr int kChunksPerRow = 8;
+
+__device__ __forceinline__ int swizzle(int row, int chunk) {
+  return chunk ^ ((row >> 1) & 7);
+}
+
+// ---------------------------------------------------------------------------
+// Work-item decode: 1-D grid -> (g, tile_m, tile_n) with the XCD round-robin
+// undone and tile rows walked in groups so that co-resident blocks share
+// operand tiles in one XCD's L2 (the reference has the same idea at
+// mlir/lib/Dialect/Rock/Transforms/GridLayoutEmitter.cpp:38-109).
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void decode_block(int tiles_m, int tiles_n, int G,
+                                             int group_m, int xcd_remap,
+                                             int &g, int &tm, int &tn) {
+  int bid = blockIdx.x;
+  const int tiles = tiles_m * tiles_n;
+  const int total = tiles * G;
+  if (xcd_remap) {
+    const int per = total >> 3;
+    if (bid < (per << 3))
+      bid = (bid & 7) * per + (bid >> 3);
+  }
+  g = bid / tiles;
+  const int t = bid - g * tiles;
+  const int group_sz = group_m * tiles_n;
+  const int grp = t / group_sz;
+  const int first_m = grp * group_m;
+  const int rows_here = min(tiles_m - first_m, group_m);
+  const int in_grp = t - grp * group_sz;
+  tm = first_m + in_grp % rows_here;
+  tn = in_grp / rows_here;
+}
+
+// ---------------------------------------------------------------------------
+// Row loaders.  Each thread owns NCH chunks of the tile: chunk column
+// c = tid & 7 (fixed), rows (tid >> 3) + i * (NT / 8).
+// ---------------------------------------------------------------------------
+template <int DT, int ROWS, int NT> struct TileGeom {
+  static constexpr int ES = MmaTraits<DT>::ES;
+  static constexpr int EPC = kChunk / ES; // elements per chunk
+  static constexpr int BKE = kRowBytes / ES; // K elements per tile
+  static constexpr int TOTAL = ROWS * kChunksPerRow;
+  static constexpr int NCH = (TOTAL + NT - 1) / NT;
+  static constexpr int ROW_STEP = NT / kChunksPerRow;
+  static_assert(NT % kChunksPerRow == 0, "thread count must be a multiple of 8");
+};
+
+// K-contiguous rows: base + row * row_stride, chunk at byte kt*128 + c*16.
+template <int DT, int ROWS, int NT> struct RowsFast {
+  using Gm = TileGeom<DT, ROWS, NT>;
+  const char *ptr[Gm::NCH];
+  bool ok[Gm::NCH];
+  int kbytes;
+  int c;
+
+  __device__ __forceinline__ void init(const void *base, int64_t row_stride,
+                                       int row0, int rows_total, int K,
+                                       int tid) {
+    c = tid & 7;
+    kbytes = K * Gm::ES;
+#pragma unroll
+    for (int i = 0; i < Gm::NCH; ++i) {
+      int r = (tid >> 3) + i * Gm::ROW_STEP;
+      int gr = row0 + r;
+      ok[i] = (r < ROWS) && (gr < rows_total);
+      int cr = min(gr, rows_total - 1);
+      ptr[i] = (const char *)base + (int64_t)cr * row_stride * Gm::ES;
+    }
+  }
+  __device__ __forceinline__ void load(int kt, v4i (&regs)[Gm::NCH]) const {
+    int off = kt * kRowBytes + c * kChunk;
+    bool kin = off < kbytes; // kbytes is a multiple of 16 on this path
+    int coff = kin ? off : 0;
+#pragma unroll
+    for (int i = 0; i < Gm::NCH; ++i) {
+      v4i v = *(const v4i *)(ptr[i] + coff);
+      regs[i] = (kin && ok[i]) ? v : v4i{0, 0, 0, 0};
+    }
+  }
+};
+
+// Assemble one chunk element by element through a caller-supplied fetch.
+template <int DT, typename F>
+__device__ __forceinline__ v4i gather_chunk(F fetch) {
+  constexpr int ES = MmaTraits<DT>::ES;
+  v4i out = {0, 0, 0, 0};
+  if constexpr (ES == 4) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      out[e] = (int)fetch(e);
+  } else if constexpr (ES == 2) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      out[e >> 1] |= (int)(fetch(e) & 0xffffu) << (16 * (e & 1));
+  } else {
+#pragma unroll
+    for (int e = 0; e < 16; ++e)
+      out[e >> 2] |= (int)(fetch(e) & 0xffu) << (8 * (e & 3));
+  }
+  return out;
+}
+
+template <int ES>
+__device__ __forceinline__ uint32_t load_elem(const void *base, int64_t idx) {
+  if constexpr (ES == 4)
+    return ((const uint32_t *)base)[idx];
+  else if constexpr (ES == 2)
+    return ((const uint16_t *)base)[idx];
+  else
+    return ((const uint8_t *)base)[idx];
+}
+
+// Arbitrary strides: element (row, k) at base[row*rs + k*ks].
+template <int DT, int ROWS, int NT> struct RowsGeneric {
+  using Gm = TileGeom<DT, ROWS, NT>;
+  const void *base;
+  int64_t rs, ks;
+  int row0, rows_total, K, tid;
+
+  __device__ __forceinline__ void init(const void *b, int64_t row_stride,
+                                       int64_t k_stride, int r0, int rt, int k,
+                                       int t) {
+    base = b; rs = row_stride; ks = k_stride; row0 = r0; rows_total = rt; K = k; tid = t;
+  }
+  __device__ __forceinline__ void load(int kt, v4i (&regs)[Gm::NCH]) const {
+    const int c = tid & 7;
+#pragma unroll
+    for (int i = 0; i < Gm::NCH; ++i) {
+      int r = (tid >> 3) + i * Gm::ROW_STEP;
+      int gr = row0 + r;
+      bool rok = (r < ROWS) && (gr < rows_total);
+      int k0 = kt * Gm::BKE + c * Gm::EPC;
+      regs[i] = gather_chunk<DT>([&](int e) -> uint32_t {
+        int k = k0 + e;
+        return (rok && k < K) ? load_elem<Gm::ES>(base, (int64_t)gr * rs + (int64_t)k * ks) : 0u;
+      });
+    }
+  }
+};
+
+// Convolution input as the implicit-GEMM A operand: row m = (n, ho, wo),
+// reduction index = (y, x, c) with c fastest.  Channel-contiguous input whose
+// channel run is a whole number of chunks, so a chunk never straddles a tap.
+template <int DT, int ROWS, int NT> struct ConvInFast {
+  using Gm = TileGeom<DT, ROWS, NT>;
+  const char *pix[Gm::NCH]; // input(n, g, c=0, 0, 0)
+  int h0[Gm::NCH], w0[Gm::NCH];
+  bool ok[Gm::NCH];
+  const RockConvParams *p;
+  int y, x, cc; // tap and channel offset of this thread's chunk at tile kt
+  int K;
+
+  __device__ __forceinline__ void init(const void *in, const RockConvParams &cp,
+                                       int g, int row0, int tid) {
+    p = &cp;
+    K = cp.K;
+    const int c = tid & 7;
+    int k0 = c * Gm::EPC;
+    int tap = k0 / cp.c;
+    cc = k0 - tap * cp.c;
+    y = tap / cp.x;
+    x = tap - y * cp.x;
+#pragma unroll
+    for (int i = 0; i < Gm::NCH; ++i) {
+      int r = (tid >> 3) + i * Gm::ROW_STEP;
+      int m = row0 + r;
+      ok[i] = (r < ROWS) && (m < cp.M);
+      int mm = min(m, cp.M - 1);
+      int n = mm / (cp.ho * cp.wo);
+      int rem = mm - n * (cp.ho * cp.wo);
+      int ho = rem / cp.wo;
+      int wo = rem - ho * cp.wo;
+      h0[i] = ho * cp.stride_h - cp.pad_h;
+      w0[i] = wo * cp.stride_w - cp.pad_w;
+      pix[i] = (const char *)in + ((int64_t)n * cp.in_ns + (int64_t)g * cp.in_gs) * Gm::ES;
+    }
+  }
+  // must be called with kt = 0, 1, 2, ... in order (tap state advances)
+  __device__ __forceinline__ void load(int kt, v4i (&regs)[Gm::NCH]) {
+    const int k0 = kt * Gm::BKE + (threadIdx.x & 7) * Gm::EPC;
+    const bool kin = k0 < K;
+    const int dh = y * p->dil_h, dw = x * p->dil_w;
+#pragma unroll
+    for (int i = 0; i < Gm::NCH; ++i) {
+      int hi = h0[i] + dh, wi = w0[i] + dw;
+      bool v = kin && ok[i] && hi >= 0 && hi < p->hi && wi >= 0 && wi < p->wi;
+      int64_t off = v ? ((int64_t)hi * p->in_hs + (int64_t)wi * p->in_ws + cc) * Gm::ES : 0;
+      v4i d = *(const v4i *)(pix[i] + off);
+      regs[i] = v ? d : v4i{0, 0, 0, 0};
+    }
+    // advance to the next tile's tap
+    cc += Gm::BKE;
+    while (cc >= p->c) {
+      cc -= p->c;
+      if (++x == p->x) { x = 0; ++y; }
+    }
+  }
+};
+
+// Decompose the reduction index for the generic convolution loaders.
+__device__ __forceinline__ void conv_split_k(const RockConvParams &p, int k,
+                                             int &c, int &y, int &x) {
+  if (p.k_order_yxc) {
+    int tap = k / p.c;
+    c = k - tap * p.c;
+    y = tap / p.x;
+    x = tap - y * p.x;
+  } else {
+    int yx = p.y * p.x;
+    c = k / yx;
+    int tap = k - c * yx;
+    y = tap / p.x;
+    x = tap - y * p.x;
+  }
+}
+
+template <int DT, int ROWS, int NT> struct ConvInGeneric {
+  using Gm = TileGeom<DT, ROWS, NT>;
+  const void *in;
+  const RockConvParams *p;
+  int g, row0, tid;
+  __device__ __forceinline__ void init(const void *i, const RockConvParams &cp,
+                                       int gg, int r0, int t) {
+    in = i; p = &cp; g = gg; row0 = r0; tid = t;
+  }
+  __device__ __forceinline__ void load(int kt, v4i (&regs)[Gm::NCH]) const {
+    const int cidx = tid & 7;
+#pragma unroll
+    for (int i = 0; i < Gm::NCH; ++i) {
+      int r = (tid >> 3) + i * Gm::ROW_STEP;
+      int m = row0 + r;
+      bool rok = (r < ROWS) && (m < p->M);
+      int mm = min(m, p->M - 1);
+      int n = mm / (p->ho * p->wo);
+      int rem = mm - n * (p->ho * p->wo);
+      int ho = rem / p->wo, wo = rem - (rem / p->wo) * p->wo;
+      int k0 = kt * Gm::BKE + cidx * Gm::EPC;
+      regs[i] = gather_chunk<DT>([&](int e) -> uint32_t {
+        int k = k0 + e;
+        if (!rok || k >= p->K) return 0u;
+        int c, y, x;
+        conv_split_k(*p, k, c, y, x);
+        int hi = ho * p->stride_h + y * p->dil_h - p->pad_h;
+        int wi = wo * p->stride_w + x * p->dil_w - p->pad_w;
+        if (hi < 0 || hi >= p->hi || wi < 0 || wi >= p->wi) return 0u;
+        int64_t idx = (int64_t)n * p->in_ns + (int64_t)g * p->in_gs + (int64_t)c * p->in_cs +
+                      (int64_t)hi * p->in_hs + (int64_t)wi * p->in_ws;
+        return load_elem<Gm::ES>(in, idx);
+      });
+    }
+  }
+};
+
+template <int DT, int ROWS, int NT> struct ConvFilGeneric {
+  using Gm = TileGeom<DT, ROWS, NT>;
+  const void *fil;
+  const RockConvParams *p;
+  int g, row0, tid;
+  __device__ __forceinline__ void init(const void *f, const RockConvParams &cp,
+                                       int gg, int r0, int t) {
+    fil = f; p = &cp; g = gg; row0 = r0; tid = t;
+  }
+  __device__ __forceinline__ void load(int kt, v4i (&regs)[Gm::NCH]) const {
+    const int cidx = tid & 7;
+#pragma unroll
+    for (int i = 0; i < Gm::NCH; ++i) {
+      int r = (tid >> 3) + i * Gm::ROW_STEP;
+      int ko = row0 + r;
+      bool rok = (r < ROWS) && (ko < p->N);
+      int k0 = kt * Gm::BKE + cidx * Gm::EPC;
+      regs[i] = gather_chunk<DT>([&](int e) -> uint32_t {
+        int k = k0 + e;
+        if (!rok || k >= p->K) return 0u;
+        int c, y, x;
+        conv_split_k(*p, k, c, y, x);
+        int64_t idx = (int64_t)g * p->fil_gs + (int64_t)ko * p->fil_ks + (int64_t)c * p->fil_cs +
+                      (int64_t)y * p->fil_ys + (int64_t)x * p->fil_xs;
+        return load_elem<Gm::ES>(fil, idx);
+      });
+    }
+  }
+};
+
+// ---------------------------------------------------------------------------
+// LDS tile store / fragment read
+// ---------------------------------------------------------------------------
+template <int DT, int ROWS, int NT>
+__device__ __forceinline__ void store_tile(char *lds, const v4i (&regs)[TileGeom<DT, ROWS, NT>::NCH], int tid) {
+  using Gm = TileGeom<DT, ROWS, NT>;
+  const int c = tid & 7;
+#pragma unroll
+  for (int i = 0; i < Gm::NCH; ++i) {
+    int r = (tid >> 3) + i * Gm::ROW_STEP;
+    if (Gm::TOTAL % NT == 0 || r < ROWS)
+      *(v4i *)(lds + r * kRowBytes + swizzle(r, c) * kChunk) = regs[i];
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ Frag<DT> read_frag(const char *lds, int row, int step, int lane_grp) {
+  Frag<DT> f;
+  if constexpr (MmaTraits<DT>::CHUNKS == 1) {
+    int chunk = step * 4 + lane_grp;
+    f.c[0] = *(const v4i *)(lds + row * kRowBytes + swizzle(row, chunk) * kChunk);
+  } else {
+    f.c[0] = *(const v4i *)(lds + row * kRowBytes + swizzle(row, lane_grp) * kChunk);
+    f.c[1] = *(const v4i *)(lds + row * kRowBytes + swizzle(row, lane_grp + 4) * kChunk);
+  }
+  return f;
+}
+
+// ---------------------------------------------------------------------------
+// Epilogue
+// ---------------------------------------------------------------------------
+template <bool INT_ACC, typename Acc>
+__device__ __forceinline__ void epilogue_store4(const Acc &acc, const RockEpilogue &e,
+                                                const void *aux, void *out_base,
+                                                int64_t off, int64_t n_stride,
+                                                int n0, int n_limit, bool vec_ok) {
+  // acc[r] belongs to output channel n0 + r
+  const int od = e.out_dtype;
+  if (INT_ACC && od == ROCK_I32) {
+    int v[4]; // exact accumulators, optional int32 bias
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      v[r] = (int)acc[r];
+      if (e.has_bias && n0 + r < n_limit)
+        v[r] += ((const int *)aux)[n0 + r];
+    }
+    int *o = (int *)out_base;
+    if (vec_ok && n0 + 3 < n_limit) {
+      *(v4i *)(o + off) = v4i{v[0], v[1], v[2], v[3]};
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n0 + r < n_limit)
+          o[off + r * n_stride] = v[r];
+    }
+    return;
+  }
+  float v[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    float f;
+    if constexpr (INT_ACC)
+      f = ((float)(int)acc[r] - (float)e.zero_point) * e.scale;
+    else
+      f = (float)acc[r] * e.scale;
+    if (e.has_bias && n0 + r < n_limit)
+      f = f + ((const float *)aux)[n0 + r];
+    if (e.relu)
+      f = fmaxf(f, 0.0f);
+    v[r] = f;
+  }
+  const bool full = vec_ok && n0 + 3 < n_limit;
+  switch (od) {
+  case ROCK_F32: {
+    float *o = (float *)out_base;
+    if (full) {
+      *(v4f *)(o + off) = v4f{v[0], v[1], v[2], v[3]};
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n0 + r < n_limit) o[off + r * n_stride] = v[r];
+    }
+    break;
+  }
+  case ROCK_F16: {
+    _Float16 *o = (_Float16 *)out_base;
+    if (full) {
+      *(v4h *)(o + off) = v4h{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n0 + r < n_limit) o[off + r * n_stride] = (_Float16)v[r];
+    }
+    break;
+  }
+  case ROCK_BF16: {
+    __bf16 *o = (__bf16 *)out_base;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (n0 + r < n_limit) o[off + r * n_stride] = (__bf16)v[r];
+    break;
+  }
+  case ROCK_I8: {
+    int8_t *o = (int8_t *)out_base;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (n0 + r < n_limit) {
+        float q = __builtin_rintf(v[r] * e.inv_quant_scale) + (float)e.out_zero_point;
+        o[off + r * n_stride] = f32_to_i8_sat(q);
+      }
+    break;
+  }
+  case ROCK_FP8: {
+    uint8_t *o = (uint8_t *)out_base;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (n0 + r < n_limit) o[off + r * n_stride] = f32_to_e4m3fn_sat(v[r]);
+    break;
+  }
+  case ROCK_BF8: {
+    uint8_t *o = (uint8_t *)out_base;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (n0 + r < n_limit) o[off + r * n_stride] = f32_to_e5m2_sat(v[r]);
+    break;
+  }
+  case ROCK_I32: { // float accumulators written as int32 are not a legal problem
+    break;
+  }
+  }
+}
+
+// ---- parameter-block adapters ------------------------------------------------
+__device__ __forceinline__ int p_batch(const RockGemmParams &p) { return p.G; }
+__device__ __forceinline__ int p_batch(const RockConvParams &p) { return p.g; }
+
+__device__ __forceinline__ bool aligned_for_vec(const void *base, int64_t row_off, int out_dtype) {
+  // 4 consecutive outputs stored as one 8/16-byte access need that alignment
+  int es = (out_dtype == ROCK_F32 || out_dtype == ROCK_I32) ? 4 : 2;
+  return ((((uintptr_t)base) + (uintptr_t)row_off * es) & (uintptr_t)(4 * es - 1)) == 0;
+}
+
+__device__ __forceinline__ void out_row_addr(const RockGemmParams &p, int g, int m, const void *base,
+                                             int64_t &row_off, int64_t &n_stride, bool &vec_ok) {
+  row_off = (int64_t)g * p.c_gs + (int64_t)m * p.c_ms;
+  n_stride = p.c_ns;
+  vec_ok = (p.c_ns == 1) && aligned_for_vec(base, row_off, p.epi.out_dtype);
+}
+
+__device__ __forceinline__ void out_row_addr(const RockConvParams &p, int g, int m, const void *base,
+                                             int64_t &row_off, int64_t &n_stride, bool &vec_ok) {
+  int n = m / (p.ho * p.wo);
+  int rem = m - n * (p.ho * p.wo);
+  int ho = rem / p.wo;
+  int wo = rem - ho * p.wo;
+  row_off = (int64_t)n * p.out_ns + (int64_t)g * p.out_gs + (int64_t)ho * p.out_hs + (int64_t)wo * p.out_ws;
+  n_stride = p.out_ks;
+  vec_ok = (p.out_ks == 1) && aligned_for_vec(base, row_off, p.epi.out_dtype);
+}
+
+template <int DT, int ROWS, int NT, int KIND>
+__device__ __forceinline__ auto make_loader_a(const void *A, const RockGemmParams &p, int g, int m0, int tid) {
+  if constexpr (KIND == LD_ROWS_FAST) {
+    RowsFast<DT, ROWS, NT> l;
+    l.init((const char *)A + (int64_t)g * p.a_gs * MmaTraits<DT>::ES, p.a_ms, m0, p.M, p.K, tid);
+    return l;
+  } else {
+    RowsGeneric<DT, ROWS, NT> l;
+    l.init((const char *)A + (int64_t)g * p.a_gs * MmaTraits<DT>::ES, p.a_ms, p.a_ks, m0, p.M, p.K, tid);
+    return l;
+  }
+}
+template <int DT, int ROWS, int NT, int KIND>
+__device__ __forceinline__ auto make_loader_b(const void *B, const RockGemmParams &p, int g, int n0, int tid) {
+  if constexpr (KIND == LD_ROWS_FAST) {
+    RowsFast<DT, ROWS, NT> l;
+    l.init((const char *)B + (int64_t)g * p.b_gs * MmaTraits<DT>::ES, p.b_ns, n0, p.N, p.K, tid);
+    return l;
+  } else {
+    RowsGeneric<DT, ROWS, NT> l;
+    l.init((const char *)B + (int64_t)g * p.b_gs * MmaTraits<DT>::ES, p.b_ns, p.b_ks, n0, p.N, p.K, tid);
+    return l;
+  }
+}
+// convolution: "A" is the input image (implicit rows), "B" the filter
+template <int DT, int ROWS, int NT, int KIND>
+__device__ __forceinline__ auto make_loader_a(const void *in, const RockConvParams &p, int g, int m0, int tid) {
+  if constexpr (KIND == LD_CONV_IN_FAST) {
+    ConvInFast<DT, ROWS, NT> l;
+    l.init(in, p, g, m0, tid);
+    return l;
+  } else {
+    ConvInGeneric<DT, ROWS, NT> l;
+    l.init(in, p, g, m0, tid);
+    return l;
+  }
+}
+template <int DT, int ROWS, int NT, int KIND>
+__device__ __forceinline__ auto make_loader_b(const void *fil, const RockConvParams &p, int g, int n0, int tid) {
+  if constexpr (KIND == LD_ROWS_FAST) {
+    RowsFast<DT, ROWS, NT> l;
+    l.init((const char *)fil + (int64_t)g * p.fil_gs * MmaTraits<DT>::ES, p.fil_ks, n0, p.N, p.K, tid);
+    return l;
+  } else {
+    ConvFilGeneric<DT, ROWS, NT> l;
+    l.init(fil, p, g, n0, tid);
+    return l;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// The kernel body.  IS_CONV selects the parameter block type.
+// ---------------------------------------------------------------------------
+template <int DT, int BM, int BN, int WAVES_M, int WAVES_N, int LDA, int LDB, typename Params>
+__device__ __forceinline__ void contraction_body(const void *Aptr, const void *Bptr, void *Cptr,
+                                                 const void *aux, const Params &p) {
+  using Tr = MmaTraits<DT>;
+  using Acc = typename Tr::Acc;
+  constexpr int NT = WAVES_M * WAVES_N * 64;
+  constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N; // wave tile
+  constexpr int MI = WTM / 16, NI = WTN / 16;
+  constexpr int STEPS = (Tr::CHUNKS == 1) ? 2 : 1; // MFMA K steps per 128-byte tile row
+  constexpr int A_BYTES = BM * kRowBytes, B_BYTES = BN * kRowBytes;
+  static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be a multiple of 16");
+
+  __shared__ __attribute__((aligned(16))) char lds[2 * (A_BYTES + B_BYTES)];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+  const int lrow = lane & 15, lgrp = lane >> 4;
+
+  int g, tm, tn;
+  decode_block(p.tiles_m, p.tiles_n, p_batch(p), p.group_m, p.xcd_remap, g, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  // ---- loaders
+  using GA = TileGeom<DT, BM, NT>;
+  using GB = TileGeom<DT, BN, NT>;
+  auto la = make_loader_a<DT, BM, NT, LDA>(Aptr, p, g, m0, tid);
+  auto lb = make_loader_b<DT, BN, NT, LDB>(Bptr, p, g, n0, tid);
+  v4i ra[GA::NCH], rb[GB::NCH];
+
+  Acc acc[MI][NI];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NI; ++j)
+      acc[i][j] = Acc{0, 0, 0, 0};
+
+  const int K = p.K;
+  const int nk = (K + GA::BKE - 1) / GA::BKE;
+
+  la.load(0, ra);
+  lb.load(0, rb);
+  store_tile<DT, BM, NT>(lds, ra, tid);
+  store_tile<DT, BN, NT>(lds + A_BYTES, rb, tid);
+  __syncthreads();
+
+  for (int kt = 0; kt < nk; ++kt) {
+    const int cur = kt & 1;
+    const char *sa = lds + cur * (A_BYTES + B_BYTES);
+    const char *sb = sa + A_BYTES;
+    const bool more = kt + 1 < nk;
+    if (more) {
+      la.load(kt + 1, ra);
+      lb.load(kt + 1, rb);
+    }
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      Frag<DT> fb[NI];
+#pragma unroll
+      for (int j = 0; j < NI; ++j)
+        fb[j] = read_frag<DT>(sb, wn * WTN + j * 16 + lrow, s, lgrp);
+#pragma unroll
+      for (int i = 0; i < MI; ++i) {
+        Frag<DT> fa = read_frag<DT>(sa, wm * WTM + i * 16 + lrow, s, lgrp);
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+          mma16<DT>(fb[j], fa, acc[i][j]);
+      }
+    }
+    if (more) {
+      char *da = lds + (cur ^ 1) * (A_BYTES + B_BYTES);
+      store_tile<DT, BM, NT>(da, ra, tid);
+      store_tile<DT, BN, NT>(da + A_BYTES, rb, tid);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane holds m = .. + lrow, n = .. + 4*lgrp + {0..3}
+  const RockEpilogue &e = p.epi;
+#pragma unroll
+  for (int i = 0; i < MI; ++i) {
+    const int m = m0 + wm * WTM + i * 16 + lrow;
+    if (m >= p.M)
+      continue;
+    int64_t row_off, n_stride;
+    bool vec_ok;
+    out_row_addr(p, g, m, Cptr, row_off, n_stride, vec_ok);
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int n = n0 + wn * WTN + j * 16 + lgrp * 4;
+      if (n >= p.N)
+        continue;
+      epilogue_store4<Tr::INT_ACC>(acc[i][j], e, aux, Cptr, row_off + (int64_t)n * n_stride,
+                                   n_stride, n, p.N, vec_ok);
+    }
+  }
+}
+
+} // namespace rk

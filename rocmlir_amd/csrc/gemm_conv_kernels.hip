@@ -1,0 +1,39 @@
+// Instantiations of the contraction kernel for one operand type.  Compiled
+// once per type with -DROCK_DT=<code> -DROCK_DTNAME=<name> into a gfx950 code
+// object; the host library picks a kernel by name from its perf-config table.
+#include "gemm_conv_kernel.h"
+
+#ifndef ROCK_DT
+#error "compile with -DROCK_DT=<operand type code> -DROCK_DTNAME=<suffix>"
+#endif
+
+#define RK_CAT_(a, b) a##b
+#define RK_CAT(a, b) RK_CAT_(a, b)
+
+#define RK_GEMM(NAME, BM, BN, WM, WN, LA, LB)                                           \
+  extern "C" __global__ __launch_bounds__(WM *WN * 64) void RK_CAT(                     \
+      RK_CAT(rock_gemm_, ROCK_DTNAME), NAME)(const void *A, const void *B, void *C,     \
+                                             const void *aux, RockGemmParams p) {       \
+    rk::contraction_body<ROCK_DT, BM, BN, WM, WN, LA, LB>(A, B, C, aux, p);             \
+  }
+
+// convolution pointer order follows the reference: filter, input, output
+#define RK_CONV(NAME, BM, BN, WM, WN, LA, LB)                                           \
+  extern "C" __global__ __launch_bounds__(WM *WN * 64) void RK_CAT(                     \
+      RK_CAT(rock_conv_, ROCK_DTNAME), NAME)(const void *fil, const void *in, void *out,\
+                                             const void *aux, RockConvParams p) {       \
+    rk::contraction_body<ROCK_DT, BM, BN, WM, WN, LA, LB>(in, fil, out, aux, p);        \
+  }
+
+RK_GEMM(_256x256_fast, 256, 256, 2, 4, rk::LD_ROWS_FAST, rk::LD_ROWS_FAST)
+RK_GEMM(_256x128_fast, 256, 128, 4, 2, rk::LD_ROWS_FAST, rk::LD_ROWS_FAST)
+RK_GEMM(_128x128_fast, 128, 128, 2, 2, rk::LD_ROWS_FAST, rk::LD_ROWS_FAST)
+RK_GEMM(_64x64_fast, 64, 64, 2, 2, rk::LD_ROWS_FAST, rk::LD_ROWS_FAST)
+RK_GEMM(_64x64_generic, 64, 64, 2, 2, rk::LD_ROWS_GENERIC, rk::LD_ROWS_GENERIC)
+
+#if ROCK_DT != 7 && ROCK_DT != 8
+RK_CONV(_256x128_fast, 256, 128, 4, 2, rk::LD_CONV_IN_FAST, rk::LD_ROWS_FAST)
+RK_CONV(_128x128_fast, 128, 128, 2, 2, rk::LD_CONV_IN_FAST, rk::LD_ROWS_FAST)
+RK_CONV(_64x64_fast, 64, 64, 2, 2, rk::LD_CONV_IN_FAST, rk::LD_ROWS_FAST)
+RK_CONV(_64x64_generic, 64, 64, 2, 2, rk::LD_CONV_IN_GENERIC, rk::LD_CONV_FIL_GENERIC)
+#endif

@@ -1,0 +1,86 @@
+// By-value parameter blocks passed to the gfx950 kernels after their pointer
+// arguments.  Shared between the host library (which fills them from the
+// parsed problem) and the device code.  Plain C layout, no padding surprises:
+// every field is 4 or 8 bytes and 8-byte fields come first.
+//
+// The reference bakes shapes into each generated kernel and passes only bare
+// pointers (mlir/lib/Dialect/Rock/Pipelines/Pipelines.cpp:246-248); the
+// hand-written kernels take the same bare pointers followed by one of these
+// blocks, which the C-ABI hands to the caller together with the code object.
+#pragma once
+#include <stdint.h>
+
+// element types; values are part of the C-ABI (rocmlir_amd.h)
+enum RockDType : int32_t {
+  ROCK_F32 = 0,
+  ROCK_F16 = 1,
+  ROCK_BF16 = 2,
+  ROCK_I8 = 3,
+  ROCK_FP8 = 4, // OCP e4m3fn
+  ROCK_BF8 = 5, // OCP e5m2
+  ROCK_I32 = 6,
+  ROCK_DTYPE_COUNT = 7
+};
+
+// Epilogue applied to the accumulator tile before the store
+// (MIGraphXToTosa.cpp:874-982 formulas; GemmToGridwise.cpp:241-263 cast).
+//   float accumulators:  v = acc * scale (+ bias[n])            -> cast
+//   int32 accumulators:  out i32: acc (+ bias_i32[n])
+//                        out float: v = (float(acc) - float(zero_point)) * scale
+//                                   (+ bias[n])                 -> cast
+//   out i8 (either):     q = clamp(roundeven(v * inv_quant_scale) + out_zero_point)
+struct RockEpilogue {
+  float scale;          // 1.0f = identity
+  float inv_quant_scale; // 1/scale of the requantisation step (out i8 only)
+  int32_t zero_point;   // subtracted from an int32 accumulator
+  int32_t out_zero_point;
+  int32_t has_bias;     // aux pointer holds one f32 (or i32 for i32 out) per output channel
+  int32_t out_dtype;    // RockDType
+  int32_t relu;         // clamp at zero after scale/bias
+  int32_t pad_;
+};
+
+struct RockGemmParams {
+  // element strides of the logical views A[g,m,k], B[g,n,k], C[g,m,n]
+  int64_t a_gs, a_ms, a_ks;
+  int64_t b_gs, b_ns, b_ks;
+  int64_t c_gs, c_ms, c_ns;
+  int32_t G, M, N, K;
+  int32_t tiles_m, tiles_n; // block tiles per batch entry
+  int32_t group_m;          // tile rows per L2 group
+  int32_t xcd_remap;        // 1: undo the round-robin block->XCD dispatch
+  RockEpilogue epi;
+};
+
+// Forward convolution as an implicit GEMM:
+//   M = N*Ho*Wo (output pixels), N = K_out per group, K = Y*X*C per group.
+// Strides are in elements of the respective tensor.
+struct RockConvParams {
+  int64_t in_ns, in_gs, in_cs, in_hs, in_ws;
+  int64_t fil_gs, fil_ks, fil_cs, fil_ys, fil_xs;
+  int64_t out_ns, out_gs, out_ks, out_hs, out_ws;
+  int32_t n, g, c, k; // c, k per group
+  int32_t hi, wi, y, x, ho, wo;
+  int32_t stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
+  int32_t M, N, K;    // implicit GEMM sizes
+  int32_t tiles_m, tiles_n;
+  int32_t group_m, xcd_remap;
+  int32_t k_order_yxc; // 1: reduction index runs (y,x,c) with c fastest; 0: (c,y,x)
+  int32_t pad_;
+  RockEpilogue epi;
+};
+
+struct RockAttentionParams {
+  // element strides of the logical views Q[g,i,d], K[g,j,d], V[g,j,e], O[g,i,e]
+  int64_t q_gs, q_is, q_ds;
+  int64_t k_gs, k_js, k_ds;
+  int64_t v_gs, v_js, v_es;
+  int64_t o_gs, o_is, o_es;
+  int64_t bias_gs, bias_is, bias_js; // optional additive bias [g,i,j] (aux pointer)
+  int32_t G, seq_q, seq_k, d_qk, d_v;
+  int32_t q_blocks;    // blocks of query rows per g
+  float scale;         // multiplies Q*K^T before the softmax
+  int32_t has_bias;
+  int32_t xcd_remap;
+  int32_t pad_;
+};

@@ -1,0 +1,1004 @@
+// Host side of librocmlir_amd.so: problem-string parsing and validation,
+// perf-config table, problem keys, code-object hand-out and a launch helper.
+//
+// It stands where the reference has ConvGenerator::parseConvConfig /
+// isApplicable (mlir/lib/Dialect/Rock/Generator/ConvGenerator.cpp:136-248,
+// 487-749), the op verifiers (mlir/lib/Dialect/Rock/IR/RockDialect.cpp:509-568,
+// 808-893,2071-2106), the tuning heuristics and problem keys
+// (mlir/lib/Dialect/Rock/Tuning/GridwiseGemmParams.cpp, RockTuningImpl.cpp:
+// 550-871) and the Miir entry points (mlir/tools/rocmlir-lib/rocmlir-lib.cpp:
+// 117-316).  There is no compiler behind it: kernels are hand-written HIP,
+// compiled ahead of time for gfx950 and embedded in this library.
+#include "../../include/rocmlir_amd.h"
+#include "kernel_params.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <sstream>
+#include <string>
+#include <vector>
+
+namespace {
+
+// --------------------------------------------------------------------------
+// error text (per thread)
+// --------------------------------------------------------------------------
+thread_local std::string g_last_error;
+
+void set_error(const std::string &msg) { g_last_error = msg; }
+
+// --------------------------------------------------------------------------
+// embedded gfx950 code objects (see blobs.S)
+// --------------------------------------------------------------------------
+#define ROCK_BLOB(n)                                                           \
+  extern "C" const char rock_hsaco_##n##_start[];                              \
+  extern "C" const char rock_hsaco_##n##_end[];
+#include "blobs.inc"
+#undef ROCK_BLOB
+
+struct Blob {
+  const char *name;
+  const char *start;
+  const char *end;
+};
+const Blob kBlobs[] = {
+#define ROCK_BLOB(n) {#n, rock_hsaco_##n##_start, rock_hsaco_##n##_end},
+#include "blobs.inc"
+#undef ROCK_BLOB
+};
+
+const Blob *find_blob(const std::string &name) {
+  for (const Blob &b : kBlobs)
+    if (name == b.name)
+      return &b;
+  return nullptr;
+}
+
+// --------------------------------------------------------------------------
+// option parsing: "--key value", "-key value", "--key=value"
+// (ConvGenerator.cpp:82-98 tokeniser, widened to rocmlir-gen's spellings)
+// --------------------------------------------------------------------------
+using OptMap = std::map<std::string, std::string>;
+
+bool parse_options(const char *text, OptMap &out) {
+  if (!text)
+    return false;
+  std::istringstream iss(text);
+  std::string tok, key;
+  while (iss >> tok) {
+    bool is_key = tok.size() > 1 && tok[0] == '-' &&
+                  !(std::isdigit((unsigned char)tok[1]) || tok[1] == '.');
+    if (is_key) {
+      if (!key.empty())
+        out[key] = "true"; // flag without a value
+      size_t p = tok.find_first_not_of('-');
+      if (p == std::string::npos)
+        return false;
+      key = tok.substr(p);
+      size_t eq = key.find('=');
+      if (eq != std::string::npos) {
+        out[key.substr(0, eq)] = key.substr(eq + 1);
+        key.clear();
+      }
+    } else {
+      if (key.empty())
+        continue; // stray value: ignored as the reference does
+      out[key] = tok;
+      key.clear();
+    }
+  }
+  if (!key.empty())
+    out[key] = "true";
+  return true;
+}
+
+bool get_int(const OptMap &m, const std::string &k, int64_t &v) {
+  auto it = m.find(k);
+  if (it == m.end())
+    return false;
+  char *end = nullptr;
+  long long r = std::strtoll(it->second.c_str(), &end, 10);
+  if (end == it->second.c_str() || *end != '\0')
+    return false;
+  v = r;
+  return true;
+}
+int64_t int_or(const OptMap &m, const std::string &k, int64_t dflt) {
+  int64_t v;
+  return get_int(m, k, v) ? v : dflt;
+}
+bool bool_or(const OptMap &m, const std::string &k, bool dflt) {
+  auto it = m.find(k);
+  if (it == m.end())
+    return dflt;
+  const std::string &s = it->second;
+  return s == "true" || s == "1" || s == "True";
+}
+bool get_float(const OptMap &m, const std::string &k, float &v) {
+  auto it = m.find(k);
+  if (it == m.end())
+    return false;
+  char *end = nullptr;
+  double r = std::strtod(it->second.c_str(), &end);
+  if (end == it->second.c_str() || *end != '\0')
+    return false;
+  v = (float)r;
+  return true;
+}
+std::string str_or(const OptMap &m, const std::string &k, const std::string &d) {
+  auto it = m.find(k);
+  return it == m.end() ? d : it->second;
+}
+
+// --------------------------------------------------------------------------
+// element types
+// --------------------------------------------------------------------------
+int parse_dtype(std::string s) {
+  // Miir spellings (ConvGenerator.cpp:569-590) and MLIR names; on gfx950 the
+  // short 8-bit float names mean the OCP formats (rocmlir-gen.cpp:3709-3729).
+  if (s == "f32" || s == "fp32") return ROCK_F32;
+  if (s == "f16" || s == "fp16") return ROCK_F16;
+  if (s == "bf16") return ROCK_BF16;
+  if (s == "i8" || s == "int8") return ROCK_I8;
+  if (s == "fp8" || s == "f8E4M3FN") return ROCK_FP8;
+  if (s == "bf8" || s == "f8E5M2") return ROCK_BF8;
+  if (s == "i32" || s == "int32") return ROCK_I32;
+  return -1;
+}
+const char *dtype_name(int t) {
+  static const char *n[] = {"f32", "f16", "bf16", "i8", "fp8", "bf8", "i32"};
+  return (t >= 0 && t < ROCK_DTYPE_COUNT) ? n[t] : "?";
+}
+int dtype_size(int t) {
+  switch (t) {
+  case ROCK_F32: case ROCK_I32: return 4;
+  case ROCK_F16: case ROCK_BF16: return 2;
+  default: return 1;
+  }
+}
+bool is_float_in(int t) { return t != ROCK_I8 && t != ROCK_I32; }
+
+// internal operand-pair code (mfma_gfx950.h): the public codes plus the two
+// mixed 8-bit float pairs; -1 if the pair has no kernel
+int operand_code(int a, int b) {
+  if (a == b && a != ROCK_I32)
+    return a;
+  if (a == ROCK_FP8 && b == ROCK_BF8) return 7;
+  if (a == ROCK_BF8 && b == ROCK_FP8) return 8;
+  return -1;
+}
+const char *operand_name(int code) {
+  static const char *n[] = {"f32", "f16", "bf16", "i8", "fp8", "bf8", "", "fp8_bf8", "bf8_fp8"};
+  return n[code];
+}
+
+// --------------------------------------------------------------------------
+// tile variants: the "small perf-config table"
+// --------------------------------------------------------------------------
+struct Tile {
+  const char *suffix; // kernel name suffix
+  int bm, bn, waves_m, waves_n;
+  int blocks_per_cu;  // co-resident blocks (LDS bound)
+  float efficiency;   // relative per-tile MFMA efficiency used by the heuristic
+  bool gemm, conv;
+};
+const Tile kFastTiles[] = {
+    {"_256x256_fast", 256, 256, 2, 4, 1, 1.00f, true, false},
+    {"_256x128_fast", 256, 128, 4, 2, 1, 0.90f, true, true},
+    {"_128x128_fast", 128, 128, 2, 2, 2, 0.75f, true, true},
+    {"_64x64_fast", 64, 64, 2, 2, 4, 0.40f, true, true},
+};
+const Tile kGenericTile = {"_64x64_generic", 64, 64, 2, 2, 4, 0.1f, true, true};
+constexpr int kNumCU = 256; // MI355X
+constexpr int kNumXCD = 8;
+
+int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
+
+// pick the tile that minimises rounds * tile_area / efficiency
+const Tile *pick_tile(int64_t M, int64_t N, int G, bool conv, const std::string &force) {
+  const Tile *best = nullptr;
+  double best_cost = 0;
+  for (const Tile &t : kFastTiles) {
+    if (conv ? !t.conv : !t.gemm)
+      continue;
+    if (!force.empty()) {
+      if (force == std::to_string(t.bm) + "x" + std::to_string(t.bn))
+        return &t;
+      continue;
+    }
+    int64_t tiles = (int64_t)ceil_div(M, t.bm) * ceil_div(N, t.bn) * G;
+    // co-resident blocks share one CU's matrix cores, so what counts is the
+    // largest number of tiles any CU has to work through
+    int64_t per_cu = (tiles + kNumCU - 1) / kNumCU;
+    double cost = (double)per_cu * t.bm * t.bn / t.efficiency;
+    if (!best || cost < best_cost) {
+      best = &t;
+      best_cost = cost;
+    }
+  }
+  return best;
+}
+
+// --------------------------------------------------------------------------
+// problems
+// --------------------------------------------------------------------------
+enum OpKind { OP_GEMM, OP_CONV, OP_ATTENTION };
+
+struct Handle {
+  OpKind op;
+  std::string arch = "gfx950";
+  int num_cu = kNumCU;
+  int kernel_id = 0;
+  // resolved kernel
+  std::string kernel_name;
+  std::string blob_name;
+  const Blob *blob = nullptr;
+  uint32_t block_size = 0, grid_size = 0;
+  int num_pointers = 0;
+  std::vector<char> params; // by-value parameter block
+  std::string perf_config;
+  std::string problem_key;
+  bool tuned = false, lowered = false;
+  // typed views of `params`
+  RockEpilogue *epi = nullptr;
+  // launch cache: device -> function
+  std::map<int, hipFunction_t> functions;
+};
+
+bool parse_epilogue(const OptMap &o, int in_a, int out_dtype, RockEpilogue &e) {
+  e.scale = 1.0f;
+  e.inv_quant_scale = 1.0f;
+  e.zero_point = 0;
+  e.out_zero_point = 0;
+  e.has_bias = bool_or(o, "bias", false) ? 1 : 0;
+  e.out_dtype = out_dtype;
+  e.relu = bool_or(o, "relu", false) ? 1 : 0;
+  e.pad_ = 0;
+  get_float(o, "scale", e.scale);
+  float qs;
+  if (get_float(o, "quant_scale", qs)) {
+    if (qs == 0.0f)
+      return false;
+    e.inv_quant_scale = 1.0f / qs;
+  }
+  e.zero_point = (int32_t)int_or(o, "zero_point", 0);
+  e.out_zero_point = (int32_t)int_or(o, "out_zero_point", 0);
+  // legality (RockDialect.cpp:539-568): float in -> float out, int in -> int
+  // out; the fused quantisation epilogue additionally lets an int8 problem
+  // leave as a float (dequantizelinear) and a float problem leave as int8
+  // (quantizelinear).
+  if (is_float_in(in_a) && out_dtype == ROCK_I32)
+    return false;
+  return true;
+}
+
+void apply_tile_grid(const Tile &t, int64_t M, int64_t N, int G, int &tiles_m, int &tiles_n,
+                     int &group_m, int &xcd_remap, uint32_t &block, uint32_t &grid) {
+  tiles_m = ceil_div(M, t.bm);
+  tiles_n = ceil_div(N, t.bn);
+  group_m = std::min(tiles_m, t.bm >= 256 ? 4 : 8);
+  int64_t total = (int64_t)tiles_m * tiles_n * G;
+  xcd_remap = total >= 2 * kNumXCD ? 1 : 0;
+  block = (uint32_t)(t.waves_m * t.waves_n * 64);
+  grid = (uint32_t)total;
+}
+
+std::string perf_string(const Tile &t, int es) {
+  // v2:MPB,NPB,KpackPB,MPW,MnPerXdl,Kpack,splitK,forceUnroll,1
+  int kpack = 16 / es;
+  int kpack_per_block = 128 / 16;
+  char buf[96];
+  std::snprintf(buf, sizeof buf, "v2:%d,%d,%d,%d,%d,%d,1,1,1", t.bm, t.bn, kpack_per_block,
+                t.bm / t.waves_m, 16, kpack);
+  return buf;
+}
+
+// "--perf_config v2:MPB,NPB,..." selects a tile by its block sizes; anything
+// that does not name an available tile falls back to the table, like the
+// reference's tuningFallback (AffixTuningParameters.cpp:129-141).
+std::string forced_tile(const OptMap &o) {
+  std::string pc = str_or(o, "perf_config", "");
+  if (pc.rfind("v2:", 0) == 0)
+    pc = pc.substr(3);
+  int a = 0, b = 0;
+  if (std::sscanf(pc.c_str(), "%d,%d", &a, &b) == 2) {
+    for (const Tile &t : kFastTiles)
+      if (t.bm == a && t.bn == b)
+        return std::to_string(a) + "x" + std::to_string(b);
+  }
+  return "";
+}
+
+// ---- GEMM -----------------------------------------------------------------
+Handle *make_gemm(const OptMap &o) {
+  std::string t = str_or(o, "t", "f32");
+  int ta, tb;
+  size_t us = t.find('_');
+  if (us != std::string::npos) {
+    ta = parse_dtype(t.substr(0, us));
+    tb = parse_dtype(t.substr(us + 1));
+  } else {
+    ta = tb = parse_dtype(t);
+  }
+  if (ta < 0 || tb < 0 || ta == ROCK_I32 || tb == ROCK_I32) {
+    set_error("gemm: unknown data type '" + t + "'");
+    return nullptr;
+  }
+  int code = operand_code(ta, tb);
+  if (code < 0) {
+    set_error("gemm: unsupported operand type pair '" + t + "'");
+    return nullptr;
+  }
+  // default output type: i8 -> i32, 8-bit floats -> f32, else the input type
+  // (rocmlir-gen.cpp:432-458)
+  int dflt_out = ta == ROCK_I8 ? ROCK_I32 : (ta == ROCK_FP8 || ta == ROCK_BF8) ? ROCK_F32 : ta;
+  std::string outs = str_or(o, "out_datatype", str_or(o, "c_dtype", ""));
+  int tc = outs.empty() ? dflt_out : parse_dtype(outs);
+  if (tc < 0) {
+    set_error("gemm: unknown output type '" + outs + "'");
+    return nullptr;
+  }
+  int64_t G = int_or(o, "g", 1), M, N, K;
+  if (!get_int(o, "m", M) || !get_int(o, "n", N) || !get_int(o, "k", K) || G <= 0 || M <= 0 ||
+      N <= 0 || K <= 0 || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX || G > INT32_MAX) {
+    set_error("gemm: -m, -n, -k (and -g) must be given and positive");
+    return nullptr;
+  }
+  bool tA = bool_or(o, "transA", false), tB = bool_or(o, "transB", false),
+       tC = bool_or(o, "transC", false);
+
+  auto *h = new Handle;
+  h->op = OP_GEMM;
+  h->params.assign(sizeof(RockGemmParams), 0);
+  auto &p = *reinterpret_cast<RockGemmParams *>(h->params.data());
+  h->epi = &p.epi;
+  if (!parse_epilogue(o, ta, tc, p.epi)) {
+    set_error("gemm: illegal input/output type combination or epilogue");
+    delete h;
+    return nullptr;
+  }
+  // storage (rocmlir-gen.cpp:2058-2080): A [G,M,K] (transA: [G,K,M]),
+  // B [G,K,N] (transB: [G,N,K]), C [G,M,N] (transC: [G,N,M])
+  p.G = (int)G; p.M = (int)M; p.N = (int)N; p.K = (int)K;
+  p.a_gs = M * K; p.a_ms = tA ? 1 : K; p.a_ks = tA ? M : 1;
+  p.b_gs = K * N; p.b_ks = tB ? 1 : N; p.b_ns = tB ? K : 1;
+  p.c_gs = M * N; p.c_ms = tC ? 1 : N; p.c_ns = tC ? M : 1;
+
+  const int es = dtype_size(ta);
+  const bool fast = p.a_ks == 1 && p.b_ks == 1 && (p.a_ms * es) % 16 == 0 &&
+                    (p.b_ns * es) % 16 == 0 && (K * es) % 16 == 0 && (p.a_gs * es) % 16 == 0 &&
+                    (p.b_gs * es) % 16 == 0;
+  const Tile *tile = fast ? pick_tile(M, N, (int)G, false, forced_tile(o)) : nullptr;
+  if (!tile)
+    tile = fast ? pick_tile(M, N, (int)G, false, "") : &kGenericTile;
+  apply_tile_grid(*tile, M, N, (int)G, p.tiles_m, p.tiles_n, p.group_m, p.xcd_remap,
+                  h->block_size, h->grid_size);
+  h->kernel_name = std::string("rock_gemm_") + operand_name(code) + tile->suffix;
+  h->blob_name = std::string("gemm_") + operand_name(code);
+  h->num_pointers = 4;
+  h->perf_config = perf_string(*tile, es);
+  // problem key (RockTuningImpl.cpp:808-862)
+  {
+    std::ostringstream k;
+    k << h->arch << '\t' << int_or(o, "num_cu", kNumCU) << '\t' << "-t " << operand_name(code)
+      << " -out_datatype " << dtype_name(tc) << " -transA " << (tA ? "true" : "false")
+      << " -transB " << (tB ? "true" : "false") << " -g " << G << " -m " << M << " -n " << N
+      << " -k " << K;
+    h->problem_key = k.str();
+  }
+  return h;
+}
+
+// ---- convolution --------------------------------------------------------------
+// letter-by-letter layout translation (ConvGenerator.cpp:641-647) widened to
+// rocmlir-gen's lowercase spellings with optional g (rocmlir-gen.cpp:837-863)
+bool canon_layout(std::string s, char channel, const char *want, std::string &out) {
+  // want: "gkcyx" / "ngchw" / "ngkhw"; `channel` is the tensor's own channel
+  // letter ('k' for filter/output second channel)
+  for (auto &ch : s)
+    ch = (char)std::tolower((unsigned char)ch);
+  const bool filter = want[0] == 'g' && want[1] == 'k';
+  std::string r;
+  for (char ch : s) {
+    char m = ch;
+    if (ch == '0') m = filter ? 'y' : 'h';
+    else if (ch == '1') m = filter ? 'x' : 'w';
+    else if (filter && ch == 'h') m = 'y';
+    else if (filter && ch == 'w') m = 'x';
+    else if (filter && ch == 'n') m = 'k';
+    else if (!filter && ch == 'y') m = 'h';
+    else if (!filter && ch == 'x') m = 'w';
+    else if (!filter && channel == 'k' && ch == 'c') m = 'k';
+    r.push_back(m);
+  }
+  if (r.find('g') == std::string::npos) {
+    if (filter) {
+      r = "g" + r;
+    } else {
+      std::string c1(1, channel);
+      if (r.size() >= 2 && r.substr(0, 2) == "n" + c1)
+        r = "ng" + c1 + r.substr(2);
+      else if (r[0] == 'n' && r.back() == channel)
+        r = r.substr(0, r.size() - 1) + "g" + c1;
+      else
+        r = "g" + r;
+    }
+  }
+  if (r.size() != 5)
+    return false;
+  std::string a = r, b = want;
+  std::sort(a.begin(), a.end());
+  std::sort(b.begin(), b.end());
+  if (a != b)
+    return false;
+  out = r;
+  return true;
+}
+
+void layout_strides(const std::string &layout, const std::string &letters, const int64_t *sizes,
+                    int64_t *strides) {
+  int64_t run = 1;
+  for (int pos = 4; pos >= 0; --pos) {
+    size_t idx = letters.find(layout[pos]);
+    strides[idx] = run;
+    run *= sizes[idx];
+  }
+}
+
+std::string key_layout(const std::string &layout, bool filter) {
+  // problem-key letters (RockTuningImpl.cpp:708-731): k->N (filter), c->C,
+  // g->G, n->N, output k->C, spatial -> 0,1
+  std::string r;
+  for (char ch : layout) {
+    switch (ch) {
+    case 'g': r.push_back('G'); break;
+    case 'n': r.push_back('N'); break;
+    case 'c': r.push_back('C'); break;
+    case 'k': r.push_back(filter ? 'N' : 'C'); break;
+    case 'y': case 'h': r.push_back('0'); break;
+    case 'x': case 'w': r.push_back('1'); break;
+    }
+  }
+  return r;
+}
+
+Handle *make_conv(const OptMap &o) {
+  // required keys (ConvGenerator.cpp:492-512); rocmlir-gen's "-t" sets all
+  // three types at once
+  std::string t_all = str_or(o, "t", "");
+  std::string in_t = str_or(o, "in_type", t_all), fil_t = str_or(o, "fil_type", t_all),
+              out_t = str_or(o, "out_type", str_or(o, "out_datatype", ""));
+  static const char *req[] = {"batchsize", "in_channels", "in_h", "in_w", "out_channels",
+                              "fil_h", "fil_w", "in_layout", "out_layout", "fil_layout"};
+  for (const char *k : req)
+    if (!o.count(k)) {
+      set_error(std::string("conv: missing --") + k);
+      return nullptr;
+    }
+  int ti = parse_dtype(in_t), tf = parse_dtype(fil_t);
+  if (ti < 0 || tf < 0 || ti != tf || ti == ROCK_I32) {
+    set_error("conv: input and filter types must be given, known and equal");
+    return nullptr;
+  }
+  int dflt_out = ti == ROCK_I8 ? ROCK_I32 : (ti == ROCK_FP8 || ti == ROCK_BF8) ? ROCK_F32 : ti;
+  int to = out_t.empty() ? dflt_out : parse_dtype(out_t);
+  if (to < 0) {
+    set_error("conv: unknown output type");
+    return nullptr;
+  }
+  std::string fl, il, ol;
+  if (!canon_layout(str_or(o, "fil_layout", ""), 'k', "gkcyx", fl) ||
+      !canon_layout(str_or(o, "in_layout", ""), 'c', "ngchw", il) ||
+      !canon_layout(str_or(o, "out_layout", ""), 'k', "ngkhw", ol)) {
+    set_error("conv: unsupported layout string (2-D, five dimensions with g)");
+    return nullptr;
+  }
+  int64_t n = int_or(o, "batchsize", 0), g = int_or(o, "groupsize", 1),
+          ct = int_or(o, "in_channels", 0), kt = int_or(o, "out_channels", 0),
+          hi = int_or(o, "in_h", 0), wi = int_or(o, "in_w", 0), y = int_or(o, "fil_h", 0),
+          x = int_or(o, "fil_w", 0);
+  int64_t dh = int_or(o, "dilation_h", 1), dw = int_or(o, "dilation_w", 1),
+          sh = int_or(o, "conv_stride_h", 1), sw = int_or(o, "conv_stride_w", 1),
+          ph = int_or(o, "padding_h", 0), pw = int_or(o, "padding_w", 0);
+  int64_t ph_r = int_or(o, "padding_h_r", ph), pw_r = int_or(o, "padding_w_r", pw);
+  ph = int_or(o, "padding_h_l", ph);
+  pw = int_or(o, "padding_w_l", pw);
+  // ConvGenerator.cpp:136-248
+  if (dh <= 0 || dw <= 0 || sh <= 0 || sw <= 0 || ph < 0 || pw < 0 || ph_r < 0 || pw_r < 0) {
+    set_error("conv: dilation and stride must be positive, padding non-negative");
+    return nullptr;
+  }
+  if (n <= 0 || g <= 0 || ct <= 0 || kt <= 0 || hi <= 0 || wi <= 0 || y <= 0 || x <= 0 ||
+      ct % g != 0 || kt % g != 0) {
+    set_error("conv: tensor dimensions must be positive and channels divisible by groups");
+    return nullptr;
+  }
+  if (hi + ph + ph_r < (y - 1) * dh + 1 || wi + pw + pw_r < (x - 1) * dw + 1) {
+    set_error("conv: input, including padding, is smaller than the filter");
+    return nullptr;
+  }
+  // output extent (ConvGenerator.h:101-108)
+  int64_t ho = (hi + ph + ph_r - (y - 1) * dh - 1) / sh + 1;
+  int64_t wo = (wi + pw + pw_r - (x - 1) * dw - 1) / sw + 1;
+  int64_t given;
+  if ((get_int(o, "out_h", given) && given != ho) || (get_int(o, "out_w", given) && given != wo)) {
+    set_error("conv: out_h/out_w do not match the value computed from the other parameters");
+    return nullptr;
+  }
+  std::string opn = str_or(o, "operation", "conv");
+  if (opn != "conv" && opn != "conv2d") {
+    set_error("conv: only the forward direction is built (" + opn + " requested)");
+    return nullptr;
+  }
+  const int64_t c = ct / g, k = kt / g;
+  const int64_t Mg = n * ho * wo, Kg = c * y * x;
+  if (Mg > INT32_MAX || Kg > INT32_MAX) {
+    set_error("conv: problem too large for 32-bit tile indices");
+    return nullptr;
+  }
+
+  auto *h = new Handle;
+  h->op = OP_CONV;
+  h->params.assign(sizeof(RockConvParams), 0);
+  auto &p = *reinterpret_cast<RockConvParams *>(h->params.data());
+  h->epi = &p.epi;
+  if (!parse_epilogue(o, ti, to, p.epi)) {
+    set_error("conv: illegal input/output type combination or epilogue");
+    delete h;
+    return nullptr;
+  }
+  p.n = (int)n; p.g = (int)g; p.c = (int)c; p.k = (int)k;
+  p.hi = (int)hi; p.wi = (int)wi; p.y = (int)y; p.x = (int)x; p.ho = (int)ho; p.wo = (int)wo;
+  p.stride_h = (int)sh; p.stride_w = (int)sw; p.pad_h = (int)ph; p.pad_w = (int)pw;
+  p.dil_h = (int)dh; p.dil_w = (int)dw;
+  p.M = (int)Mg; p.N = (int)k; p.K = (int)Kg;
+  {
+    int64_t fsz[5] = {g, k, c, y, x}, isz[5] = {n, g, c, hi, wi}, osz[5] = {n, g, k, ho, wo};
+    int64_t fs[5], is[5], os[5];
+    layout_strides(fl, "gkcyx", fsz, fs);
+    layout_strides(il, "ngchw", isz, is);
+    layout_strides(ol, "ngkhw", osz, os);
+    p.fil_gs = fs[0]; p.fil_ks = fs[1]; p.fil_cs = fs[2]; p.fil_ys = fs[3]; p.fil_xs = fs[4];
+    p.in_ns = is[0]; p.in_gs = is[1]; p.in_cs = is[2]; p.in_hs = is[3]; p.in_ws = is[4];
+    p.out_ns = os[0]; p.out_gs = os[1]; p.out_ks = os[2]; p.out_hs = os[3]; p.out_ws = os[4];
+  }
+  p.k_order_yxc = (p.in_cs == 1) ? 1 : 0;
+  const int es = dtype_size(ti);
+  auto al = [&](int64_t elems) { return (elems * es) % 16 == 0; };
+  const bool fast = p.in_cs == 1 && al(c) && al(p.in_ws) && al(p.in_hs) && al(p.in_ns) &&
+                    al(p.in_gs) && p.fil_cs == 1 && p.fil_xs == c && p.fil_ys == x * c &&
+                    al(p.fil_ks) && al(p.fil_gs);
+  const Tile *tile = fast ? pick_tile(Mg, k, (int)g, true, forced_tile(o)) : nullptr;
+  if (!tile)
+    tile = fast ? pick_tile(Mg, k, (int)g, true, "") : &kGenericTile;
+  apply_tile_grid(*tile, Mg, k, (int)g, p.tiles_m, p.tiles_n, p.group_m, p.xcd_remap,
+                  h->block_size, h->grid_size);
+  h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + tile->suffix;
+  h->blob_name = std::string("gemm_") + dtype_name(ti);
+  h->num_pointers = 4;
+  h->perf_config = perf_string(*tile, es);
+  {
+    std::ostringstream key;
+    const char *opname = ti == ROCK_F32 ? "conv" : ti == ROCK_F16 ? "convfp16"
+                       : ti == ROCK_BF16 ? "convbfp16" : ti == ROCK_I8 ? "convint8"
+                       : ti == ROCK_FP8 ? "convfp8_fp8" : "convbf8_bf8";
+    key << h->arch << '\t' << int_or(o, "num_cu", kNumCU) << '\t' << opname << " -F 1 -f "
+        << key_layout(fl, true) << " -I " << key_layout(il, false) << " -O "
+        << key_layout(ol, false) << " -n " << n << " -c " << c << " -H " << hi << " -W " << wi
+        << " -k " << k << " -y " << y << " -x " << x << " -p " << ph << " -q " << pw << " -u "
+        << sh << " -v " << sw << " -l " << dh << " -j " << dw << " -g " << g;
+    h->problem_key = key.str();
+  }
+  return h;
+}
+
+// ---- attention --------------------------------------------------------------------
+Handle *make_attention(const OptMap &o) {
+  std::string t = str_or(o, "t", "f16");
+  int ty = parse_dtype(t);
+  if (ty != ROCK_F16 && ty != ROCK_BF16) {
+    set_error("attention: only f16 and bf16 kernels are built ('" + t + "' requested)");
+    return nullptr;
+  }
+  int64_t G = int_or(o, "g", 1), sq, sk, dqk, dv;
+  if (!get_int(o, "seq_len_q", sq) || !get_int(o, "seq_len_k", sk) ||
+      !get_int(o, "head_dim_qk", dqk) || !get_int(o, "head_dim_v", dv) || G <= 0 || sq <= 0 ||
+      sk <= 0 || dqk <= 0 || dv <= 0) {
+    set_error("attention: -seq_len_q, -seq_len_k, -head_dim_qk, -head_dim_v must be positive");
+    return nullptr;
+  }
+  if (dqk > 128 || dv > 128) {
+    set_error("attention: head dimensions above 128 have no kernel");
+    return nullptr;
+  }
+  bool tQ = bool_or(o, "transQ", false), tK = bool_or(o, "transK", false),
+       tV = bool_or(o, "transV", false), tO = bool_or(o, "transO", false);
+  bool has_bias = bool_or(o, "with-attn-bias", false);
+
+  auto *h = new Handle;
+  h->op = OP_ATTENTION;
+  h->params.assign(sizeof(RockAttentionParams), 0);
+  auto &p = *reinterpret_cast<RockAttentionParams *>(h->params.data());
+  // storage (rocmlir-gen.cpp:2149-2200): Q [G,sq,d] (transQ: [G,d,sq]);
+  // K [G,d,sk] (transK: [G,sk,d]); V [G,sk,dv] (transV: [G,dv,sk]);
+  // O [G,sq,dv] (transO: [G,dv,sq])
+  p.G = (int)G; p.seq_q = (int)sq; p.seq_k = (int)sk; p.d_qk = (int)dqk; p.d_v = (int)dv;
+  p.q_gs = sq * dqk; p.q_is = tQ ? 1 : dqk; p.q_ds = tQ ? sq : 1;
+  p.k_gs = sk * dqk; p.k_js = tK ? dqk : 1; p.k_ds = tK ? 1 : sk;
+  p.v_gs = sk * dv; p.v_js = tV ? 1 : dv; p.v_es = tV ? sk : 1;
+  p.o_gs = sq * dv; p.o_is = tO ? 1 : dv; p.o_es = tO ? sq : 1;
+  p.bias_gs = sq * sk; p.bias_is = sk; p.bias_js = 1;
+  p.has_bias = has_bias ? 1 : 0;
+  p.scale = 1.0f;
+  get_float(o, "scale", p.scale);
+  p.q_blocks = ceil_div(sq, 128);
+  int64_t total = G * p.q_blocks;
+  if (total > INT32_MAX) {
+    set_error("attention: too many blocks");
+    delete h;
+    return nullptr;
+  }
+  p.xcd_remap = total >= 2 * kNumXCD ? 1 : 0;
+  const bool fast = p.q_ds == 1 && p.k_ds == 1 && p.v_es == 1 && p.o_es == 1 && dqk % 8 == 0 &&
+                    dv % 8 == 0 && p.o_is % 4 == 0;
+  const int dmax = (dqk <= 64 && dv <= 64) ? 64 : 128;
+  char name[96];
+  std::snprintf(name, sizeof name, "rock_attention_%s_d%dx%d_%s", dtype_name(ty), dmax, dmax,
+                fast ? "fast" : "generic");
+  h->kernel_name = name;
+  h->blob_name = "attention";
+  h->num_pointers = 5;
+  h->block_size = 256;
+  h->grid_size = (uint32_t)total;
+  // attn:v1:MPB_G0,MPB_G1,NPB_G0,KpackPB,MPW,MnPerXdl,Kpack,forceUnroll
+  // (G0 M tiles seq_k, G0 N tiles seq_q)
+  h->perf_config = "attn:v1:64," + std::to_string(dmax) + ",128,8,32,32,8,1";
+  {
+    std::ostringstream key;
+    auto tf = [](bool b) { return b ? "true" : "false"; };
+    key << h->arch << '\t' << int_or(o, "num_cu", kNumCU) << '\t' << "-t " << dtype_name(ty)
+        << " -transQ " << tf(tQ) << " -transK " << tf(tK) << " -transV " << tf(tV) << " -transO "
+        << tf(tO) << " -g " << G << " -seq_len_q " << sq << " -seq_len_k " << sk
+        << " -head_dim_qk " << dqk << " -head_dim_v " << dv;
+    h->problem_key = key.str();
+  }
+  return h;
+}
+
+// --------------------------------------------------------------------------
+// module cache: one hipModule per (device, code object)
+// --------------------------------------------------------------------------
+std::mutex g_module_mutex;
+std::map<std::pair<int, const Blob *>, hipModule_t> g_modules;
+
+int get_function(Handle *h, hipFunction_t *fn) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess)
+    return (int)e;
+  auto it = h->functions.find(dev);
+  if (it != h->functions.end()) {
+    *fn = it->second;
+    return 0;
+  }
+  std::lock_guard<std::mutex> lock(g_module_mutex);
+  hipModule_t mod;
+  auto key = std::make_pair(dev, h->blob);
+  auto mit = g_modules.find(key);
+  if (mit == g_modules.end()) {
+    e = hipModuleLoadData(&mod, h->blob->start);
+    if (e != hipSuccess) {
+      set_error(std::string("hipModuleLoadData failed for ") + h->blob->name + ": " +
+                hipGetErrorString(e));
+      return (int)e;
+    }
+    g_modules[key] = mod;
+  } else {
+    mod = mit->second;
+  }
+  e = hipModuleGetFunction(fn, mod, h->kernel_name.c_str());
+  if (e != hipSuccess) {
+    set_error("kernel " + h->kernel_name + " not found in code object: " + hipGetErrorString(e));
+    return (int)e;
+  }
+  h->functions[dev] = *fn;
+  return 0;
+}
+
+int launch_once(Handle *h, hipFunction_t fn, void *const *pointers, hipStream_t stream) {
+  // argument buffer: the pointers, then the parameter block (8-byte aligned)
+  char buf[8 * 8 + 512];
+  size_t off = 0;
+  for (int i = 0; i < h->num_pointers; ++i, off += 8)
+    std::memcpy(buf + off, &pointers[i], 8);
+  std::memcpy(buf + off, h->params.data(), h->params.size());
+  size_t size = off + h->params.size();
+  void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, buf, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
+                    HIP_LAUNCH_PARAM_END};
+  return (int)hipModuleLaunchKernel(fn, h->grid_size, 1, 1, h->block_size, 1, 1, 0, stream,
+                                    nullptr, config);
+}
+
+bool check_launch_args(Handle *h, void *const *pointers, int num_pointers) {
+  if (!h || !pointers || num_pointers != h->num_pointers) {
+    set_error("launch: wrong number of pointer arguments");
+    return false;
+  }
+  if (!h->lowered) {
+    set_error("launch: miirLowerBin has not been called on this handle");
+    return false;
+  }
+  // the vector paths assume 16-byte aligned tensors (true for any allocator)
+  for (int i = 0; i < num_pointers; ++i)
+    if (((uintptr_t)pointers[i] & 15) != 0) {
+      set_error("launch: tensor pointers must be 16-byte aligned");
+      return false;
+    }
+  int aux_index = 3;
+  bool need_aux = h->op == OP_ATTENTION
+                      ? reinterpret_cast<RockAttentionParams *>(h->params.data())->has_bias != 0
+                      : h->epi->has_bias != 0;
+  for (int i = 0; i < num_pointers; ++i)
+    if (!pointers[i] && (i != aux_index || need_aux)) {
+      set_error("launch: NULL tensor pointer");
+      return false;
+    }
+  return true;
+}
+
+} // namespace
+
+// ============================================================================
+// C ABI
+// ============================================================================
+extern "C" {
+
+MiirHandle miirCreateHandle(const char *options) {
+  g_last_error.clear();
+  OptMap o;
+  if (!parse_options(options, o)) {
+    set_error("could not parse the options string");
+    return nullptr;
+  }
+  // arch: "[triple:]gfxNNN[:features]" (ConvGenerator.cpp:538-552); only
+  // gfx950 has kernels here
+  std::string arch = str_or(o, "arch", "gfx950");
+  if (arch.find("gfx950") == std::string::npos) {
+    set_error("only gfx950 is supported (got '" + arch + "')");
+    return nullptr;
+  }
+  std::string op = str_or(o, "operation", "");
+  Handle *h = nullptr;
+  try {
+    if (op == "gemm")
+      h = make_gemm(o);
+    else if (op == "attention")
+      h = make_attention(o);
+    else if (op == "conv" || op == "conv2d" || op == "conv_bwd_data" || op == "conv2d_bwd_data" ||
+             op == "conv_bwd_weight" || op == "conv2d_bwd_weight")
+      h = make_conv(o);
+    else
+      set_error("unknown --operation '" + op + "'");
+  } catch (...) {
+    set_error("internal error while building the problem");
+    h = nullptr;
+  }
+  if (!h)
+    return nullptr;
+  h->kernel_id = (int)int_or(o, "kernel_id", 0);
+  if (h->kernel_id != 0) { // forward ops are single-kernel
+    set_error("kernel_id out of range");
+    delete h;
+    return nullptr;
+  }
+  h->num_cu = (int)int_or(o, "num_cu", kNumCU);
+  h->blob = find_blob(h->blob_name);
+  if (!h->blob) {
+    set_error("no code object for " + h->blob_name);
+    delete h;
+    return nullptr;
+  }
+  return h;
+}
+
+int miirGetKernelCount(MiirHandle handle) { return handle ? 1 : -1; }
+
+int miirGetWorkspaceSize(MiirHandle handle) { return handle ? 0 : -1; }
+
+MiirStatus miirLowerTuningParams(MiirHandle handle) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h)
+    return MIIR_INVALID_PARAM;
+  h->tuned = true;
+  return MIIR_SUCCESS;
+}
+
+MiirStatus miirLowerBin(MiirHandle handle) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h)
+    return MIIR_INVALID_PARAM;
+  if (!h->blob || h->blob->end <= h->blob->start)
+    return MIIR_BUILD_FAILURE;
+  h->tuned = true;
+  h->lowered = true;
+  return MIIR_SUCCESS;
+}
+
+MiirStatus miirBufferGet(MiirHandle handle, char *buffer, size_t *size) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h || !size)
+    return MIIR_INVALID_PARAM;
+  if (!h->lowered)
+    return MIIR_INVALID_MODULE;
+  size_t n = (size_t)(h->blob->end - h->blob->start);
+  if (buffer) {
+    if (*size < n)
+      return MIIR_INVALID_PARAM;
+    std::memcpy(buffer, h->blob->start, n);
+  }
+  *size = n;
+  return MIIR_SUCCESS;
+}
+
+MiirStatus miirGetExecutionDims(MiirHandle handle, size_t *global_size, size_t *local_size) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h || !global_size || !local_size)
+    return MIIR_INVALID_PARAM;
+  if (!h->tuned)
+    return MIIR_INVALID_MODULE;
+  *global_size = (size_t)h->grid_size * h->block_size;
+  *local_size = h->block_size;
+  return MIIR_SUCCESS;
+}
+
+MiirStatus miirDestroyHandle(MiirHandle handle) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h)
+    return MIIR_INVALID_PARAM;
+  delete h;
+  return MIIR_SUCCESS;
+}
+
+MiirStatus rockamdGetKernelName(MiirHandle handle, char *buffer, size_t *size) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h || !size)
+    return MIIR_INVALID_PARAM;
+  size_t n = h->kernel_name.size() + 1;
+  if (buffer) {
+    if (*size < n)
+      return MIIR_INVALID_PARAM;
+    std::memcpy(buffer, h->kernel_name.c_str(), n);
+  }
+  *size = n;
+  return MIIR_SUCCESS;
+}
+
+MiirStatus rockamdGetKernelAttrs(MiirHandle handle, uint32_t attrs[2]) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h || !attrs)
+    return MIIR_INVALID_PARAM;
+  attrs[0] = h->block_size;
+  attrs[1] = h->grid_size;
+  return MIIR_SUCCESS;
+}
+
+MiirStatus rockamdGetKernelArgs(MiirHandle handle, int *num_pointers, void *params,
+                                size_t *params_size) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h || !params_size)
+    return MIIR_INVALID_PARAM;
+  if (num_pointers)
+    *num_pointers = h->num_pointers;
+  if (params) {
+    if (*params_size < h->params.size())
+      return MIIR_INVALID_PARAM;
+    std::memcpy(params, h->params.data(), h->params.size());
+  }
+  *params_size = h->params.size();
+  return MIIR_SUCCESS;
+}
+
+static size_t copy_string(const std::string &s, char *buffer, size_t buffer_size) {
+  if (buffer && buffer_size > 0)
+    std::strncpy(buffer, s.c_str(), buffer_size);
+  return s.size();
+}
+
+size_t rockamdGetPerfConfig(MiirHandle handle, char *buffer, size_t buffer_size) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h)
+    return (size_t)-1;
+  return copy_string(h->perf_config, buffer, buffer_size);
+}
+
+size_t rockamdGetProblemKey(MiirHandle handle, char *buffer, size_t buffer_size) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h)
+    return (size_t)-1;
+  return copy_string(h->problem_key, buffer, buffer_size);
+}
+
+MiirStatus rockamdSetScale(MiirHandle handle, float scale) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h)
+    return MIIR_INVALID_PARAM;
+  if (h->op == OP_ATTENTION)
+    reinterpret_cast<RockAttentionParams *>(h->params.data())->scale = scale;
+  else
+    h->epi->scale = scale;
+  return MIIR_SUCCESS;
+}
+
+MiirStatus rockamdSetZeroPoint(MiirHandle handle, int32_t zero_point) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h || h->op == OP_ATTENTION)
+    return MIIR_INVALID_PARAM;
+  h->epi->zero_point = zero_point;
+  return MIIR_SUCCESS;
+}
+
+int rockamdLaunch(MiirHandle handle, void *const *pointers, int num_pointers, void *stream) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!check_launch_args(h, pointers, num_pointers))
+    return (int)hipErrorInvalidValue;
+  hipFunction_t fn;
+  int rc = get_function(h, &fn);
+  if (rc != 0)
+    return rc;
+  rc = launch_once(h, fn, pointers, (hipStream_t)stream);
+  if (rc != 0)
+    set_error(std::string("launch failed: ") + hipGetErrorString((hipError_t)rc));
+  return rc;
+}
+
+int rockamdBenchmark(MiirHandle handle, void *const *pointers, int num_pointers, void *stream,
+                     int warmup, int iters, float *avg_ms) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!check_launch_args(h, pointers, num_pointers) || iters <= 0 || !avg_ms)
+    return (int)hipErrorInvalidValue;
+  hipFunction_t fn;
+  int rc = get_function(h, &fn);
+  if (rc != 0)
+    return rc;
+  hipStream_t s = (hipStream_t)stream;
+  for (int i = 0; i < warmup && rc == 0; ++i)
+    rc = launch_once(h, fn, pointers, s);
+  if (rc != 0)
+    return rc;
+  hipEvent_t e0, e1;
+  if ((rc = (int)hipEventCreate(&e0)) != 0)
+    return rc;
+  if ((rc = (int)hipEventCreate(&e1)) != 0) {
+    hipEventDestroy(e0);
+    return rc;
+  }
+  rc = (int)hipEventRecord(e0, s);
+  for (int i = 0; i < iters && rc == 0; ++i)
+    rc = launch_once(h, fn, pointers, s);
+  if (rc == 0)
+    rc = (int)hipEventRecord(e1, s);
+  if (rc == 0)
+    rc = (int)hipEventSynchronize(e1);
+  float ms = 0.0f;
+  if (rc == 0)
+    rc = (int)hipEventElapsedTime(&ms, e0, e1);
+  hipEventDestroy(e0);
+  hipEventDestroy(e1);
+  if (rc != 0) {
+    set_error(std::string("benchmark failed: ") + hipGetErrorString((hipError_t)rc));
+    return rc;
+  }
+  *avg_ms = ms / (float)iters;
+  return 0;
+}
+
+const char *rockamdGetLastError(void) { return g_last_error.c_str(); }
+
+} // extern "C"
