@@ -12,8 +12,8 @@
 //   * a wave owns 32 query rows; S^T = K_tile * Q^T is computed with the
 //     32x32x16 MFMA, whose result layout gives every lane ONE query column and
 //     16 of the 32 keys of the tile (the other 16 sit in lane ^ 32);
-//   * row max / row sum are therefore per-lane loops plus one
-//     v_permlane32_swap; the running max, sum and the rescale factor are
+//   * row max / row sum are therefore per-lane loops plus one exchange with
+//     lane ^ 32; the running max, sum and the rescale factor are
 //     per-lane scalars that apply directly to the O^T accumulators, which use
 //     the same "lane = query column" layout (O^T = V^T * P^T);
 //   * P^T is packed to 16-bit floats in registers and used as the MFMA column
@@ -33,17 +33,17 @@ constexpr int kBKV = 64;  // keys per tile
 constexpr int kAttnThreads = 256;
 constexpr int kVPitch = kBKV * 2 + 16; // bytes per V^T row in LDS
 
-__device__ __forceinline__ float half_swap_max(float x) {
-  // returns max(x[lane], x[lane ^ 32]) in every lane
-  auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x),
-                                            __builtin_bit_cast(unsigned, x), false, false);
-  return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+// value of x held by lane ^ 32.  (v_permlane32_swap would do, but the
+// compiler folds its two tied operands into one register when both are the
+// same value, which turns the swap into a copy; the LDS crossbar permute has
+// no such trap and costs two instructions per K/V tile.)
+__device__ __forceinline__ float other_half(float x) {
+  const int lane = (int)(threadIdx.x & 63);
+  int v = __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __builtin_bit_cast(int, x));
+  return __builtin_bit_cast(float, v);
 }
-__device__ __forceinline__ float half_swap_sum(float x) {
-  auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x),
-                                            __builtin_bit_cast(unsigned, x), false, false);
-  return __builtin_bit_cast(float, r[0]) + __builtin_bit_cast(float, r[1]);
-}
+__device__ __forceinline__ float half_swap_max(float x) { return fmaxf(x, other_half(x)); }
+__device__ __forceinline__ float half_swap_sum(float x) { return x + other_half(x); }
 
 template <int DT>
 __device__ __forceinline__ v16f mma32(const v4i &rows, const v4i &cols, const v16f &acc) {

@@ -333,15 +333,16 @@ __device__ __forceinline__ void store_tile(char *lds, const v4i (&regs)[TileGeom
   }
 }
 
+// Fragment of one 32-row block: lane (row = lane % 32, half = lane / 32)
+// takes chunk  step*2*CHUNKS + 2*c + half  for c in [0, CHUNKS).
 template <int DT>
-__device__ __forceinline__ Frag<DT> read_frag(const char *lds, int row, int step, int lane_grp) {
+__device__ __forceinline__ Frag<DT> read_frag(const char *lds, int row, int step, int half) {
   Frag<DT> f;
-  if constexpr (MmaTraits<DT>::CHUNKS == 1) {
-    int chunk = step * 4 + lane_grp;
-    f.c[0] = *(const v4i *)(lds + row * kRowBytes + swizzle(row, chunk) * kChunk);
-  } else {
-    f.c[0] = *(const v4i *)(lds + row * kRowBytes + swizzle(row, lane_grp) * kChunk);
-    f.c[1] = *(const v4i *)(lds + row * kRowBytes + swizzle(row, lane_grp + 4) * kChunk);
+  constexpr int CH = MmaTraits<DT>::CHUNKS;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    int chunk = step * 2 * CH + 2 * c + half;
+    f.c[c] = *(const v4i *)(lds + row * kRowBytes + swizzle(row, chunk) * kChunk);
   }
   return f;
 }
@@ -349,8 +350,8 @@ __device__ __forceinline__ Frag<DT> read_frag(const char *lds, int row, int step
 // ---------------------------------------------------------------------------
 // Epilogue
 // ---------------------------------------------------------------------------
-template <bool INT_ACC, typename Acc>
-__device__ __forceinline__ void epilogue_store4(const Acc &acc, const RockEpilogue &e,
+template <bool INT_ACC, typename Acc4>
+__device__ __forceinline__ void epilogue_store4(const Acc4 &acc, const RockEpilogue &e,
                                                 const void *aux, void *out_base,
                                                 int64_t off, int64_t n_stride,
                                                 int n0, int n_limit, bool vec_ok) {
@@ -538,17 +539,17 @@ __device__ __forceinline__ void contraction_body(const void *Aptr, const void *B
   using Acc = typename Tr::Acc;
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N; // wave tile
-  constexpr int MI = WTM / 16, NI = WTN / 16;
-  constexpr int STEPS = (Tr::CHUNKS == 1) ? 2 : 1; // MFMA K steps per 128-byte tile row
+  constexpr int MI = WTM / 32, NI = WTN / 32;
+  constexpr int STEPS = kChunksPerRow / (2 * Tr::CHUNKS); // MFMA K steps per 128-byte tile row
   constexpr int A_BYTES = BM * kRowBytes, B_BYTES = BN * kRowBytes;
-  static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be a multiple of 16");
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of 32");
 
   __shared__ __attribute__((aligned(16))) char lds[2 * (A_BYTES + B_BYTES)];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int wm = wave % WAVES_M, wn = wave / WAVES_M;
-  const int lrow = lane & 15, lgrp = lane >> 4;
+  const int lrow = lane & 31, lgrp = lane >> 5;
 
   int g, tm, tn;
   decode_block(p.tiles_m, p.tiles_n, p_batch(p), p.group_m, p.xcd_remap, g, tm, tn);
@@ -566,7 +567,9 @@ __device__ __forceinline__ void contraction_body(const void *Aptr, const void *B
   for (int i = 0; i < MI; ++i)
 #pragma unroll
     for (int j = 0; j < NI; ++j)
-      acc[i][j] = Acc{0, 0, 0, 0};
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        acc[i][j][v] = 0;
 
   const int K = p.K;
   const int nk = (K + GA::BKE - 1) / GA::BKE;
@@ -591,13 +594,13 @@ __device__ __forceinline__ void contraction_body(const void *Aptr, const void *B
       Frag<DT> fb[NI];
 #pragma unroll
       for (int j = 0; j < NI; ++j)
-        fb[j] = read_frag<DT>(sb, wn * WTN + j * 16 + lrow, s, lgrp);
+        fb[j] = read_frag<DT>(sb, wn * WTN + j * 32 + lrow, s, lgrp);
 #pragma unroll
       for (int i = 0; i < MI; ++i) {
-        Frag<DT> fa = read_frag<DT>(sa, wm * WTM + i * 16 + lrow, s, lgrp);
+        Frag<DT> fa = read_frag<DT>(sa, wm * WTM + i * 32 + lrow, s, lgrp);
 #pragma unroll
         for (int j = 0; j < NI; ++j)
-          mma16<DT>(fb[j], fa, acc[i][j]);
+          mma32x32<DT>(fb[j], fa, acc[i][j]);
       }
     }
     if (more) {
@@ -608,11 +611,12 @@ __device__ __forceinline__ void contraction_body(const void *Aptr, const void *B
     __syncthreads();
   }
 
-  // ---- epilogue: lane holds m = .. + lrow, n = .. + 4*lgrp + {0..3}
+  // ---- epilogue: lane holds m = .. + lrow, n = .. + 8*q + 4*lgrp + {0..3}
   const RockEpilogue &e = p.epi;
+  using Acc4 = decltype(__builtin_shufflevector(acc[0][0], acc[0][0], 0, 1, 2, 3));
 #pragma unroll
   for (int i = 0; i < MI; ++i) {
-    const int m = m0 + wm * WTM + i * 16 + lrow;
+    const int m = m0 + wm * WTM + i * 32 + lrow;
     if (m >= p.M)
       continue;
     int64_t row_off, n_stride;
@@ -620,11 +624,16 @@ __device__ __forceinline__ void contraction_body(const void *Aptr, const void *B
     out_row_addr(p, g, m, Cptr, row_off, n_stride, vec_ok);
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
-      const int n = n0 + wn * WTN + j * 16 + lgrp * 4;
-      if (n >= p.N)
-        continue;
-      epilogue_store4<Tr::INT_ACC>(acc[i][j], e, aux, Cptr, row_off + (int64_t)n * n_stride,
-                                   n_stride, n, p.N, vec_ok);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + wn * WTN + j * 32 + q * 8 + lgrp * 4;
+        if (n >= p.N)
+          continue;
+        Acc4 a4 = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                   acc[i][j][4 * q + 3]};
+        epilogue_store4<Tr::INT_ACC>(a4, e, aux, Cptr, row_off + (int64_t)n * n_stride, n_stride,
+                                     n, p.N, vec_ok);
+      }
     }
   }
 }

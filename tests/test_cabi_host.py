@@ -1,0 +1,172 @@
+"""Host-side checks of the C ABI that need no GPU: the library loads, exports
+every symbol the header declares, follows the Miir call protocol and error
+behaviour (rocmlir-lib.cpp:117-316, rocmlir-lib-test.cpp:31-96), and renders
+perf-config / problem-key strings in the reference's grammar."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+CONV_RESNET = (
+    "--operation conv --arch amdgcn-amd-amdhsa:gfx950 --num_cu 256 --in_type fp16 --fil_type fp16 "
+    "--out_type fp16 --fil_layout GNYXC --in_layout NHWGC --out_layout NHWGC --batchsize 256 "
+    "--groupsize 1 --in_channels 128 --out_channels 128 --in_h 28 --in_w 28 --out_h 28 --out_w 28 "
+    "--fil_h 3 --fil_w 3 --dilation_h 1 --dilation_w 1 --conv_stride_h 1 --conv_stride_w 1 "
+    "--padding_h 1 --padding_w 1")
+
+
+def test_every_declared_symbol_is_exported(rock):
+    header = open(os.path.join(ROOT, "include", "rocmlir_amd.h")).read()
+    names = re.findall(r"ROCMLIR_AMD_API\s+[\w\s\*]+?\b(\w+)\s*\(", header)
+    assert len(names) >= 18
+    lib = C.CDLL(rock.library_path())
+    for n in names:
+        assert hasattr(lib, n), n
+
+
+def test_miir_protocol_conv(rock):
+    lib = rock.load_library()
+    h = lib.miirCreateHandle(CONV_RESNET.encode())
+    assert h
+    assert lib.miirGetKernelCount(h) == 1
+    assert lib.miirGetWorkspaceSize(h) == 0
+    g, l = C.c_size_t(), C.c_size_t()
+    # launch dims and the binary need the lowering calls first
+    assert lib.miirGetExecutionDims(h, C.byref(g), C.byref(l)) == 2  # MIIR_INVALID_MODULE
+    n = C.c_size_t(0)
+    assert lib.miirBufferGet(h, None, C.byref(n)) == 2
+    assert lib.miirLowerTuningParams(h) == 0
+    assert lib.miirGetExecutionDims(h, C.byref(g), C.byref(l)) == 0
+    assert l.value in (256, 512) and g.value % l.value == 0
+    assert lib.miirLowerBin(h) == 0
+    assert lib.miirBufferGet(h, None, C.byref(n)) == 0 and n.value > 1000
+    buf = C.create_string_buffer(n.value)
+    small = C.c_size_t(10)
+    assert lib.miirBufferGet(h, buf, C.byref(small)) == 1  # MIIR_INVALID_PARAM: too small
+    assert lib.miirBufferGet(h, buf, C.byref(n)) == 0
+    assert buf.raw[:4] == b"\x7fELF"  # mlir/test/mlir-rock-lib/populate_fw.mlir checks "ELF"
+    assert lib.miirDestroyHandle(h) == 0
+
+
+def test_null_handle_behaviour(rock):
+    lib = rock.load_library()
+    assert lib.miirGetKernelCount(None) == -1
+    assert lib.miirLowerBin(None) == 1
+    assert lib.miirLowerTuningParams(None) == 1
+    assert lib.miirDestroyHandle(None) == 1
+    n = C.c_size_t(0)
+    assert lib.miirBufferGet(None, None, C.byref(n)) == 1
+
+
+@pytest.mark.parametrize("bad", [
+    "",                                                        # nothing
+    "--operation conv --arch gfx950",                          # missing tensor keys
+    CONV_RESNET.replace("--out_h 28", "--out_h 27"),           # inconsistent output size
+    CONV_RESNET.replace("--conv_stride_h 1", "--conv_stride_h 0"),
+    CONV_RESNET.replace("--padding_h 1", "--padding_h -1"),
+    CONV_RESNET.replace("--in_layout NHWGC", "--in_layout NHWC3"),
+    CONV_RESNET.replace("gfx950", "gfx906"),                   # no kernels for other chips
+    CONV_RESNET.replace("--operation conv", "--operation conv_bwd_data"),
+    CONV_RESNET.replace("--fil_type fp16", "--fil_type fp32"),
+    "--operation gemm --arch gfx950 -t f32 -m 4 -n 4",         # k missing
+    "--operation gemm --arch gfx950 -t f32 -m 4 -n 4 -k 0",
+    "--operation gemm --arch gfx950 -t f16 -out_datatype i32 -m 4 -n 4 -k 4",  # float in, int out
+    "--operation gemm --arch gfx950 -t f16_i8 -m 4 -n 4 -k 4",
+    "--operation attention --arch gfx950 -t f16 -g 1 -seq_len_q 8 -seq_len_k 8 -head_dim_qk 8",
+    "--operation attention --arch gfx950 -t f16 -g 1 -seq_len_q 8 -seq_len_k 8 -head_dim_qk 256 -head_dim_v 8",
+    "--operation transpose --arch gfx950",
+    CONV_RESNET + " --kernel_id 1",
+])
+def test_bad_problems_give_null(rock, bad):
+    lib = rock.load_library()
+    assert not lib.miirCreateHandle(bad.encode())
+    assert lib.rockamdGetLastError() != b""
+    with pytest.raises(rock.RockError):
+        rock.RockKernel(bad)
+
+
+def test_baseline_configs_select_kernels(rock):
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t f32 -g 1 -m 512 -n 512 -k 512 -transB true")
+    assert k.kernel_name.startswith("rock_gemm_f32_") and k.kernel_name.endswith("_fast")
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t i8 -out_datatype f16 -g 1 -m 4096 -n 4096 "
+                        "-k 4096 -transB true -scale 0.01")
+    assert k.kernel_name == "rock_gemm_i8_256x256_fast"
+    assert (k.block_size, k.grid_size) == (512, 256)
+    assert k.execution_dims() == (512 * 256, 512)
+    assert k.perf_config == "v2:256,256,8,128,16,16,1,1,1"
+    k = rock.RockKernel(CONV_RESNET)
+    assert k.kernel_name.startswith("rock_conv_f16_") and k.kernel_name.endswith("_fast")
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t fp8 -g 1 -m 8192 -n 8192 -k 8192 -transB true")
+    assert k.kernel_name == "rock_gemm_fp8_256x256_fast" and k.grid_size == 1024
+    k = rock.RockKernel("-operation attention -arch gfx950 -t f16 -g 128 -seq_len_q 2048 -seq_len_k 2048 "
+                        "-head_dim_qk 128 -head_dim_v 128 -transK true -scale 0.08838834764831845")
+    assert k.kernel_name == "rock_attention_f16_d128x128_fast"
+    assert (k.block_size, k.grid_size, k.num_pointers) == (256, 128 * 16, 5)
+
+
+def test_generic_kernels_for_unaligned_or_transposed(rock):
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 3 -m 1024 -k 769 -n 1024 -transB true")
+    assert k.kernel_name == "rock_gemm_f16_64x64_generic"          # odd K: no 16-byte chunks
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 64 -k 64 -n 64")
+    assert k.kernel_name == "rock_gemm_f16_64x64_generic"          # B is [K,N]: not K-contiguous
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 64 -k 64 -n 64 -transA false -transB true")
+    assert k.kernel_name.endswith("_fast")
+    k = rock.RockKernel(CONV_RESNET.replace("NHWGC", "NGCHW").replace("GNYXC", "GNCHW"))
+    assert k.kernel_name == "rock_conv_f16_64x64_generic"
+
+
+def test_perf_config_override_and_fallback(rock):
+    base = "-operation gemm -arch gfx950 -t i8 -g 1 -m 4096 -n 4096 -k 4096 -transB true"
+    assert rock.RockKernel(base + " -perf_config v2:128,128,8,64,16,16,1,1,1").kernel_name == \
+        "rock_gemm_i8_128x128_fast"
+    # a config naming no available tile falls back to the table
+    assert rock.RockKernel(base + " -perf_config v2:32,32,8,16,16,16,1,1,1").kernel_name == \
+        "rock_gemm_i8_256x256_fast"
+
+
+def test_problem_keys_follow_reference_format(rock):
+    # mlir/test/rocmlir-gen/problem-key.mlir CHECK_2 / CHECK_4 (numCU in the key)
+    k = rock.RockKernel("--arch gfx950 --num_cu 304 --operation attention -seq_len_q 256 -seq_len_k 512 "
+                        "-head_dim_qk 64 -head_dim_v 32 -t f16 -g 4")
+    arch, ncu, prob = k.problem_key.split("\t")
+    assert (arch, ncu) == ("gfx950", "304")
+    assert prob == ("-t f16 -transQ false -transK false -transV false -transO false -g 4 "
+                    "-seq_len_q 256 -seq_len_k 512 -head_dim_qk 64 -head_dim_v 32")
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 1024 -n 512 -k 769 -transB true")
+    assert k.problem_key.split("\t")[2] == \
+        "-t f16 -out_datatype f16 -transA false -transB true -g 1 -m 1024 -n 512 -k 769"
+    k = rock.RockKernel(CONV_RESNET)
+    assert k.problem_key.split("\t")[2] == (
+        "convfp16 -F 1 -f GN01C -I N01GC -O N01GC -n 256 -c 128 -H 28 -W 28 -k 128 -y 3 -x 3 "
+        "-p 1 -q 1 -u 1 -v 1 -l 1 -j 1 -g 1")
+
+
+def test_param_block_and_setters(rock):
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t i8 -out_datatype f16 -g 1 -m 64 -n 64 -k 64 "
+                        "-transB true -scale 0.5 -zero_point 3")
+    import struct
+    blob = k.params()
+    assert len(blob) == k.params_size == 9 * 8 + 8 * 4 + 8 * 4
+    G, M, N, K = struct.unpack_from("4i", blob, 72)
+    assert (G, M, N, K) == (1, 64, 64, 64)
+    scale, inv_q, zp = struct.unpack_from("ffi", blob, 72 + 32)
+    assert (scale, inv_q, zp) == (0.5, 1.0, 3)
+    k.set_scale(0.25)
+    k.set_zero_point(-2)
+    scale, inv_q, zp = struct.unpack_from("ffi", k.params(), 72 + 32)
+    assert (scale, zp) == (0.25, -2)
+
+
+def test_product_does_not_touch_the_oracle():
+    """The shipped package must not import, load or link the CPU oracle."""
+    pkg = os.path.join(ROOT, "rocmlir_amd")
+    for dirpath, _, files in os.walk(pkg):
+        if "_build" in dirpath:
+            continue
+        for f in files:
+            if f.endswith((".py", ".cpp", ".h", ".hip", ".S", ".inc")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "rock_oracle" not in text and "oracle/" not in text, f

@@ -1,0 +1,82 @@
+"""GPU parity: fused attention through the C ABI vs the f32 CPU oracle.
+
+Gates: the oracle is rounded through the 16-bit output type, then relative
+RMS <= 1e-3 and max-abs <= 0.02 (the reference's f16 attention tolerances are
+RMS 0.015 / abs 0.02 / rel 0.02, PrAttentionF16.toml:3; bf16 keeps only 8
+mantissa bits, so its gate is RMS 8e-3 / abs 0.06)."""
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import check_float, quantise, to_f32, to_gpu
+
+pytestmark = pytest.mark.gpu
+GATE = {"f16": (1e-3, 0.02), "bf16": (8e-3, 0.06)}
+
+
+def _store(mat, trans):
+    return np.ascontiguousarray(mat.transpose(0, 2, 1) if trans else mat)
+
+
+def _run(rock, oracle, gpu, t, G, sq, sk, dqk, dv, scale, seed, tQ=False, tK=True, tV=False, tO=False,
+         bias=False, vones=False):
+    rng = np.random.default_rng(seed)
+    Q = rng.standard_normal((G, sq, dqk)).astype(np.float32)
+    K = rng.standard_normal((G, sk, dqk)).astype(np.float32)
+    V = np.ones((G, sk, dv), np.float32) if vones else rng.standard_normal((G, sk, dv)).astype(np.float32)
+    rq, Qq = quantise(_store(Q, tQ), t)
+    rk, Kq = quantise(_store(K, not tK), t)     # default storage is [G,d,seq_k]
+    rv, Vq = quantise(_store(V, tV), t)
+    bq = braw = None
+    if bias:
+        braw, bq = quantise(rng.standard_normal((G, sq, sk)).astype(np.float32), t)
+    out = rock.attention(to_gpu(rq, t, gpu), to_gpu(rk, t, gpu), to_gpu(rv, t, gpu), scale=scale,
+                         bias=to_gpu(braw, t, gpu) if bias else None,
+                         transQ=tQ, transK=tK, transV=tV, transO=tO)
+    torch.cuda.synchronize()
+    ref = oracle.attention(Qq, Kq, Vq, G, sq, sk, dqk, dv, scale=scale, bias_t=bq,
+                           transQ=tQ, transK=tK, transV=tV, transO=tO)
+    return to_f32(out, t), ref
+
+
+# PrAttentionF16.toml:20-67 shapes (+ ragged ones)
+SHAPES = [
+    (1, 384, 384, 64, 64), (2, 64, 64, 64, 64), (1, 256, 256, 128, 128), (3, 128, 27, 64, 32),
+    (1, 1, 1, 8, 8), (2, 100, 333, 40, 72), (1, 300, 64, 128, 64), (2, 33, 130, 16, 128),
+]
+
+
+@pytest.mark.parametrize("t", ["f16", "bf16"])
+@pytest.mark.parametrize("G,sq,sk,dqk,dv", SHAPES)
+def test_attention_shapes(rock, oracle, gpu, t, G, sq, sk, dqk, dv):
+    got, ref = _run(rock, oracle, gpu, t, G, sq, sk, dqk, dv, 1.0 / np.sqrt(dqk), 41)
+    check_float(got, ref, t, rms=GATE[t][0], max_abs=GATE[t][1])
+
+
+@pytest.mark.parametrize("tQ,tK,tV,tO", [(0, 0, 0, 0), (1, 1, 0, 0), (0, 1, 1, 0), (0, 1, 0, 1), (1, 0, 1, 1)])
+def test_attention_transposed_operands(rock, oracle, gpu, tQ, tK, tV, tO):
+    got, ref = _run(rock, oracle, gpu, "f16", 2, 72, 96, 64, 64, 0.125, 43, bool(tQ), bool(tK), bool(tV), bool(tO))
+    check_float(got, ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
+
+
+def test_attention_odd_head_dims_take_generic_kernel(rock, oracle, gpu):
+    got, ref = _run(rock, oracle, gpu, "f16", 2, 50, 70, 20, 12, 0.3, 44)
+    check_float(got, ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
+
+
+def test_attention_with_bias(rock, oracle, gpu):
+    # cross attention with scale and bias: seq_q 128, seq_k 27, d_qk 64, d_v 32
+    got, ref = _run(rock, oracle, gpu, "f16", 2, 128, 27, 64, 32, 0.125, 45, bias=True)
+    check_float(got, ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
+
+
+def test_attention_rows_of_p_sum_to_one(rock, oracle, gpu):
+    # V = ones -> O = ones exactly up to the final rounding (size-independent property)
+    got, ref = _run(rock, oracle, gpu, "f16", 2, 200, 520, 128, 128, 0.0884, 46, vones=True)
+    assert np.abs(got - 1.0).max() <= 2e-3
+
+
+def test_attention_large_scores_do_not_overflow(rock, oracle, gpu):
+    # scale 4 pushes scores to ~ +-150: exp must stay finite through the running max
+    got, ref = _run(rock, oracle, gpu, "f16", 1, 64, 256, 64, 64, 4.0, 47)
+    check_float(got, ref, "f16", rms=2e-3, max_abs=0.03)

@@ -1,0 +1,137 @@
+"""GPU parity: forward convolution through the C ABI vs the CPU oracle and the
+reference's own golden vectors."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import CODE, check_float, quantise, to_f32, to_gpu
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def _to_layout(t, canonical, layout):
+    perm = [canonical.index(ch) for ch in layout]
+    return np.ascontiguousarray(t.transpose(perm)).ravel()
+
+
+def _run(rock, oracle, gpu, t, n, g, c, k, hi, wi, y, x, stride, pad, dil, layouts, integer, seed,
+         out_dtype=None, **epi):
+    fl, il, ol = layouts
+    rng = np.random.default_rng(seed)
+    if t == "i8":
+        fil = rng.integers(-128, 128, (g, k, c, y, x)).astype(np.float32)
+        inp = rng.integers(-128, 128, (n, g, c, hi, wi)).astype(np.float32)
+    elif integer:
+        fil = rng.integers(-2, 3, (g, k, c, y, x)).astype(np.float32)
+        inp = rng.integers(-2, 3, (n, g, c, hi, wi)).astype(np.float32)
+    else:
+        fil = (rng.standard_normal((g, k, c, y, x)) * 0.1).astype(np.float32)
+        inp = (rng.standard_normal((n, g, c, hi, wi)) * 0.1).astype(np.float32)
+    raw_f, fq = quantise(_to_layout(fil, "gkcyx", fl), t)
+    raw_i, iq = quantise(_to_layout(inp, "ngchw", il), t)
+    out = rock.conv2d(to_gpu(raw_f, t, gpu), to_gpu(raw_i, t, gpu), fil_layout=fl, in_layout=il,
+                      out_layout=ol, batchsize=n, in_channels=g * c, out_channels=g * k, in_h=hi,
+                      in_w=wi, fil_h=y, fil_w=x, groupsize=g, stride=stride, padding=pad, dilation=dil,
+                      out_dtype=out_dtype, **epi)
+    torch.cuda.synchronize()
+    if t == "i8":
+        ref, ho, wo = oracle.conv_fwd(raw_f, raw_i, fl, il, ol, n, g, c, k, hi, wi, y, x, stride, pad, dil)
+    else:
+        ref, ho, wo = oracle.conv_fwd(fq, iq, fl, il, ol, n, g, c, k, hi, wi, y, x, stride, pad, dil)
+    od = out_dtype or {"i8": "i32", "fp8": "f32", "bf8": "f32"}.get(t, t)
+    assert out.numel() == ref.size
+    return out, od, ref
+
+
+def _golden():
+    with open(os.path.join(HERE, "golden", "conv_fwd_kats.json")) as f:
+        return json.load(f)
+
+
+@pytest.mark.parametrize("case", _golden(), ids=lambda c: c["source"])
+@pytest.mark.parametrize("t", ["f32", "f16", "i8"])
+def test_conv_reference_golden_vectors(rock, gpu, case, t):
+    """cpu_conv2d/*_fwd.mlir: all-ones data, the literal vector FileCheck expects."""
+    f = case["flags"]
+    n, c, k = int(f["batchsize"]), int(f["in_channels"]), int(f["out_channels"])
+    hi, wi, y, x = int(f["in_h"]), int(f["in_w"]), int(f["fil_h"]), int(f["fil_w"])
+    dt = {"f32": torch.float32, "f16": torch.float16, "i8": torch.int8}[t]
+    fil = torch.ones(k * c * y * x, dtype=dt, device=gpu)
+    inp = torch.ones(n * c * hi * wi, dtype=dt, device=gpu)
+    out = rock.conv2d(fil, inp, fil_layout=f["fil_layout"], in_layout=f["in_layout"],
+                      out_layout=f["out_layout"], batchsize=n, in_channels=c, out_channels=k,
+                      in_h=hi, in_w=wi, fil_h=y, fil_w=x,
+                      stride=(int(f["conv_stride_h"]), int(f["conv_stride_w"])),
+                      padding=(int(f["padding_h"]), int(f["padding_w"])),
+                      dilation=(int(f["dilation_h"]), int(f["dilation_w"])))
+    assert out.cpu().double().tolist() == case["expected"]
+
+
+NHWC = ("gkyxc", "nhwgc", "nhwgk")
+NCHW = ("gkcyx", "ngchw", "ngkhw")
+# (n g c k hi wi y x stride pad dil): PaddedGemmConfig.toml:23-48 and
+# conv_regression_fwd.toml:23-227 shapes, batch trimmed
+EDGE_CASES = [
+    (2, 1, 7, 64, 11, 11, 3, 3, (2, 2), (1, 1), (1, 1)),
+    (19, 1, 8, 16, 7, 7, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (2, 1, 13, 11, 7, 7, 3, 3, (1, 1), (0, 0), (1, 1)),
+    (1, 1, 15, 8, 5, 5, 3, 3, (2, 2), (1, 1), (1, 1)),
+    (1, 1, 3, 64, 56, 56, 7, 7, (2, 2), (3, 3), (1, 1)),
+    (2, 1, 3, 6, 32, 32, 7, 7, (1, 1), (0, 0), (1, 1)),
+    (2, 1, 8, 8, 16, 64, 5, 5, (2, 3), (2, 2), (1, 2)),
+    (1, 1, 16, 16, 14, 14, 14, 14, (1, 1), (1, 1), (1, 1)),
+    (3, 1, 8, 8, 4, 4, 1, 1, (3, 3), (1, 1), (2, 2)),
+    (2, 4, 64, 64, 7, 7, 1, 1, (1, 1), (0, 0), (1, 1)),
+    (2, 2, 16, 24, 9, 9, 3, 3, (1, 1), (1, 1), (1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", EDGE_CASES)
+@pytest.mark.parametrize("layouts", [NHWC, NCHW], ids=["nhwc", "nchw"])
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16", "i8"])
+def test_conv_edge_shapes_exact(rock, oracle, gpu, case, layouts, t):
+    out, od, ref = _run(rock, oracle, gpu, t, *case, layouts, True, 31)
+    if t == "i8":
+        assert oracle.verify_int(out.cpu().numpy().ravel(), ref)[0] == 0
+    else:
+        assert np.array_equal(to_f32(out, od), ref)
+
+
+MIXED = [(f, i, o) for f in ("gkcyx", "gkyxc", "gyxck") for i, o in
+         (("ngchw", "ngkhw"), ("nhwgc", "nhwgk"), ("hwcgn", "hwkgn"), ("nhwgc", "ngkhw"))]
+
+
+@pytest.mark.parametrize("layouts", MIXED, ids=lambda l: "-".join(l))
+def test_conv_mixed_layouts(rock, oracle, gpu, layouts):
+    # MixedConvLayouts.toml:14-36: N=32, C=2, K=4, 2x2 image, 2x2 filter, p1
+    out, od, ref = _run(rock, oracle, gpu, "f32", 32, 1, 2, 4, 2, 2, 2, 2, (1, 1), (1, 1), (1, 1),
+                        layouts, True, 33)
+    assert np.array_equal(to_f32(out, od), ref)
+
+
+@pytest.mark.parametrize("t", ["f16", "bf16", "f32", "fp8"])
+def test_conv_resnet_block_real_values(rock, oracle, gpu, t):
+    """ResNet50 3x3 128->128 @28x28 (conv-configs:5), batch 4: the vector-load
+    implicit-GEMM kernel with real-valued data, reference RMS gate."""
+    out, od, ref = _run(rock, oracle, gpu, t, 4, 1, 128, 128, 28, 28, 3, 3, (1, 1), (1, 1), (1, 1),
+                        NHWC, False, 35)
+    check_float(to_f32(out, od), ref, od)
+
+
+@pytest.mark.parametrize("tile", ["256,128", "128,128", "64,64"])
+def test_conv_every_fast_tile(rock, oracle, gpu, tile):
+    out, od, ref = _run(rock, oracle, gpu, "f16", 3, 2, 32, 48, 13, 11, 3, 3, (1, 2), (1, 0), (2, 1),
+                        NHWC, True, 37, perf_config="v2:%s,8,64,16,8,1,1,1" % tile)
+    assert np.array_equal(to_f32(out, od), ref)
+
+
+def test_conv_i8_dequantise_per_tensor(rock, oracle, gpu):
+    # int8 conv 3x3 s2 p1 -> dequantize (mixr-resnet-fusion-case-1-quantization.mlir chain)
+    out, od, ref = _run(rock, oracle, gpu, "i8", 2, 1, 16, 32, 14, 14, 3, 3, (2, 2), (1, 1), (1, 1),
+                        NHWC, True, 39, out_dtype="f16", scale=1.2207e-4)
+    want = oracle.round_through(oracle.dequantize(ref, 1.2207e-4, 0), CODE["f16"])
+    assert np.array_equal(to_f32(out, "f16"), want)

@@ -1,0 +1,303 @@
+"""Pins the oracle's GEMM / convolution / attention / epilogue / verifier
+restatements: the reference's own golden vectors, closed forms, library
+routines (numpy float64 matmul, torch conv2d, torch softmax) and invariants."""
+import ctypes
+import itertools
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+# ----------------------------------------------------------------- GEMM
+def _store(mat, trans):
+    """logical [G,R,C] -> storage order of the reference ([G,C,R] if trans)."""
+    return np.ascontiguousarray(mat.transpose(0, 2, 1) if trans else mat)
+
+
+@pytest.mark.parametrize("tA,tB,tC", list(itertools.product([0, 1], repeat=3)))
+def test_gemm_f32_all_transposes_vs_float64(oracle, tA, tB, tC):
+    rng = np.random.default_rng(10 + 4 * tA + 2 * tB + tC)
+    G, M, N, K = 3, 7, 5, 11
+    A = rng.uniform(-1, 1, (G, M, K)).astype(np.float32)
+    B = rng.uniform(-1, 1, (G, K, N)).astype(np.float32)
+    got = oracle.gemm(_store(A, tA), _store(B, tB), G, M, N, K, tA, tB, tC)
+    want = np.matmul(A.astype(np.float64), B.astype(np.float64))
+    want = _store(want, tC).ravel()
+    assert np.allclose(got, want, rtol=0, atol=2e-6)
+    # a transposed operand or a wrong index breaks this by O(1)
+
+
+def test_gemm_reduction_order_is_k_ascending_mul_then_add(oracle):
+    # values chosen so that any other association or an fma changes the result
+    a = np.array([[1e8, 1.0, -1e8, 1.0]], np.float32)
+    b = np.ones((4, 1), np.float32)
+    got = oracle.gemm(a, b, 1, 1, 1, 4)
+    acc = np.float32(0)
+    for k in range(4):
+        acc = np.float32(np.float32(a[0, k] * b[k, 0]) + acc)
+    assert got[0] == acc == 1.0
+    x = np.float32(1 + 2 ** -12)
+    got = oracle.gemm(np.array([[x, 1.0]], np.float32), np.array([[x], [-1.0]], np.float32), 1, 1, 1, 2)
+    assert got[0] == np.float32(np.float32(x * x) - np.float32(1.0))  # no fma
+
+
+def test_gemm_fixed_pattern_closed_form(oracle):
+    # the reference's "-rand fixed" data: {0.5,-1,0.75} cycled by flat index
+    M = N = K = 6
+    A = oracle.fill_fixed(M * K).reshape(M, K)
+    B = oracle.fill_fixed(K * N).reshape(K, N)
+    assert A.ravel()[:4].tolist() == [0.5, -1.0, 0.75, 0.5]
+    got = oracle.gemm(A, B, 1, M, N, K).reshape(M, N)
+    # K=6 is a multiple of 3, so every row of A is the pattern twice and every
+    # column of B is constant: column j of B holds pat[j % 3]
+    pat = np.array([0.5, -1.0, 0.75])
+    for j in range(N):
+        assert np.allclose(got[:, j], 2 * pat.sum() * pat[j % 3])
+
+
+def test_gemm_i8_exact_and_widened(oracle):
+    rng = np.random.default_rng(11)
+    G, M, N, K = 2, 9, 8, 300
+    A = rng.integers(-128, 128, (G, M, K), dtype=np.int8)
+    B = rng.integers(-128, 128, (G, N, K), dtype=np.int8)  # stored [G,N,K]: transB
+    got = oracle.gemm(A, B, G, M, N, K, transB=True).reshape(G, M, N)
+    want = np.einsum("gmk,gnk->gmn", A.astype(np.int64), B.astype(np.int64))
+    assert np.array_equal(got, want)
+    # -128 * -128 = 16384 does not fit in i8: proves operands are widened first
+    one = oracle.gemm(np.array([[-128]], np.int8), np.array([[-128]], np.int8), 1, 1, 1, 1)
+    assert one[0] == 16384
+
+
+def test_gemm_all_ones_quant_case(oracle):
+    # mixr-gemm-reshape-case1-quant.e2e.mlir:6 -- all-ones 5x4 . 4x3 int8 -> fifteen 4s
+    got = oracle.gemm(np.ones((5, 4), np.int8), np.ones((4, 3), np.int8), 1, 5, 3, 4)
+    assert got.tolist() == [4] * 15
+
+
+def test_gemm_row_sample(oracle):
+    rng = np.random.default_rng(12)
+    A = rng.standard_normal((16, 8)).astype(np.float32)
+    B = rng.standard_normal((8, 4)).astype(np.float32)
+    full = oracle.gemm(A, B, 1, 16, 4, 8).reshape(16, 4)
+    part = oracle.gemm(A, B, 1, 16, 4, 8, rows=(5, 9), threads=2).reshape(16, 4)
+    assert np.array_equal(part[5:9], full[5:9]) and not part[:5].any() and not part[9:].any()
+
+
+# ----------------------------------------------------------------- convolution
+def _golden_cases():
+    with open(os.path.join(HERE, "golden", "conv_fwd_kats.json")) as f:
+        return json.load(f)
+
+
+@pytest.mark.parametrize("case", _golden_cases(), ids=lambda c: c["source"])
+@pytest.mark.parametrize("dtype", ["f32", "i8"])
+def test_conv_reference_golden_vectors(oracle, case, dtype):
+    """mlir/test/rocmlir-driver/cpu_conv2d/*_fwd.mlir: all-ones data (-rand
+    none), literal expected output."""
+    f = case["flags"]
+    n, c, k = int(f["batchsize"]), int(f["in_channels"]), int(f["out_channels"])
+    hi, wi, y, x = int(f["in_h"]), int(f["in_w"]), int(f["fil_h"]), int(f["fil_w"])
+    lay = {"kyxc": "gkyxc", "kcyx": "gkcyx", "nhwc": "nhwgc", "nchw": "ngchw",
+           "nhwk": "nhwgk", "nkhw": "ngkhw"}
+    np_t = np.int8 if dtype == "i8" else np.float32
+    fil = np.ones(k * c * y * x, np_t)
+    inp = np.ones(n * c * hi * wi, np_t)
+    out, ho, wo = oracle.conv_fwd(
+        fil, inp, lay[f["fil_layout"]], lay[f["in_layout"]], lay[f["out_layout"]],
+        n, 1, c, k, hi, wi, y, x,
+        stride=(int(f["conv_stride_h"]), int(f["conv_stride_w"])),
+        pad=(int(f["padding_h"]), int(f["padding_w"])),
+        dil=(int(f["dilation_h"]), int(f["dilation_w"])))
+    assert out.size == len(case["expected"])
+    assert np.array_equal(out.astype(np.float64), np.array(case["expected"]))
+
+
+def _to_layout(t, canonical, layout):
+    """tensor with axes in `canonical` letter order -> flat array in `layout` order"""
+    perm = [canonical.index(ch) for ch in layout]
+    return np.ascontiguousarray(t.transpose(perm)).ravel()
+
+
+CONV_CASES = [
+    # n g c k hi wi y x stride pad dil
+    (2, 1, 3, 4, 9, 7, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (1, 2, 4, 6, 8, 8, 3, 2, (2, 1), (0, 1), (1, 2)),
+    (3, 4, 2, 2, 5, 6, 1, 1, (1, 1), (0, 0), (1, 1)),
+    (1, 1, 5, 3, 11, 11, 5, 5, (2, 3), (2, 2), (1, 1)),
+    (2, 1, 3, 2, 4, 4, 2, 2, (1, 1), (1, 1), (2, 2)),
+    (1, 1, 2, 3, 14, 14, 14, 14, (1, 1), (1, 1), (1, 1)),
+]
+LAYOUTS = [("gkcyx", "ngchw", "ngkhw"), ("gkyxc", "nhwgc", "nhwgk"), ("gyxck", "hwcgn", "hwkgn"),
+           ("gkcyx", "nhwgc", "ngkhw")]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+@pytest.mark.parametrize("layouts", LAYOUTS)
+def test_conv_vs_torch_conv2d(oracle, case, layouts):
+    n, g, c, k, hi, wi, y, x, stride, pad, dil = case
+    rng = np.random.default_rng(hash((case, layouts)) % 2 ** 31)
+    fil = rng.integers(-3, 4, (g, k, c, y, x)).astype(np.float32)   # exact in f32
+    inp = rng.integers(-3, 4, (n, g, c, hi, wi)).astype(np.float32)
+    fl, il, ol = layouts
+    out, ho, wo = oracle.conv_fwd(_to_layout(fil, "gkcyx", fl), _to_layout(inp, "ngchw", il),
+                                  fl, il, ol, n, g, c, k, hi, wi, y, x, stride, pad, dil)
+    ref = torch.nn.functional.conv2d(
+        torch.from_numpy(inp.reshape(n, g * c, hi, wi)).double(),
+        torch.from_numpy(fil.reshape(g * k, c, y, x)).double(),
+        stride=stride, padding=pad, dilation=dil, groups=g).numpy()
+    assert ref.shape == (n, g * k, ho, wo)
+    want = _to_layout(ref.reshape(n, g, k, ho, wo), "ngkhw", ol)
+    assert np.array_equal(out.astype(np.float64), want)
+    # int8 path on the same integers
+    out8, _, _ = oracle.conv_fwd(_to_layout(fil, "gkcyx", fl).astype(np.int8),
+                                 _to_layout(inp, "ngchw", il).astype(np.int8),
+                                 fl, il, ol, n, g, c, k, hi, wi, y, x, stride, pad, dil)
+    assert np.array_equal(out8.astype(np.float64), want)
+
+
+def test_conv_i8_widens_before_multiply(oracle):
+    # deliberate deviation from rocmlir-gen.cpp:1955-1960 (i8 multiply wraps)
+    out, _, _ = oracle.conv_fwd(np.array([-128], np.int8), np.array([-128], np.int8),
+                                "gkcyx", "ngchw", "ngkhw", 1, 1, 1, 1, 1, 1, 1, 1)
+    assert out[0] == 16384
+
+
+def test_conv_output_range_sample(oracle):
+    rng = np.random.default_rng(5)
+    fil = rng.standard_normal(4 * 3 * 3 * 3).astype(np.float32)
+    inp = rng.standard_normal(2 * 3 * 6 * 6).astype(np.float32)
+    full, _, _ = oracle.conv_fwd(fil, inp, "gkyxc", "nhwgc", "nhwgk", 2, 1, 3, 4, 6, 6, 3, 3, pad=(1, 1))
+    part, _, _ = oracle.conv_fwd(fil, inp, "gkyxc", "nhwgc", "nhwgk", 2, 1, 3, 4, 6, 6, 3, 3, pad=(1, 1),
+                                 out_range=(10, 50), threads=3)
+    assert np.array_equal(part[10:50], full[10:50]) and not part[:10].any() and not part[50:].any()
+
+
+# ----------------------------------------------------------------- attention
+def test_softmax_reference_vector(oracle):
+    # migraphx_softmax.cpu.e2e.mlir:8-9
+    got = oracle.softmax(np.array([[0, 2, 3, 1]], np.float32))[0]
+    assert np.allclose(got, [0.0320586, 0.236883, 0.643914, 0.0871443], rtol=1e-5)
+
+
+def _attn_ref64(Q, K, V, scale, bias=None):
+    S = np.einsum("gid,gjd->gij", Q.astype(np.float64), K.astype(np.float64)) * scale
+    if bias is not None:
+        S = S + bias
+    P = torch.softmax(torch.from_numpy(S), dim=-1).numpy()
+    return np.einsum("gij,gje->gie", P, V.astype(np.float64))
+
+
+@pytest.mark.parametrize("tQ,tK,tV,tO", [(0, 0, 0, 0), (0, 1, 0, 0), (1, 1, 1, 1), (1, 0, 1, 0), (0, 1, 1, 1)])
+def test_attention_vs_float64_all_layouts(oracle, tQ, tK, tV, tO):
+    rng = np.random.default_rng(20 + tQ + 2 * tK + 4 * tV + 8 * tO)
+    G, sq, sk, dqk, dv = 2, 9, 27, 8, 5
+    Q = rng.standard_normal((G, sq, dqk)).astype(np.float32)
+    K = rng.standard_normal((G, sk, dqk)).astype(np.float32)   # logical [G,sk,d]
+    V = rng.standard_normal((G, sk, dv)).astype(np.float32)
+    bias = rng.standard_normal((G, sq, sk)).astype(np.float32)
+    scale = 0.37
+    # storage: K is [G,d,sk] by default, [G,sk,d] with transK
+    got = oracle.attention(_store(Q, tQ), _store(K, not tK), _store(V, tV), G, sq, sk, dqk, dv,
+                           scale=scale, bias_t=bias, transQ=tQ, transK=tK, transV=tV, transO=tO)
+    want = _store(_attn_ref64(Q, K, V, scale, bias), tO).ravel()
+    assert np.allclose(got, want, rtol=0, atol=3e-6)
+
+
+def test_attention_invariants(oracle):
+    rng = np.random.default_rng(21)
+    G, sq, sk, d, dv = 1, 4, 16, 8, 6
+    Q = rng.standard_normal((G, sq, d)).astype(np.float32)
+    K = rng.standard_normal((G, sk, d)).astype(np.float32)
+    V = rng.standard_normal((G, sk, dv)).astype(np.float32)
+    att = lambda q, k, v, **kw: oracle.attention(q, k, v, G, sq, sk, d, dv, transK=True, **kw).reshape(G, sq, dv)
+    # rows of P sum to one
+    assert np.allclose(att(Q, K, np.ones_like(V)), 1.0, atol=1e-6)
+    # Q = 0 -> uniform weights -> column mean of V
+    assert np.allclose(att(np.zeros_like(Q), K, V), V.mean(axis=1, keepdims=True), atol=1e-6)
+    # permuting keys and values together changes nothing (up to summation order)
+    perm = rng.permutation(sk)
+    assert np.allclose(att(Q, K, V), att(Q, K[:, perm], V[:, perm]), atol=1e-6)
+    # scale tensor of constant s == scalar scale s
+    st = np.full((G, sq, sk), 0.25, np.float32)
+    assert np.array_equal(att(Q, K, V, scale_t=st), att(Q, K, V, scale=0.25))
+    # query-row sample
+    part = oracle.attention(Q, K, V, G, sq, sk, d, dv, transK=True, q_rows=(1, 3)).reshape(G, sq, dv)
+    assert np.array_equal(part[:, 1:3], att(Q, K, V)[:, 1:3]) and not part[:, 0].any()
+
+
+# ----------------------------------------------------------------- epilogue
+def test_dequantize_formula(oracle):
+    # (float(acc) - float(zp)) * scale, MIGraphXToTosa.cpp:874-902
+    acc = np.array([0, 1, -7, 100, 2 ** 26 + 3, -(2 ** 26) - 5], np.int64)
+    got = oracle.dequantize(acc, 0.01, 3)
+    want = (acc.astype(np.int32).astype(np.float32) - np.float32(3)) * np.float32(0.01)
+    assert np.array_equal(got, want)
+    assert got[1] == np.float32(-0.02)
+    # 2^26+3 is not representable in f32: the int->float conversion rounds to even
+    assert oracle.dequantize(np.array([2 ** 26 + 3], np.int64), 1.0)[0] == np.float32(2 ** 26 + 4)
+
+
+def test_quantize_formula(oracle):
+    # clamp(round_even(x * (1/scale)) + zp, -128, 127), MIGraphXToTosa.cpp:904-982
+    x = np.array([0.0, 0.25, 0.75, 1.25, -0.25, -0.75, 100.0, -100.0, 63.4], np.float32)
+    got = oracle.quantize_i8(x, 0.5, 1)
+    assert got.tolist() == [1, 1, 3, 3, 1, -1, 127, -128, 127]
+    assert oracle.quantize_i8(np.array([63.4], np.float32), 0.5, 0)[0] == 127
+    assert oracle.quantize_i8(np.array([63.2], np.float32), 0.5, 0)[0] == 126
+
+
+def test_scale_bias(oracle):
+    x = np.arange(6, dtype=np.float32).reshape(2, 3)
+    got = oracle.scale_bias(x, 2, 3, 0.5, np.array([1, 2, 3], np.float32))
+    assert np.array_equal(got, x * 0.5 + np.array([1, 2, 3], np.float32))
+
+
+# ----------------------------------------------------------------- verifier / fill
+def test_verify_float_metrics_by_hand(oracle):
+    val = np.array([1.0, 2.0, 0.0, -4.0], np.float32)
+    gpu = np.array([1.0, 2.5, 0.5, -4.0], np.float32)
+    r = oracle.verify_float(gpu, val, thr_rms=1.0, thr_abs=1.0, thr_rel=1.0)
+    # RMS = sqrt(0.25 + 0.25) / (maxMag=4 * sqrt(4))   (conv-validation-wrappers.cpp:199-200)
+    assert r.rms == pytest.approx(np.sqrt(0.5) / 8.0)
+    assert r.max_abs_diff == 0.5
+    assert r.max_rel_diff == 0.25           # val == 0 is excluded from relDiff
+    assert r.ave_abs_diff == 0.25
+    assert r.passed()
+    r = oracle.verify_float(gpu, val, thr_rms=0.01, thr_abs=1.0, thr_rel=0.1)
+    assert (r.pass_rms, r.pass_abs, r.pass_rel) == (0, 1, 0)
+
+
+def test_verify_float_inf_reference_is_fp16_max(oracle):
+    r = oracle.verify_float(np.array([65504.0], np.float32), np.array([np.inf], np.float32))
+    assert r.max_abs_diff == 0.0 and r.pass_abs
+
+
+def test_verify_int(oracle):
+    gpu = np.array([1, 2, -5, 7], np.int32)
+    val = np.array([1, 3, -5, 2 ** 31 + 7], np.int64)
+    fails, ovf, mad = oracle.verify_int(gpu, val)
+    assert (fails, ovf, mad) == (2, 1, 2 ** 31)
+    assert oracle.verify_int(gpu, gpu.astype(np.int64)) == (0, 0, 0)
+
+
+def test_fill_rand_follows_libc_rand(oracle):
+    libc = ctypes.CDLL(None)
+    libc.rand.restype = ctypes.c_int
+    oracle.seed(7)
+    ints = oracle.fill_rand(20, -5, 5, as_float=False)
+    libc.srand(7)
+    want = [float((libc.rand() % 10) - 5) for _ in range(20)]
+    assert ints.tolist() == want and ints.min() >= -5 and ints.max() < 5
+    oracle.seed(7)
+    fl = oracle.fill_rand(20, -1, 1, as_float=True)
+    libc.srand(7)
+    want = [np.float32(np.float32(2 * float(libc.rand()) / 2147483647.0) + np.float32(-1)) for _ in range(20)]
+    assert fl.tolist() == [float(w) for w in want]
+    assert oracle.fill_fixed(5, is_int=True).tolist() == [1, -1, 2, 1, -1]
+    # min == max: constant (0.1x for floats), conv-validation-wrappers.cpp:41-45
+    assert oracle.fill_rand(3, 1, 1, as_float=True).tolist() == [np.float32(0.1)] * 3
