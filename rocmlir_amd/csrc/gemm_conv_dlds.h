@@ -1,0 +1,296 @@
+// Fast path of the contraction kernel: operands stream global -> LDS without
+// passing through registers (buffer_load ... lds, 16 bytes per lane), four LDS
+// stages, so three K-steps of loads are in flight while one is multiplied.
+//
+// Same tiling and MFMA mapping as the register-staged body in
+// gemm_conv_kernel.h (which remains for arbitrary strides); what differs:
+//
+//   * K advances 64 BYTES per stage; a stage holds BM + BN rows of four
+//     16-byte chunks.  One wave-wide load instruction fills a "slab" of 16
+//     rows (1 KiB, the 64 lanes' 16 bytes land back to back in LDS).
+//   * The XOR swizzle is applied on the source side: the lane that fills
+//     physical chunk p of row r fetches logical chunk p ^ ((r >> 2) & 3), so
+//     the 32 rows an MFMA operand reads at one chunk index fall into distinct
+//     bank groups.
+//   * Zero fill (rows past the end, the K tail, convolution padding) costs no
+//     instruction: such lanes use a byte offset beyond the buffer
+//     descriptor's range and the hardware writes zeros.  This is the
+//     reference's own trick for padded loads
+//     (mlir/lib/Dialect/Rock/Transforms/SugarToLoops.cpp:1162-1267).
+//   * Synchronisation is explicit: the loads are counted with vmcnt, every
+//     iteration waits until at most two younger K-steps are outstanding,
+//     crosses ONE workgroup barrier, refills the stage that was consumed in
+//     the previous iteration, then multiplies.
+//
+// Limits checked on the host before this path is chosen: every in-range byte
+// offset relative to the block's base pointer is below 2^31.
+#pragma once
+#include "gemm_conv_kernel.h"
+
+namespace rk {
+
+constexpr int kDlRowBytes = 64;  // K bytes per row per stage
+constexpr int kDlChunks = 4;     // 16-byte chunks per row
+constexpr int kDlStages = 4;
+constexpr unsigned kOobOffset = 0x80000000u; // >= num_records: reads as zero
+
+typedef __attribute__((address_space(3))) void lds_void_t;
+
+__device__ __forceinline__ int dl_swz(int row) { return (row >> 2) & 3; }
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t dl_rsrc(const void *base) {
+  // raw buffer, 2 GiB window, dword-typed data format word used by gfx9 parts
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)kOobOffset, 0x00020000);
+}
+
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  // gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x0F70);
+}
+
+template <int ROWS, int NW> struct SlabGeom {
+  static constexpr int SLABS = ROWS / 16;
+  static constexpr int PER_WAVE = SLABS / NW;
+  static_assert(ROWS % 16 == 0 && SLABS % NW == 0, "tile rows must split into 16-row slabs per wave");
+};
+
+// K-contiguous rows (GEMM operands, KYXC filters).
+template <int DT, int ROWS, int NW> struct RowsDl {
+  using Sg = SlabGeom<ROWS, NW>;
+  static constexpr int ES = MmaTraits<DT>::ES;
+  __amdgpu_buffer_rsrc_t rsrc;
+  unsigned off[Sg::PER_WAVE]; // byte offset of this lane's chunk at K-step 0, or kOobOffset
+  int kb[Sg::PER_WAVE];       // byte offset of the chunk inside the 64-byte K-step
+  int kbytes;
+  int wave;
+
+  __device__ __forceinline__ void init(const void *base, int64_t row_stride, int row0, int rows_total,
+                                       int K, int wave_, int lane) {
+    wave = wave_;
+    kbytes = K * ES;
+    rsrc = dl_rsrc((const char *)base + (int64_t)row0 * row_stride * ES);
+#pragma unroll
+    for (int i = 0; i < Sg::PER_WAVE; ++i) {
+      int r = (wave * Sg::PER_WAVE + i) * 16 + (lane >> 2);
+      kb[i] = ((lane & 3) ^ dl_swz(r)) * kChunk;
+      off[i] = (row0 + r < rows_total) ? (unsigned)(r * (int)row_stride * ES + kb[i]) : kOobOffset;
+    }
+  }
+  __device__ __forceinline__ void issue(int kt, char *stage) {
+#pragma unroll
+    for (int i = 0; i < Sg::PER_WAVE; ++i) {
+      int k0 = kt * kDlRowBytes;
+      unsigned voff = (k0 + kb[i] < kbytes) ? off[i] + (unsigned)k0 : kOobOffset;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrc, (lds_void_t *)(stage + (wave * Sg::PER_WAVE + i) * 1024), 16, (int)voff, 0, 0, 0);
+    }
+  }
+};
+
+// Convolution input as implicit-GEMM rows: row m = (n, ho, wo), reduction
+// index (y, x, c) with c fastest; channel run is a whole number of chunks.
+template <int DT, int ROWS, int NW> struct ConvInDl {
+  using Sg = SlabGeom<ROWS, NW>;
+  static constexpr int ES = MmaTraits<DT>::ES;
+  static constexpr int EPC = kChunk / ES;
+  static constexpr int BKE = kDlRowBytes / ES;
+  __amdgpu_buffer_rsrc_t rsrc;
+  const RockConvParams *p;
+  unsigned pix[Sg::PER_WAVE]; // byte offset of input(n, g, 0, 0, 0), or kOobOffset for rows past M
+  int h0[Sg::PER_WAVE], w0[Sg::PER_WAVE];
+  int y[Sg::PER_WAVE], x[Sg::PER_WAVE], cc[Sg::PER_WAVE];
+  int wave;
+
+  __device__ __forceinline__ void init(const void *in, const RockConvParams &cp, int g, int row0,
+                                       int wave_, int lane) {
+    p = &cp;
+    wave = wave_;
+    rsrc = dl_rsrc((const char *)in + (int64_t)g * cp.in_gs * ES);
+#pragma unroll
+    for (int i = 0; i < Sg::PER_WAVE; ++i) {
+      int r = (wave * Sg::PER_WAVE + i) * 16 + (lane >> 2);
+      int m = row0 + r;
+      int mm = min(m, cp.M - 1);
+      int n = mm / (cp.ho * cp.wo);
+      int rem = mm - n * (cp.ho * cp.wo);
+      int ho = rem / cp.wo;
+      int wo = rem - ho * cp.wo;
+      h0[i] = ho * cp.stride_h - cp.pad_h;
+      w0[i] = wo * cp.stride_w - cp.pad_w;
+      pix[i] = (m < cp.M) ? (unsigned)(n * (int)cp.in_ns * ES) : kOobOffset;
+      int k0 = ((lane & 3) ^ dl_swz(r)) * EPC;
+      int tap = k0 / cp.c;
+      cc[i] = k0 - tap * cp.c;
+      y[i] = tap / cp.x;
+      x[i] = tap - y[i] * cp.x;
+    }
+  }
+  // must be called with kt = 0, 1, 2, ... in order (tap state advances)
+  __device__ __forceinline__ void issue(int kt, char *stage) {
+    (void)kt;
+#pragma unroll
+    for (int i = 0; i < Sg::PER_WAVE; ++i) {
+      int hi = h0[i] + y[i] * p->dil_h, wi = w0[i] + x[i] * p->dil_w;
+      bool v = pix[i] != kOobOffset && y[i] < p->y && hi >= 0 && hi < p->hi && wi >= 0 && wi < p->wi;
+      unsigned voff = v ? pix[i] + (unsigned)((hi * (int)p->in_hs + wi * (int)p->in_ws + cc[i]) * ES)
+                        : kOobOffset;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrc, (lds_void_t *)(stage + (wave * Sg::PER_WAVE + i) * 1024), 16, (int)voff, 0, 0, 0);
+      cc[i] += BKE;
+      while (cc[i] >= p->c) {
+        cc[i] -= p->c;
+        if (++x[i] == p->x) { x[i] = 0; ++y[i]; }
+      }
+    }
+  }
+};
+
+template <int DT, int ROWS, int NW, int KIND>
+__device__ __forceinline__ auto make_dl_a(const void *A, const RockGemmParams &p, int g, int m0, int wave, int lane) {
+  static_assert(KIND == LD_ROWS_FAST, "GEMM fast path loads K-contiguous rows");
+  RowsDl<DT, ROWS, NW> l;
+  l.init((const char *)A + (int64_t)g * p.a_gs * MmaTraits<DT>::ES, p.a_ms, m0, p.M, p.K, wave, lane);
+  return l;
+}
+template <int DT, int ROWS, int NW, int KIND>
+__device__ __forceinline__ auto make_dl_b(const void *B, const RockGemmParams &p, int g, int n0, int wave, int lane) {
+  RowsDl<DT, ROWS, NW> l;
+  l.init((const char *)B + (int64_t)g * p.b_gs * MmaTraits<DT>::ES, p.b_ns, n0, p.N, p.K, wave, lane);
+  return l;
+}
+template <int DT, int ROWS, int NW, int KIND>
+__device__ __forceinline__ auto make_dl_a(const void *in, const RockConvParams &p, int g, int m0, int wave, int lane) {
+  static_assert(KIND == LD_CONV_IN_FAST, "convolution fast path gathers channel-contiguous input");
+  ConvInDl<DT, ROWS, NW> l;
+  l.init(in, p, g, m0, wave, lane);
+  return l;
+}
+template <int DT, int ROWS, int NW, int KIND>
+__device__ __forceinline__ auto make_dl_b(const void *fil, const RockConvParams &p, int g, int n0, int wave, int lane) {
+  RowsDl<DT, ROWS, NW> l;
+  l.init((const char *)fil + (int64_t)g * p.fil_gs * MmaTraits<DT>::ES, p.fil_ks, n0, p.N, p.K, wave, lane);
+  return l;
+}
+
+// Fragment of one 32-row block out of a 64-byte-row stage: lane (row = lane % 32,
+// half = lane / 32) takes chunk  step*2*CHUNKS + 2*c + half  for c in [0, CHUNKS).
+template <int DT>
+__device__ __forceinline__ Frag<DT> dl_read_frag(const char *lds, int row, int step, int half) {
+  Frag<DT> f;
+  constexpr int CH = MmaTraits<DT>::CHUNKS;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    int chunk = step * 2 * CH + 2 * c + half;
+    f.c[c] = *(const v4i *)(lds + row * kDlRowBytes + ((chunk ^ dl_swz(row)) * kChunk));
+  }
+  return f;
+}
+
+template <int DT, int BM, int BN, int WAVES_M, int WAVES_N, int LDA, int LDB, typename Params>
+__device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void *Bptr, void *Cptr,
+                                                    const void *aux, const Params &p) {
+  using Tr = MmaTraits<DT>;
+  using Acc = typename Tr::Acc;
+  constexpr int NW = WAVES_M * WAVES_N;
+  constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N; // wave tile
+  constexpr int MI = WTM / 32, NI = WTN / 32;
+  constexpr int STEPS = kDlChunks / (2 * Tr::CHUNKS); // MFMA K steps per stage
+  constexpr int A_BYTES = BM * kDlRowBytes, B_BYTES = BN * kDlRowBytes;
+  constexpr int STAGE = A_BYTES + B_BYTES;
+  constexpr int BKE = kDlRowBytes / Tr::ES;
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of 32");
+
+  __shared__ __attribute__((aligned(1024))) char lds[kDlStages * STAGE];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+  const int lrow = lane & 31, lgrp = lane >> 5;
+
+  int g, tm, tn;
+  decode_block(p.tiles_m, p.tiles_n, p_batch(p), p.group_m, p.xcd_remap, g, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  auto la = make_dl_a<DT, BM, NW, LDA>(Aptr, p, g, m0, wave, lane);
+  auto lb = make_dl_b<DT, BN, NW, LDB>(Bptr, p, g, n0, wave, lane);
+  constexpr int LOADS_PER_STEP = SlabGeom<BM, NW>::PER_WAVE + SlabGeom<BN, NW>::PER_WAVE;
+
+  Acc acc[MI][NI];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NI; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        acc[i][j][v] = 0;
+
+  const int nk = (p.K + BKE - 1) / BKE;
+
+  // K-steps past the end are issued all the same: every lane is then out of
+  // range, no memory is touched, and the outstanding-load count stays uniform.
+#pragma unroll
+  for (int s = 0; s < kDlStages - 1; ++s) {
+    la.issue(s, lds + s * STAGE);
+    lb.issue(s, lds + s * STAGE + A_BYTES);
+  }
+
+  for (int kt = 0; kt < nk; ++kt) {
+    // this wave's loads of K-step kt have landed (two younger steps may be in flight) ...
+    wait_vmcnt<(kDlStages - 2) * LOADS_PER_STEP>();
+    // ... and so have everyone else's; everyone is also done reading step kt-1
+    __builtin_amdgcn_s_barrier();
+    {
+      char *refill = lds + ((kt + kDlStages - 1) % kDlStages) * STAGE;
+      la.issue(kt + kDlStages - 1, refill);
+      lb.issue(kt + kDlStages - 1, refill + A_BYTES);
+    }
+    const char *sa = lds + (kt % kDlStages) * STAGE;
+    const char *sb = sa + A_BYTES;
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      Frag<DT> fb[NI];
+#pragma unroll
+      for (int j = 0; j < NI; ++j)
+        fb[j] = dl_read_frag<DT>(sb, wn * WTN + j * 32 + lrow, s, lgrp);
+#pragma unroll
+      for (int i = 0; i < MI; ++i) {
+        Frag<DT> fa = dl_read_frag<DT>(sa, wm * WTM + i * 32 + lrow, s, lgrp);
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+          mma32x32<DT>(fb[j], fa, acc[i][j]);
+      }
+    }
+  }
+  // drain the out-of-range loads issued for steps >= nk before the LDS is released
+  wait_vmcnt<0>();
+
+  // ---- epilogue: lane holds m = .. + lrow, n = .. + 8*q + 4*lgrp + {0..3}
+  const RockEpilogue &e = p.epi;
+  using Acc4 = decltype(__builtin_shufflevector(acc[0][0], acc[0][0], 0, 1, 2, 3));
+#pragma unroll
+  for (int i = 0; i < MI; ++i) {
+    const int m = m0 + wm * WTM + i * 32 + lrow;
+    if (m >= p.M)
+      continue;
+    int64_t row_off, n_stride;
+    bool vec_ok;
+    out_row_addr(p, g, m, Cptr, row_off, n_stride, vec_ok);
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + wn * WTN + j * 32 + q * 8 + lgrp * 4;
+        if (n >= p.N)
+          continue;
+        Acc4 a4 = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                   acc[i][j][4 * q + 3]};
+        epilogue_store4<Tr::INT_ACC>(a4, e, aux, Cptr, row_off + (int64_t)n * n_stride, n_stride,
+                                     n, p.N, vec_ok);
+      }
+    }
+  }
+}
+
+} // namespace rk

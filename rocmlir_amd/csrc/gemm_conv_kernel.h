@@ -83,35 +83,43 @@ template <int DT, int ROWS, int NT> struct TileGeom {
 };
 
 // K-contiguous rows: base + row * row_stride, chunk at byte kt*128 + c*16.
+// Rows past the end are clamped to the last row: they only feed accumulators
+// of outputs that are never stored.  The K tail must be zero; that fix-up is
+// deferred to just before the LDS store so that the wait for the global loads
+// does not sit in front of the MFMA section.
 template <int DT, int ROWS, int NT> struct RowsFast {
   using Gm = TileGeom<DT, ROWS, NT>;
   const char *ptr[Gm::NCH];
-  bool ok[Gm::NCH];
   int kbytes;
   int c;
+  bool kin;
 
   __device__ __forceinline__ void init(const void *base, int64_t row_stride,
                                        int row0, int rows_total, int K,
                                        int tid) {
     c = tid & 7;
     kbytes = K * Gm::ES;
+    kin = true;
 #pragma unroll
     for (int i = 0; i < Gm::NCH; ++i) {
       int r = (tid >> 3) + i * Gm::ROW_STEP;
-      int gr = row0 + r;
-      ok[i] = (r < ROWS) && (gr < rows_total);
-      int cr = min(gr, rows_total - 1);
+      int cr = min(row0 + r, rows_total - 1);
       ptr[i] = (const char *)base + (int64_t)cr * row_stride * Gm::ES;
     }
   }
-  __device__ __forceinline__ void load(int kt, v4i (&regs)[Gm::NCH]) const {
+  __device__ __forceinline__ void load(int kt, v4i (&regs)[Gm::NCH]) {
     int off = kt * kRowBytes + c * kChunk;
-    bool kin = off < kbytes; // kbytes is a multiple of 16 on this path
+    kin = off < kbytes; // kbytes is a multiple of 16 on this path
     int coff = kin ? off : 0;
 #pragma unroll
-    for (int i = 0; i < Gm::NCH; ++i) {
-      v4i v = *(const v4i *)(ptr[i] + coff);
-      regs[i] = (kin && ok[i]) ? v : v4i{0, 0, 0, 0};
+    for (int i = 0; i < Gm::NCH; ++i)
+      regs[i] = *(const v4i *)(ptr[i] + coff);
+  }
+  __device__ __forceinline__ void fixup(v4i (&regs)[Gm::NCH]) const {
+    if (!kin) {
+#pragma unroll
+      for (int i = 0; i < Gm::NCH; ++i)
+        regs[i] = v4i{0, 0, 0, 0};
     }
   }
 };
@@ -173,6 +181,7 @@ template <int DT, int ROWS, int NT> struct RowsGeneric {
       });
     }
   }
+  __device__ __forceinline__ void fixup(v4i (&)[Gm::NCH]) const {}
 };
 
 // Convolution input as the implicit-GEMM A operand: row m = (n, ho, wo),
@@ -186,6 +195,7 @@ template <int DT, int ROWS, int NT> struct ConvInFast {
   const RockConvParams *p;
   int y, x, cc; // tap and channel offset of this thread's chunk at tile kt
   int K;
+  uint32_t valid; // bit i: chunk i of the tile just loaded is inside the image
 
   __device__ __forceinline__ void init(const void *in, const RockConvParams &cp,
                                        int g, int row0, int tid) {
@@ -217,20 +227,28 @@ template <int DT, int ROWS, int NT> struct ConvInFast {
     const int k0 = kt * Gm::BKE + (threadIdx.x & 7) * Gm::EPC;
     const bool kin = k0 < K;
     const int dh = y * p->dil_h, dw = x * p->dil_w;
+    uint32_t vm = 0;
 #pragma unroll
     for (int i = 0; i < Gm::NCH; ++i) {
       int hi = h0[i] + dh, wi = w0[i] + dw;
       bool v = kin && ok[i] && hi >= 0 && hi < p->hi && wi >= 0 && wi < p->wi;
       int64_t off = v ? ((int64_t)hi * p->in_hs + (int64_t)wi * p->in_ws + cc) * Gm::ES : 0;
-      v4i d = *(const v4i *)(pix[i] + off);
-      regs[i] = v ? d : v4i{0, 0, 0, 0};
+      regs[i] = *(const v4i *)(pix[i] + off);
+      vm |= (v ? 1u : 0u) << i;
     }
+    valid = vm;
     // advance to the next tile's tap
     cc += Gm::BKE;
     while (cc >= p->c) {
       cc -= p->c;
       if (++x == p->x) { x = 0; ++y; }
     }
+  }
+  // padding taps and the K tail become zeros (applied right before the LDS store)
+  __device__ __forceinline__ void fixup(v4i (&regs)[Gm::NCH]) const {
+#pragma unroll
+    for (int i = 0; i < Gm::NCH; ++i)
+      regs[i] = ((valid >> i) & 1u) ? regs[i] : v4i{0, 0, 0, 0};
   }
 };
 
@@ -286,6 +304,7 @@ template <int DT, int ROWS, int NT> struct ConvInGeneric {
       });
     }
   }
+  __device__ __forceinline__ void fixup(v4i (&)[Gm::NCH]) const {}
 };
 
 template <int DT, int ROWS, int NT> struct ConvFilGeneric {
@@ -316,6 +335,7 @@ template <int DT, int ROWS, int NT> struct ConvFilGeneric {
       });
     }
   }
+  __device__ __forceinline__ void fixup(v4i (&)[Gm::NCH]) const {}
 };
 
 // ---------------------------------------------------------------------------
@@ -576,6 +596,8 @@ __device__ __forceinline__ void contraction_body(const void *Aptr, const void *B
 
   la.load(0, ra);
   lb.load(0, rb);
+  la.fixup(ra);
+  lb.fixup(rb);
   store_tile<DT, BM, NT>(lds, ra, tid);
   store_tile<DT, BN, NT>(lds + A_BYTES, rb, tid);
   __syncthreads();
@@ -605,6 +627,8 @@ __device__ __forceinline__ void contraction_body(const void *Aptr, const void *B
     }
     if (more) {
       char *da = lds + (cur ^ 1) * (A_BYTES + B_BYTES);
+      la.fixup(ra);
+      lb.fixup(rb);
       store_tile<DT, BM, NT>(da, ra, tid);
       store_tile<DT, BN, NT>(da + A_BYTES, rb, tid);
     }

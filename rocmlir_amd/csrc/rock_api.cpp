@@ -372,9 +372,14 @@ Handle *make_gemm(const OptMap &o) {
   p.c_gs = M * N; p.c_ms = tC ? 1 : N; p.c_ns = tC ? M : 1;
 
   const int es = dtype_size(ta);
+  // vector path: K-contiguous rows of whole 16-byte chunks, and every byte
+  // offset inside one block tile (256 rows at most) below 2^31 for the buffer
+  // descriptors of the direct-to-LDS loads
+  const int64_t kMaxOff = (int64_t)1 << 31;
   const bool fast = p.a_ks == 1 && p.b_ks == 1 && (p.a_ms * es) % 16 == 0 &&
                     (p.b_ns * es) % 16 == 0 && (K * es) % 16 == 0 && (p.a_gs * es) % 16 == 0 &&
-                    (p.b_gs * es) % 16 == 0;
+                    (p.b_gs * es) % 16 == 0 && 256 * p.a_ms * es + K * es < kMaxOff &&
+                    256 * p.b_ns * es + K * es < kMaxOff;
   const Tile *tile = fast ? pick_tile(M, N, (int)G, false, forced_tile(o)) : nullptr;
   if (!tile)
     tile = fast ? pick_tile(M, N, (int)G, false, "") : &kGenericTile;
@@ -574,7 +579,10 @@ Handle *make_conv(const OptMap &o) {
   auto al = [&](int64_t elems) { return (elems * es) % 16 == 0; };
   const bool fast = p.in_cs == 1 && al(c) && al(p.in_ws) && al(p.in_hs) && al(p.in_ns) &&
                     al(p.in_gs) && p.fil_cs == 1 && p.fil_xs == c && p.fil_ys == x * c &&
-                    al(p.fil_ks) && al(p.fil_gs);
+                    al(p.fil_ks) && al(p.fil_gs) &&
+                    // byte offsets inside one group's input slice and one filter tile < 2^31
+                    (n * p.in_ns + hi * p.in_hs + wi * p.in_ws + c) * es < ((int64_t)1 << 31) &&
+                    (256 * p.fil_ks + Kg) * es < ((int64_t)1 << 31);
   const Tile *tile = fast ? pick_tile(Mg, k, (int)g, true, forced_tile(o)) : nullptr;
   if (!tile)
     tile = fast ? pick_tile(Mg, k, (int)g, true, "") : &kGenericTile;
