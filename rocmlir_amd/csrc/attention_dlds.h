@@ -1,0 +1,263 @@
+// Fast path of the fused attention kernel (unit-stride head dimension, head
+// dims multiples of 8): K and V tiles stream global -> LDS without passing
+// through registers, V is transposed by the LDS read itself, and two blocks
+// share a compute unit so that one wave's softmax overlaps another's MFMAs.
+//
+// Included by attention_kernels.hip after the helpers it uses.  Algorithm and
+// accumulator layouts are the ones described at the top of that file; what
+// changes relative to the register-staged body there:
+//
+//   * K and V tiles (64 keys x D) are stored row-major with the 16-byte chunk
+//     index XOR-ed with the key row, filled by buffer_load ... lds (hardware
+//     zero fill for keys past seq_k and head-dim padding);
+//   * the V^T row operand of the second GEMM comes from ds_read_b64_tr_b16:
+//     within a group of 16 lanes, lane i addresses 4 consecutive d of key
+//     k0 + i/4 and receives the 4 keys k0..k0+3 at d = d0 + i.  Two such reads
+//     give the 8 keys {4h..4h+3, 8+4h..8+4h+3} of a 16-key slice -- exactly
+//     the keys whose probabilities the lane holds from the first GEMM;
+//   * the running-max rescale of O is skipped while no lane's maximum moved
+//     (alpha == 1 exactly, so the result is unchanged);
+//   * without bias and with a non-negative scale the row maximum is taken on
+//     the raw scores and the scale is folded into exp2(fma(s, c, -m)).
+#pragma once
+
+namespace rk {
+
+constexpr unsigned kAttnOob = 0x80000000u;
+typedef __attribute__((address_space(3))) void attn_lds_void_t;
+typedef __attribute__((address_space(3))) v4s attn_lds_v4s_t;
+
+template <int D> struct AttnTileGeom {
+  static constexpr int CPR = D / 8;         // 16-byte chunks per row
+  static constexpr int ROWB = D * 2;        // bytes per row
+  static constexpr int TILE_B = kBKV * ROWB;
+  static constexpr int SLABS = TILE_B / 1024;
+  static constexpr int PER_WAVE = SLABS / 4;
+  static_assert(SLABS % 4 == 0, "tile must split over 4 waves");
+};
+
+// One K or V tile loader: row-major [key][d] source with unit d stride.
+template <int D> struct AttnTileLoader {
+  using Gm = AttnTileGeom<D>;
+  __amdgpu_buffer_rsrc_t rsrc;
+  unsigned off[Gm::PER_WAVE]; // byte offset at key0 = 0, or kAttnOob for head-dim padding
+  int row[Gm::PER_WAVE];
+  int pitch_b, rows_total, wave;
+
+  __device__ __forceinline__ void init(const uint16_t *base, int64_t row_stride, int rows, int d,
+                                       int wave_, int lane) {
+    wave = wave_;
+    rows_total = rows;
+    pitch_b = (int)row_stride * 2;
+    rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(base), 0, (int)kAttnOob, 0x00020000);
+#pragma unroll
+    for (int i = 0; i < Gm::PER_WAVE; ++i) {
+      int c = (wave * Gm::PER_WAVE + i) * 64 + lane; // physical chunk inside the tile
+      int r = c / Gm::CPR, pc = c - r * Gm::CPR;
+      int lc = pc ^ (r & (Gm::CPR - 1));
+      row[i] = r;
+      off[i] = (lc * 8 < d) ? (unsigned)(r * pitch_b + lc * 16) : kAttnOob;
+    }
+  }
+  __device__ __forceinline__ void issue(int key0, char *tile) {
+#pragma unroll
+    for (int i = 0; i < Gm::PER_WAVE; ++i) {
+      unsigned voff = (key0 + row[i] < rows_total) ? off[i] + (unsigned)(key0 * pitch_b) : kAttnOob;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrc, (attn_lds_void_t *)(tile + (wave * Gm::PER_WAVE + i) * 1024), 16, (int)voff, 0, 0, 0);
+    }
+  }
+};
+
+template <int DT, int D>
+__device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv, const void *Vv,
+                                                  const void *biasv, void *Ov,
+                                                  const RockAttentionParams &p) {
+  using Gm = AttnTileGeom<D>;
+  constexpr int KSTEPS = D / 16;  // MFMA K steps of the first GEMM
+  constexpr int DTILES = D / 32;  // 32-row tiles of O^T
+  constexpr int STAGE = 2 * Gm::TILE_B;
+  constexpr float kLog2e = 1.44269504088896340736f;
+
+  __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lq = lane & 31, h = lane >> 5;
+
+  int bid = blockIdx.x;
+  {
+    const int total = p.G * p.q_blocks;
+    const int per = total >> 3;
+    if (p.xcd_remap && bid < (per << 3))
+      bid = (bid & 7) * per + (bid >> 3);
+  }
+  const int g = bid / p.q_blocks;
+  const int qb = bid - g * p.q_blocks;
+  const int q_row = qb * kBQ + wave * 32 + lq;
+
+  const uint16_t *Q = (const uint16_t *)Qv + (int64_t)g * p.q_gs;
+  const uint16_t *K = (const uint16_t *)Kv + (int64_t)g * p.k_gs;
+  const uint16_t *V = (const uint16_t *)Vv + (int64_t)g * p.v_gs;
+  uint16_t *O = (uint16_t *)Ov + (int64_t)g * p.o_gs;
+  const uint16_t *bias = p.has_bias ? (const uint16_t *)biasv + (int64_t)g * p.bias_gs : nullptr;
+
+  AttnTileLoader<D> lk, lv;
+  lk.init(K, p.k_js, p.seq_k, p.d_qk, wave, lane);
+  lv.init(V, p.v_js, p.seq_k, p.d_v, wave, lane);
+  lk.issue(0, lds);
+  lv.issue(0, lds + Gm::TILE_B);
+
+  v4i qf[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks)
+    qf[ks] = load8<true>(Q, p.q_is, p.q_ds, q_row, ks * 16 + h * 8, p.seq_q, p.d_qk);
+
+  v16f o[DTILES];
+#pragma unroll
+  for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v)
+      o[dt][v] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
+
+  const float c_scale = p.scale * kLog2e;
+  const bool plain = (bias == nullptr) && (c_scale >= 0.0f); // scale folds into the exponent
+  const int nkv = (p.seq_k + kBKV - 1) / kBKV;
+
+  // lane constants of the transposing V reads
+  const int tr_i = lane & 15, tr_g = (lane >> 4) & 1;
+  const int tr_key = 4 * h + (tr_i >> 2);                  // + 32*st + 16*u (+ 8)
+  const int tr_chunk = 2 * tr_g + ((tr_i & 3) >> 1);       // + 4*dt
+  const int tr_byte = (tr_i & 1) * 8;
+
+  for (int t = 0; t < nkv; ++t) {
+    wait_vmcnt_attn0();               // this wave's part of tile t has landed ...
+    __builtin_amdgcn_s_barrier();     // ... everyone's has, and tile t-1 is no longer being read
+    const char *sk = lds + (t & 1) * STAGE;
+    const char *sv = sk + Gm::TILE_B;
+    {
+      char *nxt = lds + ((t + 1) & 1) * STAGE;
+      lk.issue((t + 1) * kBKV, nxt);  // past the end: every lane out of range, zeros, no traffic
+      lv.issue((t + 1) * kBKV, nxt + Gm::TILE_B);
+    }
+
+    // ---- S^T tiles: rows = keys, cols = queries
+    v16f s[2];
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        s[st][v] = 0.0f;
+      const int kr = st * 32 + lq;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        v4i kf = *(const v4i *)(sk + kr * Gm::ROWB + (((ks * 2 + h) ^ (kr & (Gm::CPR - 1))) * 16));
+        s[st] = mma32<DT>(kf, qf[ks], s[st]);
+      }
+    }
+
+    // ---- online softmax on this lane's 32 scores of row q_row
+    const int key_base = t * kBKV + 4 * h;
+    const bool tail = (t + 1) * kBKV > p.seq_k;
+    float mloc = -INFINITY;
+    if (!plain) {
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          int key = key_base + st * 32 + 8 * (v >> 2) + (v & 3);
+          float x = s[st][v] * c_scale;
+          if (bias != nullptr && key < p.seq_k && q_row < p.seq_q)
+            x = x + elem_to_f32<DT>(bias[(int64_t)q_row * p.bias_is + (int64_t)key * p.bias_js]) * kLog2e;
+          s[st][v] = x;
+        }
+    }
+    if (tail) {
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          int key = key_base + st * 32 + 8 * (v >> 2) + (v & 3);
+          s[st][v] = key < p.seq_k ? s[st][v] : -INFINITY;
+        }
+    }
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        mloc = fmaxf(mloc, s[st][v]);
+    float mt = half_swap_max(mloc);
+    if (plain)
+      mt = mt * c_scale;
+    const float m_new = fmaxf(m_run, mt);
+    if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+      const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+      l_run *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          o[dt][v] *= alpha;
+      m_run = m_new;
+    }
+    const float m_use = (m_run == -INFINITY) ? 0.0f : m_run;
+    const float cs = plain ? c_scale : 1.0f;
+    float psum = 0.0f;
+    uint32_t pp[2][8];
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+      for (int v = 0; v < 16; v += 2) {
+        float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[st][v], cs, -m_use));
+        float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[st][v + 1], cs, -m_use));
+        psum += p0 + p1;
+        pp[st][v >> 1] = pack2<DT>(p0, p1);
+      }
+    l_run += psum;
+
+    // ---- O^T += V^T * P^T ; K step (st,u) covers keys 32*st + 16*u + [0,16)
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        v4i pf = {(int)pp[st][4 * u + 0], (int)pp[st][4 * u + 1], (int)pp[st][4 * u + 2],
+                  (int)pp[st][4 * u + 3]};
+        const int k0 = st * 32 + u * 16 + tr_key;
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt) {
+          const int ch = 4 * dt + tr_chunk;
+          const char *a0 = sv + k0 * Gm::ROWB + ((ch ^ (k0 & (Gm::CPR - 1))) * 16) + tr_byte;
+          const char *a1 = sv + (k0 + 8) * Gm::ROWB + ((ch ^ ((k0 + 8) & (Gm::CPR - 1))) * 16) + tr_byte;
+          v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((attn_lds_v4s_t *)a0);
+          v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((attn_lds_v4s_t *)a1);
+          v2i l2 = __builtin_bit_cast(v2i, lo), h2 = __builtin_bit_cast(v2i, hi);
+          v4i vf = {l2[0], l2[1], h2[0], h2[1]};
+          o[dt] = mma32<DT>(vf, pf, o[dt]);
+        }
+      }
+  }
+  wait_vmcnt_attn0(); // drain the out-of-range loads of the step past the end
+
+  // ---- normalise and store: lane holds O[q_row][32*dt + 8*(v/4) + 4*h + v%4]
+  const float l_tot = half_swap_sum(l_run);
+  const float inv = 1.0f / l_tot;
+  if (q_row < p.seq_q) {
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+      for (int vq = 0; vq < 4; ++vq) {
+        const int e0 = dt * 32 + 8 * vq + 4 * h;
+        if (e0 >= p.d_v)
+          continue;
+        uint16_t *dst = O + (int64_t)q_row * p.o_is + e0;
+        v2i pk = {(int)pack2<DT>(o[dt][4 * vq + 0] * inv, o[dt][4 * vq + 1] * inv),
+                  (int)pack2<DT>(o[dt][4 * vq + 2] * inv, o[dt][4 * vq + 3] * inv)};
+        *(v2i *)dst = pk;
+      }
+  }
+}
+
+} // namespace rk

@@ -316,7 +316,13 @@ __device__ __forceinline__ void attention_body(const void *Qv, const void *Kv, c
   }
 }
 
+__device__ __forceinline__ void wait_vmcnt_attn0() {
+  __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0); expcnt and lgkmcnt left alone
+}
+
 } // namespace rk
+
+#include "attention_dlds.h"
 
 // pointer order follows the reference: Q, K, V, [pre-softmax bias], O
 #define RK_ATTN(DTNAME, DT, DQK, DV, FASTNAME, FAST)                                          \
@@ -327,11 +333,20 @@ __device__ __forceinline__ void attention_body(const void *Qv, const void *Kv, c
     rk::attention_body<DT, DQK, DV, FAST>(Q, K, V, bias, O, p);                               \
   }
 
-RK_ATTN(f16, MM_F16, 128, 128, fast, true)
-RK_ATTN(f16, MM_F16, 64, 64, fast, true)
+// fast variants: two blocks per compute unit (register budget 256 per lane)
+#define RK_ATTN_DL(DTNAME, DT, D)                                                             \
+  extern "C" __global__ __launch_bounds__(rk::kAttnThreads, 2) void                           \
+      rock_attention_##DTNAME##_d##D##x##D##_fast(const void *Q, const void *K, const void *V,\
+                                                  const void *bias, void *O,                  \
+                                                  RockAttentionParams p) {                    \
+    rk::attention_body_dl<DT, D>(Q, K, V, bias, O, p);                                        \
+  }
+
+RK_ATTN_DL(f16, MM_F16, 128)
+RK_ATTN_DL(f16, MM_F16, 64)
 RK_ATTN(f16, MM_F16, 128, 128, generic, false)
 RK_ATTN(f16, MM_F16, 64, 64, generic, false)
-RK_ATTN(bf16, MM_BF16, 128, 128, fast, true)
-RK_ATTN(bf16, MM_BF16, 64, 64, fast, true)
+RK_ATTN_DL(bf16, MM_BF16, 128)
+RK_ATTN_DL(bf16, MM_BF16, 64)
 RK_ATTN(bf16, MM_BF16, 128, 128, generic, false)
 RK_ATTN(bf16, MM_BF16, 64, 64, generic, false)

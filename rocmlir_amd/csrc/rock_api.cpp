@@ -655,7 +655,10 @@ Handle *make_attention(const OptMap &o) {
   }
   p.xcd_remap = total >= 2 * kNumXCD ? 1 : 0;
   const bool fast = p.q_ds == 1 && p.k_ds == 1 && p.v_es == 1 && p.o_es == 1 && dqk % 8 == 0 &&
-                    dv % 8 == 0 && p.o_is % 4 == 0;
+                    dv % 8 == 0 && p.o_is % 4 == 0 && p.k_js % 8 == 0 && p.v_js % 8 == 0 &&
+                    p.q_is % 8 == 0 &&
+                    // byte offsets inside one g slice below 2^31 (buffer descriptors)
+                    sk * p.k_js * 2 < ((int64_t)1 << 31) && sk * p.v_js * 2 < ((int64_t)1 << 31);
   const int dmax = (dqk <= 64 && dv <= 64) ? 64 : 128;
   char name[96];
   std::snprintf(name, sizeof name, "rock_attention_%s_d%dx%d_%s", dtype_name(ty), dmax, dmax,
