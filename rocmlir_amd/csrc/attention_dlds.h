@@ -8,7 +8,7 @@
 // changes relative to the register-staged body there:
 //
 //   * K and V tiles (64 keys x D) are stored row-major with the 16-byte chunk
-//     index XOR-ed with the key row, filled by buffer_load ... lds (hardware
+//     index XOR-ed with a function of the key row, filled by buffer_load ... lds (hardware
 //     zero fill for keys past seq_k and head-dim padding);
 //   * the V^T row operand of the second GEMM comes from ds_read_b64_tr_b16:
 //     within a group of 16 lanes, lane i addresses 4 consecutive d of key
@@ -36,8 +36,20 @@ template <int D> struct AttnTileGeom {
   static_assert(SLABS % 4 == 0, "tile must split over 4 waves");
 };
 
+// Chunk swizzles (XOR-ed into the 16-byte chunk index of a row).  K rows are
+// read 32 rows at one chunk index; V rows are read by the transposing load, 4
+// consecutive rows x 2 adjacent chunks per 16 lanes.  Each function spreads
+// its access pattern over distinct bank groups for the row pitch at hand
+// (256 bytes = one full bank period for D = 128, half a period for D = 64).
+template <int CPR, bool IS_V> __device__ __forceinline__ int attn_swz(int row) {
+  if constexpr (!IS_V)
+    return CPR == 16 ? (row & 15) : ((row >> 1) & 7);
+  else
+    return CPR == 16 ? ((row & 7) << 1) : (((row >> 1) & 3) << 1);
+}
+
 // One K or V tile loader: row-major [key][d] source with unit d stride.
-template <int D> struct AttnTileLoader {
+template <int D, bool IS_V> struct AttnTileLoader {
   using Gm = AttnTileGeom<D>;
   __amdgpu_buffer_rsrc_t rsrc;
   unsigned off[Gm::PER_WAVE]; // byte offset at key0 = 0, or kAttnOob for head-dim padding
@@ -54,7 +66,7 @@ template <int D> struct AttnTileLoader {
     for (int i = 0; i < Gm::PER_WAVE; ++i) {
       int c = (wave * Gm::PER_WAVE + i) * 64 + lane; // physical chunk inside the tile
       int r = c / Gm::CPR, pc = c - r * Gm::CPR;
-      int lc = pc ^ (r & (Gm::CPR - 1));
+      int lc = pc ^ attn_swz<Gm::CPR, IS_V>(r);
       row[i] = r;
       off[i] = (lc * 8 < d) ? (unsigned)(r * pitch_b + lc * 16) : kAttnOob;
     }
@@ -103,7 +115,8 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
   uint16_t *O = (uint16_t *)Ov + (int64_t)g * p.o_gs;
   const uint16_t *bias = p.has_bias ? (const uint16_t *)biasv + (int64_t)g * p.bias_gs : nullptr;
 
-  AttnTileLoader<D> lk, lv;
+  AttnTileLoader<D, false> lk;
+  AttnTileLoader<D, true> lv;
   lk.init(K, p.k_js, p.seq_k, p.d_qk, wave, lane);
   lv.init(V, p.v_js, p.seq_k, p.d_v, wave, lane);
   lk.issue(0, lds);
@@ -153,7 +166,7 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
       const int kr = st * 32 + lq;
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) {
-        v4i kf = *(const v4i *)(sk + kr * Gm::ROWB + (((ks * 2 + h) ^ (kr & (Gm::CPR - 1))) * 16));
+        v4i kf = *(const v4i *)(sk + kr * Gm::ROWB + (((ks * 2 + h) ^ attn_swz<Gm::CPR, false>(kr)) * 16));
         s[st] = mma32<DT>(kf, qf[ks], s[st]);
       }
     }
@@ -229,8 +242,8 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
 #pragma unroll
         for (int dt = 0; dt < DTILES; ++dt) {
           const int ch = 4 * dt + tr_chunk;
-          const char *a0 = sv + k0 * Gm::ROWB + ((ch ^ (k0 & (Gm::CPR - 1))) * 16) + tr_byte;
-          const char *a1 = sv + (k0 + 8) * Gm::ROWB + ((ch ^ ((k0 + 8) & (Gm::CPR - 1))) * 16) + tr_byte;
+          const char *a0 = sv + k0 * Gm::ROWB + ((ch ^ attn_swz<Gm::CPR, true>(k0)) * 16) + tr_byte;
+          const char *a1 = sv + (k0 + 8) * Gm::ROWB + ((ch ^ attn_swz<Gm::CPR, true>(k0 + 8)) * 16) + tr_byte;
           v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((attn_lds_v4s_t *)a0);
           v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((attn_lds_v4s_t *)a1);
           v2i l2 = __builtin_bit_cast(v2i, lo), h2 = __builtin_bit_cast(v2i, hi);
