@@ -25,6 +25,7 @@
 // Limits checked on the host before this path is chosen: every in-range byte
 // offset relative to the block's base pointer is below 2^31.
 #pragma once
+#include <type_traits>
 #include "gemm_conv_kernel.h"
 
 namespace rk {
@@ -269,28 +270,62 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
   // ---- epilogue: lane holds m = .. + lrow, n = .. + 8*q + 4*lgrp + {0..3}
   const RockEpilogue &e = p.epi;
   using Acc4 = decltype(__builtin_shufflevector(acc[0][0], acc[0][0], 0, 1, 2, 3));
+  const bool staged_ok = out_rows_chunk_aligned(p, Cptr, out_elem_size(e.out_dtype));
+  if (staged_ok)
+    __builtin_amdgcn_s_barrier(); // every wave is done reading the operand stages
+
+  dispatch_out_dtype<Tr::INT_ACC>(e.out_dtype, [&](auto od_const) __attribute__((always_inline)) {
+    constexpr int OD = decltype(od_const)::value;
+    if (!staged_ok) {
+      direct_epilogue<Tr::INT_ACC, OD, MI, NI, Acc4>(acc, p, g, Cptr, aux, m0 + wm * WTM + lrow,
+                                                    n0 + wn * WTN + lgrp * 4);
+      return;
+    }
+    // Staged store: each wave transposes one 32-row block of its tile at a
+    // time through a private LDS region, so that global stores are 16 bytes
+    // per lane and cover whole rows of the wave tile (WTN * ES contiguous
+    // bytes per 64/LPR lanes).
+    constexpr int ES = OutElemSize<OD>::value;
+    constexpr int ROWB = WTN * ES, PITCH = ROWB + 16;
+    constexpr int LPR = ROWB / 16, RPI = 64 / LPR;
+    constexpr int WBUF = 32 * (WTN * 4 + 16);
+    static_assert(NW * WBUF <= kDlStages * STAGE, "staging buffers must fit in the operand stages");
+    char *wbuf = lds + wave * WBUF;
+    const int rd_row = lane / LPR, rd_cb = (lane % LPR) * 16;
 #pragma unroll
-  for (int i = 0; i < MI; ++i) {
-    const int m = m0 + wm * WTM + i * 32 + lrow;
-    if (m >= p.M)
-      continue;
-    int64_t row_off, n_stride;
-    bool vec_ok;
-    out_row_addr(p, g, m, Cptr, row_off, n_stride, vec_ok);
+    for (int i = 0; i < MI; ++i) {
 #pragma unroll
-    for (int j = 0; j < NI; ++j) {
+      for (int j = 0; j < NI; ++j) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int n = n0 + wn * WTN + j * 32 + q * 8 + lgrp * 4;
-        if (n >= p.N)
-          continue;
-        Acc4 a4 = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
-                   acc[i][j][4 * q + 3]};
-        epilogue_store4<Tr::INT_ACC>(a4, e, aux, Cptr, row_off + (int64_t)n * n_stride, n_stride,
-                                     n, p.N, vec_ok);
+        for (int q = 0; q < 4; ++q) {
+          const int nloc = j * 32 + q * 8 + lgrp * 4;
+          Acc4 a4 = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                     acc[i][j][4 * q + 3]};
+          v4i raw = epilogue_convert4<Tr::INT_ACC, OD>(a4, e, aux, n0 + wn * WTN + nloc, p.N);
+          char *dst = wbuf + lrow * PITCH + nloc * ES;
+          if constexpr (ES == 4)
+            *(v4i *)dst = raw;
+          else if constexpr (ES == 2)
+            *(v2i *)dst = v2i{raw[0], raw[1]};
+          else
+            *(int *)dst = raw[0];
+        }
+      }
+#pragma unroll
+      for (int r0 = 0; r0 < 32; r0 += RPI) {
+        const int row = r0 + rd_row;
+        v4i d = *(const v4i *)(wbuf + row * PITCH + rd_cb);
+        const int m = m0 + wm * WTM + i * 32 + row;
+        const int n = n0 + wn * WTN + rd_cb / ES;
+        if (m < p.M && n < p.N) {
+          int64_t row_off, n_stride;
+          bool vec_ok;
+          out_row_addr(p, g, m, Cptr, row_off, n_stride, vec_ok);
+          *(v4i *)((char *)Cptr + (row_off + n) * ES) = d;
+        }
       }
     }
-  }
+  });
 }
 
 } // namespace rk

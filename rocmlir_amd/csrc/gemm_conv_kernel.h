@@ -20,6 +20,7 @@
 //     past the tensor; the epilogue (scale, zero point, bias, cast) runs on
 //     the accumulators in registers.
 #pragma once
+#include <type_traits>
 #include "mfma_gfx950.h"
 
 namespace rk {
@@ -368,106 +369,124 @@ __device__ __forceinline__ Frag<DT> read_frag(const char *lds, int row, int step
 }
 
 // ---------------------------------------------------------------------------
-// Epilogue
+// Epilogue: convert 4 consecutive output channels of one row, pack them in
+// the output type, store them.
 // ---------------------------------------------------------------------------
-template <bool INT_ACC, typename Acc4>
-__device__ __forceinline__ void epilogue_store4(const Acc4 &acc, const RockEpilogue &e,
-                                                const void *aux, void *out_base,
-                                                int64_t off, int64_t n_stride,
-                                                int n0, int n_limit, bool vec_ok) {
-  // acc[r] belongs to output channel n0 + r
-  const int od = e.out_dtype;
-  if (INT_ACC && od == ROCK_I32) {
-    int v[4]; // exact accumulators, optional int32 bias
+__device__ __forceinline__ int out_elem_size(int od) {
+  return (od == ROCK_F32 || od == ROCK_I32) ? 4 : (od == ROCK_F16 || od == ROCK_BF16) ? 2 : 1;
+}
+
+// acc[r] belongs to output channel n0 + r.  Returns the 4 results packed
+// back to back in the low 4*elem_size bytes.  OD (the output type) is a
+// compile-time constant so that the unrolled epilogue is straight-line code.
+template <bool INT_ACC, int OD, typename Acc4>
+__device__ __forceinline__ v4i epilogue_convert4(const Acc4 &acc, const RockEpilogue &e,
+                                                 const void *aux, int n0, int n_limit) {
+  if constexpr (INT_ACC && OD == ROCK_I32) { // exact accumulators, optional int32 bias
+    v4i v;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       v[r] = (int)acc[r];
       if (e.has_bias && n0 + r < n_limit)
         v[r] += ((const int *)aux)[n0 + r];
     }
-    int *o = (int *)out_base;
-    if (vec_ok && n0 + 3 < n_limit) {
-      *(v4i *)(o + off) = v4i{v[0], v[1], v[2], v[3]};
-    } else {
+    return v;
+  } else {
+    float v[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float f;
+      if constexpr (INT_ACC)
+        f = ((float)(int)acc[r] - (float)e.zero_point) * e.scale;
+      else
+        f = (float)acc[r] * e.scale;
+      if (e.has_bias && n0 + r < n_limit)
+        f = f + ((const float *)aux)[n0 + r];
+      if (e.relu)
+        f = fmaxf(f, 0.0f);
+      v[r] = f;
+    }
+    v4i out = {0, 0, 0, 0};
+    if constexpr (OD == ROCK_F32) {
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        if (n0 + r < n_limit)
-          o[off + r * n_stride] = v[r];
+        out[r] = __builtin_bit_cast(int, v[r]);
+    } else if constexpr (OD == ROCK_F16) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        _Float16 hv = (_Float16)v[r];
+        out[r >> 1] |= (int)__builtin_bit_cast(uint16_t, hv) << (16 * (r & 1));
+      }
+    } else if constexpr (OD == ROCK_BF16) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        __bf16 hv = (__bf16)v[r];
+        out[r >> 1] |= (int)__builtin_bit_cast(uint16_t, hv) << (16 * (r & 1));
+      }
+    } else if constexpr (OD == ROCK_I8) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float q = __builtin_rintf(v[r] * e.inv_quant_scale) + (float)e.out_zero_point;
+        out[0] |= ((int)f32_to_i8_sat(q) & 0xff) << (8 * r);
+      }
+    } else if constexpr (OD == ROCK_FP8) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        out[0] |= (int)f32_to_e4m3fn_sat(v[r]) << (8 * r);
+    } else if constexpr (OD == ROCK_BF8) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        out[0] |= (int)f32_to_e5m2_sat(v[r]) << (8 * r);
     }
+    return out;
+  }
+}
+
+// Calls f(std::integral_constant<int, OD>) for the run-time output type.
+template <bool INT_ACC, typename F>
+__device__ __forceinline__ void dispatch_out_dtype(int od, F &&f) {
+  switch (od) {
+  case ROCK_F32: f(std::integral_constant<int, ROCK_F32>{}); break;
+  case ROCK_F16: f(std::integral_constant<int, ROCK_F16>{}); break;
+  case ROCK_BF16: f(std::integral_constant<int, ROCK_BF16>{}); break;
+  case ROCK_I8: f(std::integral_constant<int, ROCK_I8>{}); break;
+  case ROCK_FP8: f(std::integral_constant<int, ROCK_FP8>{}); break;
+  case ROCK_BF8: f(std::integral_constant<int, ROCK_BF8>{}); break;
+  case ROCK_I32:
+    if constexpr (INT_ACC)
+      f(std::integral_constant<int, ROCK_I32>{});
+    break; // float accumulators written as int32 are not a legal problem
+  }
+}
+
+template <int OD> struct OutElemSize {
+  static constexpr int value = (OD == ROCK_F32 || OD == ROCK_I32) ? 4 : (OD == ROCK_F16 || OD == ROCK_BF16) ? 2 : 1;
+};
+
+// `off` is the element offset of channel n0 of this row.
+__device__ __forceinline__ void store_packed4(const v4i &raw, int es, void *out_base, int64_t off,
+                                              int64_t n_stride, int n0, int n_limit, bool vec_ok) {
+  char *o = (char *)out_base;
+  if (vec_ok && n0 + 3 < n_limit) {
+    if (es == 4)
+      *(v4i *)(o + off * 4) = raw;
+    else if (es == 2)
+      *(v2i *)(o + off * 2) = v2i{raw[0], raw[1]};
+    else
+      *(int *)(o + off) = raw[0];
     return;
   }
-  float v[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    float f;
-    if constexpr (INT_ACC)
-      f = ((float)(int)acc[r] - (float)e.zero_point) * e.scale;
+    if (n0 + r >= n_limit)
+      continue;
+    int64_t idx = off + r * n_stride;
+    if (es == 4)
+      ((int *)o)[idx] = raw[r];
+    else if (es == 2)
+      ((uint16_t *)o)[idx] = (uint16_t)((uint32_t)raw[r >> 1] >> (16 * (r & 1)));
     else
-      f = (float)acc[r] * e.scale;
-    if (e.has_bias && n0 + r < n_limit)
-      f = f + ((const float *)aux)[n0 + r];
-    if (e.relu)
-      f = fmaxf(f, 0.0f);
-    v[r] = f;
-  }
-  const bool full = vec_ok && n0 + 3 < n_limit;
-  switch (od) {
-  case ROCK_F32: {
-    float *o = (float *)out_base;
-    if (full) {
-      *(v4f *)(o + off) = v4f{v[0], v[1], v[2], v[3]};
-    } else {
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (n0 + r < n_limit) o[off + r * n_stride] = v[r];
-    }
-    break;
-  }
-  case ROCK_F16: {
-    _Float16 *o = (_Float16 *)out_base;
-    if (full) {
-      *(v4h *)(o + off) = v4h{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
-    } else {
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (n0 + r < n_limit) o[off + r * n_stride] = (_Float16)v[r];
-    }
-    break;
-  }
-  case ROCK_BF16: {
-    __bf16 *o = (__bf16 *)out_base;
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-      if (n0 + r < n_limit) o[off + r * n_stride] = (__bf16)v[r];
-    break;
-  }
-  case ROCK_I8: {
-    int8_t *o = (int8_t *)out_base;
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-      if (n0 + r < n_limit) {
-        float q = __builtin_rintf(v[r] * e.inv_quant_scale) + (float)e.out_zero_point;
-        o[off + r * n_stride] = f32_to_i8_sat(q);
-      }
-    break;
-  }
-  case ROCK_FP8: {
-    uint8_t *o = (uint8_t *)out_base;
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-      if (n0 + r < n_limit) o[off + r * n_stride] = f32_to_e4m3fn_sat(v[r]);
-    break;
-  }
-  case ROCK_BF8: {
-    uint8_t *o = (uint8_t *)out_base;
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-      if (n0 + r < n_limit) o[off + r * n_stride] = f32_to_e5m2_sat(v[r]);
-    break;
-  }
-  case ROCK_I32: { // float accumulators written as int32 are not a legal problem
-    break;
-  }
+      ((uint8_t *)o)[idx] = (uint8_t)((uint32_t)raw[0] >> (8 * r));
   }
 }
 
@@ -476,8 +495,8 @@ __device__ __forceinline__ int p_batch(const RockGemmParams &p) { return p.G; }
 __device__ __forceinline__ int p_batch(const RockConvParams &p) { return p.g; }
 
 __device__ __forceinline__ bool aligned_for_vec(const void *base, int64_t row_off, int out_dtype) {
-  // 4 consecutive outputs stored as one 8/16-byte access need that alignment
-  int es = (out_dtype == ROCK_F32 || out_dtype == ROCK_I32) ? 4 : 2;
+  // 4 consecutive outputs stored as one 4/8/16-byte access need that alignment
+  int es = out_elem_size(out_dtype);
   return ((((uintptr_t)base) + (uintptr_t)row_off * es) & (uintptr_t)(4 * es - 1)) == 0;
 }
 
@@ -497,6 +516,19 @@ __device__ __forceinline__ void out_row_addr(const RockConvParams &p, int g, int
   row_off = (int64_t)n * p.out_ns + (int64_t)g * p.out_gs + (int64_t)ho * p.out_hs + (int64_t)wo * p.out_ws;
   n_stride = p.out_ks;
   vec_ok = (p.out_ks == 1) && aligned_for_vec(base, row_off, p.epi.out_dtype);
+}
+
+// Every output row starts on a 16-byte boundary, rows are n-contiguous and a
+// row is a whole number of 16-byte pieces: the staged epilogue may write 16
+// bytes per lane.
+__device__ __forceinline__ bool out_rows_chunk_aligned(const RockGemmParams &p, const void *base, int es) {
+  return p.c_ns == 1 && (((uintptr_t)base | (uintptr_t)(p.c_ms * es) | (uintptr_t)(p.c_gs * es) |
+                          (uintptr_t)((int64_t)p.N * es)) & 15) == 0;
+}
+__device__ __forceinline__ bool out_rows_chunk_aligned(const RockConvParams &p, const void *base, int es) {
+  return p.out_ks == 1 &&
+         (((uintptr_t)base | (uintptr_t)(p.out_ns * es) | (uintptr_t)(p.out_gs * es) |
+           (uintptr_t)(p.out_hs * es) | (uintptr_t)(p.out_ws * es) | (uintptr_t)((int64_t)p.N * es)) & 15) == 0;
 }
 
 template <int DT, int ROWS, int NT, int KIND>
@@ -546,6 +578,36 @@ __device__ __forceinline__ auto make_loader_b(const void *fil, const RockConvPar
     ConvFilGeneric<DT, ROWS, NT> l;
     l.init(fil, p, g, n0, tid);
     return l;
+  }
+}
+
+// Epilogue straight from the accumulator layout: the lane owns rows
+// m_lane + 32*i and channels n_lane + 32*j + 8*q + {0..3}.
+template <bool INT_ACC, int OD, int MI, int NI, typename Acc4, typename AccArr, typename Params>
+__device__ __forceinline__ void direct_epilogue(const AccArr &acc, const Params &p, int g, void *Cptr,
+                                                const void *aux, int m_lane, int n_lane) {
+  constexpr int ES = OutElemSize<OD>::value;
+#pragma unroll
+  for (int i = 0; i < MI; ++i) {
+    const int m = m_lane + i * 32;
+    if (m >= p.M)
+      continue;
+    int64_t row_off, n_stride;
+    bool vec_ok;
+    out_row_addr(p, g, m, Cptr, row_off, n_stride, vec_ok);
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n_lane + j * 32 + q * 8;
+        if (n >= p.N)
+          continue;
+        Acc4 a4 = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                   acc[i][j][4 * q + 3]};
+        v4i raw = epilogue_convert4<INT_ACC, OD>(a4, p.epi, aux, n, p.N);
+        store_packed4(raw, ES, Cptr, row_off + (int64_t)n * n_stride, n_stride, n, p.N, vec_ok);
+      }
+    }
   }
 }
 
@@ -638,28 +700,11 @@ __device__ __forceinline__ void contraction_body(const void *Aptr, const void *B
   // ---- epilogue: lane holds m = .. + lrow, n = .. + 8*q + 4*lgrp + {0..3}
   const RockEpilogue &e = p.epi;
   using Acc4 = decltype(__builtin_shufflevector(acc[0][0], acc[0][0], 0, 1, 2, 3));
-#pragma unroll
-  for (int i = 0; i < MI; ++i) {
-    const int m = m0 + wm * WTM + i * 32 + lrow;
-    if (m >= p.M)
-      continue;
-    int64_t row_off, n_stride;
-    bool vec_ok;
-    out_row_addr(p, g, m, Cptr, row_off, n_stride, vec_ok);
-#pragma unroll
-    for (int j = 0; j < NI; ++j) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int n = n0 + wn * WTN + j * 32 + q * 8 + lgrp * 4;
-        if (n >= p.N)
-          continue;
-        Acc4 a4 = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
-                   acc[i][j][4 * q + 3]};
-        epilogue_store4<Tr::INT_ACC>(a4, e, aux, Cptr, row_off + (int64_t)n * n_stride, n_stride,
-                                     n, p.N, vec_ok);
-      }
-    }
-  }
+  dispatch_out_dtype<Tr::INT_ACC>(e.out_dtype, [&](auto od_const) __attribute__((always_inline)) {
+    constexpr int OD = decltype(od_const)::value;
+    direct_epilogue<Tr::INT_ACC, OD, MI, NI, Acc4>(acc, p, g, Cptr, aux, m0 + wm * WTM + lrow,
+                                                  n0 + wn * WTN + lgrp * 4);
+  });
 }
 
 } // namespace rk
