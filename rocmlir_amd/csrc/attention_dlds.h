@@ -8,13 +8,18 @@
 // changes relative to the register-staged body there:
 //
 //   * K and V tiles (64 keys x D) are stored row-major with the 16-byte chunk
-//     index XOR-ed with a function of the key row, filled by buffer_load ... lds (hardware
-//     zero fill for keys past seq_k and head-dim padding);
+//     index XOR-ed with a function of the key row, filled by
+//     buffer_load ... lds (hardware zero fill for keys past seq_k and for
+//     head-dim padding);
 //   * the V^T row operand of the second GEMM comes from ds_read_b64_tr_b16:
 //     within a group of 16 lanes, lane i addresses 4 consecutive d of key
 //     k0 + i/4 and receives the 4 keys k0..k0+3 at d = d0 + i.  Two such reads
 //     give the 8 keys {4h..4h+3, 8+4h..8+4h+3} of a 16-key slice -- exactly
 //     the keys whose probabilities the lane holds from the first GEMM;
+//   * every LDS read address is "per-lane offset computed once + immediate":
+//     the swizzles only depend on the low bits of the key row, which the
+//     tile / slice / stage offsets (multiples of 8 rows) do not touch, and the
+//     loop is unrolled over the two stages;
 //   * the running-max rescale of O is skipped while no lane's maximum moved
 //     (alpha == 1 exactly, so the result is unchanged);
 //   * without bias and with a non-negative scale the row maximum is taken on
@@ -25,7 +30,9 @@ namespace rk {
 
 constexpr unsigned kAttnOob = 0x80000000u;
 typedef __attribute__((address_space(3))) void attn_lds_void_t;
+typedef __attribute__((address_space(3))) char attn_lds_char_t;
 typedef __attribute__((address_space(3))) v4s attn_lds_v4s_t;
+typedef __attribute__((address_space(3))) v4i attn_lds_v4i_t;
 
 template <int D> struct AttnTileGeom {
   static constexpr int CPR = D / 8;         // 16-byte chunks per row
@@ -40,7 +47,8 @@ template <int D> struct AttnTileGeom {
 // read 32 rows at one chunk index; V rows are read by the transposing load, 4
 // consecutive rows x 2 adjacent chunks per 16 lanes.  Each function spreads
 // its access pattern over distinct bank groups for the row pitch at hand
-// (256 bytes = one full bank period for D = 128, half a period for D = 64).
+// (256 bytes = one full bank period for D = 128, half a period for D = 64),
+// and depends only on the row modulo 16 (K) or modulo 8 (V).
 template <int CPR, bool IS_V> __device__ __forceinline__ int attn_swz(int row) {
   if constexpr (!IS_V)
     return CPR == 16 ? (row & 15) : ((row >> 1) & 7);
@@ -51,17 +59,17 @@ template <int CPR, bool IS_V> __device__ __forceinline__ int attn_swz(int row) {
 // One K or V tile loader: row-major [key][d] source with unit d stride.
 template <int D, bool IS_V> struct AttnTileLoader {
   using Gm = AttnTileGeom<D>;
-  __amdgpu_buffer_rsrc_t rsrc;
-  unsigned off[Gm::PER_WAVE]; // byte offset at key0 = 0, or kAttnOob for head-dim padding
+  const char *base;
+  unsigned off[Gm::PER_WAVE]; // byte offset inside a tile, or kAttnOob for head-dim padding
   int row[Gm::PER_WAVE];
   int pitch_b, rows_total, wave;
 
-  __device__ __forceinline__ void init(const uint16_t *base, int64_t row_stride, int rows, int d,
+  __device__ __forceinline__ void init(const uint16_t *base_, int64_t row_stride, int rows, int d,
                                        int wave_, int lane) {
     wave = wave_;
     rows_total = rows;
     pitch_b = (int)row_stride * 2;
-    rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(base), 0, (int)kAttnOob, 0x00020000);
+    base = (const char *)base_;
 #pragma unroll
     for (int i = 0; i < Gm::PER_WAVE; ++i) {
       int c = (wave * Gm::PER_WAVE + i) * 64 + lane; // physical chunk inside the tile
@@ -71,15 +79,36 @@ template <int D, bool IS_V> struct AttnTileLoader {
       off[i] = (lc * 8 < d) ? (unsigned)(r * pitch_b + lc * 16) : kAttnOob;
     }
   }
-  __device__ __forceinline__ void issue(int key0, char *tile) {
+  // The descriptor is rebuilt per tile with its base at key0 (scalar work), so
+  // the per-lane offsets never change; only the last tile needs the row test.
+  __device__ __forceinline__ void issue(int key0, attn_lds_char_t *tile) {
+    __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char *>(base + (int64_t)key0 * pitch_b), 0, (int)kAttnOob, 0x00020000);
+    const int left = rows_total - key0; // rows of this tile that exist (may be <= 0)
 #pragma unroll
     for (int i = 0; i < Gm::PER_WAVE; ++i) {
-      unsigned voff = (key0 + row[i] < rows_total) ? off[i] + (unsigned)(key0 * pitch_b) : kAttnOob;
+      unsigned voff = (row[i] < left) ? off[i] : kAttnOob;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
           rsrc, (attn_lds_void_t *)(tile + (wave * Gm::PER_WAVE + i) * 1024), 16, (int)voff, 0, 0, 0);
     }
   }
 };
+
+template <int DT> __device__ __forceinline__ uint32_t pack2_fast(float a, float b) {
+  if constexpr (DT == MM_F16) {
+    typedef float v2f_t __attribute__((ext_vector_type(2)));
+    typedef _Float16 v2h_t __attribute__((ext_vector_type(2)));
+    v2f_t f = {a, b};
+    v2h_t hv = __builtin_convertvector(f, v2h_t); // round to nearest even
+    return __builtin_bit_cast(uint32_t, hv);
+  } else {
+    typedef float v2f_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 v2b_t __attribute__((ext_vector_type(2)));
+    v2f_t f = {a, b};
+    v2b_t hv = __builtin_convertvector(f, v2b_t);
+    return __builtin_bit_cast(uint32_t, hv);
+  }
+}
 
 template <int DT, int D>
 __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv, const void *Vv,
@@ -90,8 +119,10 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
   constexpr int DTILES = D / 32;  // 32-row tiles of O^T
   constexpr int STAGE = 2 * Gm::TILE_B;
   constexpr float kLog2e = 1.44269504088896340736f;
+  static_assert(2 * STAGE <= 65536, "every LDS read offset must fit the 16-bit immediate");
 
-  __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE];
+  __shared__ __attribute__((aligned(1024))) char lds_generic[2 * STAGE];
+  attn_lds_char_t *lds = (attn_lds_char_t *)lds_generic;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -127,6 +158,24 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
   for (int ks = 0; ks < KSTEPS; ++ks)
     qf[ks] = load8<true>(Q, p.q_is, p.q_ds, q_row, ks * 16 + h * 8, p.seq_q, p.d_qk);
 
+  // ---- per-lane LDS read offsets (bytes from the start of a K or V tile)
+  // K fragment of key rows 32*st + lq at chunk 2*ks + h: the swizzle depends on
+  // lq only, so "+ 32*st rows" and the stage are immediates.
+  attn_lds_char_t *kptr[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks)
+    kptr[ks] = lds + lq * Gm::ROWB + (((ks * 2 + h) ^ attn_swz<Gm::CPR, false>(lq)) * 16);
+  // V^T fragment through the transposing read: lane (i = lane % 16, g16) of
+  // half h addresses key 4*h + i/4 (+ 32*st + 16*u, + 8) at d = 32*dt + 16*g16 + 4*(i%4).
+  const int tr_i = lane & 15, tr_g = (lane >> 4) & 1;
+  const int tr_key = 4 * h + (tr_i >> 2);
+  const int tr_chunk = 2 * tr_g + ((tr_i & 3) >> 1);
+  attn_lds_char_t *vptr[DTILES];
+#pragma unroll
+  for (int dt = 0; dt < DTILES; ++dt)
+    vptr[dt] = lds + Gm::TILE_B + tr_key * Gm::ROWB +
+               (((4 * dt + tr_chunk) ^ attn_swz<Gm::CPR, true>(tr_key)) * 16) + (tr_i & 1) * 8;
+
   v16f o[DTILES];
 #pragma unroll
   for (int dt = 0; dt < DTILES; ++dt)
@@ -139,19 +188,13 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
   const bool plain = (bias == nullptr) && (c_scale >= 0.0f); // scale folds into the exponent
   const int nkv = (p.seq_k + kBKV - 1) / kBKV;
 
-  // lane constants of the transposing V reads
-  const int tr_i = lane & 15, tr_g = (lane >> 4) & 1;
-  const int tr_key = 4 * h + (tr_i >> 2);                  // + 32*st + 16*u (+ 8)
-  const int tr_chunk = 2 * tr_g + ((tr_i & 3) >> 1);       // + 4*dt
-  const int tr_byte = (tr_i & 1) * 8;
-
-  for (int t = 0; t < nkv; ++t) {
+  // one K/V tile; STG (0/1) is the LDS stage holding it
+  auto tile_step = [&](int t, auto stage_const) __attribute__((always_inline)) {
+    constexpr int STG = decltype(stage_const)::value;
     wait_vmcnt_attn0();               // this wave's part of tile t has landed ...
     __builtin_amdgcn_s_barrier();     // ... everyone's has, and tile t-1 is no longer being read
-    const char *sk = lds + (t & 1) * STAGE;
-    const char *sv = sk + Gm::TILE_B;
     {
-      char *nxt = lds + ((t + 1) & 1) * STAGE;
+      attn_lds_char_t *nxt = lds + (STG ^ 1) * STAGE;
       lk.issue((t + 1) * kBKV, nxt);  // past the end: every lane out of range, zeros, no traffic
       lv.issue((t + 1) * kBKV, nxt + Gm::TILE_B);
     }
@@ -163,10 +206,9 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
 #pragma unroll
       for (int v = 0; v < 16; ++v)
         s[st][v] = 0.0f;
-      const int kr = st * 32 + lq;
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) {
-        v4i kf = *(const v4i *)(sk + kr * Gm::ROWB + (((ks * 2 + h) ^ attn_swz<Gm::CPR, false>(kr)) * 16));
+        v4i kf = *(const attn_lds_v4i_t *)(kptr[ks] + (STG * STAGE + st * 32 * Gm::ROWB));
         s[st] = mma32<DT>(kf, qf[ks], s[st]);
       }
     }
@@ -174,7 +216,6 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
     // ---- online softmax on this lane's 32 scores of row q_row
     const int key_base = t * kBKV + 4 * h;
     const bool tail = (t + 1) * kBKV > p.seq_k;
-    float mloc = -INFINITY;
     if (!plain) {
 #pragma unroll
       for (int st = 0; st < 2; ++st)
@@ -196,6 +237,7 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
           s[st][v] = key < p.seq_k ? s[st][v] : -INFINITY;
         }
     }
+    float mloc = -INFINITY;
 #pragma unroll
     for (int st = 0; st < 2; ++st)
 #pragma unroll
@@ -227,7 +269,7 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
         float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[st][v], cs, -m_use));
         float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[st][v + 1], cs, -m_use));
         psum += p0 + p1;
-        pp[st][v >> 1] = pack2<DT>(p0, p1);
+        pp[st][v >> 1] = pack2_fast<DT>(p0, p1);
       }
     l_run += psum;
 
@@ -238,19 +280,23 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
       for (int u = 0; u < 2; ++u) {
         v4i pf = {(int)pp[st][4 * u + 0], (int)pp[st][4 * u + 1], (int)pp[st][4 * u + 2],
                   (int)pp[st][4 * u + 3]};
-        const int k0 = st * 32 + u * 16 + tr_key;
+        constexpr int kSliceB = 16 * Gm::ROWB; // 16 keys
 #pragma unroll
         for (int dt = 0; dt < DTILES; ++dt) {
-          const int ch = 4 * dt + tr_chunk;
-          const char *a0 = sv + k0 * Gm::ROWB + ((ch ^ attn_swz<Gm::CPR, true>(k0)) * 16) + tr_byte;
-          const char *a1 = sv + (k0 + 8) * Gm::ROWB + ((ch ^ attn_swz<Gm::CPR, true>(k0 + 8)) * 16) + tr_byte;
+          attn_lds_char_t *a0 = vptr[dt] + (STG * STAGE + (st * 2 + u) * kSliceB);
           v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((attn_lds_v4s_t *)a0);
-          v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((attn_lds_v4s_t *)a1);
+          v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((attn_lds_v4s_t *)(a0 + 8 * Gm::ROWB));
           v2i l2 = __builtin_bit_cast(v2i, lo), h2 = __builtin_bit_cast(v2i, hi);
           v4i vf = {l2[0], l2[1], h2[0], h2[1]};
           o[dt] = mma32<DT>(vf, pf, o[dt]);
         }
       }
+  };
+
+  for (int t = 0; t < nkv; t += 2) {
+    tile_step(t, std::integral_constant<int, 0>{});
+    if (t + 1 < nkv)
+      tile_step(t + 1, std::integral_constant<int, 1>{});
   }
   wait_vmcnt_attn0(); // drain the out-of-range loads of the step past the end
 

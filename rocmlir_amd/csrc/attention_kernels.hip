@@ -24,6 +24,7 @@
 //     operands are single conflict-free 16-byte reads;
 //   * next K/V tiles are fetched into registers while the current ones are
 //     being multiplied; two LDS stages, one barrier per tile.
+#include <type_traits>
 #include "mfma_gfx950.h"
 
 namespace rk {
