@@ -44,16 +44,17 @@ template <int D> struct AttnTileGeom {
 };
 
 // Chunk swizzles (XOR-ed into the 16-byte chunk index of a row).  K rows are
-// read 32 rows at one chunk index; V rows are read by the transposing load, 4
-// consecutive rows x 2 adjacent chunks per 16 lanes.  Each function spreads
-// its access pattern over distinct bank groups for the row pitch at hand
-// (256 bytes = one full bank period for D = 128, half a period for D = 64),
-// and depends only on the row modulo 16 (K) or modulo 8 (V).
+// read 32 rows at one chunk index.  V rows are read by the transposing load:
+// 32 lanes cover 4 consecutive rows x 4 adjacent chunks (chunk bits 0-1 come
+// from the lane), so the row index is XOR-ed into the chunk bits above them.
+// Each function spreads its access pattern over distinct bank groups for the
+// row pitch at hand (256 bytes = one full bank period for D = 128, half a
+// period for D = 64), and depends only on the row modulo 16 (K) or 8 (V).
 template <int CPR, bool IS_V> __device__ __forceinline__ int attn_swz(int row) {
   if constexpr (!IS_V)
     return CPR == 16 ? (row & 15) : ((row >> 1) & 7);
   else
-    return CPR == 16 ? ((row & 7) << 1) : (((row >> 1) & 3) << 1);
+    return CPR == 16 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2);
 }
 
 // One K or V tile loader: row-major [key][d] source with unit d stride.

@@ -1,7 +1,7 @@
 // Instantiations of the contraction kernel for one operand type.  Compiled
 // once per type with -DROCK_DT=<code> -DROCK_DTNAME=<name> into a gfx950 code
 // object; the host library picks a kernel by name from its perf-config table.
-#include "gemm_conv_dlds.h"
+#include "gemm_splitk.h"
 
 #ifndef ROCK_DT
 #error "compile with -DROCK_DT=<operand type code> -DROCK_DTNAME=<suffix>"
@@ -46,6 +46,12 @@ RK_GEMM_DL(_256x128_fast, 256, 128, 4, 2)
 RK_GEMM_DL(_128x128_fast, 128, 128, 2, 2)
 RK_GEMM_DL(_64x64_fast, 64, 64, 2, 2)
 RK_GEMM(_64x64_generic, 64, 64, 2, 2, rk::LD_ROWS_GENERIC, rk::LD_ROWS_GENERIC)
+
+// small outputs: 32x32 tile per block, K split over the block's four waves
+extern "C" __global__ __launch_bounds__(256) void RK_CAT(RK_CAT(rock_gemm_, ROCK_DTNAME), _32x32_splitk)(
+    const void *A, const void *B, void *C, const void *aux, RockGemmParams p) {
+  rk::gemm_body_splitk<ROCK_DT>(A, B, C, aux, p);
+}
 
 #if ROCK_DT != 7 && ROCK_DT != 8
 RK_CONV_DL(_256x128_fast, 256, 128, 4, 2)

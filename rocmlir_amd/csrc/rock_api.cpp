@@ -196,6 +196,8 @@ const Tile kFastTiles[] = {
     {"_64x64_fast", 64, 64, 2, 2, 4, 0.40f, true, true},
 };
 const Tile kGenericTile = {"_64x64_generic", 64, 64, 2, 2, 4, 0.1f, true, true};
+// 32x32 output tile, K split over the four waves of the block (GEMM fast path only)
+const Tile kSplitKTile = {"_32x32_splitk", 32, 32, 1, 4, 2, 0.3f, true, false};
 constexpr int kNumCU = 256; // MI355X
 constexpr int kNumXCD = 8;
 
@@ -383,12 +385,34 @@ Handle *make_gemm(const OptMap &o) {
   const Tile *tile = fast ? pick_tile(M, N, (int)G, false, forced_tile(o)) : nullptr;
   if (!tile)
     tile = fast ? pick_tile(M, N, (int)G, false, "") : &kGenericTile;
+  // Too few 64x64 tiles to occupy half the CUs and a K long enough to split:
+  // one 32x32 tile per block with the K range divided over its waves (the
+  // reference's answer to the same situation is split-K with atomics,
+  // RockTuningImpl.cpp:962-1008).
+  const bool forced = !forced_tile(o).empty();
+  const int64_t tiles64 = (int64_t)ceil_div(M, 64) * ceil_div(N, 64) * G;
+  int split_k = 1;
+  if (fast && !forced && tiles64 * 2 <= kNumCU && K * es >= 16 * 64) {
+    tile = &kSplitKTile;
+    split_k = 4;
+  }
+  if (fast && str_or(o, "perf_config", "").find("32,32,") != std::string::npos) {
+    tile = &kSplitKTile; // "-perf_config v2:32,32,..." asks for it explicitly
+    split_k = 4;
+  }
   apply_tile_grid(*tile, M, N, (int)G, p.tiles_m, p.tiles_n, p.group_m, p.xcd_remap,
                   h->block_size, h->grid_size);
+  if (split_k > 1)
+    h->block_size = 256;
   h->kernel_name = std::string("rock_gemm_") + operand_name(code) + tile->suffix;
   h->blob_name = std::string("gemm_") + operand_name(code);
   h->num_pointers = 4;
   h->perf_config = perf_string(*tile, es);
+  if (split_k > 1) { // the reference's grammar has a splitK field (7th)
+    char buf[96];
+    std::snprintf(buf, sizeof buf, "v2:32,32,4,32,32,%d,%d,1,1", 16 / es, split_k);
+    h->perf_config = buf;
+  }
   // problem key (RockTuningImpl.cpp:808-862)
   {
     std::ostringstream k;

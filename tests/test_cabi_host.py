@@ -90,7 +90,10 @@ def test_bad_problems_give_null(rock, bad):
 
 def test_baseline_configs_select_kernels(rock):
     k = rock.RockKernel("-operation gemm -arch gfx950 -t f32 -g 1 -m 512 -n 512 -k 512 -transB true")
-    assert k.kernel_name.startswith("rock_gemm_f32_") and k.kernel_name.endswith("_fast")
+    # 64 output tiles of 64x64 would leave 3/4 of the CUs idle: K is split over waves
+    assert k.kernel_name == "rock_gemm_f32_32x32_splitk"
+    assert (k.block_size, k.grid_size) == (256, 256)
+    assert k.perf_config == "v2:32,32,4,32,32,4,4,1,1"
     k = rock.RockKernel("-operation gemm -arch gfx950 -t i8 -out_datatype f16 -g 1 -m 4096 -n 4096 "
                         "-k 4096 -transB true -scale 0.01")
     assert k.kernel_name == "rock_gemm_i8_256x256_fast"
@@ -123,8 +126,11 @@ def test_perf_config_override_and_fallback(rock):
     assert rock.RockKernel(base + " -perf_config v2:128,128,8,64,16,16,1,1,1").kernel_name == \
         "rock_gemm_i8_128x128_fast"
     # a config naming no available tile falls back to the table
-    assert rock.RockKernel(base + " -perf_config v2:32,32,8,16,16,16,1,1,1").kernel_name == \
+    assert rock.RockKernel(base + " -perf_config v2:48,48,8,16,16,16,1,1,1").kernel_name == \
         "rock_gemm_i8_256x256_fast"
+    # the split-K tile can be asked for by name as well
+    assert rock.RockKernel(base + " -perf_config v2:32,32,4,32,32,16,4,1,1").kernel_name == \
+        "rock_gemm_i8_32x32_splitk"
 
 
 def test_problem_keys_follow_reference_format(rock):

@@ -90,6 +90,19 @@ def test_gemm_every_tile_variant(rock, oracle, gpu, t, tile):
         assert np.array_equal(to_f32(out, od), ref)
 
 
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16", "i8", "fp8", "bf8"])
+@pytest.mark.parametrize("G,M,N,K", [(2, 96, 70, 1040), (1, 33, 31, 4096), (1, 512, 512, 512)])
+def test_gemm_split_k_over_waves(rock, oracle, gpu, t, G, M, N, K):
+    """Few output tiles and a long K: 32x32 tile per block, K divided over the
+    block's waves and summed through LDS (ragged M, N and K tail included)."""
+    out, od, ref = _run_case(rock, oracle, gpu, t, G, M, N, K, False, True, False, True, 15,
+                             perf_config="v2:32,32,4,32,32,16,4,1,1")
+    if t == "i8":
+        assert oracle.verify_int(out.cpu().numpy().ravel(), ref)[0] == 0
+    else:  # exact f32 sums, one rounding to the output type
+        assert np.array_equal(to_f32(out, od), oracle.round_through(ref, CODE[od]))
+
+
 @pytest.mark.parametrize("t", FLOAT_TYPES)
 def test_gemm_real_values_within_reference_gate(rock, oracle, gpu, t):
     out, od, ref = _run_case(rock, oracle, gpu, t, 2, 200, 136, 512, False, True, False, False, 11)
