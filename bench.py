@@ -198,6 +198,20 @@ def main():
                 "kernel": head["kernel"].kernel_name, "kernel_ms": round(kern_ms, 5),
                 "hbm_gbps_algorithmic": round(head["min_bytes"] / (kern_ms * 1e-3) / 1e9, 1)}
 
+    # what the matrix cores alone sustain on this box (register-only MFMA chains):
+    # with constant operands, and with random bit patterns (lower clocks, power)
+    rates = {}
+
+    def issue_rate(dt):
+        if dt not in rates:
+            rates[dt] = {"constant_operands": round(rock.mfma_rate(dt, False, stream), 1),
+                         "random_operands": round(rock.mfma_rate(dt, True, stream), 1)}
+        return rates[dt]
+
+    roofline["mfma_issue_rate_measured"] = issue_rate(head["dtype"])
+    roofline["frac_of_measured_random_operand_rate"] = round(
+        achieved / roofline["mfma_issue_rate_measured"]["random_operands"], 4)
+
     per_config = {}
     if not args.only_headline:
         for name, c in cfgs.items():
@@ -206,7 +220,8 @@ def main():
             tf = c["ops"] / (ms * 1e-3) / 1e12
             per_config[name] = {"kernel": c["kernel"].kernel_name, "kernel_ms": round(ms, 5),
                                 "tflops": round(tf, 2), "peak": c["peak"], "frac_of_mfma_peak": round(tf / c["peak"], 4),
-                                "hbm_gbps_algorithmic": round(c["min_bytes"] / (ms * 1e-3) / 1e9, 1)}
+                                "hbm_gbps_algorithmic": round(c["min_bytes"] / (ms * 1e-3) / 1e9, 1),
+                                "mfma_issue_rate_measured": issue_rate(c["dtype"])}
 
     cores = os.cpu_count() or 1
     threads = min(16, cores)  # the box's CPU share for one GPU

@@ -8,7 +8,7 @@ CPU or eager fallback: if the library is missing, importing the binding
 raises.
 """
 from .api import (RockError, RockKernel, attention, conv2d, gemm,  # noqa: F401
-                  library_path, load_library)
+                  library_path, load_library, mfma_rate)
 
 __all__ = ["RockError", "RockKernel", "gemm", "conv2d", "attention",
-           "library_path", "load_library"]
+           "library_path", "load_library", "mfma_rate"]

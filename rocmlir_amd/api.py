@@ -71,6 +71,9 @@ def load_library():
         L.rockamdBenchmark.restype = C.c_int
         L.rockamdBenchmark.argtypes = [vp, C.POINTER(vp), C.c_int, vp, C.c_int,
                                        C.c_int, C.POINTER(C.c_float)]
+        L.rockamdMeasureMfmaRate.restype = C.c_int
+        L.rockamdMeasureMfmaRate.argtypes = [C.c_int, C.c_int, vp,
+                                             C.POINTER(C.c_double)]
         L.rockamdGetLastError.restype = C.c_char_p
         L.rockamdGetLastError.argtypes = []
         _lib = L
@@ -79,6 +82,21 @@ def load_library():
 
 def last_error():
     return load_library().rockamdGetLastError().decode()
+
+
+_DTYPE_CODES = {"f32": 0, "f16": 1, "bf16": 2, "i8": 3, "fp8": 4}
+
+
+def mfma_rate(dtype, random_data=False, stream=None):
+    """Sustained 32x32 MFMA issue rate in TFLOP/s (TOP/s) on the current GPU
+    for operand type `dtype`, with constant or hashed operand bits."""
+    out = C.c_double(0)
+    rc = load_library().rockamdMeasureMfmaRate(
+        _DTYPE_CODES[dtype], int(bool(random_data)),
+        getattr(stream, "cuda_stream", stream), C.byref(out))
+    if rc != 0:
+        raise RockError("rate probe failed (hip error %d): %s" % (rc, last_error()))
+    return out.value
 
 
 class RockKernel:

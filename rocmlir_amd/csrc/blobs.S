@@ -20,4 +20,5 @@ rock_hsaco_\n\()_end:
     ROCK_BLOB gemm_fp8_bf8
     ROCK_BLOB gemm_bf8_fp8
     ROCK_BLOB attention
+    ROCK_BLOB probe
     .section .note.GNU-stack,"",@progbits

@@ -1034,6 +1034,72 @@ int rockamdBenchmark(MiirHandle handle, void *const *pointers, int num_pointers,
   return 0;
 }
 
+int rockamdMeasureMfmaRate(int dtype, int random_data, void *stream, double *tera_ops) {
+  static const char *names[] = {"f32", "f16", "bf16", "i8", "fp8"};
+  // multiply-accumulates of one 32x32xK instruction per operand type
+  static const double macs[] = {32 * 32 * 2 * 4.0, 32 * 32 * 16.0, 32 * 32 * 16.0, 32 * 32 * 32.0,
+                                32 * 32 * 64.0};
+  if (dtype < 0 || dtype > ROCK_FP8 || !tera_ops) {
+    set_error("rate probe: operand type must be f32, f16, bf16, i8 or fp8");
+    return (int)hipErrorInvalidValue;
+  }
+  const Blob *blob = find_blob("probe");
+  if (!blob)
+    return (int)hipErrorInvalidValue;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess)
+    return (int)e;
+  hipModule_t mod;
+  {
+    std::lock_guard<std::mutex> lock(g_module_mutex);
+    auto key = std::make_pair(dev, blob);
+    auto it = g_modules.find(key);
+    if (it == g_modules.end()) {
+      e = hipModuleLoadData(&mod, blob->start);
+      if (e != hipSuccess)
+        return (int)e;
+      g_modules[key] = mod;
+    } else {
+      mod = it->second;
+    }
+  }
+  hipFunction_t fn;
+  std::string kname = std::string("rock_probe_mfma_") + names[dtype];
+  e = hipModuleGetFunction(&fn, mod, kname.c_str());
+  if (e != hipSuccess)
+    return (int)e;
+  const int blocks = kNumCU * 4, threads = 256, iters = 40000;
+  float *out = nullptr;
+  e = hipMalloc((void **)&out, (size_t)blocks * threads * sizeof(float));
+  if (e != hipSuccess)
+    return (int)e;
+  hipStream_t s = (hipStream_t)stream;
+  int it = iters, rnd = random_data;
+  void *args[] = {&out, &it, &rnd};
+  hipEvent_t e0, e1;
+  hipEventCreate(&e0);
+  hipEventCreate(&e1);
+  int rc = (int)hipModuleLaunchKernel(fn, blocks, 1, 1, threads, 1, 1, 0, s, args, nullptr); // warm-up
+  if (rc == 0) rc = (int)hipEventRecord(e0, s);
+  if (rc == 0) rc = (int)hipModuleLaunchKernel(fn, blocks, 1, 1, threads, 1, 1, 0, s, args, nullptr);
+  if (rc == 0) rc = (int)hipEventRecord(e1, s);
+  if (rc == 0) rc = (int)hipEventSynchronize(e1);
+  float ms = 0.0f;
+  if (rc == 0) rc = (int)hipEventElapsedTime(&ms, e0, e1);
+  hipEventDestroy(e0);
+  hipEventDestroy(e1);
+  hipFree(out);
+  if (rc != 0) {
+    set_error(std::string("rate probe failed: ") + hipGetErrorString((hipError_t)rc));
+    return rc;
+  }
+  // 4 instructions per iteration per wave, 4 waves per block
+  double ops = 2.0 * macs[dtype] * 4.0 * iters * 4.0 * blocks;
+  *tera_ops = ops / (ms * 1e-3) / 1e12;
+  return 0;
+}
+
 const char *rockamdGetLastError(void) { return g_last_error.c_str(); }
 
 } // extern "C"

@@ -190,3 +190,15 @@ def test_fp8_output_saturates(rock, oracle, gpu):
     got = to_f32(out, "fp8")
     assert np.abs(ref * 100).max() > 448 and np.abs(got).max() == 448.0
     assert np.array_equal(got, want)
+
+
+def test_mfma_rate_probe(rock, gpu):
+    """The issue-rate probe runs and reports something physically sensible:
+    positive, not above the published dense peak by more than clock headroom,
+    and not faster on random operands than on constants."""
+    peak = {"i8": 5000.0, "fp8": 5000.0, "f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
+    for dt, pk in peak.items():
+        const = rock.mfma_rate(dt, False)
+        rnd = rock.mfma_rate(dt, True)
+        assert 0.2 * pk < const < 1.1 * pk, (dt, const)
+        assert 0.2 * pk < rnd <= const * 1.05, (dt, rnd, const)
