@@ -1,17 +1,18 @@
 // Fast path of the contraction kernel: operands stream global -> LDS without
-// passing through registers (buffer_load ... lds, 16 bytes per lane), four LDS
-// stages, so three K-steps of loads are in flight while one is multiplied.
+// passing through registers (buffer_load ... lds, 16 bytes per lane) into a
+// ring of LDS stages, so K-steps of loads are in flight while one is multiplied.
 //
 // Same tiling and MFMA mapping as the register-staged body in
 // gemm_conv_kernel.h (which remains for arbitrary strides); what differs:
 //
-//   * K advances 64 BYTES per stage; a stage holds BM + BN rows of four
-//     16-byte chunks.  One wave-wide load instruction fills a "slab" of 16
-//     rows (1 KiB, the 64 lanes' 16 bytes land back to back in LDS).
+//   * K advances RB = 64 or 128 BYTES per stage (four or two stages); a stage
+//     holds BM + BN rows of RB/16 sixteen-byte chunks.  One wave-wide load
+//     instruction fills a "slab" of 1 KiB (the 64 lanes' 16 bytes land back to
+//     back in LDS): 16 rows of 64 bytes or 8 rows of 128.
 //   * The XOR swizzle is applied on the source side: the lane that fills
-//     physical chunk p of row r fetches logical chunk p ^ ((r >> 2) & 3), so
-//     the 32 rows an MFMA operand reads at one chunk index fall into distinct
-//     bank groups.
+//     physical chunk p of row r fetches logical chunk p ^ swz(r), so the 32
+//     rows an MFMA operand reads at one chunk index fall into distinct bank
+//     groups.
 //   * Zero fill (rows past the end, the K tail, convolution padding) costs no
 //     instruction: such lanes use a byte offset beyond the buffer
 //     descriptor's range and the hardware writes zeros.  This is the
@@ -30,14 +31,27 @@
 
 namespace rk {
 
-constexpr int kDlRowBytes = 64;  // K bytes per row per stage
-constexpr int kDlChunks = 4;     // 16-byte chunks per row
-constexpr int kDlStages = 4;
 constexpr unsigned kOobOffset = 0x80000000u; // >= num_records: reads as zero
 
-typedef __attribute__((address_space(3))) void lds_void_t;
+// Stage geometry.  RB = K bytes per row per stage: 64 (four stages; the big
+// tiles, whose MFMA work per K-step already dwarfs the barrier) or 128 (two
+// stages; the small tiles, which halve their barrier count and fetch whole
+// 128-byte cache lines per row).  A wave-wide load always fills 1 KiB:
+// 1024 / RB rows.
+template <int RB> struct DlGeom {
+  static_assert(RB == 64 || RB == 128, "stage rows are 64 or 128 bytes");
+  static constexpr int CHUNKS = RB / 16;
+  static constexpr int SLAB_ROWS = 1024 / RB;
+  static constexpr int STAGES = RB == 64 ? 4 : 2;
+  // XOR swizzle: the 32 rows an MFMA operand reads at one chunk index must fall
+  // into distinct bank groups (row pitch 64 B: 4 rows per 256-byte bank period;
+  // 128 B: 2 rows per period)
+  static __device__ __forceinline__ int swz(int row) {
+    return RB == 64 ? ((row >> 2) & 3) : ((row >> 1) & 7);
+  }
+};
 
-__device__ __forceinline__ int dl_swz(int row) { return (row >> 2) & 3; }
+typedef __attribute__((address_space(3))) void lds_void_t;
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t dl_rsrc(const void *base) {
   // raw buffer, 2 GiB window, dword-typed data format word used by gfx9 parts
@@ -50,15 +64,17 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x0F70);
 }
 
-template <int ROWS, int NW> struct SlabGeom {
-  static constexpr int SLABS = ROWS / 16;
+template <int ROWS, int NW, int RB> struct SlabGeom {
+  static constexpr int SLABS = ROWS / DlGeom<RB>::SLAB_ROWS;
   static constexpr int PER_WAVE = SLABS / NW;
-  static_assert(ROWS % 16 == 0 && SLABS % NW == 0, "tile rows must split into 16-row slabs per wave");
+  static_assert(ROWS % DlGeom<RB>::SLAB_ROWS == 0 && SLABS % NW == 0,
+                "tile rows must split into 1 KiB slabs per wave");
 };
 
 // K-contiguous rows (GEMM operands, KYXC filters).
-template <int DT, int ROWS, int NW> struct RowsDl {
-  using Sg = SlabGeom<ROWS, NW>;
+template <int DT, int ROWS, int NW, int RB> struct RowsDl {
+  using Sg = SlabGeom<ROWS, NW, RB>;
+  using Dg = DlGeom<RB>;
   static constexpr int ES = MmaTraits<DT>::ES;
   __amdgpu_buffer_rsrc_t rsrc;
   unsigned off[Sg::PER_WAVE]; // byte offset of this lane's chunk at K-step 0, or kOobOffset
@@ -73,15 +89,15 @@ template <int DT, int ROWS, int NW> struct RowsDl {
     rsrc = dl_rsrc((const char *)base + (int64_t)row0 * row_stride * ES);
 #pragma unroll
     for (int i = 0; i < Sg::PER_WAVE; ++i) {
-      int r = (wave * Sg::PER_WAVE + i) * 16 + (lane >> 2);
-      kb[i] = ((lane & 3) ^ dl_swz(r)) * kChunk;
+      int r = (wave * Sg::PER_WAVE + i) * Dg::SLAB_ROWS + lane / Dg::CHUNKS;
+      kb[i] = ((lane % Dg::CHUNKS) ^ Dg::swz(r)) * kChunk;
       off[i] = (row0 + r < rows_total) ? (unsigned)(r * (int)row_stride * ES + kb[i]) : kOobOffset;
     }
   }
   __device__ __forceinline__ void issue(int kt, char *stage) {
 #pragma unroll
     for (int i = 0; i < Sg::PER_WAVE; ++i) {
-      int k0 = kt * kDlRowBytes;
+      int k0 = kt * RB;
       unsigned voff = (k0 + kb[i] < kbytes) ? off[i] + (unsigned)k0 : kOobOffset;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
           rsrc, (lds_void_t *)(stage + (wave * Sg::PER_WAVE + i) * 1024), 16, (int)voff, 0, 0, 0);
@@ -91,26 +107,40 @@ template <int DT, int ROWS, int NW> struct RowsDl {
 
 // Convolution input as implicit-GEMM rows: row m = (n, ho, wo), reduction
 // index (y, x, c) with c fastest; channel run is a whole number of chunks.
-template <int DT, int ROWS, int NW> struct ConvInDl {
-  using Sg = SlabGeom<ROWS, NW>;
+//
+// When the channel run is also a whole number of K-steps (RB bytes), every lane
+// of a K-step sits in the same filter tap: the tap walk is scalar state, the
+// per-lane work of a step is one add, and the (hi, wi) bounds test runs once
+// per tap.  Otherwise each lane tracks the tap of its own chunk.
+template <int DT, int ROWS, int NW, int RB> struct ConvInDl {
+  using Sg = SlabGeom<ROWS, NW, RB>;
+  using Dg = DlGeom<RB>;
   static constexpr int ES = MmaTraits<DT>::ES;
   static constexpr int EPC = kChunk / ES;
-  static constexpr int BKE = kDlRowBytes / ES;
+  static constexpr int BKE = RB / ES;
   __amdgpu_buffer_rsrc_t rsrc;
   const RockConvParams *p;
   unsigned pix[Sg::PER_WAVE]; // byte offset of input(n, g, 0, 0, 0), or kOobOffset for rows past M
   int h0[Sg::PER_WAVE], w0[Sg::PER_WAVE];
+  // per-lane tap state (general case)
   int y[Sg::PER_WAVE], x[Sg::PER_WAVE], cc[Sg::PER_WAVE];
+  // uniform tap state (channel run = whole K-steps)
+  unsigned tapoff[Sg::PER_WAVE]; // byte offset of this lane's chunk at channel 0 of the tap, or OOB
+  int kb[Sg::PER_WAVE];
+  int uy, ux, uc0;               // tap and byte offset of the K-step inside the channel run
+  bool uniform;
   int wave;
 
   __device__ __forceinline__ void init(const void *in, const RockConvParams &cp, int g, int row0,
                                        int wave_, int lane) {
     p = &cp;
     wave = wave_;
+    uniform = (cp.c * ES) % RB == 0;
+    uy = ux = uc0 = 0;
     rsrc = dl_rsrc((const char *)in + (int64_t)g * cp.in_gs * ES);
 #pragma unroll
     for (int i = 0; i < Sg::PER_WAVE; ++i) {
-      int r = (wave * Sg::PER_WAVE + i) * 16 + (lane >> 2);
+      int r = (wave * Sg::PER_WAVE + i) * Dg::SLAB_ROWS + lane / Dg::CHUNKS;
       int m = row0 + r;
       int mm = min(m, cp.M - 1);
       int n = mm / (cp.ho * cp.wo);
@@ -120,16 +150,43 @@ template <int DT, int ROWS, int NW> struct ConvInDl {
       h0[i] = ho * cp.stride_h - cp.pad_h;
       w0[i] = wo * cp.stride_w - cp.pad_w;
       pix[i] = (m < cp.M) ? (unsigned)(n * (int)cp.in_ns * ES) : kOobOffset;
-      int k0 = ((lane & 3) ^ dl_swz(r)) * EPC;
+      int lc = (lane % Dg::CHUNKS) ^ Dg::swz(r);
+      kb[i] = lc * kChunk;
+      int k0 = lc * EPC;
       int tap = k0 / cp.c;
       cc[i] = k0 - tap * cp.c;
       y[i] = tap / cp.x;
       x[i] = tap - y[i] * cp.x;
+      tapoff[i] = kOobOffset;
     }
   }
   // must be called with kt = 0, 1, 2, ... in order (tap state advances)
   __device__ __forceinline__ void issue(int kt, char *stage) {
     (void)kt;
+    if (uniform) {
+      if (uc0 == 0) { // entering a tap: one bounds test per row
+        const int dh = uy * p->dil_h, dw = ux * p->dil_w;
+        const bool tap_ok = uy < p->y;
+#pragma unroll
+        for (int i = 0; i < Sg::PER_WAVE; ++i) {
+          int hi = h0[i] + dh, wi = w0[i] + dw;
+          bool v = tap_ok && pix[i] != kOobOffset && hi >= 0 && hi < p->hi && wi >= 0 && wi < p->wi;
+          tapoff[i] = v ? pix[i] + (unsigned)((hi * (int)p->in_hs + wi * (int)p->in_ws) * ES + kb[i])
+                        : kOobOffset;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < Sg::PER_WAVE; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rsrc, (lds_void_t *)(stage + (wave * Sg::PER_WAVE + i) * 1024), 16,
+            (int)(tapoff[i] + (unsigned)uc0), 0, 0, 0); // OOB + small stays out of range
+      uc0 += RB;
+      if (uc0 == p->c * ES) {
+        uc0 = 0;
+        if (++ux == p->x) { ux = 0; ++uy; }
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < Sg::PER_WAVE; ++i) {
       int hi = h0[i] + y[i] * p->dil_h, wi = w0[i] + x[i] * p->dil_w;
@@ -147,48 +204,48 @@ template <int DT, int ROWS, int NW> struct ConvInDl {
   }
 };
 
-template <int DT, int ROWS, int NW, int KIND>
+template <int DT, int ROWS, int NW, int RB, int KIND>
 __device__ __forceinline__ auto make_dl_a(const void *A, const RockGemmParams &p, int g, int m0, int wave, int lane) {
   static_assert(KIND == LD_ROWS_FAST, "GEMM fast path loads K-contiguous rows");
-  RowsDl<DT, ROWS, NW> l;
+  RowsDl<DT, ROWS, NW, RB> l;
   l.init((const char *)A + (int64_t)g * p.a_gs * MmaTraits<DT>::ES, p.a_ms, m0, p.M, p.K, wave, lane);
   return l;
 }
-template <int DT, int ROWS, int NW, int KIND>
+template <int DT, int ROWS, int NW, int RB, int KIND>
 __device__ __forceinline__ auto make_dl_b(const void *B, const RockGemmParams &p, int g, int n0, int wave, int lane) {
-  RowsDl<DT, ROWS, NW> l;
+  RowsDl<DT, ROWS, NW, RB> l;
   l.init((const char *)B + (int64_t)g * p.b_gs * MmaTraits<DT>::ES, p.b_ns, n0, p.N, p.K, wave, lane);
   return l;
 }
-template <int DT, int ROWS, int NW, int KIND>
+template <int DT, int ROWS, int NW, int RB, int KIND>
 __device__ __forceinline__ auto make_dl_a(const void *in, const RockConvParams &p, int g, int m0, int wave, int lane) {
   static_assert(KIND == LD_CONV_IN_FAST, "convolution fast path gathers channel-contiguous input");
-  ConvInDl<DT, ROWS, NW> l;
+  ConvInDl<DT, ROWS, NW, RB> l;
   l.init(in, p, g, m0, wave, lane);
   return l;
 }
-template <int DT, int ROWS, int NW, int KIND>
+template <int DT, int ROWS, int NW, int RB, int KIND>
 __device__ __forceinline__ auto make_dl_b(const void *fil, const RockConvParams &p, int g, int n0, int wave, int lane) {
-  RowsDl<DT, ROWS, NW> l;
+  RowsDl<DT, ROWS, NW, RB> l;
   l.init((const char *)fil + (int64_t)g * p.fil_gs * MmaTraits<DT>::ES, p.fil_ks, n0, p.N, p.K, wave, lane);
   return l;
 }
 
-// Fragment of one 32-row block out of a 64-byte-row stage: lane (row = lane % 32,
+// Fragment of one 32-row block out of a stage: lane (row = lane % 32,
 // half = lane / 32) takes chunk  step*2*CHUNKS + 2*c + half  for c in [0, CHUNKS).
-template <int DT>
+template <int DT, int RB>
 __device__ __forceinline__ Frag<DT> dl_read_frag(const char *lds, int row, int step, int half) {
   Frag<DT> f;
   constexpr int CH = MmaTraits<DT>::CHUNKS;
 #pragma unroll
   for (int c = 0; c < CH; ++c) {
     int chunk = step * 2 * CH + 2 * c + half;
-    f.c[c] = *(const v4i *)(lds + row * kDlRowBytes + ((chunk ^ dl_swz(row)) * kChunk));
+    f.c[c] = *(const v4i *)(lds + row * RB + ((chunk ^ DlGeom<RB>::swz(row)) * kChunk));
   }
   return f;
 }
 
-template <int DT, int BM, int BN, int WAVES_M, int WAVES_N, int LDA, int LDB, typename Params>
+template <int DT, int BM, int BN, int WAVES_M, int WAVES_N, int RB, int LDA, int LDB, typename Params>
 __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void *Bptr, void *Cptr,
                                                     const void *aux, const Params &p) {
   using Tr = MmaTraits<DT>;
@@ -196,10 +253,11 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N; // wave tile
   constexpr int MI = WTM / 32, NI = WTN / 32;
-  constexpr int STEPS = kDlChunks / (2 * Tr::CHUNKS); // MFMA K steps per stage
-  constexpr int A_BYTES = BM * kDlRowBytes, B_BYTES = BN * kDlRowBytes;
+  constexpr int kDlStages = DlGeom<RB>::STAGES;
+  constexpr int STEPS = DlGeom<RB>::CHUNKS / (2 * Tr::CHUNKS); // MFMA K steps per stage
+  constexpr int A_BYTES = BM * RB, B_BYTES = BN * RB;
   constexpr int STAGE = A_BYTES + B_BYTES;
-  constexpr int BKE = kDlRowBytes / Tr::ES;
+  constexpr int BKE = RB / Tr::ES;
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of 32");
 
   __shared__ __attribute__((aligned(1024))) char lds[kDlStages * STAGE];
@@ -214,9 +272,9 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
   decode_block(p.tiles_m, p.tiles_n, p_batch(p), p.group_m, p.xcd_remap, g, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
-  auto la = make_dl_a<DT, BM, NW, LDA>(Aptr, p, g, m0, wave, lane);
-  auto lb = make_dl_b<DT, BN, NW, LDB>(Bptr, p, g, n0, wave, lane);
-  constexpr int LOADS_PER_STEP = SlabGeom<BM, NW>::PER_WAVE + SlabGeom<BN, NW>::PER_WAVE;
+  auto la = make_dl_a<DT, BM, NW, RB, LDA>(Aptr, p, g, m0, wave, lane);
+  auto lb = make_dl_b<DT, BN, NW, RB, LDB>(Bptr, p, g, n0, wave, lane);
+  constexpr int LOADS_PER_STEP = SlabGeom<BM, NW, RB>::PER_WAVE + SlabGeom<BN, NW, RB>::PER_WAVE;
 
   Acc acc[MI][NI];
 #pragma unroll
@@ -254,10 +312,10 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
       Frag<DT> fb[NI];
 #pragma unroll
       for (int j = 0; j < NI; ++j)
-        fb[j] = dl_read_frag<DT>(sb, wn * WTN + j * 32 + lrow, s, lgrp);
+        fb[j] = dl_read_frag<DT, RB>(sb, wn * WTN + j * 32 + lrow, s, lgrp);
 #pragma unroll
       for (int i = 0; i < MI; ++i) {
-        Frag<DT> fa = dl_read_frag<DT>(sa, wm * WTM + i * 32 + lrow, s, lgrp);
+        Frag<DT> fa = dl_read_frag<DT, RB>(sa, wm * WTM + i * 32 + lrow, s, lgrp);
 #pragma unroll
         for (int j = 0; j < NI; ++j)
           mma32x32<DT>(fb[j], fa, acc[i][j]);

@@ -26,25 +26,25 @@
   }
 
 // fast variants: direct-to-LDS loads, K-contiguous 16-byte aligned operands
-#define RK_GEMM_DL(NAME, BM, BN, WM, WN)                                                \
+#define RK_GEMM_DL(NAME, BM, BN, WM, WN, RB)                                             \
   extern "C" __global__ __launch_bounds__(WM *WN * 64) void RK_CAT(                     \
       RK_CAT(rock_gemm_, ROCK_DTNAME), NAME)(const void *A, const void *B, void *C,     \
                                              const void *aux, RockGemmParams p) {       \
-    rk::contraction_body_dl<ROCK_DT, BM, BN, WM, WN, rk::LD_ROWS_FAST, rk::LD_ROWS_FAST>(\
+    rk::contraction_body_dl<ROCK_DT, BM, BN, WM, WN, RB, rk::LD_ROWS_FAST, rk::LD_ROWS_FAST>(\
         A, B, C, aux, p);                                                               \
   }
-#define RK_CONV_DL(NAME, BM, BN, WM, WN)                                                \
+#define RK_CONV_DL(NAME, BM, BN, WM, WN, RB)                                             \
   extern "C" __global__ __launch_bounds__(WM *WN * 64) void RK_CAT(                     \
       RK_CAT(rock_conv_, ROCK_DTNAME), NAME)(const void *fil, const void *in, void *out,\
                                              const void *aux, RockConvParams p) {       \
-    rk::contraction_body_dl<ROCK_DT, BM, BN, WM, WN, rk::LD_CONV_IN_FAST,               \
+    rk::contraction_body_dl<ROCK_DT, BM, BN, WM, WN, RB, rk::LD_CONV_IN_FAST,           \
                             rk::LD_ROWS_FAST>(in, fil, out, aux, p);                    \
   }
 
-RK_GEMM_DL(_256x256_fast, 256, 256, 2, 4)
-RK_GEMM_DL(_256x128_fast, 256, 128, 4, 2)
-RK_GEMM_DL(_128x128_fast, 128, 128, 2, 2)
-RK_GEMM_DL(_64x64_fast, 64, 64, 2, 2)
+RK_GEMM_DL(_256x256_fast, 256, 256, 2, 4, 64)
+RK_GEMM_DL(_256x128_fast, 256, 128, 4, 2, 64)
+RK_GEMM_DL(_128x128_fast, 128, 128, 2, 2, 128)
+RK_GEMM_DL(_64x64_fast, 64, 64, 2, 2, 128)
 RK_GEMM(_64x64_generic, 64, 64, 2, 2, rk::LD_ROWS_GENERIC, rk::LD_ROWS_GENERIC)
 
 // small outputs: 32x32 tile per block, K split over the block's four waves
@@ -54,8 +54,8 @@ extern "C" __global__ __launch_bounds__(256) void RK_CAT(RK_CAT(rock_gemm_, ROCK
 }
 
 #if ROCK_DT != 7 && ROCK_DT != 8
-RK_CONV_DL(_256x128_fast, 256, 128, 4, 2)
-RK_CONV_DL(_128x128_fast, 128, 128, 2, 2)
-RK_CONV_DL(_64x64_fast, 64, 64, 2, 2)
+RK_CONV_DL(_256x128_fast, 256, 128, 4, 2, 64)
+RK_CONV_DL(_128x128_fast, 128, 128, 2, 2, 128)
+RK_CONV_DL(_64x64_fast, 64, 64, 2, 2, 128)
 RK_CONV(_64x64_generic, 64, 64, 2, 2, rk::LD_CONV_IN_GENERIC, rk::LD_CONV_FIL_GENERIC)
 #endif

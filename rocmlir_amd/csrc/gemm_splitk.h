@@ -26,11 +26,13 @@ __device__ __forceinline__ void gemm_body_splitk(const void *Aptr, const void *B
   using Acc = typename Tr::Acc;
   constexpr int T = 32;      // output tile edge
   constexpr int NWAVE = 4;   // K split
-  constexpr int STEPS = kDlChunks / (2 * Tr::CHUNKS);
-  constexpr int A_BYTES = T * kDlRowBytes, STAGE = 2 * A_BYTES; // per wave
+  constexpr int RB = 64;     // K bytes per row per stage
+  constexpr int kDlStages = DlGeom<RB>::STAGES;
+  constexpr int STEPS = DlGeom<RB>::CHUNKS / (2 * Tr::CHUNKS);
+  constexpr int A_BYTES = T * RB, STAGE = 2 * A_BYTES; // per wave
   constexpr int WAVE_LDS = kDlStages * STAGE;
-  constexpr int BKE = kDlRowBytes / Tr::ES;
-  constexpr int LOADS_PER_STEP = 2 * SlabGeom<T, 1>::PER_WAVE;
+  constexpr int BKE = RB / Tr::ES;
+  constexpr int LOADS_PER_STEP = 2 * SlabGeom<T, 1, RB>::PER_WAVE;
   static_assert(WAVE_LDS >= 16 * 64 * 4, "a wave's stages must hold its partial tile");
 
   __shared__ __attribute__((aligned(1024))) char lds[NWAVE * WAVE_LDS];
@@ -47,7 +49,7 @@ __device__ __forceinline__ void gemm_body_splitk(const void *Aptr, const void *B
 
   // every wave loads whole 32-row operand tiles for its own K-steps: the
   // loaders are told they are "wave 0 of 1"
-  RowsDl<DT, T, 1> la, lb;
+  RowsDl<DT, T, 1, RB> la, lb;
   la.init((const char *)Aptr + (int64_t)g * p.a_gs * Tr::ES, p.a_ms, m0, p.M, p.K, 0, lane);
   lb.init((const char *)Bptr + (int64_t)g * p.b_gs * Tr::ES, p.b_ns, n0, p.N, p.K, 0, lane);
 
@@ -78,8 +80,8 @@ __device__ __forceinline__ void gemm_body_splitk(const void *Aptr, const void *B
     const char *sb = sa + A_BYTES;
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
-      Frag<DT> fb = dl_read_frag<DT>(sb, lrow, s, lgrp);
-      Frag<DT> fa = dl_read_frag<DT>(sa, lrow, s, lgrp);
+      Frag<DT> fb = dl_read_frag<DT, RB>(sb, lrow, s, lgrp);
+      Frag<DT> fa = dl_read_frag<DT, RB>(sa, lrow, s, lgrp);
       mma32x32<DT>(fb, fa, acc);
     }
   }
