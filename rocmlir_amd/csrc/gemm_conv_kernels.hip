@@ -41,8 +41,8 @@
                             rk::LD_ROWS_FAST>(in, fil, out, aux, p);                    \
   }
 
-RK_GEMM_DL(_256x256_fast, 256, 256, 2, 4, 64)
-RK_GEMM_DL(_256x128_fast, 256, 128, 4, 2, 64)
+RK_GEMM_DL(_256x256_fast, 256, 256, 2, 4, 128)
+RK_GEMM_DL(_256x128_fast, 256, 128, 4, 2, 128)
 RK_GEMM_DL(_128x128_fast, 128, 128, 2, 2, 128)
 RK_GEMM_DL(_64x64_fast, 64, 64, 2, 2, 128)
 RK_GEMM(_64x64_generic, 64, 64, 2, 2, rk::LD_ROWS_GENERIC, rk::LD_ROWS_GENERIC)
@@ -54,7 +54,7 @@ extern "C" __global__ __launch_bounds__(256) void RK_CAT(RK_CAT(rock_gemm_, ROCK
 }
 
 #if ROCK_DT != 7 && ROCK_DT != 8
-RK_CONV_DL(_256x128_fast, 256, 128, 4, 2, 64)
+RK_CONV_DL(_256x128_fast, 256, 128, 4, 2, 128)
 RK_CONV_DL(_128x128_fast, 128, 128, 2, 2, 128)
 RK_CONV_DL(_64x64_fast, 64, 64, 2, 2, 128)
 RK_CONV(_64x64_generic, 64, 64, 2, 2, rk::LD_CONV_IN_GENERIC, rk::LD_CONV_FIL_GENERIC)

@@ -296,7 +296,7 @@ void apply_tile_grid(const Tile &t, int64_t M, int64_t N, int G, int &tiles_m, i
 std::string perf_string(const Tile &t, int es) {
   // v2:MPB,NPB,KpackPB,MPW,MnPerXdl,Kpack,splitK,forceUnroll,1
   int kpack = 16 / es;
-  int kpack_per_block = 128 / 16;
+  int kpack_per_block = 128 / 16; // 128 K bytes per stage row, 16-byte chunks
   char buf[96];
   std::snprintf(buf, sizeof buf, "v2:%d,%d,%d,%d,%d,%d,1,1,1", t.bm, t.bn, kpack_per_block,
                 t.bm / t.waves_m, 16, kpack);
