@@ -1,6 +1,10 @@
-// Tiled MFMA contraction kernel for gfx950: GEMM and implicit-GEMM forward
-// convolution share one main loop and differ only in how a tile row is
-// addressed in global memory.
+// Tiled MFMA contraction kernel for gfx950, general-layout body: GEMM and
+// implicit-GEMM forward convolution share one main loop and differ only in
+// how a tile row is addressed in global memory.  This body gathers operands
+// element by element, so it takes ANY strides (all transposes, NCHW, odd K,
+// unaligned rows); operands made of K-contiguous 16-byte chunks take the
+// direct-to-LDS body in gemm_conv_dlds.h instead, which shares the tile
+// decode, the MFMA mapping and the epilogue defined here.
 //
 // Behaviour replaced: the reference's gridwise GEMM schedule
 // (mlir/lib/Dialect/Rock/Transforms/GridwiseGemmToBlockwise.cpp:2409-2811)
@@ -11,11 +15,11 @@
 //     element type (128 int8/fp8, 64 f16/bf16, 32 f32 elements);
 //   * global -> registers -> LDS, two LDS stages, one barrier per iteration;
 //   * LDS tile = rows of 8 sixteen-byte chunks, chunk index XOR-swizzled with
-//     the row so that the 16 lanes of an MFMA row group hit 16 distinct
-//     16-byte bank groups;
+//     the row so that the 32 rows an MFMA operand reads at one chunk index
+//     hit distinct 16-byte bank groups;
 //   * the problem's B rows feed the MFMA row operand and its A rows the
 //     column operand, so every lane ends up with 4 CONSECUTIVE n of one m and
-//     the C tile is written with 8/16-byte stores;
+//     the C tile is written with 4/8/16-byte stores;
 //   * out-of-range rows and the K tail are zero-filled on load, never read
 //     past the tensor; the epilogue (scale, zero point, bias, cast) runs on
 //     the accumulators in registers.
@@ -26,9 +30,9 @@
 namespace rk {
 
 enum LoaderKind : int {
-  LD_ROWS_FAST = 0,     // K-contiguous rows, 16-byte aligned chunks
+  LD_ROWS_FAST = 0,     // K-contiguous rows, 16-byte aligned chunks (direct-to-LDS body)
   LD_ROWS_GENERIC = 1,  // arbitrary element strides, element-wise
-  LD_CONV_IN_FAST = 2,  // convolution input, channel-contiguous, C*ES % 16 == 0
+  LD_CONV_IN_FAST = 2,  // convolution input, channel-contiguous, C*ES % 16 == 0 (direct-to-LDS body)
   LD_CONV_IN_GENERIC = 3,
   LD_CONV_FIL_GENERIC = 4
 };
@@ -81,48 +85,6 @@ template <int DT, int ROWS, int NT> struct TileGeom {
   static constexpr int NCH = (TOTAL + NT - 1) / NT;
   static constexpr int ROW_STEP = NT / kChunksPerRow;
   static_assert(NT % kChunksPerRow == 0, "thread count must be a multiple of 8");
-};
-
-// K-contiguous rows: base + row * row_stride, chunk at byte kt*128 + c*16.
-// Rows past the end are clamped to the last row: they only feed accumulators
-// of outputs that are never stored.  The K tail must be zero; that fix-up is
-// deferred to just before the LDS store so that the wait for the global loads
-// does not sit in front of the MFMA section.
-template <int DT, int ROWS, int NT> struct RowsFast {
-  using Gm = TileGeom<DT, ROWS, NT>;
-  const char *ptr[Gm::NCH];
-  int kbytes;
-  int c;
-  bool kin;
-
-  __device__ __forceinline__ void init(const void *base, int64_t row_stride,
-                                       int row0, int rows_total, int K,
-                                       int tid) {
-    c = tid & 7;
-    kbytes = K * Gm::ES;
-    kin = true;
-#pragma unroll
-    for (int i = 0; i < Gm::NCH; ++i) {
-      int r = (tid >> 3) + i * Gm::ROW_STEP;
-      int cr = min(row0 + r, rows_total - 1);
-      ptr[i] = (const char *)base + (int64_t)cr * row_stride * Gm::ES;
-    }
-  }
-  __device__ __forceinline__ void load(int kt, v4i (&regs)[Gm::NCH]) {
-    int off = kt * kRowBytes + c * kChunk;
-    kin = off < kbytes; // kbytes is a multiple of 16 on this path
-    int coff = kin ? off : 0;
-#pragma unroll
-    for (int i = 0; i < Gm::NCH; ++i)
-      regs[i] = *(const v4i *)(ptr[i] + coff);
-  }
-  __device__ __forceinline__ void fixup(v4i (&regs)[Gm::NCH]) const {
-    if (!kin) {
-#pragma unroll
-      for (int i = 0; i < Gm::NCH; ++i)
-        regs[i] = v4i{0, 0, 0, 0};
-    }
-  }
 };
 
 // Assemble one chunk element by element through a caller-supplied fetch.
@@ -182,75 +144,6 @@ template <int DT, int ROWS, int NT> struct RowsGeneric {
       });
     }
   }
-  __device__ __forceinline__ void fixup(v4i (&)[Gm::NCH]) const {}
-};
-
-// Convolution input as the implicit-GEMM A operand: row m = (n, ho, wo),
-// reduction index = (y, x, c) with c fastest.  Channel-contiguous input whose
-// channel run is a whole number of chunks, so a chunk never straddles a tap.
-template <int DT, int ROWS, int NT> struct ConvInFast {
-  using Gm = TileGeom<DT, ROWS, NT>;
-  const char *pix[Gm::NCH]; // input(n, g, c=0, 0, 0)
-  int h0[Gm::NCH], w0[Gm::NCH];
-  bool ok[Gm::NCH];
-  const RockConvParams *p;
-  int y, x, cc; // tap and channel offset of this thread's chunk at tile kt
-  int K;
-  uint32_t valid; // bit i: chunk i of the tile just loaded is inside the image
-
-  __device__ __forceinline__ void init(const void *in, const RockConvParams &cp,
-                                       int g, int row0, int tid) {
-    p = &cp;
-    K = cp.K;
-    const int c = tid & 7;
-    int k0 = c * Gm::EPC;
-    int tap = k0 / cp.c;
-    cc = k0 - tap * cp.c;
-    y = tap / cp.x;
-    x = tap - y * cp.x;
-#pragma unroll
-    for (int i = 0; i < Gm::NCH; ++i) {
-      int r = (tid >> 3) + i * Gm::ROW_STEP;
-      int m = row0 + r;
-      ok[i] = (r < ROWS) && (m < cp.M);
-      int mm = min(m, cp.M - 1);
-      int n = mm / (cp.ho * cp.wo);
-      int rem = mm - n * (cp.ho * cp.wo);
-      int ho = rem / cp.wo;
-      int wo = rem - ho * cp.wo;
-      h0[i] = ho * cp.stride_h - cp.pad_h;
-      w0[i] = wo * cp.stride_w - cp.pad_w;
-      pix[i] = (const char *)in + ((int64_t)n * cp.in_ns + (int64_t)g * cp.in_gs) * Gm::ES;
-    }
-  }
-  // must be called with kt = 0, 1, 2, ... in order (tap state advances)
-  __device__ __forceinline__ void load(int kt, v4i (&regs)[Gm::NCH]) {
-    const int k0 = kt * Gm::BKE + (threadIdx.x & 7) * Gm::EPC;
-    const bool kin = k0 < K;
-    const int dh = y * p->dil_h, dw = x * p->dil_w;
-    uint32_t vm = 0;
-#pragma unroll
-    for (int i = 0; i < Gm::NCH; ++i) {
-      int hi = h0[i] + dh, wi = w0[i] + dw;
-      bool v = kin && ok[i] && hi >= 0 && hi < p->hi && wi >= 0 && wi < p->wi;
-      int64_t off = v ? ((int64_t)hi * p->in_hs + (int64_t)wi * p->in_ws + cc) * Gm::ES : 0;
-      regs[i] = *(const v4i *)(pix[i] + off);
-      vm |= (v ? 1u : 0u) << i;
-    }
-    valid = vm;
-    // advance to the next tile's tap
-    cc += Gm::BKE;
-    while (cc >= p->c) {
-      cc -= p->c;
-      if (++x == p->x) { x = 0; ++y; }
-    }
-  }
-  // padding taps and the K tail become zeros (applied right before the LDS store)
-  __device__ __forceinline__ void fixup(v4i (&regs)[Gm::NCH]) const {
-#pragma unroll
-    for (int i = 0; i < Gm::NCH; ++i)
-      regs[i] = ((valid >> i) & 1u) ? regs[i] : v4i{0, 0, 0, 0};
-  }
 };
 
 // Decompose the reduction index for the generic convolution loaders.
@@ -305,7 +198,6 @@ template <int DT, int ROWS, int NT> struct ConvInGeneric {
       });
     }
   }
-  __device__ __forceinline__ void fixup(v4i (&)[Gm::NCH]) const {}
 };
 
 template <int DT, int ROWS, int NT> struct ConvFilGeneric {
@@ -336,7 +228,6 @@ template <int DT, int ROWS, int NT> struct ConvFilGeneric {
       });
     }
   }
-  __device__ __forceinline__ void fixup(v4i (&)[Gm::NCH]) const {}
 };
 
 // ---------------------------------------------------------------------------
@@ -533,52 +424,32 @@ __device__ __forceinline__ bool out_rows_chunk_aligned(const RockConvParams &p, 
 
 template <int DT, int ROWS, int NT, int KIND>
 __device__ __forceinline__ auto make_loader_a(const void *A, const RockGemmParams &p, int g, int m0, int tid) {
-  if constexpr (KIND == LD_ROWS_FAST) {
-    RowsFast<DT, ROWS, NT> l;
-    l.init((const char *)A + (int64_t)g * p.a_gs * MmaTraits<DT>::ES, p.a_ms, m0, p.M, p.K, tid);
-    return l;
-  } else {
-    RowsGeneric<DT, ROWS, NT> l;
-    l.init((const char *)A + (int64_t)g * p.a_gs * MmaTraits<DT>::ES, p.a_ms, p.a_ks, m0, p.M, p.K, tid);
-    return l;
-  }
+  static_assert(KIND == LD_ROWS_GENERIC, "K-contiguous operands take the direct-to-LDS body");
+  RowsGeneric<DT, ROWS, NT> l;
+  l.init((const char *)A + (int64_t)g * p.a_gs * MmaTraits<DT>::ES, p.a_ms, p.a_ks, m0, p.M, p.K, tid);
+  return l;
 }
 template <int DT, int ROWS, int NT, int KIND>
 __device__ __forceinline__ auto make_loader_b(const void *B, const RockGemmParams &p, int g, int n0, int tid) {
-  if constexpr (KIND == LD_ROWS_FAST) {
-    RowsFast<DT, ROWS, NT> l;
-    l.init((const char *)B + (int64_t)g * p.b_gs * MmaTraits<DT>::ES, p.b_ns, n0, p.N, p.K, tid);
-    return l;
-  } else {
-    RowsGeneric<DT, ROWS, NT> l;
-    l.init((const char *)B + (int64_t)g * p.b_gs * MmaTraits<DT>::ES, p.b_ns, p.b_ks, n0, p.N, p.K, tid);
-    return l;
-  }
+  static_assert(KIND == LD_ROWS_GENERIC, "K-contiguous operands take the direct-to-LDS body");
+  RowsGeneric<DT, ROWS, NT> l;
+  l.init((const char *)B + (int64_t)g * p.b_gs * MmaTraits<DT>::ES, p.b_ns, p.b_ks, n0, p.N, p.K, tid);
+  return l;
 }
 // convolution: "A" is the input image (implicit rows), "B" the filter
 template <int DT, int ROWS, int NT, int KIND>
 __device__ __forceinline__ auto make_loader_a(const void *in, const RockConvParams &p, int g, int m0, int tid) {
-  if constexpr (KIND == LD_CONV_IN_FAST) {
-    ConvInFast<DT, ROWS, NT> l;
-    l.init(in, p, g, m0, tid);
-    return l;
-  } else {
-    ConvInGeneric<DT, ROWS, NT> l;
-    l.init(in, p, g, m0, tid);
-    return l;
-  }
+  static_assert(KIND == LD_CONV_IN_GENERIC, "channel-contiguous input takes the direct-to-LDS body");
+  ConvInGeneric<DT, ROWS, NT> l;
+  l.init(in, p, g, m0, tid);
+  return l;
 }
 template <int DT, int ROWS, int NT, int KIND>
 __device__ __forceinline__ auto make_loader_b(const void *fil, const RockConvParams &p, int g, int n0, int tid) {
-  if constexpr (KIND == LD_ROWS_FAST) {
-    RowsFast<DT, ROWS, NT> l;
-    l.init((const char *)fil + (int64_t)g * p.fil_gs * MmaTraits<DT>::ES, p.fil_ks, n0, p.N, p.K, tid);
-    return l;
-  } else {
-    ConvFilGeneric<DT, ROWS, NT> l;
-    l.init(fil, p, g, n0, tid);
-    return l;
-  }
+  static_assert(KIND == LD_CONV_FIL_GENERIC, "K-contiguous filters take the direct-to-LDS body");
+  ConvFilGeneric<DT, ROWS, NT> l;
+  l.init(fil, p, g, n0, tid);
+  return l;
 }
 
 // Epilogue straight from the accumulator layout: the lane owns rows
@@ -658,8 +529,6 @@ __device__ __forceinline__ void contraction_body(const void *Aptr, const void *B
 
   la.load(0, ra);
   lb.load(0, rb);
-  la.fixup(ra);
-  lb.fixup(rb);
   store_tile<DT, BM, NT>(lds, ra, tid);
   store_tile<DT, BN, NT>(lds + A_BYTES, rb, tid);
   __syncthreads();
@@ -689,8 +558,6 @@ __device__ __forceinline__ void contraction_body(const void *Aptr, const void *B
     }
     if (more) {
       char *da = lds + (cur ^ 1) * (A_BYTES + B_BYTES);
-      la.fixup(ra);
-      lb.fixup(rb);
       store_tile<DT, BM, NT>(da, ra, tid);
       store_tile<DT, BN, NT>(da + A_BYTES, rb, tid);
     }
