@@ -62,8 +62,9 @@ template <int D, bool IS_V> struct AttnTileLoader {
   using Gm = AttnTileGeom<D>;
   const char *base;
   unsigned off[Gm::PER_WAVE]; // byte offset inside a tile, or kAttnOob for head-dim padding
-  int row[Gm::PER_WAVE];
+  int row0;                   // tile row of this lane's first chunk; chunk i is ROWS_PER_SLAB*i further
   int pitch_b, rows_total, wave;
+  static constexpr int ROWS_PER_SLAB = 64 / Gm::CPR;
 
   __device__ __forceinline__ void init(const uint16_t *base_, int64_t row_stride, int rows, int d,
                                        int wave_, int lane) {
@@ -76,7 +77,8 @@ template <int D, bool IS_V> struct AttnTileLoader {
       int c = (wave * Gm::PER_WAVE + i) * 64 + lane; // physical chunk inside the tile
       int r = c / Gm::CPR, pc = c - r * Gm::CPR;
       int lc = pc ^ attn_swz<Gm::CPR, IS_V>(r);
-      row[i] = r;
+      if (i == 0)
+        row0 = r;
       off[i] = (lc * 8 < d) ? (unsigned)(r * pitch_b + lc * 16) : kAttnOob;
     }
   }
@@ -88,7 +90,7 @@ template <int D, bool IS_V> struct AttnTileLoader {
     const int left = rows_total - key0; // rows of this tile that exist (may be <= 0)
 #pragma unroll
     for (int i = 0; i < Gm::PER_WAVE; ++i) {
-      unsigned voff = (row[i] < left) ? off[i] : kAttnOob;
+      unsigned voff = (row0 + i * ROWS_PER_SLAB < left) ? off[i] : kAttnOob;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
           rsrc, (attn_lds_void_t *)(tile + (wave * Gm::PER_WAVE + i) * 1024), 16, (int)voff, 0, 0, 0);
     }
@@ -111,7 +113,9 @@ template <int DT> __device__ __forceinline__ uint32_t pack2_fast(float a, float 
   }
 }
 
-template <int DT, int D>
+// PLAIN: no bias and a non-negative scale, so the row maximum can be taken on
+// the raw scores and the scale folded into the exponent.
+template <int DT, int D, bool PLAIN>
 __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv, const void *Vv,
                                                   const void *biasv, void *Ov,
                                                   const RockAttentionParams &p) {
@@ -120,9 +124,14 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
   constexpr int DTILES = D / 32;  // 32-row tiles of O^T
   constexpr int STAGE = 2 * Gm::TILE_B;
   constexpr float kLog2e = 1.44269504088896340736f;
+  // The plain kernel software-pipelines the two GEMMs (see tile_step); the
+  // bias kernel needs its registers for the bias gather and keeps the simple
+  // order "scores, softmax, PV" per tile.
+  constexpr bool PIPE = PLAIN;
   static_assert(2 * STAGE <= 65536, "every LDS read offset must fit the 16-bit immediate");
 
   __shared__ __attribute__((aligned(1024))) char lds_generic[2 * STAGE];
+
   attn_lds_char_t *lds = (attn_lds_char_t *)lds_generic;
 
   const int tid = threadIdx.x;
@@ -153,6 +162,8 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
   lv.init(V, p.v_js, p.seq_k, p.d_v, wave, lane);
   lk.issue(0, lds);
   lv.issue(0, lds + Gm::TILE_B);
+  if constexpr (PIPE)
+    lk.issue(kBKV, lds + 2 * Gm::TILE_B);
 
   v4i qf[KSTEPS];
 #pragma unroll
@@ -162,20 +173,17 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
   // ---- per-lane LDS read offsets (bytes from the start of a K or V tile)
   // K fragment of key rows 32*st + lq at chunk 2*ks + h: the swizzle depends on
   // lq only, so "+ 32*st rows" and the stage are immediates.
-  attn_lds_char_t *kptr[KSTEPS];
-#pragma unroll
-  for (int ks = 0; ks < KSTEPS; ++ks)
-    kptr[ks] = lds + lq * Gm::ROWB + (((ks * 2 + h) ^ attn_swz<Gm::CPR, false>(lq)) * 16);
+  attn_lds_char_t *const krow = lds + lq * Gm::ROWB;
+  const int kswz = (h ^ attn_swz<Gm::CPR, false>(lq)) * 16; // chunk 2*ks + h: ks XORs in as a constant
+  auto kptr = [&](int ks) __attribute__((always_inline)) { return krow + (kswz ^ (ks * 32)); };
   // V^T fragment through the transposing read: lane (i = lane % 16, g16) of
   // half h addresses key 4*h + i/4 (+ 32*st + 16*u, + 8) at d = 32*dt + 16*g16 + 4*(i%4).
   const int tr_i = lane & 15, tr_g = (lane >> 4) & 1;
   const int tr_key = 4 * h + (tr_i >> 2);
   const int tr_chunk = 2 * tr_g + ((tr_i & 3) >> 1);
-  attn_lds_char_t *vptr[DTILES];
-#pragma unroll
-  for (int dt = 0; dt < DTILES; ++dt)
-    vptr[dt] = lds + Gm::TILE_B + tr_key * Gm::ROWB +
-               (((4 * dt + tr_chunk) ^ attn_swz<Gm::CPR, true>(tr_key)) * 16) + (tr_i & 1) * 8;
+  attn_lds_char_t *const vrow = lds + Gm::TILE_B + tr_key * Gm::ROWB + (tr_i & 1) * 8;
+  const int vswz = (tr_chunk ^ attn_swz<Gm::CPR, true>(tr_key)) * 16; // chunk 4*dt + tr_chunk
+  auto vptr = [&](int dt) __attribute__((always_inline)) { return vrow + (vswz ^ (dt * 64)); };
 
   v16f o[DTILES];
 #pragma unroll
@@ -186,22 +194,12 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
   float m_run = -INFINITY, l_run = 0.0f;
 
   const float c_scale = p.scale * kLog2e;
-  const bool plain = (bias == nullptr) && (c_scale >= 0.0f); // scale folds into the exponent
+  constexpr bool plain = PLAIN;
   const int nkv = (p.seq_k + kBKV - 1) / kBKV;
 
-  // one K/V tile; STG (0/1) is the LDS stage holding it
-  auto tile_step = [&](int t, auto stage_const) __attribute__((always_inline)) {
-    constexpr int STG = decltype(stage_const)::value;
-    wait_vmcnt_attn0();               // this wave's part of tile t has landed ...
-    __builtin_amdgcn_s_barrier();     // ... everyone's has, and tile t-1 is no longer being read
-    {
-      attn_lds_char_t *nxt = lds + (STG ^ 1) * STAGE;
-      lk.issue((t + 1) * kBKV, nxt);  // past the end: every lane out of range, zeros, no traffic
-      lv.issue((t + 1) * kBKV, nxt + Gm::TILE_B);
-    }
-
-    // ---- S^T tiles: rows = keys, cols = queries
-    v16f s[2];
+  // S^T tiles of the K tile in LDS slot SLOT: rows = keys, cols = queries
+  auto scores = [&](auto slot_const, v16f(&s)[2]) __attribute__((always_inline)) {
+    constexpr int SLOT = decltype(slot_const)::value;
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
 #pragma unroll
@@ -209,23 +207,52 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
         s[st][v] = 0.0f;
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) {
-        v4i kf = *(const attn_lds_v4i_t *)(kptr[ks] + (STG * STAGE + st * 32 * Gm::ROWB));
+        v4i kf = *(const attn_lds_v4i_t *)(kptr(ks) + (SLOT * STAGE + st * 32 * Gm::ROWB));
         s[st] = mma32<DT>(kf, qf[ks], s[st]);
       }
+    }
+  };
+
+  // One step of the software pipeline.  On entry `s` holds the scores of tile
+  // t (their MFMAs possibly still in flight), K[t+1] and V[t] have been
+  // requested.  The step requests K[t+2] and V[t+1], issues the score MFMAs of
+  // tile t+1 into `s_next`, and only then runs the softmax of tile t, so the
+  // matrix pipe works on the next tile while the vector ALU exponentiates
+  // this one.  K[t] and V[t] live in slot t%2 = PAR of their rings.
+  auto tile_step = [&](int t, auto par_const, auto last_const, v16f(&s_in)[2], v16f(&s_next)[2])
+                       __attribute__((always_inline)) {
+    v16f s_here[2];
+    v16f(&s)[2] = PIPE ? s_in : s_here;
+    constexpr int PAR = decltype(par_const)::value;
+    constexpr bool LAST = decltype(last_const)::value; // no tile t+1: nothing to issue ahead
+    constexpr int STG = PAR;
+    wait_loads_and_lds_reads();       // this wave's parts of K[t+1] and V[t] have landed ...
+    __builtin_amdgcn_s_barrier();     // ... everyone's have; K[t] and V[t-1] are no longer read
+    if constexpr (!PIPE) {
+      // plain double buffering: request tile t+1, then compute tile t's scores
+      lk.issue((t + 1) * kBKV, lds + (PAR ^ 1) * STAGE); // past the end: zeros, no traffic
+      lv.issue((t + 1) * kBKV, lds + (PAR ^ 1) * STAGE + Gm::TILE_B);
+      scores(std::integral_constant<int, PAR>{}, s);
+    } else if constexpr (!LAST) {
+      lk.issue((t + 2) * kBKV, lds + PAR * STAGE); // past the end: zeros, no traffic
+      lv.issue((t + 1) * kBKV, lds + (PAR ^ 1) * STAGE + Gm::TILE_B);
     }
 
     // ---- online softmax on this lane's 32 scores of row q_row
     const int key_base = t * kBKV + 4 * h;
-    const bool tail = (t + 1) * kBKV > p.seq_k;
-    if (!plain) {
+    const bool tail = LAST && (t + 1) * kBKV > p.seq_k; // only the last tile can be ragged
+    if constexpr (!plain) {
+      // element offsets inside one g slice of the bias fit 32 bits (host check)
+      const unsigned bias_js = (unsigned)p.bias_js;
+      const unsigned boff = (unsigned)q_row * (unsigned)p.bias_is + (unsigned)key_base * bias_js;
 #pragma unroll
       for (int st = 0; st < 2; ++st)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          int key = key_base + st * 32 + 8 * (v >> 2) + (v & 3);
+          const int kofs = st * 32 + 8 * (v >> 2) + (v & 3);
           float x = s[st][v] * c_scale;
-          if (bias != nullptr && key < p.seq_k && q_row < p.seq_q)
-            x = x + elem_to_f32<DT>(bias[(int64_t)q_row * p.bias_is + (int64_t)key * p.bias_js]) * kLog2e;
+          if (bias != nullptr && key_base + kofs < p.seq_k && q_row < p.seq_q)
+            x = x + elem_to_f32<DT>(bias[boff + (unsigned)kofs * bias_js]) * kLog2e;
           s[st][v] = x;
         }
     }
@@ -238,17 +265,26 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
           s[st][v] = key < p.seq_k ? s[st][v] : -INFINITY;
         }
     }
-    float mloc = -INFINITY;
+    // row maximum: four independent chains, then across the two wave halves
+    float mc[4];
 #pragma unroll
-    for (int st = 0; st < 2; ++st)
+    for (int c = 0; c < 4; ++c)
+      mc[c] = fmaxf(s[c >> 1][(c & 1) * 8], s[c >> 1][(c & 1) * 8 + 1]);
 #pragma unroll
-      for (int v = 0; v < 16; ++v)
-        mloc = fmaxf(mloc, s[st][v]);
-    float mt = half_swap_max(mloc);
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+      for (int v = 2; v < 8; ++v)
+        mc[c] = fmaxf(mc[c], s[c >> 1][(c & 1) * 8 + v]);
+    float mt = half_swap_max_fast(fmaxf(fmaxf(mc[0], mc[1]), fmaxf(mc[2], mc[3])));
     if (plain)
       mt = mt * c_scale;
-    const float m_new = fmaxf(m_run, mt);
-    if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+    // The running maximum only moves when some row's maximum grew by more
+    // than kSlack (log2 units): until then p = 2^(s - m_run) <= 2^kSlack,
+    // harmless in f16/bf16 and in the f32 sums, and the final division by the
+    // row sum cancels the stale maximum exactly.
+    constexpr float kSlack = 8.0f;
+    if (__builtin_amdgcn_ballot_w64(mt > m_run + kSlack) != 0) {
+      const float m_new = fmaxf(m_run, mt);
       const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
       const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
       l_run *= alpha;
@@ -259,6 +295,9 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
           o[dt][v] *= alpha;
       m_run = m_new;
     }
+    // same basic block as the exponentials below: the scheduler interleaves
+    if constexpr (PIPE && !LAST)
+      scores(std::integral_constant<int, PAR ^ 1>{}, s_next);
     const float m_use = (m_run == -INFINITY) ? 0.0f : m_run;
     const float cs = plain ? c_scale : 1.0f;
     float psum = 0.0f;
@@ -284,7 +323,7 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
         constexpr int kSliceB = 16 * Gm::ROWB; // 16 keys
 #pragma unroll
         for (int dt = 0; dt < DTILES; ++dt) {
-          attn_lds_char_t *a0 = vptr[dt] + (STG * STAGE + (st * 2 + u) * kSliceB);
+          attn_lds_char_t *a0 = vptr(dt) + (STG * STAGE + (st * 2 + u) * kSliceB);
           v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((attn_lds_v4s_t *)a0);
           v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((attn_lds_v4s_t *)(a0 + 8 * Gm::ROWB));
           v2i l2 = __builtin_bit_cast(v2i, lo), h2 = __builtin_bit_cast(v2i, hi);
@@ -294,10 +333,32 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
       }
   };
 
-  for (int t = 0; t < nkv; t += 2) {
-    tile_step(t, std::integral_constant<int, 0>{});
-    if (t + 1 < nkv)
-      tile_step(t + 1, std::integral_constant<int, 1>{});
+  v16f s_even[2], s_odd[2];
+  if constexpr (PIPE) {
+    wait_vmcnt_attn0();
+    __builtin_amdgcn_s_barrier();
+    scores(std::integral_constant<int, 0>{}, s_even);
+  }
+  using C0 = std::integral_constant<int, 0>;
+  using C1 = std::integral_constant<int, 1>;
+  int t = 0;
+  if constexpr (!PIPE) {
+    for (; t < nkv; t += 2) {
+      tile_step(t, C0{}, std::true_type{}, s_even, s_odd);
+      if (t + 1 < nkv)
+        tile_step(t + 1, C1{}, std::true_type{}, s_odd, s_even);
+    }
+  } else {
+  for (; t + 2 < nkv; t += 2) {
+    tile_step(t, C0{}, std::false_type{}, s_even, s_odd);
+    tile_step(t + 1, C1{}, std::false_type{}, s_odd, s_even);
+  }
+  if (t + 1 < nkv) {
+    tile_step(t, C0{}, std::false_type{}, s_even, s_odd);
+    tile_step(t + 1, C1{}, std::true_type{}, s_odd, s_even);
+  } else {
+    tile_step(t, C0{}, std::true_type{}, s_even, s_odd);
+  }
   }
   wait_vmcnt_attn0(); // drain the out-of-range loads of the step past the end
 

@@ -43,6 +43,24 @@ __device__ __forceinline__ float other_half(float x) {
   int v = __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __builtin_bit_cast(int, x));
   return __builtin_bit_cast(float, v);
 }
+// Both halves of the wave through one v_permlane32_swap: with a = b = x in two
+// different registers the instruction leaves a = [x.lo, x.lo] and
+// b = [x.hi, x.hi].  Written as assembly: the compiler builtin folds the two
+// equal operands into one register and then drops the combine that follows.
+// The s_nop pair covers the wait states the instruction needs after a VALU
+// write of its operands and before a VALU read of its results, which the
+// compiler's hazard pass cannot see inside an asm block.
+__device__ __forceinline__ void both_halves(float x, float &lo, float &hi) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  lo = a;
+  hi = b;
+}
+__device__ __forceinline__ float half_swap_max_fast(float x) {
+  float lo, hi;
+  both_halves(x, lo, hi);
+  return fmaxf(lo, hi);
+}
 __device__ __forceinline__ float half_swap_max(float x) { return fmaxf(x, other_half(x)); }
 __device__ __forceinline__ float half_swap_sum(float x) { return x + other_half(x); }
 
@@ -320,6 +338,13 @@ __device__ __forceinline__ void attention_body(const void *Qv, const void *Kv, c
 __device__ __forceinline__ void wait_vmcnt_attn0() {
   __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0); expcnt and lgkmcnt left alone
 }
+// Before the barrier that hands an LDS tile back to the loaders: this wave's
+// loads have landed AND its LDS reads have returned.  Without the second part
+// a read issued just before the barrier can still sit in the LDS queue when
+// another wave's refill of that tile lands.
+__device__ __forceinline__ void wait_loads_and_lds_reads() {
+  __builtin_amdgcn_s_waitcnt(0x0070); // vmcnt(0) lgkmcnt(0); expcnt left alone
+}
 
 } // namespace rk
 
@@ -335,19 +360,23 @@ __device__ __forceinline__ void wait_vmcnt_attn0() {
   }
 
 // fast variants: two blocks per compute unit (register budget 256 per lane)
-#define RK_ATTN_DL(DTNAME, DT, D)                                                             \
+#define RK_ATTN_DL(DTNAME, DT, D, SUFFIX, PLAIN)                                              \
   extern "C" __global__ __launch_bounds__(rk::kAttnThreads, 2) void                           \
-      rock_attention_##DTNAME##_d##D##x##D##_fast(const void *Q, const void *K, const void *V,\
-                                                  const void *bias, void *O,                  \
-                                                  RockAttentionParams p) {                    \
-    rk::attention_body_dl<DT, D>(Q, K, V, bias, O, p);                                        \
+      rock_attention_##DTNAME##_d##D##x##D##_##SUFFIX(const void *Q, const void *K,           \
+                                                      const void *V, const void *bias,        \
+                                                      void *O, RockAttentionParams p) {       \
+    rk::attention_body_dl<DT, D, PLAIN>(Q, K, V, bias, O, p);                                 \
   }
 
-RK_ATTN_DL(f16, MM_F16, 128)
-RK_ATTN_DL(f16, MM_F16, 64)
+RK_ATTN_DL(f16, MM_F16, 128, fast, true)
+RK_ATTN_DL(f16, MM_F16, 128, fast_bias, false)
+RK_ATTN_DL(f16, MM_F16, 64, fast, true)
+RK_ATTN_DL(f16, MM_F16, 64, fast_bias, false)
 RK_ATTN(f16, MM_F16, 128, 128, generic, false)
 RK_ATTN(f16, MM_F16, 64, 64, generic, false)
-RK_ATTN_DL(bf16, MM_BF16, 128)
-RK_ATTN_DL(bf16, MM_BF16, 64)
+RK_ATTN_DL(bf16, MM_BF16, 128, fast, true)
+RK_ATTN_DL(bf16, MM_BF16, 128, fast_bias, false)
+RK_ATTN_DL(bf16, MM_BF16, 64, fast, true)
+RK_ATTN_DL(bf16, MM_BF16, 64, fast_bias, false)
 RK_ATTN(bf16, MM_BF16, 128, 128, generic, false)
 RK_ATTN(bf16, MM_BF16, 64, 64, generic, false)

@@ -683,11 +683,13 @@ Handle *make_attention(const OptMap &o) {
                     dv % 8 == 0 && p.o_is % 4 == 0 && p.k_js % 8 == 0 && p.v_js % 8 == 0 &&
                     p.q_is % 8 == 0 &&
                     // byte offsets inside one g slice below 2^31 (buffer descriptors)
-                    sk * p.k_js * 2 < ((int64_t)1 << 31) && sk * p.v_js * 2 < ((int64_t)1 << 31);
+                    sk * p.k_js * 2 < ((int64_t)1 << 31) && sk * p.v_js * 2 < ((int64_t)1 << 31) &&
+                    // the bias gather indexes one g slice with 32-bit element offsets
+                    (!has_bias || sq * sk < ((int64_t)1 << 31));
   const int dmax = (dqk <= 64 && dv <= 64) ? 64 : 128;
   char name[96];
   std::snprintf(name, sizeof name, "rock_attention_%s_d%dx%d_%s", dtype_name(ty), dmax, dmax,
-                fast ? "fast" : "generic");
+                !fast ? "generic" : (!p.has_bias && p.scale >= 0.0f) ? "fast" : "fast_bias");
   h->kernel_name = name;
   h->blob_name = "attention";
   h->num_pointers = 5;
