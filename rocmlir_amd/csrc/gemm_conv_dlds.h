@@ -64,6 +64,15 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x0F70);
 }
 
+// vmcnt(N) and lgkmcnt(0) together: the form used before a barrier that hands
+// an LDS stage back to the loaders.  The LDS reads of that stage were issued
+// before the barrier, but a read can still sit in the LDS queue when another
+// wave's refill lands unless its issuer has waited for the data.
+template <int N> __device__ __forceinline__ void wait_vmcnt_and_lds_reads() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x0070);
+}
+
 template <int ROWS, int NW, int RB> struct SlabGeom {
   static constexpr int SLABS = ROWS / DlGeom<RB>::SLAB_ROWS;
   static constexpr int PER_WAVE = SLABS / NW;
@@ -297,7 +306,7 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
 
   for (int kt = 0; kt < nk; ++kt) {
     // this wave's loads of K-step kt have landed (two younger steps may be in flight) ...
-    wait_vmcnt<(kDlStages - 2) * LOADS_PER_STEP>();
+    wait_vmcnt_and_lds_reads<(kDlStages - 2) * LOADS_PER_STEP>();
     // ... and so have everyone else's; everyone is also done reading step kt-1
     __builtin_amdgcn_s_barrier();
     {

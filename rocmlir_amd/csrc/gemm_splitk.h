@@ -68,8 +68,9 @@ __device__ __forceinline__ void gemm_body_splitk(const void *Aptr, const void *B
     lb.issue(k_begin + s, wlds + s * STAGE + A_BYTES);
   }
   for (int i = 0; i < per_wave; ++i) {
-    // this wave's loads of step i have landed; nobody else touches its stages
-    wait_vmcnt<(kDlStages - 2) * LOADS_PER_STEP>();
+    // this wave's loads of step i have landed and its reads of the stage about
+    // to be refilled have returned; nobody else touches its stages
+    wait_vmcnt_and_lds_reads<(kDlStages - 2) * LOADS_PER_STEP>();
     {
       char *refill = wlds + ((i + kDlStages - 1) % kDlStages) * STAGE;
       const int kt = (i + kDlStages - 1 < per_wave) ? k_begin + i + kDlStages - 1 : nk; // nk = out of range
