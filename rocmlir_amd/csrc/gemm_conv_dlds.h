@@ -281,9 +281,17 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
   decode_block(p.tiles_m, p.tiles_n, p_batch(p), p.group_m, p.xcd_remap, g, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
-  auto la = make_dl_a<DT, BM, NW, RB, LDA>(Aptr, p, g, m0, wave, lane);
-  auto lb = make_dl_b<DT, BN, NW, RB, LDB>(Bptr, p, g, n0, wave, lane);
-  constexpr int LOADS_PER_STEP = SlabGeom<BM, NW, RB>::PER_WAVE + SlabGeom<BN, NW, RB>::PER_WAVE;
+  // Eight-wave blocks put two waves on every SIMD.  Only the upper four issue
+  // loads: a burst of load instructions from all eight backs up in the
+  // texture path and stalls every wave at once, idling the matrix pipe; this
+  // way the lower wave of each SIMD starts its MFMAs right after the barrier
+  // and the upper one follows when its loads are out.
+  constexpr int NLOAD = NW == 8 ? 4 : NW;
+  const bool loader = wave >= NW - NLOAD;
+  const int lwave = loader ? wave - (NW - NLOAD) : 0;
+  auto la = make_dl_a<DT, BM, NLOAD, RB, LDA>(Aptr, p, g, m0, lwave, lane);
+  auto lb = make_dl_b<DT, BN, NLOAD, RB, LDB>(Bptr, p, g, n0, lwave, lane);
+  constexpr int LOADS_PER_STEP = SlabGeom<BM, NLOAD, RB>::PER_WAVE + SlabGeom<BN, NLOAD, RB>::PER_WAVE;
 
   Acc acc[MI][NI];
 #pragma unroll
@@ -300,8 +308,10 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
   // range, no memory is touched, and the outstanding-load count stays uniform.
 #pragma unroll
   for (int s = 0; s < kDlStages - 1; ++s) {
-    la.issue(s, lds + s * STAGE);
-    lb.issue(s, lds + s * STAGE + A_BYTES);
+    if (loader) {
+      la.issue(s, lds + s * STAGE);
+      lb.issue(s, lds + s * STAGE + A_BYTES);
+    }
   }
 
   for (int kt = 0; kt < nk; ++kt) {
@@ -309,7 +319,7 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
     wait_vmcnt_and_lds_reads<(kDlStages - 2) * LOADS_PER_STEP>();
     // ... and so have everyone else's; everyone is also done reading step kt-1
     __builtin_amdgcn_s_barrier();
-    {
+    if (loader) {
       char *refill = lds + ((kt + kDlStages - 1) % kDlStages) * STAGE;
       la.issue(kt + kDlStages - 1, refill);
       lb.issue(kt + kDlStages - 1, refill + A_BYTES);
