@@ -157,8 +157,14 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-headline", action="store_true", help="skip the other four configs")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
-    ap.add_argument("--traffic-bytes", type=float, default=None,
-                    help="HBM bytes per launch of the headline kernel from rocprofv3 --pmc runs")
+    ap.add_argument("--traffic-bytes", type=float, default=134.5e6,
+                    help="HBM bytes per launch of the headline kernel: FETCH_SIZE + WRITE_SIZE of "
+                         "rocprofv3 --pmc runs of this command, each scaled by the same counter's reading "
+                         "for a plain copy (--calibrate-copy); the default is the committed measurement "
+                         "(profiles/gemm_i8_256x256_c2_hbm_traffic.txt)")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
+                    help="only run a plain device-to-device copy of MIB MiB five times (the known-size "
+                         "kernel that FETCH_SIZE / WRITE_SIZE readings are scaled by) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (every box has one); --gpus %d is not "
@@ -172,6 +178,14 @@ def main():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.calibrate_copy:
+        src = torch.ones(args.calibrate_copy << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes": src.numel(), "launches": 5}))
+        return
     cfgs = make_configs(torch, rock, dev)
     head_name = "c2_gemm_i8_4096_f16out"
     head = cfgs[head_name]
