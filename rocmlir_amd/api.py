@@ -320,10 +320,12 @@ def conv2d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize,
            in_channels, out_channels, in_h, in_w, fil_h, fil_w, groupsize=1,
            stride=(1, 1), padding=(0, 0), dilation=(1, 1), out_dtype=None,
            scale=None, zero_point=0, bias=None, relu=False, quant_scale=None,
-           out_zero_point=0, out=None, perf_config=None, stream=None):
+           out_zero_point=0, out=None, perf_config=None, stream=None,
+           info=None):
     """Forward convolution; tensors are flat device buffers laid out as the
     layout strings say (Miir / rocmlir-gen spelling, e.g. 'gkyxc', 'nhwgc',
-    'NGCHW').  Returns the flat output tensor."""
+    'NGCHW').  Returns the flat output tensor.  A dict passed as `info`
+    receives the name and perf_config of the kernel that ran."""
     import torch
     t = _dtype_name(inp.dtype)
     ho = (in_h + 2 * padding[0] - (fil_h - 1) * dilation[0] - 1) // stride[0] + 1
@@ -345,6 +347,9 @@ def conv2d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize,
     opts += _epilogue_flags(scale, zero_point, bias, relu, quant_scale,
                             out_zero_point)
     k = _kernel(opts)
+    if info is not None:
+        info["kernel_name"] = k.kernel_name
+        info["perf_config"] = k.perf_config
     if out_dtype is None:
         out_dtype = {"i8": "i32", "fp8": "f32", "bf8": "f32"}.get(t, t)
     if out is None:

@@ -254,6 +254,85 @@ __device__ __forceinline__ Frag<DT> dl_read_frag(const char *lds, int row, int s
   return f;
 }
 
+// Epilogue of the direct-to-LDS bodies: lane holds m = m_wave + 32*i + lrow,
+// n = n_wave + 32*j + 8*q + 4*lgrp + {0..3}.  `lds` is the block's operand
+// ring (LDS_BYTES), free once every wave has passed the barrier at the top;
+// NWAVES waves call this, each with its own `wave` index in [0, NWAVES).  A
+// wave of the block that holds no accumulators and does not call it must
+// still execute that barrier: it does so when dl_epilogue_staged() is true.
+template <typename Params>
+__device__ __forceinline__ bool dl_epilogue_staged(const Params &p, const void *Cptr) {
+  return out_rows_chunk_aligned(p, Cptr, out_elem_size(p.epi.out_dtype));
+}
+
+template <int DT, int MI, int NI, int NWAVES, int LDS_BYTES, typename Params>
+__device__ __forceinline__ void dl_epilogue(typename MmaTraits<DT>::Acc (&acc)[MI][NI], const Params &p, int g,
+                                            void *Cptr, const void *aux, int m_wave, int n_wave, char *lds,
+                                            int wave, int lane) {
+  using Tr = MmaTraits<DT>;
+  constexpr int WTN = NI * 32;
+  const int lrow = lane & 31, lgrp = lane >> 5;
+  const RockEpilogue &e = p.epi;
+  using Acc4 = decltype(__builtin_shufflevector(acc[0][0], acc[0][0], 0, 1, 2, 3));
+  const bool staged_ok = dl_epilogue_staged(p, Cptr);
+  if (staged_ok)
+    __builtin_amdgcn_s_barrier(); // every wave is done reading the operand stages
+
+  dispatch_out_dtype<Tr::INT_ACC>(e.out_dtype, [&](auto od_const) __attribute__((always_inline)) {
+    constexpr int OD = decltype(od_const)::value;
+    if (!staged_ok) {
+      direct_epilogue<Tr::INT_ACC, OD, MI, NI, Acc4>(acc, p, g, Cptr, aux, m_wave + lrow,
+                                                    n_wave + lgrp * 4);
+      return;
+    }
+    // Staged store: each wave transposes one 32-row block of its tile at a
+    // time through a private LDS region, so that global stores are 16 bytes
+    // per lane and cover whole rows of the wave tile (WTN * ES contiguous
+    // bytes per 64/LPR lanes).
+    constexpr int ES = OutElemSize<OD>::value;
+    constexpr int ROWB = WTN * ES, PITCH = ROWB + 16;
+    constexpr int LPR = ROWB / 16, RPI = 64 / LPR;
+    constexpr int WBUF = 32 * (WTN * 4 + 16);
+    static_assert(NWAVES * WBUF <= LDS_BYTES, "staging buffers must fit in the operand stages");
+    char *wbuf = lds + wave * WBUF;
+    const int rd_row = lane / LPR, rd_cb = (lane % LPR) * 16;
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+#pragma unroll
+      for (int j = 0; j < NI; ++j) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int nloc = j * 32 + q * 8 + lgrp * 4;
+          Acc4 a4 = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                     acc[i][j][4 * q + 3]};
+          v4i raw = epilogue_convert4<Tr::INT_ACC, OD>(a4, e, aux, n_wave + nloc, p.N);
+          char *dst = wbuf + lrow * PITCH + nloc * ES;
+          if constexpr (ES == 4)
+            *(v4i *)dst = raw;
+          else if constexpr (ES == 2)
+            *(v2i *)dst = v2i{raw[0], raw[1]};
+          else
+            *(int *)dst = raw[0];
+        }
+      }
+#pragma unroll
+      for (int r0 = 0; r0 < 32; r0 += RPI) {
+        const int row = r0 + rd_row;
+        v4i d = *(const v4i *)(wbuf + row * PITCH + rd_cb);
+        const int m = m_wave + i * 32 + row;
+        const int n = n_wave + rd_cb / ES;
+        if (m < p.M && n < p.N) {
+          int64_t row_off, n_stride;
+          bool vec_ok;
+          out_row_addr(p, g, m, Cptr, row_off, n_stride, vec_ok);
+          *(v4i *)((char *)Cptr + (row_off + n) * ES) = d;
+        }
+      }
+    }
+  });
+}
+
+
 template <int DT, int BM, int BN, int WAVES_M, int WAVES_N, int RB, int LDA, int LDB, typename Params>
 __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void *Bptr, void *Cptr,
                                                     const void *aux, const Params &p) {
@@ -344,65 +423,8 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
   // drain the out-of-range loads issued for steps >= nk before the LDS is released
   wait_vmcnt<0>();
 
-  // ---- epilogue: lane holds m = .. + lrow, n = .. + 8*q + 4*lgrp + {0..3}
-  const RockEpilogue &e = p.epi;
-  using Acc4 = decltype(__builtin_shufflevector(acc[0][0], acc[0][0], 0, 1, 2, 3));
-  const bool staged_ok = out_rows_chunk_aligned(p, Cptr, out_elem_size(e.out_dtype));
-  if (staged_ok)
-    __builtin_amdgcn_s_barrier(); // every wave is done reading the operand stages
-
-  dispatch_out_dtype<Tr::INT_ACC>(e.out_dtype, [&](auto od_const) __attribute__((always_inline)) {
-    constexpr int OD = decltype(od_const)::value;
-    if (!staged_ok) {
-      direct_epilogue<Tr::INT_ACC, OD, MI, NI, Acc4>(acc, p, g, Cptr, aux, m0 + wm * WTM + lrow,
-                                                    n0 + wn * WTN + lgrp * 4);
-      return;
-    }
-    // Staged store: each wave transposes one 32-row block of its tile at a
-    // time through a private LDS region, so that global stores are 16 bytes
-    // per lane and cover whole rows of the wave tile (WTN * ES contiguous
-    // bytes per 64/LPR lanes).
-    constexpr int ES = OutElemSize<OD>::value;
-    constexpr int ROWB = WTN * ES, PITCH = ROWB + 16;
-    constexpr int LPR = ROWB / 16, RPI = 64 / LPR;
-    constexpr int WBUF = 32 * (WTN * 4 + 16);
-    static_assert(NW * WBUF <= kDlStages * STAGE, "staging buffers must fit in the operand stages");
-    char *wbuf = lds + wave * WBUF;
-    const int rd_row = lane / LPR, rd_cb = (lane % LPR) * 16;
-#pragma unroll
-    for (int i = 0; i < MI; ++i) {
-#pragma unroll
-      for (int j = 0; j < NI; ++j) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int nloc = j * 32 + q * 8 + lgrp * 4;
-          Acc4 a4 = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
-                     acc[i][j][4 * q + 3]};
-          v4i raw = epilogue_convert4<Tr::INT_ACC, OD>(a4, e, aux, n0 + wn * WTN + nloc, p.N);
-          char *dst = wbuf + lrow * PITCH + nloc * ES;
-          if constexpr (ES == 4)
-            *(v4i *)dst = raw;
-          else if constexpr (ES == 2)
-            *(v2i *)dst = v2i{raw[0], raw[1]};
-          else
-            *(int *)dst = raw[0];
-        }
-      }
-#pragma unroll
-      for (int r0 = 0; r0 < 32; r0 += RPI) {
-        const int row = r0 + rd_row;
-        v4i d = *(const v4i *)(wbuf + row * PITCH + rd_cb);
-        const int m = m0 + wm * WTM + i * 32 + row;
-        const int n = n0 + wn * WTN + rd_cb / ES;
-        if (m < p.M && n < p.N) {
-          int64_t row_off, n_stride;
-          bool vec_ok;
-          out_row_addr(p, g, m, Cptr, row_off, n_stride, vec_ok);
-          *(v4i *)((char *)Cptr + (row_off + n) * ES) = d;
-        }
-      }
-    }
-  });
+  dl_epilogue<DT, MI, NI, NW, kDlStages * STAGE>(acc, p, g, Cptr, aux, m0 + wm * WTM, n0 + wn * WTN, lds, wave,
+                                                 lane);
 }
 
 } // namespace rk

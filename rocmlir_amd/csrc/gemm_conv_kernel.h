@@ -400,11 +400,17 @@ __device__ __forceinline__ void out_row_addr(const RockGemmParams &p, int g, int
 
 __device__ __forceinline__ void out_row_addr(const RockConvParams &p, int g, int m, const void *base,
                                              int64_t &row_off, int64_t &n_stride, bool &vec_ok) {
-  int n = m / (p.ho * p.wo);
-  int rem = m - n * (p.ho * p.wo);
-  int ho = rem / p.wo;
-  int wo = rem - ho * p.wo;
-  row_off = (int64_t)n * p.out_ns + (int64_t)g * p.out_gs + (int64_t)ho * p.out_hs + (int64_t)wo * p.out_ws;
+  if (p.out_hs == (int64_t)p.wo * p.out_ws && p.out_ns == (int64_t)p.ho * p.out_hs) {
+    // pixels of one group are equally spaced in memory (NHWC-like outputs):
+    // the pixel index addresses the row directly, no division
+    row_off = (int64_t)g * p.out_gs + (int64_t)m * p.out_ws;
+  } else {
+    int n = m / (p.ho * p.wo);
+    int rem = m - n * (p.ho * p.wo);
+    int ho = rem / p.wo;
+    int wo = rem - ho * p.wo;
+    row_off = (int64_t)n * p.out_ns + (int64_t)g * p.out_gs + (int64_t)ho * p.out_hs + (int64_t)wo * p.out_ws;
+  }
   n_stride = p.out_ks;
   vec_ok = (p.out_ks == 1) && aligned_for_vec(base, row_off, p.epi.out_dtype);
 }

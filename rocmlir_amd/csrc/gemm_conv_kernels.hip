@@ -2,6 +2,7 @@
 // once per type with -DROCK_DT=<code> -DROCK_DTNAME=<name> into a gfx950 code
 // object; the host library picks a kernel by name from its perf-config table.
 #include "gemm_splitk.h"
+#include "conv_direct.h"
 
 #ifndef ROCK_DT
 #error "compile with -DROCK_DT=<operand type code> -DROCK_DTNAME=<suffix>"
@@ -58,4 +59,9 @@ RK_CONV_DL(_256x128_fast, 256, 128, 4, 2, 128)
 RK_CONV_DL(_128x128_fast, 128, 128, 2, 2, 128)
 RK_CONV_DL(_64x64_fast, 64, 64, 2, 2, 128)
 RK_CONV(_64x64_generic, 64, 64, 2, 2, rk::LD_CONV_IN_GENERIC, rk::LD_CONV_FIL_GENERIC)
+// input window resident in LDS: 224 output pixels x 128 channels per block
+extern "C" __global__ __launch_bounds__(512) void RK_CAT(RK_CAT(rock_conv_, ROCK_DTNAME), _direct224)(
+    const void *fil, const void *in, void *out, const void *aux, RockConvParams p) {
+  rk::conv_direct_body<ROCK_DT, 7, 2>(in, fil, out, aux, p);
+}
 #endif

@@ -66,7 +66,7 @@ struct RockConvParams {
   int32_t tiles_m, tiles_n;
   int32_t group_m, xcd_remap;
   int32_t k_order_yxc; // 1: reduction index runs (y,x,c) with c fastest; 0: (c,y,x)
-  int32_t pad_;
+  int32_t rows_per_tile; // window-resident kernel: output rows (n, ho) per block; else 0
   RockEpilogue epi;
 };
 

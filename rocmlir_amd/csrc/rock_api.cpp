@@ -200,6 +200,8 @@ const Tile kGenericTile = {"_64x64_generic", 64, 64, 2, 2, 4, 0.1f, true, true};
 // 32x32 output tile, K split over the four waves of the block (GEMM fast path only)
 const Tile kSplitKTile = {"_32x32_splitk", 32, 32, 1, 4, 2, 0.3f, true, false};
 constexpr int kNumCU = 256; // MI355X
+constexpr int kDirectTilePixels = 224;          // conv_direct.h: 7 blocks of 32 output pixels
+constexpr int64_t kDirectWindowBytes = 96 * 1024; // and its LDS window
 constexpr int kNumXCD = 8;
 
 int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
@@ -617,6 +619,52 @@ Handle *make_conv(const OptMap &o) {
   h->blob_name = std::string("gemm_") + dtype_name(ti);
   h->num_pointers = 4;
   h->perf_config = perf_string(*tile, es);
+
+  // Window-resident kernel (conv_direct.h), chosen by "-perf_config
+  // v2:224,128,...": stride 1, dilation 1, a filter of more than one tap,
+  // channel run a power of two of 128..1024 bytes, output width within the
+  // 224-pixel tile and a window of TH + 2(Y-1) padded rows (a tile may
+  // straddle two images) within 96 KiB of LDS.  On the ResNet 3x3 layer of
+  // the benchmark it runs within a few percent of the implicit-GEMM kernel,
+  // so the table does not pick it by itself; a request that cannot be met
+  // falls back to the table like any other perf_config.
+  {
+    const int64_t cbytes = c * es;
+    const int64_t th = std::min<int64_t>(ho, wo > 0 ? kDirectTilePixels / wo : 0);
+    const int64_t row_pitch = ((wi + 2 * pw) * cbytes + 1023) / 1024 * 1024; // whole 1 KiB load slabs
+    const int64_t window = (th + 2 * (y - 1)) * row_pitch;
+    const bool direct_ok = fast && sh == 1 && sw == 1 && dh == 1 && dw == 1 && y * x > 1 &&
+                           cbytes >= 128 && cbytes <= 1024 && (cbytes & (cbytes - 1)) == 0 &&
+                           th >= 1 && window <= kDirectWindowBytes && row_pitch <= 32 * 1024;
+    const bool asked = str_or(o, "perf_config", "").find("224,128,") != std::string::npos;
+    if (direct_ok && asked) {
+      // rows per tile: the most that fit, unless a slightly shorter tile fills
+      // the last round of blocks better (cost = rounds x (rows + ~2 rows of
+      // window halo and epilogue per tile))
+      int64_t best_th = th;
+      const int64_t per_round = (int64_t)kNumCU;
+      auto cost = [&](int64_t rows) {
+        int64_t tiles = (int64_t)ceil_div(n * ho, rows) * ceil_div(k, 128) * g;
+        return ((tiles + per_round - 1) / per_round) * (rows + 2);
+      };
+      for (int64_t rows = th - 1; rows >= std::max<int64_t>(1, th / 2); --rows)
+        if (cost(rows) < cost(best_th))
+          best_th = rows;
+      const int64_t th = best_th;
+      p.rows_per_tile = (int)th;
+      p.tiles_m = ceil_div(n * ho, th);
+      p.tiles_n = ceil_div(k, 128);
+      p.group_m = std::min(p.tiles_m, 8);
+      int64_t total = (int64_t)p.tiles_m * p.tiles_n * g;
+      p.xcd_remap = total >= 2 * kNumXCD ? 1 : 0;
+      h->block_size = 512;
+      h->grid_size = (uint32_t)total;
+      h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + "_direct224";
+      char buf[96];
+      std::snprintf(buf, sizeof buf, "v2:224,128,8,224,32,%d,1,1,1", 16 / es);
+      h->perf_config = buf;
+    }
+  }
   {
     std::ostringstream key;
     const char *opname = ti == ROCK_F32 ? "conv" : ti == ROCK_F16 ? "convfp16"

@@ -129,6 +129,58 @@ def test_conv_every_fast_tile(rock, oracle, gpu, tile):
     assert np.array_equal(to_f32(out, od), ref)
 
 
+# The window-resident kernel ("-perf_config v2:224,128,..."): stride 1, dilation 1.
+# (n g pixel_bytes k hi wi y x pad); the channel count follows from the element size.
+WINDOW_CASES = [
+    (3, 1, 128, 128, 28, 28, 3, 3, (1, 1)),  # 8-row tiles over 28-row images: tiles straddle images
+    (5, 1, 256, 96, 9, 7, 3, 3, (1, 1)),     # whole small images per tile, 96 of 128 output channels
+    (4, 1, 128, 32, 30, 30, 3, 3, (0, 1)),   # 28x30 outputs, padding in one direction only
+    (3, 1, 128, 64, 10, 12, 3, 3, (1, 1)),   # 18-row tiles capped at the image height of 10
+    (7, 1, 128, 48, 6, 50, 3, 3, (1, 1)),    # 4-row tiles against 6-row images: tiles straddle images
+    (2, 2, 128, 40, 12, 20, 3, 5, (1, 2)),   # two groups, 3x5 filter
+    (2, 1, 128, 130, 10, 33, 2, 2, (0, 0)),  # even filter, no padding, two blocks of output channels
+    (1, 1, 512, 64, 6, 6, 5, 5, (2, 2)),     # 512-byte pixels, 5x5 filter
+]
+
+
+@pytest.mark.parametrize("case", WINDOW_CASES)
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16", "i8"])
+def test_conv_window_resident_kernel_exact(rock, oracle, gpu, case, t):
+    n, g, pixel_bytes, k, hi, wi, y, x, pad = case
+    c = pixel_bytes // {"f32": 4, "f16": 2, "bf16": 2, "i8": 1}[t]
+    info = {}
+    out, od, ref = _run(rock, oracle, gpu, t, n, g, c, k, hi, wi, y, x, (1, 1), pad, (1, 1), NHWC, True, 41,
+                        perf_config="v2:224,128,8,224,32,8,1,1,1", info=info)
+    assert info["kernel_name"] == "rock_conv_%s_direct224" % t
+    if t == "i8":
+        assert oracle.verify_int(out.cpu().numpy().ravel(), ref)[0] == 0
+    else:
+        # integer data: every partial sum is exact in f32; only the final
+        # narrowing rounds (sums of up to 1152 terms exceed bf16's 8 bits)
+        assert np.array_equal(to_f32(out, od), oracle.round_through(ref, CODE[od]))
+
+
+def test_conv_window_resident_kernel_real_values_and_epilogue(rock, oracle, gpu):
+    """Real-valued f16 data through the window-resident kernel with a ReLU and
+    an f32 output, against the oracle with the reference's RMS gate."""
+    info = {}
+    out, od, ref = _run(rock, oracle, gpu, "f16", 4, 1, 128, 128, 28, 28, 3, 3, (1, 1), (1, 1), (1, 1),
+                        NHWC, False, 43, out_dtype="f32", relu=True, perf_config="v2:224,128,8,224,32,8,1,1,1",
+                        info=info)
+    assert info["kernel_name"] == "rock_conv_f16_direct224"
+    check_float(to_f32(out, od), np.maximum(ref, 0.0), od)
+
+
+def test_conv_window_resident_request_falls_back(rock, oracle, gpu):
+    """A stride-2 problem cannot use the window-resident kernel: the request
+    falls back to the table (tuningFallback, AffixTuningParameters.cpp:129-141)."""
+    info = {}
+    out, od, ref = _run(rock, oracle, gpu, "f16", 2, 1, 64, 32, 14, 14, 3, 3, (2, 2), (1, 1), (1, 1),
+                        NHWC, True, 45, perf_config="v2:224,128,8,224,32,8,1,1,1", info=info)
+    assert "direct" not in info["kernel_name"]
+    assert np.array_equal(to_f32(out, od), ref)
+
+
 def test_conv_i8_dequantise_per_tensor(rock, oracle, gpu):
     # int8 conv 3x3 s2 p1 -> dequantize (mixr-resnet-fusion-case-1-quantization.mlir chain)
     out, od, ref = _run(rock, oracle, gpu, "i8", 2, 1, 16, 32, 14, 14, 3, 3, (2, 2), (1, 1), (1, 1),
