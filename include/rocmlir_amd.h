@@ -136,6 +136,57 @@ ROCMLIR_AMD_API MiirStatus rockamdSetScale(MiirHandle handle, float scale);
 ROCMLIR_AMD_API MiirStatus rockamdSetZeroPoint(MiirHandle handle, int32_t zero_point);
 
 /* ---------------------------------------------------------------------------
+ * 2b. Tuning surface (mlir-c/Dialect/Rock.h:39-148; implementation
+ *     mlir/lib/Dialect/Rock/Tuning/RockTuningImpl.cpp:461-548,902-1015).
+ *     The reference enumerates a grid of block/wave tile sizes; here the
+ *     space of a problem is the list of hand-written kernels it can run on,
+ *     each named by a perf_config string in the reference's "v2:" grammar.
+ * ------------------------------------------------------------------------- */
+typedef void *RockamdTuningSpace;
+typedef void *RockamdTuningTable;
+
+/* RocmlirTuningParamSetKind (RockEnums.h:19-23); both kinds return the same short list. */
+enum { ROCKAMD_TUNING_QUICK = 0, ROCKAMD_TUNING_FULL = 1 };
+/* RocmlirSplitKSelectionLikelihood (RockEnums.h:26) */
+enum { ROCKAMD_SPLITK_NEVER = 0, ROCKAMD_SPLITK_MAYBE = 1, ROCKAMD_SPLITK_ALWAYS = 2 };
+
+/* mlirRockTuningSpaceCreate / mlirRockTuningGetNumParams /
+ * mlirRockTuningParamGet + mlirRockTuningParamToString / mlirRockTuningSpaceDestroy
+ * (Rock.h:39-84).  Entry 0 is the kernel the built-in table picks.  ToString
+ * copies like strncpy (no terminator if the buffer is too small) and returns
+ * the full length, (size_t)-1 for a bad position. */
+ROCMLIR_AMD_API RockamdTuningSpace rockamdTuningSpaceCreate(MiirHandle handle, int kind);
+ROCMLIR_AMD_API unsigned rockamdTuningGetNumParams(RockamdTuningSpace space);
+ROCMLIR_AMD_API size_t rockamdTuningParamToString(RockamdTuningSpace space, unsigned pos, char *buffer,
+                                                  size_t buffer_size);
+ROCMLIR_AMD_API void rockamdTuningSpaceDestroy(RockamdTuningSpace space);
+
+/* mlirRockTuningSetFromStr (Rock.h:90-92): re-resolves the handle's kernel
+ * under the given perf_config; a string that names no applicable kernel falls
+ * back to the table (AffixTuningParameters.cpp:129-141).  Returns 1 on
+ * success; fetch the code object, launch dimensions and parameter block again. */
+ROCMLIR_AMD_API int rockamdTuningSetFromStr(MiirHandle handle, const char *perf_config);
+
+/* mlirRockTuningTableCreate / Destroy / mlirRockTuningUpdateTable /
+ * mlirRockTuningSetFromTable (Rock.h:94-117): an in-memory map from problem
+ * key (rockamdGetProblemKey) to the best perf_config seen.  Update returns 1
+ * if the entry was stored, 0 if a better-performing one exists; SetFromTable
+ * returns 1 if the problem was found and applied. */
+ROCMLIR_AMD_API RockamdTuningTable rockamdTuningTableCreate(void);
+ROCMLIR_AMD_API void rockamdTuningTableDestroy(RockamdTuningTable table);
+ROCMLIR_AMD_API int rockamdTuningUpdateTable(RockamdTuningTable table, const char *problem_key,
+                                             const char *perf_config, float time);
+ROCMLIR_AMD_API int rockamdTuningSetFromTable(RockamdTuningTable table, MiirHandle handle);
+
+/* mlirIsSplitKFaster (Rock.h:136-142, RockTuningImpl.cpp:962-1008), answered
+ * for this library's split-K kernel (K divided over the waves of one block):
+ * ALWAYS when the built-in table itself would choose it (64x64 tiles would
+ * occupy at most half the CUs and K is at least 1 KiB), MAYBE while the tile
+ * count does not exceed the CUs, NEVER otherwise.  element_size in bytes. */
+ROCMLIR_AMD_API int rockamdIsSplitKFaster(int64_t g, int64_t m, int64_t n, int64_t k, int64_t num_cu,
+                                          int element_size);
+
+/* ---------------------------------------------------------------------------
  * 3. Launch helpers (the client side of rocmlir-tuning-driver.cpp:131-185)
  * ------------------------------------------------------------------------- */
 

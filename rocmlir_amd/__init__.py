@@ -12,3 +12,4 @@ from .api import (RockError, RockKernel, attention, conv2d, gemm,  # noqa: F401
 
 __all__ = ["RockError", "RockKernel", "gemm", "conv2d", "attention",
            "library_path", "load_library", "mfma_rate"]
+# rocmlir_amd.tuning (tuning table + in-process tuner) is imported on demand

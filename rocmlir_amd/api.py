@@ -76,6 +76,27 @@ def load_library():
                                              C.POINTER(C.c_double)]
         L.rockamdGetLastError.restype = C.c_char_p
         L.rockamdGetLastError.argtypes = []
+        L.rockamdTuningSpaceCreate.restype = vp
+        L.rockamdTuningSpaceCreate.argtypes = [vp, C.c_int]
+        L.rockamdTuningGetNumParams.restype = C.c_uint
+        L.rockamdTuningGetNumParams.argtypes = [vp]
+        L.rockamdTuningParamToString.restype = sz
+        L.rockamdTuningParamToString.argtypes = [vp, C.c_uint, C.c_char_p, sz]
+        L.rockamdTuningSpaceDestroy.restype = None
+        L.rockamdTuningSpaceDestroy.argtypes = [vp]
+        L.rockamdTuningSetFromStr.restype = C.c_int
+        L.rockamdTuningSetFromStr.argtypes = [vp, C.c_char_p]
+        L.rockamdTuningTableCreate.restype = vp
+        L.rockamdTuningTableCreate.argtypes = []
+        L.rockamdTuningTableDestroy.restype = None
+        L.rockamdTuningTableDestroy.argtypes = [vp]
+        L.rockamdTuningUpdateTable.restype = C.c_int
+        L.rockamdTuningUpdateTable.argtypes = [vp, C.c_char_p, C.c_char_p,
+                                               C.c_float]
+        L.rockamdTuningSetFromTable.restype = C.c_int
+        L.rockamdTuningSetFromTable.argtypes = [vp, vp]
+        L.rockamdIsSplitKFaster.restype = C.c_int
+        L.rockamdIsSplitKFaster.argtypes = [C.c_int64] * 5 + [C.c_int]
         _lib = L
         return _lib
 
@@ -113,6 +134,12 @@ class RockKernel:
         if not self._h:
             raise RockError("miirCreateHandle failed: %s [%s]"
                             % (last_error(), options))
+        self._refresh()
+
+    def _refresh(self):
+        """(Re)reads what describes the resolved kernel; called after
+        creation and after a perf_config has been applied."""
+        L = load_library()
         if L.miirLowerTuningParams(self._h) != MIIR_SUCCESS:
             raise RockError("miirLowerTuningParams failed")
         if L.miirLowerBin(self._h) != MIIR_SUCCESS:
@@ -176,6 +203,35 @@ class RockKernel:
         if rc != MIIR_SUCCESS:
             raise RockError("miirGetExecutionDims failed (%d)" % rc)
         return g.value, l.value
+
+    # ---- tuning (mlir-c/Dialect/Rock.h:39-117) -------------------------------
+    def tuning_space(self, full=False):
+        """perf_config strings of the kernels this problem can run on; the
+        first is the built-in table's choice."""
+        L = load_library()
+        sp = L.rockamdTuningSpaceCreate(self._h, 1 if full else 0)
+        if not sp:
+            raise RockError("rockamdTuningSpaceCreate failed")
+        try:
+            out = []
+            for i in range(L.rockamdTuningGetNumParams(sp)):
+                buf = C.create_string_buffer(128)
+                n = L.rockamdTuningParamToString(sp, i, buf, 128)
+                if n == C.c_size_t(-1).value or n >= 128:
+                    raise RockError("rockamdTuningParamToString failed")
+                out.append(buf.value.decode())
+            return out
+        finally:
+            L.rockamdTuningSpaceDestroy(sp)
+
+    def set_perf_config(self, perf_config):
+        """Re-resolves the kernel under `perf_config`
+        (mlirRockTuningSetFromStr); unknown strings fall back to the table."""
+        if not load_library().rockamdTuningSetFromStr(self._h,
+                                                      perf_config.encode()):
+            raise RockError("rockamdTuningSetFromStr(%r) failed: %s"
+                            % (perf_config, last_error()))
+        self._refresh()
 
     def set_scale(self, scale):
         load_library().rockamdSetScale(self._h, float(scale))

@@ -251,6 +251,7 @@ struct Handle {
   std::string perf_config;
   std::string problem_key;
   bool tuned = false, lowered = false;
+  OptMap options; // the parsed problem, kept so that a perf_config can be applied later
   // typed views of `params`
   RockEpilogue *epi = nullptr;
   // launch cache: device -> function
@@ -839,20 +840,8 @@ bool check_launch_args(Handle *h, void *const *pointers, int num_pointers) {
   return true;
 }
 
-} // namespace
-
-// ============================================================================
-// C ABI
-// ============================================================================
-extern "C" {
-
-MiirHandle miirCreateHandle(const char *options) {
-  g_last_error.clear();
-  OptMap o;
-  if (!parse_options(options, o)) {
-    set_error("could not parse the options string");
-    return nullptr;
-  }
+// problem description -> resolved kernel; NULL with the error set on failure
+Handle *build_handle(const OptMap &o) {
   // arch: "[triple:]gfxNNN[:features]" (ConvGenerator.cpp:538-552); only
   // gfx950 has kernels here
   std::string arch = str_or(o, "arch", "gfx950");
@@ -891,7 +880,69 @@ MiirHandle miirCreateHandle(const char *options) {
     delete h;
     return nullptr;
   }
+  h->options = o;
   return h;
+}
+
+// The perf_config strings worth trying for a problem: one per distinct kernel
+// the problem can run on (a request that does not fit falls back to the
+// table's choice and is dropped as a duplicate).  The reference enumerates
+// its parameter grid instead (createGemmTuningRangeBF / the quick lists,
+// RockTuningImpl.cpp:461-548); here the grid is the handful of hand-written
+// tiles.
+std::vector<std::string> tuning_candidates(const Handle &h) {
+  std::vector<std::string> requests;
+  requests.push_back(""); // the table's own choice comes first
+  if (h.op != OP_ATTENTION) {
+    for (const Tile &t : kFastTiles)
+      requests.push_back(perf_string(t, 1));
+    requests.push_back("v2:32,32,4,32,32,16,4,1,1");    // K split over the block's waves (GEMM)
+    requests.push_back("v2:224,128,8,224,32,16,1,1,1"); // window-resident convolution
+  }
+  std::vector<std::string> out, seen;
+  const std::string keep_error = g_last_error;
+  for (const std::string &r : requests) {
+    OptMap o = h.options;
+    o.erase("perf_config");
+    if (!r.empty())
+      o["perf_config"] = r;
+    Handle *c = build_handle(o);
+    if (!c)
+      continue;
+    if (std::find(seen.begin(), seen.end(), c->kernel_name) == seen.end()) {
+      seen.push_back(c->kernel_name);
+      out.push_back(c->perf_config);
+    }
+    delete c;
+  }
+  g_last_error = keep_error;
+  return out;
+}
+
+struct TuningSpace {
+  std::vector<std::string> params;
+};
+
+// problem key -> best perf_config seen and its time (mlirRockTuningUpdateTable keeps only the best)
+struct TuningTable {
+  std::map<std::string, std::pair<std::string, float>> best;
+};
+
+} // namespace
+
+// ============================================================================
+// C ABI
+// ============================================================================
+extern "C" {
+
+MiirHandle miirCreateHandle(const char *options) {
+  g_last_error.clear();
+  OptMap o;
+  if (!parse_options(options, o)) {
+    set_error("could not parse the options string");
+    return nullptr;
+  }
+  return build_handle(o);
 }
 
 int miirGetKernelCount(MiirHandle handle) { return handle ? 1 : -1; }
@@ -1149,6 +1200,85 @@ int rockamdMeasureMfmaRate(int dtype, int random_data, void *stream, double *ter
   double ops = 2.0 * macs[dtype] * 4.0 * iters * 4.0 * blocks;
   *tera_ops = ops / (ms * 1e-3) / 1e12;
   return 0;
+}
+
+// ---- tuning surface ---------------------------------------------------------
+RockamdTuningSpace rockamdTuningSpaceCreate(MiirHandle handle, int kind) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h || (kind != ROCKAMD_TUNING_QUICK && kind != ROCKAMD_TUNING_FULL))
+    return nullptr;
+  auto *sp = new TuningSpace;
+  sp->params = tuning_candidates(*h); // the quick and the full list coincide: a handful of kernels
+  return sp;
+}
+
+unsigned rockamdTuningGetNumParams(RockamdTuningSpace space) {
+  return space ? (unsigned)static_cast<TuningSpace *>(space)->params.size() : 0u;
+}
+
+size_t rockamdTuningParamToString(RockamdTuningSpace space, unsigned pos, char *buffer, size_t buffer_size) {
+  auto *sp = static_cast<TuningSpace *>(space);
+  if (!sp || pos >= sp->params.size())
+    return (size_t)-1;
+  const std::string &s = sp->params[pos];
+  if (buffer && buffer_size)
+    std::strncpy(buffer, s.c_str(), buffer_size);
+  return s.size();
+}
+
+void rockamdTuningSpaceDestroy(RockamdTuningSpace space) { delete static_cast<TuningSpace *>(space); }
+
+int rockamdTuningSetFromStr(MiirHandle handle, const char *perf_config) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h || !perf_config)
+    return 0;
+  OptMap o = h->options;
+  o["perf_config"] = perf_config;
+  Handle *n = build_handle(o);
+  if (!n)
+    return 0;
+  *n->epi = *h->epi; // scalars changed with rockamdSetScale / SetZeroPoint stay
+  *h = std::move(*n); // params moves with its buffer, so the typed views stay valid
+  delete n;
+  return 1;
+}
+
+RockamdTuningTable rockamdTuningTableCreate(void) { return new TuningTable; }
+
+void rockamdTuningTableDestroy(RockamdTuningTable table) { delete static_cast<TuningTable *>(table); }
+
+int rockamdTuningUpdateTable(RockamdTuningTable table, const char *problem_key, const char *perf_config,
+                             float time) {
+  auto *t = static_cast<TuningTable *>(table);
+  if (!t || !problem_key || !perf_config)
+    return 0;
+  auto it = t->best.find(problem_key);
+  if (it != t->best.end() && it->second.second <= time)
+    return 0; // a better-performing entry exists
+  t->best[problem_key] = std::make_pair(std::string(perf_config), time);
+  return 1;
+}
+
+int rockamdTuningSetFromTable(RockamdTuningTable table, MiirHandle handle) {
+  auto *t = static_cast<TuningTable *>(table);
+  auto *h = static_cast<Handle *>(handle);
+  if (!t || !h)
+    return 0;
+  auto it = t->best.find(h->problem_key);
+  if (it == t->best.end())
+    return 0;
+  return rockamdTuningSetFromStr(handle, it->second.first.c_str());
+}
+
+int rockamdIsSplitKFaster(int64_t g, int64_t m, int64_t n, int64_t k, int64_t num_cu, int element_size) {
+  if (g <= 0 || m <= 0 || n <= 0 || k <= 0 || num_cu <= 0 || element_size <= 0)
+    return ROCKAMD_SPLITK_NEVER;
+  if (k * element_size < 16 * 64)
+    return ROCKAMD_SPLITK_NEVER; // a K range this short gives each wave less than one 64-byte step
+  const int64_t tiles64 = (int64_t)ceil_div(m, 64) * ceil_div(n, 64) * g;
+  if (tiles64 * 2 <= num_cu)
+    return ROCKAMD_SPLITK_ALWAYS; // make_gemm's own rule: 64x64 tiles would leave half the CUs idle
+  return tiles64 <= num_cu ? ROCKAMD_SPLITK_MAYBE : ROCKAMD_SPLITK_NEVER;
 }
 
 const char *rockamdGetLastError(void) { return g_last_error.c_str(); }

@@ -166,6 +166,93 @@ def test_param_block_and_setters(rock):
     assert (scale, zp) == (0.25, -2)
 
 
+def test_tuning_space_lists_the_kernels_a_problem_can_run_on(rock):
+    """mlirRockTuningSpaceCreate / GetNumParams / ParamGet / ToString
+    (mlir-c/Dialect/Rock.h:39-84): entry 0 is the table's choice, every entry
+    selects a different kernel, and strings follow the v2 grammar."""
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 4096 -n 4096 -k 4096 -transB true")
+    space = k.tuning_space()
+    assert space[0] == k.perf_config
+    assert space == k.tuning_space(full=True)
+    names = []
+    for perf in space:
+        assert re.fullmatch(r"v2:\d+(,\d+){8}", perf)
+        k.set_perf_config(perf)
+        assert k.perf_config == perf
+        names.append(k.kernel_name)
+    assert len(set(names)) == len(names) == 5  # four tiles and the K-split kernel
+    # a convolution the window-resident kernel can run offers it; attention has one kernel
+    assert "v2:224,128,8,224,32,8,1,1,1" in rock.RockKernel(CONV_RESNET).tuning_space()
+    att = rock.RockKernel("--arch gfx950 --operation attention -seq_len_q 256 -seq_len_k 512 "
+                          "-head_dim_qk 64 -head_dim_v 64 -t f16 -g 4 -transK true")
+    assert att.tuning_space() == [att.perf_config]
+    # operands that are not K-contiguous only have the generic kernel
+    gen = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 256 -n 256 -k 256")
+    assert gen.tuning_space() == [gen.perf_config]
+    # raw entry points: bad position, short buffer
+    lib = rock.load_library()
+    sp = lib.rockamdTuningSpaceCreate(k._h, 0)
+    assert lib.rockamdTuningGetNumParams(sp) == 5
+    assert lib.rockamdTuningParamToString(sp, 99, None, 0) == C.c_size_t(-1).value
+    buf = C.create_string_buffer(b"\xff" * 8, 8)
+    n = lib.rockamdTuningParamToString(sp, 0, buf, 4)
+    assert n == len(space[0]) and buf.raw[:4] == space[0][:4].encode() and buf.raw[4:] == b"\xff" * 4
+    lib.rockamdTuningSpaceDestroy(sp)
+    assert lib.rockamdTuningSpaceCreate(None, 0) is None
+    assert lib.rockamdTuningSpaceCreate(k._h, 7) is None
+
+
+def test_set_perf_config_keeps_epilogue_scalars_and_launch_geometry(rock):
+    import struct
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t i8 -out_datatype f16 -g 1 -m 1024 -n 1024 -k 1024 "
+                        "-transB true -scale 0.5")
+    k.set_scale(0.125)
+    k.set_perf_config("v2:64,64,8,32,16,16,1,1,1")
+    assert k.kernel_name == "rock_gemm_i8_64x64_fast"
+    assert (k.block_size, k.grid_size) == (256, 16 * 16)
+    assert k.execution_dims() == (256 * 256, 256)
+    assert struct.unpack_from("f", k.params(), 72 + 32)[0] == 0.125
+    assert len(k.code_object()) > 1000
+
+
+def test_tuning_table_keeps_the_best_entry(rock, tmp_path):
+    """mlirRockTuningUpdateTable / SetFromTable (Rock.h:94-117)."""
+    from rocmlir_amd import tuning
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 4096 -n 4096 -k 4096 -transB true")
+    other = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 512 -n 4096 -k 4096 -transB true")
+    t = tuning.TuningTable()
+    assert not t.apply(k)
+    assert t.update(k.problem_key, "v2:64,64,8,32,16,8,1,1,1", 2.0)
+    assert t.update(k.problem_key, "v2:128,128,8,64,16,8,1,1,1", 1.0)      # faster: replaces
+    assert not t.update(k.problem_key, "v2:64,64,8,32,16,8,1,1,1", 1.5)   # slower: refused
+    assert t.apply(k) and k.kernel_name == "rock_gemm_f16_128x128_fast"
+    untouched = other.kernel_name
+    assert not t.apply(other) and other.kernel_name == untouched
+    # the text form is the reference's four-column tuning database
+    path = tmp_path / "gfx950.tuning"
+    t.save(str(path))
+    line = path.read_text().splitlines()
+    assert len(line) == 1 and line[0].split("\t") == ["gfx950", "256", k.problem_key.split("\t")[2],
+                                                      "v2:128,128,8,64,16,8,1,1,1"]
+    again = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 4096 -n 4096 -k 4096 -transB true")
+    assert tuning.TuningTable.load(str(path)).apply(again)
+    assert again.kernel_name == "rock_gemm_f16_128x128_fast"
+
+
+def test_split_k_likelihood(rock):
+    """mlirIsSplitKFaster (Rock.h:136-142) for this library's K-split kernel:
+    ALWAYS exactly where the built-in table picks it."""
+    lib = rock.load_library()
+    never, maybe, always = 0, 1, 2
+    assert lib.rockamdIsSplitKFaster(1, 512, 512, 512, 256, 4) == always
+    assert rock.RockKernel("-operation gemm -arch gfx950 -t f32 -g 1 -m 512 -n 512 -k 512 "
+                           "-transB true").kernel_name.endswith("_splitk")
+    assert lib.rockamdIsSplitKFaster(1, 1024, 1024, 4096, 256, 2) == maybe
+    assert lib.rockamdIsSplitKFaster(1, 4096, 4096, 4096, 256, 1) == never
+    assert lib.rockamdIsSplitKFaster(1, 64, 64, 64, 256, 2) == never   # K too short to split
+    assert lib.rockamdIsSplitKFaster(0, 64, 64, 4096, 256, 2) == never
+
+
 def test_product_does_not_touch_the_oracle():
     """The shipped package must not import, load or link the CPU oracle."""
     pkg = os.path.join(ROOT, "rocmlir_amd")
