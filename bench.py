@@ -168,7 +168,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (every box has one); --gpus %d is not "
-                 "supported -- the path shards without exchange (see DESIGN.md) but no multi-GPU "
+                 "supported -- the path shards without exchange (GEMM by rows, conv by batch, attention "
+                 "by batch x heads) but no multi-GPU "
                  "figure is produced here" % args.gpus)
 
     import torch
