@@ -336,11 +336,13 @@ def _epilogue_flags(scale, zero_point, bias, relu, quant_scale, out_zero_point):
 
 def gemm(a, b, *, transA=False, transB=False, transC=False, out_dtype=None,
          scale=None, zero_point=0, bias=None, relu=False, quant_scale=None,
-         out_zero_point=0, out=None, perf_config=None, stream=None):
+         out_zero_point=0, out=None, perf_config=None, stream=None,
+         info=None):
     """C = epilogue(A x B) with the reference's storage conventions
     (rocmlir-gen.cpp:2058-2080): a is [G,M,K] ([G,K,M] if transA), b is
     [G,K,N] ([G,N,K] if transB), result [G,M,N] ([G,N,M] if transC).
-    2-D inputs mean G = 1."""
+    2-D inputs mean G = 1.  A dict passed as `info` receives the name and
+    perf_config of the kernel that ran."""
     import torch
     a3 = a if a.dim() == 3 else a.unsqueeze(0)
     b3 = b if b.dim() == 3 else b.unsqueeze(0)
@@ -363,6 +365,9 @@ def gemm(a, b, *, transA=False, transB=False, transC=False, out_dtype=None,
     opts += _epilogue_flags(scale, zero_point, bias, relu, quant_scale,
                             out_zero_point)
     k = _kernel(opts)
+    if info is not None:
+        info["kernel_name"] = k.kernel_name
+        info["perf_config"] = k.perf_config
     if out_dtype is None:
         out_dtype = {"i8": "i32", "fp8": "f32", "bf8": "f32"}.get(ta, ta)
     shape = (G, N, M) if transC else (G, M, N)

@@ -213,18 +213,151 @@ template <int DT, int ROWS, int NW, int RB> struct ConvInDl {
   }
 };
 
+// ---------------------------------------------------------------------------
+// K-major operands (A stored [K, M], B stored [K, N]: the contiguous index is
+// the tile's row index, not K).  A stage holds the same bytes as for a
+// K-contiguous operand, but as KR = RB/ES rows of k, each COLS*ES bytes of
+// consecutive m (or n).  MFMA fragments need 16 bytes of consecutive k per
+// lane, so they come out of LDS through the transposing reads
+// (ds_read_b64_tr_b16 / _b8: 16 lanes fetch a 4 x 16 block of 16-bit or an
+// 8 x 16 block of 8-bit elements and each lane receives one column), 32-bit
+// elements through four scalar reads.  The reference reaches the same layouts
+// through its generic coordinate transforms (GridwiseGemmToBlockwise.cpp:
+// 2602-2760 loads "KxD" tiles for either operand orientation).
+// ---------------------------------------------------------------------------
+template <int DT, int COLS, int RB> struct KmGeom {
+  static constexpr int ES = MmaTraits<DT>::ES;
+  static constexpr int ROWB = COLS * ES;  // bytes per k-row
+  static constexpr int KR = RB / ES;      // k-rows per stage
+  static constexpr int CPR = ROWB / kChunk;
+  static constexpr int SLAB_ROWS = 1024 / ROWB;
+  static_assert(ROWB >= 64 && ROWB <= 1024 && 1024 % ROWB == 0, "a 1 KiB load slab is a whole number of k-rows");
+  // Chunk swizzle.  A transposing read touches 4 (16-bit) or 8 (8-bit)
+  // consecutive k-rows at the same columns; rows are a multiple of the bank
+  // period apart, so each of those rows is moved to its own 64- or 32-byte
+  // column group.  The 32-bit path reads one row per instruction and only has
+  // to keep the two wave halves (4 rows apart) on different bank halves.
+  static __device__ __forceinline__ int swz(int row) {
+    int x = ES == 2 ? ((row & 3) << 2) : ES == 1 ? ((row & 7) << 1) : (((row >> 2) & 1) << 3);
+    return x & (CPR - 1);
+  }
+};
+
+template <int DT, int COLS, int NW, int RB> struct ColsDl {
+  using Kg = KmGeom<DT, COLS, RB>;
+  struct Sg { // same slab count as a K-contiguous tile of the same bytes
+    static constexpr int SLABS = COLS * RB / 1024;
+    static constexpr int PER_WAVE = SLABS / NW;
+    static_assert(SLABS % NW == 0, "stage must split into 1 KiB slabs per wave");
+  };
+  static constexpr int ES = Kg::ES;
+  __amdgpu_buffer_rsrc_t rsrc;
+  unsigned off[Sg::PER_WAVE]; // byte offset of this lane's chunk at K-step 0, or kOobOffset
+  int krow[Sg::PER_WAVE];     // k-row of the chunk inside a stage
+  int kstride_b;              // bytes between consecutive k
+  int K;
+  int wave;
+
+  __device__ __forceinline__ void init(const void *base, int64_t k_stride, int col0, int cols_total, int K_,
+                                       int wave_, int lane) {
+    wave = wave_;
+    K = K_;
+    kstride_b = (int)k_stride * ES;
+    rsrc = dl_rsrc((const char *)base + (int64_t)col0 * ES);
+#pragma unroll
+    for (int i = 0; i < Sg::PER_WAVE; ++i) {
+      const int idx = (wave * Sg::PER_WAVE + i) * 64 + lane; // physical chunk inside the stage
+      const int r = idx / Kg::CPR, pc = idx % Kg::CPR;
+      const int lc = pc ^ Kg::swz(r);                        // logical chunk this lane fetches
+      krow[i] = r;
+      const bool col_ok = col0 + (lc + 1) * (kChunk / ES) <= cols_total;
+      off[i] = col_ok ? (unsigned)(r * kstride_b + lc * kChunk) : kOobOffset;
+    }
+  }
+  __device__ __forceinline__ void issue(int kt, char *stage) {
+    const int k0 = kt * Kg::KR;
+#pragma unroll
+    for (int i = 0; i < Sg::PER_WAVE; ++i) {
+      unsigned voff = (k0 + krow[i] < K) ? off[i] + (unsigned)(k0 * kstride_b) : kOobOffset;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrc, (lds_void_t *)(stage + (wave * Sg::PER_WAVE + i) * 1024), 16, (int)voff, 0, 0, 0);
+    }
+  }
+};
+
+typedef __attribute__((address_space(3))) v4s km_lds_v4s_t;
+typedef __attribute__((address_space(3))) v2i km_lds_v2i_t;
+
+// Fragment of the 32 columns [colblock, colblock + 32) of a K-major stage, same
+// k assignment as dl_read_frag: lane (col = lane % 32, half = lane / 32) gets
+// the 16 bytes of k-chunk  step*2*CHUNKS + 2*c + half.
+template <int DT, int COLS, int RB>
+__device__ __forceinline__ Frag<DT> dl_read_frag_km(const char *stage, int colblock, int step, int lane) {
+  using Kg = KmGeom<DT, COLS, RB>;
+  constexpr int ES = Kg::ES, CH = MmaTraits<DT>::CHUNKS;
+  const int l16 = lane & 15, g16 = (lane >> 4) & 1, half = lane >> 5;
+  Frag<DT> f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int kb = (step * 2 * CH + 2 * c + half) * (kChunk / ES); // first k-row of the chunk
+    if constexpr (ES == 2) {
+      const int colbyte = (colblock + 16 * g16 + 4 * (l16 & 3)) * 2;
+      v2i part[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int row = kb + 4 * j + (l16 >> 2);
+        const char *a = stage + row * Kg::ROWB + ((((colbyte >> 4) ^ Kg::swz(row))) << 4) + (colbyte & 15);
+        part[j] = __builtin_bit_cast(v2i, __builtin_amdgcn_ds_read_tr16_b64_v4i16((km_lds_v4s_t *)a));
+      }
+      f.c[c] = v4i{part[0][0], part[0][1], part[1][0], part[1][1]};
+    } else if constexpr (ES == 1) {
+      const int colbyte = colblock + 16 * g16 + 8 * (l16 & 1);
+      v2i part[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int row = kb + 8 * j + (l16 >> 1);
+        const char *a = stage + row * Kg::ROWB + ((((colbyte >> 4) ^ Kg::swz(row))) << 4) + (colbyte & 15);
+        part[j] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((km_lds_v2i_t *)a);
+      }
+      f.c[c] = v4i{part[0][0], part[0][1], part[1][0], part[1][1]};
+    } else {
+      const int colbyte = (colblock + (lane & 31)) * 4;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int row = kb + t;
+        f.c[c][t] = *(const int *)(stage + row * Kg::ROWB + ((((colbyte >> 4) ^ Kg::swz(row))) << 4) + (colbyte & 15));
+      }
+    }
+  }
+  return f;
+}
+
 template <int DT, int ROWS, int NW, int RB, int KIND>
 __device__ __forceinline__ auto make_dl_a(const void *A, const RockGemmParams &p, int g, int m0, int wave, int lane) {
-  static_assert(KIND == LD_ROWS_FAST, "GEMM fast path loads K-contiguous rows");
-  RowsDl<DT, ROWS, NW, RB> l;
-  l.init((const char *)A + (int64_t)g * p.a_gs * MmaTraits<DT>::ES, p.a_ms, m0, p.M, p.K, wave, lane);
-  return l;
+  static_assert(KIND == LD_ROWS_FAST || KIND == LD_COLS_FAST, "GEMM fast paths: K-contiguous or K-major");
+  const char *base = (const char *)A + (int64_t)g * p.a_gs * MmaTraits<DT>::ES;
+  if constexpr (KIND == LD_COLS_FAST) {
+    ColsDl<DT, ROWS, NW, RB> l;
+    l.init(base, p.a_ks, m0, p.M, p.K, wave, lane);
+    return l;
+  } else {
+    RowsDl<DT, ROWS, NW, RB> l;
+    l.init(base, p.a_ms, m0, p.M, p.K, wave, lane);
+    return l;
+  }
 }
 template <int DT, int ROWS, int NW, int RB, int KIND>
 __device__ __forceinline__ auto make_dl_b(const void *B, const RockGemmParams &p, int g, int n0, int wave, int lane) {
-  RowsDl<DT, ROWS, NW, RB> l;
-  l.init((const char *)B + (int64_t)g * p.b_gs * MmaTraits<DT>::ES, p.b_ns, n0, p.N, p.K, wave, lane);
-  return l;
+  const char *base = (const char *)B + (int64_t)g * p.b_gs * MmaTraits<DT>::ES;
+  if constexpr (KIND == LD_COLS_FAST) {
+    ColsDl<DT, ROWS, NW, RB> l;
+    l.init(base, p.b_ks, n0, p.N, p.K, wave, lane);
+    return l;
+  } else {
+    RowsDl<DT, ROWS, NW, RB> l;
+    l.init(base, p.b_ns, n0, p.N, p.K, wave, lane);
+    return l;
+  }
 }
 template <int DT, int ROWS, int NW, int RB, int KIND>
 __device__ __forceinline__ auto make_dl_a(const void *in, const RockConvParams &p, int g, int m0, int wave, int lane) {
@@ -370,7 +503,7 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
   const int lwave = loader ? wave - (NW - NLOAD) : 0;
   auto la = make_dl_a<DT, BM, NLOAD, RB, LDA>(Aptr, p, g, m0, lwave, lane);
   auto lb = make_dl_b<DT, BN, NLOAD, RB, LDB>(Bptr, p, g, n0, lwave, lane);
-  constexpr int LOADS_PER_STEP = SlabGeom<BM, NLOAD, RB>::PER_WAVE + SlabGeom<BN, NLOAD, RB>::PER_WAVE;
+  constexpr int LOADS_PER_STEP = decltype(la)::Sg::PER_WAVE + decltype(lb)::Sg::PER_WAVE;
 
   Acc acc[MI][NI];
 #pragma unroll
@@ -409,11 +542,19 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
     for (int s = 0; s < STEPS; ++s) {
       Frag<DT> fb[NI];
 #pragma unroll
-      for (int j = 0; j < NI; ++j)
-        fb[j] = dl_read_frag<DT, RB>(sb, wn * WTN + j * 32 + lrow, s, lgrp);
+      for (int j = 0; j < NI; ++j) {
+        if constexpr (LDB == LD_COLS_FAST)
+          fb[j] = dl_read_frag_km<DT, BN, RB>(sb, wn * WTN + j * 32, s, lane);
+        else
+          fb[j] = dl_read_frag<DT, RB>(sb, wn * WTN + j * 32 + lrow, s, lgrp);
+      }
 #pragma unroll
       for (int i = 0; i < MI; ++i) {
-        Frag<DT> fa = dl_read_frag<DT, RB>(sa, wm * WTM + i * 32 + lrow, s, lgrp);
+        Frag<DT> fa;
+        if constexpr (LDA == LD_COLS_FAST)
+          fa = dl_read_frag_km<DT, BM, RB>(sa, wm * WTM + i * 32, s, lane);
+        else
+          fa = dl_read_frag<DT, RB>(sa, wm * WTM + i * 32 + lrow, s, lgrp);
 #pragma unroll
         for (int j = 0; j < NI; ++j)
           mma32x32<DT>(fb[j], fa, acc[i][j]);

@@ -42,10 +42,25 @@
                             rk::LD_ROWS_FAST>(in, fil, out, aux, p);                    \
   }
 
+// K-major operands: LA / LB name how A and B are stored
+#define RK_GEMM_DL_X(NAME, BM, BN, WM, WN, RB, LA, LB)                                   \
+  extern "C" __global__ __launch_bounds__(WM *WN * 64) void RK_CAT(                     \
+      RK_CAT(rock_gemm_, ROCK_DTNAME), NAME)(const void *A, const void *B, void *C,     \
+                                             const void *aux, RockGemmParams p) {       \
+    rk::contraction_body_dl<ROCK_DT, BM, BN, WM, WN, RB, LA, LB>(A, B, C, aux, p);      \
+  }
+#define RK_GEMM_DL_TRANSPOSED(TILE, BM, BN, WM, WN)                                                  \
+  RK_GEMM_DL_X(RK_CAT(TILE, _fast_nn), BM, BN, WM, WN, 128, rk::LD_ROWS_FAST, rk::LD_COLS_FAST)      \
+  RK_GEMM_DL_X(RK_CAT(TILE, _fast_tn), BM, BN, WM, WN, 128, rk::LD_COLS_FAST, rk::LD_COLS_FAST)      \
+  RK_GEMM_DL_X(RK_CAT(TILE, _fast_tt), BM, BN, WM, WN, 128, rk::LD_COLS_FAST, rk::LD_ROWS_FAST)
+
 RK_GEMM_DL(_256x256_fast, 256, 256, 2, 4, 128)
 RK_GEMM_DL(_256x128_fast, 256, 128, 4, 2, 128)
 RK_GEMM_DL(_128x128_fast, 128, 128, 2, 2, 128)
 RK_GEMM_DL(_64x64_fast, 64, 64, 2, 2, 128)
+RK_GEMM_DL_TRANSPOSED(_256x256, 256, 256, 2, 4)
+RK_GEMM_DL_TRANSPOSED(_128x128, 128, 128, 2, 2)
+RK_GEMM_DL_TRANSPOSED(_64x64, 64, 64, 2, 2)
 RK_GEMM(_64x64_generic, 64, 64, 2, 2, rk::LD_ROWS_GENERIC, rk::LD_ROWS_GENERIC)
 
 // small outputs: 32x32 tile per block, K split over the block's four waves

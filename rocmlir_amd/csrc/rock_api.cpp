@@ -207,11 +207,14 @@ constexpr int kNumXCD = 8;
 int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
 // pick the tile that minimises rounds * tile_area / efficiency
-const Tile *pick_tile(int64_t M, int64_t N, int G, bool conv, const std::string &force) {
+// `k_major`: the problem has a K-major operand; those kernels exist for the square tiles only
+const Tile *pick_tile(int64_t M, int64_t N, int G, bool conv, const std::string &force, bool k_major = false) {
   const Tile *best = nullptr;
   double best_cost = 0;
   for (const Tile &t : kFastTiles) {
     if (conv ? !t.conv : !t.gemm)
+      continue;
+    if (k_major && t.bm != t.bn)
       continue;
     if (!force.empty()) {
       if (force == std::to_string(t.bm) + "x" + std::to_string(t.bn))
@@ -382,13 +385,22 @@ Handle *make_gemm(const OptMap &o) {
   // offset inside one block tile (256 rows at most) below 2^31 for the buffer
   // descriptors of the direct-to-LDS loads
   const int64_t kMaxOff = (int64_t)1 << 31;
-  const bool fast = p.a_ks == 1 && p.b_ks == 1 && (p.a_ms * es) % 16 == 0 &&
-                    (p.b_ns * es) % 16 == 0 && (K * es) % 16 == 0 && (p.a_gs * es) % 16 == 0 &&
-                    (p.b_gs * es) % 16 == 0 && 256 * p.a_ms * es + K * es < kMaxOff &&
-                    256 * p.b_ns * es + K * es < kMaxOff;
-  const Tile *tile = fast ? pick_tile(M, N, (int)G, false, forced_tile(o)) : nullptr;
+  auto al16 = [&](int64_t elems) { return (elems * es) % 16 == 0; };
+  // each operand either K-contiguous (rows of whole chunks) or K-major (its
+  // M / N index contiguous, k-rows of whole chunks: the transposing-read path)
+  const bool a_rows = p.a_ks == 1 && al16(p.a_ms) && al16(K) && al16(p.a_gs) && 256 * p.a_ms * es + K * es < kMaxOff;
+  const bool b_rows = p.b_ks == 1 && al16(p.b_ns) && al16(K) && al16(p.b_gs) && 256 * p.b_ns * es + K * es < kMaxOff;
+  const bool a_cols = p.a_ms == 1 && al16(p.a_ks) && al16(M) && al16(p.a_gs) && K * p.a_ks * es + 256 * es < kMaxOff;
+  const bool b_cols = p.b_ns == 1 && al16(p.b_ks) && al16(N) && al16(p.b_gs) && K * p.b_ks * es + 256 * es < kMaxOff;
+  const bool fast = a_rows && b_rows;
+  // storage suffix of the K-major variants: n = as the reference stores it by default
+  const char *storage = nullptr;
+  if (!fast && (a_rows || a_cols) && (b_rows || b_cols))
+    storage = a_rows ? "_nn" : b_rows ? "_tt" : "_tn";
+  const bool tiled = fast || storage;
+  const Tile *tile = tiled ? pick_tile(M, N, (int)G, false, forced_tile(o), storage != nullptr) : nullptr;
   if (!tile)
-    tile = fast ? pick_tile(M, N, (int)G, false, "") : &kGenericTile;
+    tile = tiled ? pick_tile(M, N, (int)G, false, "", storage != nullptr) : &kGenericTile;
   // Too few 64x64 tiles to occupy half the CUs and a K long enough to split:
   // one 32x32 tile per block with the K range divided over its waves (the
   // reference's answer to the same situation is split-K with atomics,
@@ -408,7 +420,7 @@ Handle *make_gemm(const OptMap &o) {
                   h->block_size, h->grid_size);
   if (split_k > 1)
     h->block_size = 256;
-  h->kernel_name = std::string("rock_gemm_") + operand_name(code) + tile->suffix;
+  h->kernel_name = std::string("rock_gemm_") + operand_name(code) + tile->suffix + (storage ? storage : "");
   h->blob_name = std::string("gemm_") + operand_name(code);
   h->num_pointers = 4;
   h->perf_config = perf_string(*tile, es);

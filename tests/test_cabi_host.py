@@ -113,10 +113,14 @@ def test_baseline_configs_select_kernels(rock):
 def test_generic_kernels_for_unaligned_or_transposed(rock):
     k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 3 -m 1024 -k 769 -n 1024 -transB true")
     assert k.kernel_name == "rock_gemm_f16_64x64_generic"          # odd K: no 16-byte chunks
-    k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 64 -k 64 -n 64")
-    assert k.kernel_name == "rock_gemm_f16_64x64_generic"          # B is [K,N]: not K-contiguous
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 64 -k 64 -n 60")
+    assert k.kernel_name == "rock_gemm_f16_64x64_generic"          # B is [K,N] with rows of 120 bytes
     k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 64 -k 64 -n 64 -transA false -transB true")
     assert k.kernel_name.endswith("_fast")
+    # K-major operands of whole 16-byte chunks take the transposing-read kernels
+    for flags, suffix in (("", "_fast_nn"), ("-transA true", "_fast_tn"), ("-transA true -transB true", "_fast_tt")):
+        k = rock.RockKernel("-operation gemm -arch gfx950 -t i8 -g 1 -m 4096 -k 4096 -n 4096 " + flags)
+        assert k.kernel_name == "rock_gemm_i8_256x256" + suffix
     k = rock.RockKernel(CONV_RESNET.replace("NHWGC", "NGCHW").replace("GNYXC", "GNCHW"))
     assert k.kernel_name == "rock_conv_f16_64x64_generic"
 
@@ -186,8 +190,10 @@ def test_tuning_space_lists_the_kernels_a_problem_can_run_on(rock):
     att = rock.RockKernel("--arch gfx950 --operation attention -seq_len_q 256 -seq_len_k 512 "
                           "-head_dim_qk 64 -head_dim_v 64 -t f16 -g 4 -transK true")
     assert att.tuning_space() == [att.perf_config]
-    # operands that are not K-contiguous only have the generic kernel
-    gen = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 256 -n 256 -k 256")
+    # K-major operands have the three square tiles; unaligned ones only the generic kernel
+    nn = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 256 -n 256 -k 256")
+    assert len(nn.tuning_space()) == 3
+    gen = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 256 -n 250 -k 256")
     assert gen.tuning_space() == [gen.perf_config]
     # raw entry points: bad position, short buffer
     lib = rock.load_library()

@@ -61,6 +61,42 @@ def test_gemm_transposes_exact(rock, oracle, gpu, t, tA, tB, tC):
         assert np.array_equal(got, ref)
 
 
+# K-major operands (A stored [K,M] and/or B stored [K,N], the reference's
+# default B): the transposing-read kernels, every tile, ragged tiles and K tails.
+KM_STORAGE = {"nn": (False, False), "tn": (True, False), "tt": (True, True)}
+KM_SHAPES = [(1, 256, 256, 256), (2, 144, 208, 208), (1, 304, 80, 1008), (1, 64, 48, 80)]
+
+
+@pytest.mark.parametrize("tile", ["256,256", "128,128", "64,64"])
+@pytest.mark.parametrize("storage", sorted(KM_STORAGE))
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16", "i8", "fp8", "bf8", "fp8_bf8"])
+def test_gemm_k_major_operands_exact(rock, oracle, gpu, t, storage, tile):
+    tA, tB = KM_STORAGE[storage]
+    for G, M, N, K in KM_SHAPES:
+        if storage == "tn":
+            K -= 3   # both operands K-major: any K, the tail rows are zero-filled
+        info = {}
+        out, od, ref = _run_case(rock, oracle, gpu, t, G, M, N, K, tA, tB, False, True, 11,
+                                 perf_config="v2:%s,8,64,16,8,1,1,1" % tile, info=info)
+        assert info["kernel_name"] == "rock_gemm_%s_%s_fast_%s" % (t, tile.replace(",", "x"), storage)
+        if t == "i8":
+            assert oracle.verify_int(out.cpu().numpy().ravel(), ref)[0] == 0, (G, M, N, K)
+        else:  # exact sums; only the narrowing to the output type rounds
+            assert np.array_equal(to_f32(out, od), oracle.round_through(ref, CODE[od])), (G, M, N, K)
+
+
+def test_gemm_k_major_real_values_with_epilogue(rock, oracle, gpu):
+    """Default reference layout (no transposes), real-valued f16 data, scale +
+    bias + ReLU into f32: the reference's RMS gate."""
+    info = {}
+    bias = torch.linspace(-1.0, 1.0, 320, device=gpu)
+    out, od, ref = _run_case(rock, oracle, gpu, "f16", 1, 384, 320, 512, False, False, False, False, 13,
+                             out_dtype="f32", scale=0.5, bias=bias, relu=True, info=info)
+    assert info["kernel_name"].endswith("_fast_nn")
+    want = np.maximum(ref.reshape(384, 320) * 0.5 + bias.cpu().numpy()[None, :], 0.0)
+    check_float(to_f32(out, od), want.ravel(), od)
+
+
 SHAPES = [
     (1, 1, 1, 1), (1, 16, 16, 16), (1, 64, 64, 128), (1, 65, 63, 129), (3, 128, 96, 200),
     (1, 256, 256, 512), (1, 300, 520, 272), (2, 512, 128, 64), (1, 1000, 24, 48),
