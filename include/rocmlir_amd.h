@@ -128,6 +128,22 @@ ROCMLIR_AMD_API size_t rockamdGetPerfConfig(MiirHandle handle, char *buffer, siz
  * Returns the full length, or (size_t)-1 on failure. */
 ROCMLIR_AMD_API size_t rockamdGetProblemKey(MiirHandle handle, char *buffer, size_t buffer_size);
 
+/* Multi-kernel problems.  As in the reference (rocmlir-lib.cpp:150-199: one
+ * handle per "--kernel_id i", i < miirGetKernelCount, all kernels sharing
+ * miirGetWorkspaceSize bytes of scratch), a problem may lower to several
+ * kernels: a convolution whose filter or input is not channel-contiguous
+ * (gkcyx / ngchw, the reference's default layouts) is run as one layout-
+ * conversion kernel per such tensor followed by the vector contraction kernel
+ * ("--layout_conversion false" keeps the single element-wise kernel).  Every
+ * kernel of the problem is launched, in kernel_id order on one stream, with
+ * the SAME caller list: the problem's pointers followed by the workspace
+ * pointer.  This call says how many pointers the caller list has, how many
+ * the kernel itself takes, and for each of those which caller pointer it is
+ * (source[i]) plus a byte offset; rockamdLaunch applies the map itself.  For
+ * single-kernel problems the map is the identity. */
+ROCMLIR_AMD_API MiirStatus rockamdGetPointerMap(MiirHandle handle, int *caller_pointers, int *kernel_pointers,
+                                                int32_t *source, int64_t *offset);
+
 /* Epilogue scalars can be changed after creation (they live in the by-value
  * parameter block; fetch it again after a change).  Formulas:
  * MIGraphXToTosa.cpp:874-982.  No counterpart entry point in the reference,

@@ -44,6 +44,9 @@ def device_jobs():
                 ["-o", os.path.join(BUILD, "attention.hsaco"),
                  os.path.join(CSRC, "attention_kernels.hip")])
     jobs.append([HIPCC] + DEVICE_FLAGS +
+                ["-o", os.path.join(BUILD, "relayout.hsaco"),
+                 os.path.join(CSRC, "relayout_kernels.hip")])
+    jobs.append([HIPCC] + DEVICE_FLAGS +
                 ["-o", os.path.join(BUILD, "probe.hsaco"),
                  os.path.join(CSRC, "probe_kernels.hip")])
     return jobs

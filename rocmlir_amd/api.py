@@ -95,6 +95,11 @@ def load_library():
                                                C.c_float]
         L.rockamdTuningSetFromTable.restype = C.c_int
         L.rockamdTuningSetFromTable.argtypes = [vp, vp]
+        L.rockamdGetPointerMap.restype = C.c_int
+        L.rockamdGetPointerMap.argtypes = [vp, C.POINTER(C.c_int),
+                                           C.POINTER(C.c_int),
+                                           C.POINTER(C.c_int32),
+                                           C.POINTER(C.c_int64)]
         L.rockamdIsSplitKFaster.restype = C.c_int
         L.rockamdIsSplitKFaster.argtypes = [C.c_int64] * 5 + [C.c_int]
         _lib = L
@@ -156,6 +161,13 @@ class RockKernel:
         L.rockamdGetKernelArgs(self._h, C.byref(npt), None, C.byref(psz))
         self.num_pointers = npt.value
         self.params_size = psz.value
+        # multi-kernel problems: kernels of the problem, its workspace, and the
+        # caller pointer list every one of its kernels is launched with
+        self.kernel_count = L.miirGetKernelCount(self._h)
+        self.workspace_bytes = L.miirGetWorkspaceSize(self._h)
+        ncall = C.c_int(0)
+        L.rockamdGetPointerMap(self._h, C.byref(ncall), None, None, None)
+        self.caller_pointers = ncall.value
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
@@ -241,9 +253,9 @@ class RockKernel:
 
     # ---- launch --------------------------------------------------------------
     def _pointer_array(self, args):
-        if len(args) != self.num_pointers:
+        if len(args) != self.caller_pointers:
             raise RockError("kernel %s takes %d pointer arguments, got %d"
-                            % (self.kernel_name, self.num_pointers, len(args)))
+                            % (self.kernel_name, self.caller_pointers, len(args)))
         arr = (C.c_void_p * len(args))()
         for i, a in enumerate(args):
             if a is None:
@@ -284,6 +296,43 @@ class RockKernel:
         return ms.value
 
 
+class RockProgram:
+    """All kernels of one problem (miirGetKernelCount handles, one per
+    --kernel_id) plus the workspace they share; launch() runs them in order
+    on one stream.  Single-kernel problems behave like their RockKernel."""
+
+    def __init__(self, options):
+        first = RockKernel(options)
+        self.kernels = [first] + [RockKernel("%s --kernel_id %d" % (options, i))
+                                  for i in range(1, first.kernel_count)]
+        self.workspace_bytes = first.workspace_bytes
+        self._workspace = None
+
+    @property
+    def main(self):
+        """The contraction kernel (the last of the problem)."""
+        return self.kernels[-1]
+
+    def _args(self, args):
+        if len(self.kernels) == 1 and self.main.caller_pointers == len(args):
+            return args
+        if self._workspace is None:
+            import torch
+            dev = next(a.device for a in args if a is not None and not isinstance(a, int))
+            self._workspace = torch.empty(max(self.workspace_bytes, 16), dtype=torch.uint8, device=dev)
+        return tuple(args) + (self._workspace,)
+
+    def launch(self, *args, stream=None):
+        full = self._args(args)
+        for k in self.kernels:
+            k.launch(*full, stream=stream)
+
+    def benchmark(self, *args, warmup=3, iters=20, stream=None):
+        """Sum of the kernels' average times in milliseconds."""
+        full = self._args(args)
+        return sum(k.benchmark(*full, warmup=warmup, iters=iters, stream=stream) for k in self.kernels)
+
+
 # ---------------------------------------------------------------------------
 # torch front ends
 # ---------------------------------------------------------------------------
@@ -295,6 +344,16 @@ def _kernel(options):
     if k is None:
         k = _kernel_cache[options] = RockKernel(options)
     return k
+
+
+_program_cache = {}
+
+
+def _program(options):
+    p = _program_cache.get(options)
+    if p is None:
+        p = _program_cache[options] = RockProgram(options)
+    return p
 
 
 def _dtype_name(dt):
@@ -407,16 +466,18 @@ def conv2d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize,
         opts += " --perf_config %s" % perf_config
     opts += _epilogue_flags(scale, zero_point, bias, relu, quant_scale,
                             out_zero_point)
-    k = _kernel(opts)
+    prog = _program(opts)
+    k = prog.main
     if info is not None:
         info["kernel_name"] = k.kernel_name
         info["perf_config"] = k.perf_config
+        info["kernels"] = [x.kernel_name for x in prog.kernels]
     if out_dtype is None:
         out_dtype = {"i8": "i32", "fp8": "f32", "bf8": "f32"}.get(t, t)
     if out is None:
         out = torch.empty(batchsize * out_channels * ho * wo,
                           dtype=_torch_dtype(out_dtype), device=inp.device)
-    k.launch(fil.contiguous(), inp.contiguous(), out, bias, stream=stream)
+    prog.launch(fil.contiguous(), inp.contiguous(), out, bias, stream=stream)
     return out
 
 

@@ -20,5 +20,6 @@ rock_hsaco_\n\()_end:
     ROCK_BLOB gemm_fp8_bf8
     ROCK_BLOB gemm_bf8_fp8
     ROCK_BLOB attention
+    ROCK_BLOB relayout
     ROCK_BLOB probe
     .section .note.GNU-stack,"",@progbits

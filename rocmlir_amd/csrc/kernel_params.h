@@ -70,6 +70,19 @@ struct RockConvParams {
   RockEpilogue epi;
 };
 
+// Layout conversion of a 5-D tensor (the utility "converting copy" of the
+// reference's multi-kernel flows, ConvGenerator.cpp:279-344): element (i0..i4)
+// moves from src[sum i_d * src_stride[d]] to dst[sum i_d * dst_stride[d]].
+// The dimension that is contiguous in the source and the one that is
+// contiguous in the destination are tiled 32 x 32 through LDS so that both
+// sides are accessed in whole rows; the other three dimensions index tiles.
+struct RockRelayoutParams {
+  int64_t src_stride[5], dst_stride[5]; // in elements
+  int32_t size[5];
+  int32_t src_fast, dst_fast; // dimension indices; equal when no transposition is needed
+  int32_t pad_;
+};
+
 struct RockAttentionParams {
   // element strides of the logical views Q[g,i,d], K[g,j,d], V[g,j,e], O[g,i,e]
   int64_t q_gs, q_is, q_ds;

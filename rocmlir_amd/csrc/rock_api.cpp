@@ -237,7 +237,7 @@ const Tile *pick_tile(int64_t M, int64_t N, int G, bool conv, const std::string 
 // --------------------------------------------------------------------------
 // problems
 // --------------------------------------------------------------------------
-enum OpKind { OP_GEMM, OP_CONV, OP_ATTENTION };
+enum OpKind { OP_GEMM, OP_CONV, OP_ATTENTION, OP_RELAYOUT };
 
 struct Handle {
   OpKind op;
@@ -255,6 +255,18 @@ struct Handle {
   std::string problem_key;
   bool tuned = false, lowered = false;
   OptMap options; // the parsed problem, kept so that a perf_config can be applied later
+  // multi-kernel problems (layout conversion + contraction): every kernel of
+  // the problem is launched with the same caller pointer list, the problem's
+  // tensors followed by one workspace pointer; ptr_map says where each of
+  // THIS kernel's pointers comes from.  Single-kernel problems: identity.
+  int kernel_count = 1;
+  size_t workspace_bytes = 0;
+  int caller_pointers = 0; // 0 = same as num_pointers
+  struct PtrSrc {
+    int source;     // index into the caller's list
+    int64_t offset; // bytes added to it
+  };
+  std::vector<PtrSrc> ptr_map;
   // typed views of `params`
   RockEpilogue *epi = nullptr;
   // launch cache: device -> function
@@ -614,15 +626,109 @@ Handle *make_conv(const OptMap &o) {
     p.in_ns = is[0]; p.in_gs = is[1]; p.in_cs = is[2]; p.in_hs = is[3]; p.in_ws = is[4];
     p.out_ns = os[0]; p.out_gs = os[1]; p.out_ks = os[2]; p.out_hs = os[3]; p.out_ws = os[4];
   }
-  p.k_order_yxc = (p.in_cs == 1) ? 1 : 0;
   const int es = dtype_size(ti);
   auto al = [&](int64_t elems) { return (elems * es) % 16 == 0; };
-  const bool fast = p.in_cs == 1 && al(c) && al(p.in_ws) && al(p.in_hs) && al(p.in_ns) &&
-                    al(p.in_gs) && p.fil_cs == 1 && p.fil_xs == c && p.fil_ys == x * c &&
-                    al(p.fil_ks) && al(p.fil_gs) &&
-                    // byte offsets inside one group's input slice and one filter tile < 2^31
-                    (n * p.in_ns + hi * p.in_hs + wi * p.in_ws + c) * es < ((int64_t)1 << 31) &&
-                    (256 * p.fil_ks + Kg) * es < ((int64_t)1 << 31);
+  auto conv_fast = [&](const RockConvParams &q) {
+    return q.in_cs == 1 && al(c) && al(q.in_ws) && al(q.in_hs) && al(q.in_ns) && al(q.in_gs) &&
+           q.fil_cs == 1 && q.fil_xs == c && q.fil_ys == x * c && al(q.fil_ks) && al(q.fil_gs) &&
+           // byte offsets inside one group's input slice and one filter tile < 2^31
+           (n * q.in_ns + hi * q.in_hs + wi * q.in_ws + c) * es < ((int64_t)1 << 31) &&
+           (256 * q.fil_ks + Kg) * es < ((int64_t)1 << 31);
+  };
+  bool fast = conv_fast(p);
+
+  // Layout-conversion plan.  A problem whose filter or input is not
+  // channel-contiguous (the reference's default gkcyx / ngchw) would run the
+  // element-wise kernel; if the channel-contiguous form qualifies for the
+  // vector kernels, the tensors are first copied into that form in a
+  // workspace by one relayout kernel each, and the contraction kernel reads
+  // the copies (and writes the caller's output layout directly).  This is the
+  // reference's multi-kernel protocol (miirGetKernelCount / --kernel_id /
+  // miirGetWorkspaceSize, rocmlir-lib.cpp:150-199) which it uses for its
+  // backward convolutions with their utility kernels.
+  {
+    RockConvParams q = p;
+    const int64_t fsz[5] = {g, k, c, y, x}, isz[5] = {n, g, c, hi, wi};
+    int64_t fs[5], is[5];
+    layout_strides("gkyxc", "gkcyx", fsz, fs);
+    layout_strides("nhwgc", "ngchw", isz, is);
+    q.fil_gs = fs[0]; q.fil_ks = fs[1]; q.fil_cs = fs[2]; q.fil_ys = fs[3]; q.fil_xs = fs[4];
+    q.in_ns = is[0]; q.in_gs = is[1]; q.in_cs = is[2]; q.in_hs = is[3]; q.in_ws = is[4];
+    const bool need_f = !(p.fil_cs == 1 && p.fil_xs == c && p.fil_ys == x * c && al(p.fil_ks) && al(p.fil_gs));
+    const bool need_i = !(p.in_cs == 1 && al(p.in_ws) && al(p.in_hs) && al(p.in_ns) && al(p.in_gs));
+    const int64_t fil_bytes = (g * k * c * y * x * es + 255) / 256 * 256;
+    const int64_t in_bytes = (n * g * c * hi * wi * es + 255) / 256 * 256;
+    if (!fast && conv_fast(q) && bool_or(o, "layout_conversion", true)) {
+      if (!need_f) { // keep the caller's filter
+        q.fil_gs = p.fil_gs; q.fil_ks = p.fil_ks; q.fil_cs = p.fil_cs; q.fil_ys = p.fil_ys; q.fil_xs = p.fil_xs;
+      }
+      if (!need_i) {
+        q.in_ns = p.in_ns; q.in_gs = p.in_gs; q.in_cs = p.in_cs; q.in_hs = p.in_hs; q.in_ws = p.in_ws;
+      }
+      const int n_relayout = (need_f ? 1 : 0) + (need_i ? 1 : 0);
+      const int64_t off_f = 0, off_i = need_f ? fil_bytes : 0;
+      h->kernel_count = n_relayout + 1;
+      h->workspace_bytes = (size_t)((need_f ? fil_bytes : 0) + (need_i ? in_bytes : 0));
+      h->caller_pointers = 5; // filter, input, output, bias, workspace
+      const int kid = (int)int_or(o, "kernel_id", 0);
+      const bool is_f = need_f && kid == 0, is_i = need_i && kid == (need_f ? 1 : 0);
+      if (is_f || is_i) {
+        // this handle is one of the conversion kernels
+        RockRelayoutParams r;
+        std::memset(&r, 0, sizeof r);
+        const int64_t *sz = is_f ? fsz : isz; // sizes in the letter order of the canonical layout string below
+        // dimensions listed in destination (channel-contiguous) order
+        const int order_f[5] = {0, 1, 3, 4, 2}, order_i[5] = {0, 3, 4, 1, 2}; // g k y x c ; n h w g c
+        const int64_t src_f[5] = {p.fil_gs, p.fil_ks, p.fil_cs, p.fil_ys, p.fil_xs};
+        const int64_t src_i[5] = {p.in_ns, p.in_gs, p.in_cs, p.in_hs, p.in_ws};
+        int64_t dst = 1;
+        for (int d = 4; d >= 0; --d) {
+          const int letter = is_f ? order_f[d] : order_i[d];
+          r.size[d] = (int32_t)sz[letter];
+          r.src_stride[d] = is_f ? src_f[letter] : src_i[letter];
+          r.dst_stride[d] = dst;
+          dst *= sz[letter];
+        }
+        r.dst_fast = 4;
+        r.src_fast = 4;
+        for (int d = 0; d < 5; ++d) // the source's contiguous dimension (ties: the longest)
+          if (r.src_stride[d] == 1 && (r.src_stride[r.src_fast] != 1 || r.size[d] > r.size[r.src_fast]))
+            r.src_fast = d;
+        int64_t blocks = 1;
+        for (int d = 0; d < 5; ++d) {
+          if (d == r.src_fast)
+            blocks *= r.src_fast == r.dst_fast ? (r.size[d] + 1023) / 1024 : (r.size[d] + 31) / 32;
+          else if (d == r.dst_fast)
+            blocks *= (r.size[d] + 31) / 32;
+          else
+            blocks *= r.size[d];
+        }
+        if (blocks > INT32_MAX) {
+          set_error("conv: tensor too large for the layout-conversion kernel");
+          delete h;
+          return nullptr;
+        }
+        h->op = OP_RELAYOUT;
+        h->epi = nullptr;
+        h->params.assign(sizeof r, 0);
+        std::memcpy(h->params.data(), &r, sizeof r);
+        h->kernel_name = std::string("rock_relayout_b") + std::to_string(es);
+        h->blob_name = "relayout";
+        h->block_size = 256;
+        h->grid_size = (uint32_t)blocks;
+        h->num_pointers = 2;
+        h->ptr_map = {{is_f ? 0 : 1, 0}, {4, is_f ? off_f : off_i}};
+        h->perf_config = "";
+        h->problem_key = std::string("relayout ") + (is_f ? "filter " : "input ") + (is_f ? fl : il);
+        return h;
+      }
+      // this handle is the contraction kernel reading the converted tensors
+      p = q;
+      fast = true;
+      h->ptr_map = {{need_f ? 4 : 0, need_f ? off_f : 0}, {need_i ? 4 : 1, need_i ? off_i : 0}, {2, 0}, {3, 0}};
+    }
+  }
+  p.k_order_yxc = (p.in_cs == 1) ? 1 : 0;
   const Tile *tile = fast ? pick_tile(Mg, k, (int)g, true, forced_tile(o)) : nullptr;
   if (!tile)
     tile = fast ? pick_tile(Mg, k, (int)g, true, "") : &kGenericTile;
@@ -815,8 +921,11 @@ int launch_once(Handle *h, hipFunction_t fn, void *const *pointers, hipStream_t 
   // argument buffer: the pointers, then the parameter block (8-byte aligned)
   char buf[8 * 8 + 512];
   size_t off = 0;
-  for (int i = 0; i < h->num_pointers; ++i, off += 8)
-    std::memcpy(buf + off, &pointers[i], 8);
+  for (int i = 0; i < h->num_pointers; ++i, off += 8) {
+    const void *ptr = h->ptr_map.empty() ? pointers[i]
+                                         : (const char *)pointers[h->ptr_map[i].source] + h->ptr_map[i].offset;
+    std::memcpy(buf + off, &ptr, 8);
+  }
   std::memcpy(buf + off, h->params.data(), h->params.size());
   size_t size = off + h->params.size();
   void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, buf, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
@@ -826,7 +935,8 @@ int launch_once(Handle *h, hipFunction_t fn, void *const *pointers, hipStream_t 
 }
 
 bool check_launch_args(Handle *h, void *const *pointers, int num_pointers) {
-  if (!h || !pointers || num_pointers != h->num_pointers) {
+  const int expected = h ? (h->caller_pointers ? h->caller_pointers : h->num_pointers) : 0;
+  if (!h || !pointers || num_pointers != expected) {
     set_error("launch: wrong number of pointer arguments");
     return false;
   }
@@ -843,7 +953,7 @@ bool check_launch_args(Handle *h, void *const *pointers, int num_pointers) {
   int aux_index = 3;
   bool need_aux = h->op == OP_ATTENTION
                       ? reinterpret_cast<RockAttentionParams *>(h->params.data())->has_bias != 0
-                      : h->epi->has_bias != 0;
+                      : (h->epi && h->epi->has_bias != 0);
   for (int i = 0; i < num_pointers; ++i)
     if (!pointers[i] && (i != aux_index || need_aux)) {
       set_error("launch: NULL tensor pointer");
@@ -880,7 +990,7 @@ Handle *build_handle(const OptMap &o) {
   if (!h)
     return nullptr;
   h->kernel_id = (int)int_or(o, "kernel_id", 0);
-  if (h->kernel_id != 0) { // forward ops are single-kernel
+  if (h->kernel_id < 0 || h->kernel_id >= h->kernel_count) {
     set_error("kernel_id out of range");
     delete h;
     return nullptr;
@@ -957,9 +1067,16 @@ MiirHandle miirCreateHandle(const char *options) {
   return build_handle(o);
 }
 
-int miirGetKernelCount(MiirHandle handle) { return handle ? 1 : -1; }
+int miirGetKernelCount(MiirHandle handle) {
+  return handle ? static_cast<Handle *>(handle)->kernel_count : -1;
+}
 
-int miirGetWorkspaceSize(MiirHandle handle) { return handle ? 0 : -1; }
+int miirGetWorkspaceSize(MiirHandle handle) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h)
+    return -1;
+  return h->workspace_bytes > (size_t)INT32_MAX ? -1 : (int)h->workspace_bytes;
+}
 
 MiirStatus miirLowerTuningParams(MiirHandle handle) {
   auto *h = static_cast<Handle *>(handle);
@@ -1074,20 +1191,40 @@ size_t rockamdGetProblemKey(MiirHandle handle, char *buffer, size_t buffer_size)
   return copy_string(h->problem_key, buffer, buffer_size);
 }
 
+MiirStatus rockamdGetPointerMap(MiirHandle handle, int *caller_pointers, int *kernel_pointers,
+                                int32_t *source, int64_t *offset) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h)
+    return MIIR_INVALID_PARAM;
+  if (caller_pointers)
+    *caller_pointers = h->caller_pointers ? h->caller_pointers : h->num_pointers;
+  if (kernel_pointers)
+    *kernel_pointers = h->num_pointers;
+  for (int i = 0; i < h->num_pointers; ++i) {
+    if (source)
+      source[i] = h->ptr_map.empty() ? i : h->ptr_map[i].source;
+    if (offset)
+      offset[i] = h->ptr_map.empty() ? 0 : h->ptr_map[i].offset;
+  }
+  return MIIR_SUCCESS;
+}
+
 MiirStatus rockamdSetScale(MiirHandle handle, float scale) {
   auto *h = static_cast<Handle *>(handle);
   if (!h)
     return MIIR_INVALID_PARAM;
   if (h->op == OP_ATTENTION)
     reinterpret_cast<RockAttentionParams *>(h->params.data())->scale = scale;
-  else
+  else if (h->epi)
     h->epi->scale = scale;
+  else
+    return MIIR_INVALID_PARAM; // a layout-conversion kernel has no epilogue
   return MIIR_SUCCESS;
 }
 
 MiirStatus rockamdSetZeroPoint(MiirHandle handle, int32_t zero_point) {
   auto *h = static_cast<Handle *>(handle);
-  if (!h || h->op == OP_ATTENTION)
+  if (!h || h->op == OP_ATTENTION || !h->epi)
     return MIIR_INVALID_PARAM;
   h->epi->zero_point = zero_point;
   return MIIR_SUCCESS;
@@ -1249,7 +1386,8 @@ int rockamdTuningSetFromStr(MiirHandle handle, const char *perf_config) {
   Handle *n = build_handle(o);
   if (!n)
     return 0;
-  *n->epi = *h->epi; // scalars changed with rockamdSetScale / SetZeroPoint stay
+  if (n->epi && h->epi)
+    *n->epi = *h->epi; // scalars changed with rockamdSetScale / SetZeroPoint stay
   *h = std::move(*n); // params moves with its buffer, so the typed views stay valid
   delete n;
   return 1;

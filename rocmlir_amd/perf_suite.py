@@ -112,7 +112,7 @@ def conv_problem(line, t, layout):
 
 def run_problem(rock, torch, dev, opts, shapes, flops, warmup, iters):
     try:
-        kern = rock.RockKernel(opts)
+        prog = rock.RockProgram(opts)  # every kernel of the problem and its workspace
     except rock.RockError as e:
         return {"status": "no kernel", "error": str(e).split(" [")[0]}
     # the last tensor in pointer order is the output; the bias slot stays empty
@@ -120,8 +120,8 @@ def run_problem(rock, torch, dev, opts, shapes, flops, warmup, iters):
     args = [None if s is None else
             torch.empty(s[0], device=dev, dtype=_torch_dtype(torch, s[1])) if i == last else _rand(torch, s[0], s[1], dev)
             for i, s in enumerate(shapes)]
-    ms = kern.benchmark(*args, warmup=warmup, iters=iters)
-    return {"status": "ok", "kernel": kern.kernel_name, "ms": round(ms, 5),
+    ms = prog.benchmark(*args, warmup=warmup, iters=iters)
+    return {"status": "ok", "kernel": prog.main.kernel_name, "kernels": len(prog.kernels), "ms": round(ms, 5),
             "tflops": round(flops / (ms * 1e-3) / 1e12, 2)}
 
 

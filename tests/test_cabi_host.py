@@ -121,8 +121,45 @@ def test_generic_kernels_for_unaligned_or_transposed(rock):
     for flags, suffix in (("", "_fast_nn"), ("-transA true", "_fast_tn"), ("-transA true -transB true", "_fast_tt")):
         k = rock.RockKernel("-operation gemm -arch gfx950 -t i8 -g 1 -m 4096 -k 4096 -n 4096 " + flags)
         assert k.kernel_name == "rock_gemm_i8_256x256" + suffix
-    k = rock.RockKernel(CONV_RESNET.replace("NHWGC", "NGCHW").replace("GNYXC", "GNCHW"))
-    assert k.kernel_name == "rock_conv_f16_64x64_generic"
+    nchw = CONV_RESNET.replace("NHWGC", "NGCHW").replace("GNYXC", "GNCHW")
+    assert rock.RockKernel(nchw + " --layout_conversion false").kernel_name == "rock_conv_f16_64x64_generic"
+    k = rock.RockKernel(CONV_RESNET.replace("--in_channels 128", "--in_channels 100").replace("NHWGC", "NGCHW"))
+    assert k.kernel_name == "rock_conv_f16_64x64_generic"    # 200-byte channel runs: no vector form to convert to
+
+
+def test_layout_conversion_plan_follows_the_multi_kernel_protocol(rock):
+    """NCHW tensors (the reference's default layouts): one conversion kernel
+    per tensor, then the vector contraction kernel, behind miirGetKernelCount /
+    --kernel_id / miirGetWorkspaceSize (rocmlir-lib.cpp:150-199)."""
+    lib = rock.load_library()
+    nchw = CONV_RESNET.replace("NHWGC", "NGCHW").replace("GNYXC", "GNCHW")
+    ks = [rock.RockKernel(nchw + " --kernel_id %d" % i) for i in range(3)]
+    assert [k.kernel_name for k in ks] == ["rock_relayout_b2", "rock_relayout_b2", "rock_conv_f16_128x128_fast"]
+    fil_bytes, in_bytes = 128 * 128 * 9 * 2, 256 * 128 * 28 * 28 * 2
+    for k in ks:
+        assert k.kernel_count == 3 and k.caller_pointers == 5
+        assert k.workspace_bytes == lib.miirGetWorkspaceSize(k._h) == fil_bytes + in_bytes
+    maps = []
+    for k in ks:
+        ncall, nk = C.c_int(), C.c_int()
+        src, off = (C.c_int32 * 8)(), (C.c_int64 * 8)()
+        assert lib.rockamdGetPointerMap(k._h, C.byref(ncall), C.byref(nk), src, off) == 0
+        assert ncall.value == 5 and nk.value == k.num_pointers
+        maps.append([(src[i], off[i]) for i in range(nk.value)])
+    assert maps == [[(0, 0), (4, 0)], [(1, 0), (4, fil_bytes)],
+                    [(4, 0), (4, fil_bytes), (2, 0), (3, 0)]]
+    with pytest.raises(rock.RockError, match="kernel_id out of range"):
+        rock.RockKernel(nchw + " --kernel_id 3")
+    # only the input needs converting when the filter is already channel-contiguous
+    mixed = CONV_RESNET.replace("--in_layout NHWGC", "--in_layout NGCHW")
+    ks = [rock.RockKernel(mixed + " --kernel_id %d" % i) for i in range(2)]
+    assert [k.kernel_name for k in ks] == ["rock_relayout_b2", "rock_conv_f16_128x128_fast"]
+    assert ks[0].workspace_bytes == in_bytes
+    # single-kernel problems: identity map, no workspace
+    k = rock.RockKernel(CONV_RESNET)
+    assert (k.kernel_count, k.workspace_bytes, k.caller_pointers) == (1, 0, 4)
+    # a conversion kernel has no epilogue scalars to set
+    assert lib.rockamdSetScale(rock.RockKernel(nchw)._h, C.c_float(2.0)) != 0
 
 
 def test_perf_config_override_and_fallback(rock):
