@@ -70,10 +70,13 @@ typedef void *MiirHandle;
  * failure, as the reference does. */
 ROCMLIR_AMD_API MiirHandle miirCreateHandle(const char *options);
 
-/* Miir.h:56 -- number of kernels the operation needs; -1 for a NULL handle. */
+/* Miir.h:56 -- number of kernels the operation needs (1, or up to 3 for a
+ * convolution run through the layout-conversion plan, see
+ * rockamdGetPointerMap); -1 for a NULL handle. */
 ROCMLIR_AMD_API int miirGetKernelCount(MiirHandle handle);
 
-/* Miir.h:65 -- workspace bytes (always 0 for the forward ops built here). */
+/* Miir.h:65 -- workspace bytes shared by the kernels of the problem (0 for
+ * single-kernel problems); -1 for a NULL handle or a size beyond int. */
 ROCMLIR_AMD_API int miirGetWorkspaceSize(MiirHandle handle);
 
 /* Miir.h:70 -- resolves the perf config (table lookup); needed before
