@@ -138,6 +138,10 @@ template <int DT, int ROWS, int NW, int RB> struct ConvInDl {
   int kb[Sg::PER_WAVE];
   int uy, ux, uc0;               // tap and byte offset of the K-step inside the channel run
   bool uniform;
+  // what one K-step (BKE elements) advances a per-lane tap by: whole filter
+  // rows, taps within a row, channels within a tap
+  int step_y, step_x, step_c;
+  bool padded; // some window reaches outside the image
   int wave;
 
   __device__ __forceinline__ void init(const void *in, const RockConvParams &cp, int g, int row0,
@@ -146,6 +150,15 @@ template <int DT, int ROWS, int NW, int RB> struct ConvInDl {
     wave = wave_;
     uniform = (cp.c * ES) % RB == 0;
     uy = ux = uc0 = 0;
+    {
+      const int taps = BKE / cp.c;
+      step_c = BKE - taps * cp.c;
+      step_y = taps / cp.x;
+      step_x = taps - step_y * cp.x;
+    }
+    padded = cp.pad_h != 0 || cp.pad_w != 0 ||
+             (cp.ho - 1) * cp.stride_h + (cp.y - 1) * cp.dil_h >= cp.hi ||
+             (cp.wo - 1) * cp.stride_w + (cp.x - 1) * cp.dil_w >= cp.wi;
     rsrc = dl_rsrc((const char *)in + (int64_t)g * cp.in_gs * ES);
 #pragma unroll
     for (int i = 0; i < Sg::PER_WAVE; ++i) {
@@ -196,19 +209,24 @@ template <int DT, int ROWS, int NW, int RB> struct ConvInDl {
       }
       return;
     }
+    // per-lane taps: a K-step moves every lane's chunk on by the same
+    // (taps, channels) amount, so the walk is branch-free
 #pragma unroll
     for (int i = 0; i < Sg::PER_WAVE; ++i) {
       int hi = h0[i] + y[i] * p->dil_h, wi = w0[i] + x[i] * p->dil_w;
-      bool v = pix[i] != kOobOffset && y[i] < p->y && hi >= 0 && hi < p->hi && wi >= 0 && wi < p->wi;
+      bool v = pix[i] != kOobOffset && y[i] < p->y;
+      if (padded) // uniform
+        v = v && hi >= 0 && hi < p->hi && wi >= 0 && wi < p->wi;
       unsigned voff = v ? pix[i] + (unsigned)((hi * (int)p->in_hs + wi * (int)p->in_ws + cc[i]) * ES)
                         : kOobOffset;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
           rsrc, (lds_void_t *)(stage + (wave * Sg::PER_WAVE + i) * 1024), 16, (int)voff, 0, 0, 0);
-      cc[i] += BKE;
-      while (cc[i] >= p->c) {
-        cc[i] -= p->c;
-        if (++x[i] == p->x) { x[i] = 0; ++y[i]; }
-      }
+      cc[i] += step_c;
+      const int carry = cc[i] >= p->c ? 1 : 0;
+      cc[i] -= carry ? p->c : 0;
+      x[i] += step_x + carry;
+      y[i] += step_y;
+      if (x[i] >= p->x) { x[i] -= p->x; ++y[i]; }
     }
   }
 };

@@ -73,14 +73,20 @@ struct RockConvParams {
 // Layout conversion of a 5-D tensor (the utility "converting copy" of the
 // reference's multi-kernel flows, ConvGenerator.cpp:279-344): element (i0..i4)
 // moves from src[sum i_d * src_stride[d]] to dst[sum i_d * dst_stride[d]].
-// The dimension that is contiguous in the source and the one that is
-// contiguous in the destination are tiled 32 x 32 through LDS so that both
-// sides are accessed in whole rows; the other three dimensions index tiles.
+// The destination may be longer than the source along a dimension (channel
+// padding): positions at or beyond src_size read as zero.
+enum RockRelayoutMode {
+  RELAYOUT_TRANSPOSE = 0, // contiguous dimensions differ: tile_d x (1024/tile_d) tiles through LDS
+  RELAYOUT_COPY = 1,      // both contiguous along dimension 4: one 16-byte destination chunk per thread
+  RELAYOUT_TRANSPOSE_VEC = 2, // as TRANSPOSE with 128-byte tile rows and 16-byte accesses
+};
 struct RockRelayoutParams {
   int64_t src_stride[5], dst_stride[5]; // in elements
-  int32_t size[5];
-  int32_t src_fast, dst_fast; // dimension indices; equal when no transposition is needed
-  int32_t pad_;
+  int32_t size[5];                      // of the destination
+  int32_t src_size[5];
+  int32_t src_fast, dst_fast; // dimension indices
+  int32_t mode;               // RockRelayoutMode
+  int32_t tile_d;             // RELAYOUT_TRANSPOSE: tile extent along dst_fast (8, 16 or 32)
 };
 
 struct RockAttentionParams {

@@ -594,8 +594,10 @@ Handle *make_conv(const OptMap &o) {
     set_error("conv: only the forward direction is built (" + opn + " requested)");
     return nullptr;
   }
-  const int64_t c = ct / g, k = kt / g;
-  const int64_t Mg = n * ho * wo, Kg = c * y * x;
+  const int64_t c_problem = ct / g, k = kt / g; // channels per group as the problem states them
+  int64_t c = c_problem;                        // ... and as the contraction kernel sees them (may be padded)
+  const int64_t Mg = n * ho * wo;
+  int64_t Kg = c * y * x;
   if (Mg > INT32_MAX || Kg > INT32_MAX) {
     set_error("conv: problem too large for 32-bit tile indices");
     return nullptr;
@@ -628,14 +630,14 @@ Handle *make_conv(const OptMap &o) {
   }
   const int es = dtype_size(ti);
   auto al = [&](int64_t elems) { return (elems * es) % 16 == 0; };
-  auto conv_fast = [&](const RockConvParams &q) {
-    return q.in_cs == 1 && al(c) && al(q.in_ws) && al(q.in_hs) && al(q.in_ns) && al(q.in_gs) &&
-           q.fil_cs == 1 && q.fil_xs == c && q.fil_ys == x * c && al(q.fil_ks) && al(q.fil_gs) &&
+  auto conv_fast = [&](const RockConvParams &q, int64_t cc) {
+    return q.in_cs == 1 && al(cc) && al(q.in_ws) && al(q.in_hs) && al(q.in_ns) && al(q.in_gs) &&
+           q.fil_cs == 1 && q.fil_xs == cc && q.fil_ys == x * cc && al(q.fil_ks) && al(q.fil_gs) &&
            // byte offsets inside one group's input slice and one filter tile < 2^31
-           (n * q.in_ns + hi * q.in_hs + wi * q.in_ws + c) * es < ((int64_t)1 << 31) &&
-           (256 * q.fil_ks + Kg) * es < ((int64_t)1 << 31);
+           (n * q.in_ns + hi * q.in_hs + wi * q.in_ws + cc) * es < ((int64_t)1 << 31) &&
+           (256 * q.fil_ks + cc * y * x) * es < ((int64_t)1 << 31);
   };
-  bool fast = conv_fast(p);
+  bool fast = conv_fast(p, c);
 
   // Layout-conversion plan.  A problem whose filter or input is not
   // channel-contiguous (the reference's default gkcyx / ngchw) would run the
@@ -647,18 +649,24 @@ Handle *make_conv(const OptMap &o) {
   // miirGetWorkspaceSize, rocmlir-lib.cpp:150-199) which it uses for its
   // backward convolutions with their utility kernels.
   {
+    // channel runs that are not whole 16-byte chunks (the 3-channel first layer
+    // of a CNN) are zero-padded up to one by the conversion kernels
+    const int64_t cp = (c * es + 15) / 16 * 16 / es;
     RockConvParams q = p;
-    const int64_t fsz[5] = {g, k, c, y, x}, isz[5] = {n, g, c, hi, wi};
+    q.c = (int)cp;
+    q.K = (int)(cp * y * x);
+    const int64_t fsz[5] = {g, k, cp, y, x}, isz[5] = {n, g, cp, hi, wi};        // converted tensors
+    const int64_t fsz_src[5] = {g, k, c, y, x}, isz_src[5] = {n, g, c, hi, wi};  // the caller's
     int64_t fs[5], is[5];
     layout_strides("gkyxc", "gkcyx", fsz, fs);
     layout_strides("nhwgc", "ngchw", isz, is);
     q.fil_gs = fs[0]; q.fil_ks = fs[1]; q.fil_cs = fs[2]; q.fil_ys = fs[3]; q.fil_xs = fs[4];
     q.in_ns = is[0]; q.in_gs = is[1]; q.in_cs = is[2]; q.in_hs = is[3]; q.in_ws = is[4];
-    const bool need_f = !(p.fil_cs == 1 && p.fil_xs == c && p.fil_ys == x * c && al(p.fil_ks) && al(p.fil_gs));
-    const bool need_i = !(p.in_cs == 1 && al(p.in_ws) && al(p.in_hs) && al(p.in_ns) && al(p.in_gs));
-    const int64_t fil_bytes = (g * k * c * y * x * es + 255) / 256 * 256;
-    const int64_t in_bytes = (n * g * c * hi * wi * es + 255) / 256 * 256;
-    if (!fast && conv_fast(q) && bool_or(o, "layout_conversion", true)) {
+    const bool need_f = cp != c || !(p.fil_cs == 1 && p.fil_xs == c && p.fil_ys == x * c && al(p.fil_ks) && al(p.fil_gs));
+    const bool need_i = cp != c || !(p.in_cs == 1 && al(p.in_ws) && al(p.in_hs) && al(p.in_ns) && al(p.in_gs));
+    const int64_t fil_bytes = (g * k * cp * y * x * es + 255) / 256 * 256;
+    const int64_t in_bytes = (n * g * cp * hi * wi * es + 255) / 256 * 256;
+    if (!fast && cp * y * x <= INT32_MAX && conv_fast(q, cp) && bool_or(o, "layout_conversion", true)) {
       if (!need_f) { // keep the caller's filter
         q.fil_gs = p.fil_gs; q.fil_ks = p.fil_ks; q.fil_cs = p.fil_cs; q.fil_ys = p.fil_ys; q.fil_xs = p.fil_xs;
       }
@@ -676,18 +684,45 @@ Handle *make_conv(const OptMap &o) {
         // this handle is one of the conversion kernels
         RockRelayoutParams r;
         std::memset(&r, 0, sizeof r);
-        const int64_t *sz = is_f ? fsz : isz; // sizes in the letter order of the canonical layout string below
+        const int64_t *sz = is_f ? fsz : isz;             // sizes in the letter order "gkcyx" / "ngchw"
+        const int64_t *sz_src = is_f ? fsz_src : isz_src; // the source is shorter along c when padding
         // dimensions listed in destination (channel-contiguous) order
         const int order_f[5] = {0, 1, 3, 4, 2}, order_i[5] = {0, 3, 4, 1, 2}; // g k y x c ; n h w g c
         const int64_t src_f[5] = {p.fil_gs, p.fil_ks, p.fil_cs, p.fil_ys, p.fil_xs};
         const int64_t src_i[5] = {p.in_ns, p.in_gs, p.in_cs, p.in_hs, p.in_ws};
+        struct Dim { int64_t size, src_size, ss, ds; };
+        std::vector<Dim> dims;
         int64_t dst = 1;
         for (int d = 4; d >= 0; --d) {
           const int letter = is_f ? order_f[d] : order_i[d];
-          r.size[d] = (int32_t)sz[letter];
-          r.src_stride[d] = is_f ? src_f[letter] : src_i[letter];
-          r.dst_stride[d] = dst;
+          dims.insert(dims.begin(), Dim{sz[letter], sz_src[letter], is_f ? src_f[letter] : src_i[letter], dst});
           dst *= sz[letter];
+        }
+        // drop unit dimensions and fold neighbours that are laid out back to back
+        // on both sides (h and w of an NCHW image) into one, so that the tiled
+        // dimensions are as long as the layouts allow
+        for (size_t d = 0; d + 1 < dims.size();) // the channel dimension stays last
+          if (dims[d].size == 1)
+            dims.erase(dims.begin() + d);
+          else
+            ++d;
+        for (size_t d = 0; d + 1 < dims.size();) {
+          const Dim &o = dims[d], &i = dims[d + 1];
+          if (i.src_size == i.size && o.ss == i.size * i.ss && o.ds == i.size * i.ds &&
+              o.size * i.size <= INT32_MAX) {
+            dims[d] = Dim{o.size * i.size, o.src_size * i.size, i.ss, i.ds};
+            dims.erase(dims.begin() + d + 1);
+          } else {
+            ++d;
+          }
+        }
+        while (dims.size() < 5)
+          dims.insert(dims.begin(), Dim{1, 1, 0, 0});
+        for (int d = 0; d < 5; ++d) {
+          r.size[d] = (int32_t)dims[d].size;
+          r.src_size[d] = (int32_t)dims[d].src_size;
+          r.src_stride[d] = dims[d].ss;
+          r.dst_stride[d] = dims[d].ds;
         }
         r.dst_fast = 4;
         r.src_fast = 4;
@@ -695,13 +730,31 @@ Handle *make_conv(const OptMap &o) {
           if (r.src_stride[d] == 1 && (r.src_stride[r.src_fast] != 1 || r.size[d] > r.size[r.src_fast]))
             r.src_fast = d;
         int64_t blocks = 1;
-        for (int d = 0; d < 5; ++d) {
-          if (d == r.src_fast)
-            blocks *= r.src_fast == r.dst_fast ? (r.size[d] + 1023) / 1024 : (r.size[d] + 31) / 32;
-          else if (d == r.dst_fast)
-            blocks *= (r.size[d] + 31) / 32;
-          else
-            blocks *= r.size[d];
+        if (r.src_fast == r.dst_fast) {
+          // the destination's channel runs are whole 16-byte chunks by construction of cp
+          r.mode = RELAYOUT_COPY;
+          const int64_t chunks = (int64_t)r.size[2] * r.size[3] * (r.size[4] * es / 16);
+          if (chunks > INT32_MAX) {
+            set_error("conv: tensor too large for the layout-conversion kernel");
+            delete h;
+            return nullptr;
+          }
+          blocks = (chunks + 255) / 256 * r.size[1] * r.size[0];
+        } else {
+          // short channel runs: narrow tiles, element-wise; otherwise 128-byte
+          // tile rows with 16-byte accesses
+          const bool vec = r.size[r.dst_fast] > 16 && r.src_stride[r.src_fast] == 1;
+          r.mode = vec ? RELAYOUT_TRANSPOSE_VEC : RELAYOUT_TRANSPOSE;
+          r.tile_d = vec ? 128 / es : r.size[r.dst_fast] <= 8 ? 8 : r.size[r.dst_fast] <= 16 ? 16 : 32;
+          const int tile_s = vec ? 128 / es : 1024 / r.tile_d;
+          for (int d = 0; d < 5; ++d) {
+            if (d == r.src_fast)
+              blocks *= (r.size[d] + tile_s - 1) / tile_s;
+            else if (d == r.dst_fast)
+              blocks *= (r.size[d] + r.tile_d - 1) / r.tile_d;
+            else
+              blocks *= r.size[d];
+          }
         }
         if (blocks > INT32_MAX) {
           set_error("conv: tensor too large for the layout-conversion kernel");
@@ -724,6 +777,8 @@ Handle *make_conv(const OptMap &o) {
       }
       // this handle is the contraction kernel reading the converted tensors
       p = q;
+      c = cp;
+      Kg = cp * y * x;
       fast = true;
       h->ptr_map = {{need_f ? 4 : 0, need_f ? off_f : 0}, {need_i ? 4 : 1, need_i ? off_i : 0}, {2, 0}, {3, 0}};
     }
@@ -791,7 +846,7 @@ Handle *make_conv(const OptMap &o) {
                        : ti == ROCK_FP8 ? "convfp8_fp8" : "convbf8_bf8";
     key << h->arch << '\t' << int_or(o, "num_cu", kNumCU) << '\t' << opname << " -F 1 -f "
         << key_layout(fl, true) << " -I " << key_layout(il, false) << " -O "
-        << key_layout(ol, false) << " -n " << n << " -c " << c << " -H " << hi << " -W " << wi
+        << key_layout(ol, false) << " -n " << n << " -c " << c_problem << " -H " << hi << " -W " << wi
         << " -k " << k << " -y " << y << " -x " << x << " -p " << ph << " -q " << pw << " -u "
         << sh << " -v " << sw << " -l " << dh << " -j " << dw << " -g " << g;
     h->problem_key = key.str();

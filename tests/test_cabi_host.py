@@ -123,8 +123,38 @@ def test_generic_kernels_for_unaligned_or_transposed(rock):
         assert k.kernel_name == "rock_gemm_i8_256x256" + suffix
     nchw = CONV_RESNET.replace("NHWGC", "NGCHW").replace("GNYXC", "GNCHW")
     assert rock.RockKernel(nchw + " --layout_conversion false").kernel_name == "rock_conv_f16_64x64_generic"
-    k = rock.RockKernel(CONV_RESNET.replace("--in_channels 128", "--in_channels 100").replace("NHWGC", "NGCHW"))
-    assert k.kernel_name == "rock_conv_f16_64x64_generic"    # 200-byte channel runs: no vector form to convert to
+    odd = CONV_RESNET.replace("--in_channels 128", "--in_channels 100")
+    assert rock.RockKernel(odd + " --layout_conversion false").kernel_name == "rock_conv_f16_64x64_generic"
+
+
+def test_layout_conversion_pads_channel_runs_to_whole_chunks(rock):
+    """Channel runs that are not a multiple of 16 bytes (3-channel images, 100
+    channels of f16) are zero-padded by the conversion kernels, so the vector
+    contraction kernel runs with the padded count; the problem key keeps the
+    caller's."""
+    first = ("--operation conv --arch gfx950 --in_type fp16 --fil_type fp16 --out_type fp16 --fil_layout GNYXC "
+             "--in_layout NHWGC --out_layout NHWGK --batchsize 4 --groupsize 1 --in_channels 3 --out_channels 64 "
+             "--in_h 230 --in_w 230 --fil_h 7 --fil_w 7 --dilation_h 1 --dilation_w 1 --conv_stride_h 2 "
+             "--conv_stride_w 2 --padding_h 0 --padding_w 0")
+    ks = [rock.RockKernel(first + " --kernel_id %d" % i) for i in range(3)]
+    assert [k.kernel_name for k in ks[:2]] == ["rock_relayout_b2", "rock_relayout_b2"]
+    assert ks[2].kernel_name.startswith("rock_conv_f16_") and ks[2].kernel_name.endswith("_fast")
+    fil_bytes, in_bytes = 64 * 7 * 7 * 8 * 2, 4 * 230 * 230 * 8 * 2   # 3 -> 8 channels
+    for k in ks:
+        assert k.kernel_count == 3 and k.workspace_bytes == fil_bytes + in_bytes
+    # n, h and w fold into one dimension; one thread per 16-byte chunk, 256 chunks a block
+    assert ks[1].grid_size == -(-4 * 230 * 230 // 256)
+    assert " -c 3 " in ks[2].problem_key
+    # NCHW with the same channels: h and w fold; transposing tiles of 8 channels x 128 pixels
+    k = rock.RockKernel(first.replace("NHWGC", "NGCHW") + " --kernel_id 1")
+    assert k.kernel_name == "rock_relayout_b2" and k.grid_size == -(-230 * 230 // 128) * 4
+    # 128 channels: 64 x 64 tiles of 16-bit elements over (channel, folded pixel)
+    nchw = CONV_RESNET.replace("NHWGC", "NGCHW").replace("GNYXC", "GNCHW")
+    k = rock.RockKernel(nchw + " --kernel_id 1")
+    assert k.grid_size == -(-28 * 28 // 64) * (128 // 64) * 256
+    # int8: 16 channels a chunk
+    k8 = rock.RockKernel(first.replace("fp16 --fil_type fp16 --out_type fp16", "i8 --fil_type i8 --out_type i32"))
+    assert k8.workspace_bytes == 64 * 7 * 7 * 16 + (4 * 230 * 230 * 16 + 255) // 256 * 256
 
 
 def test_layout_conversion_plan_follows_the_multi_kernel_protocol(rock):

@@ -113,6 +113,39 @@ def test_conv_mixed_layouts(rock, oracle, gpu, layouts):
     assert np.array_equal(to_f32(out, od), ref)
 
 
+# Channel counts whose runs are not whole 16-byte chunks: the conversion
+# kernels zero-pad them (3 -> 8 f16 / 16 i8 / 4 f32 channels, 100 -> 104 f16).
+# (n g c k hi wi y x stride pad dil)
+PADDED_CASES = [
+    (2, 1, 3, 32, 20, 300, 7, 7, (2, 2), (3, 3), (1, 1)),    # rows longer than one transposing tile
+    (1, 3, 5, 16, 9, 9, 3, 3, (1, 1), (1, 1), (1, 1)),       # groups
+    (1, 1, 100, 24, 6, 6, 3, 3, (1, 1), (1, 1), (1, 1)),     # several chunks a pixel, the last one partial
+    (3, 2, 1, 8, 12, 12, 5, 5, (1, 1), (2, 2), (1, 1)),      # depth-wise-like single channel
+]
+PADDED_LAYOUTS = [NHWC, NCHW, ("gyxck", "hwcgn", "hwkgn"), ("gkcyx", "nhwgc", "ngkhw")]
+
+
+@pytest.mark.parametrize("case", PADDED_CASES)
+@pytest.mark.parametrize("layouts", PADDED_LAYOUTS, ids=lambda l: "-".join(l))
+@pytest.mark.parametrize("t", ["f32", "f16", "i8"])
+def test_conv_channel_padding_exact(rock, oracle, gpu, case, layouts, t):
+    out, od, ref = _run(rock, oracle, gpu, t, *case, layouts, True, 41)
+    if t == "i8":
+        assert oracle.verify_int(out.cpu().numpy().ravel(), ref)[0] == 0
+    else:
+        assert np.array_equal(to_f32(out, od), ref)
+
+
+def test_conv_channel_padding_takes_the_vector_kernel(rock, oracle, gpu):
+    """ResNet50's first layer (conv-configs:1, batch trimmed), real values; the
+    plan's kernels are the two conversions and a vector contraction kernel."""
+    info = {}
+    out, od, ref = _run(rock, oracle, gpu, "f16", 4, 1, 3, 64, 230, 230, 7, 7, (2, 2), (0, 0), (1, 1),
+                        NCHW, False, 43, info=info)
+    assert info["kernels"][:2] == ["rock_relayout_b2", "rock_relayout_b2"] and info["kernels"][2].endswith("_fast")
+    check_float(to_f32(out, od), ref, od)
+
+
 @pytest.mark.parametrize("t", ["f16", "bf16", "f32", "fp8"])
 def test_conv_resnet_block_real_values(rock, oracle, gpu, t):
     """ResNet50 3x3 128->128 @28x28 (conv-configs:5), batch 4: the vector-load
