@@ -337,6 +337,61 @@ std::string forced_tile(const OptMap &o) {
   return "";
 }
 
+// Chooses the kernel, tile and grid for a GEMM whose sizes and strides are
+// already in p.  Returns false when only the element-wise kernel fits.
+bool plan_gemm_kernel(Handle *h, RockGemmParams &p, int code, int es, const OptMap &o) {
+  const int64_t M = p.M, N = p.N, K = p.K, G = p.G;
+  // vector path: K-contiguous rows of whole 16-byte chunks, and every byte
+  // offset inside one block tile (256 rows at most) below 2^31 for the buffer
+  // descriptors of the direct-to-LDS loads
+  const int64_t kMaxOff = (int64_t)1 << 31;
+  auto al16 = [&](int64_t elems) { return (elems * es) % 16 == 0; };
+  // each operand either K-contiguous (rows of whole chunks) or K-major (its
+  // M / N index contiguous, k-rows of whole chunks: the transposing-read path)
+  const bool a_rows = p.a_ks == 1 && al16(p.a_ms) && al16(K) && al16(p.a_gs) && 256 * p.a_ms * es + K * es < kMaxOff;
+  const bool b_rows = p.b_ks == 1 && al16(p.b_ns) && al16(K) && al16(p.b_gs) && 256 * p.b_ns * es + K * es < kMaxOff;
+  const bool a_cols = p.a_ms == 1 && al16(p.a_ks) && al16(M) && al16(p.a_gs) && K * p.a_ks * es + 256 * es < kMaxOff;
+  const bool b_cols = p.b_ns == 1 && al16(p.b_ks) && al16(N) && al16(p.b_gs) && K * p.b_ks * es + 256 * es < kMaxOff;
+  const bool fast = a_rows && b_rows;
+  // storage suffix of the K-major variants: n = as the reference stores it by default
+  const char *storage = nullptr;
+  if (!fast && (a_rows || a_cols) && (b_rows || b_cols))
+    storage = a_rows ? "_nn" : b_rows ? "_tt" : "_tn";
+  const bool tiled = fast || storage;
+  const Tile *tile = tiled ? pick_tile(M, N, p.G, false, forced_tile(o), storage != nullptr) : nullptr;
+  if (!tile)
+    tile = tiled ? pick_tile(M, N, p.G, false, "", storage != nullptr) : &kGenericTile;
+  // Too few 64x64 tiles to occupy half the CUs and a K long enough to split:
+  // one 32x32 tile per block with the K range divided over its waves (the
+  // reference's answer to the same situation is split-K with atomics,
+  // RockTuningImpl.cpp:962-1008).
+  const bool forced = !forced_tile(o).empty();
+  const int64_t tiles64 = (int64_t)ceil_div(M, 64) * ceil_div(N, 64) * G;
+  int split_k = 1;
+  if (fast && !forced && tiles64 * 2 <= kNumCU && K * es >= 16 * 64) {
+    tile = &kSplitKTile;
+    split_k = 4;
+  }
+  if (fast && str_or(o, "perf_config", "").find("32,32,") != std::string::npos) {
+    tile = &kSplitKTile; // "-perf_config v2:32,32,..." asks for it explicitly
+    split_k = 4;
+  }
+  apply_tile_grid(*tile, M, N, p.G, p.tiles_m, p.tiles_n, p.group_m, p.xcd_remap,
+                  h->block_size, h->grid_size);
+  if (split_k > 1)
+    h->block_size = 256;
+  h->kernel_name = std::string("rock_gemm_") + operand_name(code) + tile->suffix + (storage ? storage : "");
+  h->blob_name = std::string("gemm_") + operand_name(code);
+  h->num_pointers = 4;
+  h->perf_config = perf_string(*tile, es);
+  if (split_k > 1) { // the reference's grammar has a splitK field (7th)
+    char buf[96];
+    std::snprintf(buf, sizeof buf, "v2:32,32,4,32,32,%d,%d,1,1", 16 / es, split_k);
+    h->perf_config = buf;
+  }
+  return tiled;
+}
+
 // ---- GEMM -----------------------------------------------------------------
 Handle *make_gemm(const OptMap &o) {
   std::string t = str_or(o, "t", "f32");
@@ -392,55 +447,7 @@ Handle *make_gemm(const OptMap &o) {
   p.b_gs = K * N; p.b_ks = tB ? 1 : N; p.b_ns = tB ? K : 1;
   p.c_gs = M * N; p.c_ms = tC ? 1 : N; p.c_ns = tC ? M : 1;
 
-  const int es = dtype_size(ta);
-  // vector path: K-contiguous rows of whole 16-byte chunks, and every byte
-  // offset inside one block tile (256 rows at most) below 2^31 for the buffer
-  // descriptors of the direct-to-LDS loads
-  const int64_t kMaxOff = (int64_t)1 << 31;
-  auto al16 = [&](int64_t elems) { return (elems * es) % 16 == 0; };
-  // each operand either K-contiguous (rows of whole chunks) or K-major (its
-  // M / N index contiguous, k-rows of whole chunks: the transposing-read path)
-  const bool a_rows = p.a_ks == 1 && al16(p.a_ms) && al16(K) && al16(p.a_gs) && 256 * p.a_ms * es + K * es < kMaxOff;
-  const bool b_rows = p.b_ks == 1 && al16(p.b_ns) && al16(K) && al16(p.b_gs) && 256 * p.b_ns * es + K * es < kMaxOff;
-  const bool a_cols = p.a_ms == 1 && al16(p.a_ks) && al16(M) && al16(p.a_gs) && K * p.a_ks * es + 256 * es < kMaxOff;
-  const bool b_cols = p.b_ns == 1 && al16(p.b_ks) && al16(N) && al16(p.b_gs) && K * p.b_ks * es + 256 * es < kMaxOff;
-  const bool fast = a_rows && b_rows;
-  // storage suffix of the K-major variants: n = as the reference stores it by default
-  const char *storage = nullptr;
-  if (!fast && (a_rows || a_cols) && (b_rows || b_cols))
-    storage = a_rows ? "_nn" : b_rows ? "_tt" : "_tn";
-  const bool tiled = fast || storage;
-  const Tile *tile = tiled ? pick_tile(M, N, (int)G, false, forced_tile(o), storage != nullptr) : nullptr;
-  if (!tile)
-    tile = tiled ? pick_tile(M, N, (int)G, false, "", storage != nullptr) : &kGenericTile;
-  // Too few 64x64 tiles to occupy half the CUs and a K long enough to split:
-  // one 32x32 tile per block with the K range divided over its waves (the
-  // reference's answer to the same situation is split-K with atomics,
-  // RockTuningImpl.cpp:962-1008).
-  const bool forced = !forced_tile(o).empty();
-  const int64_t tiles64 = (int64_t)ceil_div(M, 64) * ceil_div(N, 64) * G;
-  int split_k = 1;
-  if (fast && !forced && tiles64 * 2 <= kNumCU && K * es >= 16 * 64) {
-    tile = &kSplitKTile;
-    split_k = 4;
-  }
-  if (fast && str_or(o, "perf_config", "").find("32,32,") != std::string::npos) {
-    tile = &kSplitKTile; // "-perf_config v2:32,32,..." asks for it explicitly
-    split_k = 4;
-  }
-  apply_tile_grid(*tile, M, N, (int)G, p.tiles_m, p.tiles_n, p.group_m, p.xcd_remap,
-                  h->block_size, h->grid_size);
-  if (split_k > 1)
-    h->block_size = 256;
-  h->kernel_name = std::string("rock_gemm_") + operand_name(code) + tile->suffix + (storage ? storage : "");
-  h->blob_name = std::string("gemm_") + operand_name(code);
-  h->num_pointers = 4;
-  h->perf_config = perf_string(*tile, es);
-  if (split_k > 1) { // the reference's grammar has a splitK field (7th)
-    char buf[96];
-    std::snprintf(buf, sizeof buf, "v2:32,32,4,32,32,%d,%d,1,1", 16 / es, split_k);
-    h->perf_config = buf;
-  }
+  plan_gemm_kernel(h, p, code, dtype_size(ta), o);
   // problem key (RockTuningImpl.cpp:808-862)
   {
     std::ostringstream k;
@@ -638,6 +645,45 @@ Handle *make_conv(const OptMap &o) {
            (256 * q.fil_ks + cc * y * x) * es < ((int64_t)1 << 31);
   };
   bool fast = conv_fast(p, c);
+
+  auto set_problem_key = [&] {
+    std::ostringstream key;
+    const char *opname = ti == ROCK_F32 ? "conv" : ti == ROCK_F16 ? "convfp16"
+                       : ti == ROCK_BF16 ? "convbfp16" : ti == ROCK_I8 ? "convint8"
+                       : ti == ROCK_FP8 ? "convfp8_fp8" : "convbf8_bf8";
+    key << h->arch << '\t' << int_or(o, "num_cu", kNumCU) << '\t' << opname << " -F 1 -f "
+        << key_layout(fl, true) << " -I " << key_layout(il, false) << " -O "
+        << key_layout(ol, false) << " -n " << n << " -c " << c_problem << " -H " << hi << " -W " << wi
+        << " -k " << k << " -y " << y << " -x " << x << " -p " << ph << " -q " << pw << " -u "
+        << sh << " -v " << sw << " -l " << dh << " -j " << dw << " -g " << g;
+    h->problem_key = key.str();
+  };
+
+  // A 1x1 filter with unit stride, no padding and one group over images whose
+  // pixels are contiguous (NCHW): image n's output is filter[k, c] x
+  // input_n[c, h*w], a batched GEMM with the filter shared by the batch and the
+  // second operand stored K-major.  The transposing-read GEMM kernels take it
+  // as it lies: no conversion, no workspace.  (A per-channel bias would run
+  // along GEMM rows, which the epilogue does not do; such problems convert.)
+  if (!fast && y == 1 && x == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && g == 1 && !p.epi.has_bias &&
+      p.in_ws == 1 && p.in_hs == wi && p.out_ws == 1 && p.out_hs == wo && hi * wi <= INT32_MAX &&
+      bool_or(o, "pointwise_as_gemm", true)) {
+    RockGemmParams gp;
+    std::memset(&gp, 0, sizeof gp);
+    gp.G = (int)n; gp.M = (int)k; gp.N = (int)(hi * wi); gp.K = (int)c;
+    gp.a_gs = 0; gp.a_ms = p.fil_ks; gp.a_ks = p.fil_cs;
+    gp.b_gs = p.in_ns; gp.b_ns = 1; gp.b_ks = p.in_cs;
+    gp.c_gs = p.out_ns; gp.c_ms = p.out_ks; gp.c_ns = 1;
+    gp.epi = p.epi;
+    if (plan_gemm_kernel(h, gp, operand_code(ti, ti), es, o)) {
+      h->op = OP_GEMM;
+      h->params.assign(sizeof gp, 0); // p is gone from here on
+      std::memcpy(h->params.data(), &gp, sizeof gp);
+      h->epi = &reinterpret_cast<RockGemmParams *>(h->params.data())->epi;
+      set_problem_key();
+      return h;
+    }
+  }
 
   // Layout-conversion plan.  A problem whose filter or input is not
   // channel-contiguous (the reference's default gkcyx / ngchw) would run the
@@ -839,18 +885,7 @@ Handle *make_conv(const OptMap &o) {
       h->perf_config = buf;
     }
   }
-  {
-    std::ostringstream key;
-    const char *opname = ti == ROCK_F32 ? "conv" : ti == ROCK_F16 ? "convfp16"
-                       : ti == ROCK_BF16 ? "convbfp16" : ti == ROCK_I8 ? "convint8"
-                       : ti == ROCK_FP8 ? "convfp8_fp8" : "convbf8_bf8";
-    key << h->arch << '\t' << int_or(o, "num_cu", kNumCU) << '\t' << opname << " -F 1 -f "
-        << key_layout(fl, true) << " -I " << key_layout(il, false) << " -O "
-        << key_layout(ol, false) << " -n " << n << " -c " << c_problem << " -H " << hi << " -W " << wi
-        << " -k " << k << " -y " << y << " -x " << x << " -p " << ph << " -q " << pw << " -u "
-        << sh << " -v " << sw << " -l " << dh << " -j " << dw << " -g " << g;
-    h->problem_key = key.str();
-  }
+  set_problem_key();
   return h;
 }
 

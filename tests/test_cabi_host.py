@@ -127,6 +127,26 @@ def test_generic_kernels_for_unaligned_or_transposed(rock):
     assert rock.RockKernel(odd + " --layout_conversion false").kernel_name == "rock_conv_f16_64x64_generic"
 
 
+def test_pointwise_nchw_convolution_is_a_k_major_gemm(rock):
+    """1x1, stride 1, no padding, one group, NCHW: filter[k,c] x image[c,h*w]
+    batched over n on the transposing-read GEMM kernel, one kernel, no workspace."""
+    pw = ("--operation conv --arch gfx950 --in_type fp16 --fil_type fp16 --out_type fp16 --fil_layout GNCYX "
+          "--in_layout NGCHW --out_layout NGCHW --batchsize 256 --groupsize 1 --in_channels 256 --out_channels 64 "
+          "--in_h 56 --in_w 56 --fil_h 1 --fil_w 1 --dilation_h 1 --dilation_w 1 --conv_stride_h 1 "
+          "--conv_stride_w 1 --padding_h 0 --padding_w 0")
+    k = rock.RockKernel(pw)
+    assert k.kernel_name.startswith("rock_gemm_f16_") and k.kernel_name.endswith("_fast_nn")
+    assert (k.kernel_count, k.workspace_bytes, k.num_pointers) == (1, 0, 4)
+    assert "convfp16" in k.problem_key and " -y 1 -x 1 " in k.problem_key
+    # anything the GEMM form cannot express converts instead
+    for change in (("--conv_stride_h 1", "--conv_stride_h 2"), ("--padding_w 0", "--padding_w 1"),
+                   ("--in_h 56 --in_w 56", "--in_h 7 --in_w 7"), ("--out_layout NGCHW", "--out_layout NHWGC")):
+        k = rock.RockKernel(pw.replace(*change))
+        assert k.kernel_count == 3, change
+    assert rock.RockKernel(pw + " --bias true").kernel_count == 3
+    assert rock.RockKernel(pw + " --pointwise_as_gemm false").kernel_count == 3
+
+
 def test_layout_conversion_pads_channel_runs_to_whole_chunks(rock):
     """Channel runs that are not a multiple of 16 bytes (3-channel images, 100
     channels of f16) are zero-padded by the conversion kernels, so the vector

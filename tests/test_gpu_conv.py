@@ -113,6 +113,32 @@ def test_conv_mixed_layouts(rock, oracle, gpu, layouts):
     assert np.array_equal(to_f32(out, od), ref)
 
 
+# 1x1 filters over NCHW images run as a batched GEMM with a K-major second
+# operand (no conversion kernels).  (n c k hi wi)
+POINTWISE_CASES = [(3, 64, 48, 8, 8), (2, 32, 200, 12, 12), (5, 16, 16, 16, 4), (1, 128, 300, 28, 28)]
+
+
+@pytest.mark.parametrize("case", POINTWISE_CASES)
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16", "i8"])
+def test_conv_pointwise_nchw_as_gemm_exact(rock, oracle, gpu, case, t):
+    n, c, k, hi, wi = case
+    info = {}
+    out, od, ref = _run(rock, oracle, gpu, t, n, 1, c, k, hi, wi, 1, 1, (1, 1), (0, 0), (1, 1), NCHW, True, 45,
+                        info=info)
+    assert info["kernels"] == [info["kernel_name"]] and info["kernel_name"].startswith("rock_gemm_")
+    assert info["kernel_name"].endswith("_fast_nn")
+    if t == "i8":
+        assert oracle.verify_int(out.cpu().numpy().ravel(), ref)[0] == 0
+    else:
+        assert np.array_equal(to_f32(out, od), oracle.round_through(ref, CODE[od]))
+
+
+def test_conv_pointwise_nchw_real_values_with_epilogue(rock, oracle, gpu):
+    out, od, ref = _run(rock, oracle, gpu, "f16", 4, 1, 256, 64, 56, 56, 1, 1, (1, 1), (0, 0), (1, 1), NCHW, False,
+                        47, scale=0.5, relu=True)
+    check_float(to_f32(out, od), np.maximum(ref * 0.5, 0.0), od)
+
+
 # Channel counts whose runs are not whole 16-byte chunks: the conversion
 # kernels zero-pad them (3 -> 8 f16 / 16 i8 / 4 f32 channels, 100 -> 104 f16).
 # (n g c k hi wi y x stride pad dil)
