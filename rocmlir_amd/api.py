@@ -376,7 +376,8 @@ def _torch_dtype(name):
             "fp8": torch.float8_e4m3fn, "bf8": torch.float8_e5m2}[name]
 
 
-def _epilogue_flags(scale, zero_point, bias, relu, quant_scale, out_zero_point):
+def _epilogue_flags(scale, zero_point, bias, relu, quant_scale, out_zero_point,
+                    activation=None, clip=None, residual=None, residual_op="add"):
     s = ""
     if scale is not None:
         s += " -scale %.9g" % scale
@@ -390,17 +391,28 @@ def _epilogue_flags(scale, zero_point, bias, relu, quant_scale, out_zero_point):
         s += " -bias true"
     if relu:
         s += " -relu true"
+    if activation:
+        s += " -activation %s" % activation
+    if clip is not None:
+        s += " -activation clip -clip_min %.9g -clip_max %.9g" % tuple(clip)
+    if residual is not None:
+        s += " -residual %s" % residual_op
     return s
 
 
 def gemm(a, b, *, transA=False, transB=False, transC=False, out_dtype=None,
          scale=None, zero_point=0, bias=None, relu=False, quant_scale=None,
-         out_zero_point=0, out=None, perf_config=None, stream=None,
+         out_zero_point=0, activation=None, clip=None, residual=None,
+         residual_op="add", out=None, perf_config=None, stream=None,
          info=None):
     """C = epilogue(A x B) with the reference's storage conventions
     (rocmlir-gen.cpp:2058-2080): a is [G,M,K] ([G,K,M] if transA), b is
     [G,K,N] ([G,N,K] if transB), result [G,M,N] ([G,N,M] if transC).
-    2-D inputs mean G = 1.  A dict passed as `info` receives the name and
+    2-D inputs mean G = 1.  The epilogue runs scale / zero point, per-column
+    `bias`, `residual` (a tensor shaped and typed like the result, combined by
+    `residual_op` "add" or "mul"), then `activation` ("relu", "sigmoid",
+    "tanh", "erf", "gelu", "exp") or `clip=(lo, hi)`, then the narrowing to
+    the output type.  A dict passed as `info` receives the name and
     perf_config of the kernel that ran."""
     import torch
     a3 = a if a.dim() == 3 else a.unsqueeze(0)
@@ -422,7 +434,8 @@ def gemm(a, b, *, transA=False, transB=False, transC=False, out_dtype=None,
     if perf_config:
         opts += " -perf_config %s" % perf_config
     opts += _epilogue_flags(scale, zero_point, bias, relu, quant_scale,
-                            out_zero_point)
+                            out_zero_point, activation, clip, residual,
+                            residual_op)
     k = _kernel(opts)
     if info is not None:
         info["kernel_name"] = k.kernel_name
@@ -432,7 +445,12 @@ def gemm(a, b, *, transA=False, transB=False, transC=False, out_dtype=None,
     shape = (G, N, M) if transC else (G, M, N)
     if out is None:
         out = torch.empty(shape, dtype=_torch_dtype(out_dtype), device=a.device)
-    k.launch(a3, b3, out, bias, stream=stream)
+    if residual is None:
+        k.launch(a3, b3, out, bias, stream=stream)
+    else:
+        if residual.dtype != out.dtype or residual.numel() != out.numel():
+            raise RockError("gemm: the residual must have the result's type and size")
+        k.launch(a3, b3, out, bias, residual.contiguous(), stream=stream)
     return out if a.dim() == 3 else out.squeeze(0)
 
 
@@ -440,11 +458,13 @@ def conv2d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize,
            in_channels, out_channels, in_h, in_w, fil_h, fil_w, groupsize=1,
            stride=(1, 1), padding=(0, 0), dilation=(1, 1), out_dtype=None,
            scale=None, zero_point=0, bias=None, relu=False, quant_scale=None,
-           out_zero_point=0, out=None, perf_config=None, stream=None,
+           out_zero_point=0, activation=None, clip=None, residual=None,
+           residual_op="add", out=None, perf_config=None, stream=None,
            info=None):
     """Forward convolution; tensors are flat device buffers laid out as the
     layout strings say (Miir / rocmlir-gen spelling, e.g. 'gkyxc', 'nhwgc',
-    'NGCHW').  Returns the flat output tensor.  A dict passed as `info`
+    'NGCHW').  Epilogue arguments as for gemm(); the residual is laid out
+    like the output.  Returns the flat output tensor.  A dict passed as `info`
     receives the name and perf_config of the kernel that ran."""
     import torch
     t = _dtype_name(inp.dtype)
@@ -465,7 +485,8 @@ def conv2d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize,
     if perf_config:
         opts += " --perf_config %s" % perf_config
     opts += _epilogue_flags(scale, zero_point, bias, relu, quant_scale,
-                            out_zero_point)
+                            out_zero_point, activation, clip, residual,
+                            residual_op)
     prog = _program(opts)
     k = prog.main
     if info is not None:
@@ -477,7 +498,12 @@ def conv2d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize,
     if out is None:
         out = torch.empty(batchsize * out_channels * ho * wo,
                           dtype=_torch_dtype(out_dtype), device=inp.device)
-    prog.launch(fil.contiguous(), inp.contiguous(), out, bias, stream=stream)
+    if residual is None:
+        prog.launch(fil.contiguous(), inp.contiguous(), out, bias, stream=stream)
+    else:
+        if residual.dtype != out.dtype or residual.numel() != out.numel():
+            raise RockError("conv2d: the residual must have the output's type and size")
+        prog.launch(fil.contiguous(), inp.contiguous(), out, bias, residual.contiguous(), stream=stream)
     return out
 
 

@@ -42,9 +42,9 @@ namespace rk {
 constexpr int kDirectWindowBytes = 96 * 1024;
 constexpr int kDirectSlabsPerWave = 8; // a window row is at most 32 KiB
 
-template <int DT, int TMB, int MSPLIT>
+template <int DT, int TMB, int MSPLIT, bool RICH = false>
 __device__ __forceinline__ void conv_direct_body(const void *in, const void *fil, void *out, const void *aux,
-                                                 const RockConvParams &p) {
+                                                 const void *res, const RockConvParams &p) {
   using Tr = MmaTraits<DT>;
   using Acc = typename Tr::Acc;
   constexpr int ES = Tr::ES;
@@ -227,7 +227,7 @@ __device__ __forceinline__ void conv_direct_body(const void *in, const void *fil
   // ---- epilogue: the tile is the contiguous pixel range [r0*Wo, r_end*Wo) of the implicit GEMM's M
   RockConvParams pe = p;
   pe.M = r_end * p.wo;
-  dl_epilogue<DT, TMW, 1, NWAVE, NS * B_STAGE>(acc, pe, g, out, aux, r0 * p.wo + mh * TMW * 32, n0 + nb * 32, ring,
+  dl_epilogue<DT, TMW, 1, NWAVE, NS * B_STAGE, RICH>(acc, pe, g, out, aux, res, r0 * p.wo + mh * TMW * 32, n0 + nb * 32, ring,
                                                wave, lane);
 }
 

@@ -408,17 +408,175 @@ __device__ __forceinline__ Frag<DT> dl_read_frag(const char *lds, int row, int s
 // Epilogue of the direct-to-LDS bodies: lane holds m = m_wave + 32*i + lrow,
 // n = n_wave + 32*j + 8*q + 4*lgrp + {0..3}.  `lds` is the block's operand
 // ring (LDS_BYTES), free once every wave has passed the barrier at the top;
-// NWAVES waves call this, each with its own `wave` index in [0, NWAVES).  A
-// wave of the block that holds no accumulators and does not call it must
-// still execute that barrier: it does so when dl_epilogue_staged() is true.
+// NWAVES waves call this, each with its own `wave` index in [0, NWAVES); it
+// contains a workgroup barrier, so every wave of the block must call it.
 template <typename Params>
 __device__ __forceinline__ bool dl_epilogue_staged(const Params &p, const void *Cptr) {
   return out_rows_chunk_aligned(p, Cptr, out_elem_size(p.epi.out_dtype));
 }
 
+// Epilogue with a residual tensor or a transcendental activation.  Unrolled
+// over the accumulator registers, such an epilogue would repeat its loads,
+// address arithmetic and math routines for every group of four outputs (128
+// times in the largest tile, once more per output type) and dominate the code
+// object and its build time.  Instead everything but the register moves is
+// rolled: per 32-row block of the wave tile, the raw accumulators are parked in
+// the wave's LDS region (16 bytes per lane per group, lane-private), ONE loop
+// runs the whole epilogue on each group with the output type as a run-time
+// switch and leaves the packed result in its slot, and the results take the
+// same staged or direct store as the plain epilogue.  The loop over blocks is
+// rolled too; only the parking is specialised per block.
+template <int ES, int NI, typename Params>
+__device__ __forceinline__ void dl_rich_store(const Params &p, int g, void *Cptr, char *wbuf, int m_block,
+                                              int n_wave, int lane, bool staged_ok) {
+  constexpr int WTN = NI * 32;
+  constexpr int ROWB = WTN * ES, PITCH = ROWB + 16;
+  constexpr int LPR = ROWB / 16, RPI = 64 / LPR;
+  const int lrow = lane & 31, lgrp = lane >> 5;
+  const int rd_row = lane / LPR, rd_cb = (lane % LPR) * 16;
+  v4i raw[NI * 4];
+#pragma unroll
+  for (int t = 0; t < NI * 4; ++t)
+    raw[t] = *(const v4i *)(wbuf + (t * 64 + lane) * 16);
+  if (!staged_ok) {
+    const int m = m_block + lrow;
+    if (m < p.M) {
+      int64_t row_off, n_stride;
+      bool vec_ok;
+      out_row_addr(p, g, m, Cptr, row_off, n_stride, vec_ok);
+#pragma unroll
+      for (int t = 0; t < NI * 4; ++t) {
+        const int n = n_wave + (t >> 2) * 32 + (t & 3) * 8 + lgrp * 4;
+        if (n < p.N)
+          store_packed4(raw[t], ES, Cptr, row_off + (int64_t)n * n_stride, n_stride, n, p.N, vec_ok);
+      }
+    }
+    return;
+  }
+  // transposition through the same buffer: every lane of the wave has read
+  // its slots (LDS operations of one wave complete in order)
+#pragma unroll
+  for (int t = 0; t < NI * 4; ++t) {
+    const int nloc = (t >> 2) * 32 + (t & 3) * 8 + lgrp * 4;
+    char *dst = wbuf + lrow * PITCH + nloc * ES;
+    if constexpr (ES == 4)
+      *(v4i *)dst = raw[t];
+    else if constexpr (ES == 2)
+      *(v2i *)dst = v2i{raw[t][0], raw[t][1]};
+    else
+      *(int *)dst = raw[t][0];
+  }
+#pragma unroll
+  for (int r0 = 0; r0 < 32; r0 += RPI) {
+    const int row = r0 + rd_row;
+    v4i d = *(const v4i *)(wbuf + row * PITCH + rd_cb);
+    const int m = m_block + row;
+    const int n = n_wave + rd_cb / ES;
+    if (m < p.M && n < p.N) {
+      int64_t row_off, n_stride;
+      bool vec_ok;
+      out_row_addr(p, g, m, Cptr, row_off, n_stride, vec_ok);
+      *(v4i *)((char *)Cptr + (row_off + n) * ES) = d;
+    }
+  }
+}
+
 template <int DT, int MI, int NI, int NWAVES, int LDS_BYTES, typename Params>
+__device__ __forceinline__ void dl_epilogue_rich(typename MmaTraits<DT>::Acc (&acc)[MI][NI], const Params &p, int g,
+                                                 void *Cptr, const void *aux, const void *res, int m_wave,
+                                                 int n_wave, char *lds, int wave, int lane, bool staged_ok) {
+  using Tr = MmaTraits<DT>;
+  constexpr int WTN = NI * 32;
+  constexpr int WBUF = 32 * (WTN * 4 + 16);
+  static_assert(NWAVES * WBUF <= LDS_BYTES, "staging buffers must fit in the operand stages");
+  static_assert(NI * 4 * 1024 <= WBUF, "parked accumulators must fit in the wave's staging buffer");
+  using Acc4 = decltype(__builtin_shufflevector(acc[0][0], acc[0][0], 0, 1, 2, 3));
+  const RockEpilogue &e = p.epi;
+  const int lrow = lane & 31, lgrp = lane >> 5;
+  char *wbuf = lds + wave * WBUF;
+  const int od = e.out_dtype;
+  const bool slow = activation_is_slow(e);
+#pragma unroll 1
+  for (int i = 0; i < MI; ++i) {
+    // park block i: the only step that names registers
+    static_for<MI>([&](auto ic) __attribute__((always_inline)) {
+      if (i == ic.value) {
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            Acc4 a4 = {acc[ic.value][j][4 * q + 0], acc[ic.value][j][4 * q + 1], acc[ic.value][j][4 * q + 2],
+                       acc[ic.value][j][4 * q + 3]};
+            *(Acc4 *)(wbuf + ((j * 4 + q) * 64 + lane) * 16) = a4;
+          }
+        }
+      }
+    });
+    const int m = m_wave + i * 32 + lrow;
+    const void *res_row = nullptr;
+    int64_t row_off = 0, n_stride = 1;
+    if (m < p.M && e.residual_op) {
+      bool unused;
+      out_row_addr(p, g, m, Cptr, row_off, n_stride, unused);
+      res_row = res;
+    }
+#pragma unroll 1
+    for (int t = 0; t < NI * 4; ++t) {
+      char *slot = wbuf + (t * 64 + lane) * 16;
+      const int n = n_wave + (t >> 2) * 32 + (t & 3) * 8 + lgrp * 4;
+      const Acc4 a4 = *(const Acc4 *)slot;
+      const int64_t res_off = row_off + (int64_t)n * n_stride;
+      if (Tr::INT_ACC && od == ROCK_I32) {
+        if constexpr (Tr::INT_ACC)
+          *(v4i *)slot = epilogue_convert4<true, ROCK_I32>(a4, e, aux, n, p.N, res_row, res_off, n_stride);
+        continue;
+      }
+      float v[4];
+      epilogue_affine4<Tr::INT_ACC, ROCK_DTYPE_COUNT>(a4, e, aux, n, p.N, nullptr, 0, 1, v);
+      if (res_row) {
+        *(v4f *)slot = v4f{v[0], v[1], v[2], v[3]};
+#pragma unroll 1
+        for (int r = 0; r < 4; ++r) {
+          if (n + r < p.N) {
+            float *f = (float *)slot + r;
+            const float rv = load_out_elem_rt(res_row, res_off + r * n_stride, od);
+            *f = e.residual_op == ROCK_RES_ADD ? *f + rv : *f * rv;
+          }
+        }
+        const v4f x = *(const v4f *)slot;
+        v[0] = x[0]; v[1] = x[1]; v[2] = x[2]; v[3] = x[3];
+      }
+      if (slow) { // one copy of the routine: loop over the slot, not over registers
+        *(v4f *)slot = v4f{v[0], v[1], v[2], v[3]};
+#pragma unroll 1
+        for (int r = 0; r < 4; ++r) {
+          float *f = (float *)slot + r;
+          *f = activation_slow(*f, e.activation);
+        }
+        const v4f x = *(const v4f *)slot;
+        v[0] = x[0]; v[1] = x[1]; v[2] = x[2]; v[3] = x[3];
+      } else if (e.activation) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          v[r] = activation_fast(v[r], e);
+      }
+      *(v4i *)slot = epilogue_pack4_rt(v, od, e);
+    }
+    const int es = out_elem_size(od);
+    if (es == 4)
+      dl_rich_store<4, NI>(p, g, Cptr, wbuf, m_wave + i * 32, n_wave, lane, staged_ok);
+    else if (es == 2)
+      dl_rich_store<2, NI>(p, g, Cptr, wbuf, m_wave + i * 32, n_wave, lane, staged_ok);
+    else
+      dl_rich_store<1, NI>(p, g, Cptr, wbuf, m_wave + i * 32, n_wave, lane, staged_ok);
+  }
+}
+
+// RICH kernels are separate instantiations (kernel name suffix "_e") so that
+// the plain kernels' register allocation is untouched by the rich path.
+template <int DT, int MI, int NI, int NWAVES, int LDS_BYTES, bool RICH = false, typename Params>
 __device__ __forceinline__ void dl_epilogue(typename MmaTraits<DT>::Acc (&acc)[MI][NI], const Params &p, int g,
-                                            void *Cptr, const void *aux, int m_wave, int n_wave, char *lds,
+                                            void *Cptr, const void *aux, const void *res, int m_wave, int n_wave, char *lds,
                                             int wave, int lane) {
   using Tr = MmaTraits<DT>;
   constexpr int WTN = NI * 32;
@@ -426,14 +584,21 @@ __device__ __forceinline__ void dl_epilogue(typename MmaTraits<DT>::Acc (&acc)[M
   const RockEpilogue &e = p.epi;
   using Acc4 = decltype(__builtin_shufflevector(acc[0][0], acc[0][0], 0, 1, 2, 3));
   const bool staged_ok = dl_epilogue_staged(p, Cptr);
+  if constexpr (RICH) {
+    __builtin_amdgcn_s_barrier(); // every wave is done reading the operand stages
+    dl_epilogue_rich<DT, MI, NI, NWAVES, LDS_BYTES>(acc, p, g, Cptr, aux, res, m_wave, n_wave, lds, wave, lane,
+                                                    staged_ok);
+    return;
+  }
   if (staged_ok)
     __builtin_amdgcn_s_barrier(); // every wave is done reading the operand stages
 
   dispatch_out_dtype<Tr::INT_ACC>(e.out_dtype, [&](auto od_const) __attribute__((always_inline)) {
     constexpr int OD = decltype(od_const)::value;
+    // plain epilogue (scale, bias, relu / clip, narrowing): unrolled over the registers
     if (!staged_ok) {
-      direct_epilogue<Tr::INT_ACC, OD, MI, NI, Acc4>(acc, p, g, Cptr, aux, m_wave + lrow,
-                                                    n_wave + lgrp * 4);
+      direct_epilogue<Tr::INT_ACC, OD, MI, NI, Acc4, false>(acc, p, g, Cptr, aux, nullptr, m_wave + lrow,
+                                                           n_wave + lgrp * 4);
       return;
     }
     // Staged store: each wave transposes one 32-row block of its tile at a
@@ -484,9 +649,10 @@ __device__ __forceinline__ void dl_epilogue(typename MmaTraits<DT>::Acc (&acc)[M
 }
 
 
-template <int DT, int BM, int BN, int WAVES_M, int WAVES_N, int RB, int LDA, int LDB, typename Params>
+template <int DT, int BM, int BN, int WAVES_M, int WAVES_N, int RB, int LDA, int LDB, bool RICH = false,
+          typename Params>
 __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void *Bptr, void *Cptr,
-                                                    const void *aux, const Params &p) {
+                                                    const void *aux, const void *res, const Params &p) {
   using Tr = MmaTraits<DT>;
   using Acc = typename Tr::Acc;
   constexpr int NW = WAVES_M * WAVES_N;
@@ -582,7 +748,7 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
   // drain the out-of-range loads issued for steps >= nk before the LDS is released
   wait_vmcnt<0>();
 
-  dl_epilogue<DT, MI, NI, NW, kDlStages * STAGE>(acc, p, g, Cptr, aux, m0 + wm * WTM, n0 + wn * WTN, lds, wave,
+  dl_epilogue<DT, MI, NI, NW, kDlStages * STAGE, RICH>(acc, p, g, Cptr, aux, res, m0 + wm * WTM, n0 + wn * WTN, lds, wave,
                                                  lane);
 }
 

@@ -268,69 +268,179 @@ __device__ __forceinline__ int out_elem_size(int od) {
   return (od == ROCK_F32 || od == ROCK_I32) ? 4 : (od == ROCK_F16 || od == ROCK_BF16) ? 2 : 1;
 }
 
-// acc[r] belongs to output channel n0 + r.  Returns the 4 results packed
-// back to back in the low 4*elem_size bytes.  OD (the output type) is a
-// compile-time constant so that the unrolled epilogue is straight-line code.
+// relu and clip cost an instruction or two and are applied where the
+// accumulators sit.  The transcendental activations are long routines; a
+// copy per accumulator element of an unrolled epilogue would dominate the code
+// object, so the tiled kernels run them in a rolled loop over values parked in
+// LDS (dl_epilogue) and the element-wise kernels call them out of line.
+__device__ __forceinline__ bool activation_is_slow(const RockEpilogue &e) { return e.activation > ROCK_ACT_CLIP; }
+
+// relu and clip are one clamp: the host resolves the bounds (relu: [0, +inf))
+__device__ __forceinline__ float activation_fast(float v, const RockEpilogue &e) {
+  return fminf(fmaxf(v, e.act_lo), e.act_hi);
+}
+
+__device__ __forceinline__ float activation_slow(float v, int activation) {
+  switch (activation) { // uniform
+  case ROCK_ACT_SIGMOID: return 1.0f / (1.0f + expf(-v));
+  case ROCK_ACT_TANH: return tanhf(v);
+  case ROCK_ACT_ERF: return erff(v);
+  case ROCK_ACT_GELU: return 0.5f * v * (1.0f + erff(v * 0.70710678118654752f));
+  case ROCK_ACT_EXP: return expf(v);
+  default: return v;
+  }
+}
+__device__ __attribute__((noinline)) float activation_slow_call(float v, int activation) {
+  return activation_slow(v, activation);
+}
+
+// One element of a tensor of the output type, widened.
+template <int OD> __device__ __forceinline__ float load_out_elem(const void *base, int64_t idx) {
+  if constexpr (OD == ROCK_F32)
+    return ((const float *)base)[idx];
+  else if constexpr (OD == ROCK_F16)
+    return (float)((const _Float16 *)base)[idx];
+  else if constexpr (OD == ROCK_BF16)
+    return __builtin_bit_cast(float, (uint32_t)((const uint16_t *)base)[idx] << 16);
+  else if constexpr (OD == ROCK_I8)
+    return (float)((const int8_t *)base)[idx];
+  else if constexpr (OD == ROCK_FP8)
+    return e4m3fn_to_f32(((const uint8_t *)base)[idx]);
+  else if constexpr (OD == ROCK_BF8)
+    return e5m2_to_f32(((const uint8_t *)base)[idx]);
+  else
+    return (float)((const int *)base)[idx];
+}
+
+// The same with the type as a run-time value (uniform across the block).
+__device__ __forceinline__ float load_out_elem_rt(const void *base, int64_t idx, int od) {
+  switch (od) {
+  case ROCK_F32: return load_out_elem<ROCK_F32>(base, idx);
+  case ROCK_F16: return load_out_elem<ROCK_F16>(base, idx);
+  case ROCK_BF16: return load_out_elem<ROCK_BF16>(base, idx);
+  case ROCK_I8: return load_out_elem<ROCK_I8>(base, idx);
+  case ROCK_FP8: return load_out_elem<ROCK_FP8>(base, idx);
+  case ROCK_BF8: return load_out_elem<ROCK_BF8>(base, idx);
+  default: return load_out_elem<ROCK_I32>(base, idx);
+  }
+}
+
+template <int N, typename F> __device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (N > 0) {
+    static_for<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+}
+
+// Steps 1-3 of the epilogue for 4 consecutive output channels of one row:
+// acc[r] belongs to channel n0 + r.  `res` is the residual tensor and res_off
+// the element offset of (row, n0) in it, channels res_ns apart; null when the
+// epilogue names no residual operation or the row is out of range.
 template <bool INT_ACC, int OD, typename Acc4>
+__device__ __forceinline__ void epilogue_affine4(const Acc4 &acc, const RockEpilogue &e, const void *aux,
+                                                 int n0, int n_limit, const void *res, int64_t res_off,
+                                                 int64_t res_ns, float (&v)[4]) {
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    float f;
+    if constexpr (INT_ACC)
+      f = ((float)(int)acc[r] - (float)e.zero_point) * e.scale;
+    else
+      f = (float)acc[r] * e.scale;
+    if (e.has_bias && n0 + r < n_limit)
+      f = f + ((const float *)aux)[n0 + r];
+    if (res && n0 + r < n_limit) {
+      const float rv = load_out_elem<OD>(res, res_off + r * res_ns);
+      f = e.residual_op == ROCK_RES_ADD ? f + rv : f * rv;
+    }
+    v[r] = f;
+  }
+}
+
+// Step 5: 4 values narrowed to the output type and packed back to back in the
+// low 4*elem_size bytes.
+template <int OD> __device__ __forceinline__ v4i epilogue_pack4(const float (&v)[4], const RockEpilogue &e) {
+  v4i out = {0, 0, 0, 0};
+  if constexpr (OD == ROCK_F32 || OD == ROCK_I32) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      out[r] = __builtin_bit_cast(int, v[r]);
+  } else if constexpr (OD == ROCK_F16) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      _Float16 hv = (_Float16)v[r];
+      out[r >> 1] |= (int)__builtin_bit_cast(uint16_t, hv) << (16 * (r & 1));
+    }
+  } else if constexpr (OD == ROCK_BF16) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      __bf16 hv = (__bf16)v[r];
+      out[r >> 1] |= (int)__builtin_bit_cast(uint16_t, hv) << (16 * (r & 1));
+    }
+  } else if constexpr (OD == ROCK_I8) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float q = __builtin_rintf(v[r] * e.inv_quant_scale) + (float)e.out_zero_point;
+      out[0] |= ((int)f32_to_i8_sat(q) & 0xff) << (8 * r);
+    }
+  } else if constexpr (OD == ROCK_FP8) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      out[0] |= (int)f32_to_e4m3fn_sat(v[r]) << (8 * r);
+  } else if constexpr (OD == ROCK_BF8) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      out[0] |= (int)f32_to_e5m2_sat(v[r]) << (8 * r);
+  }
+  return out;
+}
+
+__device__ __forceinline__ v4i epilogue_pack4_rt(const float (&v)[4], int od, const RockEpilogue &e) {
+  switch (od) {
+  case ROCK_F32: return epilogue_pack4<ROCK_F32>(v, e);
+  case ROCK_F16: return epilogue_pack4<ROCK_F16>(v, e);
+  case ROCK_BF16: return epilogue_pack4<ROCK_BF16>(v, e);
+  case ROCK_I8: return epilogue_pack4<ROCK_I8>(v, e);
+  case ROCK_FP8: return epilogue_pack4<ROCK_FP8>(v, e);
+  default: return epilogue_pack4<ROCK_BF8>(v, e);
+  }
+}
+
+// The whole epilogue for 4 channels.  OD (the output type) is a compile-time
+// constant so that the unrolled epilogue is straight-line code.  SLOW_CALL:
+// transcendental activations are applied here through an out-of-line call
+// (element-wise kernels); otherwise the caller has dealt with them.
+template <bool INT_ACC, int OD, bool SLOW_CALL = false, typename Acc4>
 __device__ __forceinline__ v4i epilogue_convert4(const Acc4 &acc, const RockEpilogue &e,
-                                                 const void *aux, int n0, int n_limit) {
-  if constexpr (INT_ACC && OD == ROCK_I32) { // exact accumulators, optional int32 bias
+                                                 const void *aux, int n0, int n_limit,
+                                                 const void *res = nullptr, int64_t res_off = 0,
+                                                 int64_t res_ns = 1) {
+  if constexpr (INT_ACC && OD == ROCK_I32) { // exact accumulators, optional int32 bias and residual
     v4i v;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       v[r] = (int)acc[r];
       if (e.has_bias && n0 + r < n_limit)
         v[r] += ((const int *)aux)[n0 + r];
+      if (res && n0 + r < n_limit) {
+        const int rv = ((const int *)res)[res_off + r * res_ns];
+        v[r] = e.residual_op == ROCK_RES_ADD ? v[r] + rv : v[r] * rv;
+      }
     }
     return v;
   } else {
     float v[4];
+    epilogue_affine4<INT_ACC, OD>(acc, e, aux, n0, n_limit, res, res_off, res_ns, v);
+    if (SLOW_CALL && activation_is_slow(e)) {
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      float f;
-      if constexpr (INT_ACC)
-        f = ((float)(int)acc[r] - (float)e.zero_point) * e.scale;
-      else
-        f = (float)acc[r] * e.scale;
-      if (e.has_bias && n0 + r < n_limit)
-        f = f + ((const float *)aux)[n0 + r];
-      if (e.relu)
-        f = fmaxf(f, 0.0f);
-      v[r] = f;
+      for (int r = 0; r < 4; ++r)
+        v[r] = activation_slow_call(v[r], e.activation);
+    } else if (e.activation) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        v[r] = activation_fast(v[r], e);
     }
-    v4i out = {0, 0, 0, 0};
-    if constexpr (OD == ROCK_F32) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        out[r] = __builtin_bit_cast(int, v[r]);
-    } else if constexpr (OD == ROCK_F16) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        _Float16 hv = (_Float16)v[r];
-        out[r >> 1] |= (int)__builtin_bit_cast(uint16_t, hv) << (16 * (r & 1));
-      }
-    } else if constexpr (OD == ROCK_BF16) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        __bf16 hv = (__bf16)v[r];
-        out[r >> 1] |= (int)__builtin_bit_cast(uint16_t, hv) << (16 * (r & 1));
-      }
-    } else if constexpr (OD == ROCK_I8) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float q = __builtin_rintf(v[r] * e.inv_quant_scale) + (float)e.out_zero_point;
-        out[0] |= ((int)f32_to_i8_sat(q) & 0xff) << (8 * r);
-      }
-    } else if constexpr (OD == ROCK_FP8) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        out[0] |= (int)f32_to_e4m3fn_sat(v[r]) << (8 * r);
-    } else if constexpr (OD == ROCK_BF8) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        out[0] |= (int)f32_to_e5m2_sat(v[r]) << (8 * r);
-    }
-    return out;
+    return epilogue_pack4<OD>(v, e);
   }
 }
 
@@ -461,9 +571,9 @@ __device__ __forceinline__ auto make_loader_b(const void *fil, const RockConvPar
 
 // Epilogue straight from the accumulator layout: the lane owns rows
 // m_lane + 32*i and channels n_lane + 32*j + 8*q + {0..3}.
-template <bool INT_ACC, int OD, int MI, int NI, typename Acc4, typename AccArr, typename Params>
+template <bool INT_ACC, int OD, int MI, int NI, typename Acc4, bool SLOW_CALL = true, typename AccArr, typename Params>
 __device__ __forceinline__ void direct_epilogue(const AccArr &acc, const Params &p, int g, void *Cptr,
-                                                const void *aux, int m_lane, int n_lane) {
+                                                const void *aux, const void *res, int m_lane, int n_lane) {
   constexpr int ES = OutElemSize<OD>::value;
 #pragma unroll
   for (int i = 0; i < MI; ++i) {
@@ -482,7 +592,8 @@ __device__ __forceinline__ void direct_epilogue(const AccArr &acc, const Params 
           continue;
         Acc4 a4 = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
                    acc[i][j][4 * q + 3]};
-        v4i raw = epilogue_convert4<INT_ACC, OD>(a4, p.epi, aux, n, p.N);
+        v4i raw = epilogue_convert4<INT_ACC, OD, SLOW_CALL>(a4, p.epi, aux, n, p.N, p.epi.residual_op ? res : nullptr,
+                                                 row_off + (int64_t)n * n_stride, n_stride);
         store_packed4(raw, ES, Cptr, row_off + (int64_t)n * n_stride, n_stride, n, p.N, vec_ok);
       }
     }
@@ -494,7 +605,7 @@ __device__ __forceinline__ void direct_epilogue(const AccArr &acc, const Params 
 // ---------------------------------------------------------------------------
 template <int DT, int BM, int BN, int WAVES_M, int WAVES_N, int LDA, int LDB, typename Params>
 __device__ __forceinline__ void contraction_body(const void *Aptr, const void *Bptr, void *Cptr,
-                                                 const void *aux, const Params &p) {
+                                                 const void *aux, const void *res, const Params &p) {
   using Tr = MmaTraits<DT>;
   using Acc = typename Tr::Acc;
   constexpr int NT = WAVES_M * WAVES_N * 64;
@@ -576,7 +687,7 @@ __device__ __forceinline__ void contraction_body(const void *Aptr, const void *B
   using Acc4 = decltype(__builtin_shufflevector(acc[0][0], acc[0][0], 0, 1, 2, 3));
   dispatch_out_dtype<Tr::INT_ACC>(e.out_dtype, [&](auto od_const) __attribute__((always_inline)) {
     constexpr int OD = decltype(od_const)::value;
-    direct_epilogue<Tr::INT_ACC, OD, MI, NI, Acc4>(acc, p, g, Cptr, aux, m0 + wm * WTM + lrow,
+    direct_epilogue<Tr::INT_ACC, OD, MI, NI, Acc4>(acc, p, g, Cptr, aux, res, m0 + wm * WTM + lrow,
                                                   n0 + wn * WTN + lgrp * 4);
   });
 }

@@ -19,9 +19,9 @@
 
 namespace rk {
 
-template <int DT>
+template <int DT, bool RICH = false>
 __device__ __forceinline__ void gemm_body_splitk(const void *Aptr, const void *Bptr, void *Cptr,
-                                                 const void *aux, const RockGemmParams &p) {
+                                                 const void *aux, const void *res, const RockGemmParams &p) {
   using Tr = MmaTraits<DT>;
   using Acc = typename Tr::Acc;
   constexpr int T = 32;      // output tile edge
@@ -111,7 +111,9 @@ __device__ __forceinline__ void gemm_body_splitk(const void *Aptr, const void *B
   Acc tile[1][1] = {{acc}};
   dispatch_out_dtype<Tr::INT_ACC>(p.epi.out_dtype, [&](auto od_const) __attribute__((always_inline)) {
     constexpr int OD = decltype(od_const)::value;
-    direct_epilogue<Tr::INT_ACC, OD, 1, 1, Acc4>(tile, p, g, Cptr, aux, m0 + lrow, n0 + lgrp * 4);
+    // RICH (kernel suffix "_e"): residual tensor and out-of-line transcendental activations
+    direct_epilogue<Tr::INT_ACC, OD, 1, 1, Acc4, RICH>(tile, p, g, Cptr, aux, RICH ? res : nullptr, m0 + lrow,
+                                                       n0 + lgrp * 4);
   });
 }
 

@@ -23,12 +23,32 @@ enum RockDType : int32_t {
 };
 
 // Epilogue applied to the accumulator tile before the store
-// (MIGraphXToTosa.cpp:874-982 formulas; GemmToGridwise.cpp:241-263 cast).
-//   float accumulators:  v = acc * scale (+ bias[n])            -> cast
-//   int32 accumulators:  out i32: acc (+ bias_i32[n])
-//                        out float: v = (float(acc) - float(zero_point)) * scale
-//                                   (+ bias[n])                 -> cast
-//   out i8 (either):     q = clamp(roundeven(v * inv_quant_scale) + out_zero_point)
+// (MIGraphXToTosa.cpp:874-982 formulas; GemmToGridwise.cpp:241-263 cast; the
+// element-wise operations MIGraphX fuses behind a contraction,
+// MIGraphXToTosa.cpp:1009-1016 relu, :1089-1100 clip, :1283-1295 add, mul,
+// erf, exp, sigmoid, tanh).  Steps, in this order:
+//   1. float accumulators:  v = acc * scale
+//      int32 accumulators:  v = (float(acc) - float(zero_point)) * scale
+//   2. v += bias[n]                       one value per output channel
+//   3. v = v + r  or  v * r               r = residual tensor, same type and
+//                                         layout as the output
+//   4. v = activation(v)
+//   5. out i8:  q = clamp(roundeven(v * inv_quant_scale) + out_zero_point)
+//      else:    round to the output type
+// int32 accumulators leaving as int32 skip 1, 4 and 5 and take 2 and 3 in
+// integer arithmetic.
+enum RockActivation : int32_t {
+  ROCK_ACT_NONE = 0,
+  ROCK_ACT_RELU = 1,    // max(v, 0)
+  ROCK_ACT_CLIP = 2,    // min(max(v, act_lo), act_hi)
+  ROCK_ACT_SIGMOID = 3, // 1 / (1 + exp(-v))
+  ROCK_ACT_TANH = 4,
+  ROCK_ACT_ERF = 5,
+  ROCK_ACT_GELU = 6,    // 0.5 v (1 + erf(v / sqrt 2)), the mul/erf/add chain of a traced GELU
+  ROCK_ACT_EXP = 7,
+};
+enum RockResidualOp : int32_t { ROCK_RES_NONE = 0, ROCK_RES_ADD = 1, ROCK_RES_MUL = 2 };
+
 struct RockEpilogue {
   float scale;          // 1.0f = identity
   float inv_quant_scale; // 1/scale of the requantisation step (out i8 only)
@@ -36,8 +56,9 @@ struct RockEpilogue {
   int32_t out_zero_point;
   int32_t has_bias;     // aux pointer holds one f32 (or i32 for i32 out) per output channel
   int32_t out_dtype;    // RockDType
-  int32_t relu;         // clamp at zero after scale/bias
-  int32_t pad_;
+  int32_t activation;   // RockActivation
+  int32_t residual_op;  // RockResidualOp; the residual pointer follows the bias pointer
+  float act_lo, act_hi; // clamp applied for relu [0, +inf) and clip [lo, hi]; (-inf, +inf) otherwise
 };
 
 struct RockGemmParams {

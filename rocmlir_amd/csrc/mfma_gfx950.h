@@ -132,6 +132,12 @@ __device__ __forceinline__ uint8_t f32_to_e5m2_sat(float v) {
   int packed = __builtin_amdgcn_cvt_pk_bf8_f32(v, v, 0, false);
   return (uint8_t)(packed & 0xff);
 }
+__device__ __forceinline__ float e4m3fn_to_f32(uint8_t v) {
+  return __builtin_amdgcn_cvt_f32_fp8((int)v, 0);
+}
+__device__ __forceinline__ float e5m2_to_f32(uint8_t v) {
+  return __builtin_amdgcn_cvt_f32_bf8((int)v, 0);
+}
 __device__ __forceinline__ int8_t f32_to_i8_sat(float v) {
   float r = __builtin_rintf(v); // ties to even
   r = fminf(fmaxf(r, -128.0f), 127.0f);

@@ -280,8 +280,41 @@ bool parse_epilogue(const OptMap &o, int in_a, int out_dtype, RockEpilogue &e) {
   e.out_zero_point = 0;
   e.has_bias = bool_or(o, "bias", false) ? 1 : 0;
   e.out_dtype = out_dtype;
-  e.relu = bool_or(o, "relu", false) ? 1 : 0;
-  e.pad_ = 0;
+  // element-wise tail: "-activation relu|clip|sigmoid|tanh|erf|gelu|exp"
+  // ("-relu true" is the older spelling), "-clip_min/-clip_max" for clip,
+  // "-residual add|mul" for a second tensor shaped like the output
+  e.activation = bool_or(o, "relu", false) ? ROCK_ACT_RELU : ROCK_ACT_NONE;
+  e.act_lo = 0.0f;
+  e.act_hi = 0.0f;
+  {
+    static const std::pair<const char *, int> kActs[] = {
+        {"none", ROCK_ACT_NONE}, {"relu", ROCK_ACT_RELU}, {"clip", ROCK_ACT_CLIP}, {"sigmoid", ROCK_ACT_SIGMOID},
+        {"tanh", ROCK_ACT_TANH}, {"erf", ROCK_ACT_ERF},   {"gelu", ROCK_ACT_GELU}, {"exp", ROCK_ACT_EXP}};
+    const std::string act = str_or(o, "activation", "");
+    bool known = act.empty();
+    for (const auto &a : kActs)
+      if (act == a.first) {
+        e.activation = a.second;
+        known = true;
+      }
+    if (!known)
+      return false;
+    e.act_lo = -INFINITY;
+    e.act_hi = INFINITY;
+    if (e.activation == ROCK_ACT_RELU)
+      e.act_lo = 0.0f;
+    if (e.activation == ROCK_ACT_CLIP) {
+      if (!get_float(o, "clip_min", e.act_lo) || !get_float(o, "clip_max", e.act_hi) || e.act_lo > e.act_hi)
+        return false;
+    }
+    const std::string res = str_or(o, "residual", "none");
+    if (res != "none" && res != "add" && res != "mul")
+      return false;
+    e.residual_op = res == "add" ? ROCK_RES_ADD : res == "mul" ? ROCK_RES_MUL : ROCK_RES_NONE;
+    // integers leaving as integers take no float step
+    if (out_dtype == ROCK_I32 && e.activation != ROCK_ACT_NONE)
+      return false;
+  }
   get_float(o, "scale", e.scale);
   float qs;
   if (get_float(o, "quant_scale", qs)) {
@@ -337,6 +370,29 @@ std::string forced_tile(const OptMap &o) {
   return "";
 }
 
+// The tiled kernels exist twice: with the plain epilogue unrolled over their
+// accumulators, and ("_e") with the rolled epilogue that a residual tensor or a
+// transcendental activation needs.  The element-wise kernels handle both in
+// one.
+const char *rich_suffix(const RockEpilogue &e, bool tiled_kernel) {
+  return tiled_kernel && (e.residual_op != ROCK_RES_NONE || e.activation > ROCK_ACT_CLIP) ? "_e" : "";
+}
+
+// The contraction kernels take five pointers: two operands, the output, the
+// per-channel bias and the residual tensor.  A caller passes the residual
+// only when the problem names one; otherwise the library fills that slot
+// with NULL.
+void set_contraction_pointers(Handle *h, const RockEpilogue &e) {
+  h->num_pointers = 5;
+  if (e.residual_op) {
+    h->caller_pointers = 0; // all five, in order
+    h->ptr_map.clear();
+  } else {
+    h->caller_pointers = 4;
+    h->ptr_map = {{0, 0}, {1, 0}, {2, 0}, {3, 0}, {-1, 0}};
+  }
+}
+
 // Chooses the kernel, tile and grid for a GEMM whose sizes and strides are
 // already in p.  Returns false when only the element-wise kernel fits.
 bool plan_gemm_kernel(Handle *h, RockGemmParams &p, int code, int es, const OptMap &o) {
@@ -380,9 +436,10 @@ bool plan_gemm_kernel(Handle *h, RockGemmParams &p, int code, int es, const OptM
                   h->block_size, h->grid_size);
   if (split_k > 1)
     h->block_size = 256;
-  h->kernel_name = std::string("rock_gemm_") + operand_name(code) + tile->suffix + (storage ? storage : "");
+  h->kernel_name = std::string("rock_gemm_") + operand_name(code) + tile->suffix + (storage ? storage : "") +
+                   rich_suffix(p.epi, tiled);
   h->blob_name = std::string("gemm_") + operand_name(code);
-  h->num_pointers = 4;
+  set_contraction_pointers(h, p.epi);
   h->perf_config = perf_string(*tile, es);
   if (split_k > 1) { // the reference's grammar has a splitK field (7th)
     char buf[96];
@@ -645,6 +702,7 @@ Handle *make_conv(const OptMap &o) {
            (256 * q.fil_ks + cc * y * x) * es < ((int64_t)1 << 31);
   };
   bool fast = conv_fast(p, c);
+  bool planned = false; // the layout-conversion plan fixes the pointer map itself
 
   auto set_problem_key = [&] {
     std::ostringstream key;
@@ -723,7 +781,10 @@ Handle *make_conv(const OptMap &o) {
       const int64_t off_f = 0, off_i = need_f ? fil_bytes : 0;
       h->kernel_count = n_relayout + 1;
       h->workspace_bytes = (size_t)((need_f ? fil_bytes : 0) + (need_i ? in_bytes : 0));
-      h->caller_pointers = 5; // filter, input, output, bias, workspace
+      // filter, input, output, bias, [residual,] workspace
+      const int ws = p.epi.residual_op ? 5 : 4;
+      h->caller_pointers = ws + 1;
+      planned = true;
       const int kid = (int)int_or(o, "kernel_id", 0);
       const bool is_f = need_f && kid == 0, is_i = need_i && kid == (need_f ? 1 : 0);
       if (is_f || is_i) {
@@ -816,7 +877,7 @@ Handle *make_conv(const OptMap &o) {
         h->block_size = 256;
         h->grid_size = (uint32_t)blocks;
         h->num_pointers = 2;
-        h->ptr_map = {{is_f ? 0 : 1, 0}, {4, is_f ? off_f : off_i}};
+        h->ptr_map = {{is_f ? 0 : 1, 0}, {ws, is_f ? off_f : off_i}};
         h->perf_config = "";
         h->problem_key = std::string("relayout ") + (is_f ? "filter " : "input ") + (is_f ? fl : il);
         return h;
@@ -826,7 +887,8 @@ Handle *make_conv(const OptMap &o) {
       c = cp;
       Kg = cp * y * x;
       fast = true;
-      h->ptr_map = {{need_f ? 4 : 0, need_f ? off_f : 0}, {need_i ? 4 : 1, need_i ? off_i : 0}, {2, 0}, {3, 0}};
+      h->ptr_map = {{need_f ? ws : 0, need_f ? off_f : 0}, {need_i ? ws : 1, need_i ? off_i : 0}, {2, 0}, {3, 0},
+                    {p.epi.residual_op ? 4 : -1, 0}};
     }
   }
   p.k_order_yxc = (p.in_cs == 1) ? 1 : 0;
@@ -835,9 +897,11 @@ Handle *make_conv(const OptMap &o) {
     tile = fast ? pick_tile(Mg, k, (int)g, true, "") : &kGenericTile;
   apply_tile_grid(*tile, Mg, k, (int)g, p.tiles_m, p.tiles_n, p.group_m, p.xcd_remap,
                   h->block_size, h->grid_size);
-  h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + tile->suffix;
+  h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + tile->suffix + rich_suffix(p.epi, fast);
   h->blob_name = std::string("gemm_") + dtype_name(ti);
-  h->num_pointers = 4;
+  h->num_pointers = 5;
+  if (!planned)
+    set_contraction_pointers(h, p.epi);
   h->perf_config = perf_string(*tile, es);
 
   // Window-resident kernel (conv_direct.h), chosen by "-perf_config
@@ -879,7 +943,7 @@ Handle *make_conv(const OptMap &o) {
       p.xcd_remap = total >= 2 * kNumXCD ? 1 : 0;
       h->block_size = 512;
       h->grid_size = (uint32_t)total;
-      h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + "_direct224";
+      h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + "_direct224" + rich_suffix(p.epi, true);
       char buf[96];
       std::snprintf(buf, sizeof buf, "v2:224,128,8,224,32,%d,1,1,1", 16 / es);
       h->perf_config = buf;
@@ -1012,8 +1076,9 @@ int launch_once(Handle *h, hipFunction_t fn, void *const *pointers, hipStream_t 
   char buf[8 * 8 + 512];
   size_t off = 0;
   for (int i = 0; i < h->num_pointers; ++i, off += 8) {
-    const void *ptr = h->ptr_map.empty() ? pointers[i]
-                                         : (const char *)pointers[h->ptr_map[i].source] + h->ptr_map[i].offset;
+    const void *ptr = h->ptr_map.empty()           ? pointers[i]
+                      : h->ptr_map[i].source < 0   ? nullptr
+                                                   : (const char *)pointers[h->ptr_map[i].source] + h->ptr_map[i].offset;
     std::memcpy(buf + off, &ptr, 8);
   }
   std::memcpy(buf + off, h->params.data(), h->params.size());
@@ -1049,7 +1114,7 @@ bool check_launch_args(Handle *h, void *const *pointers, int num_pointers) {
       set_error("launch: NULL tensor pointer");
       return false;
     }
-  return true;
+  return true; // (a residual, when the problem names one, is pointer 4 and covered by the loop)
 }
 
 // problem description -> resolved kernel; NULL with the error set on failure

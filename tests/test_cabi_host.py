@@ -136,7 +136,7 @@ def test_pointwise_nchw_convolution_is_a_k_major_gemm(rock):
           "--conv_stride_w 1 --padding_h 0 --padding_w 0")
     k = rock.RockKernel(pw)
     assert k.kernel_name.startswith("rock_gemm_f16_") and k.kernel_name.endswith("_fast_nn")
-    assert (k.kernel_count, k.workspace_bytes, k.num_pointers) == (1, 0, 4)
+    assert (k.kernel_count, k.workspace_bytes, k.num_pointers, k.caller_pointers) == (1, 0, 5, 4)
     assert "convfp16" in k.problem_key and " -y 1 -x 1 " in k.problem_key
     # anything the GEMM form cannot express converts instead
     for change in (("--conv_stride_h 1", "--conv_stride_h 2"), ("--padding_w 0", "--padding_w 1"),
@@ -196,8 +196,20 @@ def test_layout_conversion_plan_follows_the_multi_kernel_protocol(rock):
         assert lib.rockamdGetPointerMap(k._h, C.byref(ncall), C.byref(nk), src, off) == 0
         assert ncall.value == 5 and nk.value == k.num_pointers
         maps.append([(src[i], off[i]) for i in range(nk.value)])
+    # the contraction kernel's fifth pointer is the residual tensor: none here (-1 = pass NULL)
     assert maps == [[(0, 0), (4, 0)], [(1, 0), (4, fil_bytes)],
-                    [(4, 0), (4, fil_bytes), (2, 0), (3, 0)]]
+                    [(4, 0), (4, fil_bytes), (2, 0), (3, 0), (-1, 0)]]
+    # with a residual the caller's list grows to six and the workspace moves to its end
+    ks = [rock.RockKernel(nchw + " --residual add --kernel_id %d" % i) for i in range(3)]
+    maps = []
+    for k in ks:
+        ncall, nk = C.c_int(), C.c_int()
+        src, off = (C.c_int32 * 8)(), (C.c_int64 * 8)()
+        assert lib.rockamdGetPointerMap(k._h, C.byref(ncall), C.byref(nk), src, off) == 0
+        assert ncall.value == 6
+        maps.append([(src[i], off[i]) for i in range(nk.value)])
+    assert maps == [[(0, 0), (5, 0)], [(1, 0), (5, fil_bytes)],
+                    [(5, 0), (5, fil_bytes), (2, 0), (3, 0), (4, 0)]]
     with pytest.raises(rock.RockError, match="kernel_id out of range"):
         rock.RockKernel(nchw + " --kernel_id 3")
     # only the input needs converting when the filter is already channel-contiguous
@@ -210,6 +222,39 @@ def test_layout_conversion_plan_follows_the_multi_kernel_protocol(rock):
     assert (k.kernel_count, k.workspace_bytes, k.caller_pointers) == (1, 0, 4)
     # a conversion kernel has no epilogue scalars to set
     assert lib.rockamdSetScale(rock.RockKernel(nchw)._h, C.c_float(2.0)) != 0
+
+
+def test_elementwise_epilogue_options(rock):
+    """The element-wise tail MIGraphX fuses behind a contraction
+    (MIGraphXToTosa.cpp:1009-1016, 1089-1100, 1283-1295): activation names,
+    clip bounds, a residual tensor as a fifth pointer."""
+    base = "-operation gemm -arch gfx950 -t f16 -g 1 -m 256 -n 256 -k 256 -transB true"
+    k = rock.RockKernel(base)
+    assert (k.num_pointers, k.caller_pointers) == (5, 4)
+    # relu and clip are a clamp in the plain kernel; the transcendental ones and a
+    # residual take the kernel's rolled-epilogue twin ("_e")
+    for act in ("relu", "none", "clip -clip_min 0 -clip_max 6"):
+        assert rock.RockKernel(base + " -activation " + act).kernel_name == k.kernel_name
+    for act in ("sigmoid", "tanh", "erf", "gelu", "exp"):
+        assert rock.RockKernel(base + " -activation " + act).kernel_name == k.kernel_name + "_e"
+    assert rock.RockKernel(base + " -residual add").kernel_name == k.kernel_name + "_e"
+    assert rock.RockKernel(base + " -activation clip -clip_min 0 -clip_max 6").caller_pointers == 4
+    # the element-wise kernels handle every epilogue themselves
+    odd = base.replace("-k 256", "-k 255")
+    assert rock.RockKernel(odd + " -activation erf").kernel_name == rock.RockKernel(odd).kernel_name
+    assert rock.RockKernel(odd).kernel_name.endswith("_generic")
+    for bad in (" -activation swish", " -activation clip", " -activation clip -clip_min 2 -clip_max 1",
+                " -residual sub"):
+        with pytest.raises(rock.RockError):
+            rock.RockKernel(base + bad)
+    for op in ("add", "mul"):
+        assert rock.RockKernel(base + " -residual " + op).caller_pointers == 5
+    # integer results stay integer: no float activation, but an integer residual is fine
+    i8 = "-operation gemm -arch gfx950 -t i8 -g 1 -m 256 -n 256 -k 256 -transB true"
+    with pytest.raises(rock.RockError):
+        rock.RockKernel(i8 + " -activation tanh")
+    assert rock.RockKernel(i8 + " -residual add").caller_pointers == 5
+    assert rock.RockKernel(i8 + " -out_datatype f16 -scale 0.01 -activation tanh").caller_pointers == 4
 
 
 def test_perf_config_override_and_fallback(rock):
@@ -246,7 +291,7 @@ def test_param_block_and_setters(rock):
                         "-transB true -scale 0.5 -zero_point 3")
     import struct
     blob = k.params()
-    assert len(blob) == k.params_size == 9 * 8 + 8 * 4 + 8 * 4
+    assert len(blob) == k.params_size == 9 * 8 + 8 * 4 + 10 * 4   # strides, sizes/tiling, epilogue
     G, M, N, K = struct.unpack_from("4i", blob, 72)
     assert (G, M, N, K) == (1, 64, 64, 64)
     scale, inv_q, zp = struct.unpack_from("ffi", blob, 72 + 32)

@@ -301,3 +301,21 @@ def test_fill_rand_follows_libc_rand(oracle):
     assert oracle.fill_fixed(5, is_int=True).tolist() == [1, -1, 2, 1, -1]
     # min == max: constant (0.1x for floats), conv-validation-wrappers.cpp:41-45
     assert oracle.fill_rand(3, 1, 1, as_float=True).tolist() == [np.float32(0.1)] * 3
+
+
+def test_rand_fill_reproduces_the_reference_erf_vector():
+    """mixr-gemm-erf_f32.mlir runs `-rand 3` (srand(3), integers in [-5, 5),
+    arguments filled in order) through dot + erf and FileChecks the printed
+    result: reproducing it pins the fill's generator, range and order."""
+    import json
+    import math
+    import os
+    from oracle import rock_oracle as o
+    here = os.path.dirname(os.path.abspath(__file__))
+    case = next(c for c in json.load(open(os.path.join(here, "golden", "fusion_kats.json")))
+                if c["source"].endswith("erf_f32.mlir"))
+    o.seed(int(case["rand"]))
+    a = o.fill_rand(case["m"] * case["k"], -5, 5, False)
+    b = o.fill_rand(case["k"] * case["n"], -5, 5, False)
+    c = o.gemm(a, b, 1, case["m"], case["n"], case["k"])
+    assert [float("%.6g" % math.erf(v)) for v in np.asarray(c).ravel()] == case["expected"]
