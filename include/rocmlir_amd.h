@@ -65,7 +65,13 @@ typedef void *MiirHandle;
  * out_datatype, g, m, k, n, transA, transB, transC; g, seq_len_q, seq_len_k,
  * head_dim_qk, head_dim_v, transQ, transK, transV, transO, with-attn-bias.
  * Epilogue keys (all optional): scale, zero_point, quant_scale,
- * out_zero_point, bias, relu.  A single leading dash and "key=value" are
+ * out_zero_point, bias, relu; and the element-wise operations MIGraphX fuses
+ * behind a contraction (MIGraphXToTosa.cpp:1009-1016, 1089-1100, 1283-1295):
+ * activation {relu|clip|sigmoid|tanh|erf|gelu|exp} with clip_min / clip_max
+ * for clip, residual {add|mul} for a second tensor of the output's type and
+ * layout.  Order: scale and zero point, bias, residual, activation,
+ * narrowing.  Convolution-only switches: layout_conversion {true|false},
+ * pointwise_as_gemm {true|false}.  A single leading dash and "key=value" are
  * accepted as well.  Returns NULL on any parse, validation or support
  * failure, as the reference does. */
 ROCMLIR_AMD_API MiirHandle miirCreateHandle(const char *options);
@@ -111,9 +117,13 @@ ROCMLIR_AMD_API MiirStatus rockamdGetKernelName(MiirHandle handle, char *buffer,
 ROCMLIR_AMD_API MiirStatus rockamdGetKernelAttrs(MiirHandle handle, uint32_t attrs[2]);
 
 /* Kernel argument list: `num_pointers` bare device pointers in op order
- * (GEMM: A, B, C, aux; conv: filter, input, output, aux; attention: Q, K, V,
- * aux, O -- aux is the bias vector / pre-softmax bias tensor, NULL when
- * unused), followed by ONE by-value parameter block of `*params_size` bytes.
+ * (GEMM: A, B, C, aux, residual; conv: filter, input, output, aux, residual;
+ * attention: Q, K, V, aux, O -- aux is the bias vector / pre-softmax bias
+ * tensor, residual the tensor of "--residual"; NULL when unused), followed by
+ * ONE by-value parameter block of `*params_size` bytes.  What the CALLER
+ * passes to rockamdLaunch can be shorter: a problem without "--residual"
+ * passes four pointers and the library fills the fifth with NULL
+ * (rockamdGetPointerMap reports it as source -1).
  * Two-call protocol: params == NULL writes the size only.  The reference
  * bakes shapes into the kernel and passes pointers only (Pipelines.cpp:
  * 246-248); this block is the documented extension that replaces that. */
@@ -142,8 +152,12 @@ ROCMLIR_AMD_API size_t rockamdGetProblemKey(MiirHandle handle, char *buffer, siz
  * the SAME caller list: the problem's pointers followed by the workspace
  * pointer.  This call says how many pointers the caller list has, how many
  * the kernel itself takes, and for each of those which caller pointer it is
- * (source[i]) plus a byte offset; rockamdLaunch applies the map itself.  For
- * single-kernel problems the map is the identity. */
+ * (source[i]) plus a byte offset; rockamdLaunch applies the map itself.
+ * source[i] == -1 means NULL (the residual slot of a problem without one).
+ * With "--residual" the caller list is A, B, C, aux, residual[, workspace].
+ * A convolution with a 1x1 filter, unit stride, no padding, one group and no
+ * bias over NCHW tensors needs no conversion: it runs as ONE batched GEMM
+ * kernel (filter x image, the image stored K-major). */
 ROCMLIR_AMD_API MiirStatus rockamdGetPointerMap(MiirHandle handle, int *caller_pointers, int *kernel_pointers,
                                                 int32_t *source, int64_t *offset);
 
