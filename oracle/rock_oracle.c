@@ -492,6 +492,112 @@ ORC_EXPORT int orc_conv_fwd_i8(const int8_t *fil, const int8_t *in,
 }
 
 /* ------------------------------------------------------------------ */
+/* backward convolutions (same generator, rocmlir-gen.cpp:1715-1997)   */
+/* ------------------------------------------------------------------ */
+/* Backward data: loop nest = the five INPUT dimensions in input-layout order,
+ * then k, then y, x (rocmlir-gen.cpp:1817-1821);
+ *   out_tmp = in_idx + pad - fil_idx * dilation          (:1895-1897)
+ * contributes only when out_tmp % stride == 0 and out_tmp / stride lies in
+ * [0, out extent) (:1786-1804); in += filter * out (:1938-1945, :1965-1969). */
+ORC_EXPORT int orc_conv_bwd_data_f32(const float *fil, float *in, const float *out, const char *fil_layout,
+                                     const char *in_layout, const char *out_layout, const orc_conv_dims *d,
+                                     int threads) {
+  int64_t fs[5], is[5], os[5];
+  int64_t fsz[5] = {d->g, d->k, d->c, d->y, d->x};
+  int64_t isz[5] = {d->n, d->g, d->c, d->hi, d->wi};
+  int64_t osz[5] = {d->n, d->g, d->k, d->ho, d->wo};
+  if (layout_strides(fil_layout, "gkcyx", fsz, fs) || layout_strides(in_layout, "ngchw", isz, is) ||
+      layout_strides(out_layout, "ngkhw", osz, os))
+    return -1;
+  int ord[5];
+  int64_t ext[5];
+  for (int p = 0; p < 5; ++p) {
+    ord[p] = (int)(strchr("ngchw", in_layout[p]) - "ngchw");
+    ext[p] = isz[ord[p]];
+  }
+  int64_t total = ext[0] * ext[1] * ext[2] * ext[3] * ext[4];
+  int nt = orc_threads(threads);
+  (void)nt;
+  _Pragma("omp parallel for num_threads(nt) schedule(static)")
+  for (int64_t flat = 0; flat < total; ++flat) {
+    int64_t idx[5]; /* n g c h w */
+    int64_t rem = flat;
+    for (int p = 4; p >= 0; --p) {
+      idx[ord[p]] = rem % ext[p];
+      rem /= ext[p];
+    }
+    int64_t n = idx[0], g = idx[1], c = idx[2], hi = idx[3], wi = idx[4];
+    float acc = 0.0f;
+    for (int64_t k = 0; k < d->k; ++k)
+      for (int64_t y = 0; y < d->y; ++y)
+        for (int64_t x = 0; x < d->x; ++x) {
+          int64_t th = hi + d->pad_h - y * d->dil_h, tw = wi + d->pad_w - x * d->dil_w;
+          if (th < 0 || tw < 0 || th % d->stride_h != 0 || tw % d->stride_w != 0)
+            continue;
+          int64_t ho = th / d->stride_h, wo = tw / d->stride_w;
+          if (ho >= d->ho || wo >= d->wo)
+            continue;
+          float fv = fil[g * fs[0] + k * fs[1] + c * fs[2] + y * fs[3] + x * fs[4]];
+          float ov = out[n * os[0] + g * os[1] + k * os[2] + ho * os[3] + wo * os[4]];
+          float prod = fv * ov;
+          acc = acc + prod;
+        }
+    in[n * is[0] + g * is[1] + c * is[2] + hi * is[3] + wi * is[4]] = acc;
+  }
+  return 0;
+}
+
+/* Backward weight: loop nest = the five FILTER dimensions in filter-layout
+ * order, then n, then ho, wo (rocmlir-gen.cpp:1822-1826);
+ *   in_idx = out_idx * stride + fil_idx * dilation - pad  (:1905-1910)
+ * in bounds (:1786-1804); filter += out * in (:1930-1937, :1965-1969). */
+ORC_EXPORT int orc_conv_bwd_weight_f32(float *fil, const float *in, const float *out, const char *fil_layout,
+                                       const char *in_layout, const char *out_layout, const orc_conv_dims *d,
+                                       int threads) {
+  int64_t fs[5], is[5], os[5];
+  int64_t fsz[5] = {d->g, d->k, d->c, d->y, d->x};
+  int64_t isz[5] = {d->n, d->g, d->c, d->hi, d->wi};
+  int64_t osz[5] = {d->n, d->g, d->k, d->ho, d->wo};
+  if (layout_strides(fil_layout, "gkcyx", fsz, fs) || layout_strides(in_layout, "ngchw", isz, is) ||
+      layout_strides(out_layout, "ngkhw", osz, os))
+    return -1;
+  int ord[5];
+  int64_t ext[5];
+  for (int p = 0; p < 5; ++p) {
+    ord[p] = (int)(strchr("gkcyx", fil_layout[p]) - "gkcyx");
+    ext[p] = fsz[ord[p]];
+  }
+  int64_t total = ext[0] * ext[1] * ext[2] * ext[3] * ext[4];
+  int nt = orc_threads(threads);
+  (void)nt;
+  _Pragma("omp parallel for num_threads(nt) schedule(static)")
+  for (int64_t flat = 0; flat < total; ++flat) {
+    int64_t idx[5]; /* g k c y x */
+    int64_t rem = flat;
+    for (int p = 4; p >= 0; --p) {
+      idx[ord[p]] = rem % ext[p];
+      rem /= ext[p];
+    }
+    int64_t g = idx[0], k = idx[1], c = idx[2], y = idx[3], x = idx[4];
+    float acc = 0.0f;
+    for (int64_t n = 0; n < d->n; ++n)
+      for (int64_t ho = 0; ho < d->ho; ++ho)
+        for (int64_t wo = 0; wo < d->wo; ++wo) {
+          int64_t hi = ho * d->stride_h + y * d->dil_h - d->pad_h;
+          int64_t wi = wo * d->stride_w + x * d->dil_w - d->pad_w;
+          if (hi < 0 || hi >= d->hi || wi < 0 || wi >= d->wi)
+            continue;
+          float ov = out[n * os[0] + g * os[1] + k * os[2] + ho * os[3] + wo * os[4]];
+          float iv = in[n * is[0] + g * is[1] + c * is[2] + hi * is[3] + wi * is[4]];
+          float prod = ov * iv;
+          acc = acc + prod;
+        }
+    fil[g * fs[0] + k * fs[1] + c * fs[2] + y * fs[3] + x * fs[4]] = acc;
+  }
+  return 0;
+}
+
+/* ------------------------------------------------------------------ */
 /* attention (rocmlir-gen.cpp:2507-2638)                               */
 /* ------------------------------------------------------------------ */
 /* Storage shapes (rocmlir-gen.cpp:2149-2200):

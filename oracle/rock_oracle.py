@@ -82,6 +82,11 @@ def lib():
         L.orc_conv_fwd_f32.restype = C.c_int
         L.orc_conv_fwd_i8.argtypes = conv_args
         L.orc_conv_fwd_i8.restype = C.c_int
+        bwd_args = [vp, vp, vp, C.c_char_p, C.c_char_p, C.c_char_p,
+                    C.POINTER(ConvDims), C.c_int]
+        for nm in ("orc_conv_bwd_data_f32", "orc_conv_bwd_weight_f32"):
+            getattr(L, nm).argtypes = bwd_args
+            getattr(L, nm).restype = C.c_int
         L.orc_attention_f32.argtypes = [vp, vp, vp, vp, vp, f32, vp, i64, i64,
                                         i64, i64, i64, C.c_int, C.c_int,
                                         C.c_int, C.c_int, i64, i64, C.c_int]
@@ -188,6 +193,40 @@ def conv_fwd(fil, inp, fil_layout, in_layout, out_layout, n, g, c, k, hi, wi,
     if rc != 0:
         raise ValueError("bad layout string")
     return out, ho, wo
+
+
+def conv_bwd_data(fil, out, fil_layout, in_layout, out_layout, n, g, c, k, hi,
+                  wi, y, x, stride=(1, 1), pad=(0, 0), dil=(1, 1), threads=0):
+    """Gradient with respect to the input: (flat input-shaped array, ho, wo)."""
+    ho = conv_out_dim(hi, y, pad[0], pad[0], stride[0], dil[0])
+    wo = conv_out_dim(wi, x, pad[1], pad[1], stride[1], dil[1])
+    d = ConvDims(n, g, c, k, hi, wi, y, x, ho, wo, stride[0], stride[1],
+                 pad[0], pad[1], dil[0], dil[1])
+    fil, out = _c(fil, np.float32), _c(out, np.float32)
+    assert fil.size == g * k * c * y * x and out.size == n * g * k * ho * wo
+    inp = np.zeros(n * g * c * hi * wi, np.float32)
+    rc = lib().orc_conv_bwd_data_f32(_p(fil), _p(inp), _p(out), fil_layout.encode(), in_layout.encode(),
+                                     out_layout.encode(), C.byref(d), threads)
+    if rc != 0:
+        raise ValueError("bad layout string")
+    return inp, ho, wo
+
+
+def conv_bwd_weight(inp, out, fil_layout, in_layout, out_layout, n, g, c, k, hi,
+                    wi, y, x, stride=(1, 1), pad=(0, 0), dil=(1, 1), threads=0):
+    """Gradient with respect to the filter: (flat filter-shaped array, ho, wo)."""
+    ho = conv_out_dim(hi, y, pad[0], pad[0], stride[0], dil[0])
+    wo = conv_out_dim(wi, x, pad[1], pad[1], stride[1], dil[1])
+    d = ConvDims(n, g, c, k, hi, wi, y, x, ho, wo, stride[0], stride[1],
+                 pad[0], pad[1], dil[0], dil[1])
+    inp, out = _c(inp, np.float32), _c(out, np.float32)
+    assert inp.size == n * g * c * hi * wi and out.size == n * g * k * ho * wo
+    fil = np.zeros(g * k * c * y * x, np.float32)
+    rc = lib().orc_conv_bwd_weight_f32(_p(fil), _p(inp), _p(out), fil_layout.encode(), in_layout.encode(),
+                                       out_layout.encode(), C.byref(d), threads)
+    if rc != 0:
+        raise ValueError("bad layout string")
+    return fil, ho, wo
 
 
 # ---- attention ------------------------------------------------------------

@@ -517,6 +517,98 @@ Handle *make_gemm(const OptMap &o) {
   return h;
 }
 
+// Makes h a layout-conversion kernel: a 5-D tensor, dimensions listed in the
+// destination's order (the last one contiguous there, the destination dense),
+// read through src_stride and zero-filled beyond src_size.  Strides may be
+// negative (a flipped filter); the caller adds the matching base offset to the
+// source pointer.  Returns false with the error set when the tensor is too
+// large for the kernel's 32-bit indices.
+bool fill_relayout_handle(Handle *h, const int64_t size[5], const int64_t src_size[5],
+                          const int64_t src_stride[5], int es) {
+  RockRelayoutParams r;
+  std::memset(&r, 0, sizeof r);
+  struct Dim { int64_t size, src_size, ss, ds; };
+  std::vector<Dim> dims;
+  int64_t dst = 1;
+  for (int d = 4; d >= 0; --d) {
+    dims.insert(dims.begin(), Dim{size[d], src_size[d], src_stride[d], dst});
+    dst *= size[d];
+  }
+  // drop unit dimensions and fold neighbours that are laid out back to back
+  // on both sides (h and w of an NCHW image) into one, so that the tiled
+  // dimensions are as long as the layouts allow
+  for (size_t d = 0; d + 1 < dims.size();) // the channel dimension stays last
+    if (dims[d].size == 1)
+      dims.erase(dims.begin() + d);
+    else
+      ++d;
+  for (size_t d = 0; d + 1 < dims.size();) {
+    const Dim &o = dims[d], &i = dims[d + 1];
+    if (i.src_size == i.size && o.ss == i.size * i.ss && o.ds == i.size * i.ds &&
+        o.size * i.size <= INT32_MAX) {
+      dims[d] = Dim{o.size * i.size, o.src_size * i.size, i.ss, i.ds};
+      dims.erase(dims.begin() + d + 1);
+    } else {
+      ++d;
+    }
+  }
+  while (dims.size() < 5)
+    dims.insert(dims.begin(), Dim{1, 1, 0, 0});
+  for (int d = 0; d < 5; ++d) {
+    r.size[d] = (int32_t)dims[d].size;
+    r.src_size[d] = (int32_t)dims[d].src_size;
+    r.src_stride[d] = dims[d].ss;
+    r.dst_stride[d] = dims[d].ds;
+  }
+  r.dst_fast = 4;
+  r.src_fast = 4;
+  for (int d = 0; d < 5; ++d) // the source's contiguous dimension (ties: the longest)
+    if (r.src_stride[d] == 1 && (r.src_stride[r.src_fast] != 1 || r.size[d] > r.size[r.src_fast]))
+      r.src_fast = d;
+  int64_t blocks = 1;
+  if (r.src_fast == r.dst_fast) {
+    // the destination's channel runs are whole 16-byte chunks by construction of cp
+    r.mode = RELAYOUT_COPY;
+    const int64_t chunks = (int64_t)r.size[2] * r.size[3] * (r.size[4] * es / 16);
+    if (chunks > INT32_MAX) {
+      set_error("conv: tensor too large for the layout-conversion kernel");
+      return false;
+    }
+    blocks = (chunks + 255) / 256 * r.size[1] * r.size[0];
+  } else {
+    // short channel runs: narrow tiles, element-wise; otherwise 128-byte
+    // tile rows with 16-byte accesses
+    const bool vec = r.size[r.dst_fast] > 16 && r.src_stride[r.src_fast] == 1;
+    r.mode = vec ? RELAYOUT_TRANSPOSE_VEC : RELAYOUT_TRANSPOSE;
+    r.tile_d = vec ? 128 / es : r.size[r.dst_fast] <= 8 ? 8 : r.size[r.dst_fast] <= 16 ? 16 : 32;
+    const int tile_s = vec ? 128 / es : 1024 / r.tile_d;
+    for (int d = 0; d < 5; ++d) {
+      if (d == r.src_fast)
+        blocks *= (r.size[d] + tile_s - 1) / tile_s;
+      else if (d == r.dst_fast)
+        blocks *= (r.size[d] + r.tile_d - 1) / r.tile_d;
+      else
+        blocks *= r.size[d];
+    }
+  }
+  if (blocks > INT32_MAX) {
+    set_error("conv: tensor too large for the layout-conversion kernel");
+    return false;
+  }
+  h->op = OP_RELAYOUT;
+  h->epi = nullptr;
+  h->params.assign(sizeof r, 0);
+  std::memcpy(h->params.data(), &r, sizeof r);
+  h->kernel_name = std::string("rock_relayout_b") + std::to_string(es);
+  h->blob_name = "relayout";
+  h->block_size = 256;
+  h->grid_size = (uint32_t)blocks;
+  h->num_pointers = 2;
+  h->caller_pointers = 0;
+  h->perf_config = "";
+  return true;
+}
+
 // ---- convolution --------------------------------------------------------------
 // letter-by-letter layout translation (ConvGenerator.cpp:641-647) widened to
 // rocmlir-gen's lowercase spellings with optional g (rocmlir-gen.cpp:837-863)
@@ -789,96 +881,26 @@ Handle *make_conv(const OptMap &o) {
       const bool is_f = need_f && kid == 0, is_i = need_i && kid == (need_f ? 1 : 0);
       if (is_f || is_i) {
         // this handle is one of the conversion kernels
-        RockRelayoutParams r;
-        std::memset(&r, 0, sizeof r);
         const int64_t *sz = is_f ? fsz : isz;             // sizes in the letter order "gkcyx" / "ngchw"
         const int64_t *sz_src = is_f ? fsz_src : isz_src; // the source is shorter along c when padding
         // dimensions listed in destination (channel-contiguous) order
         const int order_f[5] = {0, 1, 3, 4, 2}, order_i[5] = {0, 3, 4, 1, 2}; // g k y x c ; n h w g c
         const int64_t src_f[5] = {p.fil_gs, p.fil_ks, p.fil_cs, p.fil_ys, p.fil_xs};
         const int64_t src_i[5] = {p.in_ns, p.in_gs, p.in_cs, p.in_hs, p.in_ws};
-        struct Dim { int64_t size, src_size, ss, ds; };
-        std::vector<Dim> dims;
-        int64_t dst = 1;
-        for (int d = 4; d >= 0; --d) {
-          const int letter = is_f ? order_f[d] : order_i[d];
-          dims.insert(dims.begin(), Dim{sz[letter], sz_src[letter], is_f ? src_f[letter] : src_i[letter], dst});
-          dst *= sz[letter];
-        }
-        // drop unit dimensions and fold neighbours that are laid out back to back
-        // on both sides (h and w of an NCHW image) into one, so that the tiled
-        // dimensions are as long as the layouts allow
-        for (size_t d = 0; d + 1 < dims.size();) // the channel dimension stays last
-          if (dims[d].size == 1)
-            dims.erase(dims.begin() + d);
-          else
-            ++d;
-        for (size_t d = 0; d + 1 < dims.size();) {
-          const Dim &o = dims[d], &i = dims[d + 1];
-          if (i.src_size == i.size && o.ss == i.size * i.ss && o.ds == i.size * i.ds &&
-              o.size * i.size <= INT32_MAX) {
-            dims[d] = Dim{o.size * i.size, o.src_size * i.size, i.ss, i.ds};
-            dims.erase(dims.begin() + d + 1);
-          } else {
-            ++d;
-          }
-        }
-        while (dims.size() < 5)
-          dims.insert(dims.begin(), Dim{1, 1, 0, 0});
+        int64_t rsize[5], rsrc_size[5], rstride[5];
         for (int d = 0; d < 5; ++d) {
-          r.size[d] = (int32_t)dims[d].size;
-          r.src_size[d] = (int32_t)dims[d].src_size;
-          r.src_stride[d] = dims[d].ss;
-          r.dst_stride[d] = dims[d].ds;
+          const int letter = is_f ? order_f[d] : order_i[d];
+          rsize[d] = sz[letter];
+          rsrc_size[d] = sz_src[letter];
+          rstride[d] = is_f ? src_f[letter] : src_i[letter];
         }
-        r.dst_fast = 4;
-        r.src_fast = 4;
-        for (int d = 0; d < 5; ++d) // the source's contiguous dimension (ties: the longest)
-          if (r.src_stride[d] == 1 && (r.src_stride[r.src_fast] != 1 || r.size[d] > r.size[r.src_fast]))
-            r.src_fast = d;
-        int64_t blocks = 1;
-        if (r.src_fast == r.dst_fast) {
-          // the destination's channel runs are whole 16-byte chunks by construction of cp
-          r.mode = RELAYOUT_COPY;
-          const int64_t chunks = (int64_t)r.size[2] * r.size[3] * (r.size[4] * es / 16);
-          if (chunks > INT32_MAX) {
-            set_error("conv: tensor too large for the layout-conversion kernel");
-            delete h;
-            return nullptr;
-          }
-          blocks = (chunks + 255) / 256 * r.size[1] * r.size[0];
-        } else {
-          // short channel runs: narrow tiles, element-wise; otherwise 128-byte
-          // tile rows with 16-byte accesses
-          const bool vec = r.size[r.dst_fast] > 16 && r.src_stride[r.src_fast] == 1;
-          r.mode = vec ? RELAYOUT_TRANSPOSE_VEC : RELAYOUT_TRANSPOSE;
-          r.tile_d = vec ? 128 / es : r.size[r.dst_fast] <= 8 ? 8 : r.size[r.dst_fast] <= 16 ? 16 : 32;
-          const int tile_s = vec ? 128 / es : 1024 / r.tile_d;
-          for (int d = 0; d < 5; ++d) {
-            if (d == r.src_fast)
-              blocks *= (r.size[d] + tile_s - 1) / tile_s;
-            else if (d == r.dst_fast)
-              blocks *= (r.size[d] + r.tile_d - 1) / r.tile_d;
-            else
-              blocks *= r.size[d];
-          }
-        }
-        if (blocks > INT32_MAX) {
-          set_error("conv: tensor too large for the layout-conversion kernel");
+        const int callers = h->caller_pointers;
+        if (!fill_relayout_handle(h, rsize, rsrc_size, rstride, es)) {
           delete h;
           return nullptr;
         }
-        h->op = OP_RELAYOUT;
-        h->epi = nullptr;
-        h->params.assign(sizeof r, 0);
-        std::memcpy(h->params.data(), &r, sizeof r);
-        h->kernel_name = std::string("rock_relayout_b") + std::to_string(es);
-        h->blob_name = "relayout";
-        h->block_size = 256;
-        h->grid_size = (uint32_t)blocks;
-        h->num_pointers = 2;
+        h->caller_pointers = callers;
         h->ptr_map = {{is_f ? 0 : 1, 0}, {ws, is_f ? off_f : off_i}};
-        h->perf_config = "";
         h->problem_key = std::string("relayout ") + (is_f ? "filter " : "input ") + (is_f ? fl : il);
         return h;
       }

@@ -1,7 +1,8 @@
-"""Extracts the forward-convolution known-answer vectors that the reference's
-own CPU tests hold (mlir/test/rocmlir-driver/cpu_conv2d/*_fwd.mlir: the RUN
-line's problem flags and the literal output vector FileCheck expects) into
-conv_fwd_kats.json.  Run in the build container, where /root/reference is
+"""Extracts the convolution known-answer vectors that the reference's own CPU
+tests hold (mlir/test/rocmlir-driver/cpu_conv2d/*.mlir: the RUN line's
+problem flags and the literal output vector FileCheck expects) into
+conv_fwd_kats.json (forward) and conv_bwd_kats.json (backward data and
+backward weight; flags carry the operation).  Run in the build container, where /root/reference is
 mounted; the JSON (data only) is what the tests read.
 
     python tests/golden/make_conv_kats.py
@@ -12,15 +13,17 @@ import re
 
 REF = "/root/reference/mlir/test/rocmlir-driver/cpu_conv2d"
 FILES = ["kyxc_nhwc_nhwk_fwd.mlir", "kcyx_nchw_nkhw_fwd.mlir"]
+BWD_FILES = ["kyxc_nhwc_nhwk_bwd_data.mlir", "kcyx_nchw_nkhw_bwd_data.mlir",
+             "kyxc_nhwc_nhwk_bwd_weight.mlir", "kcyx_nchw_nkhw_bwd_weight.mlir"]
 FLAGS = ["fil_layout", "in_layout", "out_layout", "batchsize", "in_channels",
          "out_channels", "in_h", "in_w", "fil_h", "fil_w", "dilation_h",
          "dilation_w", "padding_h", "padding_w", "conv_stride_h",
-         "conv_stride_w", "groupsize", "rand", "t"]
+         "conv_stride_w", "groupsize", "rand", "t", "operation"]
 
 
-def main():
+def extract(files, out_name):
     cases = []
-    for fname in FILES:
+    for fname in files:
         text = open(os.path.join(REF, fname)).read().splitlines()
         pending = None
         for line in text:
@@ -37,11 +40,15 @@ def main():
                 pending["expected"] = [float(v) for v in m.group(2).split(",")]
                 cases.append(pending)
                 pending = None
-    out = os.path.join(os.path.dirname(os.path.abspath(__file__)),
-                       "conv_fwd_kats.json")
+    out = os.path.join(os.path.dirname(os.path.abspath(__file__)), out_name)
     with open(out, "w") as f:
         json.dump(cases, f, separators=(",", ":"))
     print("wrote %d cases to %s" % (len(cases), out))
+
+
+def main():
+    extract(FILES, "conv_fwd_kats.json")
+    extract(BWD_FILES, "conv_bwd_kats.json")
 
 
 if __name__ == "__main__":

@@ -160,6 +160,65 @@ def test_conv_vs_torch_conv2d(oracle, case, layouts):
     assert np.array_equal(out8.astype(np.float64), want)
 
 
+def _bwd_golden_cases():
+    with open(os.path.join(HERE, "golden", "conv_bwd_kats.json")) as f:
+        return json.load(f)
+
+
+@pytest.mark.parametrize("case", _bwd_golden_cases(), ids=lambda c: c["source"])
+def test_conv_backward_reference_golden_vectors(oracle, case):
+    """mlir/test/rocmlir-driver/cpu_conv2d/*_bwd_data.mlir, *_bwd_weight.mlir:
+    all-ones data (-rand none), the literal gradient FileCheck expects."""
+    f = case["flags"]
+    n, c, k = int(f["batchsize"]), int(f["in_channels"]), int(f["out_channels"])
+    hi, wi, y, x = int(f["in_h"]), int(f["in_w"]), int(f["fil_h"]), int(f["fil_w"])
+    lay = {"kyxc": "gkyxc", "kcyx": "gkcyx", "nhwc": "nhwgc", "nchw": "ngchw",
+           "nhwk": "nhwgk", "nkhw": "ngkhw"}
+    geom = dict(stride=(int(f["conv_stride_h"]), int(f["conv_stride_w"])),
+                pad=(int(f["padding_h"]), int(f["padding_w"])),
+                dil=(int(f["dilation_h"]), int(f["dilation_w"])))
+    ho = oracle.conv_out_dim(hi, y, geom["pad"][0], geom["pad"][0], geom["stride"][0], geom["dil"][0])
+    wo = oracle.conv_out_dim(wi, x, geom["pad"][1], geom["pad"][1], geom["stride"][1], geom["dil"][1])
+    layouts = (lay[f["fil_layout"]], lay[f["in_layout"]], lay[f["out_layout"]])
+    dy = np.ones(n * k * ho * wo, np.float32)
+    if f["operation"] == "conv_bwd_data":
+        got, _, _ = oracle.conv_bwd_data(np.ones(k * c * y * x, np.float32), dy, *layouts,
+                                         n, 1, c, k, hi, wi, y, x, **geom)
+    else:
+        got, _, _ = oracle.conv_bwd_weight(np.ones(n * c * hi * wi, np.float32), dy, *layouts,
+                                           n, 1, c, k, hi, wi, y, x, **geom)
+    assert got.size == len(case["expected"])
+    assert np.array_equal(got.astype(np.float64), np.array(case["expected"]))
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+@pytest.mark.parametrize("layouts", LAYOUTS)
+def test_conv_backward_vs_torch_grad(oracle, case, layouts):
+    """torch.nn.grad.conv2d_input / conv2d_weight (library routines) on
+    integer-valued data in float64: every sum exact."""
+    n, g, c, k, hi, wi, y, x, stride, pad, dil = case
+    rng = np.random.default_rng(hash((case, layouts, "bwd")) % 2 ** 31)
+    ho = oracle.conv_out_dim(hi, y, pad[0], pad[0], stride[0], dil[0])
+    wo = oracle.conv_out_dim(wi, x, pad[1], pad[1], stride[1], dil[1])
+    fil = rng.integers(-3, 4, (g, k, c, y, x)).astype(np.float32)
+    inp = rng.integers(-3, 4, (n, g, c, hi, wi)).astype(np.float32)
+    dy = rng.integers(-3, 4, (n, g, k, ho, wo)).astype(np.float32)
+    fl, il, ol = layouts
+    t_in = torch.from_numpy(inp.reshape(n, g * c, hi, wi)).double()
+    t_fil = torch.from_numpy(fil.reshape(g * k, c, y, x)).double()
+    t_dy = torch.from_numpy(dy.reshape(n, g * k, ho, wo)).double()
+    dx, _, _ = oracle.conv_bwd_data(_to_layout(fil, "gkcyx", fl), _to_layout(dy, "ngkhw", ol), fl, il, ol,
+                                    n, g, c, k, hi, wi, y, x, stride, pad, dil)
+    ref = torch.nn.grad.conv2d_input(t_in.shape, t_fil, t_dy, stride=stride, padding=pad, dilation=dil,
+                                     groups=g).numpy()
+    assert np.array_equal(dx.astype(np.float64), _to_layout(ref.reshape(n, g, c, hi, wi), "ngchw", il))
+    dw, _, _ = oracle.conv_bwd_weight(_to_layout(inp, "ngchw", il), _to_layout(dy, "ngkhw", ol), fl, il, ol,
+                                      n, g, c, k, hi, wi, y, x, stride, pad, dil)
+    ref = torch.nn.grad.conv2d_weight(t_in, t_fil.shape, t_dy, stride=stride, padding=pad, dilation=dil,
+                                      groups=g).numpy()
+    assert np.array_equal(dw.astype(np.float64), _to_layout(ref.reshape(g, k, c, y, x), "gkcyx", fl))
+
+
 def test_conv_i8_widens_before_multiply(oracle):
     # deliberate deviation from rocmlir-gen.cpp:1955-1960 (i8 multiply wraps)
     out, _, _ = oracle.conv_fwd(np.array([-128], np.int8), np.array([-128], np.int8),
