@@ -314,8 +314,8 @@ class RockProgram:
         return self.kernels[-1]
 
     def _args(self, args):
-        if len(self.kernels) == 1 and self.main.caller_pointers == len(args):
-            return args
+        if self.kernels[0].caller_pointers == len(args):
+            return args   # no workspace pointer in this problem's caller list
         if self._workspace is None:
             import torch
             dev = next(a.device for a in args if a is not None and not isinstance(a, int))
@@ -534,4 +534,60 @@ def attention(q, k, v, *, scale=1.0, bias=None, transQ=False, transK=False,
     if out is None:
         out = torch.empty(shape, dtype=q.dtype, device=q.device)
     kern.launch(q, k, v, bias, out, stream=stream)
+    return out
+
+
+def _conv_options(operation, t, fil_layout, in_layout, out_layout, batchsize, groupsize, in_channels, out_channels,
+                  in_h, in_w, fil_h, fil_w, stride, padding, dilation):
+    return ("--operation %s --arch gfx950 --in_type %s --fil_type %s --out_type %s"
+            " --fil_layout %s --in_layout %s --out_layout %s --batchsize %d"
+            " --groupsize %d --in_channels %d --out_channels %d --in_h %d"
+            " --in_w %d --fil_h %d --fil_w %d --dilation_h %d --dilation_w %d"
+            " --conv_stride_h %d --conv_stride_w %d --padding_h %d --padding_w %d"
+            % (operation, t, t, t, fil_layout, in_layout, out_layout, batchsize, groupsize, in_channels,
+               out_channels, in_h, in_w, fil_h, fil_w, dilation[0], dilation[1], stride[0], stride[1],
+               padding[0], padding[1]))
+
+
+def conv2d_bwd_data(fil, dout, *, fil_layout, in_layout, out_layout, batchsize, in_channels, out_channels, in_h,
+                    in_w, fil_h, fil_w, groupsize=1, stride=(1, 1), padding=(0, 0), dilation=(1, 1), out=None,
+                    layout_conversion=True, stream=None, info=None):
+    """Gradient of conv2d with respect to its input (rocmlir-gen / Miir
+    operation conv_bwd_data): `dout` is the gradient of the output, laid out
+    as `out_layout` says; returns the flat input-shaped gradient."""
+    import torch
+    t = _dtype_name(dout.dtype)
+    opts = _conv_options("conv_bwd_data", t, fil_layout, in_layout, out_layout, batchsize, groupsize, in_channels,
+                         out_channels, in_h, in_w, fil_h, fil_w, stride, padding, dilation)
+    if not layout_conversion:
+        opts += " --layout_conversion false"
+    prog = _program(opts)
+    if info is not None:
+        info["kernels"] = [k.kernel_name for k in prog.kernels]
+        info["workspace_bytes"] = prog.workspace_bytes
+    if out is None:
+        out = torch.empty(batchsize * in_channels * in_h * in_w, dtype=dout.dtype, device=dout.device)
+    prog.launch(fil.contiguous(), out, dout.contiguous(), None, stream=stream)
+    return out
+
+
+def conv2d_bwd_weight(inp, dout, *, fil_layout, in_layout, out_layout, batchsize, in_channels, out_channels, in_h,
+                      in_w, fil_h, fil_w, groupsize=1, stride=(1, 1), padding=(0, 0), dilation=(1, 1), out=None,
+                      layout_conversion=True, stream=None, info=None):
+    """Gradient of conv2d with respect to its filter (operation
+    conv_bwd_weight); returns the flat filter-shaped gradient."""
+    import torch
+    t = _dtype_name(dout.dtype)
+    opts = _conv_options("conv_bwd_weight", t, fil_layout, in_layout, out_layout, batchsize, groupsize, in_channels,
+                         out_channels, in_h, in_w, fil_h, fil_w, stride, padding, dilation)
+    if not layout_conversion:
+        opts += " --layout_conversion false"
+    prog = _program(opts)
+    if info is not None:
+        info["kernels"] = [k.kernel_name for k in prog.kernels]
+        info["workspace_bytes"] = prog.workspace_bytes
+    if out is None:
+        out = torch.empty(out_channels * (in_channels // groupsize) * fil_h * fil_w, dtype=dout.dtype,
+                          device=dout.device)
+    prog.launch(out, inp.contiguous(), dout.contiguous(), None, stream=stream)
     return out

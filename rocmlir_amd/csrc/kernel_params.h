@@ -110,6 +110,24 @@ struct RockRelayoutParams {
   int32_t tile_d;             // RELAYOUT_TRANSPOSE: tile extent along dst_fast (8, 16 or 32)
 };
 
+// Utility kernels of the backward convolutions (the reference's zero-init and
+// converting-copy utility kernels, ConvGenerator.cpp:279-344, 434-480).
+// rock_fill_zero(dst, p): clears `bytes` bytes.
+struct RockFillParams {
+  int64_t bytes;
+};
+// rock_reduce_splits(partials, dst, p): partial sums of a K-split contraction,
+// `splits` dense f32 arrays of size[0]*size[1]*size[2]*size[3] elements each
+// `split_stride` elements apart, are added in split order and written in the
+// destination's type to dst[sum i_d * dst_stride[d]].
+struct RockReduceParams {
+  int64_t split_stride;
+  int64_t dst_stride[4];
+  int32_t size[4];
+  int32_t splits;
+  int32_t out_dtype; // RockDType: f32, f16 or bf16
+};
+
 struct RockAttentionParams {
   // element strides of the logical views Q[g,i,d], K[g,j,d], V[g,j,e], O[g,i,e]
   int64_t q_gs, q_is, q_ds;

@@ -1,5 +1,6 @@
-// Layout conversion kernels (1-, 2- and 4-byte elements): see
-// RockRelayoutParams in kernel_params.h.
+// Utility kernels: layout conversion (1-, 2- and 4-byte elements), zero fill
+// and the reduction of K-split partial sums: see RockRelayoutParams,
+// RockFillParams and RockReduceParams in kernel_params.h.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include "kernel_params.h"
@@ -205,4 +206,40 @@ extern "C" __global__ __launch_bounds__(256) void rock_relayout_b2(const void *s
 extern "C" __global__ __launch_bounds__(256) void rock_relayout_b4(const void *src, void *dst,
                                                                     RockRelayoutParams p) {
   relayout_body<uint32_t>((const uint32_t *)src, (uint32_t *)dst, p);
+}
+
+// 16 bytes per thread; the tail of a size that is not a multiple of 16 byte by byte
+extern "C" __global__ __launch_bounds__(256) void rock_fill_zero(void *dst, RockFillParams p) {
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 16;
+  if (i + 16 <= p.bytes) {
+    *(uint4 *)((char *)dst + i) = uint4{0, 0, 0, 0};
+  } else {
+    for (int64_t b = i; b < p.bytes; ++b)
+      ((char *)dst)[b] = 0;
+  }
+}
+
+// one output element per thread
+extern "C" __global__ __launch_bounds__(256) void rock_reduce_splits(const float *partials, void *dst,
+                                                                     RockReduceParams p) {
+  const int64_t total = (int64_t)p.size[0] * p.size[1] * p.size[2] * p.size[3];
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total)
+    return;
+  float acc = 0.0f;
+  for (int s = 0; s < p.splits; ++s)
+    acc = acc + partials[(int64_t)s * p.split_stride + i];
+  int64_t rem = i, off = 0;
+#pragma unroll
+  for (int d = 3; d >= 0; --d) {
+    off += (rem % p.size[d]) * p.dst_stride[d];
+    rem /= p.size[d];
+  }
+  if (p.out_dtype == ROCK_F32) {
+    ((float *)dst)[off] = acc;
+  } else if (p.out_dtype == ROCK_F16) {
+    ((_Float16 *)dst)[off] = (_Float16)acc;
+  } else {
+    ((__bf16 *)dst)[off] = (__bf16)acc;
+  }
 }

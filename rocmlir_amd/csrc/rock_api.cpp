@@ -682,6 +682,399 @@ std::string key_layout(const std::string &layout, bool filter) {
   return r;
 }
 
+// ---- backward convolutions ------------------------------------------------------
+// Both gradients are forward convolutions over re-labelled views of the
+// problem's tensors, so they run on the forward kernels; what the views cannot
+// express directly (channel-contiguous operands for the vector kernels,
+// flipped filters, a reduction split over blocks) goes through the utility
+// kernels and the multi-kernel protocol.  The reference lowers them through
+// its own gridwise GEMM with dedicated coordinate transforms
+// (ConvToGemm.cpp:530-1131) plus zero-init / converting-copy utility kernels
+// (ConvGenerator.cpp:279-344, 434-480).
+struct ConvProblem {
+  int ti; // element type of all three tensors
+  std::string fl, il, ol;
+  int64_t n, g, c, k, hi, wi, y, x, ho, wo, sh, sw, ph, pw, dh, dw;
+  int64_t fs[5], is[5], os[5]; // element strides in letter order gkcyx / ngchw / ngkhw
+};
+
+int64_t floor_div(int64_t a, int64_t b) { return a >= 0 ? a / b : -((-a + b - 1) / b); }
+
+bool conv_view_fast(const RockConvParams &q, int es) {
+  auto al = [&](int64_t elems) { return (elems * es) % 16 == 0; };
+  const int64_t cc = q.c;
+  return q.in_cs == 1 && al(cc) && al(q.in_ws) && al(q.in_hs) && al(q.in_ns) && al(q.in_gs) && q.fil_cs == 1 &&
+         q.fil_xs == cc && q.fil_ys == (int64_t)q.x * cc && al(q.fil_ks) && al(q.fil_gs) &&
+         ((int64_t)q.n * q.in_ns + (int64_t)q.hi * q.in_hs + (int64_t)q.wi * q.in_ws + cc) * es < ((int64_t)1 << 31) &&
+         (256 * q.fil_ks + cc * q.y * q.x) * es < ((int64_t)1 << 31);
+}
+
+// Kernel, tile and grid for a forward convolution given entirely by its
+// parameter block (sizes, strides, epilogue).  False when the sizes exceed the
+// kernels' 32-bit indices.
+bool select_view_conv_kernel(Handle *h, RockConvParams &p, int ti, const OptMap &o) {
+  const int es = dtype_size(ti);
+  const int64_t Mg = (int64_t)p.n * p.ho * p.wo, Kg = (int64_t)p.c * p.y * p.x;
+  if (Mg > INT32_MAX || Kg > INT32_MAX) {
+    set_error("conv: problem too large for 32-bit tile indices");
+    return false;
+  }
+  p.M = (int)Mg; p.N = p.k; p.K = (int)Kg;
+  const bool fast = conv_view_fast(p, es);
+  p.k_order_yxc = (p.in_cs == 1) ? 1 : 0;
+  p.rows_per_tile = 0;
+  const Tile *tile = fast ? pick_tile(Mg, p.k, p.g, true, forced_tile(o)) : nullptr;
+  if (!tile)
+    tile = fast ? pick_tile(Mg, p.k, p.g, true, "") : &kGenericTile;
+  apply_tile_grid(*tile, Mg, p.k, p.g, p.tiles_m, p.tiles_n, p.group_m, p.xcd_remap, h->block_size, h->grid_size);
+  h->op = OP_CONV;
+  h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + tile->suffix;
+  h->blob_name = std::string("gemm_") + dtype_name(ti);
+  h->num_pointers = 5;
+  h->perf_config = perf_string(*tile, es);
+  return true;
+}
+
+std::string conv_problem_key(const Handle *h, const OptMap &o, const ConvProblem &cp, int direction) {
+  std::ostringstream key;
+  const int ti = cp.ti;
+  const char *opname = ti == ROCK_F32 ? "conv" : ti == ROCK_F16 ? "convfp16" : ti == ROCK_BF16 ? "convbfp16"
+                     : ti == ROCK_I8 ? "convint8" : ti == ROCK_FP8 ? "convfp8_fp8" : "convbf8_bf8";
+  key << h->arch << '\t' << int_or(o, "num_cu", kNumCU) << '\t' << opname << " -F " << direction << " -f "
+      << key_layout(cp.fl, true) << " -I " << key_layout(cp.il, false) << " -O " << key_layout(cp.ol, false)
+      << " -n " << cp.n << " -c " << cp.c << " -H " << cp.hi << " -W " << cp.wi << " -k " << cp.k << " -y "
+      << cp.y << " -x " << cp.x << " -p " << cp.ph << " -q " << cp.pw << " -u " << cp.sh << " -v " << cp.sw
+      << " -l " << cp.dh << " -j " << cp.dw << " -g " << cp.g;
+  return key.str();
+}
+
+void default_epilogue(RockEpilogue &e, int out_dtype) {
+  std::memset(&e, 0, sizeof e);
+  e.scale = 1.0f;
+  e.inv_quant_scale = 1.0f;
+  e.out_dtype = out_dtype;
+  e.act_lo = -INFINITY;
+  e.act_hi = INFINITY;
+}
+
+Handle *conv_handle_from_view(const RockConvParams &q, int ti, const OptMap &o) {
+  auto *h = new Handle;
+  h->params.assign(sizeof(RockConvParams), 0);
+  auto &p = *reinterpret_cast<RockConvParams *>(h->params.data());
+  p = q;
+  h->epi = &p.epi;
+  if (!select_view_conv_kernel(h, p, ti, o)) {
+    delete h;
+    return nullptr;
+  }
+  return h;
+}
+
+Handle *utility_fill_handle(int64_t bytes) {
+  auto *h = new Handle;
+  RockFillParams f{bytes};
+  h->op = OP_RELAYOUT;
+  h->epi = nullptr;
+  h->params.assign(sizeof f, 0);
+  std::memcpy(h->params.data(), &f, sizeof f);
+  h->kernel_name = "rock_fill_zero";
+  h->blob_name = "relayout";
+  h->block_size = 256;
+  h->grid_size = (uint32_t)((bytes + 16 * 256 - 1) / (16 * 256));
+  h->num_pointers = 1;
+  h->perf_config = "";
+  return h;
+}
+
+int64_t align256(int64_t bytes) { return (bytes + 255) / 256 * 256; }
+
+// One spatial axis of the backward-data decomposition.  Input positions with
+// (i + pad) % stride == r receive only the filter taps y with
+// (r - y * dilation) % stride == 0: y = y_first + t * y_step, t < T, which
+// reach output position a + o_first - t * dd for i = stride * a + r - pad.
+struct BwdAxis {
+  int64_t T = 0, y_first = 0, y_step = 1, o_first = 0, dd = 1, a_min = 0, A = 0;
+};
+BwdAxis bwd_data_axis(int64_t r, int64_t stride, int64_t dil, int64_t Y, int64_t pad, int64_t in_len) {
+  BwdAxis a;
+  for (int64_t y = 0; y < Y; ++y) {
+    if (floor_div(r - y * dil, stride) * stride != r - y * dil)
+      continue;
+    if (a.T == 0)
+      a.y_first = y;
+    else if (a.T == 1)
+      a.y_step = y - a.y_first;
+    ++a.T;
+  }
+  if (a.T > 0)
+    a.o_first = floor_div(r - a.y_first * dil, stride);
+  a.dd = a.T > 1 ? a.y_step * dil / stride : 1;
+  a.a_min = floor_div(pad - r + stride - 1, stride);
+  const int64_t a_max = floor_div(in_len - 1 + pad - r, stride);
+  a.A = std::max<int64_t>(0, a_max - a.a_min + 1);
+  return a;
+}
+
+// Gradient with respect to the input.  Pointer order as the forward problem:
+// filter, input (written), output (the incoming gradient), unused, [workspace].
+// For every phase (rh, rw) of (input position + padding) modulo the stride, the
+// input positions of that phase are a stride-1 convolution of the output
+// gradient with the flipped sub-filter of the taps that reach them
+// (the reference makes one kernel per such phase too: kernel_id selects it,
+// ConvToGemm.cpp:735-1131).  Phases without taps are left at zero by a
+// zero-fill kernel that runs first.
+Handle *make_conv_bwd_data(const OptMap &o, const ConvProblem &cp) {
+  const int es = dtype_size(cp.ti);
+  const int kid = (int)int_or(o, "kernel_id", 0);
+  struct Phase {
+    BwdAxis h, w;
+    int64_t rh, rw;
+  };
+  std::vector<Phase> phases;
+  bool need_fill = false;
+  for (int64_t rh = 0; rh < cp.sh; ++rh)
+    for (int64_t rw = 0; rw < cp.sw; ++rw) {
+      Phase ph{bwd_data_axis(rh, cp.sh, cp.dh, cp.y, cp.ph, cp.hi), bwd_data_axis(rw, cp.sw, cp.dw, cp.x, cp.pw, cp.wi),
+               rh, rw};
+      if (ph.h.A == 0 || ph.w.A == 0)
+        continue; // no input position in this phase
+      if (ph.h.T == 0 || ph.w.T == 0) {
+        need_fill = true; // positions no tap reaches
+        continue;
+      }
+      phases.push_back(ph);
+    }
+  // the convolution of one phase over the caller's tensors as they lie
+  auto phase_view = [&](const Phase &ph, int64_t &fil_off, int64_t &out_off) {
+    RockConvParams q;
+    std::memset(&q, 0, sizeof q);
+    q.n = (int)cp.n; q.g = (int)cp.g; q.c = (int)cp.k; q.k = (int)cp.c;
+    q.hi = (int)cp.ho; q.wi = (int)cp.wo; q.y = (int)ph.h.T; q.x = (int)ph.w.T;
+    q.ho = (int)ph.h.A; q.wo = (int)ph.w.A;
+    q.stride_h = q.stride_w = 1;
+    q.dil_h = (int)ph.h.dd; q.dil_w = (int)ph.w.dd;
+    q.pad_h = (int)((ph.h.T - 1) * ph.h.dd - ph.h.o_first - ph.h.a_min);
+    q.pad_w = (int)((ph.w.T - 1) * ph.w.dd - ph.w.o_first - ph.w.a_min);
+    q.in_ns = cp.os[0]; q.in_gs = cp.os[1]; q.in_cs = cp.os[2]; q.in_hs = cp.os[3]; q.in_ws = cp.os[4];
+    q.fil_gs = cp.fs[0]; q.fil_ks = cp.fs[2]; q.fil_cs = cp.fs[1];
+    q.fil_ys = -ph.h.y_step * cp.fs[3]; q.fil_xs = -ph.w.y_step * cp.fs[4];
+    fil_off = (ph.h.y_first + (ph.h.T - 1) * ph.h.y_step) * cp.fs[3] +
+              (ph.w.y_first + (ph.w.T - 1) * ph.w.y_step) * cp.fs[4];
+    q.out_ns = cp.is[0]; q.out_gs = cp.is[1]; q.out_ks = cp.is[2];
+    q.out_hs = cp.sh * cp.is[3]; q.out_ws = cp.sw * cp.is[4];
+    out_off = (cp.sh * ph.h.a_min + ph.rh - cp.ph) * cp.is[3] + (cp.sw * ph.w.a_min + ph.rw - cp.pw) * cp.is[4];
+    default_epilogue(q.epi, cp.ti);
+    return q;
+  };
+  // the same with the sub-filter and the output gradient converted to the
+  // vector kernels' form (reduction channel k contiguous, whole 16-byte chunks)
+  const int64_t kp = (cp.k * es + 15) / 16 * 16 / es;
+  auto al = [&](int64_t elems) { return (elems * es) % 16 == 0; };
+  const bool dy_as_is = cp.os[2] == 1 && kp == cp.k && al(cp.os[4]) && al(cp.os[3]) && al(cp.os[0]) && al(cp.os[1]);
+  const int64_t dy_bytes = dy_as_is ? 0 : align256(cp.n * cp.ho * cp.wo * cp.g * kp * es);
+  auto phase_fast_view = [&](const Phase &ph, int64_t &out_off) {
+    int64_t unused;
+    RockConvParams q = phase_view(ph, unused, out_off);
+    q.c = (int)kp;
+    q.fil_cs = 1; q.fil_xs = kp; q.fil_ys = ph.w.T * kp; q.fil_ks = ph.h.T * ph.w.T * kp; q.fil_gs = cp.c * q.fil_ks;
+    if (!dy_as_is) {
+      q.in_cs = 1; q.in_gs = kp; q.in_ws = cp.g * kp; q.in_hs = cp.wo * q.in_ws; q.in_ns = cp.ho * q.in_hs;
+    }
+    return q;
+  };
+  bool fast = bool_or(o, "layout_conversion", true);
+  for (const Phase &ph : phases) {
+    int64_t unused;
+    fast = fast && conv_view_fast(phase_fast_view(ph, unused), es);
+  }
+  // kernel list
+  const int first_phase = (need_fill ? 1 : 0) + (fast && !dy_as_is ? 1 : 0);
+  const int per_phase = fast ? 2 : 1;
+  const int count = first_phase + per_phase * (int)phases.size();
+  int64_t workspace = 0;
+  std::vector<int64_t> fil_ws(phases.size(), 0);
+  if (fast) {
+    workspace = dy_bytes;
+    for (size_t i = 0; i < phases.size(); ++i) {
+      fil_ws[i] = workspace;
+      workspace += align256(cp.g * cp.c * phases[i].h.T * phases[i].w.T * kp * es);
+    }
+  }
+  if (count == 0 || kid < 0 || kid >= count) {
+    set_error(count == 0 ? "conv_bwd_data: empty problem" : "conv: kernel_id out of range");
+    return nullptr;
+  }
+  Handle *h = nullptr;
+  const int ws = 4; // filter, input, output, unused, workspace
+  int idx = kid;
+  if (need_fill && idx-- == 0) {
+    h = utility_fill_handle(cp.n * cp.g * cp.c * cp.hi * cp.wi * es);
+    h->ptr_map = {{1, 0}};
+    h->problem_key = "zero fill of the input gradient";
+  } else if (fast && !dy_as_is && idx-- == 0) {
+    h = new Handle;
+    const int64_t size[5] = {cp.n, cp.ho, cp.wo, cp.g, kp}, src_size[5] = {cp.n, cp.ho, cp.wo, cp.g, cp.k};
+    const int64_t stride[5] = {cp.os[0], cp.os[3], cp.os[4], cp.os[1], cp.os[2]};
+    if (!fill_relayout_handle(h, size, src_size, stride, es)) {
+      delete h;
+      return nullptr;
+    }
+    h->ptr_map = {{2, 0}, {ws, 0}};
+    h->problem_key = "relayout output gradient " + cp.ol;
+  } else {
+    const Phase &ph = phases[idx / per_phase];
+    const int64_t fil_dst = fil_ws[idx / per_phase];
+    int64_t fil_off, out_off;
+    const RockConvParams generic = phase_view(ph, fil_off, out_off);
+    if (fast && idx % 2 == 0) {
+      // flipped sub-filter -> [g][c][T_h][T_w][kp]
+      h = new Handle;
+      const int64_t size[5] = {cp.g, cp.c, ph.h.T, ph.w.T, kp}, src_size[5] = {cp.g, cp.c, ph.h.T, ph.w.T, cp.k};
+      const int64_t stride[5] = {generic.fil_gs, generic.fil_ks, generic.fil_ys, generic.fil_xs, generic.fil_cs};
+      if (!fill_relayout_handle(h, size, src_size, stride, es)) {
+        delete h;
+        return nullptr;
+      }
+      h->ptr_map = {{0, fil_off * es}, {ws, fil_dst}};
+      h->problem_key = "relayout filter phase " + std::to_string(ph.rh) + "," + std::to_string(ph.rw);
+    } else {
+      int64_t off2;
+      h = conv_handle_from_view(fast ? phase_fast_view(ph, off2) : generic, cp.ti, o);
+      if (!h)
+        return nullptr;
+      h->ptr_map = {fast ? Handle::PtrSrc{ws, fil_dst} : Handle::PtrSrc{0, fil_off * es},
+                    (fast && !dy_as_is) ? Handle::PtrSrc{ws, 0} : Handle::PtrSrc{2, 0},
+                    {1, out_off * es}, {-1, 0}, {-1, 0}};
+      h->problem_key = conv_problem_key(h, o, cp, 2);
+    }
+  }
+  h->kernel_count = count;
+  h->workspace_bytes = (size_t)workspace;
+  h->caller_pointers = workspace ? 5 : 4;
+  return h;
+}
+
+// Gradient with respect to the filter.  Pointer order as the forward problem:
+// filter (written), input, output (the incoming gradient), unused, [workspace].
+//   dW[k, c, y, x] = sum over n, ho, wo of  X[n, c, ho*s + y*d - p, ...] * dY[n, k, ho, wo]
+// is a forward convolution with the roles re-labelled: its batch is c, its
+// reduction channel n, its "filter" the output gradient (spatial size ho x wo),
+// its output spatial size y x x, its stride the dilation and its dilation the
+// stride.  For the vector kernels both operands are copied with n contiguous;
+// with one group the reduction over n is split into S chunks that run as the
+// groups of that convolution into f32 partial sums, added up in split order by
+// a reduction kernel (the reference's answer is atomic adds into a zero-filled
+// f32 workspace, ConvGenerator.cpp:434-480).
+Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
+  const int es = dtype_size(cp.ti);
+  const int kid = (int)int_or(o, "kernel_id", 0);
+  RockConvParams q;
+  std::memset(&q, 0, sizeof q);
+  q.n = (int)cp.c; q.g = (int)cp.g; q.c = (int)cp.n; q.k = (int)cp.k;
+  q.hi = (int)cp.hi; q.wi = (int)cp.wi; q.y = (int)cp.ho; q.x = (int)cp.wo; q.ho = (int)cp.y; q.wo = (int)cp.x;
+  q.stride_h = (int)cp.dh; q.stride_w = (int)cp.dw; q.dil_h = (int)cp.sh; q.dil_w = (int)cp.sw;
+  q.pad_h = (int)cp.ph; q.pad_w = (int)cp.pw;
+  q.in_ns = cp.is[2]; q.in_gs = cp.is[1]; q.in_cs = cp.is[0]; q.in_hs = cp.is[3]; q.in_ws = cp.is[4];
+  q.fil_gs = cp.os[1]; q.fil_ks = cp.os[2]; q.fil_cs = cp.os[0]; q.fil_ys = cp.os[3]; q.fil_xs = cp.os[4];
+  q.out_ns = cp.fs[2]; q.out_gs = cp.fs[0]; q.out_ks = cp.fs[1]; q.out_hs = cp.fs[3]; q.out_ws = cp.fs[4];
+  default_epilogue(q.epi, cp.ti);
+
+  // split of the reduction over n (one group only: the splits take the group index)
+  int64_t S = 1;
+  if (cp.g == 1) {
+    const int64_t base = (int64_t)ceil_div(cp.c * cp.y * cp.x, 128) * ceil_div(cp.k, 128);
+    while (S < 64 && cp.n % (2 * S) == 0 && cp.n / (2 * S) >= 8 && base * S < 2 * kNumCU)
+      S *= 2;
+  }
+  const int64_t G2 = cp.g == 1 ? S : cp.g, n_per = cp.n / S;
+  const int64_t np = (n_per * es + 15) / 16 * 16 / es;
+  RockConvParams f = q; // converted operands
+  f.g = (int)G2; f.c = (int)np;
+  f.in_cs = 1; f.in_gs = np; f.in_ws = G2 * np; f.in_hs = cp.wi * f.in_ws; f.in_ns = cp.hi * f.in_hs;
+  f.fil_cs = 1; f.fil_xs = np; f.fil_ys = cp.wo * np; f.fil_ks = cp.ho * f.fil_ys; f.fil_gs = cp.k * f.fil_ks;
+  const int64_t dw_elems = cp.c * cp.y * cp.x * cp.k;
+  if (S > 1) { // f32 partial sums [S][c][y][x][k]
+    f.out_ks = 1; f.out_ws = cp.k; f.out_hs = cp.x * cp.k; f.out_ns = cp.y * f.out_hs; f.out_gs = dw_elems;
+    f.epi.out_dtype = ROCK_F32;
+  }
+  const bool fast = bool_or(o, "layout_conversion", true) && conv_view_fast(f, es) &&
+                    (int64_t)np * cp.ho * cp.wo <= INT32_MAX;
+  if (!fast)
+    S = 1;
+  const int64_t x_bytes = align256(cp.c * cp.hi * cp.wi * G2 * np * es);
+  const int64_t dy_bytes = align256(G2 * cp.k * cp.ho * cp.wo * np * es);
+  const int64_t part_bytes = S > 1 ? align256(S * dw_elems * 4) : 0;
+  const int count = fast ? (S > 1 ? 4 : 3) : 1;
+  const int64_t workspace = fast ? x_bytes + dy_bytes + part_bytes : 0;
+  if (kid < 0 || kid >= count) {
+    set_error("conv: kernel_id out of range");
+    return nullptr;
+  }
+  const int ws = 4;
+  const int64_t group_is = cp.g == 1 ? n_per * cp.is[0] : cp.is[1], group_os = cp.g == 1 ? n_per * cp.os[0] : cp.os[1];
+  Handle *h = nullptr;
+  if (!fast) {
+    h = conv_handle_from_view(q, cp.ti, o);
+    if (!h)
+      return nullptr;
+    h->ptr_map = {{2, 0}, {1, 0}, {0, 0}, {-1, 0}, {-1, 0}};
+    h->problem_key = conv_problem_key(h, o, cp, 4);
+  } else if (kid == 0) { // input -> [c][hi][wi][G2][np]
+    h = new Handle;
+    const int64_t size[5] = {cp.c, cp.hi, cp.wi, G2, np}, src_size[5] = {cp.c, cp.hi, cp.wi, G2, n_per};
+    const int64_t stride[5] = {cp.is[2], cp.is[3], cp.is[4], group_is, cp.is[0]};
+    if (!fill_relayout_handle(h, size, src_size, stride, es)) {
+      delete h;
+      return nullptr;
+    }
+    h->ptr_map = {{1, 0}, {ws, 0}};
+    h->problem_key = "relayout input " + cp.il;
+  } else if (kid == 1) { // output gradient -> [G2][k][ho][wo][np]
+    h = new Handle;
+    const int64_t size[5] = {G2, cp.k, cp.ho, cp.wo, np}, src_size[5] = {G2, cp.k, cp.ho, cp.wo, n_per};
+    const int64_t stride[5] = {group_os, cp.os[2], cp.os[3], cp.os[4], cp.os[0]};
+    if (!fill_relayout_handle(h, size, src_size, stride, es)) {
+      delete h;
+      return nullptr;
+    }
+    h->ptr_map = {{2, 0}, {ws, x_bytes}};
+    h->problem_key = "relayout output gradient " + cp.ol;
+  } else if (kid == 2) {
+    h = conv_handle_from_view(f, cp.ti, o);
+    if (!h)
+      return nullptr;
+    h->ptr_map = {{ws, x_bytes}, {ws, 0}, S > 1 ? Handle::PtrSrc{ws, x_bytes + dy_bytes} : Handle::PtrSrc{0, 0},
+                  {-1, 0}, {-1, 0}};
+    h->problem_key = conv_problem_key(h, o, cp, 4);
+  } else {
+    h = new Handle;
+    RockReduceParams r;
+    std::memset(&r, 0, sizeof r);
+    r.split_stride = dw_elems;
+    r.size[0] = (int)cp.c; r.size[1] = (int)cp.y; r.size[2] = (int)cp.x; r.size[3] = (int)cp.k;
+    r.dst_stride[0] = cp.fs[2]; r.dst_stride[1] = cp.fs[3]; r.dst_stride[2] = cp.fs[4]; r.dst_stride[3] = cp.fs[1];
+    r.splits = (int)S;
+    r.out_dtype = cp.ti;
+    h->op = OP_RELAYOUT;
+    h->epi = nullptr;
+    h->params.assign(sizeof r, 0);
+    std::memcpy(h->params.data(), &r, sizeof r);
+    h->kernel_name = "rock_reduce_splits";
+    h->blob_name = "relayout";
+    h->block_size = 256;
+    h->grid_size = (uint32_t)((dw_elems + 255) / 256);
+    h->num_pointers = 2;
+    h->perf_config = "";
+    h->ptr_map = {{ws, x_bytes + dy_bytes}, {0, 0}};
+    h->problem_key = "reduction of the split partial sums";
+  }
+  h->kernel_count = count;
+  h->workspace_bytes = (size_t)workspace;
+  h->caller_pointers = workspace ? 5 : 4;
+  return h;
+}
+
+
 Handle *make_conv(const OptMap &o) {
   // required keys (ConvGenerator.cpp:492-512); rocmlir-gen's "-t" sets all
   // three types at once
@@ -747,8 +1140,24 @@ Handle *make_conv(const OptMap &o) {
   }
   std::string opn = str_or(o, "operation", "conv");
   if (opn != "conv" && opn != "conv2d") {
-    set_error("conv: only the forward direction is built (" + opn + " requested)");
-    return nullptr;
+    // the gradients (rocmlir-gen's conv_bwd_data / conv_bwd_weight, Miir's operation key)
+    if (ph_r != ph || pw_r != pw) {
+      set_error("conv: the backward kernels take symmetric padding only");
+      return nullptr;
+    }
+    if (ti != to || (ti != ROCK_F32 && ti != ROCK_F16 && ti != ROCK_BF16)) {
+      set_error("conv: the backward kernels take f32, f16 or bf16 for all three tensors");
+      return nullptr;
+    }
+    ConvProblem cp;
+    cp.ti = ti; cp.fl = fl; cp.il = il; cp.ol = ol;
+    cp.n = n; cp.g = g; cp.c = ct / g; cp.k = kt / g; cp.hi = hi; cp.wi = wi; cp.y = y; cp.x = x; cp.ho = ho; cp.wo = wo;
+    cp.sh = sh; cp.sw = sw; cp.ph = ph; cp.pw = pw; cp.dh = dh; cp.dw = dw;
+    const int64_t fsz[5] = {g, cp.k, cp.c, y, x}, isz[5] = {n, g, cp.c, hi, wi}, osz[5] = {n, g, cp.k, ho, wo};
+    layout_strides(fl, "gkcyx", fsz, cp.fs);
+    layout_strides(il, "ngchw", isz, cp.is);
+    layout_strides(ol, "ngkhw", osz, cp.os);
+    return opn.find("bwd_data") != std::string::npos ? make_conv_bwd_data(o, cp) : make_conv_bwd_weight(o, cp);
   }
   const int64_t c_problem = ct / g, k = kt / g; // channels per group as the problem states them
   int64_t c = c_problem;                        // ... and as the contraction kernel sees them (may be padded)

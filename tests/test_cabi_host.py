@@ -69,7 +69,8 @@ def test_null_handle_behaviour(rock):
     CONV_RESNET.replace("--padding_h 1", "--padding_h -1"),
     CONV_RESNET.replace("--in_layout NHWGC", "--in_layout NHWC3"),
     CONV_RESNET.replace("gfx950", "gfx906"),                   # no kernels for other chips
-    CONV_RESNET.replace("--operation conv", "--operation conv_bwd_data"),
+    CONV_RESNET.replace("--operation conv", "--operation conv_bwd_data").replace("fp16", "i8"),  # float gradients only
+    CONV_RESNET.replace("--operation conv", "--operation conv_bwd_weight") + " --kernel_id 4",
     CONV_RESNET.replace("--fil_type fp16", "--fil_type fp32"),
     "--operation gemm --arch gfx950 -t f32 -m 4 -n 4",         # k missing
     "--operation gemm --arch gfx950 -t f32 -m 4 -n 4 -k 0",
@@ -222,6 +223,38 @@ def test_layout_conversion_plan_follows_the_multi_kernel_protocol(rock):
     assert (k.kernel_count, k.workspace_bytes, k.caller_pointers) == (1, 0, 4)
     # a conversion kernel has no epilogue scalars to set
     assert lib.rockamdSetScale(rock.RockKernel(nchw)._h, C.c_float(2.0)) != 0
+
+
+def test_backward_convolution_plans(rock):
+    """conv_bwd_data / conv_bwd_weight behind the multi-kernel protocol
+    (rocmlir-lib.cpp:150-199): kernel lists, workspace, problem keys with the
+    reference's direction codes (RockTuningImpl.cpp:759-772)."""
+    bwd_data = CONV_RESNET.replace("--operation conv", "--operation conv_bwd_data")
+    ks = [rock.RockKernel(bwd_data + " --kernel_id %d" % i) for i in range(2)]
+    assert [k.kernel_name for k in ks] == ["rock_relayout_b2", "rock_conv_f16_128x128_fast"]
+    assert all(k.kernel_count == 2 and k.workspace_bytes == 128 * 128 * 9 * 2 and k.caller_pointers == 5 for k in ks)
+    assert "convfp16 -F 2 " in ks[1].problem_key
+    # stride 2: one sub-filter conversion and one convolution per phase of the input grid
+    s2 = bwd_data.replace("--conv_stride_h 1 --conv_stride_w 1", "--conv_stride_h 2 --conv_stride_w 2") \
+                 .replace("--out_h 28 --out_w 28", "--out_h 14 --out_w 14")
+    k = rock.RockKernel(s2)
+    assert k.kernel_count == 8
+    # 1x1 filter, stride 2: three phases get no tap and are cleared by the zero-fill kernel
+    s3 = s2.replace("--fil_h 3 --fil_w 3", "--fil_h 1 --fil_w 1").replace("--padding_h 1 --padding_w 1",
+                                                                          "--padding_h 0 --padding_w 0")
+    names = [rock.RockKernel(s3 + " --kernel_id %d" % i).kernel_name for i in range(rock.RockKernel(s3).kernel_count)]
+    assert names == ["rock_fill_zero", "rock_relayout_b2", "rock_conv_f16_256x128_fast"]
+    # tensors as they lie: one element-wise kernel per phase, no workspace pointer
+    k = rock.RockKernel(s2 + " --layout_conversion false")
+    assert (k.kernel_count, k.workspace_bytes, k.caller_pointers) == (4, 0, 4)
+    assert k.kernel_name == "rock_conv_f16_64x64_generic"
+    bwd_w = CONV_RESNET.replace("--operation conv", "--operation conv_bwd_weight")
+    names = [rock.RockKernel(bwd_w + " --kernel_id %d" % i).kernel_name for i in range(4)]
+    assert names[:2] == ["rock_relayout_b2", "rock_relayout_b2"] and names[3] == "rock_reduce_splits"
+    assert names[2].startswith("rock_conv_f16_") and names[2].endswith("_fast")
+    assert "convfp16 -F 4 " in rock.RockKernel(bwd_w + " --kernel_id 2").problem_key
+    k = rock.RockKernel(bwd_w + " --layout_conversion false")
+    assert (k.kernel_count, k.workspace_bytes, k.kernel_name) == (1, 0, "rock_conv_f16_64x64_generic")
 
 
 def test_elementwise_epilogue_options(rock):

@@ -1,0 +1,145 @@
+"""GPU parity: backward-data and backward-weight convolution through the C ABI
+(operations conv_bwd_data / conv_bwd_weight) vs the CPU oracle.
+
+First the reference's own literal vectors (cpu_conv2d/*_bwd_data.mlir,
+*_bwd_weight.mlir), then integer-valued data, where every partial sum is exact
+in f32 whatever the order, over strides, dilations, padding, groups, layouts
+and both routes (vector kernels behind the conversion kernels, element-wise
+kernel on the tensors as they lie); real-valued data to the reference's RMS
+gate."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import CODE, check_float, quantise, to_f32, to_gpu
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+NHWC = ("gkyxc", "nhwgc", "nhwgk")
+NCHW = ("gkcyx", "ngchw", "ngkhw")
+
+
+def _to_layout(t, canonical, layout):
+    return np.ascontiguousarray(t.transpose([canonical.index(ch) for ch in layout])).ravel()
+
+
+def _golden():
+    with open(os.path.join(HERE, "golden", "conv_bwd_kats.json")) as f:
+        return json.load(f)
+
+
+@pytest.mark.parametrize("case", _golden(), ids=lambda c: c["source"])
+@pytest.mark.parametrize("t", ["f32", "f16"])
+def test_conv_backward_reference_golden_vectors(rock, oracle, gpu, case, t):
+    f = case["flags"]
+    n, c, k = int(f["batchsize"]), int(f["in_channels"]), int(f["out_channels"])
+    hi, wi, y, x = int(f["in_h"]), int(f["in_w"]), int(f["fil_h"]), int(f["fil_w"])
+    stride = (int(f["conv_stride_h"]), int(f["conv_stride_w"]))
+    pad = (int(f["padding_h"]), int(f["padding_w"]))
+    dil = (int(f["dilation_h"]), int(f["dilation_w"]))
+    ho = oracle.conv_out_dim(hi, y, pad[0], pad[0], stride[0], dil[0])
+    wo = oracle.conv_out_dim(wi, x, pad[1], pad[1], stride[1], dil[1])
+    dt = {"f32": torch.float32, "f16": torch.float16}[t]
+    kw = dict(fil_layout=f["fil_layout"], in_layout=f["in_layout"], out_layout=f["out_layout"], batchsize=n,
+              in_channels=c, out_channels=k, in_h=hi, in_w=wi, fil_h=y, fil_w=x, stride=stride, padding=pad,
+              dilation=dil)
+    dy = torch.ones(n * k * ho * wo, dtype=dt, device=gpu)
+    if f["operation"] == "conv_bwd_data":
+        got = rock.conv2d_bwd_data(torch.ones(k * c * y * x, dtype=dt, device=gpu), dy, **kw)
+    else:
+        got = rock.conv2d_bwd_weight(torch.ones(n * c * hi * wi, dtype=dt, device=gpu), dy, **kw)
+    assert got.cpu().double().tolist() == case["expected"]
+
+
+# (n g c k hi wi y x stride pad dil)
+CASES = [
+    (2, 1, 16, 24, 9, 9, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (3, 1, 8, 16, 12, 10, 3, 3, (2, 2), (1, 1), (1, 1)),      # ResNet down-sampling 3x3
+    (2, 1, 16, 8, 8, 8, 1, 1, (2, 2), (0, 0), (1, 1)),        # 1x1 stride 2: three of four phases stay zero
+    (1, 1, 3, 8, 21, 21, 7, 7, (2, 2), (3, 3), (1, 1)),       # first layer, odd channel count
+    (2, 2, 8, 8, 11, 13, 5, 5, (2, 3), (2, 2), (1, 2)),       # groups, mixed stride / dilation
+    (2, 1, 8, 8, 10, 10, 3, 3, (2, 2), (2, 2), (2, 2)),       # stride and dilation share a factor
+    (1, 1, 5, 7, 9, 9, 3, 3, (3, 3), (0, 0), (1, 1)),         # stride = filter size
+    (8, 1, 16, 16, 6, 6, 3, 3, (1, 1), (1, 1), (1, 1)),       # batch large enough to split the weight reduction
+    (4, 1, 16, 16, 5, 5, 2, 2, (1, 1), (0, 0), (2, 2)),
+]
+LAYOUTS = [NHWC, NCHW, ("gyxck", "hwcgn", "hwkgn")]
+
+
+def _tensors(case, layouts, t, seed, integer=True):
+    n, g, c, k, hi, wi, y, x, stride, pad, dil = case
+    fl, il, ol = layouts
+    ho = (hi + 2 * pad[0] - (y - 1) * dil[0] - 1) // stride[0] + 1
+    wo = (wi + 2 * pad[1] - (x - 1) * dil[1] - 1) // stride[1] + 1
+    rng = np.random.default_rng(seed)
+    if integer:
+        fil = rng.integers(-2, 3, (g, k, c, y, x)).astype(np.float32)
+        inp = rng.integers(-2, 3, (n, g, c, hi, wi)).astype(np.float32)
+        dy = rng.integers(-2, 3, (n, g, k, ho, wo)).astype(np.float32)
+    else:
+        fil = (rng.standard_normal((g, k, c, y, x)) * 0.1).astype(np.float32)
+        inp = (rng.standard_normal((n, g, c, hi, wi)) * 0.1).astype(np.float32)
+        dy = (rng.standard_normal((n, g, k, ho, wo)) * 0.1).astype(np.float32)
+    return (quantise(_to_layout(fil, "gkcyx", fl), t), quantise(_to_layout(inp, "ngchw", il), t),
+            quantise(_to_layout(dy, "ngkhw", ol), t), ho, wo)
+
+
+def _kw(case, layouts):
+    n, g, c, k, hi, wi, y, x, stride, pad, dil = case
+    return dict(fil_layout=layouts[0], in_layout=layouts[1], out_layout=layouts[2], batchsize=n, groupsize=g,
+                in_channels=g * c, out_channels=g * k, in_h=hi, in_w=wi, fil_h=y, fil_w=x, stride=stride,
+                padding=pad, dilation=dil)
+
+
+@pytest.mark.parametrize("convert", [True, False], ids=["converted", "as-is"])
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("layouts", LAYOUTS, ids=lambda l: l[1])
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16"])
+def test_conv_bwd_data_exact(rock, oracle, gpu, case, layouts, t, convert):
+    n, g, c, k, hi, wi, y, x, stride, pad, dil = case
+    (raw_f, fq), _, (raw_dy, dyq), ho, wo = _tensors(case, layouts, t, 71)
+    info = {}
+    got = rock.conv2d_bwd_data(to_gpu(raw_f, t, gpu), to_gpu(raw_dy, t, gpu), layout_conversion=convert, info=info,
+                               **_kw(case, layouts))
+    torch.cuda.synchronize()
+    ref, _, _ = oracle.conv_bwd_data(fq, dyq, *layouts, n, g, c, k, hi, wi, y, x, stride, pad, dil)
+    assert np.array_equal(to_f32(got, t), oracle.round_through(ref, CODE[t]))
+    if not convert:
+        assert not any(name.startswith("rock_relayout") for name in info["kernels"])
+
+
+@pytest.mark.parametrize("convert", [True, False], ids=["converted", "as-is"])
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("layouts", LAYOUTS, ids=lambda l: l[1])
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16"])
+def test_conv_bwd_weight_exact(rock, oracle, gpu, case, layouts, t, convert):
+    n, g, c, k, hi, wi, y, x, stride, pad, dil = case
+    _, (raw_i, iq), (raw_dy, dyq), ho, wo = _tensors(case, layouts, t, 73)
+    info = {}
+    got = rock.conv2d_bwd_weight(to_gpu(raw_i, t, gpu), to_gpu(raw_dy, t, gpu), layout_conversion=convert,
+                                 info=info, **_kw(case, layouts))
+    torch.cuda.synchronize()
+    ref, _, _ = oracle.conv_bwd_weight(iq, dyq, *layouts, n, g, c, k, hi, wi, y, x, stride, pad, dil)
+    assert np.array_equal(to_f32(got, t), oracle.round_through(ref, CODE[t]))
+    assert (len(info["kernels"]) == 1) == (not convert) or "generic" in info["kernels"][-1]
+
+
+@pytest.mark.parametrize("t", ["f16", "f32"])
+def test_conv_backward_resnet_block_real_values(rock, oracle, gpu, t):
+    """ResNet50 3x3 128->128 @28x28 (conv-configs:5), batch 16: both gradients
+    on the vector kernels (split weight reduction included), the reference's RMS gate."""
+    case = (16, 1, 128, 128, 28, 28, 3, 3, (1, 1), (1, 1), (1, 1))
+    n, g, c, k, hi, wi, y, x, stride, pad, dil = case
+    (raw_f, fq), (raw_i, iq), (raw_dy, dyq), ho, wo = _tensors(case, NHWC, t, 75, integer=False)
+    info = {}
+    dx = rock.conv2d_bwd_data(to_gpu(raw_f, t, gpu), to_gpu(raw_dy, t, gpu), info=info, **_kw(case, NHWC))
+    assert info["kernels"][-1].endswith("_fast")
+    ref, _, _ = oracle.conv_bwd_data(fq, dyq, *NHWC, n, g, c, k, hi, wi, y, x, stride, pad, dil)
+    check_float(to_f32(dx, t), ref, t)
+    dw = rock.conv2d_bwd_weight(to_gpu(raw_i, t, gpu), to_gpu(raw_dy, t, gpu), info=info, **_kw(case, NHWC))
+    assert info["kernels"][-1] == "rock_reduce_splits" and info["kernels"][-2].endswith("_fast")
+    ref, _, _ = oracle.conv_bwd_weight(iq, dyq, *NHWC, n, g, c, k, hi, wi, y, x, stride, pad, dil)
+    check_float(to_f32(dw, t), ref, t)
