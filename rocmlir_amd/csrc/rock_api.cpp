@@ -979,6 +979,107 @@ Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
   q.out_ns = cp.fs[2]; q.out_gs = cp.fs[0]; q.out_ks = cp.fs[1]; q.out_hs = cp.fs[3]; q.out_ws = cp.fs[4];
   default_epilogue(q.epi, cp.ti);
 
+  // 1x1 filter, unit stride, no padding, one group, pixels equally spaced in
+  // both tensors: dW[k, c] = sum over pixels of dY[pixel, k] * X[pixel, c] is a
+  // plain GEMM over the tensors as they lie -- both operands K-major when the
+  // channels are contiguous (NHWC), both K-contiguous when the pixels are
+  // (NCHW, one GEMM per image).  The pixel range is cut into S batch entries
+  // whose f32 partial results the reduction kernel adds up.
+  {
+    const bool lin_x = cp.is[3] == cp.wi * cp.is[4], lin_y = cp.os[3] == cp.wo * cp.os[4];
+    const bool all_x = lin_x && cp.is[0] == cp.hi * cp.is[3], all_y = lin_y && cp.os[0] == cp.ho * cp.os[3];
+    if (cp.y == 1 && cp.x == 1 && cp.sh == 1 && cp.sw == 1 && cp.ph == 0 && cp.pw == 0 && cp.g == 1 && lin_x && lin_y &&
+        bool_or(o, "pointwise_as_gemm", true)) {
+      const int64_t P = cp.hi * cp.wi;
+      const bool whole = all_x && all_y; // pixels of all images form one equally spaced run
+      const int64_t Ktot = whole ? cp.n * P : P;
+      // enough batch entries to fill the chip, each a divisor's share of the pixels
+      int64_t S = 1;
+      if (whole) {
+        const int64_t tiles = (int64_t)ceil_div(cp.k, 128) * ceil_div(cp.c, 128);
+        const int64_t want = std::max<int64_t>(1, std::min<int64_t>(2 * kNumCU / tiles, Ktot / 256));
+        for (int64_t d = want; d >= 1; --d)
+          if (Ktot % d == 0) {
+            S = d;
+            break;
+          }
+      } else {
+        S = cp.n;
+      }
+      const int64_t Ks = whole ? Ktot / S : P;
+      RockGemmParams gp;
+      std::memset(&gp, 0, sizeof gp);
+      gp.G = (int)S; gp.M = (int)cp.k; gp.N = (int)cp.c; gp.K = (int)Ks;
+      gp.a_ms = cp.os[2]; gp.a_ks = cp.os[4]; gp.a_gs = whole ? Ks * cp.os[4] : cp.os[0];
+      gp.b_ns = cp.is[2]; gp.b_ks = cp.is[4]; gp.b_gs = whole ? Ks * cp.is[4] : cp.is[0];
+      const int64_t dw = cp.k * cp.c;
+      if (S > 1) {
+        gp.c_ms = cp.c; gp.c_ns = 1; gp.c_gs = dw;
+        default_epilogue(gp.epi, ROCK_F32);
+      } else {
+        gp.c_ms = cp.fs[1]; gp.c_ns = cp.fs[2]; gp.c_gs = 0;
+        default_epilogue(gp.epi, cp.ti);
+      }
+      const int count = S > 1 ? 2 : 1;
+      const int64_t workspace = S > 1 ? align256(S * dw * 4) : 0;
+      auto *h = new Handle;
+      bool ok = false;
+      if (kid == 0) {
+        ok = Ks <= INT32_MAX && plan_gemm_kernel(h, gp, operand_code(cp.ti, cp.ti), es, o);
+        if (ok) {
+          h->op = OP_GEMM;
+          h->params.assign(sizeof gp, 0);
+          std::memcpy(h->params.data(), &gp, sizeof gp);
+          h->epi = &reinterpret_cast<RockGemmParams *>(h->params.data())->epi;
+          h->ptr_map = {{2, 0}, {1, 0}, S > 1 ? Handle::PtrSrc{4, 0} : Handle::PtrSrc{0, 0}, {-1, 0}, {-1, 0}};
+          h->problem_key = conv_problem_key(h, o, cp, 4);
+        }
+      } else if (kid == 1 && S > 1) {
+        // only reached when kernel 0 took this route as well (same decision below)
+        RockGemmParams probe = gp;
+        Handle tmp;
+        ok = Ks <= INT32_MAX && plan_gemm_kernel(&tmp, probe, operand_code(cp.ti, cp.ti), es, o);
+        if (ok) {
+          RockReduceParams r;
+          std::memset(&r, 0, sizeof r);
+          r.split_stride = dw;
+          r.size[0] = 1; r.size[1] = 1; r.size[2] = (int)cp.k; r.size[3] = (int)cp.c;
+          r.dst_stride[2] = cp.fs[1]; r.dst_stride[3] = cp.fs[2];
+          r.splits = (int)S;
+          r.out_dtype = cp.ti;
+          h->op = OP_RELAYOUT;
+          h->epi = nullptr;
+          h->params.assign(sizeof r, 0);
+          std::memcpy(h->params.data(), &r, sizeof r);
+          h->kernel_name = "rock_reduce_splits";
+          h->blob_name = "relayout";
+          h->block_size = 256;
+          h->grid_size = (uint32_t)((dw + 255) / 256);
+          h->num_pointers = 2;
+          h->perf_config = "";
+          h->ptr_map = {{4, 0}, {0, 0}};
+          h->problem_key = "reduction of the split partial sums";
+        }
+      } else {
+        // does the route apply at all?  (a kernel_id beyond its list is an error, not a fallback)
+        RockGemmParams probe = gp;
+        Handle tmp;
+        if (Ks <= INT32_MAX && plan_gemm_kernel(&tmp, probe, operand_code(cp.ti, cp.ti), es, o)) {
+          delete h;
+          set_error("conv: kernel_id out of range");
+          return nullptr;
+        }
+      }
+      if (ok) {
+        h->kernel_count = count;
+        h->workspace_bytes = (size_t)workspace;
+        h->caller_pointers = workspace ? 5 : 4;
+        return h;
+      }
+      delete h; // operands not in whole 16-byte chunks: the general route below
+    }
+  }
+
   // split of the reduction over n (one group only: the splits take the group index)
   int64_t S = 1;
   if (cp.g == 1) {

@@ -10,7 +10,8 @@ same three kinds of config lines are accepted,
                -head_dim_qk 128 -head_dim_v 128"   (perfRunner.py:590-622)
   conv        "-n 256 -c 128 -H 28 -W 28 -k 128 -y 3 -x 3 -p 1 -q 1 -u 1 -v 1
                -l 1 -j 1 -g 1 -m conv -t 1"        (MIOpenDriver letters,
-              perfRunner.py:261-307,387-470; layouts from --layouts)
+              perfRunner.py:261-307,387-470; layouts from --layouts; -F 1,
+              2 or 4, or --direction, picks forward, backward data, backward weight)
 
 every problem goes through the C ABI, is timed with HIP events on synthetic
 data, and is reported with the reference's FLOP formulas
@@ -85,13 +86,16 @@ _CONV_TYPES = {"conv": "f32", "convfp16": "f16", "convbfp16": "bf16", "convint8"
 _LAYOUTS = {"NCHW": ("gkcyx", "ngchw", "ngkhw"), "NHWC": ("gkyxc", "nhwgc", "nhwgk")}
 
 
-def conv_problem(line, t, layout):
+def conv_problem(line, t, layout, direction_flag=None):
+    if direction_flag:
+        line = line + " -F " + direction_flag
     toks = shlex.split(line)
     if toks and not toks[0].startswith("-"):  # leading "convfp16"-style type word
         t = _CONV_TYPES.get(toks[0], t)
     f = _flags(line)
-    if f.get("F", "1") != "1":
-        raise ValueError("only the forward direction (-F 1) is built")
+    direction = {"1": "conv", "2": "conv_bwd_data", "4": "conv_bwd_weight"}.get(f.get("F", "1"))
+    if direction is None:
+        raise ValueError("-F must be 1 (forward), 2 (backward data) or 4 (backward weight)")
     fl, il, ol = _LAYOUTS[layout]
     n, c, hi, wi, k = int(f["n"]), int(f["c"]), int(f["H"]), int(f["W"]), int(f["k"])
     y, x, g = int(f["y"]), int(f["x"]), int(f.get("g", 1))
@@ -100,13 +104,14 @@ def conv_problem(line, t, layout):
     ho = (hi + 2 * ph - (y - 1) * dh - 1) // sh + 1
     wo = (wi + 2 * pw - (x - 1) * dw - 1) // sw + 1
     name = {"f32": "f32", "f16": "fp16", "bf16": "bf16", "i8": "i8"}[t]
-    opts = ("--operation conv --arch gfx950 --in_type %s --fil_type %s --out_type %s --fil_layout %s --in_layout %s "
+    opts = ("--operation " + direction + " --arch gfx950 --in_type %s --fil_type %s --out_type %s --fil_layout %s --in_layout %s "
             "--out_layout %s --batchsize %d --groupsize %d --in_channels %d --out_channels %d --in_h %d --in_w %d "
             "--fil_h %d --fil_w %d --dilation_h %d --dilation_w %d --conv_stride_h %d --conv_stride_w %d "
             "--padding_h %d --padding_w %d"
             % (name, name, {"i8": "i32"}.get(t, name), fl, il, ol, n, g, c, k, hi, wi, y, x, dh, dw, sh, sw, ph, pw))
-    # pointer order filter, input, output, bias
-    shapes = [((k * (c // g) * y * x,), t), ((n * c * hi * wi,), t), ((n * k * ho * wo,), _out_type(t)), None]
+    # pointer order filter, input, output, bias; the written tensor comes last in `shapes`' order of use
+    out_t = _out_type(t) if direction == "conv" else t
+    shapes = [((k * (c // g) * y * x,), t), ((n * c * hi * wi,), t), ((n * k * ho * wo,), out_t), None]
     return opts, shapes, 2.0 * n * (c // g) * k * ho * wo * y * x
 
 
@@ -115,13 +120,16 @@ def run_problem(rock, torch, dev, opts, shapes, flops, warmup, iters):
         prog = rock.RockProgram(opts)  # every kernel of the problem and its workspace
     except rock.RockError as e:
         return {"status": "no kernel", "error": str(e).split(" [")[0]}
-    # the last tensor in pointer order is the output; the bias slot stays empty
+    # the last tensor in pointer order is left uninitialised (the forward output; for the
+    # gradients every tensor holds some data, which is all timing needs); the bias slot stays empty
     last = max(i for i, s in enumerate(shapes) if s is not None)
     args = [None if s is None else
             torch.empty(s[0], device=dev, dtype=_torch_dtype(torch, s[1])) if i == last else _rand(torch, s[0], s[1], dev)
             for i, s in enumerate(shapes)]
     ms = prog.benchmark(*args, warmup=warmup, iters=iters)
-    return {"status": "ok", "kernel": prog.main.kernel_name, "kernels": len(prog.kernels), "ms": round(ms, 5),
+    contraction = [k.kernel_name for k in prog.kernels if k.kernel_name.startswith(("rock_conv", "rock_gemm",
+                                                                                     "rock_attention"))]
+    return {"status": "ok", "kernel": contraction[-1], "kernels": len(prog.kernels), "ms": round(ms, 5),
             "tflops": round(flops / (ms * 1e-3) / 1e12, 2)}
 
 
@@ -131,6 +139,8 @@ def main(argv=None):
     ap.add_argument("--op", choices=["gemm", "conv", "attention"], required=True)
     ap.add_argument("--types", default="f16", help="comma-separated element types for lines that name none")
     ap.add_argument("--layouts", default="NHWC", help="conv only: comma-separated subset of NHWC,NCHW")
+    ap.add_argument("--direction", choices=["1", "2", "4"], default=None,
+                    help="conv only: run every line forward (1), backward data (2) or backward weight (4)")
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--max-bytes", type=float, default=8e9, help="skip problems whose tensors exceed this")
@@ -151,7 +161,7 @@ def main(argv=None):
                     elif args.op == "attention":
                         opts, shapes, flops = attention_problem(line, t)
                     else:
-                        opts, shapes, flops = conv_problem(line, t, layout)
+                        opts, shapes, flops = conv_problem(line, t, layout, args.direction)
                 except (KeyError, ValueError) as e:
                     print(json.dumps({"config": line, "status": "unparsed", "error": str(e)}), flush=True)
                     continue

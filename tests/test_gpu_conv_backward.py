@@ -65,6 +65,8 @@ CASES = [
     (1, 1, 5, 7, 9, 9, 3, 3, (3, 3), (0, 0), (1, 1)),         # stride = filter size
     (8, 1, 16, 16, 6, 6, 3, 3, (1, 1), (1, 1), (1, 1)),       # batch large enough to split the weight reduction
     (4, 1, 16, 16, 5, 5, 2, 2, (1, 1), (0, 0), (2, 2)),
+    (4, 1, 16, 24, 6, 6, 1, 1, (1, 1), (0, 0), (1, 1)),       # pointwise: the weight gradient is a split GEMM
+    (3, 1, 64, 48, 8, 8, 1, 1, (1, 1), (0, 0), (1, 1)),
 ]
 LAYOUTS = [NHWC, NCHW, ("gyxck", "hwcgn", "hwkgn")]
 
@@ -124,7 +126,12 @@ def test_conv_bwd_weight_exact(rock, oracle, gpu, case, layouts, t, convert):
     torch.cuda.synchronize()
     ref, _, _ = oracle.conv_bwd_weight(iq, dyq, *layouts, n, g, c, k, hi, wi, y, x, stride, pad, dil)
     assert np.array_equal(to_f32(got, t), oracle.round_through(ref, CODE[t]))
-    assert (len(info["kernels"]) == 1) == (not convert) or "generic" in info["kernels"][-1]
+    if (c, hi) == (64, 8) and layouts in (NHWC, NCHW):
+        # pointwise with whole 16-byte runs: a GEMM over the tensors as they lie, its split
+        # partial sums added by the reduction kernel
+        assert info["kernels"][0].startswith("rock_gemm_") and not any("relayout" in k for k in info["kernels"])
+    elif not convert and not info["kernels"][0].startswith("rock_gemm_"):
+        assert len(info["kernels"]) == 1
 
 
 @pytest.mark.parametrize("t", ["f16", "f32"])
