@@ -56,7 +56,9 @@ typedef void *MiirHandle;
 
 /* Miir.h:50 (impl rocmlir-lib.cpp:117-154).  `options` is a whitespace
  * separated "--key value" list.  Convolution keys are the reference's
- * (ConvGenerator.cpp:492-661): operation, arch, num_cu, kernel_id,
+ * (ConvGenerator.cpp:492-661): operation {conv|conv_bwd_data|conv_bwd_weight}
+ * (the gradients take f32, f16 or bf16, the forward problem's keys and pointer
+ * order, and usually several kernels: see rockamdGetPointerMap), arch, num_cu, kernel_id,
  * kernel_name, perf_config, in_type/fil_type/out_type, in_layout/fil_layout/
  * out_layout, batchsize, groupsize, in_channels, out_channels, in_h, in_w,
  * out_h, out_w, fil_h, fil_w, dilation_{h,w}, conv_stride_{h,w},
