@@ -507,9 +507,11 @@ def conv2d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize,
     return out
 
 
-def attention(q, k, v, *, scale=1.0, bias=None, transQ=False, transK=False,
+def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, transQ=False, transK=False,
               transV=False, transO=False, out=None, stream=None):
-    """O = softmax(scale * Q K + bias) V with the reference's storage
+    """O = softmax(scale * scale_tensor * Q K + bias) V (bias and scale_tensor
+    optional [G,seq_q,seq_k] tensors, rocmlir-gen's -with-attn-bias /
+    -with-attn-scale) with the reference's storage
     conventions (rocmlir-gen.cpp:2149-2200): q [G,seq_q,d] ([G,d,seq_q] if
     transQ); k [G,d,seq_k] ([G,seq_k,d] if transK -- the usual row-major keys);
     v [G,seq_k,dv] ([G,dv,seq_k] if transV); result [G,seq_q,dv]
@@ -529,11 +531,16 @@ def attention(q, k, v, *, scale=1.0, bias=None, transQ=False, transK=False,
                tf(transO), scale))
     if bias is not None:
         opts += " -with-attn-bias true"
+    if scale_tensor is not None:
+        opts += " -with-attn-scale true"
     kern = _kernel(opts)
     shape = (G, dv, sq) if transO else (G, sq, dv)
     if out is None:
         out = torch.empty(shape, dtype=q.dtype, device=q.device)
-    kern.launch(q, k, v, bias, out, stream=stream)
+    if scale_tensor is None:
+        kern.launch(q, k, v, bias, out, stream=stream)
+    else:
+        kern.launch(q, k, v, scale_tensor.contiguous(), bias, out, stream=stream)
     return out
 
 

@@ -117,7 +117,7 @@ template <int DT> __device__ __forceinline__ uint32_t pack2_fast(float a, float 
 // the raw scores and the scale folded into the exponent.
 template <int DT, int D, bool PLAIN>
 __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv, const void *Vv,
-                                                  const void *biasv, void *Ov,
+                                                  const void *scalev, const void *biasv, void *Ov,
                                                   const RockAttentionParams &p) {
   using Gm = AttnTileGeom<D>;
   constexpr int KSTEPS = D / 16;  // MFMA K steps of the first GEMM
@@ -155,6 +155,7 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
   const uint16_t *V = (const uint16_t *)Vv + (int64_t)g * p.v_gs;
   uint16_t *O = (uint16_t *)Ov + (int64_t)g * p.o_gs;
   const uint16_t *bias = p.has_bias ? (const uint16_t *)biasv + (int64_t)g * p.bias_gs : nullptr;
+  const uint16_t *scale_t = p.has_scale_tensor ? (const uint16_t *)scalev + (int64_t)g * p.bias_gs : nullptr;
 
   AttnTileLoader<D, false> lk;
   AttnTileLoader<D, true> lv;
@@ -250,8 +251,12 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int kofs = st * 32 + 8 * (v >> 2) + (v & 3);
-          float x = s[st][v] * c_scale;
-          if (bias != nullptr && key_base + kofs < p.seq_k && q_row < p.seq_q)
+          float x = s[st][v];
+          const bool in_range = key_base + kofs < p.seq_k && q_row < p.seq_q;
+          if (scale_t != nullptr && in_range)
+            x = x * elem_to_f32<DT>(scale_t[boff + (unsigned)kofs * bias_js]);
+          x = x * c_scale;
+          if (bias != nullptr && in_range)
             x = x + elem_to_f32<DT>(bias[boff + (unsigned)kofs * bias_js]) * kLog2e;
           s[st][v] = x;
         }

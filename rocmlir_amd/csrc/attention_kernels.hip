@@ -114,7 +114,7 @@ __device__ __forceinline__ v4i load8(const uint16_t *base, int64_t rs, int64_t c
 
 template <int DT, int DQK, int DV, bool FAST>
 __device__ __forceinline__ void attention_body(const void *Qv, const void *Kv, const void *Vv,
-                                               const void *biasv, void *Ov,
+                                               const void *scalev, const void *biasv, void *Ov,
                                                const RockAttentionParams &p) {
   constexpr int KCH = DQK / 8;              // 16-byte chunks per K row
   constexpr int KPITCH = DQK * 2 + 16;      // bytes
@@ -152,6 +152,7 @@ __device__ __forceinline__ void attention_body(const void *Qv, const void *Kv, c
   const uint16_t *V = (const uint16_t *)Vv + (int64_t)g * p.v_gs;
   uint16_t *O = (uint16_t *)Ov + (int64_t)g * p.o_gs;
   const uint16_t *bias = p.has_bias ? (const uint16_t *)biasv + (int64_t)g * p.bias_gs : nullptr;
+  const uint16_t *scale_t = p.has_scale_tensor ? (const uint16_t *)scalev + (int64_t)g * p.bias_gs : nullptr;
 
   // ---- Q^T fragments: column operand, lane = query row, 8 d per K step
   v4i qf[KSTEPS];
@@ -257,7 +258,11 @@ __device__ __forceinline__ void attention_body(const void *Qv, const void *Kv, c
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         int key = key_base + st * 32 + 8 * (v >> 2) + (v & 3);
-        float x = s[st][v] * c_scale;
+        float x = s[st][v];
+        // op order of the reference: * scale tensor, * scale, + bias (rocmlir-gen.cpp:2565-2590)
+        if (scale_t != nullptr && key < p.seq_k && q_row < p.seq_q)
+          x = x * elem_to_f32<DT>(scale_t[(int64_t)q_row * p.bias_is + (int64_t)key * p.bias_js]);
+        x = x * c_scale;
         if (bias != nullptr && key < p.seq_k && q_row < p.seq_q)
           x = x + elem_to_f32<DT>(bias[(int64_t)q_row * p.bias_is + (int64_t)key * p.bias_js]) *
                       1.44269504088896340736f;
@@ -350,22 +355,24 @@ __device__ __forceinline__ void wait_loads_and_lds_reads() {
 
 #include "attention_dlds.h"
 
-// pointer order follows the reference: Q, K, V, [pre-softmax bias], O
+// pointer order follows the reference: Q, K, V, [pre-softmax scale tensor], [pre-softmax bias], O
 #define RK_ATTN(DTNAME, DT, DQK, DV, FASTNAME, FAST)                                          \
   extern "C" __global__ __launch_bounds__(rk::kAttnThreads) void                              \
       rock_attention_##DTNAME##_d##DQK##x##DV##_##FASTNAME(const void *Q, const void *K,     \
-                                                           const void *V, const void *bias,  \
-                                                           void *O, RockAttentionParams p) { \
-    rk::attention_body<DT, DQK, DV, FAST>(Q, K, V, bias, O, p);                               \
+                                                           const void *V, const void *scale, \
+                                                           const void *bias, void *O,        \
+                                                           RockAttentionParams p) {          \
+    rk::attention_body<DT, DQK, DV, FAST>(Q, K, V, scale, bias, O, p);                        \
   }
 
 // fast variants: two blocks per compute unit (register budget 256 per lane)
 #define RK_ATTN_DL(DTNAME, DT, D, SUFFIX, PLAIN)                                              \
   extern "C" __global__ __launch_bounds__(rk::kAttnThreads, 2) void                           \
       rock_attention_##DTNAME##_d##D##x##D##_##SUFFIX(const void *Q, const void *K,           \
-                                                      const void *V, const void *bias,        \
-                                                      void *O, RockAttentionParams p) {       \
-    rk::attention_body_dl<DT, D, PLAIN>(Q, K, V, bias, O, p);                                 \
+                                                      const void *V, const void *scale,       \
+                                                      const void *bias, void *O,              \
+                                                      RockAttentionParams p) {                \
+    rk::attention_body_dl<DT, D, PLAIN>(Q, K, V, scale, bias, O, p);                          \
   }
 
 RK_ATTN_DL(f16, MM_F16, 128, fast, true)

@@ -134,11 +134,11 @@ struct RockAttentionParams {
   int64_t k_gs, k_js, k_ds;
   int64_t v_gs, v_js, v_es;
   int64_t o_gs, o_is, o_es;
-  int64_t bias_gs, bias_is, bias_js; // optional additive bias [g,i,j] (aux pointer)
+  int64_t bias_gs, bias_is, bias_js; // optional pre-softmax tensors [g,i,j]: additive bias, multiplicative scale
   int32_t G, seq_q, seq_k, d_qk, d_v;
   int32_t q_blocks;    // blocks of query rows per g
   float scale;         // multiplies Q*K^T before the softmax
   int32_t has_bias;
   int32_t xcd_remap;
-  int32_t pad_;
+  int32_t has_scale_tensor; // scores are multiplied element-wise by the scale tensor before `scale`
 };

@@ -1507,6 +1507,9 @@ Handle *make_attention(const OptMap &o) {
   bool tQ = bool_or(o, "transQ", false), tK = bool_or(o, "transK", false),
        tV = bool_or(o, "transV", false), tO = bool_or(o, "transO", false);
   bool has_bias = bool_or(o, "with-attn-bias", false);
+  // "-with-attn-scale": a full [G, seq_q, seq_k] tensor multiplied into the
+  // scores before the softmax (rocmlir-gen.cpp:2185-2196), besides the scalar "-scale"
+  bool has_scale_t = bool_or(o, "with-attn-scale", false);
 
   auto *h = new Handle;
   h->op = OP_ATTENTION;
@@ -1522,6 +1525,7 @@ Handle *make_attention(const OptMap &o) {
   p.o_gs = sq * dv; p.o_is = tO ? 1 : dv; p.o_es = tO ? sq : 1;
   p.bias_gs = sq * sk; p.bias_is = sk; p.bias_js = 1;
   p.has_bias = has_bias ? 1 : 0;
+  p.has_scale_tensor = has_scale_t ? 1 : 0;
   p.scale = 1.0f;
   get_float(o, "scale", p.scale);
   p.q_blocks = ceil_div(sq, 128);
@@ -1538,14 +1542,22 @@ Handle *make_attention(const OptMap &o) {
                     // byte offsets inside one g slice below 2^31 (buffer descriptors)
                     sk * p.k_js * 2 < ((int64_t)1 << 31) && sk * p.v_js * 2 < ((int64_t)1 << 31) &&
                     // the bias gather indexes one g slice with 32-bit element offsets
-                    (!has_bias || sq * sk < ((int64_t)1 << 31));
+                    ((!has_bias && !has_scale_t) || sq * sk < ((int64_t)1 << 31));
   const int dmax = (dqk <= 64 && dv <= 64) ? 64 : 128;
   char name[96];
   std::snprintf(name, sizeof name, "rock_attention_%s_d%dx%d_%s", dtype_name(ty), dmax, dmax,
-                !fast ? "generic" : (!p.has_bias && p.scale >= 0.0f) ? "fast" : "fast_bias");
+                !fast ? "generic" : (!p.has_bias && !has_scale_t && p.scale >= 0.0f) ? "fast" : "fast_bias");
   h->kernel_name = name;
   h->blob_name = "attention";
-  h->num_pointers = 5;
+  // kernel pointers: Q, K, V, scale tensor, bias, O; a caller passes the scale
+  // tensor only when the problem names one
+  h->num_pointers = 6;
+  if (has_scale_t) {
+    h->caller_pointers = 0;
+  } else {
+    h->caller_pointers = 5;
+    h->ptr_map = {{0, 0}, {1, 0}, {2, 0}, {-1, 0}, {3, 0}, {4, 0}};
+  }
   h->block_size = 256;
   h->grid_size = (uint32_t)total;
   // attn:v1:MPB_G0,MPB_G1,NPB_G0,KpackPB,MPW,MnPerXdl,Kpack,forceUnroll
@@ -1637,10 +1649,13 @@ bool check_launch_args(Handle *h, void *const *pointers, int num_pointers) {
       set_error("launch: tensor pointers must be 16-byte aligned");
       return false;
     }
-  int aux_index = 3;
-  bool need_aux = h->op == OP_ATTENTION
-                      ? reinterpret_cast<RockAttentionParams *>(h->params.data())->has_bias != 0
-                      : (h->epi && h->epi->has_bias != 0);
+  int aux_index = 3; // the bias slot, which may be NULL when the problem has no bias
+  bool need_aux = h->epi && h->epi->has_bias != 0;
+  if (h->op == OP_ATTENTION) {
+    const auto *ap = reinterpret_cast<RockAttentionParams *>(h->params.data());
+    need_aux = ap->has_bias != 0;
+    aux_index = ap->has_scale_tensor ? 4 : 3;
+  }
   for (int i = 0; i < num_pointers; ++i)
     if (!pointers[i] && (i != aux_index || need_aux)) {
       set_error("launch: NULL tensor pointer");

@@ -108,7 +108,7 @@ def test_baseline_configs_select_kernels(rock):
     k = rock.RockKernel("-operation attention -arch gfx950 -t f16 -g 128 -seq_len_q 2048 -seq_len_k 2048 "
                         "-head_dim_qk 128 -head_dim_v 128 -transK true -scale 0.08838834764831845")
     assert k.kernel_name == "rock_attention_f16_d128x128_fast"
-    assert (k.block_size, k.grid_size, k.num_pointers) == (256, 128 * 16, 5)
+    assert (k.block_size, k.grid_size, k.num_pointers, k.caller_pointers) == (256, 128 * 16, 6, 5)
 
 
 def test_generic_kernels_for_unaligned_or_transposed(rock):
@@ -223,6 +223,18 @@ def test_layout_conversion_plan_follows_the_multi_kernel_protocol(rock):
     assert (k.kernel_count, k.workspace_bytes, k.caller_pointers) == (1, 0, 4)
     # a conversion kernel has no epilogue scalars to set
     assert lib.rockamdSetScale(rock.RockKernel(nchw)._h, C.c_float(2.0)) != 0
+
+
+def test_attention_pre_softmax_tensors(rock):
+    """-with-attn-scale / -with-attn-bias (rocmlir-gen.cpp:2185-2196): the
+    caller list is Q, K, V, [scale tensor], bias slot, O."""
+    base = ("-operation attention -arch gfx950 -t f16 -g 4 -seq_len_q 256 -seq_len_k 256 -head_dim_qk 64 "
+            "-head_dim_v 64 -transK true")
+    assert rock.RockKernel(base).kernel_name == "rock_attention_f16_d64x64_fast"
+    k = rock.RockKernel(base + " -with-attn-bias true")
+    assert (k.kernel_name, k.caller_pointers) == ("rock_attention_f16_d64x64_fast_bias", 5)
+    k = rock.RockKernel(base + " -with-attn-scale true")
+    assert (k.kernel_name, k.caller_pointers, k.num_pointers) == ("rock_attention_f16_d64x64_fast_bias", 6, 6)
 
 
 def test_backward_convolution_plans(rock):

@@ -19,7 +19,7 @@ def _store(mat, trans):
 
 
 def _run(rock, oracle, gpu, t, G, sq, sk, dqk, dv, scale, seed, tQ=False, tK=True, tV=False, tO=False,
-         bias=False, vones=False):
+         bias=False, vones=False, scale_tensor=False):
     rng = np.random.default_rng(seed)
     Q = rng.standard_normal((G, sq, dqk)).astype(np.float32)
     K = rng.standard_normal((G, sk, dqk)).astype(np.float32)
@@ -30,11 +30,15 @@ def _run(rock, oracle, gpu, t, G, sq, sk, dqk, dv, scale, seed, tQ=False, tK=Tru
     bq = braw = None
     if bias:
         braw, bq = quantise(rng.standard_normal((G, sq, sk)).astype(np.float32), t)
+    sq_ = sraw = None
+    if scale_tensor:
+        sraw, sq_ = quantise(rng.uniform(-1.5, 1.5, (G, sq, sk)).astype(np.float32), t)
     out = rock.attention(to_gpu(rq, t, gpu), to_gpu(rk, t, gpu), to_gpu(rv, t, gpu), scale=scale,
                          bias=to_gpu(braw, t, gpu) if bias else None,
+                         scale_tensor=to_gpu(sraw, t, gpu) if scale_tensor else None,
                          transQ=tQ, transK=tK, transV=tV, transO=tO)
     torch.cuda.synchronize()
-    ref = oracle.attention(Qq, Kq, Vq, G, sq, sk, dqk, dv, scale=scale, bias_t=bq,
+    ref = oracle.attention(Qq, Kq, Vq, G, sq, sk, dqk, dv, scale=scale, bias_t=bq, scale_t=sq_,
                            transQ=tQ, transK=tK, transV=tV, transO=tO)
     return to_f32(out, t), ref
 
@@ -67,6 +71,17 @@ def test_attention_odd_head_dims_take_generic_kernel(rock, oracle, gpu):
 def test_attention_with_bias(rock, oracle, gpu):
     # cross attention with scale and bias: seq_q 128, seq_k 27, d_qk 64, d_v 32
     got, ref = _run(rock, oracle, gpu, "f16", 2, 128, 27, 64, 32, 0.125, 45, bias=True)
+    check_float(got, ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
+
+
+@pytest.mark.parametrize("bias", [False, True])
+@pytest.mark.parametrize("shape", [(2, 128, 27, 64, 32), (1, 300, 200, 128, 128), (2, 50, 70, 20, 12)],
+                         ids=["cross", "d128", "generic"])
+def test_attention_with_scale_tensor(rock, oracle, gpu, shape, bias):
+    """-with-attn-scale: a [G,seq_q,seq_k] tensor multiplied into the scores
+    before the softmax (rocmlir-gen.cpp:2185-2196, 2368-2382), alone and with a bias."""
+    G, sq, sk, dqk, dv = shape
+    got, ref = _run(rock, oracle, gpu, "f16", G, sq, sk, dqk, dv, 0.125, 49, bias=bias, scale_tensor=True)
     check_float(got, ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
 
 
