@@ -88,6 +88,11 @@ ROCMLIR_AMD_API int miirGetKernelCount(MiirHandle handle);
  * single-kernel problems); -1 for a NULL handle or a size beyond int. */
 ROCMLIR_AMD_API int miirGetWorkspaceSize(MiirHandle handle);
 
+/* The same as a size_t ((size_t)-1 for a NULL handle): the score workspace of
+ * attention run as three kernels can exceed what Miir.h:65's int holds.  No
+ * counterpart in the reference. */
+ROCMLIR_AMD_API size_t rockamdGetWorkspaceSize64(MiirHandle handle);
+
 /* Miir.h:70 -- resolves the perf config (table lookup); needed before
  * miirGetExecutionDims, as in the reference flow. */
 ROCMLIR_AMD_API MiirStatus miirLowerTuningParams(MiirHandle handle);

@@ -47,6 +47,8 @@ def load_library():
                      "miirDestroyHandle"):
             getattr(L, name).restype = C.c_int
             getattr(L, name).argtypes = [vp]
+        L.rockamdGetWorkspaceSize64.restype = sz
+        L.rockamdGetWorkspaceSize64.argtypes = [vp]
         L.miirBufferGet.restype = C.c_int
         L.miirBufferGet.argtypes = [vp, C.c_char_p, C.POINTER(sz)]
         L.miirGetExecutionDims.restype = C.c_int
@@ -164,7 +166,7 @@ class RockKernel:
         # multi-kernel problems: kernels of the problem, its workspace, and the
         # caller pointer list every one of its kernels is launched with
         self.kernel_count = L.miirGetKernelCount(self._h)
-        self.workspace_bytes = L.miirGetWorkspaceSize(self._h)
+        self.workspace_bytes = L.rockamdGetWorkspaceSize64(self._h)
         ncall = C.c_int(0)
         L.rockamdGetPointerMap(self._h, C.byref(ncall), None, None, None)
         self.caller_pointers = ncall.value
@@ -533,7 +535,7 @@ def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, transQ=False,
         opts += " -with-attn-bias true"
     if scale_tensor is not None:
         opts += " -with-attn-scale true"
-    kern = _kernel(opts)
+    kern = _program(opts)   # one fused kernel, or three for head dimensions above 128 and f32
     shape = (G, dv, sq) if transO else (G, sq, dv)
     if out is None:
         out = torch.empty(shape, dtype=q.dtype, device=q.device)

@@ -128,6 +128,22 @@ struct RockReduceParams {
   int32_t out_dtype; // RockDType: f32, f16 or bf16
 };
 
+// rock_softmax_rows(S, scale_tensor, bias, p): the middle kernel of attention
+// run as three kernels (head dimensions beyond the fused kernel's, f32).  S
+// holds G*seq_q rows of seq_k f32 scores, `row_pitch` floats apart; row by row
+//   x_j = S_j * scale_tensor_j * scale + bias_j ; P_j = exp(x_j - max) / sum
+// and P is written IN PLACE in the element type `dtype` from the start of the
+// row (so rows of P are row_pitch * 4 bytes apart).
+struct RockSoftmaxParams {
+  int64_t row_pitch;
+  int64_t t_gs, t_is, t_js; // element strides of the [g, i, j] scale tensor and bias
+  int32_t G, seq_q, seq_k;
+  float scale;
+  int32_t has_bias, has_scale_tensor;
+  int32_t dtype; // RockDType of P, the scale tensor and the bias: f32, f16 or bf16
+  int32_t pad_;
+};
+
 struct RockAttentionParams {
   // element strides of the logical views Q[g,i,d], K[g,j,d], V[g,j,e], O[g,i,e]
   int64_t q_gs, q_is, q_ds;

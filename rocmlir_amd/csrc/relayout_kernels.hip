@@ -243,3 +243,75 @@ extern "C" __global__ __launch_bounds__(256) void rock_reduce_splits(const float
     ((__bf16 *)dst)[off] = (__bf16)acc;
   }
 }
+
+namespace {
+__device__ __forceinline__ float load_as_f32(const void *base, int64_t idx, int dtype) {
+  if (dtype == ROCK_F32)
+    return ((const float *)base)[idx];
+  if (dtype == ROCK_F16)
+    return (float)((const _Float16 *)base)[idx];
+  return __builtin_bit_cast(float, (uint32_t)((const uint16_t *)base)[idx] << 16);
+}
+
+__device__ __forceinline__ float block_reduce(float v, bool take_max, float *scratch) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float o = __shfl_xor(v, off, 64);
+    v = take_max ? fmaxf(v, o) : v + o;
+  }
+  __syncthreads(); // scratch may still be read from the previous reduction
+  if ((threadIdx.x & 63) == 0)
+    scratch[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float r = scratch[0];
+#pragma unroll
+  for (int w = 1; w < 4; ++w)
+    r = take_max ? fmaxf(r, scratch[w]) : r + scratch[w];
+  return r;
+}
+} // namespace
+
+// One block per row, three passes over it (maximum, sum, normalise); the last
+// pass loads a chunk of scores into registers before any thread overwrites the
+// narrower results over them.
+extern "C" __global__ __launch_bounds__(256) void rock_softmax_rows(float *S, const void *scale_t, const void *bias,
+                                                                    RockSoftmaxParams p) {
+  __shared__ float scratch[4];
+  const int64_t row = blockIdx.x;
+  const int g = (int)(row / p.seq_q), i = (int)(row - (int64_t)g * p.seq_q);
+  float *s = S + row * p.row_pitch;
+  const int64_t t_off = (int64_t)g * p.t_gs + (int64_t)i * p.t_is;
+  auto score = [&](int j) {
+    float x = s[j];
+    if (p.has_scale_tensor)
+      x = x * load_as_f32(scale_t, t_off + (int64_t)j * p.t_js, p.dtype);
+    x = x * p.scale;
+    if (p.has_bias)
+      x = x + load_as_f32(bias, t_off + (int64_t)j * p.t_js, p.dtype);
+    return x;
+  };
+  float m = -INFINITY;
+  for (int j = threadIdx.x; j < p.seq_k; j += 256)
+    m = fmaxf(m, score(j));
+  m = block_reduce(m, true, scratch);
+  float l = 0.0f;
+  for (int j = threadIdx.x; j < p.seq_k; j += 256)
+    l = l + expf(score(j) - m);
+  l = block_reduce(l, false, scratch);
+  const float inv = 1.0f / l;
+  for (int j0 = 0; j0 < p.seq_k; j0 += 256) {
+    const int j = j0 + (int)threadIdx.x;
+    float e = 0.0f;
+    if (j < p.seq_k)
+      e = expf(score(j) - m) * inv;
+    __syncthreads(); // every score of this chunk is in a register
+    if (j < p.seq_k) {
+      if (p.dtype == ROCK_F32)
+        s[j] = e;
+      else if (p.dtype == ROCK_F16)
+        ((_Float16 *)s)[j] = (_Float16)e;
+      else
+        ((__bf16 *)s)[j] = (__bf16)e;
+    }
+  }
+}

@@ -1485,12 +1485,97 @@ Handle *make_conv(const OptMap &o) {
   return h;
 }
 
+// Attention outside the fused kernel's reach (head dimensions above 128, f32):
+// three kernels over a workspace of G * seq_q * seq_k f32 scores -- the GEMM
+// Q K^T, a row softmax that applies scale tensor, scale and bias and narrows
+// the probabilities in place, and the GEMM P V.  The reference fuses every
+// shape (GridwiseGemmToBlockwise.cpp:1607-2403); its validator computes these
+// same three steps (rocmlir-gen.cpp:2565-2620).
+Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, int64_t sk, int64_t dqk, int64_t dv,
+                               bool tQ, bool tK, bool tV, bool tO, bool has_bias, bool has_scale_t) {
+  const int es = dtype_size(ty);
+  const int kid = (int)int_or(o, "kernel_id", 0);
+  if (kid < 0 || kid > 2) {
+    set_error("attention: kernel_id out of range");
+    return nullptr;
+  }
+  if (sq * sk > INT32_MAX * (int64_t)4 || G * sq > INT32_MAX) {
+    set_error("attention: score matrix too large for the three-kernel form");
+    return nullptr;
+  }
+  float scale = 1.0f;
+  get_float(o, "scale", scale);
+  // caller list: Q, K, V, [scale tensor], bias slot, O, workspace
+  const int i_bias = has_scale_t ? 4 : 3, i_out = i_bias + 1, i_ws = i_out + 1;
+  const int64_t pitch_p = 4 / es; // elements of P per f32 score: P lies in place, rows sk * 4 bytes apart
+  auto *h = new Handle;
+  if (kid == 1) {
+    RockSoftmaxParams r;
+    std::memset(&r, 0, sizeof r);
+    r.row_pitch = sk;
+    r.t_gs = sq * sk; r.t_is = sk; r.t_js = 1;
+    r.G = (int)G; r.seq_q = (int)sq; r.seq_k = (int)sk;
+    r.scale = scale;
+    r.has_bias = has_bias ? 1 : 0;
+    r.has_scale_tensor = has_scale_t ? 1 : 0;
+    r.dtype = ty;
+    h->op = OP_RELAYOUT;
+    h->epi = nullptr;
+    h->params.assign(sizeof r, 0);
+    std::memcpy(h->params.data(), &r, sizeof r);
+    h->kernel_name = "rock_softmax_rows";
+    h->blob_name = "relayout";
+    h->block_size = 256;
+    h->grid_size = (uint32_t)(G * sq);
+    h->num_pointers = 3;
+    h->perf_config = "";
+    h->ptr_map = {{i_ws, 0}, {has_scale_t ? 3 : -1, 0}, {has_bias ? i_bias : -1, 0}};
+    h->problem_key = "row softmax of the attention scores";
+  } else {
+    RockGemmParams gp;
+    std::memset(&gp, 0, sizeof gp);
+    gp.G = (int)G;
+    if (kid == 0) { // S[g,i,j] = sum_d Q[g,i,d] K[g,j,d], f32
+      gp.M = (int)sq; gp.N = (int)sk; gp.K = (int)dqk;
+      gp.a_gs = sq * dqk; gp.a_ms = tQ ? 1 : dqk; gp.a_ks = tQ ? sq : 1;
+      gp.b_gs = sk * dqk; gp.b_ns = tK ? dqk : 1; gp.b_ks = tK ? 1 : sk;
+      gp.c_gs = sq * sk; gp.c_ms = sk; gp.c_ns = 1;
+      default_epilogue(gp.epi, ROCK_F32);
+    } else { // O[g,i,e] = sum_j P[g,i,j] V[g,j,e]
+      gp.M = (int)sq; gp.N = (int)dv; gp.K = (int)sk;
+      gp.a_gs = sq * sk * pitch_p; gp.a_ms = sk * pitch_p; gp.a_ks = 1;
+      gp.b_gs = sk * dv; gp.b_ns = tV ? sk : 1; gp.b_ks = tV ? 1 : dv;
+      gp.c_gs = sq * dv; gp.c_ms = tO ? 1 : dv; gp.c_ns = tO ? sq : 1;
+      default_epilogue(gp.epi, ty);
+    }
+    plan_gemm_kernel(h, gp, operand_code(ty, ty), es, o);
+    if (kid == 0)
+      h->ptr_map = {{0, 0}, {1, 0}, {i_ws, 0}, {-1, 0}, {-1, 0}};
+    else
+      h->ptr_map = {{i_ws, 0}, {2, 0}, {i_out, 0}, {-1, 0}, {-1, 0}};
+    h->op = OP_GEMM;
+    h->params.assign(sizeof gp, 0);
+    std::memcpy(h->params.data(), &gp, sizeof gp);
+    h->epi = &reinterpret_cast<RockGemmParams *>(h->params.data())->epi;
+    std::ostringstream key;
+    auto tf = [](bool b) { return b ? "true" : "false"; };
+    key << h->arch << '\t' << int_or(o, "num_cu", kNumCU) << '\t' << "-t " << dtype_name(ty) << " -transQ " << tf(tQ)
+        << " -transK " << tf(tK) << " -transV " << tf(tV) << " -transO " << tf(tO) << " -g " << G << " -seq_len_q "
+        << sq << " -seq_len_k " << sk << " -head_dim_qk " << dqk << " -head_dim_v " << dv;
+    h->problem_key = key.str();
+  }
+  h->kernel_count = 3;
+  h->workspace_bytes = (size_t)(G * sq * sk * 4);
+  h->caller_pointers = i_ws + 1;
+  return h;
+}
+
 // ---- attention --------------------------------------------------------------------
 Handle *make_attention(const OptMap &o) {
   std::string t = str_or(o, "t", "f16");
   int ty = parse_dtype(t);
-  if (ty != ROCK_F16 && ty != ROCK_BF16) {
-    set_error("attention: only f16 and bf16 kernels are built ('" + t + "' requested)");
+  if (ty != ROCK_F16 && ty != ROCK_BF16 && ty != ROCK_F32) {
+    set_error("attention: f16, bf16 and f32 kernels are built ('" + t + "' requested)");
     return nullptr;
   }
   int64_t G = int_or(o, "g", 1), sq, sk, dqk, dv;
@@ -1500,16 +1585,14 @@ Handle *make_attention(const OptMap &o) {
     set_error("attention: -seq_len_q, -seq_len_k, -head_dim_qk, -head_dim_v must be positive");
     return nullptr;
   }
-  if (dqk > 128 || dv > 128) {
-    set_error("attention: head dimensions above 128 have no kernel");
-    return nullptr;
-  }
   bool tQ = bool_or(o, "transQ", false), tK = bool_or(o, "transK", false),
        tV = bool_or(o, "transV", false), tO = bool_or(o, "transO", false);
   bool has_bias = bool_or(o, "with-attn-bias", false);
   // "-with-attn-scale": a full [G, seq_q, seq_k] tensor multiplied into the
   // scores before the softmax (rocmlir-gen.cpp:2185-2196), besides the scalar "-scale"
   bool has_scale_t = bool_or(o, "with-attn-scale", false);
+  if (ty == ROCK_F32 || dqk > 128 || dv > 128)
+    return make_attention_unfused(o, ty, G, sq, sk, dqk, dv, tQ, tK, tV, tO, has_bias, has_scale_t);
 
   auto *h = new Handle;
   h->op = OP_ATTENTION;
@@ -1778,6 +1861,11 @@ int miirGetWorkspaceSize(MiirHandle handle) {
   if (!h)
     return -1;
   return h->workspace_bytes > (size_t)INT32_MAX ? -1 : (int)h->workspace_bytes;
+}
+
+size_t rockamdGetWorkspaceSize64(MiirHandle handle) {
+  auto *h = static_cast<Handle *>(handle);
+  return h ? h->workspace_bytes : (size_t)-1;
 }
 
 MiirStatus miirLowerTuningParams(MiirHandle handle) {

@@ -77,7 +77,9 @@ def test_null_handle_behaviour(rock):
     "--operation gemm --arch gfx950 -t f16 -out_datatype i32 -m 4 -n 4 -k 4",  # float in, int out
     "--operation gemm --arch gfx950 -t f16_i8 -m 4 -n 4 -k 4",
     "--operation attention --arch gfx950 -t f16 -g 1 -seq_len_q 8 -seq_len_k 8 -head_dim_qk 8",
-    "--operation attention --arch gfx950 -t f16 -g 1 -seq_len_q 8 -seq_len_k 8 -head_dim_qk 256 -head_dim_v 8",
+    "--operation attention --arch gfx950 -t i8 -g 1 -seq_len_q 8 -seq_len_k 8 -head_dim_qk 64 -head_dim_v 8",
+    "--operation attention --arch gfx950 -t f16 -g 1 -seq_len_q 8 -seq_len_k 8 -head_dim_qk 256 -head_dim_v 8 "
+    "--kernel_id 3",
     "--operation transpose --arch gfx950",
     CONV_RESNET + " --kernel_id 1",
 ])
@@ -235,6 +237,23 @@ def test_attention_pre_softmax_tensors(rock):
     assert (k.kernel_name, k.caller_pointers) == ("rock_attention_f16_d64x64_fast_bias", 5)
     k = rock.RockKernel(base + " -with-attn-scale true")
     assert (k.kernel_name, k.caller_pointers, k.num_pointers) == ("rock_attention_f16_d64x64_fast_bias", 6, 6)
+
+
+def test_attention_as_three_kernels(rock):
+    """Head dimensions above 128 and f32 (attention-configs' sdxl vae lines):
+    GEMM, row softmax in place over an f32 score workspace, GEMM."""
+    vae = ("-operation attention -arch gfx950 -t %s -g 1 -seq_len_q 16384 -seq_len_k 16384 -head_dim_qk 512 "
+           "-head_dim_v 512 -transK true")
+    for t in ("f16", "f32"):
+        ks = [rock.RockKernel(vae % t + " -kernel_id %d" % i) for i in range(3)]
+        assert ks[0].kernel_name.startswith("rock_gemm_%s_" % t) and ks[0].kernel_name.endswith("_fast")
+        assert ks[1].kernel_name == "rock_softmax_rows" and ks[1].grid_size == 16384
+        assert ks[2].kernel_name.startswith("rock_gemm_%s_" % t) and ks[2].kernel_name.endswith("_fast_nn")
+        assert all(k.kernel_count == 3 and k.workspace_bytes == 16384 * 16384 * 4 and k.caller_pointers == 6
+                   for k in ks)
+    lib = rock.load_library()
+    k = rock.RockKernel((vae % "f16").replace("-g 1 ", "-g 4 "))
+    assert k.workspace_bytes == 4 * 16384 * 16384 * 4 and lib.miirGetWorkspaceSize(k._h) == -1   # beyond an int
 
 
 def test_backward_convolution_plans(rock):

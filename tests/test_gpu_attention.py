@@ -85,6 +85,27 @@ def test_attention_with_scale_tensor(rock, oracle, gpu, shape, bias):
     check_float(got, ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
 
 
+@pytest.mark.parametrize("t", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("shape", [(2, 200, 333, 256, 256), (1, 130, 520, 512, 512), (3, 64, 100, 40, 72)],
+                         ids=["d256", "d512", "small"])
+def test_attention_three_kernel_form(rock, oracle, gpu, t, shape):
+    """Head dimensions above 128, and every f32 problem: GEMM, row softmax, GEMM."""
+    G, sq, sk, dqk, dv = shape
+    if t != "f32" and dqk <= 128:
+        pytest.skip("the fused kernel takes this one")
+    gate = {"f16": GATE["f16"], "bf16": GATE["bf16"], "f32": (3e-5, 1e-4)}[t]
+    got, ref = _run(rock, oracle, gpu, t, G, sq, sk, dqk, dv, 1.0 / np.sqrt(dqk), 51)
+    check_float(got, ref, t, rms=gate[0], max_abs=gate[1])
+
+
+def test_attention_three_kernel_form_with_bias_and_scale_tensor(rock, oracle, gpu):
+    got, ref = _run(rock, oracle, gpu, "f16", 2, 100, 150, 256, 192, 0.07, 53, bias=True, scale_tensor=True)
+    check_float(got, ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
+    got, ref = _run(rock, oracle, gpu, "f32", 2, 96, 80, 64, 64, 0.125, 55, tQ=True, tK=False, tV=True, tO=True,
+                    bias=True)
+    check_float(got, ref, "f32", rms=3e-5, max_abs=1e-4)
+
+
 def test_attention_rows_of_p_sum_to_one(rock, oracle, gpu):
     # V = ones -> O = ones exactly up to the final rounding (size-independent property)
     got, ref = _run(rock, oracle, gpu, "f16", 2, 200, 520, 128, 128, 0.0884, 46, vones=True)
