@@ -424,48 +424,41 @@ __device__ __forceinline__ bool dl_epilogue_staged(const Params &p, const void *
 // the wave's LDS region (16 bytes per lane per group, lane-private), ONE loop
 // runs the whole epilogue on each group with the output type as a run-time
 // switch and leaves the packed result in its slot, and the results take the
-// same staged or direct store as the plain epilogue.  The loop over blocks is
-// rolled too; only the parking is specialised per block.
+// same staged or direct store as the plain epilogue.
+// Store side of the rolled epilogue, the element size a run-time value.
+// dl_rich_emit places one slot's packed results: straight into global memory
+// when the output rows cannot take 16-byte stores, else at their transposed
+// position in the wave's LDS buffer, from where dl_rich_flush writes whole rows.
+struct DlRichRow { // the lane's own output row of the current block
+  int64_t row_off, n_stride;
+  bool in_range, vec_ok;
+};
+template <int NI, typename Params>
+__device__ __forceinline__ void dl_rich_emit(const Params &p, void *Cptr, char *wbuf, const v4i &raw, int t, int es,
+                                             const DlRichRow &row, int n_wave, int lane, bool staged_ok) {
+  const int lrow = lane & 31, lgrp = lane >> 5;
+  const int nloc = (t >> 2) * 32 + (t & 3) * 8 + lgrp * 4;
+  if (!staged_ok) {
+    const int n = n_wave + nloc;
+    if (row.in_range && n < p.N)
+      store_packed4(raw, es, Cptr, row.row_off + (int64_t)n * row.n_stride, row.n_stride, n, p.N, row.vec_ok);
+    return;
+  }
+  char *dst = wbuf + lrow * (NI * 32 * es + 16) + nloc * es;
+  if (es == 4)
+    *(v4i *)dst = raw;
+  else if (es == 2)
+    *(v2i *)dst = v2i{raw[0], raw[1]};
+  else
+    *(int *)dst = raw[0];
+}
 template <int ES, int NI, typename Params>
-__device__ __forceinline__ void dl_rich_store(const Params &p, int g, void *Cptr, char *wbuf, int m_block,
-                                              int n_wave, int lane, bool staged_ok) {
+__device__ __forceinline__ void dl_rich_flush(const Params &p, int g, void *Cptr, char *wbuf, int m_block,
+                                              int n_wave, int lane) {
   constexpr int WTN = NI * 32;
   constexpr int ROWB = WTN * ES, PITCH = ROWB + 16;
   constexpr int LPR = ROWB / 16, RPI = 64 / LPR;
-  const int lrow = lane & 31, lgrp = lane >> 5;
   const int rd_row = lane / LPR, rd_cb = (lane % LPR) * 16;
-  v4i raw[NI * 4];
-#pragma unroll
-  for (int t = 0; t < NI * 4; ++t)
-    raw[t] = *(const v4i *)(wbuf + (t * 64 + lane) * 16);
-  if (!staged_ok) {
-    const int m = m_block + lrow;
-    if (m < p.M) {
-      int64_t row_off, n_stride;
-      bool vec_ok;
-      out_row_addr(p, g, m, Cptr, row_off, n_stride, vec_ok);
-#pragma unroll
-      for (int t = 0; t < NI * 4; ++t) {
-        const int n = n_wave + (t >> 2) * 32 + (t & 3) * 8 + lgrp * 4;
-        if (n < p.N)
-          store_packed4(raw[t], ES, Cptr, row_off + (int64_t)n * n_stride, n_stride, n, p.N, vec_ok);
-      }
-    }
-    return;
-  }
-  // transposition through the same buffer: every lane of the wave has read
-  // its slots (LDS operations of one wave complete in order)
-#pragma unroll
-  for (int t = 0; t < NI * 4; ++t) {
-    const int nloc = (t >> 2) * 32 + (t & 3) * 8 + lgrp * 4;
-    char *dst = wbuf + lrow * PITCH + nloc * ES;
-    if constexpr (ES == 4)
-      *(v4i *)dst = raw[t];
-    else if constexpr (ES == 2)
-      *(v2i *)dst = v2i{raw[t][0], raw[t][1]};
-    else
-      *(int *)dst = raw[t][0];
-  }
 #pragma unroll
   for (int r0 = 0; r0 < 32; r0 += RPI) {
     const int row = r0 + rd_row;
@@ -481,6 +474,59 @@ __device__ __forceinline__ void dl_rich_store(const Params &p, int g, void *Cptr
   }
 }
 
+// The residual values of one 32-row block in the accumulator layout: slot t
+// holds the 4 channels n_wave + (t/4)*32 + (t%4)*8 + lgrp*4 + {0..3} of the
+// lane's row, as raw elements packed back to back.  Whole, aligned groups
+// only (the caller checks); all loads sit in one basic block per element
+// size so that they are in flight together.
+template <int NI>
+__device__ __forceinline__ void dl_load_residual_block(v4i (&rr)[NI * 4], const char *row, int es, int n_wave,
+                                                       int lgrp) {
+  auto one = [&](auto es_const) __attribute__((always_inline)) {
+    constexpr int ES = decltype(es_const)::value;
+#pragma unroll
+    for (int t = 0; t < NI * 4; ++t) {
+      const int n = n_wave + (t >> 2) * 32 + (t & 3) * 8 + lgrp * 4;
+      const char *src = row + n * ES;
+      v4i r = {0, 0, 0, 0};
+      if constexpr (ES == 4)
+        r = *(const v4i *)src;
+      else if constexpr (ES == 2) {
+        const v2i x = *(const v2i *)src;
+        r[0] = x[0];
+        r[1] = x[1];
+      } else
+        r[0] = *(const int *)src;
+      rr[t] = r;
+    }
+  };
+  if (es == 4)
+    one(std::integral_constant<int, 4>{});
+  else if (es == 2)
+    one(std::integral_constant<int, 2>{});
+  else
+    one(std::integral_constant<int, 1>{});
+}
+
+// 4 packed elements of the output type widened (the inverse of epilogue_pack4)
+__device__ __forceinline__ void unpack4_rt(const v4i &raw, int od, float (&f)[4]) {
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const uint32_t h = (uint32_t)raw[k >> 1] >> (16 * (k & 1));
+    const uint8_t b = (uint8_t)((uint32_t)raw[0] >> (8 * k));
+    const int word = raw[k]; // a copy: bit-casting the vector element itself reads element 0
+    switch (od) {
+    case ROCK_F32: f[k] = __builtin_bit_cast(float, word); break;
+    case ROCK_F16: f[k] = (float)__builtin_bit_cast(_Float16, (uint16_t)h); break;
+    case ROCK_BF16: f[k] = __builtin_bit_cast(float, h << 16); break;
+    case ROCK_I8: f[k] = (float)(int8_t)b; break;
+    case ROCK_FP8: f[k] = e4m3fn_to_f32(b); break;
+    case ROCK_BF8: f[k] = e5m2_to_f32(b); break;
+    default: f[k] = (float)word; break;
+    }
+  }
+}
+
 template <int DT, int MI, int NI, int NWAVES, int LDS_BYTES, typename Params>
 __device__ __forceinline__ void dl_epilogue_rich(typename MmaTraits<DT>::Acc (&acc)[MI][NI], const Params &p, int g,
                                                  void *Cptr, const void *aux, const void *res, int m_wave,
@@ -489,87 +535,167 @@ __device__ __forceinline__ void dl_epilogue_rich(typename MmaTraits<DT>::Acc (&a
   constexpr int WTN = NI * 32;
   constexpr int WBUF = 32 * (WTN * 4 + 16);
   static_assert(NWAVES * WBUF <= LDS_BYTES, "staging buffers must fit in the operand stages");
-  static_assert(NI * 4 * 1024 <= WBUF, "parked accumulators must fit in the wave's staging buffer");
+  static_assert(NI * 4 * 1024 <= WBUF, "parked values must fit in the wave's staging buffer");
   using Acc4 = decltype(__builtin_shufflevector(acc[0][0], acc[0][0], 0, 1, 2, 3));
   const RockEpilogue &e = p.epi;
   const int lrow = lane & 31, lgrp = lane >> 5;
   char *wbuf = lds + wave * WBUF;
   const int od = e.out_dtype;
+  const int es = out_elem_size(od);
   const bool slow = activation_is_slow(e);
-#pragma unroll 1
-  for (int i = 0; i < MI; ++i) {
-    // park block i: the only step that names registers
-    static_for<MI>([&](auto ic) __attribute__((always_inline)) {
-      if (i == ic.value) {
+  const bool int_out = Tr::INT_ACC && od == ROCK_I32;
+  // Unrolled over the blocks at compile time (a loop the compiler leaves
+  // rolled would index the accumulator registers dynamically, which sends them
+  // through scratch memory); the bulk of each block's code is the rolled slot
+  // loop below.
+  // Per block: the lane's own row and its residual values.  Rows whose groups
+  // of four are whole and aligned (the usual case) load them as vectors, all
+  // in flight together and one block ahead of their use; otherwise element by
+  // element in the slot loop.
+  DlRichRow rows[MI];
+  bool res_vecs[MI];
+  v4i rr2[2][NI * 4];
+  auto prefetch = [&](auto ibc) __attribute__((always_inline)) {
+    constexpr int ib = decltype(ibc)::value;
+    const int m = m_wave + ib * 32 + lrow;
+    DlRichRow row{0, 1, m < p.M, false};
+    if (row.in_range)
+      out_row_addr(p, g, m, Cptr, row.row_off, row.n_stride, row.vec_ok);
+    bool rv = false;
+    if (e.residual_op && row.in_range) {
+      const char *rowp = (const char *)res + row.row_off * es;
+      rv = row.n_stride == 1 && (((uintptr_t)rowp) & (uintptr_t)(4 * es - 1)) == 0 && n_wave + WTN <= p.N;
+      if (rv)
+        dl_load_residual_block<NI>(rr2[ib & 1], rowp, es, n_wave, lgrp);
+    }
+    rows[ib] = row;
+    res_vecs[ib] = rv;
+  };
+  prefetch(std::integral_constant<int, 0>{});
+  static_for<MI>([&](auto ic) __attribute__((always_inline)) {
+    constexpr int i = decltype(ic)::value;
+    if constexpr (i + 1 < MI)
+      prefetch(std::integral_constant<int, i + 1>{});
+    const DlRichRow row = rows[i];
+    const bool res_vec = res_vecs[i];
+    v4i(&rr)[NI * 4] = rr2[i & 1];
+    const bool with_res = e.residual_op && row.in_range;
+    const int64_t res_off = row.row_off, res_ns = row.n_stride;
+    // Steps 1-3 where the accumulators sit.  With a clamp-type activation and
+    // no ragged residual in this wave the results are finished in registers;
+    // otherwise they are parked in LDS as f32 and finished by the rolled slot
+    // loop, the single copy of the activation routines.
+    const bool ragged = with_res && !res_vec;
+    const bool park = !int_out && (slow || __builtin_amdgcn_ballot_w64(ragged) != 0);
+    const bool park_int = int_out && __builtin_amdgcn_ballot_w64(ragged) != 0;
 #pragma unroll
-        for (int j = 0; j < NI; ++j) {
+    for (int j = 0; j < NI; ++j) {
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            Acc4 a4 = {acc[ic.value][j][4 * q + 0], acc[ic.value][j][4 * q + 1], acc[ic.value][j][4 * q + 2],
-                       acc[ic.value][j][4 * q + 3]};
-            *(Acc4 *)(wbuf + ((j * 4 + q) * 64 + lane) * 16) = a4;
+      for (int q = 0; q < 4; ++q) {
+        const int t = j * 4 + q;
+        const int n = n_wave + j * 32 + q * 8 + lgrp * 4;
+        Acc4 a4 = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+        char *slot = wbuf + (t * 64 + lane) * 16;
+        if (int_out) {
+          if constexpr (Tr::INT_ACC) {
+            v4i v = epilogue_convert4<true, ROCK_I32>(a4, e, aux, n, p.N);
+            if (res_vec) {
+#pragma unroll
+              for (int k = 0; k < 4; ++k)
+                v[k] = e.residual_op == ROCK_RES_ADD ? v[k] + rr[t][k] : v[k] * rr[t][k];
+            }
+            if (park_int)
+              *(v4i *)slot = v;
+            else
+              dl_rich_emit<NI>(p, Cptr, wbuf, v, t, es, row, n_wave, lane, staged_ok);
+          }
+        } else {
+          float v[4];
+          epilogue_affine4<Tr::INT_ACC, ROCK_DTYPE_COUNT>(a4, e, aux, n, p.N, nullptr, 0, 1, v);
+          if (res_vec) {
+            float rf[4];
+            unpack4_rt(rr[t], od, rf);
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+              v[k] = e.residual_op == ROCK_RES_ADD ? v[k] + rf[k] : v[k] * rf[k];
+          }
+          if (park) {
+            *(v4f *)slot = v4f{v[0], v[1], v[2], v[3]};
+          } else {
+            if (e.activation) {
+#pragma unroll
+              for (int k = 0; k < 4; ++k)
+                v[k] = activation_fast(v[k], e);
+            }
+            dl_rich_emit<NI>(p, Cptr, wbuf, epilogue_pack4_rt(v, od, e), t, es, row, n_wave, lane, staged_ok);
           }
         }
       }
-    });
-    const int m = m_wave + i * 32 + lrow;
-    const void *res_row = nullptr;
-    int64_t row_off = 0, n_stride = 1;
-    if (m < p.M && e.residual_op) {
-      bool unused;
-      out_row_addr(p, g, m, Cptr, row_off, n_stride, unused);
-      res_row = res;
     }
+    if (park || park_int) {
+      if (ragged) { // ragged or unaligned rows: one residual element at a time
 #pragma unroll 1
-    for (int t = 0; t < NI * 4; ++t) {
-      char *slot = wbuf + (t * 64 + lane) * 16;
-      const int n = n_wave + (t >> 2) * 32 + (t & 3) * 8 + lgrp * 4;
-      const Acc4 a4 = *(const Acc4 *)slot;
-      const int64_t res_off = row_off + (int64_t)n * n_stride;
-      if (Tr::INT_ACC && od == ROCK_I32) {
-        if constexpr (Tr::INT_ACC)
-          *(v4i *)slot = epilogue_convert4<true, ROCK_I32>(a4, e, aux, n, p.N, res_row, res_off, n_stride);
-        continue;
-      }
-      float v[4];
-      epilogue_affine4<Tr::INT_ACC, ROCK_DTYPE_COUNT>(a4, e, aux, n, p.N, nullptr, 0, 1, v);
-      if (res_row) {
-        *(v4f *)slot = v4f{v[0], v[1], v[2], v[3]};
+        for (int t = 0; t < NI * 4; ++t) {
+          char *slot = wbuf + (t * 64 + lane) * 16;
+          const int n = n_wave + (t >> 2) * 32 + (t & 3) * 8 + lgrp * 4;
 #pragma unroll 1
-        for (int r = 0; r < 4; ++r) {
-          if (n + r < p.N) {
-            float *f = (float *)slot + r;
-            const float rv = load_out_elem_rt(res_row, res_off + r * n_stride, od);
-            *f = e.residual_op == ROCK_RES_ADD ? *f + rv : *f * rv;
+          for (int r = 0; r < 4; ++r) {
+            if (n + r >= p.N)
+              continue;
+            const int64_t idx = res_off + (int64_t)(n + r) * res_ns;
+            if (int_out) {
+              int *f = (int *)slot + r;
+              const int rv = ((const int *)res)[idx];
+              *f = e.residual_op == ROCK_RES_ADD ? *f + rv : *f * rv;
+            } else {
+              float *f = (float *)slot + r;
+              const float rv = load_out_elem_rt(res, idx, od);
+              *f = e.residual_op == ROCK_RES_ADD ? *f + rv : *f * rv;
+            }
           }
         }
-        const v4f x = *(const v4f *)slot;
-        v[0] = x[0]; v[1] = x[1]; v[2] = x[2]; v[3] = x[3];
       }
-      if (slow) { // one copy of the routine: loop over the slot, not over registers
-        *(v4f *)slot = v4f{v[0], v[1], v[2], v[3]};
+      if (!int_out) {
 #pragma unroll 1
-        for (int r = 0; r < 4; ++r) {
-          float *f = (float *)slot + r;
-          *f = activation_slow(*f, e.activation);
-        }
-        const v4f x = *(const v4f *)slot;
-        v[0] = x[0]; v[1] = x[1]; v[2] = x[2]; v[3] = x[3];
-      } else if (e.activation) {
+        for (int t = 0; t < NI * 4; ++t) {
+          char *slot = wbuf + (t * 64 + lane) * 16;
+          if (slow) {
+#pragma unroll 1
+            for (int r = 0; r < 4; ++r) {
+              float *f = (float *)slot + r;
+              *f = activation_slow(*f, e.activation);
+            }
+          }
+          const v4f x = *(const v4f *)slot;
+          float v[4] = {x[0], x[1], x[2], x[3]};
+          if (!slow && e.activation) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          v[r] = activation_fast(v[r], e);
+            for (int r = 0; r < 4; ++r)
+              v[r] = activation_fast(v[r], e);
+          }
+          *(v4i *)slot = epilogue_pack4_rt(v, od, e);
+        }
       }
-      *(v4i *)slot = epilogue_pack4_rt(v, od, e);
+      // results back into registers, then to their store positions: every lane
+      // has read its slots before any overwrites them (LDS operations of one
+      // wave complete in order)
+      v4i raw[NI * 4];
+#pragma unroll
+      for (int t = 0; t < NI * 4; ++t)
+        raw[t] = *(const v4i *)(wbuf + (t * 64 + lane) * 16);
+#pragma unroll
+      for (int t = 0; t < NI * 4; ++t)
+        dl_rich_emit<NI>(p, Cptr, wbuf, raw[t], t, es, row, n_wave, lane, staged_ok);
     }
-    const int es = out_elem_size(od);
-    if (es == 4)
-      dl_rich_store<4, NI>(p, g, Cptr, wbuf, m_wave + i * 32, n_wave, lane, staged_ok);
-    else if (es == 2)
-      dl_rich_store<2, NI>(p, g, Cptr, wbuf, m_wave + i * 32, n_wave, lane, staged_ok);
-    else
-      dl_rich_store<1, NI>(p, g, Cptr, wbuf, m_wave + i * 32, n_wave, lane, staged_ok);
-  }
+    if (staged_ok) {
+      if (es == 4)
+        dl_rich_flush<4, NI>(p, g, Cptr, wbuf, m_wave + i * 32, n_wave, lane);
+      else if (es == 2)
+        dl_rich_flush<2, NI>(p, g, Cptr, wbuf, m_wave + i * 32, n_wave, lane);
+      else
+        dl_rich_flush<1, NI>(p, g, Cptr, wbuf, m_wave + i * 32, n_wave, lane);
+    }
+  });
 }
 
 // RICH kernels are separate instantiations (kernel name suffix "_e") so that

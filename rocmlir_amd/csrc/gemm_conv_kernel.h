@@ -282,7 +282,7 @@ __device__ __forceinline__ float activation_fast(float v, const RockEpilogue &e)
 
 __device__ __forceinline__ float activation_slow(float v, int activation) {
   switch (activation) { // uniform
-  case ROCK_ACT_SIGMOID: return 1.0f / (1.0f + expf(-v));
+  case ROCK_ACT_SIGMOID: return __frcp_rn(1.0f + __expf(-v)); // hardware exp2 and reciprocal: ~1e-7 relative
   case ROCK_ACT_TANH: return tanhf(v);
   case ROCK_ACT_ERF: return erff(v);
   case ROCK_ACT_GELU: return 0.5f * v * (1.0f + erff(v * 0.70710678118654752f));
@@ -340,6 +340,20 @@ template <bool INT_ACC, int OD, typename Acc4>
 __device__ __forceinline__ void epilogue_affine4(const Acc4 &acc, const RockEpilogue &e, const void *aux,
                                                  int n0, int n_limit, const void *res, int64_t res_off,
                                                  int64_t res_ns, float (&v)[4]) {
+  // the four bias values as one 16-byte load where the group is whole (n0 is a
+  // multiple of 4 and the vector starts on a 16-byte boundary like its tensor)
+  float b4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (e.has_bias) {
+    if (n0 + 3 < n_limit) {
+      const v4f b = *(const v4f *)((const float *)aux + n0);
+      b4[0] = b[0]; b4[1] = b[1]; b4[2] = b[2]; b4[3] = b[3];
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n0 + r < n_limit)
+          b4[r] = ((const float *)aux)[n0 + r];
+    }
+  }
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     float f;
@@ -347,8 +361,8 @@ __device__ __forceinline__ void epilogue_affine4(const Acc4 &acc, const RockEpil
       f = ((float)(int)acc[r] - (float)e.zero_point) * e.scale;
     else
       f = (float)acc[r] * e.scale;
-    if (e.has_bias && n0 + r < n_limit)
-      f = f + ((const float *)aux)[n0 + r];
+    if (e.has_bias)
+      f = f + b4[r];
     if (res && n0 + r < n_limit) {
       const float rv = load_out_elem<OD>(res, res_off + r * res_ns);
       f = e.residual_op == ROCK_RES_ADD ? f + rv : f * rv;

@@ -374,8 +374,10 @@ std::string forced_tile(const OptMap &o) {
 // accumulators, and ("_e") with the rolled epilogue that a residual tensor or a
 // transcendental activation needs.  The element-wise kernels handle both in
 // one.
-const char *rich_suffix(const RockEpilogue &e, bool tiled_kernel) {
-  return tiled_kernel && (e.residual_op != ROCK_RES_NONE || e.activation > ROCK_ACT_CLIP) ? "_e" : "";
+const char *rich_suffix(const RockEpilogue &e, bool tiled_kernel, const OptMap &o) {
+  // "-rolled_epilogue true" asks for the twin regardless (it handles every epilogue)
+  return tiled_kernel && (e.residual_op != ROCK_RES_NONE || e.activation > ROCK_ACT_CLIP ||
+                          bool_or(o, "rolled_epilogue", false)) ? "_e" : "";
 }
 
 // The contraction kernels take five pointers: two operands, the output, the
@@ -437,7 +439,7 @@ bool plan_gemm_kernel(Handle *h, RockGemmParams &p, int code, int es, const OptM
   if (split_k > 1)
     h->block_size = 256;
   h->kernel_name = std::string("rock_gemm_") + operand_name(code) + tile->suffix + (storage ? storage : "") +
-                   rich_suffix(p.epi, tiled);
+                   rich_suffix(p.epi, tiled, o);
   h->blob_name = std::string("gemm_") + operand_name(code);
   set_contraction_pointers(h, p.epi);
   h->perf_config = perf_string(*tile, es);
@@ -1429,7 +1431,7 @@ Handle *make_conv(const OptMap &o) {
     tile = fast ? pick_tile(Mg, k, (int)g, true, "") : &kGenericTile;
   apply_tile_grid(*tile, Mg, k, (int)g, p.tiles_m, p.tiles_n, p.group_m, p.xcd_remap,
                   h->block_size, h->grid_size);
-  h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + tile->suffix + rich_suffix(p.epi, fast);
+  h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + tile->suffix + rich_suffix(p.epi, fast, o);
   h->blob_name = std::string("gemm_") + dtype_name(ti);
   h->num_pointers = 5;
   if (!planned)
@@ -1475,7 +1477,7 @@ Handle *make_conv(const OptMap &o) {
       p.xcd_remap = total >= 2 * kNumXCD ? 1 : 0;
       h->block_size = 512;
       h->grid_size = (uint32_t)total;
-      h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + "_direct224" + rich_suffix(p.epi, true);
+      h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + "_direct224" + rich_suffix(p.epi, true, o);
       char buf[96];
       std::snprintf(buf, sizeof buf, "v2:224,128,8,224,32,%d,1,1,1", 16 / es);
       h->perf_config = buf;
