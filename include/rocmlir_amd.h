@@ -66,7 +66,10 @@ typedef void *MiirHandle;
  * reference's rocmlir-gen flag names (rocmlir-gen.cpp:90-561): t,
  * out_datatype, g, m, k, n, transA, transB, transC; g, seq_len_q, seq_len_k,
  * head_dim_qk, head_dim_v, transQ, transK, transV, transO, with-attn-bias,
- * with-attn-scale (pointer order Q, K, V, [scale tensor], bias slot, O).
+ * with-attn-scale (pointer order Q, K, V, [scale tensor], bias slot, O);
+ * attention types f16, bf16, f32, and i8 = int8 Q and K with f16 V / O, the
+ * scores dequantised as (acc - zero_point) * scale.  Head dimensions above
+ * 128, f32 and i8 run as three kernels over a score workspace.
  * Epilogue keys (all optional): scale, zero_point, quant_scale,
  * out_zero_point, bias, relu; and the element-wise operations MIGraphX fuses
  * behind a contraction (MIGraphXToTosa.cpp:1009-1016, 1089-1100, 1283-1295):

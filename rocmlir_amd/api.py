@@ -509,7 +509,7 @@ def conv2d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize,
     return out
 
 
-def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, transQ=False, transK=False,
+def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, zero_point=0, transQ=False, transK=False,
               transV=False, transO=False, out=None, stream=None):
     """O = softmax(scale * scale_tensor * Q K + bias) V (bias and scale_tensor
     optional [G,seq_q,seq_k] tensors, rocmlir-gen's -with-attn-bias /
@@ -517,7 +517,8 @@ def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, transQ=False,
     conventions (rocmlir-gen.cpp:2149-2200): q [G,seq_q,d] ([G,d,seq_q] if
     transQ); k [G,d,seq_k] ([G,seq_k,d] if transK -- the usual row-major keys);
     v [G,seq_k,dv] ([G,dv,seq_k] if transV); result [G,seq_q,dv]
-    ([G,dv,seq_q] if transO)."""
+    ([G,dv,seq_q] if transO).  int8 q and k (with f16 v, bias, scale_tensor)
+    select the quantised first GEMM: the scores are (acc - zero_point) * scale."""
     import torch
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     G = q.shape[0]
@@ -535,10 +536,12 @@ def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, transQ=False,
         opts += " -with-attn-bias true"
     if scale_tensor is not None:
         opts += " -with-attn-scale true"
+    if zero_point:
+        opts += " -zero_point %d" % zero_point
     kern = _program(opts)   # one fused kernel, or three for head dimensions above 128 and f32
     shape = (G, dv, sq) if transO else (G, sq, dv)
     if out is None:
-        out = torch.empty(shape, dtype=q.dtype, device=q.device)
+        out = torch.empty(shape, dtype=v.dtype, device=q.device)
     if scale_tensor is None:
         kern.launch(q, k, v, bias, out, stream=stream)
     else:

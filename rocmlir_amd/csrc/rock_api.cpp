@@ -1495,6 +1495,13 @@ Handle *make_conv(const OptMap &o) {
 // same three steps (rocmlir-gen.cpp:2565-2620).
 Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, int64_t sk, int64_t dqk, int64_t dv,
                                bool tQ, bool tK, bool tV, bool tO, bool has_bias, bool has_scale_t) {
+  // "-t i8": Q and K are int8, their product is dequantised before the softmax
+  // ((acc - zero_point) * scale, the scalars rocmlir-gen passes as [1,1,1]
+  // tensors, rocmlir-gen.cpp:2173-2184, 2353-2367); V, the pre-softmax tensors
+  // and O are f16
+  const int tq = ty;
+  if (ty == ROCK_I8)
+    ty = ROCK_F16;
   const int es = dtype_size(ty);
   const int kid = (int)int_or(o, "kernel_id", 0);
   if (kid < 0 || kid > 2) {
@@ -1543,6 +1550,7 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
       gp.b_gs = sk * dqk; gp.b_ns = tK ? dqk : 1; gp.b_ks = tK ? 1 : sk;
       gp.c_gs = sq * sk; gp.c_ms = sk; gp.c_ns = 1;
       default_epilogue(gp.epi, ROCK_F32);
+      gp.epi.zero_point = (int32_t)int_or(o, "zero_point", 0); // i8: scores leave as float(acc) - zero_point
     } else { // O[g,i,e] = sum_j P[g,i,j] V[g,j,e]
       gp.M = (int)sq; gp.N = (int)dv; gp.K = (int)sk;
       gp.a_gs = sq * sk * pitch_p; gp.a_ms = sk * pitch_p; gp.a_ks = 1;
@@ -1550,7 +1558,8 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
       gp.c_gs = sq * dv; gp.c_ms = tO ? 1 : dv; gp.c_ns = tO ? sq : 1;
       default_epilogue(gp.epi, ty);
     }
-    plan_gemm_kernel(h, gp, operand_code(ty, ty), es, o);
+    const int tg = kid == 0 ? tq : ty;
+    plan_gemm_kernel(h, gp, operand_code(tg, tg), dtype_size(tg), o);
     if (kid == 0)
       h->ptr_map = {{0, 0}, {1, 0}, {i_ws, 0}, {-1, 0}, {-1, 0}};
     else
@@ -1561,7 +1570,7 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
     h->epi = &reinterpret_cast<RockGemmParams *>(h->params.data())->epi;
     std::ostringstream key;
     auto tf = [](bool b) { return b ? "true" : "false"; };
-    key << h->arch << '\t' << int_or(o, "num_cu", kNumCU) << '\t' << "-t " << dtype_name(ty) << " -transQ " << tf(tQ)
+    key << h->arch << '\t' << int_or(o, "num_cu", kNumCU) << '\t' << "-t " << dtype_name(tq) << " -transQ " << tf(tQ)
         << " -transK " << tf(tK) << " -transV " << tf(tV) << " -transO " << tf(tO) << " -g " << G << " -seq_len_q "
         << sq << " -seq_len_k " << sk << " -head_dim_qk " << dqk << " -head_dim_v " << dv;
     h->problem_key = key.str();
@@ -1576,8 +1585,8 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
 Handle *make_attention(const OptMap &o) {
   std::string t = str_or(o, "t", "f16");
   int ty = parse_dtype(t);
-  if (ty != ROCK_F16 && ty != ROCK_BF16 && ty != ROCK_F32) {
-    set_error("attention: f16, bf16 and f32 kernels are built ('" + t + "' requested)");
+  if (ty != ROCK_F16 && ty != ROCK_BF16 && ty != ROCK_F32 && ty != ROCK_I8) {
+    set_error("attention: f16, bf16, f32 and i8 (quantised first GEMM) kernels are built ('" + t + "' requested)");
     return nullptr;
   }
   int64_t G = int_or(o, "g", 1), sq, sk, dqk, dv;
@@ -1593,7 +1602,7 @@ Handle *make_attention(const OptMap &o) {
   // "-with-attn-scale": a full [G, seq_q, seq_k] tensor multiplied into the
   // scores before the softmax (rocmlir-gen.cpp:2185-2196), besides the scalar "-scale"
   bool has_scale_t = bool_or(o, "with-attn-scale", false);
-  if (ty == ROCK_F32 || dqk > 128 || dv > 128)
+  if (ty == ROCK_F32 || ty == ROCK_I8 || dqk > 128 || dv > 128)
     return make_attention_unfused(o, ty, G, sq, sk, dqk, dv, tQ, tK, tV, tO, has_bias, has_scale_t);
 
   auto *h = new Handle;

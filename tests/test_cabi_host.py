@@ -77,7 +77,7 @@ def test_null_handle_behaviour(rock):
     "--operation gemm --arch gfx950 -t f16 -out_datatype i32 -m 4 -n 4 -k 4",  # float in, int out
     "--operation gemm --arch gfx950 -t f16_i8 -m 4 -n 4 -k 4",
     "--operation attention --arch gfx950 -t f16 -g 1 -seq_len_q 8 -seq_len_k 8 -head_dim_qk 8",
-    "--operation attention --arch gfx950 -t i8 -g 1 -seq_len_q 8 -seq_len_k 8 -head_dim_qk 64 -head_dim_v 8",
+    "--operation attention --arch gfx950 -t fp8 -g 1 -seq_len_q 8 -seq_len_k 8 -head_dim_qk 64 -head_dim_v 8",
     "--operation attention --arch gfx950 -t f16 -g 1 -seq_len_q 8 -seq_len_k 8 -head_dim_qk 256 -head_dim_v 8 "
     "--kernel_id 3",
     "--operation transpose --arch gfx950",
@@ -251,6 +251,10 @@ def test_attention_as_three_kernels(rock):
         assert ks[2].kernel_name.startswith("rock_gemm_%s_" % t) and ks[2].kernel_name.endswith("_fast_nn")
         assert all(k.kernel_count == 3 and k.workspace_bytes == 16384 * 16384 * 4 and k.caller_pointers == 6
                    for k in ks)
+    # int8 first GEMM: int8 contraction into f32 scores, f16 from there on
+    q8 = [rock.RockKernel("-operation attention -arch gfx950 -t i8 -g 2 -seq_len_q 128 -seq_len_k 128 -head_dim_qk 64 "
+                          "-head_dim_v 64 -transK true -zero_point 3 -scale 0.001 -kernel_id %d" % i) for i in range(3)]
+    assert q8[0].kernel_name.startswith("rock_gemm_i8_") and q8[2].kernel_name.startswith("rock_gemm_f16_")
     lib = rock.load_library()
     k = rock.RockKernel((vae % "f16").replace("-g 1 ", "-g 4 "))
     assert k.workspace_bytes == 4 * 16384 * 16384 * 4 and lib.miirGetWorkspaceSize(k._h) == -1   # beyond an int

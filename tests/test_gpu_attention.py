@@ -106,6 +106,33 @@ def test_attention_three_kernel_form_with_bias_and_scale_tensor(rock, oracle, gp
     check_float(got, ref, "f32", rms=3e-5, max_abs=1e-4)
 
 
+@pytest.mark.parametrize("shape", [(1, 64, 64, 32, 32), (2, 100, 130, 64, 48), (1, 200, 77, 256, 64)],
+                         ids=["mixr", "ragged", "d256"])
+@pytest.mark.parametrize("bias", [False, True])
+def test_attention_int8_first_gemm(rock, oracle, gpu, shape, bias):
+    """-t i8 (mixr-attention-first-gemm-i8-f16.mlir): Q K^T in int8 -> int32,
+    dequantised with a zero point and an f16-valued scale before the softmax,
+    f16 V and output.  The oracle gets the same scores through a bias that
+    carries -zero_point * scale."""
+    G, sq, sk, dqk, dv = shape
+    rng = np.random.default_rng(57)
+    Q = rng.integers(-128, 128, (G, sq, dqk)).astype(np.int8)
+    K = rng.integers(-128, 128, (G, sk, dqk)).astype(np.int8)
+    V = rng.standard_normal((G, sk, dv)).astype(np.float32)
+    rv, Vq = quantise(V, "f16")
+    zp, scale = 37, float(np.float16(3.0e-4))
+    braw = bq = None
+    if bias:
+        braw, bq = quantise(rng.standard_normal((G, sq, sk)).astype(np.float32), "f16")
+    out = rock.attention(torch.from_numpy(Q).to(gpu), torch.from_numpy(K).to(gpu), to_gpu(rv, "f16", gpu),
+                         scale=scale, zero_point=zp, bias=to_gpu(braw, "f16", gpu) if bias else None, transK=True)
+    torch.cuda.synchronize()
+    shift = np.full((G, sq, sk), -zp * scale, np.float32) + (bq.reshape(G, sq, sk) if bias else 0.0)
+    ref = oracle.attention(Q.astype(np.float32), K.astype(np.float32), Vq, G, sq, sk, dqk, dv, scale=scale,
+                           bias_t=shift.astype(np.float32), transK=True)
+    check_float(to_f32(out, "f16"), ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
+
+
 def test_attention_rows_of_p_sum_to_one(rock, oracle, gpu):
     # V = ones -> O = ones exactly up to the final rounding (size-independent property)
     got, ref = _run(rock, oracle, gpu, "f16", 2, 200, 520, 128, 128, 0.0884, 46, vones=True)
