@@ -406,7 +406,7 @@ def gemm(a, b, *, transA=False, transB=False, transC=False, out_dtype=None,
          scale=None, zero_point=0, bias=None, relu=False, quant_scale=None,
          out_zero_point=0, activation=None, clip=None, residual=None,
          residual_op="add", out=None, perf_config=None, stream=None,
-         info=None):
+         info=None, split_k=True):
     """C = epilogue(A x B) with the reference's storage conventions
     (rocmlir-gen.cpp:2058-2080): a is [G,M,K] ([G,K,M] if transA), b is
     [G,K,N] ([G,N,K] if transB), result [G,M,N] ([G,N,M] if transC).
@@ -435,24 +435,28 @@ def gemm(a, b, *, transA=False, transB=False, transC=False, out_dtype=None,
         opts += " -out_datatype %s" % out_dtype
     if perf_config:
         opts += " -perf_config %s" % perf_config
+    if not split_k:
+        opts += " -split_k false"
     opts += _epilogue_flags(scale, zero_point, bias, relu, quant_scale,
                             out_zero_point, activation, clip, residual,
                             residual_op)
-    k = _kernel(opts)
+    prog = _program(opts)   # one kernel, or two when the reduction is split over blocks
+    k = prog.kernels[0]
     if info is not None:
         info["kernel_name"] = k.kernel_name
         info["perf_config"] = k.perf_config
+        info["kernels"] = [x.kernel_name for x in prog.kernels]
     if out_dtype is None:
         out_dtype = {"i8": "i32", "fp8": "f32", "bf8": "f32"}.get(ta, ta)
     shape = (G, N, M) if transC else (G, M, N)
     if out is None:
         out = torch.empty(shape, dtype=_torch_dtype(out_dtype), device=a.device)
     if residual is None:
-        k.launch(a3, b3, out, bias, stream=stream)
+        prog.launch(a3, b3, out, bias, stream=stream)
     else:
         if residual.dtype != out.dtype or residual.numel() != out.numel():
             raise RockError("gemm: the residual must have the result's type and size")
-        k.launch(a3, b3, out, bias, residual.contiguous(), stream=stream)
+        prog.launch(a3, b3, out, bias, residual.contiguous(), stream=stream)
     return out if a.dim() == 3 else out.squeeze(0)
 
 

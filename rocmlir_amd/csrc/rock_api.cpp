@@ -370,6 +370,17 @@ std::string forced_tile(const OptMap &o) {
   return "";
 }
 
+void default_epilogue(RockEpilogue &e, int out_dtype) {
+  std::memset(&e, 0, sizeof e);
+  e.scale = 1.0f;
+  e.inv_quant_scale = 1.0f;
+  e.out_dtype = out_dtype;
+  e.act_lo = -INFINITY;
+  e.act_hi = INFINITY;
+}
+
+int64_t align256(int64_t bytes) { return (bytes + 255) / 256 * 256; }
+
 // The tiled kernels exist twice: with the plain epilogue unrolled over their
 // accumulators, and ("_e") with the rolled epilogue that a residual tensor or a
 // transcendental activation needs.  The element-wise kernels handle both in
@@ -508,6 +519,80 @@ Handle *make_gemm(const OptMap &o) {
 
   plan_gemm_kernel(h, p, code, dtype_size(ta), o);
   // problem key (RockTuningImpl.cpp:808-862)
+  auto set_key = [&](Handle *hh) {
+    std::ostringstream k;
+    k << hh->arch << '\t' << int_or(o, "num_cu", kNumCU) << '\t' << "-t " << operand_name(code)
+      << " -out_datatype " << dtype_name(tc) << " -transA " << (tA ? "true" : "false")
+      << " -transB " << (tB ? "true" : "false") << " -g " << G << " -m " << M << " -n " << N
+      << " -k " << K;
+    hh->problem_key = k.str();
+  };
+  // Split of the reduction over blocks.  A single floating-point GEMM with few
+  // output tiles and a long K leaves most of the chip idle; its K range is cut
+  // into S batch entries writing f32 partial results into a workspace, which
+  // the reduction kernel adds up in split order (the reference reaches the same
+  // parallelism with atomic adds into a pre-filled C, RockTuningImpl.cpp:962-1008,
+  // Rock.cpp:167-198).  Only with the identity epilogue, which commutes with the sum.
+  {
+    const int es = dtype_size(ta);
+    const RockEpilogue &e = p.epi;
+    const bool identity = e.scale == 1.0f && !e.has_bias && e.activation == ROCK_ACT_NONE &&
+                          e.residual_op == ROCK_RES_NONE && (tc == ROCK_F32 || tc == ROCK_F16 || tc == ROCK_BF16);
+    const bool tiled = h->kernel_name.find("_fast") != std::string::npos;
+    const int64_t tiles64 = (int64_t)ceil_div(M, 64) * ceil_div(N, 64);
+    int64_t S = 1;
+    if (G == 1 && is_float_in(ta) && is_float_in(tb) && identity && tiled && tiles64 * 4 <= kNumCU &&
+        forced_tile(o).empty() && bool_or(o, "split_k", true)) {
+      const int64_t want = std::min<int64_t>(2 * kNumCU / tiles64, K / 512);
+      for (int64_t d = want; d >= 2; --d)
+        if (K % d == 0 && ((K / d) * es) % 64 == 0) {
+          S = d;
+          break;
+        }
+    }
+    if (S > 1) {
+      const int kid = (int)int_or(o, "kernel_id", 0);
+      if (kid < 0 || kid > 1) {
+        set_error("gemm: kernel_id out of range");
+        delete h;
+        return nullptr;
+      }
+      const int64_t Ks = K / S, cstride_m = p.c_ms, cstride_n = p.c_ns;
+      if (kid == 0) {
+        p.G = (int)S; p.K = (int)Ks;
+        p.a_gs = Ks * p.a_ks; p.b_gs = Ks * p.b_ks;
+        p.c_gs = M * N; p.c_ms = N; p.c_ns = 1;
+        default_epilogue(p.epi, ROCK_F32);
+        plan_gemm_kernel(h, p, code, es, o);
+        h->ptr_map = {{0, 0}, {1, 0}, {4, 0}, {-1, 0}, {-1, 0}};
+        set_key(h);
+      } else {
+        RockReduceParams r;
+        std::memset(&r, 0, sizeof r);
+        r.split_stride = M * N;
+        r.size[0] = 1; r.size[1] = 1; r.size[2] = (int)M; r.size[3] = (int)N;
+        r.dst_stride[2] = cstride_m; r.dst_stride[3] = cstride_n;
+        r.splits = (int)S;
+        r.out_dtype = tc;
+        h->op = OP_RELAYOUT;
+        h->epi = nullptr;
+        h->params.assign(sizeof r, 0);
+        std::memcpy(h->params.data(), &r, sizeof r);
+        h->kernel_name = "rock_reduce_splits";
+        h->blob_name = "relayout";
+        h->block_size = 256;
+        h->grid_size = (uint32_t)((M * N + 255) / 256);
+        h->num_pointers = 2;
+        h->perf_config = "";
+        h->ptr_map = {{4, 0}, {2, 0}};
+        h->problem_key = "reduction of the split partial sums";
+      }
+      h->kernel_count = 2;
+      h->workspace_bytes = (size_t)align256(S * M * N * 4);
+      h->caller_pointers = 5; // A, B, C, unused, workspace
+      return h;
+    }
+  }
   {
     std::ostringstream k;
     k << h->arch << '\t' << int_or(o, "num_cu", kNumCU) << '\t' << "-t " << operand_name(code)
@@ -750,15 +835,6 @@ std::string conv_problem_key(const Handle *h, const OptMap &o, const ConvProblem
   return key.str();
 }
 
-void default_epilogue(RockEpilogue &e, int out_dtype) {
-  std::memset(&e, 0, sizeof e);
-  e.scale = 1.0f;
-  e.inv_quant_scale = 1.0f;
-  e.out_dtype = out_dtype;
-  e.act_lo = -INFINITY;
-  e.act_hi = INFINITY;
-}
-
 Handle *conv_handle_from_view(const RockConvParams &q, int ti, const OptMap &o) {
   auto *h = new Handle;
   h->params.assign(sizeof(RockConvParams), 0);
@@ -787,8 +863,6 @@ Handle *utility_fill_handle(int64_t bytes) {
   h->perf_config = "";
   return h;
 }
-
-int64_t align256(int64_t bytes) { return (bytes + 255) / 256 * 256; }
 
 // One spatial axis of the backward-data decomposition.  Input positions with
 // (i + pad) % stride == r receive only the filter taps y with

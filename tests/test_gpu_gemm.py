@@ -238,3 +238,21 @@ def test_mfma_rate_probe(rock, gpu):
         rnd = rock.mfma_rate(dt, True)
         assert 0.2 * pk < const < 1.1 * pk, (dt, const)
         assert 0.2 * pk < rnd <= const * 1.05, (dt, rnd, const)
+
+
+@pytest.mark.parametrize("t,od", [("f16", "f16"), ("bf16", "f32"), ("f32", "f32"), ("fp8", "f32")])
+@pytest.mark.parametrize("tA,tB", [(False, False), (True, False), (True, True)])
+def test_gemm_split_over_blocks_exact(rock, oracle, gpu, t, od, tA, tB):
+    """Few output tiles, long K, K-major storage: the reduction is cut into batch
+    entries whose f32 partial results the reduction kernel adds (two kernels)."""
+    G, M, N, K = 1, 128, 192, 8192
+    info = {}
+    out, od_, ref = _run_case(rock, oracle, gpu, t, G, M, N, K, tA, tB, False, True, 17, out_dtype=od, info=info)
+    assert info["kernels"][1] == "rock_reduce_splits" and "_fast_" in info["kernels"][0]
+    assert np.array_equal(to_f32(out, od), oracle.round_through(ref, CODE[od]))
+    # the split can be declined
+    info = {}
+    out, _, _ = _run_case(rock, oracle, gpu, t, G, M, N, K, tA, tB, False, True, 17, out_dtype=od, info=info,
+                          split_k=False)
+    assert len(info["kernels"]) == 1
+    assert np.array_equal(to_f32(out, od), oracle.round_through(ref, CODE[od]))
