@@ -226,6 +226,12 @@ const Tile *pick_tile(int64_t M, int64_t N, int G, bool conv, const std::string 
     // largest number of tiles any CU has to work through
     int64_t per_cu = (tiles + kNumCU - 1) / kNumCU;
     double cost = (double)per_cu * t.bm * t.bn / t.efficiency;
+    // a compute unit with a single four-wave block resident (one wave per
+    // SIMD) cannot keep its matrix pipes busy: nothing overlaps a wave's LDS
+    // reads and barriers
+    const int64_t resident = std::min<int64_t>(per_cu, t.blocks_per_cu);
+    if (resident * t.waves_m * t.waves_n < 8)
+      cost /= 0.7;
     if (!best || cost < best_cost) {
       best = &t;
       best_cost = cost;
