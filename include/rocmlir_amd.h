@@ -141,6 +141,15 @@ ROCMLIR_AMD_API MiirStatus rockamdGetKernelAttrs(MiirHandle handle, uint32_t att
 ROCMLIR_AMD_API MiirStatus rockamdGetKernelArgs(MiirHandle handle, int *num_pointers,
                                 void *params, size_t *params_size);
 
+/* The caller's pointer list described, one entry per pointer rockamdLaunch
+ * takes (index < caller_pointers of rockamdGetPointerMap): element type
+ * (RockDType value of kernel_params.h: 0 f32, 1 f16, 2 bf16, 3 i8, 4 fp8,
+ * 5 bf8, 6 i32; -1 = bytes, the workspace), rank (<= 5) and dimensions in
+ * storage order, outermost first -- what mlirGetKernelInfo reports per
+ * argument (MIGraphX.cpp:54-90).  Any of the out-pointers may be NULL. */
+ROCMLIR_AMD_API MiirStatus rockamdGetArgumentInfo(MiirHandle handle, int index, int *dtype, int *rank,
+                                                  int64_t *dims);
+
 /* perf-config string of the selected kernel in the reference's grammar
  * ("v2:MPB,NPB,KpackPB,MPW,MnPerXdl,Kpack,splitK,forceUnroll,1" or
  * "attn:v1:...", RockAttrDefs.td:241-329).  strncpy semantics, returns the

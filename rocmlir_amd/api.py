@@ -49,6 +49,9 @@ def load_library():
             getattr(L, name).argtypes = [vp]
         L.rockamdGetWorkspaceSize64.restype = sz
         L.rockamdGetWorkspaceSize64.argtypes = [vp]
+        L.rockamdGetArgumentInfo.restype = C.c_int
+        L.rockamdGetArgumentInfo.argtypes = [vp, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int),
+                                             C.POINTER(C.c_int64)]
         L.miirBufferGet.restype = C.c_int
         L.miirBufferGet.argtypes = [vp, C.c_char_p, C.POINTER(sz)]
         L.miirGetExecutionDims.restype = C.c_int
@@ -246,6 +249,16 @@ class RockKernel:
             raise RockError("rockamdTuningSetFromStr(%r) failed: %s"
                             % (perf_config, last_error()))
         self._refresh()
+
+    def arguments(self):
+        """[(dtype code, dims)] for every pointer launch() takes (rockamdGetArgumentInfo)."""
+        out = []
+        for i in range(self.caller_pointers):
+            dt, rank, dims = C.c_int(), C.c_int(), (C.c_int64 * 5)()
+            if load_library().rockamdGetArgumentInfo(self._h, i, C.byref(dt), C.byref(rank), dims) != 0:
+                raise RockError("rockamdGetArgumentInfo(%d) failed" % i)
+            out.append((dt.value, list(dims[:rank.value])))
+        return out
 
     def set_scale(self, scale):
         load_library().rockamdSetScale(self._h, float(scale))

@@ -273,6 +273,13 @@ struct Handle {
     int64_t offset; // bytes added to it
   };
   std::vector<PtrSrc> ptr_map;
+  // the caller's pointer list described: element type (RockDType, -1 = bytes)
+  // and dimensions in storage order, outermost first
+  struct ArgInfo {
+    int dtype;
+    std::vector<int64_t> dims;
+  };
+  std::vector<ArgInfo> args;
   // typed views of `params`
   RockEpilogue *epi = nullptr;
   // launch cache: device -> function
@@ -1838,6 +1845,81 @@ bool check_launch_args(Handle *h, void *const *pointers, int num_pointers) {
   return true; // (a residual, when the problem names one, is pointer 4 and covered by the loop)
 }
 
+// What the caller's pointers are, for clients that size and check their
+// buffers from the handle (the per-argument rank and dimensions MIGraphX reads
+// with mlirGetKernelInfo, mlir/lib/CAPI/Dialect/MIGraphX.cpp:54-90).
+void describe_arguments(const OptMap &o, Handle *h) {
+  using A = Handle::ArgInfo;
+  const std::string op = str_or(o, "operation", "");
+  auto with_workspace = [&] {
+    if (h->workspace_bytes)
+      h->args.push_back(A{-1, {(int64_t)h->workspace_bytes}});
+  };
+  if (op == "gemm") {
+    std::string t = str_or(o, "t", "f32");
+    size_t us = t.find('_');
+    const int ta = parse_dtype(us == std::string::npos ? t : t.substr(0, us));
+    const int tb = parse_dtype(us == std::string::npos ? t : t.substr(us + 1));
+    const int tc = h->epi ? h->epi->out_dtype : -1;
+    const int64_t G = int_or(o, "g", 1), M = int_or(o, "m", 0), N = int_or(o, "n", 0), K = int_or(o, "k", 0);
+    const bool tA = bool_or(o, "transA", false), tB = bool_or(o, "transB", false), tC = bool_or(o, "transC", false);
+    std::string outs = str_or(o, "out_datatype", str_or(o, "c_dtype", ""));
+    const int dflt = ta == ROCK_I8 ? ROCK_I32 : (ta == ROCK_FP8 || ta == ROCK_BF8) ? ROCK_F32 : ta;
+    const int out_t = outs.empty() ? dflt : parse_dtype(outs);
+    (void)tc;
+    h->args = {A{ta, tA ? std::vector<int64_t>{G, K, M} : std::vector<int64_t>{G, M, K}},
+               A{tb, tB ? std::vector<int64_t>{G, N, K} : std::vector<int64_t>{G, K, N}},
+               A{out_t, tC ? std::vector<int64_t>{G, N, M} : std::vector<int64_t>{G, M, N}},
+               A{out_t == ROCK_I32 ? ROCK_I32 : ROCK_F32, {N}}};
+    if (str_or(o, "residual", "none") != "none")
+      h->args.push_back(A{out_t, h->args[2].dims});
+    with_workspace();
+  } else if (op == "attention") {
+    const int t = parse_dtype(str_or(o, "t", "f16"));
+    const int tv = t == ROCK_I8 ? ROCK_F16 : t;
+    const int64_t G = int_or(o, "g", 1), sq = int_or(o, "seq_len_q", 0), sk = int_or(o, "seq_len_k", 0),
+                  dqk = int_or(o, "head_dim_qk", 0), dv = int_or(o, "head_dim_v", 0);
+    auto mat = [&](bool tr, int64_t r, int64_t c) { return tr ? std::vector<int64_t>{G, c, r} : std::vector<int64_t>{G, r, c}; };
+    h->args = {A{t, mat(bool_or(o, "transQ", false), sq, dqk)}, A{t, mat(!bool_or(o, "transK", false), sk, dqk)},
+               A{tv, mat(bool_or(o, "transV", false), sk, dv)}};
+    if (bool_or(o, "with-attn-scale", false))
+      h->args.push_back(A{tv, {G, sq, sk}});
+    h->args.push_back(A{tv, {G, sq, sk}}); // bias slot
+    h->args.push_back(A{tv, mat(bool_or(o, "transO", false), sq, dv)});
+    with_workspace();
+  } else { // convolutions: filter, input, output in the order of their layout strings
+    std::string t_all = str_or(o, "t", "");
+    const int ti = parse_dtype(str_or(o, "in_type", t_all)), tf = parse_dtype(str_or(o, "fil_type", t_all));
+    std::string out_t = str_or(o, "out_type", str_or(o, "out_datatype", ""));
+    const int dflt = ti == ROCK_I8 ? ROCK_I32 : (ti == ROCK_FP8 || ti == ROCK_BF8) ? ROCK_F32 : ti;
+    const int to = out_t.empty() ? dflt : parse_dtype(out_t);
+    std::string fl, il, ol;
+    if (!canon_layout(str_or(o, "fil_layout", ""), 'k', "gkcyx", fl) || !canon_layout(str_or(o, "in_layout", ""), 'c', "ngchw", il) ||
+        !canon_layout(str_or(o, "out_layout", ""), 'k', "ngkhw", ol))
+      return;
+    const int64_t n = int_or(o, "batchsize", 0), g = int_or(o, "groupsize", 1), c = int_or(o, "in_channels", 0) / g,
+                  k = int_or(o, "out_channels", 0) / g, hi = int_or(o, "in_h", 0), wi = int_or(o, "in_w", 0),
+                  y = int_or(o, "fil_h", 0), x = int_or(o, "fil_w", 0);
+    const int64_t dh = int_or(o, "dilation_h", 1), dw = int_or(o, "dilation_w", 1), sh = int_or(o, "conv_stride_h", 1),
+                  sw = int_or(o, "conv_stride_w", 1);
+    const int64_t ph = int_or(o, "padding_h_l", int_or(o, "padding_h", 0)), pw = int_or(o, "padding_w_l", int_or(o, "padding_w", 0));
+    const int64_t ph_r = int_or(o, "padding_h_r", int_or(o, "padding_h", 0)), pw_r = int_or(o, "padding_w_r", int_or(o, "padding_w", 0));
+    const int64_t ho = (hi + ph + ph_r - (y - 1) * dh - 1) / sh + 1, wo = (wi + pw + pw_r - (x - 1) * dw - 1) / sw + 1;
+    auto dims = [](const std::string &layout, const char *letters, const int64_t *sizes) {
+      std::vector<int64_t> d;
+      for (char ch : layout)
+        d.push_back(sizes[std::strchr(letters, ch) - letters]);
+      return d;
+    };
+    const int64_t fsz[5] = {g, k, c, y, x}, isz[5] = {n, g, c, hi, wi}, osz[5] = {n, g, k, ho, wo};
+    h->args = {A{tf, dims(fl, "gkcyx", fsz)}, A{ti, dims(il, "ngchw", isz)}, A{to, dims(ol, "ngkhw", osz)},
+               A{to == ROCK_I32 ? ROCK_I32 : ROCK_F32, {g * k}}};
+    if (str_or(o, "residual", "none") != "none")
+      h->args.push_back(A{to, h->args[2].dims});
+    with_workspace();
+  }
+}
+
 // problem description -> resolved kernel; NULL with the error set on failure
 Handle *build_handle(const OptMap &o) {
   // arch: "[triple:]gfxNNN[:features]" (ConvGenerator.cpp:538-552); only
@@ -1879,6 +1961,7 @@ Handle *build_handle(const OptMap &o) {
     return nullptr;
   }
   h->options = o;
+  describe_arguments(o, h);
   return h;
 }
 
@@ -2049,6 +2132,21 @@ MiirStatus rockamdGetKernelArgs(MiirHandle handle, int *num_pointers, void *para
     std::memcpy(params, h->params.data(), h->params.size());
   }
   *params_size = h->params.size();
+  return MIIR_SUCCESS;
+}
+
+MiirStatus rockamdGetArgumentInfo(MiirHandle handle, int index, int *dtype, int *rank, int64_t *dims) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h || index < 0 || index >= (int)h->args.size())
+    return MIIR_INVALID_PARAM;
+  const auto &a = h->args[index];
+  if (dtype)
+    *dtype = a.dtype;
+  if (rank)
+    *rank = (int)a.dims.size();
+  if (dims)
+    for (size_t i = 0; i < a.dims.size(); ++i)
+      dims[i] = a.dims[i];
   return MIIR_SUCCESS;
 }
 

@@ -227,6 +227,26 @@ def test_layout_conversion_plan_follows_the_multi_kernel_protocol(rock):
     assert lib.rockamdSetScale(rock.RockKernel(nchw)._h, C.c_float(2.0)) != 0
 
 
+def test_argument_info_describes_the_caller_list(rock):
+    """Element type and dimensions per pointer, as mlirGetKernelInfo reports
+    them per kernel argument (MIGraphX.cpp:54-90)."""
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t i8 -out_datatype f16 -g 2 -m 64 -n 48 -k 32 -transB true "
+                        "-scale 0.01 -residual add")
+    assert k.arguments() == [(3, [2, 64, 32]), (3, [2, 48, 32]), (1, [2, 64, 48]), (0, [48]), (1, [2, 64, 48])]
+    k = rock.RockKernel(CONV_RESNET)
+    assert k.arguments() == [(1, [1, 128, 3, 3, 128]), (1, [256, 28, 28, 1, 128]), (1, [256, 28, 28, 1, 128]),
+                             (0, [128])]
+    nchw = CONV_RESNET.replace("NHWGC", "NGCHW").replace("GNYXC", "GNCHW")
+    args = rock.RockKernel(nchw + " --kernel_id 1").arguments()     # every kernel of a plan: the same list
+    assert args[1] == (1, [256, 1, 128, 28, 28]) and args[4] == (-1, [rock.RockKernel(nchw).workspace_bytes])
+    k = rock.RockKernel("-operation attention -arch gfx950 -t f16 -g 4 -seq_len_q 256 -seq_len_k 77 -head_dim_qk 64 "
+                        "-head_dim_v 32 -transK true -with-attn-scale true")
+    assert k.arguments() == [(1, [4, 256, 64]), (1, [4, 77, 64]), (1, [4, 77, 32]), (1, [4, 256, 77]),
+                             (1, [4, 256, 77]), (1, [4, 256, 32])]
+    lib = rock.load_library()
+    assert lib.rockamdGetArgumentInfo(k._h, 6, None, None, None) != 0
+
+
 def test_attention_pre_softmax_tensors(rock):
     """-with-attn-scale / -with-attn-bias (rocmlir-gen.cpp:2185-2196): the
     caller list is Q, K, V, [scale tensor], bias slot, O."""
