@@ -716,12 +716,60 @@ __device__ __forceinline__ void dl_epilogue(typename MmaTraits<DT>::Acc (&acc)[M
                                                     staged_ok);
     return;
   }
-  if (staged_ok)
+  const bool cols_ok = !staged_ok && out_cols_chunk_aligned(p, Cptr, out_elem_size(e.out_dtype));
+  if (staged_ok || cols_ok)
     __builtin_amdgcn_s_barrier(); // every wave is done reading the operand stages
 
   dispatch_out_dtype<Tr::INT_ACC>(e.out_dtype, [&](auto od_const) __attribute__((always_inline)) {
     constexpr int OD = decltype(od_const)::value;
     // plain epilogue (scale, bias, relu / clip, narrowing): unrolled over the registers
+    if (cols_ok) {
+      // m-contiguous output (NCHW-style convolution output, transposed C): each
+      // 32-row block goes through the wave's LDS region as [channel][row], and
+      // leaves as 16-byte vectors of consecutive rows
+      constexpr int ES = OutElemSize<OD>::value;
+      constexpr int MP = 32 * ES + (ES == 4 ? 0 : 16); // bytes per channel row in LDS
+      constexpr int VPR = 32 * ES / 16;                // 16-byte vectors per channel row
+      constexpr int WBUF = 32 * (WTN * 4 + 16);
+      static_assert(WTN * MP <= WBUF && NWAVES * WBUF <= LDS_BYTES, "transposed block must fit in the wave's region");
+      char *wbuf = lds + wave * WBUF;
+#pragma unroll
+      for (int i = 0; i < MI; ++i) {
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int nloc = j * 32 + q * 8 + lgrp * 4;
+            Acc4 a4 = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                       acc[i][j][4 * q + 3]};
+            const v4i raw = epilogue_convert4<Tr::INT_ACC, OD>(a4, e, aux, n_wave + nloc, p.N);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              char *dst = wbuf + (nloc + r) * MP + lrow * ES;
+              if constexpr (ES == 4)
+                *(int *)dst = raw[r];
+              else if constexpr (ES == 2)
+                *(uint16_t *)dst = (uint16_t)((uint32_t)raw[r >> 1] >> (16 * (r & 1)));
+              else
+                *(uint8_t *)dst = (uint8_t)((uint32_t)raw[0] >> (8 * r));
+            }
+          }
+        }
+#pragma unroll
+        for (int it = 0; it < WTN * VPR / 64; ++it) {
+          const int v = it * 64 + lane;
+          const int nloc = v / VPR, mloc = (v % VPR) * (16 / ES);
+          const v4i d = *(const v4i *)(wbuf + nloc * MP + mloc * ES);
+          const int m = m_wave + i * 32 + mloc, n = n_wave + nloc;
+          if (m < p.M && n < p.N) {
+            int64_t off, n_stride;
+            out_col_addr(p, g, m, off, n_stride);
+            *(v4i *)((char *)Cptr + (off + (int64_t)n * n_stride) * ES) = d;
+          }
+        }
+      }
+      return;
+    }
     if (!staged_ok) {
       direct_epilogue<Tr::INT_ACC, OD, MI, NI, Acc4, false>(acc, p, g, Cptr, aux, nullptr, m_wave + lrow,
                                                            n_wave + lgrp * 4);

@@ -553,6 +553,30 @@ __device__ __forceinline__ bool out_rows_chunk_aligned(const RockConvParams &p, 
            (uintptr_t)(p.out_hs * es) | (uintptr_t)(p.out_ws * es) | (uintptr_t)((int64_t)p.N * es)) & 15) == 0;
 }
 
+// The output is contiguous along m (rows of the implicit GEMM), not along n:
+// a transposed C, or an NCHW-style convolution output whose pixels are
+// contiguous per channel.  16 bytes' worth of consecutive m must start on a
+// 16-byte boundary and stay inside one image.
+__device__ __forceinline__ bool out_cols_chunk_aligned(const RockGemmParams &p, const void *base, int es) {
+  return p.c_ms == 1 && (((uintptr_t)base | (uintptr_t)(p.c_ns * es) | (uintptr_t)(p.c_gs * es) |
+                          (uintptr_t)((int64_t)p.M * es)) & 15) == 0;
+}
+__device__ __forceinline__ bool out_cols_chunk_aligned(const RockConvParams &p, const void *base, int es) {
+  return p.out_ws == 1 && p.out_hs == (int64_t)p.wo &&
+         (((uintptr_t)base | (uintptr_t)(p.out_ns * es) | (uintptr_t)(p.out_gs * es) | (uintptr_t)(p.out_ks * es) |
+           (uintptr_t)((int64_t)p.ho * p.wo * es)) & 15) == 0;
+}
+// element offset of output (g, m, n = 0) and the stride between channels, for m-contiguous outputs
+__device__ __forceinline__ void out_col_addr(const RockGemmParams &p, int g, int m, int64_t &off, int64_t &n_stride) {
+  off = (int64_t)g * p.c_gs + m;
+  n_stride = p.c_ns;
+}
+__device__ __forceinline__ void out_col_addr(const RockConvParams &p, int g, int m, int64_t &off, int64_t &n_stride) {
+  const int img = m / (p.ho * p.wo);
+  off = (int64_t)img * p.out_ns + (int64_t)g * p.out_gs + (m - img * (p.ho * p.wo));
+  n_stride = p.out_ks;
+}
+
 template <int DT, int ROWS, int NT, int KIND>
 __device__ __forceinline__ auto make_loader_a(const void *A, const RockGemmParams &p, int g, int m0, int tid) {
   static_assert(KIND == LD_ROWS_GENERIC, "K-contiguous operands take the direct-to-LDS body");

@@ -665,6 +665,14 @@ bool fill_relayout_handle(Handle *h, const int64_t size[5], const int64_t src_si
   for (int d = 0; d < 5; ++d) // the source's contiguous dimension (ties: the longest)
     if (r.src_stride[d] == 1 && (r.src_stride[r.src_fast] != 1 || r.size[d] > r.size[r.src_fast]))
       r.src_fast = d;
+  if (r.src_stride[r.src_fast] != 1) {
+    // no unit-stride dimension (every other pixel of a row, a flipped filter):
+    // tile along the one whose elements lie closest together
+    for (int d = 0; d < 5; ++d)
+      if (r.size[d] > 1 && r.src_stride[d] != 0 &&
+          std::llabs(r.src_stride[d]) < std::llabs(r.src_stride[r.src_fast]))
+        r.src_fast = d;
+  }
   int64_t blocks = 1;
   if (r.src_fast == r.dst_fast) {
     // the destination's channel runs are whole 16-byte chunks by construction of cp
@@ -915,6 +923,60 @@ BwdAxis bwd_data_axis(int64_t r, int64_t stride, int64_t dil, int64_t Y, int64_t
 Handle *make_conv_bwd_data(const OptMap &o, const ConvProblem &cp) {
   const int es = dtype_size(cp.ti);
   const int kid = (int)int_or(o, "kernel_id", 0);
+  // 1x1 filter, unit stride, no padding, one group: dX[pixel, c] = sum over k
+  // of dY[pixel, k] * W[k, c] is a GEMM over the tensors as they lie.  With
+  // contiguous pixels (NCHW) it runs per image as W^T x dY_n, both operands
+  // K-major; with contiguous channels (NHWC) as dY x W with the filter
+  // K-major, over all images at once when their pixels are equally spaced.
+  // One kernel, no workspace.
+  if (cp.y == 1 && cp.x == 1 && cp.sh == 1 && cp.sw == 1 && cp.ph == 0 && cp.pw == 0 && cp.g == 1 &&
+      cp.hi * cp.wi <= INT32_MAX && cp.n * cp.hi * cp.wi <= INT32_MAX && bool_or(o, "pointwise_as_gemm", true) &&
+      bool_or(o, "layout_conversion", true)) {
+    const int64_t P = cp.hi * cp.wi;
+    const bool lin_x = cp.is[3] == cp.wi * cp.is[4], lin_y = cp.os[3] == cp.wo * cp.os[4];
+    RockGemmParams gp;
+    std::memset(&gp, 0, sizeof gp);
+    bool shaped = false, pixels = false;
+    if (lin_x && lin_y && cp.is[4] == 1 && cp.os[4] == 1) { // pixels contiguous
+      pixels = true;
+      gp.G = (int)cp.n; gp.M = (int)cp.c; gp.N = (int)P; gp.K = (int)cp.k;
+      gp.a_gs = 0; gp.a_ms = cp.fs[2]; gp.a_ks = cp.fs[1];
+      gp.b_gs = cp.os[0]; gp.b_ns = 1; gp.b_ks = cp.os[2];
+      gp.c_gs = cp.is[0]; gp.c_ms = cp.is[2]; gp.c_ns = 1;
+      shaped = true;
+    } else if (lin_x && lin_y && cp.is[2] == 1 && cp.os[2] == 1) { // channels contiguous
+      const bool whole = cp.is[0] == P * cp.is[4] && cp.os[0] == P * cp.os[4];
+      gp.G = whole ? 1 : (int)cp.n; gp.M = (int)(whole ? cp.n * P : P); gp.N = (int)cp.c; gp.K = (int)cp.k;
+      gp.a_gs = whole ? 0 : cp.os[0]; gp.a_ms = cp.os[4]; gp.a_ks = 1;
+      gp.b_gs = 0; gp.b_ns = cp.fs[2]; gp.b_ks = cp.fs[1];
+      gp.c_gs = whole ? 0 : cp.is[0]; gp.c_ms = cp.is[4]; gp.c_ns = 1;
+      shaped = true;
+    }
+    if (shaped) {
+      default_epilogue(gp.epi, cp.ti);
+      auto *h = new Handle;
+      if (plan_gemm_kernel(h, gp, operand_code(cp.ti, cp.ti), es, o)) {
+        if (kid != 0) {
+          delete h;
+          set_error("conv: kernel_id out of range");
+          return nullptr;
+        }
+        h->op = OP_GEMM;
+        h->params.assign(sizeof gp, 0);
+        std::memcpy(h->params.data(), &gp, sizeof gp);
+        h->epi = &reinterpret_cast<RockGemmParams *>(h->params.data())->epi;
+        // GEMM A, B, C from the caller's filter, input (written), output
+        h->ptr_map = pixels ? std::vector<Handle::PtrSrc>{{0, 0}, {2, 0}, {1, 0}, {-1, 0}, {-1, 0}}
+                            : std::vector<Handle::PtrSrc>{{2, 0}, {0, 0}, {1, 0}, {-1, 0}, {-1, 0}};
+        h->problem_key = conv_problem_key(h, o, cp, 2);
+        h->kernel_count = 1;
+        h->workspace_bytes = 0;
+        h->caller_pointers = 4;
+        return h;
+      }
+      delete h;
+    }
+  }
   struct Phase {
     BwdAxis h, w;
     int64_t rh, rw;
@@ -1450,17 +1512,25 @@ Handle *make_conv(const OptMap &o) {
     RockConvParams q = p;
     q.c = (int)cp;
     q.K = (int)(cp * y * x);
-    const int64_t fsz[5] = {g, k, cp, y, x}, isz[5] = {n, g, cp, hi, wi};        // converted tensors
-    const int64_t fsz_src[5] = {g, k, c, y, x}, isz_src[5] = {n, g, c, hi, wi};  // the caller's
+    const bool need_i = cp != c || !(p.in_cs == 1 && al(p.in_ws) && al(p.in_hs) && al(p.in_ns) && al(p.in_gs));
+    // a strided 1x1 filter without padding reads one pixel in stride_h * stride_w:
+    // the conversion copies only those, and the contraction runs with unit stride
+    const bool shrink = need_i && y == 1 && x == 1 && ph == 0 && pw == 0 && ph_r == 0 && pw_r == 0 && (sh > 1 || sw > 1);
+    const int64_t hi2 = shrink ? ho : hi, wi2 = shrink ? wo : wi;
+    if (shrink) {
+      q.hi = (int)ho; q.wi = (int)wo;
+      q.stride_h = q.stride_w = 1;
+    }
+    const int64_t fsz[5] = {g, k, cp, y, x}, isz[5] = {n, g, cp, hi2, wi2};        // converted tensors
+    const int64_t fsz_src[5] = {g, k, c, y, x}, isz_src[5] = {n, g, c, hi2, wi2};  // the caller's
     int64_t fs[5], is[5];
     layout_strides("gkyxc", "gkcyx", fsz, fs);
     layout_strides("nhwgc", "ngchw", isz, is);
     q.fil_gs = fs[0]; q.fil_ks = fs[1]; q.fil_cs = fs[2]; q.fil_ys = fs[3]; q.fil_xs = fs[4];
     q.in_ns = is[0]; q.in_gs = is[1]; q.in_cs = is[2]; q.in_hs = is[3]; q.in_ws = is[4];
     const bool need_f = cp != c || !(p.fil_cs == 1 && p.fil_xs == c && p.fil_ys == x * c && al(p.fil_ks) && al(p.fil_gs));
-    const bool need_i = cp != c || !(p.in_cs == 1 && al(p.in_ws) && al(p.in_hs) && al(p.in_ns) && al(p.in_gs));
     const int64_t fil_bytes = (g * k * cp * y * x * es + 255) / 256 * 256;
-    const int64_t in_bytes = (n * g * cp * hi * wi * es + 255) / 256 * 256;
+    const int64_t in_bytes = (n * g * cp * hi2 * wi2 * es + 255) / 256 * 256;
     if (!fast && cp * y * x <= INT32_MAX && conv_fast(q, cp) && bool_or(o, "layout_conversion", true)) {
       if (!need_f) { // keep the caller's filter
         q.fil_gs = p.fil_gs; q.fil_ks = p.fil_ks; q.fil_cs = p.fil_cs; q.fil_ys = p.fil_ys; q.fil_xs = p.fil_xs;
@@ -1485,7 +1555,7 @@ Handle *make_conv(const OptMap &o) {
         // dimensions listed in destination (channel-contiguous) order
         const int order_f[5] = {0, 1, 3, 4, 2}, order_i[5] = {0, 3, 4, 1, 2}; // g k y x c ; n h w g c
         const int64_t src_f[5] = {p.fil_gs, p.fil_ks, p.fil_cs, p.fil_ys, p.fil_xs};
-        const int64_t src_i[5] = {p.in_ns, p.in_gs, p.in_cs, p.in_hs, p.in_ws};
+        const int64_t src_i[5] = {p.in_ns, p.in_gs, p.in_cs, p.in_hs * (shrink ? sh : 1), p.in_ws * (shrink ? sw : 1)};
         int64_t rsize[5], rsrc_size[5], rstride[5];
         for (int d = 0; d < 5; ++d) {
           const int letter = is_f ? order_f[d] : order_i[d];

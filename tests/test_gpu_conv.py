@@ -87,6 +87,9 @@ EDGE_CASES = [
     (3, 1, 8, 8, 4, 4, 1, 1, (3, 3), (1, 1), (2, 2)),
     (2, 4, 64, 64, 7, 7, 1, 1, (1, 1), (0, 0), (1, 1)),
     (2, 2, 16, 24, 9, 9, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (2, 1, 16, 24, 9, 9, 1, 1, (2, 2), (0, 0), (1, 1)),      # strided pointwise: the conversion copies the used pixels only
+    (2, 1, 16, 24, 8, 10, 1, 1, (2, 3), (0, 0), (1, 1)),
+    (2, 1, 8, 16, 1, 50, 1, 5, (1, 2), (0, 2), (1, 1)),      # a 1-D convolution written as 2-D with height 1
 ]
 
 

@@ -67,6 +67,7 @@ CASES = [
     (4, 1, 16, 16, 5, 5, 2, 2, (1, 1), (0, 0), (2, 2)),
     (4, 1, 16, 24, 6, 6, 1, 1, (1, 1), (0, 0), (1, 1)),       # pointwise: the weight gradient is a split GEMM
     (3, 1, 64, 48, 8, 8, 1, 1, (1, 1), (0, 0), (1, 1)),
+    (2, 1, 128, 192, 16, 16, 1, 1, (1, 1), (0, 0), (1, 1)),   # pointwise, more than one tile
 ]
 LAYOUTS = [NHWC, NCHW, ("gyxck", "hwcgn", "hwkgn")]
 
@@ -111,6 +112,9 @@ def test_conv_bwd_data_exact(rock, oracle, gpu, case, layouts, t, convert):
     assert np.array_equal(to_f32(got, t), oracle.round_through(ref, CODE[t]))
     if not convert:
         assert not any(name.startswith("rock_relayout") for name in info["kernels"])
+    elif (y, x, c % 64, hi % 8) == (1, 1, 0, 0) and stride == (1, 1) and layouts in (NHWC, NCHW):
+        # pointwise with whole 16-byte runs: one GEMM over the tensors as they lie
+        assert len(info["kernels"]) == 1 and info["kernels"][0].startswith("rock_gemm_")
 
 
 @pytest.mark.parametrize("convert", [True, False], ids=["converted", "as-is"])
@@ -126,7 +130,7 @@ def test_conv_bwd_weight_exact(rock, oracle, gpu, case, layouts, t, convert):
     torch.cuda.synchronize()
     ref, _, _ = oracle.conv_bwd_weight(iq, dyq, *layouts, n, g, c, k, hi, wi, y, x, stride, pad, dil)
     assert np.array_equal(to_f32(got, t), oracle.round_through(ref, CODE[t]))
-    if (c, hi) == (64, 8) and layouts in (NHWC, NCHW):
+    if (y, x, c % 64, hi % 8) == (1, 1, 0, 0) and layouts in (NHWC, NCHW):
         # pointwise with whole 16-byte runs: a GEMM over the tensors as they lie, its split
         # partial sums added by the reduction kernel
         assert info["kernels"][0].startswith("rock_gemm_") and not any("relayout" in k for k in info["kernels"])
