@@ -62,7 +62,11 @@ typedef void *MiirHandle;
  * kernel_name, perf_config, in_type/fil_type/out_type, in_layout/fil_layout/
  * out_layout, batchsize, groupsize, in_channels, out_channels, in_h, in_w,
  * out_h, out_w, fil_h, fil_w, dilation_{h,w}, conv_stride_{h,w},
- * padding_{h,w}.  `--operation gemm` and `--operation attention` take the
+ * padding_{h,w}.  With in_d / fil_d (and out_d, dilation_d, conv_stride_d,
+ * padding_d; rocmlir-gen.cpp:171-294) the forward convolution runs over three
+ * spatial dimensions and the layouts have six letters (ngc012 / gkc012 /
+ * ngk012, h w d and y x z accepted for 0 1 2): several kernels over a
+ * workspace, same pointer order.  `--operation gemm` and `--operation attention` take the
  * reference's rocmlir-gen flag names (rocmlir-gen.cpp:90-561): t,
  * out_datatype, g, m, k, n, transA, transB, transC; g, seq_len_q, seq_len_k,
  * head_dim_qk, head_dim_v, transQ, transK, transV, transO, with-attn-bias,
@@ -144,7 +148,7 @@ ROCMLIR_AMD_API MiirStatus rockamdGetKernelArgs(MiirHandle handle, int *num_poin
 /* The caller's pointer list described, one entry per pointer rockamdLaunch
  * takes (index < caller_pointers of rockamdGetPointerMap): element type
  * (RockDType value of kernel_params.h: 0 f32, 1 f16, 2 bf16, 3 i8, 4 fp8,
- * 5 bf8, 6 i32; -1 = bytes, the workspace), rank (<= 5) and dimensions in
+ * 5 bf8, 6 i32; -1 = bytes, the workspace), rank (<= 6) and dimensions in
  * storage order, outermost first -- what mlirGetKernelInfo reports per
  * argument (MIGraphX.cpp:54-90).  Any of the out-pointers may be NULL. */
 ROCMLIR_AMD_API MiirStatus rockamdGetArgumentInfo(MiirHandle handle, int index, int *dtype, int *rank,

@@ -229,6 +229,40 @@ def conv_bwd_weight(inp, out, fil_layout, in_layout, out_layout, n, g, c, k, hi,
     return fil, ho, wo
 
 
+def conv3d(fil, inp, fil_layout, in_layout, out_layout, n, g, c, k, in_size, fil_size,
+           stride=(1, 1, 1), pad=(0, 0, 0), dil=(1, 1, 1)):
+    """Forward convolution over three spatial dimensions, the arithmetic the
+    reference checks its 3-D rock.conv against (linalg.conv_3d in
+    mlir/test/Dialect/Rock/integration/conv3d-test-from-rocmlir-gen.mlir:12-20,
+    grouped and strided as rocmlir-gen.cpp:171-294 parameterises it).  Flat
+    arrays laid out as six-letter strings over g k c 0 1 2 / n g c 0 1 2 /
+    n g k 0 1 2 say; numpy, one slice product per filter tap, sums in f64 (tests
+    use integer-valued data where the order of the sum cannot matter, and a
+    tolerance otherwise).  Returns (flat output, output sizes)."""
+    outs = tuple(conv_out_dim(in_size[a], fil_size[a], pad[a], pad[a], stride[a], dil[a]) for a in range(3))
+
+    def canon(flat, layout, letters, sizes):
+        shape = [sizes[letters.index(ch)] for ch in layout]
+        arr = np.asarray(flat, np.float64).reshape(shape)
+        return arr.transpose([layout.index(ch) for ch in letters])
+
+    f = canon(fil, fil_layout, "gkc012", (g, k, c) + tuple(fil_size))
+    x = canon(inp, in_layout, "ngc012", (n, g, c) + tuple(in_size))
+    xp = np.zeros((n, g, c) + tuple(in_size[a] + 2 * pad[a] for a in range(3)))
+    xp[:, :, :, pad[0]:pad[0] + in_size[0], pad[1]:pad[1] + in_size[1], pad[2]:pad[2] + in_size[2]] = x
+    out = np.zeros((n, g, k) + outs)
+    for t0 in range(fil_size[0]):
+        for t1 in range(fil_size[1]):
+            for t2 in range(fil_size[2]):
+                win = xp[:, :, :,
+                         t0 * dil[0]:t0 * dil[0] + (outs[0] - 1) * stride[0] + 1:stride[0],
+                         t1 * dil[1]:t1 * dil[1] + (outs[1] - 1) * stride[1] + 1:stride[1],
+                         t2 * dil[2]:t2 * dil[2] + (outs[2] - 1) * stride[2] + 1:stride[2]]
+                out += np.einsum("ngcabd,gkc->ngkabd", win, f[:, :, :, t0, t1, t2])
+    flat = out.transpose(["ngk012".index(ch) for ch in out_layout]).astype(np.float32).ravel()
+    return flat, outs
+
+
 # ---- attention ------------------------------------------------------------
 def attention(Q, K, V, G, sq, sk, dqk, dv, scale=1.0, scale_t=None,
               bias_t=None, transQ=False, transK=False, transV=False,

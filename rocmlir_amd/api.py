@@ -254,7 +254,7 @@ class RockKernel:
         """[(dtype code, dims)] for every pointer launch() takes (rockamdGetArgumentInfo)."""
         out = []
         for i in range(self.caller_pointers):
-            dt, rank, dims = C.c_int(), C.c_int(), (C.c_int64 * 5)()
+            dt, rank, dims = C.c_int(), C.c_int(), (C.c_int64 * 6)()
             if load_library().rockamdGetArgumentInfo(self._h, i, C.byref(dt), C.byref(rank), dims) != 0:
                 raise RockError("rockamdGetArgumentInfo(%d) failed" % i)
             out.append((dt.value, list(dims[:rank.value])))
@@ -563,6 +563,43 @@ def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, zero_point=0,
         kern.launch(q, k, v, bias, out, stream=stream)
     else:
         kern.launch(q, k, v, scale_tensor.contiguous(), bias, out, stream=stream)
+    return out
+
+
+def conv3d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize, in_channels, out_channels, in_size,
+           fil_size, groupsize=1, stride=(1, 1, 1), padding=(0, 0, 0), dilation=(1, 1, 1), out_dtype=None,
+           scale=None, zero_point=0, bias=None, relu=False, quant_scale=None, out_zero_point=0,
+           activation=None, clip=None, out=None, perf_config=None, stream=None, info=None):
+    """Forward convolution over three spatial dimensions.  Sizes, strides,
+    padding and dilation are (h, w, d) triples; the layout strings have six
+    letters ('ngc012' / 'gkc012' / 'ngk012' in rocmlir-gen's spelling, h w d
+    and y x z accepted for 0 1 2).  Epilogue arguments as for conv2d(), without
+    a residual tensor.  Returns the flat output tensor."""
+    import torch
+    t = _dtype_name(inp.dtype)
+    outs = [(in_size[a] + 2 * padding[a] - (fil_size[a] - 1) * dilation[a] - 1) // stride[a] + 1 for a in range(3)]
+    opts = ("--operation conv --arch gfx950 --in_type %s --fil_type %s --fil_layout %s --in_layout %s"
+            " --out_layout %s --batchsize %d --groupsize %d --in_channels %d --out_channels %d"
+            % (t, _dtype_name(fil.dtype), fil_layout, in_layout, out_layout, batchsize, groupsize, in_channels,
+               out_channels))
+    for a, s in enumerate("hwd"):
+        opts += (" --in_%s %d --fil_%s %d --out_%s %d --dilation_%s %d --conv_stride_%s %d --padding_%s %d"
+                 % (s, in_size[a], s, fil_size[a], s, outs[a], s, dilation[a], s, stride[a], s, padding[a]))
+    if out_dtype is not None:
+        opts += " --out_type %s" % out_dtype
+    if perf_config:
+        opts += " --perf_config %s" % perf_config
+    opts += _epilogue_flags(scale, zero_point, bias, relu, quant_scale, out_zero_point, activation, clip, None, "add")
+    prog = _program(opts)
+    if info is not None:
+        info["kernels"] = [x.kernel_name for x in prog.kernels]
+        info["workspace_bytes"] = prog.workspace_bytes
+    if out_dtype is None:
+        out_dtype = {"i8": "i32", "fp8": "f32", "bf8": "f32"}.get(t, t)
+    if out is None:
+        out = torch.empty(batchsize * out_channels * outs[0] * outs[1] * outs[2], dtype=_torch_dtype(out_dtype),
+                          device=inp.device)
+    prog.launch(fil.contiguous(), inp.contiguous(), out, bias, stream=stream)
     return out
 
 

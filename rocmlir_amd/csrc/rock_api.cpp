@@ -618,20 +618,23 @@ Handle *make_gemm(const OptMap &o) {
 }
 
 // Makes h a layout-conversion kernel: a 5-D tensor, dimensions listed in the
-// destination's order (the last one contiguous there, the destination dense),
+// destination's order (the last one contiguous there, the destination dense
+// unless dst_stride says otherwise),
 // read through src_stride and zero-filled beyond src_size.  Strides may be
 // negative (a flipped filter); the caller adds the matching base offset to the
 // source pointer.  Returns false with the error set when the tensor is too
 // large for the kernel's 32-bit indices.
 bool fill_relayout_handle(Handle *h, const int64_t size[5], const int64_t src_size[5],
-                          const int64_t src_stride[5], int es) {
+                          const int64_t src_stride[5], int es, const int64_t *dst_stride = nullptr) {
   RockRelayoutParams r;
   std::memset(&r, 0, sizeof r);
   struct Dim { int64_t size, src_size, ss, ds; };
   std::vector<Dim> dims;
   int64_t dst = 1;
+  // dst_stride: a destination that is a slice of a larger dense tensor (last
+  // dimension still contiguous, every stride a whole number of 16-byte chunks)
   for (int d = 4; d >= 0; --d) {
-    dims.insert(dims.begin(), Dim{size[d], src_size[d], src_stride[d], dst});
+    dims.insert(dims.begin(), Dim{size[d], src_size[d], src_stride[d], dst_stride ? dst_stride[d] : dst});
     dst *= size[d];
   }
   // drop unit dimensions and fold neighbours that are laid out back to back
@@ -673,9 +676,18 @@ bool fill_relayout_handle(Handle *h, const int64_t size[5], const int64_t src_si
           std::llabs(r.src_stride[d]) < std::llabs(r.src_stride[r.src_fast]))
         r.src_fast = d;
   }
+  if (r.src_fast == r.dst_fast && ((int64_t)r.size[4] * es) % 16 != 0) {
+    // runs along the shared contiguous dimension that are not whole 16-byte
+    // chunks (an output with 12 f16 channels): element-wise tiles over that
+    // dimension and the longest other one
+    r.src_fast = 3;
+    for (int d = 0; d < 4; ++d)
+      if (r.size[d] > r.size[r.src_fast])
+        r.src_fast = d;
+  }
   int64_t blocks = 1;
   if (r.src_fast == r.dst_fast) {
-    // the destination's channel runs are whole 16-byte chunks by construction of cp
+    // whole 16-byte chunks along the contiguous dimension (by construction of cp)
     r.mode = RELAYOUT_COPY;
     const int64_t chunks = (int64_t)r.size[2] * r.size[3] * (r.size[4] * es / 16);
     if (chunks > INT32_MAX) {
@@ -766,7 +778,7 @@ bool canon_layout(std::string s, char channel, const char *want, std::string &ou
 void layout_strides(const std::string &layout, const std::string &letters, const int64_t *sizes,
                     int64_t *strides) {
   int64_t run = 1;
-  for (int pos = 4; pos >= 0; --pos) {
+  for (int pos = (int)layout.size() - 1; pos >= 0; --pos) {
     size_t idx = letters.find(layout[pos]);
     strides[idx] = run;
     run *= sizes[idx];
@@ -1327,7 +1339,304 @@ Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
 }
 
 
+// ---- 3-D convolution ----------------------------------------------------------
+// Layout strings of six letters (rocmlir-gen's "ngc012" / "gkc012" / "ngk012",
+// rocmlir-gen.cpp:865-877; h, w, d and y, x, z are accepted for 0, 1, 2).
+bool canon_layout3(std::string s, char channel, bool filter, std::string &out) {
+  std::string r;
+  for (char raw : s) {
+    char ch = (char)std::tolower((unsigned char)raw);
+    if (ch == 'h' || ch == 'y') ch = '0';
+    else if (ch == 'w' || ch == 'x') ch = '1';
+    else if (ch == 'd' || ch == 'z') ch = '2';
+    else if (filter && ch == 'n') ch = 'k';
+    else if (!filter && channel == 'k' && ch == 'c') ch = 'k';
+    r.push_back(ch);
+  }
+  if (r.find('g') == std::string::npos) {
+    const std::string c1(1, channel);
+    if (filter)
+      r = "g" + r;
+    else if (r.size() >= 2 && r.substr(0, 2) == "n" + c1)
+      r = "ng" + c1 + r.substr(2);
+    else if (!r.empty() && r[0] == 'n' && r.back() == channel)
+      r = r.substr(0, r.size() - 1) + "g" + c1;
+    else
+      r = "g" + r;
+  }
+  std::string a = r, b = filter ? "gkc012" : std::string("ng") + channel + "012";
+  std::sort(a.begin(), a.end());
+  std::sort(b.begin(), b.end());
+  if (a != b)
+    return false;
+  out = r;
+  return true;
+}
+
+// Forward convolution over three spatial dimensions (the reference takes them
+// through the same rock.conv with a third spatial index, rocmlir-gen.cpp:171-294).
+// The contraction kernels walk two spatial dimensions, so the third is
+// unfolded into the channels by the conversion kernels: the workspace holds
+//   T[n, do, hi, wi, g, z, c] = input[n, g, c, hi, wi, do*stride_d + z*dil_d - pad_d]
+// (zero where that depth lies in the padding, c padded to whole 16-byte
+// chunks) and the filter as F[g, k, y, x, z, c], after which the problem is a
+// 2-D convolution with batch n*Do and Z*c channels per group.  Its output
+// rows are the caller's when the output's batch stride is Do depth strides
+// (channels-last layouts, or one image); otherwise it writes
+// O[n, do, ho, wo, g, k] into the workspace and a last conversion kernel
+// brings that into the caller's layout.  Kernels: [zero fill of T], one
+// conversion per (z, g) slice, the filter conversion (one per group when g
+// and k are not neighbours in the filter's layout), the contraction, [the
+// output conversion].
+Handle *make_conv3d(const OptMap &o) {
+  std::string t_all = str_or(o, "t", "");
+  std::string in_t = str_or(o, "in_type", t_all), fil_t = str_or(o, "fil_type", t_all),
+              out_t = str_or(o, "out_type", str_or(o, "out_datatype", ""));
+  static const char *req[] = {"batchsize", "in_channels", "in_h", "in_w", "in_d", "out_channels",
+                              "fil_h", "fil_w", "fil_d", "in_layout", "out_layout", "fil_layout"};
+  for (const char *k : req)
+    if (!o.count(k)) {
+      set_error(std::string("conv: missing --") + k);
+      return nullptr;
+    }
+  const std::string opn = str_or(o, "operation", "conv");
+  if (opn != "conv" && opn != "conv3d") {
+    set_error("conv: only the forward direction is built for three spatial dimensions");
+    return nullptr;
+  }
+  const int ti = parse_dtype(in_t), tf = parse_dtype(fil_t);
+  if (ti < 0 || tf < 0 || ti != tf || ti == ROCK_I32) {
+    set_error("conv: input and filter types must be given, known and equal");
+    return nullptr;
+  }
+  const int dflt_out = ti == ROCK_I8 ? ROCK_I32 : (ti == ROCK_FP8 || ti == ROCK_BF8) ? ROCK_F32 : ti;
+  const int to = out_t.empty() ? dflt_out : parse_dtype(out_t);
+  RockEpilogue epi;
+  if (to < 0 || !parse_epilogue(o, ti, to, epi)) {
+    set_error("conv: illegal input/output type combination or epilogue");
+    return nullptr;
+  }
+  if (epi.residual_op != ROCK_RES_NONE) {
+    set_error("conv: a residual tensor is not taken with three spatial dimensions");
+    return nullptr;
+  }
+  std::string fl, il, ol;
+  if (!canon_layout3(str_or(o, "fil_layout", ""), 'k', true, fl) ||
+      !canon_layout3(str_or(o, "in_layout", ""), 'c', false, il) ||
+      !canon_layout3(str_or(o, "out_layout", ""), 'k', false, ol)) {
+    set_error("conv: unsupported layout string (3-D, six dimensions with g)");
+    return nullptr;
+  }
+  const int64_t n = int_or(o, "batchsize", 0), g = int_or(o, "groupsize", 1), ct = int_or(o, "in_channels", 0),
+                kt = int_or(o, "out_channels", 0);
+  // spatial dimensions in the order 0 (h), 1 (w), 2 (d)
+  static const char *ax[3] = {"h", "w", "d"};
+  int64_t in[3], fil[3], out[3], dil[3], str[3], pl[3], pr[3];
+  for (int a = 0; a < 3; ++a) {
+    const std::string s = ax[a];
+    in[a] = int_or(o, ("in_" + s).c_str(), 0);
+    fil[a] = int_or(o, ("fil_" + s).c_str(), 0);
+    dil[a] = int_or(o, ("dilation_" + s).c_str(), 1);
+    str[a] = int_or(o, ("conv_stride_" + s).c_str(), 1);
+    const int64_t both = int_or(o, ("padding_" + s).c_str(), 0);
+    pl[a] = int_or(o, ("padding_" + s + "_l").c_str(), both);
+    pr[a] = int_or(o, ("padding_" + s + "_r").c_str(), both);
+    if (dil[a] <= 0 || str[a] <= 0 || pl[a] < 0 || pr[a] < 0) {
+      set_error("conv: dilation and stride must be positive, padding non-negative");
+      return nullptr;
+    }
+    if (in[a] <= 0 || fil[a] <= 0) {
+      set_error("conv: tensor dimensions must be positive and channels divisible by groups");
+      return nullptr;
+    }
+    if (in[a] + pl[a] + pr[a] < (fil[a] - 1) * dil[a] + 1) {
+      set_error("conv: input, including padding, is smaller than the filter");
+      return nullptr;
+    }
+    out[a] = (in[a] + pl[a] + pr[a] - (fil[a] - 1) * dil[a] - 1) / str[a] + 1;
+    int64_t given;
+    if (get_int(o, ("out_" + s).c_str(), given) && given != out[a]) {
+      set_error("conv: out_h/out_w/out_d do not match the value computed from the other parameters");
+      return nullptr;
+    }
+  }
+  if (n <= 0 || g <= 0 || ct <= 0 || kt <= 0 || ct % g != 0 || kt % g != 0) {
+    set_error("conv: tensor dimensions must be positive and channels divisible by groups");
+    return nullptr;
+  }
+  if (!bool_or(o, "layout_conversion", true)) {
+    set_error("conv: three spatial dimensions run through the conversion kernels only");
+    return nullptr;
+  }
+  const int64_t c = ct / g, k = kt / g;
+  const int64_t Hi = in[0], Wi = in[1], Di = in[2], Y = fil[0], X = fil[1], Z = fil[2], Ho = out[0], Wo = out[1],
+                Do = out[2];
+  int64_t fs[6], is[6], os[6];
+  {
+    const int64_t fsz[6] = {g, k, c, Y, X, Z}, isz[6] = {n, g, c, Hi, Wi, Di}, osz[6] = {n, g, k, Ho, Wo, Do};
+    layout_strides(fl, "gkc012", fsz, fs);
+    layout_strides(il, "ngc012", isz, is);
+    layout_strides(ol, "ngk012", osz, os);
+  }
+  const int es = dtype_size(ti), eso = dtype_size(to);
+  const int64_t cp = (c * es + 15) / 16 * 16 / es;
+  // the filter converts in one kernel when g and k fold into one dimension, else per group
+  const bool fil_folds = g == 1 || fs[0] == k * fs[1];
+  const int fil_kernels = fil_folds ? 1 : (int)g;
+  // workspace: T, F, [O]
+  const int64_t t_pix = g * Z * cp; // elements per (n, do, hi, wi)
+  const int64_t t_bytes = align256(n * Do * Hi * Wi * t_pix * es);
+  const int64_t f_bytes = align256(g * k * Y * X * Z * cp * es);
+  const bool out_direct = n == 1 || os[0] == Do * os[5];
+  const int64_t o_bytes = out_direct ? 0 : align256(n * Do * Ho * Wo * g * k * eso);
+  if (n * Do > INT32_MAX || Z * cp > INT32_MAX || t_bytes / es > ((int64_t)1 << 40)) {
+    set_error("conv: problem too large for 32-bit tile indices");
+    return nullptr;
+  }
+  // slices of T: for tap z the output depths whose input depth exists
+  struct Slice { int64_t z, g, lo, cnt; };
+  std::vector<Slice> slices;
+  bool need_fill = false;
+  for (int64_t z = 0; z < Z; ++z) {
+    const int64_t shift = z * dil[2] - pl[2]; // input depth = do * stride + shift
+    const int64_t lo = shift >= 0 ? 0 : (-shift + str[2] - 1) / str[2];
+    const int64_t hi_d = std::min(Do - 1, floor_div(Di - 1 - shift, str[2]));
+    const int64_t cnt = hi_d - lo + 1;
+    if (cnt < Do)
+      need_fill = true;
+    if (cnt > 0)
+      for (int64_t gi = 0; gi < g; ++gi)
+        slices.push_back(Slice{z, gi, lo, cnt});
+  }
+  const int first_slice = need_fill ? 1 : 0;
+  const int i_filter = first_slice + (int)slices.size(), i_conv = i_filter + fil_kernels;
+  const int count = i_conv + 1 + (out_direct ? 0 : 1);
+  const int kid = (int)int_or(o, "kernel_id", 0);
+  if (kid < 0 || kid >= count) {
+    set_error("conv: kernel_id out of range");
+    return nullptr;
+  }
+  const int ws = 4; // caller list: filter, input, output, bias, workspace
+  Handle *h = nullptr;
+  if (need_fill && kid == 0) {
+    h = utility_fill_handle(t_bytes);
+    h->ptr_map = {{ws, 0}};
+    h->problem_key = "zero fill of the unfolded input";
+  } else if (kid < i_filter) {
+    const Slice &sl = slices[kid - first_slice];
+    h = new Handle;
+    const int64_t size[5] = {n, sl.cnt, Hi, Wi, cp}, src_size[5] = {n, sl.cnt, Hi, Wi, c};
+    const int64_t stride[5] = {is[0], str[2] * is[5], is[3], is[4], is[2]};
+    const int64_t dstride[5] = {Do * Hi * Wi * t_pix, Hi * Wi * t_pix, Wi * t_pix, t_pix, 1};
+    if (!fill_relayout_handle(h, size, src_size, stride, es, dstride)) {
+      delete h;
+      return nullptr;
+    }
+    const int64_t src_off = sl.g * is[1] + (sl.lo * str[2] + sl.z * dil[2] - pl[2]) * is[5];
+    const int64_t dst_off = sl.lo * Hi * Wi * t_pix + (sl.g * Z + sl.z) * cp;
+    h->ptr_map = {{1, src_off * es}, {ws, dst_off * es}};
+    h->problem_key = "unfold input depth tap " + std::to_string(sl.z) + " group " + std::to_string(sl.g);
+  } else if (kid < i_conv) {
+    h = new Handle;
+    const int64_t gi = kid - i_filter, rows = fil_folds ? g * k : k;
+    const int64_t size[5] = {rows, Y, X, Z, cp}, src_size[5] = {rows, Y, X, Z, c};
+    const int64_t stride[5] = {fs[1], fs[3], fs[4], fs[5], fs[2]};
+    if (!fill_relayout_handle(h, size, src_size, stride, es)) {
+      delete h;
+      return nullptr;
+    }
+    h->ptr_map = {{0, gi * fs[0] * es}, {ws, t_bytes + gi * k * Y * X * Z * cp * es}};
+    h->problem_key = "relayout filter " + fl;
+  } else if (kid == i_conv) {
+    RockConvParams q;
+    std::memset(&q, 0, sizeof q);
+    q.n = (int)(n * Do); q.g = (int)g; q.c = (int)(Z * cp); q.k = (int)k;
+    q.hi = (int)Hi; q.wi = (int)Wi; q.y = (int)Y; q.x = (int)X; q.ho = (int)Ho; q.wo = (int)Wo;
+    q.stride_h = (int)str[0]; q.stride_w = (int)str[1]; q.pad_h = (int)pl[0]; q.pad_w = (int)pl[1];
+    q.dil_h = (int)dil[0]; q.dil_w = (int)dil[1];
+    q.in_cs = 1; q.in_gs = Z * cp; q.in_ws = t_pix; q.in_hs = Wi * t_pix; q.in_ns = Hi * Wi * t_pix;
+    q.fil_cs = 1; q.fil_xs = Z * cp; q.fil_ys = X * q.fil_xs; q.fil_ks = Y * q.fil_ys; q.fil_gs = k * q.fil_ks;
+    if (out_direct) {
+      q.out_ns = os[5]; q.out_gs = os[1]; q.out_ks = os[2]; q.out_hs = os[3]; q.out_ws = os[4];
+    } else {
+      q.out_ks = 1; q.out_gs = k; q.out_ws = g * k; q.out_hs = Wo * q.out_ws; q.out_ns = Ho * q.out_hs;
+    }
+    q.epi = epi;
+    h = conv_handle_from_view(q, ti, o);
+    if (!h)
+      return nullptr;
+    const bool tiled = h->kernel_name.find("generic") == std::string::npos;
+    h->kernel_name += rich_suffix(epi, tiled, o);
+    h->ptr_map = {{ws, t_bytes}, {ws, 0}, out_direct ? Handle::PtrSrc{2, 0} : Handle::PtrSrc{ws, t_bytes + f_bytes},
+                  {3, 0}, {-1, 0}};
+    std::ostringstream key;
+    const char *opname = ti == ROCK_F32 ? "conv" : ti == ROCK_F16 ? "convfp16" : ti == ROCK_BF16 ? "convbfp16"
+                       : ti == ROCK_I8 ? "convint8" : ti == ROCK_FP8 ? "convfp8_fp8" : "convbf8_bf8";
+    auto key_letters = [](const std::string &layout, bool filter) {
+      std::string r;
+      for (char ch : layout)
+        r.push_back(ch == 'g' ? 'G' : ch == 'n' ? 'N' : ch == 'c' ? 'C' : ch == 'k' ? (filter ? 'N' : 'C') : ch);
+      return r;
+    };
+    key << h->arch << '\t' << int_or(o, "num_cu", kNumCU) << '\t' << opname << " -F 1 -f " << key_letters(fl, true)
+        << " -I " << key_letters(il, false) << " -O " << key_letters(ol, false) << " -n " << n << " -c " << c
+        << " -H " << Hi << " -W " << Wi << " -k " << k << " -y " << Y << " -x " << X << " -p " << pl[0] << " -q "
+        << pl[1] << " -u " << str[0] << " -v " << str[1] << " -l " << dil[0] << " -j " << dil[1] << " -g " << g
+        // the reference's key stops here (RockTuningImpl.cpp:775-808); the depth fields keep 3-D problems apart
+        << " --in_d " << Di << " --fil_d " << Z << " --padding_d " << pl[2] << " --conv_stride_d " << str[2]
+        << " --dilation_d " << dil[2];
+    h->problem_key = key.str();
+  } else {
+    // O[n, do, ho, wo, g, k] -> the caller's layout: dimensions in the caller's
+    // order, unit ones dropped, (g, k) and neighbouring spatial dimensions folded
+    struct Dim { int64_t size, ss; };
+    std::vector<Dim> dims;
+    const int64_t osz[6] = {n, g, k, Ho, Wo, Do};
+    const int64_t oss[6] = {Do * Ho * Wo * g * k, k, 1, Wo * g * k, g * k, Ho * Wo * g * k}; // of O, letter order ngk012
+    for (char ch : ol) {
+      const size_t idx = std::string("ngk012").find(ch);
+      dims.push_back(Dim{osz[idx], oss[idx]});
+    }
+    for (size_t d = 0; d + 1 < dims.size();)
+      if (dims[d].size == 1)
+        dims.erase(dims.begin() + d);
+      else
+        ++d;
+    for (size_t d = 0; d + 1 < dims.size() && dims.size() > 5;)
+      if (dims[d].ss == dims[d + 1].size * dims[d + 1].ss) {
+        dims[d] = Dim{dims[d].size * dims[d + 1].size, dims[d + 1].ss};
+        dims.erase(dims.begin() + d + 1);
+      } else {
+        ++d;
+      }
+    if (dims.size() > 5) {
+      set_error("conv: this 3-D output layout needs more than five independent dimensions");
+      return nullptr;
+    }
+    while (dims.size() < 5)
+      dims.insert(dims.begin(), Dim{1, 0});
+    int64_t size[5], stride[5];
+    for (int d = 0; d < 5; ++d) {
+      size[d] = dims[d].size;
+      stride[d] = dims[d].ss;
+    }
+    h = new Handle;
+    if (!fill_relayout_handle(h, size, size, stride, eso)) {
+      delete h;
+      return nullptr;
+    }
+    h->ptr_map = {{ws, t_bytes + f_bytes}, {2, 0}};
+    h->problem_key = "relayout output " + ol;
+  }
+  h->kernel_count = count;
+  h->workspace_bytes = (size_t)(t_bytes + f_bytes + o_bytes);
+  h->caller_pointers = 5;
+  return h;
+}
+
 Handle *make_conv(const OptMap &o) {
+  if (o.count("in_d") || o.count("fil_d"))
+    return make_conv3d(o);
   // required keys (ConvGenerator.cpp:492-512); rocmlir-gen's "-t" sets all
   // three types at once
   std::string t_all = str_or(o, "t", "");
@@ -1956,6 +2265,39 @@ void describe_arguments(const OptMap &o, Handle *h) {
       h->args.push_back(A{tv, {G, sq, sk}});
     h->args.push_back(A{tv, {G, sq, sk}}); // bias slot
     h->args.push_back(A{tv, mat(bool_or(o, "transO", false), sq, dv)});
+    with_workspace();
+  } else if (o.count("in_d") || o.count("fil_d")) { // three spatial dimensions: six-dimensional tensors
+    std::string t_all = str_or(o, "t", "");
+    const int ti = parse_dtype(str_or(o, "in_type", t_all)), tf = parse_dtype(str_or(o, "fil_type", t_all));
+    std::string out_t = str_or(o, "out_type", str_or(o, "out_datatype", ""));
+    const int dflt = ti == ROCK_I8 ? ROCK_I32 : (ti == ROCK_FP8 || ti == ROCK_BF8) ? ROCK_F32 : ti;
+    const int to = out_t.empty() ? dflt : parse_dtype(out_t);
+    std::string fl, il, ol;
+    if (!canon_layout3(str_or(o, "fil_layout", ""), 'k', true, fl) || !canon_layout3(str_or(o, "in_layout", ""), 'c', false, il) ||
+        !canon_layout3(str_or(o, "out_layout", ""), 'k', false, ol))
+      return;
+    const int64_t n = int_or(o, "batchsize", 0), g = int_or(o, "groupsize", 1), c = int_or(o, "in_channels", 0) / g,
+                  k = int_or(o, "out_channels", 0) / g;
+    int64_t fsz[6] = {g, k, c, 0, 0, 0}, isz[6] = {n, g, c, 0, 0, 0}, osz[6] = {n, g, k, 0, 0, 0};
+    static const char *ax[3] = {"h", "w", "d"};
+    for (int a = 0; a < 3; ++a) {
+      const std::string s = ax[a];
+      const int64_t in = int_or(o, ("in_" + s).c_str(), 0), fil = int_or(o, ("fil_" + s).c_str(), 0),
+                    dil = int_or(o, ("dilation_" + s).c_str(), 1), str = int_or(o, ("conv_stride_" + s).c_str(), 1),
+                    both = int_or(o, ("padding_" + s).c_str(), 0), pl = int_or(o, ("padding_" + s + "_l").c_str(), both),
+                    pr = int_or(o, ("padding_" + s + "_r").c_str(), both);
+      fsz[3 + a] = fil;
+      isz[3 + a] = in;
+      osz[3 + a] = (in + pl + pr - (fil - 1) * dil - 1) / str + 1;
+    }
+    auto dims = [](const std::string &layout, const char *letters, const int64_t *sizes) {
+      std::vector<int64_t> d;
+      for (char ch : layout)
+        d.push_back(sizes[std::strchr(letters, ch) - letters]);
+      return d;
+    };
+    h->args = {A{tf, dims(fl, "gkc012", fsz)}, A{ti, dims(il, "ngc012", isz)}, A{to, dims(ol, "ngk012", osz)},
+               A{to == ROCK_I32 ? ROCK_I32 : ROCK_F32, {g * k}}};
     with_workspace();
   } else { // convolutions: filter, input, output in the order of their layout strings
     std::string t_all = str_or(o, "t", "");
