@@ -160,6 +160,44 @@ def test_conv_vs_torch_conv2d(oracle, case, layouts):
     assert np.array_equal(out8.astype(np.float64), want)
 
 
+CONV3D_CASES = [
+    (2, 2, 3, 4, (5, 6, 7), (3, 2, 3), (1, 2, 2), (1, 0, 2), (1, 2, 1)),
+    (1, 1, 4, 5, (6, 6, 6), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
+    (2, 1, 2, 3, (7, 5, 9), (1, 3, 5), (2, 1, 3), (0, 1, 2), (1, 1, 1)),
+]
+CONV3D_LAYOUTS = [("gkc012", "ngc012", "ngk012"), ("gk012c", "n012gc", "n012gk"), ("g012ck", "n2g01c", "ngk201")]
+
+
+@pytest.mark.parametrize("case", CONV3D_CASES)
+@pytest.mark.parametrize("layouts", CONV3D_LAYOUTS, ids=lambda l: l[1])
+def test_conv3d_vs_torch_conv3d(oracle, case, layouts):
+    """torch.nn.functional.conv3d (a library routine) on integer-valued data in
+    float64: every sum exact, so a wrong index, stride or padding side shows."""
+    n, g, c, k, ins, fs, stride, pad, dil = case
+    rng = np.random.default_rng(hash((case, layouts)) % 2 ** 31)
+    fil = rng.integers(-3, 4, (g, k, c) + fs).astype(np.float32)
+    inp = rng.integers(-3, 4, (n, g, c) + ins).astype(np.float32)
+    fl, il, ol = layouts
+    out, outs = oracle.conv3d(_to_layout(fil, "gkc012", fl), _to_layout(inp, "ngc012", il), fl, il, ol,
+                              n, g, c, k, ins, fs, stride, pad, dil)
+    ref = torch.nn.functional.conv3d(torch.from_numpy(inp.reshape((n, g * c) + ins)).double(),
+                                     torch.from_numpy(fil.reshape((g * k, c) + fs)).double(),
+                                     stride=stride, padding=pad, dilation=dil, groups=g).numpy()
+    assert ref.shape == (n, g * k) + outs
+    assert np.array_equal(out.astype(np.float64), _to_layout(ref.reshape((n, g, k) + outs), "ngk012", ol))
+
+
+def test_conv3d_with_depth_one_is_the_2d_oracle(oracle):
+    n, g, c, k, hi, wi, y, x = 2, 2, 3, 4, 6, 7, 3, 2
+    rng = np.random.default_rng(17)
+    fil = rng.integers(-3, 4, g * k * c * y * x).astype(np.float32)
+    inp = rng.integers(-3, 4, n * g * c * hi * wi).astype(np.float32)
+    want, ho, wo = oracle.conv_fwd(fil, inp, "gkcyx", "ngchw", "ngkhw", n, g, c, k, hi, wi, y, x, (2, 1), (1, 0), (1, 2))
+    got, outs = oracle.conv3d(fil, inp, "gkc012", "ngc012", "ngk012", n, g, c, k, (hi, wi, 1), (y, x, 1),
+                              (2, 1, 1), (1, 0, 0), (1, 2, 1))
+    assert outs == (ho, wo, 1) and np.array_equal(got, want)
+
+
 def _bwd_golden_cases():
     with open(os.path.join(HERE, "golden", "conv_bwd_kats.json")) as f:
         return json.load(f)
