@@ -1129,6 +1129,64 @@ Handle *make_conv_bwd_data(const OptMap &o, const ConvProblem &cp) {
 // a reduction kernel (the reference's answer is atomic adds into a zero-filled
 // f32 workspace, ConvGenerator.cpp:434-480).
 Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
+  // A strided 1x1 filter without padding touches one input pixel in
+  // stride_h * stride_w.  A first kernel gathers those into the workspace
+  // (ho x wo pixels, channels last when the channel runs are whole 16-byte
+  // chunks, else in the caller's letter order); what remains is the
+  // unit-stride problem over the gathered tensor, planned as such (a split GEMM
+  // over the tensors as they lie when the runs are whole 16-byte chunks).
+  if (cp.y == 1 && cp.x == 1 && cp.ph == 0 && cp.pw == 0 && (cp.sh > 1 || cp.sw > 1) &&
+      bool_or(o, "layout_conversion", true) && bool_or(o, "pointwise_as_gemm", true)) {
+    const int es = dtype_size(cp.ti);
+    const int kid = (int)int_or(o, "kernel_id", 0);
+    ConvProblem inner = cp;
+    inner.hi = cp.ho; inner.wi = cp.wo; inner.sh = inner.sw = 1;
+    const int64_t isz[5] = {cp.n, cp.g, cp.c, cp.ho, cp.wo};
+    if ((cp.c * es) % 16 == 0)
+      inner.il = "nhwgc"; // channel runs of whole chunks: the form the GEMM route reads best
+    layout_strides(inner.il, "ngchw", isz, inner.is);
+    const int64_t gathered = align256(cp.n * cp.g * cp.c * cp.ho * cp.wo * es);
+    OptMap o2 = o;
+    o2["kernel_id"] = std::to_string(kid == 0 ? 0 : kid - 1);
+    Handle *sub = make_conv_bwd_weight(o2, inner);
+    if (!sub)
+      return nullptr;
+    const int count = sub->kernel_count + 1;
+    const size_t workspace = (size_t)gathered + sub->workspace_bytes;
+    if (kid == 0) {
+      delete sub;
+      auto *h = new Handle;
+      int64_t size[5], stride[5];
+      for (int d = 0; d < 5; ++d) { // dimensions in the order of the gathered tensor's layout
+        const size_t idx = std::string("ngchw").find(inner.il[d]);
+        size[d] = isz[idx];
+        stride[d] = cp.is[idx] * (idx == 3 ? cp.sh : idx == 4 ? cp.sw : 1);
+      }
+      if (!fill_relayout_handle(h, size, size, stride, es)) {
+        delete h;
+        return nullptr;
+      }
+      h->ptr_map = {{1, 0}, {4, 0}};
+      h->problem_key = "gather of the input pixels a strided 1x1 filter reads";
+      h->kernel_count = count;
+      h->workspace_bytes = workspace;
+      h->caller_pointers = 5;
+      return h;
+    }
+    // the inner plan's input is the gathered tensor, its workspace lies behind it
+    for (auto &src : sub->ptr_map) {
+      if (src.source == 4)
+        src.offset += gathered;
+      else if (src.source == 1)
+        src = Handle::PtrSrc{4, src.offset};
+    }
+    if (sub->op != OP_RELAYOUT)
+      sub->problem_key = conv_problem_key(sub, o, cp, 4);
+    sub->kernel_count = count;
+    sub->workspace_bytes = workspace;
+    sub->caller_pointers = 5;
+    return sub;
+  }
   const int es = dtype_size(cp.ti);
   const int kid = (int)int_or(o, "kernel_id", 0);
   RockConvParams q;
@@ -1239,7 +1297,66 @@ Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
         h->caller_pointers = workspace ? 5 : 4;
         return h;
       }
-      delete h; // operands not in whole 16-byte chunks: the general route below
+      delete h; // operands not in whole 16-byte chunks
+      // Pixel runs that are not whole chunks (14x14 and 7x7 images in NCHW)
+      // while the channel runs are: the tensors that are not channels-last are
+      // copied into that form in the workspace and the problem is planned
+      // again over the copies (all pixels of all images then form one run).
+      const bool cl_in = cp.is[2] == 1, cl_out = cp.os[2] == 1;
+      if ((!cl_in || !cl_out) && (cp.c * es) % 16 == 0 && (cp.k * es) % 16 == 0 &&
+          bool_or(o, "layout_conversion", true)) {
+        ConvProblem inner = cp;
+        const int64_t isz[5] = {cp.n, cp.g, cp.c, cp.hi, cp.wi}, osz[5] = {cp.n, cp.g, cp.k, cp.ho, cp.wo};
+        if (!cl_in) {
+          inner.il = "nhwgc";
+          layout_strides(inner.il, "ngchw", isz, inner.is);
+        }
+        if (!cl_out) {
+          inner.ol = "nhwgk";
+          layout_strides(inner.ol, "ngkhw", osz, inner.os);
+        }
+        const int64_t x_bytes = cl_in ? 0 : align256(cp.n * cp.c * cp.hi * cp.wi * es);
+        const int64_t y_bytes = cl_out ? 0 : align256(cp.n * cp.k * cp.ho * cp.wo * es);
+        const int pre = (cl_in ? 0 : 1) + (cl_out ? 0 : 1);
+        OptMap o2 = o;
+        o2["kernel_id"] = std::to_string(std::max(0, kid - pre));
+        Handle *sub = make_conv_bwd_weight(o2, inner);
+        if (!sub)
+          return nullptr;
+        const int total = sub->kernel_count + pre;
+        const size_t ws_total = (size_t)(x_bytes + y_bytes) + sub->workspace_bytes;
+        if (kid < pre) {
+          delete sub;
+          const bool input = kid == 0 && !cl_in;
+          auto *c2 = new Handle;
+          const int64_t size_x[5] = {cp.n, cp.hi, cp.wi, cp.g, cp.c}, size_y[5] = {cp.n, cp.ho, cp.wo, cp.g, cp.k};
+          const int64_t str_x[5] = {cp.is[0], cp.is[3], cp.is[4], cp.is[1], cp.is[2]};
+          const int64_t str_y[5] = {cp.os[0], cp.os[3], cp.os[4], cp.os[1], cp.os[2]};
+          if (!fill_relayout_handle(c2, input ? size_x : size_y, input ? size_x : size_y, input ? str_x : str_y, es)) {
+            delete c2;
+            return nullptr;
+          }
+          c2->ptr_map = input ? std::vector<Handle::PtrSrc>{{1, 0}, {4, 0}}
+                              : std::vector<Handle::PtrSrc>{{2, 0}, {4, x_bytes}};
+          c2->problem_key = input ? "relayout input " + cp.il : "relayout output gradient " + cp.ol;
+          sub = c2;
+        } else {
+          for (auto &src : sub->ptr_map) {
+            if (src.source == 4)
+              src.offset += x_bytes + y_bytes;
+            else if (src.source == 1 && !cl_in)
+              src = Handle::PtrSrc{4, src.offset};
+            else if (src.source == 2 && !cl_out)
+              src = Handle::PtrSrc{4, x_bytes + src.offset};
+          }
+          if (sub->op != OP_RELAYOUT)
+            sub->problem_key = conv_problem_key(sub, o, cp, 4);
+        }
+        sub->kernel_count = total;
+        sub->workspace_bytes = ws_total;
+        sub->caller_pointers = 5;
+        return sub;
+      }
     }
   }
 

@@ -68,6 +68,8 @@ CASES = [
     (4, 1, 16, 24, 6, 6, 1, 1, (1, 1), (0, 0), (1, 1)),       # pointwise: the weight gradient is a split GEMM
     (3, 1, 64, 48, 8, 8, 1, 1, (1, 1), (0, 0), (1, 1)),
     (2, 1, 128, 192, 16, 16, 1, 1, (1, 1), (0, 0), (1, 1)),   # pointwise, more than one tile
+    (2, 1, 64, 128, 16, 16, 1, 1, (2, 2), (0, 0), (1, 1)),    # strided pointwise: a quarter of the pixels is read
+    (3, 2, 8, 8, 9, 12, 1, 1, (2, 3), (0, 0), (1, 1)),        # ... with groups, odd sizes, unequal strides
 ]
 LAYOUTS = [NHWC, NCHW, ("gyxck", "hwcgn", "hwkgn")]
 
@@ -130,10 +132,13 @@ def test_conv_bwd_weight_exact(rock, oracle, gpu, case, layouts, t, convert):
     torch.cuda.synchronize()
     ref, _, _ = oracle.conv_bwd_weight(iq, dyq, *layouts, n, g, c, k, hi, wi, y, x, stride, pad, dil)
     assert np.array_equal(to_f32(got, t), oracle.round_through(ref, CODE[t]))
-    if (y, x, c % 64, hi % 8) == (1, 1, 0, 0) and layouts in (NHWC, NCHW):
+    if (y, x, c % 64, hi % 8) == (1, 1, 0, 0) and layouts in (NHWC, NCHW) and stride == (1, 1):
         # pointwise with whole 16-byte runs: a GEMM over the tensors as they lie, its split
         # partial sums added by the reduction kernel
         assert info["kernels"][0].startswith("rock_gemm_") and not any("relayout" in k for k in info["kernels"])
+    elif (y, x, c % 64, hi % 16) == (1, 1, 0, 0) and layouts in (NHWC, NCHW) and convert:
+        # strided pointwise: the pixels read are gathered first, then the same GEMM
+        assert info["kernels"][0].startswith("rock_relayout") and info["kernels"][1].startswith("rock_gemm_")
     elif not convert and not info["kernels"][0].startswith("rock_gemm_"):
         assert len(info["kernels"]) == 1
 
