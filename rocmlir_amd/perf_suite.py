@@ -24,6 +24,7 @@ import argparse
 import json
 import shlex
 import sys
+import time
 
 
 def _flags(line):
@@ -115,7 +116,7 @@ def conv_problem(line, t, layout, direction_flag=None):
     return opts, shapes, 2.0 * n * (c // g) * k * ho * wo * y * x
 
 
-def run_problem(rock, torch, dev, opts, shapes, flops, warmup, iters):
+def run_problem(rock, torch, dev, opts, shapes, flops, warmup, iters, warm_ms=0.0):
     try:
         prog = rock.RockProgram(opts)  # every kernel of the problem and its workspace
     except rock.RockError as e:
@@ -126,6 +127,12 @@ def run_problem(rock, torch, dev, opts, shapes, flops, warmup, iters):
     args = [None if s is None else
             torch.empty(s[0], device=dev, dtype=_torch_dtype(torch, s[1])) if i == last else _rand(torch, s[0], s[1], dev)
             for i, s in enumerate(shapes)]
+    # the shader clock leaves its idle state only after some tens of milliseconds of load
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < warm_ms:
+        for _ in range(10):
+            prog.launch(*args)
+        torch.cuda.synchronize()
     ms = prog.benchmark(*args, warmup=warmup, iters=iters)
     contraction = [k.kernel_name for k in prog.kernels if k.kernel_name.startswith(("rock_conv", "rock_gemm",
                                                                                      "rock_attention"))]
@@ -143,6 +150,8 @@ def main(argv=None):
                     help="conv only: run every line forward (1), backward data (2) or backward weight (4)")
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--iters", type=int, default=20)
+    ap.add_argument("--warm-ms", type=float, default=30.0,
+                    help="keep the GPU busy with the problem for this long before timing it (clock ramp-up)")
     ap.add_argument("--max-bytes", type=float, default=8e9, help="skip problems whose tensors exceed this")
     args = ap.parse_args(argv)
 
@@ -173,7 +182,7 @@ def main(argv=None):
                 if nbytes > args.max_bytes:
                     print(json.dumps({"problem": opts, "status": "skipped", "bytes": nbytes}), flush=True)
                     continue
-                res = run_problem(rock, torch, dev, opts, shapes, flops, args.warmup, args.iters)
+                res = run_problem(rock, torch, dev, opts, shapes, flops, args.warmup, args.iters, args.warm_ms)
                 res["problem"] = opts
                 print(json.dumps(res), flush=True)
                 torch.cuda.empty_cache()
