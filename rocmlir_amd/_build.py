@@ -52,10 +52,13 @@ def device_jobs():
     return jobs
 
 
-def build(jobs=8, verbose=False):
+def build(jobs=8, verbose=False, host_only=False, only=None):
+    """host_only: relink rock_api.cpp against the code objects already built;
+    only: rebuild just the code objects whose file name contains this string."""
     os.makedirs(BUILD, exist_ok=True)
+    todo = [] if host_only else [j for j in device_jobs() if only is None or only in os.path.basename(j[-2])]
     with ThreadPoolExecutor(max_workers=jobs) as pool:
-        for out in pool.map(_run, device_jobs()):
+        for out in pool.map(_run, todo):
             if verbose and out.strip():
                 print(out)
     blobs_o = os.path.join(BUILD, "blobs.o")
@@ -72,4 +75,5 @@ def build(jobs=8, verbose=False):
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    only = [a.split("=", 1)[1] for a in sys.argv[1:] if a.startswith("--only=")]
+    print(build(verbose=True, host_only="--host-only" in sys.argv[1:], only=only[0] if only else None))

@@ -896,27 +896,51 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
     }
     const char *sa = lds + (kt % kDlStages) * STAGE;
     const char *sb = sa + A_BYTES;
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      Frag<DT> fb[NI];
+    // the fragments of MFMA step s + 1 are fetched while the MFMAs of step s run
+    Frag<DT> fa[2][MI], fb[2][NI];
+    auto fetch = [&](int s, Frag<DT> *a, Frag<DT> *b) {
 #pragma unroll
       for (int j = 0; j < NI; ++j) {
         if constexpr (LDB == LD_COLS_FAST)
-          fb[j] = dl_read_frag_km<DT, BN, RB>(sb, wn * WTN + j * 32, s, lane);
+          b[j] = dl_read_frag_km<DT, BN, RB>(sb, wn * WTN + j * 32, s, lane);
         else
-          fb[j] = dl_read_frag<DT, RB>(sb, wn * WTN + j * 32 + lrow, s, lgrp);
+          b[j] = dl_read_frag<DT, RB>(sb, wn * WTN + j * 32 + lrow, s, lgrp);
       }
 #pragma unroll
       for (int i = 0; i < MI; ++i) {
-        Frag<DT> fa;
         if constexpr (LDA == LD_COLS_FAST)
-          fa = dl_read_frag_km<DT, BM, RB>(sa, wm * WTM + i * 32, s, lane);
+          a[i] = dl_read_frag_km<DT, BM, RB>(sa, wm * WTM + i * 32, s, lane);
         else
-          fa = dl_read_frag<DT, RB>(sa, wm * WTM + i * 32 + lrow, s, lgrp);
+          a[i] = dl_read_frag<DT, RB>(sa, wm * WTM + i * 32 + lrow, s, lgrp);
+      }
+    };
+    fetch(0, fa[0], fb[0]);
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      if (s + 1 < STEPS)
+        fetch(s + 1, fa[(s + 1) & 1], fb[(s + 1) & 1]);
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < NI; ++j)
-          mma32x32<DT>(fb[j], fa, acc[i][j]);
+          mma32x32<DT>(fb[s & 1][j], fa[s & 1][i], acc[i][j]);
+    }
+    // Issue order for the scheduler: the first step's fragment reads, then per
+    // step one LDS read of the next step's fragments after every MFMA until
+    // they are all out, then the step's remaining MFMAs.
+    if constexpr (LDA != LD_COLS_FAST && LDB != LD_COLS_FAST && MI * NI >= MI + NI) {
+      __builtin_amdgcn_sched_group_barrier(0x100, MI + NI, 0);
+#pragma unroll
+      for (int s = 0; s + 1 < STEPS; ++s) {
+#pragma unroll
+        for (int r = 0; r < MI + NI; ++r) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        if constexpr (MI * NI > MI + NI)
+          __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - (MI + NI), 0);
       }
+      __builtin_amdgcn_sched_group_barrier(0x008, MI * NI, 0);
     }
   }
   // drain the out-of-range loads issued for steps >= nk before the LDS is released
