@@ -249,3 +249,26 @@ def test_conv_i8_dequantise_per_tensor(rock, oracle, gpu):
                         NHWC, True, 39, out_dtype="f16", scale=1.2207e-4)
     want = oracle.round_through(oracle.dequantize(ref, 1.2207e-4, 0), CODE["f16"])
     assert np.array_equal(to_f32(out, "f16"), want)
+
+
+# NCHW-style outputs (pixels contiguous per channel) whose pixel runs are whole
+# 16-byte chunks leave the tiled kernels as 16-byte vectors of consecutive
+# pixels: one- and four-byte output elements (the two-byte ones run in every
+# NCHW case above), with and without the layout-conversion kernels in front.
+@pytest.mark.parametrize("in_layouts", [NCHW, ("gkyxc", "nhwgc", "ngkhw")], ids=["nchw", "nhwc-in"])
+@pytest.mark.parametrize("t,od", [("i8", "i8"), ("i8", "i32"), ("f16", "f32"), ("f16", "fp8")])
+def test_conv_pixel_contiguous_output_vector_store_exact(rock, oracle, gpu, t, od, in_layouts):
+    n, g, c, k, hi, wi = 3, 1, 32, 72, 16, 16
+    if od == "i8":
+        out, _, ref = _run(rock, oracle, gpu, t, n, g, c, k, hi, wi, 3, 3, (1, 1), (1, 1), (1, 1), in_layouts, True,
+                           141, out_dtype="i8", scale=0.001, quant_scale=0.5, out_zero_point=-3)
+        want = oracle.quantize_i8(oracle.dequantize(ref, 0.001, 0), 0.5, -3)
+        assert np.array_equal(out.cpu().numpy().ravel(), want.ravel())
+    elif od == "i32":
+        out, _, ref = _run(rock, oracle, gpu, t, n, g, c, k, hi, wi, 3, 3, (1, 1), (1, 1), (1, 1), in_layouts, True, 142)
+        assert np.array_equal(out.cpu().numpy().ravel(), ref.ravel())
+    else:
+        out, _, ref = _run(rock, oracle, gpu, t, n, g, c, k, hi, wi, 3, 3, (1, 1), (1, 1), (1, 1), in_layouts, True,
+                           143, out_dtype=od, scale=0.25)
+        want = oracle.round_through(np.asarray(ref, np.float32) * np.float32(0.25), CODE[od])
+        assert np.array_equal(to_f32(out, od), want)

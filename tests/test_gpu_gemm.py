@@ -256,3 +256,31 @@ def test_gemm_split_over_blocks_exact(rock, oracle, gpu, t, od, tA, tB):
                           split_k=False)
     assert len(info["kernels"]) == 1
     assert np.array_equal(to_f32(out, od), oracle.round_through(ref, CODE[od]))
+
+
+# Transposed C with rows of whole 16-byte chunks leaves the tiled kernels as
+# 16-byte vectors of consecutive m (the path NCHW-style convolution outputs
+# take as well): every output element size, every tile, a batch, ragged N.
+@pytest.mark.parametrize("tile", ["256,256", "128,128", "64,64"])
+@pytest.mark.parametrize("t,od", [("f16", "f16"), ("f16", "f32"), ("bf16", "bf16"), ("f16", "fp8"), ("f16", "bf8"),
+                                  ("i8", "i32"), ("i8", "f16"), ("f32", "f32")])
+def test_gemm_transposed_output_vector_store_exact(rock, oracle, gpu, t, od, tile):
+    G, M, N, K = 2, 304, 88, 96
+    info = {}
+    epi = dict(scale=0.25) if od != "i32" else {}
+    out, _, ref = _run_case(rock, oracle, gpu, t, G, M, N, K, False, True, True, True, 131, out_dtype=od,
+                            perf_config="v2:%s,8,64,16,8,1,1,1" % tile, info=info, **epi)
+    assert "_fast" in info["kernel_name"] and tile.replace(",", "x") in info["kernel_name"]
+    if od == "i32":
+        assert np.array_equal(out.cpu().numpy().ravel(), ref.ravel())
+    else:
+        want = oracle.round_through(np.asarray(ref, np.float32) * np.float32(0.25), CODE[od])
+        assert np.array_equal(to_f32(out, od), want)
+
+
+def test_gemm_transposed_output_requantised_to_i8(rock, oracle, gpu):
+    G, M, N, K = 1, 128, 80, 64
+    out, od, ref = _run_case(rock, oracle, gpu, "i8", G, M, N, K, False, True, True, True, 133, out_dtype="i8",
+                             scale=0.001, quant_scale=0.5, out_zero_point=-3)
+    want = oracle.quantize_i8(oracle.dequantize(ref, 0.001, 0), 0.5, -3)
+    assert np.array_equal(out.cpu().numpy().ravel(), want.ravel())
