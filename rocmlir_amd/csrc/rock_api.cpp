@@ -225,7 +225,13 @@ const Tile *pick_tile(int64_t M, int64_t N, int G, bool conv, const std::string 
     // co-resident blocks share one CU's matrix cores, so what counts is the
     // largest number of tiles any CU has to work through
     int64_t per_cu = (tiles + kNumCU - 1) / kNumCU;
-    double cost = (double)per_cu * t.bm * t.bn / t.efficiency;
+    // The 256x128 tile's figure comes from GEMMs.  As an implicit-GEMM
+    // convolution tile it lost to 128x128 on every problem of the reference's
+    // convolution list where this model had preferred it (13 of 40, by 4-30 %):
+    // one resident block per CU leaves the im2col address work of its loader
+    // waves with nothing to hide behind.
+    const double efficiency = (conv && t.bm == 256) ? 0.62 : t.efficiency;
+    double cost = (double)per_cu * t.bm * t.bn / efficiency;
     // a compute unit with a single four-wave block resident (one wave per
     // SIMD) cannot keep its matrix pipes busy: nothing overlaps a wave's LDS
     // reads and barriers

@@ -298,7 +298,7 @@ def test_backward_convolution_plans(rock):
     s3 = s2.replace("--fil_h 3 --fil_w 3", "--fil_h 1 --fil_w 1").replace("--padding_h 1 --padding_w 1",
                                                                           "--padding_h 0 --padding_w 0")
     names = [rock.RockKernel(s3 + " --kernel_id %d" % i).kernel_name for i in range(rock.RockKernel(s3).kernel_count)]
-    assert names == ["rock_fill_zero", "rock_relayout_b2", "rock_conv_f16_256x128_fast"]
+    assert names == ["rock_fill_zero", "rock_relayout_b2", "rock_conv_f16_128x128_fast"]
     # tensors as they lie: one element-wise kernel per phase, no workspace pointer
     k = rock.RockKernel(s2 + " --layout_conversion false")
     assert (k.kernel_count, k.workspace_bytes, k.caller_pointers) == (4, 0, 4)
