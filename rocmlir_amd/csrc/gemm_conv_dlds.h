@@ -815,7 +815,9 @@ __device__ __forceinline__ void dl_epilogue(typename MmaTraits<DT>::Acc (&acc)[M
           int64_t row_off, n_stride;
           bool vec_ok;
           out_row_addr(p, g, m, Cptr, row_off, n_stride, vec_ok);
-          *(v4i *)((char *)Cptr + (row_off + n) * ES) = d;
+          // streaming hint: the kernel never reads its output back, and the burst of
+          // whole-row stores that every block issues at the same moment drains faster
+          __builtin_nontemporal_store(d, (v4i *)((char *)Cptr + (row_off + n) * ES));
         }
       }
     }
