@@ -161,7 +161,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-headline", action="store_true", help="skip the other four configs")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
-    ap.add_argument("--traffic-bytes", type=float, default=134.5e6,
+    ap.add_argument("--traffic-bytes", type=float, default=134.7e6,
                     help="HBM bytes per launch of the headline kernel: FETCH_SIZE + WRITE_SIZE of "
                          "rocprofv3 --pmc runs of this command, each scaled by the same counter's reading "
                          "for a plain copy (--calibrate-copy); the default is the committed measurement "
