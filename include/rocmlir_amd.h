@@ -156,8 +156,9 @@ ROCMLIR_AMD_API MiirStatus rockamdGetArgumentInfo(MiirHandle handle, int index, 
 
 /* perf-config string of the selected kernel in the reference's grammar
  * ("v2:MPB,NPB,KpackPB,MPW,MnPerXdl,Kpack,splitK,forceUnroll,1" or
- * "attn:v1:...", RockAttrDefs.td:241-329).  strncpy semantics, returns the
- * full length like mlirRockTuningParamToString (Rock.h:60-75). */
+ * "attn:v1:...", RockAttrDefs.td:241-329).  Copies what fits, always
+ * terminates the buffer and returns the full length like
+ * mlirRockTuningParamToString (Rock.h:60-75). */
 ROCMLIR_AMD_API size_t rockamdGetPerfConfig(MiirHandle handle, char *buffer, size_t buffer_size);
 
 /* Tuning problem key, "<arch>\t<numCU>\t<problem>" in the reference's format
@@ -202,16 +203,22 @@ ROCMLIR_AMD_API MiirStatus rockamdSetZeroPoint(MiirHandle handle, int32_t zero_p
 typedef void *RockamdTuningSpace;
 typedef void *RockamdTuningTable;
 
-/* RocmlirTuningParamSetKind (RockEnums.h:19-23); both kinds return the same short list. */
-enum { ROCKAMD_TUNING_QUICK = 0, ROCKAMD_TUNING_FULL = 1 };
+/* RocmlirTuningParamSetKind (RockEnums.h:19-23).  Quick: the built-in table's
+ * choice and its two likeliest alternatives; Full: one entry per kernel the
+ * problem can run on; Exhaustive: Full, and every tile once more as its twin
+ * with the rolled epilogue (eighth field, forceUnroll, 0). */
+enum { ROCKAMD_TUNING_QUICK = 0, ROCKAMD_TUNING_FULL = 1, ROCKAMD_TUNING_EXHAUSTIVE = 2 };
 /* RocmlirSplitKSelectionLikelihood (RockEnums.h:26) */
 enum { ROCKAMD_SPLITK_NEVER = 0, ROCKAMD_SPLITK_MAYBE = 1, ROCKAMD_SPLITK_ALWAYS = 2 };
 
 /* mlirRockTuningSpaceCreate / mlirRockTuningGetNumParams /
  * mlirRockTuningParamGet + mlirRockTuningParamToString / mlirRockTuningSpaceDestroy
- * (Rock.h:39-84).  Entry 0 is the kernel the built-in table picks.  ToString
- * copies like strncpy (no terminator if the buffer is too small) and returns
- * the full length, (size_t)-1 for a bad position. */
+ * (Rock.h:39-84).  Entry 0 is the kernel the built-in table picks.  GEMM and
+ * convolution entries are "v2:" strings, attention entries "attn:v1:" strings
+ * (RockAttrDefs.td:241-329); both are accepted back by "--perf_config" and
+ * rockamdTuningSetFromStr.  ToString copies what fits, always terminates the
+ * buffer and returns the full length ((size_t)-1 for a bad position): a
+ * result >= buffer_size means the text was cut. */
 ROCMLIR_AMD_API RockamdTuningSpace rockamdTuningSpaceCreate(MiirHandle handle, int kind);
 ROCMLIR_AMD_API unsigned rockamdTuningGetNumParams(RockamdTuningSpace space);
 ROCMLIR_AMD_API size_t rockamdTuningParamToString(RockamdTuningSpace space, unsigned pos, char *buffer,
@@ -234,6 +241,26 @@ ROCMLIR_AMD_API void rockamdTuningTableDestroy(RockamdTuningTable table);
 ROCMLIR_AMD_API int rockamdTuningUpdateTable(RockamdTuningTable table, const char *problem_key,
                                              const char *perf_config, float time);
 ROCMLIR_AMD_API int rockamdTuningSetFromTable(RockamdTuningTable table, MiirHandle handle);
+
+/* mlirIsModuleFusible (Rock.h:145-147, RockTuningImpl.cpp:1010-1015): may the
+ * handle's element-wise tail (scale, bias, residual, activation) stay fused
+ * when the problem runs under `perf_config`?  The reference says no when the
+ * string asks for a split reduction, whose partial sums meet through atomic
+ * adds; here a requested split sums its partial tiles inside the block before
+ * the epilogue, so the answer is 1 for every string the problem resolves
+ * under and 0 only for a NULL handle or string. */
+ROCMLIR_AMD_API int rockamdIsFusible(MiirHandle handle, const char *perf_config);
+
+/* mlirGetNumPrefillArgs / mlirGetPrefillArgsInfo (Rock.h:149-158): arguments
+ * whose memory must hold an initial value before the launch.  The reference
+ * needs a zero-filled output for its atomic split-K; no kernel of this
+ * library accumulates into memory it has not written (split reductions go
+ * through a workspace and a reduction kernel, the zero fill of the strided
+ * backward-data phases is a kernel of the problem's own list), so the count
+ * is 0 and the info call writes nothing. */
+ROCMLIR_AMD_API size_t rockamdGetNumPrefillArgs(MiirHandle handle);
+ROCMLIR_AMD_API void rockamdGetPrefillArgsInfo(MiirHandle handle, size_t *indices, float *init_values,
+                                               size_t length);
 
 /* mlirIsSplitKFaster (Rock.h:136-142, RockTuningImpl.cpp:962-1008), answered
  * for this library's split-K kernel (K divided over the waves of one block):

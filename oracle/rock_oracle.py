@@ -170,11 +170,14 @@ def conv_out_dim(in_len, fil_len, pad_l, pad_r, stride, dil):
 
 def conv_fwd(fil, inp, fil_layout, in_layout, out_layout, n, g, c, k, hi, wi,
              y, x, stride=(1, 1), pad=(0, 0), dil=(1, 1), out_range=None,
-             threads=0):
+             threads=0, pad_r=None):
     """c and k are PER-GROUP channel counts.  Layout strings: permutations of
-    'gkcyx' / 'ngchw' / 'ngkhw'.  Returns (flat output, ho, wo)."""
-    ho = conv_out_dim(hi, y, pad[0], pad[0], stride[0], dil[0])
-    wo = conv_out_dim(wi, x, pad[1], pad[1], stride[1], dil[1])
+    'gkcyx' / 'ngchw' / 'ngkhw'.  `pad` is the top / left padding and, unless
+    `pad_r` gives the bottom / right one, that one too.  Returns (flat output,
+    ho, wo)."""
+    pad_r = pad if pad_r is None else pad_r
+    ho = conv_out_dim(hi, y, pad[0], pad_r[0], stride[0], dil[0])
+    wo = conv_out_dim(wi, x, pad[1], pad_r[1], stride[1], dil[1])
     d = ConvDims(n, g, c, k, hi, wi, y, x, ho, wo, stride[0], stride[1],
                  pad[0], pad[1], dil[0], dil[1])
     total = n * g * k * ho * wo

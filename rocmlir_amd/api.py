@@ -105,6 +105,12 @@ def load_library():
                                            C.POINTER(C.c_int),
                                            C.POINTER(C.c_int32),
                                            C.POINTER(C.c_int64)]
+        L.rockamdIsFusible.restype = C.c_int
+        L.rockamdIsFusible.argtypes = [vp, C.c_char_p]
+        L.rockamdGetNumPrefillArgs.restype = sz
+        L.rockamdGetNumPrefillArgs.argtypes = [vp]
+        L.rockamdGetPrefillArgsInfo.restype = None
+        L.rockamdGetPrefillArgsInfo.argtypes = [vp, C.POINTER(sz), C.POINTER(C.c_float), sz]
         L.rockamdIsSplitKFaster.restype = C.c_int
         L.rockamdIsSplitKFaster.argtypes = [C.c_int64] * 5 + [C.c_int]
         _lib = L
@@ -222,11 +228,14 @@ class RockKernel:
         return g.value, l.value
 
     # ---- tuning (mlir-c/Dialect/Rock.h:39-117) -------------------------------
-    def tuning_space(self, full=False):
+    TUNING_KINDS = {"quick": 0, "full": 1, "exhaustive": 2}
+
+    def tuning_space(self, kind="full"):
         """perf_config strings of the kernels this problem can run on; the
-        first is the built-in table's choice."""
+        first is the built-in table's choice.  kind: "quick" (at most three
+        entries), "full" (every kernel) or "exhaustive" (RockEnums.h:19-23)."""
         L = load_library()
-        sp = L.rockamdTuningSpaceCreate(self._h, 1 if full else 0)
+        sp = L.rockamdTuningSpaceCreate(self._h, self.TUNING_KINDS[kind])
         if not sp:
             raise RockError("rockamdTuningSpaceCreate failed")
         try:
@@ -479,16 +488,19 @@ def conv2d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize,
            scale=None, zero_point=0, bias=None, relu=False, quant_scale=None,
            out_zero_point=0, activation=None, clip=None, residual=None,
            residual_op="add", out=None, perf_config=None, stream=None,
-           info=None):
+           info=None, padding_r=None):
     """Forward convolution; tensors are flat device buffers laid out as the
     layout strings say (Miir / rocmlir-gen spelling, e.g. 'gkyxc', 'nhwgc',
     'NGCHW').  Epilogue arguments as for gemm(); the residual is laid out
-    like the output.  Returns the flat output tensor.  A dict passed as `info`
+    like the output.  `padding` is the top / left padding and, unless
+    `padding_r` gives the bottom / right one (--padding_h_r / --padding_w_r),
+    that one too.  Returns the flat output tensor.  A dict passed as `info`
     receives the name and perf_config of the kernel that ran."""
     import torch
     t = _dtype_name(inp.dtype)
-    ho = (in_h + 2 * padding[0] - (fil_h - 1) * dilation[0] - 1) // stride[0] + 1
-    wo = (in_w + 2 * padding[1] - (fil_w - 1) * dilation[1] - 1) // stride[1] + 1
+    pr = padding if padding_r is None else padding_r
+    ho = (in_h + padding[0] + pr[0] - (fil_h - 1) * dilation[0] - 1) // stride[0] + 1
+    wo = (in_w + padding[1] + pr[1] - (fil_w - 1) * dilation[1] - 1) // stride[1] + 1
     opts = ("--operation conv --arch gfx950 --in_type %s --fil_type %s"
             " --fil_layout %s --in_layout %s --out_layout %s --batchsize %d"
             " --groupsize %d --in_channels %d --out_channels %d --in_h %d"
@@ -499,6 +511,8 @@ def conv2d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize,
                batchsize, groupsize, in_channels, out_channels, in_h, in_w, ho,
                wo, fil_h, fil_w, dilation[0], dilation[1], stride[0], stride[1],
                padding[0], padding[1]))
+    if padding_r is not None:
+        opts += " --padding_h_r %d --padding_w_r %d" % (pr[0], pr[1])
     if out_dtype is not None:
         opts += " --out_type %s" % out_dtype
     if perf_config:

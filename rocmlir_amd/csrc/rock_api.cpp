@@ -363,13 +363,34 @@ void apply_tile_grid(const Tile &t, int64_t M, int64_t N, int G, int &tiles_m, i
   grid = (uint32_t)total;
 }
 
-std::string perf_string(const Tile &t, int es) {
+// field `index` (0-based) of "--perf_config [v2:]a,b,c,...", or dflt
+int64_t perf_field(const OptMap &o, int index, int64_t dflt) {
+  std::string pc = str_or(o, "perf_config", "");
+  if (pc.rfind("v2:", 0) == 0)
+    pc = pc.substr(3);
+  else if (pc.find(':') != std::string::npos)
+    return dflt; // another grammar (attn:v1:...)
+  std::istringstream iss(pc);
+  std::string part;
+  for (int i = 0; std::getline(iss, part, ','); ++i)
+    if (i == index) {
+      char *end = nullptr;
+      long long v = std::strtoll(part.c_str(), &end, 10);
+      return (end != part.c_str() && *end == '\0') ? v : dflt;
+    }
+  return dflt;
+}
+
+std::string perf_string(const Tile &t, int es, const OptMap *o = nullptr) {
   // v2:MPB,NPB,KpackPB,MPW,MnPerXdl,Kpack,splitK,forceUnroll,1
+  // forceUnroll: 1 = the kernel whose epilogue is unrolled over its
+  // accumulators wherever the problem's epilogue allows it, 0 = the "_e" twin
+  // with the rolled epilogue whatever the epilogue (see rich_suffix)
   int kpack = 16 / es;
   int kpack_per_block = 128 / 16; // 128 K bytes per stage row, 16-byte chunks
   char buf[96];
-  std::snprintf(buf, sizeof buf, "v2:%d,%d,%d,%d,%d,%d,1,1,1", t.bm, t.bn, kpack_per_block,
-                t.bm / t.waves_m, 16, kpack);
+  std::snprintf(buf, sizeof buf, "v2:%d,%d,%d,%d,%d,%d,1,%d,1", t.bm, t.bn, kpack_per_block,
+                t.bm / t.waves_m, 16, kpack, (o && perf_field(*o, 7, 1) == 0) ? 0 : 1);
   return buf;
 }
 
@@ -389,6 +410,17 @@ std::string forced_tile(const OptMap &o) {
   return "";
 }
 
+// true when "--perf_config [v2:]MPB,NPB,..." names exactly this block tile
+// (the first two fields; later fields of a reference-style string, such as
+// MPerWave = 32, must not match)
+bool requested_tile_is(const OptMap &o, int bm, int bn) {
+  std::string pc = str_or(o, "perf_config", "");
+  if (pc.rfind("v2:", 0) == 0)
+    pc = pc.substr(3);
+  int a = 0, b = 0;
+  return std::sscanf(pc.c_str(), "%d,%d", &a, &b) == 2 && a == bm && b == bn;
+}
+
 void default_epilogue(RockEpilogue &e, int out_dtype) {
   std::memset(&e, 0, sizeof e);
   e.scale = 1.0f;
@@ -405,9 +437,10 @@ int64_t align256(int64_t bytes) { return (bytes + 255) / 256 * 256; }
 // transcendental activation needs.  The element-wise kernels handle both in
 // one.
 const char *rich_suffix(const RockEpilogue &e, bool tiled_kernel, const OptMap &o) {
-  // "-rolled_epilogue true" asks for the twin regardless (it handles every epilogue)
+  // "-rolled_epilogue true", or a perf_config whose eighth field (forceUnroll)
+  // is 0, asks for the twin regardless (it handles every epilogue)
   return tiled_kernel && (e.residual_op != ROCK_RES_NONE || e.activation > ROCK_ACT_CLIP ||
-                          bool_or(o, "rolled_epilogue", false)) ? "_e" : "";
+                          bool_or(o, "rolled_epilogue", false) || perf_field(o, 7, 1) == 0) ? "_e" : "";
 }
 
 // The contraction kernels take five pointers: two operands, the output, the
@@ -460,7 +493,7 @@ bool plan_gemm_kernel(Handle *h, RockGemmParams &p, int code, int es, const OptM
     tile = &kSplitKTile;
     split_k = 4;
   }
-  if (fast && str_or(o, "perf_config", "").find("32,32,") != std::string::npos) {
+  if (fast && requested_tile_is(o, kSplitKTile.bm, kSplitKTile.bn)) {
     tile = &kSplitKTile; // "-perf_config v2:32,32,..." asks for it explicitly
     split_k = 4;
   }
@@ -472,13 +505,48 @@ bool plan_gemm_kernel(Handle *h, RockGemmParams &p, int code, int es, const OptM
                    rich_suffix(p.epi, tiled, o);
   h->blob_name = std::string("gemm_") + operand_name(code);
   set_contraction_pointers(h, p.epi);
-  h->perf_config = perf_string(*tile, es);
+  h->perf_config = perf_string(*tile, es, &o);
   if (split_k > 1) { // the reference's grammar has a splitK field (7th)
     char buf[96];
     std::snprintf(buf, sizeof buf, "v2:32,32,4,32,32,%d,%d,1,1", 16 / es, split_k);
     h->perf_config = buf;
   }
   return tiled;
+}
+
+// ---- attention kernel variants and their perf_config strings ---------------
+// "attn:v1:MPB_G0,MPB_G1,NPB_G0,KpackPB,MPW,MnPerXdl,Kpack,forceUnroll"
+// (RockAttrDefs.td:241-329; G0 M tiles seq_k, G1 M the head dimension, G0 N
+// seq_q).  The hand-written kernels all take 64 keys x 128 queries per step;
+// what a string selects is the head-dimension instantiation (MPB_G1 = 64 or
+// 128), the element-wise kernel (KpackPB = 1) and, through forceUnroll, the
+// order of work inside a key tile: 1 = the next tile's score MFMAs are issued
+// ahead of this tile's softmax (only without bias / scale tensor and with a
+// non-negative scale), 0 = scores, softmax, PV per tile.
+struct AttnVariant {
+  const char *kind; // kernel-name suffix
+  int kpack_pb, force_unroll;
+};
+const AttnVariant kAttnVariants[] = {{"fast", 8, 1}, {"fast_bias", 8, 0}, {"generic", 1, 1}};
+
+std::string attn_perf_string(const AttnVariant &v, int dmax) {
+  char buf[96];
+  std::snprintf(buf, sizeof buf, "attn:v1:64,%d,128,%d,32,32,%d,%d", dmax, v.kpack_pb, v.kpack_pb == 1 ? 1 : 8,
+                v.force_unroll);
+  return buf;
+}
+
+// Parses "attn:v1:..." (eight fields); false when the string is another grammar or malformed.
+bool parse_attn_perf(const std::string &pc, int &dmax, int &kpack_pb, int &force_unroll) {
+  if (pc.rfind("attn:v1:", 0) != 0)
+    return false;
+  int f[8];
+  if (std::sscanf(pc.c_str() + 8, "%d,%d,%d,%d,%d,%d,%d,%d", &f[0], &f[1], &f[2], &f[3], &f[4], &f[5], &f[6], &f[7]) != 8)
+    return false;
+  dmax = f[1];
+  kpack_pb = f[3];
+  force_unroll = f[7];
+  return true;
 }
 
 // ---- GEMM -----------------------------------------------------------------
@@ -536,7 +604,7 @@ Handle *make_gemm(const OptMap &o) {
   p.b_gs = K * N; p.b_ks = tB ? 1 : N; p.b_ns = tB ? K : 1;
   p.c_gs = M * N; p.c_ms = tC ? 1 : N; p.c_ns = tC ? M : 1;
 
-  plan_gemm_kernel(h, p, code, dtype_size(ta), o);
+  const bool vector_kernel = plan_gemm_kernel(h, p, code, dtype_size(ta), o);
   // problem key (RockTuningImpl.cpp:808-862)
   auto set_key = [&](Handle *hh) {
     std::ostringstream k;
@@ -557,10 +625,16 @@ Handle *make_gemm(const OptMap &o) {
     const RockEpilogue &e = p.epi;
     const bool identity = e.scale == 1.0f && !e.has_bias && e.activation == ROCK_ACT_NONE &&
                           e.residual_op == ROCK_RES_NONE && (tc == ROCK_F32 || tc == ROCK_F16 || tc == ROCK_BF16);
-    const bool tiled = h->kernel_name.find("_fast") != std::string::npos;
+    // any vector storage, including the K-contiguous one for which the planner
+    // has just chosen the split over the waves of a block: the sub-problems
+    // are planned again below and may still take that kernel, now S times over
+    const bool tiled = vector_kernel;
     const int64_t tiles64 = (int64_t)ceil_div(M, 64) * ceil_div(N, 64);
+    // ... unless that kernel's 32x32 tiles already occupy half the chip by themselves
+    const bool wave_split = h->kernel_name.find(kSplitKTile.suffix) != std::string::npos;
+    const bool wave_split_fills = wave_split && (int64_t)ceil_div(M, 32) * ceil_div(N, 32) * 2 > kNumCU;
     int64_t S = 1;
-    if (G == 1 && is_float_in(ta) && is_float_in(tb) && identity && tiled && tiles64 * 4 <= kNumCU &&
+    if (G == 1 && is_float_in(ta) && is_float_in(tb) && identity && tiled && !wave_split_fills && tiles64 * 4 <= kNumCU &&
         forced_tile(o).empty() && bool_or(o, "split_k", true)) {
       const int64_t want = std::min<int64_t>(2 * kNumCU / tiles64, K / 512);
       for (int64_t d = want; d >= 2; --d)
@@ -857,7 +931,7 @@ bool select_view_conv_kernel(Handle *h, RockConvParams &p, int ti, const OptMap 
   h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + tile->suffix;
   h->blob_name = std::string("gemm_") + dtype_name(ti);
   h->num_pointers = 5;
-  h->perf_config = perf_string(*tile, es);
+  h->perf_config = perf_string(*tile, es, &o);
   return true;
 }
 
@@ -2025,7 +2099,7 @@ Handle *make_conv(const OptMap &o) {
   h->num_pointers = 5;
   if (!planned)
     set_contraction_pointers(h, p.epi);
-  h->perf_config = perf_string(*tile, es);
+  h->perf_config = perf_string(*tile, es, &o);
 
   // Window-resident kernel (conv_direct.h), chosen by "-perf_config
   // v2:224,128,...": stride 1, dilation 1, a filter of more than one tap,
@@ -2040,10 +2114,12 @@ Handle *make_conv(const OptMap &o) {
     const int64_t th = std::min<int64_t>(ho, wo > 0 ? kDirectTilePixels / wo : 0);
     const int64_t row_pitch = ((wi + 2 * pw) * cbytes + 1023) / 1024 * 1024; // whole 1 KiB load slabs
     const int64_t window = (th + 2 * (y - 1)) * row_pitch;
+    // the kernel sizes its window from the left / top padding alone: both sides must be equal
     const bool direct_ok = fast && sh == 1 && sw == 1 && dh == 1 && dw == 1 && y * x > 1 &&
+                           ph_r == ph && pw_r == pw &&
                            cbytes >= 128 && cbytes <= 1024 && (cbytes & (cbytes - 1)) == 0 &&
                            th >= 1 && window <= kDirectWindowBytes && row_pitch <= 32 * 1024;
-    const bool asked = str_or(o, "perf_config", "").find("224,128,") != std::string::npos;
+    const bool asked = requested_tile_is(o, kDirectTilePixels, 128);
     if (direct_ok && asked) {
       // rows per tile: the most that fit, unless a slightly shorter tile fills
       // the last round of blocks better (cost = rounds x (rows + ~2 rows of
@@ -2226,10 +2302,24 @@ Handle *make_attention(const OptMap &o) {
                     sk * p.k_js * 2 < ((int64_t)1 << 31) && sk * p.v_js * 2 < ((int64_t)1 << 31) &&
                     // the bias gather indexes one g slice with 32-bit element offsets
                     ((!has_bias && !has_scale_t) || sq * sk < ((int64_t)1 << 31));
-  const int dmax = (dqk <= 64 && dv <= 64) ? 64 : 128;
+  int dmax = (dqk <= 64 && dv <= 64) ? 64 : 128;
+  const bool plain_ok = !p.has_bias && !has_scale_t && p.scale >= 0.0f;
+  const AttnVariant *variant = !fast ? &kAttnVariants[2] : plain_ok ? &kAttnVariants[0] : &kAttnVariants[1];
+  {
+    // a perf_config that names a kernel this problem can run on selects it;
+    // anything else falls back to the table (AffixTuningParameters.cpp:129-141)
+    int want_d, want_kpack, want_unroll;
+    if (parse_attn_perf(str_or(o, "perf_config", ""), want_d, want_kpack, want_unroll)) {
+      if ((want_d == 64 || want_d == 128) && want_d >= dmax)
+        dmax = want_d;
+      if (want_kpack == 1)
+        variant = &kAttnVariants[2];
+      else if (fast && want_kpack == 8)
+        variant = (want_unroll != 0 && plain_ok) ? &kAttnVariants[0] : &kAttnVariants[1];
+    }
+  }
   char name[96];
-  std::snprintf(name, sizeof name, "rock_attention_%s_d%dx%d_%s", dtype_name(ty), dmax, dmax,
-                !fast ? "generic" : (!p.has_bias && !has_scale_t && p.scale >= 0.0f) ? "fast" : "fast_bias");
+  std::snprintf(name, sizeof name, "rock_attention_%s_d%dx%d_%s", dtype_name(ty), dmax, dmax, variant->kind);
   h->kernel_name = name;
   h->blob_name = "attention";
   // kernel pointers: Q, K, V, scale tensor, bias, O; a caller passes the scale
@@ -2245,7 +2335,7 @@ Handle *make_attention(const OptMap &o) {
   h->grid_size = (uint32_t)total;
   // attn:v1:MPB_G0,MPB_G1,NPB_G0,KpackPB,MPW,MnPerXdl,Kpack,forceUnroll
   // (G0 M tiles seq_k, G0 N tiles seq_q)
-  h->perf_config = "attn:v1:64," + std::to_string(dmax) + ",128,8,32,32,8,1";
+  h->perf_config = attn_perf_string(*variant, dmax);
   {
     std::ostringstream key;
     auto tf = [](bool b) { return b ? "true" : "false"; };
@@ -2506,14 +2596,26 @@ Handle *build_handle(const OptMap &o) {
 // its parameter grid instead (createGemmTuningRangeBF / the quick lists,
 // RockTuningImpl.cpp:461-548); here the grid is the handful of hand-written
 // tiles.
-std::vector<std::string> tuning_candidates(const Handle &h) {
+std::vector<std::string> tuning_candidates(const Handle &h, int kind) {
   std::vector<std::string> requests;
   requests.push_back(""); // the table's own choice comes first
-  if (h.op != OP_ATTENTION) {
+  if (h.op == OP_ATTENTION) {
+    for (int dmax : {64, 128})
+      for (const AttnVariant &v : kAttnVariants)
+        requests.push_back(attn_perf_string(v, dmax));
+  } else {
     for (const Tile &t : kFastTiles)
       requests.push_back(perf_string(t, 1));
     requests.push_back("v2:32,32,4,32,32,16,4,1,1");    // K split over the block's waves (GEMM)
     requests.push_back("v2:224,128,8,224,32,16,1,1,1"); // window-resident convolution
+    if (kind == ROCKAMD_TUNING_EXHAUSTIVE) {
+      // every tile once more as its twin with the rolled epilogue (forceUnroll 0)
+      for (const Tile &t : kFastTiles) {
+        std::string pc = perf_string(t, 1);
+        pc[pc.size() - 3] = '0';
+        requests.push_back(pc);
+      }
+    }
   }
   std::vector<std::string> out, seen;
   const std::string keep_error = g_last_error;
@@ -2532,6 +2634,11 @@ std::vector<std::string> tuning_candidates(const Handle &h) {
     delete c;
   }
   g_last_error = keep_error;
+  // Quick: the table's choice and its two nearest alternatives in the order
+  // above (largest tiles first), as the reference's quick lists hold a handful
+  // of likely winners (RockTuningImpl.cpp:401-459)
+  if (kind == ROCKAMD_TUNING_QUICK && out.size() > 3)
+    out.resize(3);
   return out;
 }
 
@@ -2542,6 +2649,7 @@ struct TuningSpace {
 // problem key -> best perf_config seen and its time (mlirRockTuningUpdateTable keeps only the best)
 struct TuningTable {
   std::map<std::string, std::pair<std::string, float>> best;
+  std::mutex mutex; // several tuning threads may share one table (RockTuningImpl.cpp:902-931 takes a RW lock)
 };
 
 } // namespace
@@ -2685,9 +2793,16 @@ MiirStatus rockamdGetArgumentInfo(MiirHandle handle, int index, int *dtype, int 
   return MIIR_SUCCESS;
 }
 
+// Copies as much of s as fits and ALWAYS terminates it; returns the full
+// length, so a result >= buffer_size tells the caller the text was cut.  (The
+// reference's strncpy, mlir/lib/CAPI/Dialect/Rock.cpp:86,142, leaves a short
+// buffer unterminated; with a buffer that is large enough the two agree.)
 static size_t copy_string(const std::string &s, char *buffer, size_t buffer_size) {
-  if (buffer && buffer_size > 0)
-    std::strncpy(buffer, s.c_str(), buffer_size);
+  if (buffer && buffer_size > 0) {
+    const size_t n = std::min(s.size(), buffer_size - 1);
+    std::memcpy(buffer, s.data(), n);
+    buffer[n] = '\0';
+  }
   return s.size();
 }
 
@@ -2727,9 +2842,25 @@ MiirStatus rockamdSetScale(MiirHandle handle, float scale) {
   auto *h = static_cast<Handle *>(handle);
   if (!h)
     return MIIR_INVALID_PARAM;
-  if (h->op == OP_ATTENTION)
-    reinterpret_cast<RockAttentionParams *>(h->params.data())->scale = scale;
-  else if (h->epi)
+  if (h->op == OP_ATTENTION) {
+    auto *ap = reinterpret_cast<RockAttentionParams *>(h->params.data());
+    ap->scale = scale;
+    // The plain fused kernel takes the row maximum of the raw scores and
+    // scales afterwards, which is only right for a non-negative scale: a sign
+    // change moves the handle to or from the kernel that scales first.
+    const std::string plain = "_fast", scaled = "_fast_bias";
+    std::string &name = h->kernel_name;
+    auto ends_with = [&](const std::string &suffix) {
+      return name.size() >= suffix.size() && name.compare(name.size() - suffix.size(), suffix.size(), suffix) == 0;
+    };
+    if (scale < 0.0f && ends_with(plain)) {
+      name += "_bias";
+      h->functions.clear();
+    } else if (scale >= 0.0f && ends_with(scaled) && !ap->has_bias && !ap->has_scale_tensor) {
+      name.erase(name.size() - 5);
+      h->functions.clear();
+    }
+  } else if (h->epi)
     h->epi->scale = scale;
   else
     return MIIR_INVALID_PARAM; // a layout-conversion kernel has no epilogue
@@ -2868,10 +2999,10 @@ int rockamdMeasureMfmaRate(int dtype, int random_data, void *stream, double *ter
 // ---- tuning surface ---------------------------------------------------------
 RockamdTuningSpace rockamdTuningSpaceCreate(MiirHandle handle, int kind) {
   auto *h = static_cast<Handle *>(handle);
-  if (!h || (kind != ROCKAMD_TUNING_QUICK && kind != ROCKAMD_TUNING_FULL))
+  if (!h || (kind != ROCKAMD_TUNING_QUICK && kind != ROCKAMD_TUNING_FULL && kind != ROCKAMD_TUNING_EXHAUSTIVE))
     return nullptr;
   auto *sp = new TuningSpace;
-  sp->params = tuning_candidates(*h); // the quick and the full list coincide: a handful of kernels
+  sp->params = tuning_candidates(*h, kind);
   return sp;
 }
 
@@ -2883,10 +3014,7 @@ size_t rockamdTuningParamToString(RockamdTuningSpace space, unsigned pos, char *
   auto *sp = static_cast<TuningSpace *>(space);
   if (!sp || pos >= sp->params.size())
     return (size_t)-1;
-  const std::string &s = sp->params[pos];
-  if (buffer && buffer_size)
-    std::strncpy(buffer, s.c_str(), buffer_size);
-  return s.size();
+  return copy_string(sp->params[pos], buffer, buffer_size);
 }
 
 void rockamdTuningSpaceDestroy(RockamdTuningSpace space) { delete static_cast<TuningSpace *>(space); }
@@ -2916,6 +3044,7 @@ int rockamdTuningUpdateTable(RockamdTuningTable table, const char *problem_key, 
   auto *t = static_cast<TuningTable *>(table);
   if (!t || !problem_key || !perf_config)
     return 0;
+  std::lock_guard<std::mutex> lock(t->mutex);
   auto it = t->best.find(problem_key);
   if (it != t->best.end() && it->second.second <= time)
     return 0; // a better-performing entry exists
@@ -2928,10 +3057,15 @@ int rockamdTuningSetFromTable(RockamdTuningTable table, MiirHandle handle) {
   auto *h = static_cast<Handle *>(handle);
   if (!t || !h)
     return 0;
-  auto it = t->best.find(h->problem_key);
-  if (it == t->best.end())
-    return 0;
-  return rockamdTuningSetFromStr(handle, it->second.first.c_str());
+  std::string perf_config;
+  {
+    std::lock_guard<std::mutex> lock(t->mutex);
+    auto it = t->best.find(h->problem_key);
+    if (it == t->best.end())
+      return 0;
+    perf_config = it->second.first;
+  }
+  return rockamdTuningSetFromStr(handle, perf_config.c_str());
 }
 
 int rockamdIsSplitKFaster(int64_t g, int64_t m, int64_t n, int64_t k, int64_t num_cu, int element_size) {
@@ -2943,6 +3077,37 @@ int rockamdIsSplitKFaster(int64_t g, int64_t m, int64_t n, int64_t k, int64_t nu
   if (tiles64 * 2 <= num_cu)
     return ROCKAMD_SPLITK_ALWAYS; // make_gemm's own rule: 64x64 tiles would leave half the CUs idle
   return tiles64 <= num_cu ? ROCKAMD_SPLITK_MAYBE : ROCKAMD_SPLITK_NEVER;
+}
+
+int rockamdIsFusible(MiirHandle handle, const char *perf_config) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h || !perf_config)
+    return 0;
+  // The reference refuses an element-wise tail behind a split reduction
+  // because its partial sums meet in memory through atomic adds
+  // (RockTuningImpl.cpp:1010-1015).  Here a requested split (seventh field of
+  // the perf_config > 1) is the kernel that divides K over the waves of one
+  // block and sums the partial tiles in LDS BEFORE the epilogue, and the split
+  // over blocks through a workspace is only ever planned for an identity
+  // epilogue: whatever the handle resolves to under the string keeps its tail.
+  OptMap o = h->options;
+  o["perf_config"] = perf_config;
+  const std::string keep_error = g_last_error;
+  Handle *c = build_handle(o);
+  g_last_error = keep_error;
+  if (!c)
+    return 0;
+  delete c;
+  return 1;
+}
+
+size_t rockamdGetNumPrefillArgs(MiirHandle handle) {
+  (void)handle; // no kernel of this library accumulates into memory it has not written itself
+  return 0;
+}
+
+void rockamdGetPrefillArgsInfo(MiirHandle handle, size_t *indices, float *init_values, size_t length) {
+  (void)handle; (void)indices; (void)init_values; (void)length; // nothing to report: the count is zero
 }
 
 const char *rockamdGetLastError(void) { return g_last_error.c_str(); }

@@ -70,12 +70,12 @@ class TuningTable:
         return t
 
 
-def tune(kernel, *args, table=None, warmup=5, iters=20, stream=None):
-    """Times every entry of `kernel`'s tuning space on the given device
-    buffers, leaves the fastest applied, records it in `table` if given, and
-    returns [(perf_config, kernel_name, ms), ...] fastest first."""
+def tune(kernel, *args, table=None, warmup=5, iters=20, stream=None, kind="full"):
+    """Times every entry of `kernel`'s tuning space (of the given kind) on the
+    given device buffers, leaves the fastest applied, records it in `table` if
+    given, and returns [(perf_config, kernel_name, ms), ...] fastest first."""
     results = []
-    for perf in kernel.tuning_space():
+    for perf in kernel.tuning_space(kind):
         kernel.set_perf_config(perf)
         ms = kernel.benchmark(*args, warmup=warmup, iters=iters, stream=stream)
         results.append((kernel.perf_config, kernel.kernel_name, ms))

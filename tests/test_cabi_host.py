@@ -397,7 +397,10 @@ def test_tuning_space_lists_the_kernels_a_problem_can_run_on(rock):
     k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 4096 -n 4096 -k 4096 -transB true")
     space = k.tuning_space()
     assert space[0] == k.perf_config
-    assert space == k.tuning_space(full=True)
+    # RocmlirTuningParamSetKind (RockEnums.h:19-23): quick is a prefix of full, exhaustive holds full
+    quick, exhaustive = k.tuning_space("quick"), k.tuning_space("exhaustive")
+    assert quick == space[:3]
+    assert exhaustive[:len(space)] == space
     names = []
     for perf in space:
         assert re.fullmatch(r"v2:\d+(,\d+){8}", perf)
@@ -405,11 +408,38 @@ def test_tuning_space_lists_the_kernels_a_problem_can_run_on(rock):
         assert k.perf_config == perf
         names.append(k.kernel_name)
     assert len(set(names)) == len(names) == 5  # four tiles and the K-split kernel
-    # a convolution the window-resident kernel can run offers it; attention has one kernel
+    # a convolution the window-resident kernel can run offers it
     assert "v2:224,128,8,224,32,8,1,1,1" in rock.RockKernel(CONV_RESNET).tuning_space()
+    # exhaustive: every tile once more as the twin with the rolled epilogue (forceUnroll 0)
+    assert len(exhaustive) == len(space) + 4 and "v2:256,256,8,128,16,8,1,0,1" in exhaustive
+    k.set_perf_config("v2:256,256,8,128,16,8,1,0,1")
+    assert k.kernel_name == "rock_gemm_f16_256x256_fast_e" and k.perf_config == "v2:256,256,8,128,16,8,1,0,1"
+    # attention: the three kernels a plain problem can run on, in "attn:v1:" strings that
+    # are accepted back (RockAttrDefs.td:241-329, parser RockDialect.cpp:2122-2170); a head
+    # dimension of 64 can also run on the 128 instantiation
     att = rock.RockKernel("--arch gfx950 --operation attention -seq_len_q 256 -seq_len_k 512 "
-                          "-head_dim_qk 64 -head_dim_v 64 -t f16 -g 4 -transK true")
-    assert att.tuning_space() == [att.perf_config]
+                          "-head_dim_qk 128 -head_dim_v 128 -t f16 -g 4 -transK true")
+    sp = att.tuning_space()
+    assert sp[0] == att.perf_config == "attn:v1:64,128,128,8,32,32,8,1" and len(sp) == 3
+    kernels = []
+    for perf in sp:
+        assert re.fullmatch(r"attn:v1:\d+(,\d+){7}", perf)
+        att.set_perf_config(perf)
+        assert att.perf_config == perf
+        kernels.append(att.kernel_name)
+    assert kernels == ["rock_attention_f16_d128x128_fast", "rock_attention_f16_d128x128_fast_bias",
+                       "rock_attention_f16_d128x128_generic"]
+    att64 = rock.RockKernel("--arch gfx950 --operation attention -seq_len_q 256 -seq_len_k 512 "
+                            "-head_dim_qk 64 -head_dim_v 64 -t f16 -g 4 -transK true")
+    assert len(att64.tuning_space()) == 6
+    att64.set_perf_config("attn:v1:64,128,128,8,32,32,8,1")
+    assert att64.kernel_name == "rock_attention_f16_d128x128_fast"
+    # with a bias the pipelined kernel is not on offer, and asking for it falls back
+    attb = rock.RockKernel("--arch gfx950 --operation attention -seq_len_q 256 -seq_len_k 512 "
+                           "-head_dim_qk 128 -head_dim_v 128 -t f16 -g 4 -transK true -with-attn-bias true")
+    assert len(attb.tuning_space()) == 2
+    attb.set_perf_config("attn:v1:64,128,128,8,32,32,8,1")
+    assert attb.kernel_name == "rock_attention_f16_d128x128_fast_bias"
     # K-major operands have the three square tiles; unaligned ones only the generic kernel
     nn = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 256 -n 256 -k 256")
     assert len(nn.tuning_space()) == 3
@@ -417,15 +447,21 @@ def test_tuning_space_lists_the_kernels_a_problem_can_run_on(rock):
     assert gen.tuning_space() == [gen.perf_config]
     # raw entry points: bad position, short buffer
     lib = rock.load_library()
-    sp = lib.rockamdTuningSpaceCreate(k._h, 0)
+    sp = lib.rockamdTuningSpaceCreate(k._h, 1)
     assert lib.rockamdTuningGetNumParams(sp) == 5
     assert lib.rockamdTuningParamToString(sp, 99, None, 0) == C.c_size_t(-1).value
+    # a short buffer gets what fits, terminated; the full length comes back
     buf = C.create_string_buffer(b"\xff" * 8, 8)
     n = lib.rockamdTuningParamToString(sp, 0, buf, 4)
-    assert n == len(space[0]) and buf.raw[:4] == space[0][:4].encode() and buf.raw[4:] == b"\xff" * 4
+    assert n == len(space[0]) and buf.raw[:3] == space[0][:3].encode() and buf.raw[3] == 0
+    assert buf.raw[4:] == b"\xff" * 4
     lib.rockamdTuningSpaceDestroy(sp)
     assert lib.rockamdTuningSpaceCreate(None, 0) is None
     assert lib.rockamdTuningSpaceCreate(k._h, 7) is None
+    for getter in (lib.rockamdGetPerfConfig, lib.rockamdGetProblemKey):
+        buf = C.create_string_buffer(b"\xff" * 8, 8)
+        n = getter(k._h, buf, 5)
+        assert n > 5 and buf.raw[4] == 0 and buf.raw[5:] == b"\xff" * 3
 
 
 def test_set_perf_config_keeps_epilogue_scalars_and_launch_geometry(rock):
@@ -489,3 +525,141 @@ def test_product_does_not_touch_the_oracle():
             if f.endswith((".py", ".cpp", ".h", ".hip", ".S", ".inc")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "rock_oracle" not in text and "oracle/" not in text, f
+
+
+def test_window_resident_request_with_asymmetric_padding_falls_back(rock):
+    """The window-resident kernel sizes its LDS window from the top / left
+    padding alone, so a problem whose two sides differ must not get it."""
+    asym = (CONV_RESNET.replace("--padding_h 1", "--padding_h_l 0 --padding_h_r 1")
+            .replace("--fil_h 3", "--fil_h 2").replace("--out_h 28", "--out_h 28"))
+    base = rock.RockKernel(asym)
+    asked = rock.RockKernel(asym + " --perf_config v2:224,128,8,224,32,8,1,1,1")
+    assert "direct224" not in asked.kernel_name and asked.kernel_name == base.kernel_name
+    assert "v2:224,128,8,224,32,8,1,1,1" not in base.tuning_space()
+    sym = rock.RockKernel(CONV_RESNET + " --perf_config v2:224,128,8,224,32,8,1,1,1")
+    assert sym.kernel_name == "rock_conv_f16_direct224"
+
+
+def test_reference_style_perf_config_keeps_its_tile(rock):
+    """A reference-style string carries MPerWave = 32 and MnPerXdl = 32 in its
+    fourth and fifth fields; only the FIRST two fields name the block tile."""
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 4096 -n 4096 -k 4096 -transB true "
+                        "-perf_config v2:64,64,8,32,32,8,1,1,1")
+    assert k.kernel_name == "rock_gemm_f16_64x64_fast" and k.grid_size == 64 * 64
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 4096 -n 4096 -k 4096 -transB true "
+                        "-perf_config v2:32,32,4,32,32,8,4,1,1")
+    assert k.kernel_name == "rock_gemm_f16_32x32_splitk"
+    conv = rock.RockKernel(CONV_RESNET + " --perf_config v2:128,128,8,224,128,8,1,1,1")
+    assert conv.kernel_name == "rock_conv_f16_128x128_fast"
+
+
+def test_reduction_split_over_blocks_covers_both_storages(rock):
+    """A single float GEMM with few output tiles and a long K is cut over
+    blocks whichever way its operands are stored."""
+    for flags in ("-transB true", ""):
+        k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 128 -n 128 -k 16384 " + flags)
+        assert k.kernel_count == 2 and k.workspace_bytes > 0, flags
+        assert k.grid_size >= 128, (flags, k.kernel_name, k.grid_size)
+        red = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 128 -n 128 -k 16384 %s -kernel_id 1" % flags)
+        assert red.kernel_name == "rock_reduce_splits"
+    one = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 128 -n 128 -k 16384 -transB true -split_k false")
+    assert one.kernel_count == 1 and one.kernel_name == "rock_gemm_f16_32x32_splitk"
+
+
+def test_attention_scale_sign_selects_the_kernel(rock):
+    """The plain fused kernel takes the row maximum before scaling, which needs
+    a non-negative scale; rockamdSetScale moves the handle when the sign changes."""
+    opts = ("-operation attention -arch gfx950 -t f16 -g 2 -seq_len_q 256 -seq_len_k 256 "
+            "-head_dim_qk 64 -head_dim_v 64 -transK true -scale 0.125")
+    k = rock.RockKernel(opts)
+    assert k.kernel_name == "rock_attention_f16_d64x64_fast"
+    k.set_scale(-0.125)
+    k._refresh()
+    assert k.kernel_name == "rock_attention_f16_d64x64_fast_bias"
+    k.set_scale(0.5)
+    k._refresh()
+    assert k.kernel_name == "rock_attention_f16_d64x64_fast"
+    b = rock.RockKernel(opts + " -with-attn-bias true")
+    b.set_scale(0.5)
+    b._refresh()
+    assert b.kernel_name == "rock_attention_f16_d64x64_fast_bias"
+
+
+def test_fusibility_and_prefill_queries(rock):
+    """mlirIsModuleFusible / mlirGetNumPrefillArgs (mlir-c/Dialect/Rock.h:145-158)."""
+    lib = rock.load_library()
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 128 -n 128 -k 4096 -transB true "
+                        "-bias true -activation relu")
+    assert lib.rockamdIsFusible(k._h, b"v2:32,32,4,32,32,8,4,1,1") == 1   # split inside the block: tail stays
+    assert lib.rockamdIsFusible(k._h, b"v2:128,128,8,64,16,8,1,1,1") == 1
+    assert lib.rockamdIsFusible(None, b"v2:128,128,8,64,16,8,1,1,1") == 0
+    assert lib.rockamdIsFusible(k._h, None) == 0
+    assert lib.rockamdGetNumPrefillArgs(k._h) == 0
+    idx, val = (C.c_size_t * 2)(7, 7), (C.c_float * 2)(7.0, 7.0)
+    lib.rockamdGetPrefillArgsInfo(k._h, idx, val, 0)
+    assert list(idx) == [7, 7]
+
+
+def test_operands_beyond_31_bit_offsets_leave_the_vector_kernels(rock):
+    """The direct-to-LDS loads address a block's operand rows with 32-bit byte
+    offsets below 2^31: 256 rows plus one of about 8 MiB each cannot, and such a
+    problem must run on the element-wise kernel instead."""
+    ok = rock.RockKernel("-operation gemm -arch gfx950 -t i8 -g 1 -m 256 -n 256 -k 8355840 -transB true")
+    assert "_generic" not in ok.kernel_name
+    big = rock.RockKernel("-operation gemm -arch gfx950 -t i8 -g 1 -m 256 -n 256 -k 8356096 -transB true")
+    assert big.kernel_name == "rock_gemm_i8_64x64_generic"
+    km = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 1048576 -n 256 -k 2048 -transA true -transB true")
+    assert km.kernel_name == "rock_gemm_f16_64x64_generic"   # K-major A: k * M * 2 bytes passes 2^31
+
+
+def test_handles_from_eight_threads(rock):
+    """The header promises that entry points may be called from several threads
+    (one handle per thread): create, query, re-tune and destroy concurrently."""
+    import threading
+    errors = []
+
+    def work(i):
+        try:
+            for j in range(40):
+                m = 64 * (1 + (i + j) % 9)
+                k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m %d -n 256 -k 512 -transB true" % m)
+                assert k.grid_size > 0 and k.kernel_name.startswith("rock_gemm_f16_")
+                space = k.tuning_space()
+                k.set_perf_config(space[-1])
+                assert k.perf_config == space[-1]
+                bad = rock.load_library().miirCreateHandle(b"--operation gemm --arch gfx950 -t f16 -m 4")
+                assert not bad and rock.api.last_error() != ""
+                del k
+        except Exception as e:  # noqa: BLE001 - collected for the main thread
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+
+
+def test_tuning_table_shared_by_threads(rock):
+    """mlirRockTuningUpdateTable keeps the best entry under a lock
+    (RockTuningImpl.cpp:902-931): concurrent updates of one key must end with the minimum."""
+    import threading
+    from rocmlir_amd.tuning import TuningTable
+    lib = rock.load_library()
+    table = TuningTable()
+    key = b"gfx950\t256\t-t f16 -out_datatype f16 -transA false -transB true -g 1 -m 64 -n 256 -k 512"
+
+    def work(i):
+        for j in range(200):
+            t = 1.0 + ((i * 200 + j) * 7919 % 1000) / 10.0
+            lib.rockamdTuningUpdateTable(table._t, key, b"v2:64,64,8,32,16,8,1,1,1" if t > 1.0 else
+                                         b"v2:128,128,8,64,16,8,1,1,1", C.c_float(t))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert lib.rockamdTuningUpdateTable(table._t, key, b"v2:64,64,8,32,16,8,1,1,1", C.c_float(1.0)) == 0
+    assert lib.rockamdTuningUpdateTable(table._t, key, b"v2:64,64,8,32,16,8,1,1,1", C.c_float(0.5)) == 1

@@ -19,7 +19,7 @@ def _to_layout(t, canonical, layout):
 
 
 def _run(rock, oracle, gpu, t, n, g, c, k, hi, wi, y, x, stride, pad, dil, layouts, integer, seed,
-         out_dtype=None, **epi):
+         out_dtype=None, pad_r=None, **epi):
     fl, il, ol = layouts
     rng = np.random.default_rng(seed)
     if t == "i8":
@@ -36,12 +36,13 @@ def _run(rock, oracle, gpu, t, n, g, c, k, hi, wi, y, x, stride, pad, dil, layou
     out = rock.conv2d(to_gpu(raw_f, t, gpu), to_gpu(raw_i, t, gpu), fil_layout=fl, in_layout=il,
                       out_layout=ol, batchsize=n, in_channels=g * c, out_channels=g * k, in_h=hi,
                       in_w=wi, fil_h=y, fil_w=x, groupsize=g, stride=stride, padding=pad, dilation=dil,
-                      out_dtype=out_dtype, **epi)
+                      out_dtype=out_dtype, padding_r=pad_r, **epi)
     torch.cuda.synchronize()
     if t == "i8":
-        ref, ho, wo = oracle.conv_fwd(raw_f, raw_i, fl, il, ol, n, g, c, k, hi, wi, y, x, stride, pad, dil)
+        ref, ho, wo = oracle.conv_fwd(raw_f, raw_i, fl, il, ol, n, g, c, k, hi, wi, y, x, stride, pad, dil,
+                                      pad_r=pad_r)
     else:
-        ref, ho, wo = oracle.conv_fwd(fq, iq, fl, il, ol, n, g, c, k, hi, wi, y, x, stride, pad, dil)
+        ref, ho, wo = oracle.conv_fwd(fq, iq, fl, il, ol, n, g, c, k, hi, wi, y, x, stride, pad, dil, pad_r=pad_r)
     od = out_dtype or {"i8": "i32", "fp8": "f32", "bf8": "f32"}.get(t, t)
     assert out.numel() == ref.size
     return out, od, ref
@@ -102,6 +103,29 @@ def test_conv_edge_shapes_exact(rock, oracle, gpu, case, layouts, t):
         assert oracle.verify_int(out.cpu().numpy().ravel(), ref)[0] == 0
     else:
         assert np.array_equal(to_f32(out, od), ref)
+
+
+# (n g c k hi wi y x stride pad_left dil pad_right)
+ASYM_PAD_CASES = [
+    (2, 1, 64, 128, 14, 14, 2, 2, (1, 1), (0, 0), (1, 1), (1, 1)),   # "same" padding of an even filter
+    (3, 1, 16, 32, 9, 11, 3, 3, (2, 2), (0, 1), (1, 1), (1, 2)),
+    (2, 2, 8, 16, 7, 7, 3, 2, (1, 1), (2, 0), (1, 2), (0, 1)),
+]
+
+
+@pytest.mark.parametrize("case", ASYM_PAD_CASES)
+@pytest.mark.parametrize("layouts", [NHWC, NCHW], ids=["nhwc", "nchw"])
+@pytest.mark.parametrize("perf", [None, "v2:224,128,8,224,32,8,1,1,1"], ids=["table", "direct224-asked"])
+def test_conv_asymmetric_padding_exact(rock, oracle, gpu, case, layouts, perf):
+    """--padding_h_l / _r, --padding_w_l / _r with different values on the two
+    sides.  A request for the window-resident kernel, which only knows
+    symmetric padding, must fall back and still be exact."""
+    *shape, pad_r = case
+    info = {}
+    out, od, ref = _run(rock, oracle, gpu, "f16", *shape, layouts, True, 77, pad_r=pad_r, perf_config=perf,
+                        info=info)
+    assert "direct224" not in info["kernel_name"]
+    assert np.array_equal(to_f32(out, od), ref)
 
 
 MIXED = [(f, i, o) for f in ("gkcyx", "gkyxc", "gyxck") for i, o in

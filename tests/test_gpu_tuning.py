@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 
 def test_tuner_gemm_every_candidate_exact_and_best_applied(rock, oracle, gpu):
     from rocmlir_amd import tuning
-    M, N, K = 384, 320, 1536
+    M, N, K = 384, 384, 1536   # 144 tiles of 32x32: the K-split kernel alone fills the chip, one kernel
     rng = np.random.default_rng(51)
     ra, aq = quantise(rng.integers(-3, 4, (M, K)).astype(np.float32), "f16")
     rb, bq = quantise(rng.integers(-3, 4, (N, K)).astype(np.float32), "f16")
