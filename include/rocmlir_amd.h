@@ -281,6 +281,27 @@ ROCMLIR_AMD_API int rockamdIsSplitKFaster(int64_t g, int64_t m, int64_t n, int64
 ROCMLIR_AMD_API int rockamdLaunch(MiirHandle handle, void *const *pointers, int num_pointers,
                   void *stream);
 
+/* rockamdLaunch for callers that cannot allocate device memory: code under HIP
+ * graph capture, serving loops and harnesses that forbid hipMalloc.  It has
+ * no counterpart in the reference.  A problem of several kernels
+ * (miirGetKernelCount > 1) passes intermediate results through a workspace
+ * that rockamdLaunch's caller allocates and passes last; this entry point
+ * takes the problem's own pointers only (one fewer than rockamdLaunch when the
+ * problem has a workspace) and uses an array of
+ * ROCKAMD_STATIC_WORKSPACE_BYTES bytes in the library's own device image
+ * instead.  It calls no allocating routine, except that the first call for a
+ * handle on a device loads the handle's code object and resolves the array's
+ * address: make that call outside a capture.  A problem whose workspace is
+ * larger fails with hipErrorInvalidValue and a message in
+ * rockamdGetLastError; nothing is launched.  Each GPU holds one such array
+ * until the process ends and all calls on that GPU share it: launch the
+ * kernels of one problem in kernel_id order on one stream, and do not let two
+ * problems with workspaces overlap in time on one GPU (they race on it).  A
+ * problem without a workspace behaves exactly as under rockamdLaunch. */
+#define ROCKAMD_STATIC_WORKSPACE_BYTES ((size_t)64 << 20)
+ROCMLIR_AMD_API int rockamdLaunchStaticWorkspace(MiirHandle handle, void *const *pointers, int num_pointers,
+                                                 void *stream);
+
 /* Timed loop with HIP events on `stream`: `warmup` untimed launches, then
  * `iters` launches between one start/stop event pair; writes the average
  * milliseconds per launch.  Synchronises the stream. */

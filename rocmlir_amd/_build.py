@@ -61,13 +61,18 @@ def build(jobs=8, verbose=False, host_only=False, only=None):
         for out in pool.map(_run, todo):
             if verbose and out.strip():
                 print(out)
+    # the one source with host and device code in one object: the static workspace
+    static_o = os.path.join(BUILD, "static_workspace.o")
+    _run([HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden",
+          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+          "-c", os.path.join(CSRC, "static_workspace.hip"), "-o", static_o])
     blobs_o = os.path.join(BUILD, "blobs.o")
     _run(["gcc", "-c", "-x", "assembler-with-cpp", "-I", BUILD,
           os.path.join(CSRC, "blobs.S"), "-o", blobs_o])
     _run([HIPCC, "-O2", "-std=c++17", "-fPIC", "-shared", "-x", "c++",
           "-D__HIP_PLATFORM_AMD__", "-fvisibility=hidden",
           "-I", os.path.join(ROCM, "include"),
-          os.path.join(CSRC, "rock_api.cpp"), "-x", "none", blobs_o,
+          os.path.join(CSRC, "rock_api.cpp"), "-x", "none", blobs_o, static_o,
           "-L", os.path.join(ROCM, "lib"), "-lamdhip64",
           "-Wl,-rpath," + os.path.join(ROCM, "lib"),
           "-o", LIB])

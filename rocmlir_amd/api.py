@@ -73,6 +73,8 @@ def load_library():
         L.rockamdSetZeroPoint.argtypes = [vp, C.c_int32]
         L.rockamdLaunch.restype = C.c_int
         L.rockamdLaunch.argtypes = [vp, C.POINTER(vp), C.c_int, vp]
+        L.rockamdLaunchStaticWorkspace.restype = C.c_int
+        L.rockamdLaunchStaticWorkspace.argtypes = [vp, C.POINTER(vp), C.c_int, vp]
         L.rockamdBenchmark.restype = C.c_int
         L.rockamdBenchmark.argtypes = [vp, C.POINTER(vp), C.c_int, vp, C.c_int,
                                        C.c_int, C.POINTER(C.c_float)]

@@ -11,6 +11,7 @@
 // compiled ahead of time for gfx950 and embedded in this library.
 #include "../../include/rocmlir_amd.h"
 #include "kernel_params.h"
+#include "rock_internal.h"
 
 #include <hip/hip_runtime_api.h>
 
@@ -2653,6 +2654,44 @@ struct TuningTable {
 };
 
 } // namespace
+
+// see rock_internal.h
+int rock_launch_with_workspace(void *handle, void *const *pointers, int num_pointers, void *workspace,
+                               size_t capacity, void *stream) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h || !pointers) {
+    set_error("launch: NULL handle or pointer list");
+    return (int)hipErrorInvalidValue;
+  }
+  const int expected = h->caller_pointers ? h->caller_pointers : h->num_pointers;
+  const bool has_workspace = h->workspace_bytes != 0;
+  void *full[16];
+  if (num_pointers != expected - (has_workspace ? 1 : 0) || expected > 16) {
+    set_error("launch: wrong number of pointer arguments (the workspace is not one of them here)");
+    return (int)hipErrorInvalidValue;
+  }
+  if (h->workspace_bytes > capacity) {
+    char msg[160];
+    std::snprintf(msg, sizeof msg, "launch: the problem needs a workspace of %zu bytes, the built-in one holds %zu",
+                  h->workspace_bytes, capacity);
+    set_error(msg);
+    return (int)hipErrorInvalidValue;
+  }
+  for (int i = 0; i < num_pointers; ++i)
+    full[i] = pointers[i];
+  if (has_workspace)
+    full[num_pointers] = workspace; // the workspace closes every multi-kernel problem's caller list
+  if (!check_launch_args(h, full, expected))
+    return (int)hipErrorInvalidValue;
+  hipFunction_t fn;
+  int rc = get_function(h, &fn);
+  if (rc != 0)
+    return rc;
+  rc = launch_once(h, fn, full, (hipStream_t)stream);
+  if (rc != 0)
+    set_error(std::string("launch failed: ") + hipGetErrorString((hipError_t)rc));
+  return rc;
+}
 
 // ============================================================================
 // C ABI
