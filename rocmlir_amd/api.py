@@ -430,7 +430,7 @@ def gemm(a, b, *, transA=False, transB=False, transC=False, out_dtype=None,
          scale=None, zero_point=0, bias=None, relu=False, quant_scale=None,
          out_zero_point=0, activation=None, clip=None, residual=None,
          residual_op="add", out=None, perf_config=None, stream=None,
-         info=None, split_k=True):
+         info=None, split_k=True, layout_conversion=True):
     """C = epilogue(A x B) with the reference's storage conventions
     (rocmlir-gen.cpp:2058-2080): a is [G,M,K] ([G,K,M] if transA), b is
     [G,K,N] ([G,N,K] if transB), result [G,M,N] ([G,N,M] if transC).
@@ -439,7 +439,10 @@ def gemm(a, b, *, transA=False, transB=False, transC=False, out_dtype=None,
     `residual_op` "add" or "mul"), then `activation` ("relu", "sigmoid",
     "tanh", "erf", "gelu", "exp") or `clip=(lo, hi)`, then the narrowing to
     the output type.  A dict passed as `info` receives the name and
-    perf_config of the kernel that ran."""
+    perf_config of the GEMM kernel that ran and the names of all kernels of
+    the problem (operands that are not whole 16-byte chunks are first copied
+    into padded ones unless `layout_conversion` is False; a long reduction
+    over few output tiles is split over blocks unless `split_k` is False)."""
     import torch
     a3 = a if a.dim() == 3 else a.unsqueeze(0)
     b3 = b if b.dim() == 3 else b.unsqueeze(0)
@@ -461,11 +464,13 @@ def gemm(a, b, *, transA=False, transB=False, transC=False, out_dtype=None,
         opts += " -perf_config %s" % perf_config
     if not split_k:
         opts += " -split_k false"
+    if not layout_conversion:
+        opts += " -layout_conversion false"
     opts += _epilogue_flags(scale, zero_point, bias, relu, quant_scale,
                             out_zero_point, activation, clip, residual,
                             residual_op)
-    prog = _program(opts)   # one kernel, or two when the reduction is split over blocks
-    k = prog.kernels[0]
+    prog = _program(opts)   # one kernel, or several: padded operand copies, a reduction split over blocks
+    k = next(x for x in prog.kernels if x.kernel_name.startswith("rock_gemm_"))
     if info is not None:
         info["kernel_name"] = k.kernel_name
         info["perf_config"] = k.perf_config

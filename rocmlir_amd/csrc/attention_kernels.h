@@ -24,6 +24,7 @@
 //     operands are single conflict-free 16-byte reads;
 //   * next K/V tiles are fetched into registers while the current ones are
 //     being multiplied; two LDS stages, one barrier per tile.
+#pragma once
 #include <type_traits>
 #include "mfma_gfx950.h"
 
@@ -365,7 +366,10 @@ __device__ __forceinline__ void wait_loads_and_lds_reads() {
     rk::attention_body<DT, DQK, DV, FAST>(Q, K, V, scale, bias, O, p);                        \
   }
 
-// fast variants: two blocks per compute unit (register budget 256 per lane)
+// fast variants: two blocks per compute unit (register budget 256 per lane).
+// The build (rocmlir_amd/_build.py holds the list) compiles every kernel into a
+// code object of its own from a small source that includes this file and
+// invokes one of the two macros.
 #define RK_ATTN_DL(DTNAME, DT, D, SUFFIX, PLAIN)                                              \
   extern "C" __global__ __launch_bounds__(rk::kAttnThreads, 2) void                           \
       rock_attention_##DTNAME##_d##D##x##D##_##SUFFIX(const void *Q, const void *K,           \
@@ -374,16 +378,3 @@ __device__ __forceinline__ void wait_loads_and_lds_reads() {
                                                       RockAttentionParams p) {                \
     rk::attention_body_dl<DT, D, PLAIN>(Q, K, V, scale, bias, O, p);                          \
   }
-
-RK_ATTN_DL(f16, MM_F16, 128, fast, true)
-RK_ATTN_DL(f16, MM_F16, 128, fast_bias, false)
-RK_ATTN_DL(f16, MM_F16, 64, fast, true)
-RK_ATTN_DL(f16, MM_F16, 64, fast_bias, false)
-RK_ATTN(f16, MM_F16, 128, 128, generic, false)
-RK_ATTN(f16, MM_F16, 64, 64, generic, false)
-RK_ATTN_DL(bf16, MM_BF16, 128, fast, true)
-RK_ATTN_DL(bf16, MM_BF16, 128, fast_bias, false)
-RK_ATTN_DL(bf16, MM_BF16, 64, fast, true)
-RK_ATTN_DL(bf16, MM_BF16, 64, fast_bias, false)
-RK_ATTN(bf16, MM_BF16, 128, 128, generic, false)
-RK_ATTN(bf16, MM_BF16, 64, 64, generic, false)

@@ -1,5 +1,7 @@
 /* Places each compiled gfx950 code object in .rodata between a start and an
- * end symbol.  Assembled with -I <directory holding the .hsaco files>. */
+ * end symbol.  Assembled with -I <build directory>, which holds the .hsaco
+ * files and blobs_list.S, the generated list of "ROCK_BLOB <kernel name>"
+ * lines (one code object per kernel). */
     .macro ROCK_BLOB n
     .global rock_hsaco_\n\()_start
     .global rock_hsaco_\n\()_end
@@ -11,15 +13,5 @@ rock_hsaco_\n\()_end:
     .endm
 
     .section .rodata
-    ROCK_BLOB gemm_f32
-    ROCK_BLOB gemm_f16
-    ROCK_BLOB gemm_bf16
-    ROCK_BLOB gemm_i8
-    ROCK_BLOB gemm_fp8
-    ROCK_BLOB gemm_bf8
-    ROCK_BLOB gemm_fp8_bf8
-    ROCK_BLOB gemm_bf8_fp8
-    ROCK_BLOB attention
-    ROCK_BLOB relayout
-    ROCK_BLOB probe
+#include "blobs_list.S"
     .section .note.GNU-stack,"",@progbits

@@ -110,6 +110,14 @@ struct RockRelayoutParams {
   int32_t tile_d;             // RELAYOUT_TRANSPOSE: tile extent along dst_fast (8, 16 or 32)
 };
 
+// rock_relayout_pair_b{1,2,4}(src0, dst0, src1, dst1, p): two conversions in one
+// launch; blocks [0, first_blocks) run `first`, the others `second`.
+struct RockRelayoutPairParams {
+  RockRelayoutParams first, second;
+  int32_t first_blocks;
+  int32_t pad_;
+};
+
 // Utility kernels of the backward convolutions (the reference's zero-init and
 // converting-copy utility kernels, ConvGenerator.cpp:279-344, 434-480).
 // rock_fill_zero(dst, p): clears `bytes` bytes.

@@ -54,8 +54,24 @@ __device__ __forceinline__ void probe_body(float *out, int iters, int random_dat
                                                                            int random_data) { \
     probe_body<DT>(out, iters, random_data);                                                 \
   }
+// one code object per kernel: the build compiles this file once per operand
+// type with -DROCK_KERNEL=<RockDType value> (the preprocessor does not see the enumerators)
+#ifndef ROCK_KERNEL
+#define ROCK_KERNEL -1
+#endif
+#define RK_SELECTED(n) (ROCK_KERNEL < 0 || ROCK_KERNEL == (n))
+#if RK_SELECTED(0) // MM_F32
 RK_PROBE(f32, MM_F32)
+#endif
+#if RK_SELECTED(1) // MM_F16
 RK_PROBE(f16, MM_F16)
+#endif
+#if RK_SELECTED(2) // MM_BF16
 RK_PROBE(bf16, MM_BF16)
+#endif
+#if RK_SELECTED(3) // MM_I8
 RK_PROBE(i8, MM_I8)
+#endif
+#if RK_SELECTED(4) // MM_FP8
 RK_PROBE(fp8, MM_FP8)
+#endif

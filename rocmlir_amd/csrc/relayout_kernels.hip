@@ -5,6 +5,15 @@
 #include <stdint.h>
 #include "kernel_params.h"
 
+// Every kernel goes into a code object of its own: the build compiles this
+// file once per kernel with -DROCK_KERNEL=<n>, n counting the kernels below
+// from 0 in file order (rocmlir_amd/_build.py holds the matching list of
+// names and checks each object's symbol against it).
+#ifndef ROCK_KERNEL
+#define ROCK_KERNEL -1
+#endif
+#define RK_SELECTED(n) (ROCK_KERNEL < 0 || ROCK_KERNEL == (n))
+
 namespace {
 
 // RELAYOUT_TRANSPOSE: one block moves a tile of tile_d x (1024 / tile_d)
@@ -15,14 +24,14 @@ namespace {
 // the src_fast tiles, then dst_fast tiles, then the remaining three
 // dimensions in index order.
 template <typename T>
-__device__ __forceinline__ void relayout_transpose(const T *src, T *dst, const RockRelayoutParams &p) {
+__device__ __forceinline__ void relayout_transpose(const T *src, T *dst, const RockRelayoutParams &p, unsigned block) {
   __shared__ T tile[1024 + 128];
   const int sf = p.src_fast, df = p.dst_fast;
   const int td = p.tile_d, ts = 1024 / td; // both powers of two
   const int td_shift = __builtin_ctz(td), ts_shift = 10 - td_shift;
   const int size_s = p.size[sf], size_d = p.size[df];
   const int src_s = p.src_size[sf], src_d = p.src_size[df]; // shorter than the destination when padding
-  unsigned b = blockIdx.x;
+  unsigned b = block;
   const unsigned tiles_s = (size_s + ts - 1) >> ts_shift, tiles_d = (size_d + td - 1) >> td_shift;
   const int org_s = (int)(b % tiles_s) << ts_shift;
   b /= tiles_s;
@@ -71,7 +80,7 @@ __device__ __forceinline__ void relayout_transpose(const T *src, T *dst, const R
 // element by element elsewhere.  Requires unit stride of src_fast in the source
 // and of dst_fast in the destination.
 template <typename T>
-__device__ __forceinline__ void relayout_transpose_vec(const T *src, T *dst, const RockRelayoutParams &p) {
+__device__ __forceinline__ void relayout_transpose_vec(const T *src, T *dst, const RockRelayoutParams &p, unsigned block) {
   constexpr int V = 16 / (int)sizeof(T); // elements per 16-byte vector
   constexpr int TILE = 8 * V;            // tile side in elements
   constexpr int PITCH = TILE + V;        // keeps LDS rows 16-byte aligned
@@ -79,7 +88,7 @@ __device__ __forceinline__ void relayout_transpose_vec(const T *src, T *dst, con
   const int sf = p.src_fast, df = p.dst_fast;
   const int size_s = p.size[sf], size_d = p.size[df];
   const int src_s = p.src_size[sf], src_d = p.src_size[df];
-  unsigned b = blockIdx.x;
+  unsigned b = block;
   const unsigned tiles_s = (size_s + TILE - 1) / TILE, tiles_d = (size_d + TILE - 1) / TILE;
   const int org_s = (int)(b % tiles_s) * TILE;
   b /= tiles_s;
@@ -153,12 +162,12 @@ __device__ __forceinline__ void relayout_transpose_vec(const T *src, T *dst, con
 // beyond the source's length.  blockIdx.x enumerates groups of 256 chunks over
 // the flattened dimensions (2, 3, chunk), then dimensions 1 and 0.
 template <typename T>
-__device__ __forceinline__ void relayout_copy(const T *src, T *dst, const RockRelayoutParams &p) {
+__device__ __forceinline__ void relayout_copy(const T *src, T *dst, const RockRelayoutParams &p, unsigned block) {
   constexpr int EPC = 16 / (int)sizeof(T); // elements per chunk
   const unsigned chunks4 = (unsigned)p.size[4] / EPC;
   const unsigned inner = (unsigned)p.size[2] * (unsigned)p.size[3] * chunks4;
   const unsigned per = (inner + 255) / 256;
-  unsigned b = blockIdx.x;
+  unsigned b = block;
   unsigned q = (b % per) * 256 + threadIdx.x;
   b /= per;
   const unsigned i1 = b % (unsigned)p.size[1], i0 = b / (unsigned)p.size[1];
@@ -184,31 +193,50 @@ __device__ __forceinline__ void relayout_copy(const T *src, T *dst, const RockRe
 }
 
 template <typename T>
-__device__ __forceinline__ void relayout_body(const T *src, T *dst, const RockRelayoutParams &p) {
+__device__ __forceinline__ void relayout_body(const T *src, T *dst, const RockRelayoutParams &p,
+                                              unsigned block = blockIdx.x) {
   if (p.mode == RELAYOUT_COPY)
-    relayout_copy<T>(src, dst, p);
+    relayout_copy<T>(src, dst, p, block);
   else if (p.mode == RELAYOUT_TRANSPOSE_VEC)
-    relayout_transpose_vec<T>(src, dst, p);
+    relayout_transpose_vec<T>(src, dst, p, block);
   else
-    relayout_transpose<T>(src, dst, p);
+    relayout_transpose<T>(src, dst, p, block);
+}
+
+// Two conversions in one launch (both operands of a GEMM copied into padded
+// rows): blocks [0, first_blocks) convert the first tensor, the rest the second.
+template <typename T>
+__device__ __forceinline__ void relayout_pair_body(const void *src0, void *dst0, const void *src1, void *dst1,
+                                                   const RockRelayoutPairParams &p) {
+  if (blockIdx.x < (unsigned)p.first_blocks) // uniform per block
+    relayout_body<T>((const T *)src0, (T *)dst0, p.first, blockIdx.x);
+  else
+    relayout_body<T>((const T *)src1, (T *)dst1, p.second, blockIdx.x - (unsigned)p.first_blocks);
 }
 
 } // namespace
 
+#if RK_SELECTED(0)
 extern "C" __global__ __launch_bounds__(256) void rock_relayout_b1(const void *src, void *dst,
                                                                     RockRelayoutParams p) {
   relayout_body<uint8_t>((const uint8_t *)src, (uint8_t *)dst, p);
 }
+#endif
+#if RK_SELECTED(1)
 extern "C" __global__ __launch_bounds__(256) void rock_relayout_b2(const void *src, void *dst,
                                                                     RockRelayoutParams p) {
   relayout_body<uint16_t>((const uint16_t *)src, (uint16_t *)dst, p);
 }
+#endif
+#if RK_SELECTED(2)
 extern "C" __global__ __launch_bounds__(256) void rock_relayout_b4(const void *src, void *dst,
                                                                     RockRelayoutParams p) {
   relayout_body<uint32_t>((const uint32_t *)src, (uint32_t *)dst, p);
 }
+#endif
 
 // 16 bytes per thread; the tail of a size that is not a multiple of 16 byte by byte
+#if RK_SELECTED(3)
 extern "C" __global__ __launch_bounds__(256) void rock_fill_zero(void *dst, RockFillParams p) {
   const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 16;
   if (i + 16 <= p.bytes) {
@@ -218,8 +246,10 @@ extern "C" __global__ __launch_bounds__(256) void rock_fill_zero(void *dst, Rock
       ((char *)dst)[b] = 0;
   }
 }
+#endif
 
 // one output element per thread
+#if RK_SELECTED(4)
 extern "C" __global__ __launch_bounds__(256) void rock_reduce_splits(const float *partials, void *dst,
                                                                      RockReduceParams p) {
   const int64_t total = (int64_t)p.size[0] * p.size[1] * p.size[2] * p.size[3];
@@ -243,6 +273,7 @@ extern "C" __global__ __launch_bounds__(256) void rock_reduce_splits(const float
     ((__bf16 *)dst)[off] = (__bf16)acc;
   }
 }
+#endif
 
 namespace {
 __device__ __forceinline__ float load_as_f32(const void *base, int64_t idx, int dtype) {
@@ -274,6 +305,7 @@ __device__ __forceinline__ float block_reduce(float v, bool take_max, float *scr
 // One block per row, three passes over it (maximum, sum, normalise); the last
 // pass loads a chunk of scores into registers before any thread overwrites the
 // narrower results over them.
+#if RK_SELECTED(5)
 extern "C" __global__ __launch_bounds__(256) void rock_softmax_rows(float *S, const void *scale_t, const void *bias,
                                                                     RockSoftmaxParams p) {
   __shared__ float scratch[4];
@@ -315,3 +347,22 @@ extern "C" __global__ __launch_bounds__(256) void rock_softmax_rows(float *S, co
     }
   }
 }
+#endif
+#if RK_SELECTED(6)
+extern "C" __global__ __launch_bounds__(256) void rock_relayout_pair_b1(const void *src0, void *dst0, const void *src1,
+                                                                         void *dst1, RockRelayoutPairParams p) {
+  relayout_pair_body<uint8_t>(src0, dst0, src1, dst1, p);
+}
+#endif
+#if RK_SELECTED(7)
+extern "C" __global__ __launch_bounds__(256) void rock_relayout_pair_b2(const void *src0, void *dst0, const void *src1,
+                                                                         void *dst1, RockRelayoutPairParams p) {
+  relayout_pair_body<uint16_t>(src0, dst0, src1, dst1, p);
+}
+#endif
+#if RK_SELECTED(8)
+extern "C" __global__ __launch_bounds__(256) void rock_relayout_pair_b4(const void *src0, void *dst0, const void *src1,
+                                                                         void *dst1, RockRelayoutPairParams p) {
+  relayout_pair_body<uint32_t>(src0, dst0, src1, dst1, p);
+}
+#endif

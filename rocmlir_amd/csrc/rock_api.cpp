@@ -36,7 +36,9 @@ thread_local std::string g_last_error;
 void set_error(const std::string &msg) { g_last_error = msg; }
 
 // --------------------------------------------------------------------------
-// embedded gfx950 code objects (see blobs.S)
+// embedded gfx950 code objects, one per kernel and named after it (blobs.S;
+// blobs.inc is the list the build generates).  The reference hands out one
+// kernel per code object (rocmlir-lib.cpp:292-316); so does miirBufferGet.
 // --------------------------------------------------------------------------
 #define ROCK_BLOB(n)                                                           \
   extern "C" const char rock_hsaco_##n##_start[];                              \
@@ -45,7 +47,7 @@ void set_error(const std::string &msg) { g_last_error = msg; }
 #undef ROCK_BLOB
 
 struct Blob {
-  const char *name;
+  const char *name; // the kernel's symbol
   const char *start;
   const char *end;
 };
@@ -55,11 +57,15 @@ const Blob kBlobs[] = {
 #undef ROCK_BLOB
 };
 
-const Blob *find_blob(const std::string &name) {
-  for (const Blob &b : kBlobs)
-    if (name == b.name)
-      return &b;
-  return nullptr;
+const Blob *find_blob(const std::string &kernel_name) {
+  static const std::map<std::string, const Blob *> index = [] {
+    std::map<std::string, const Blob *> m;
+    for (const Blob &b : kBlobs)
+      m[b.name] = &b;
+    return m;
+  }();
+  auto it = index.find(kernel_name);
+  return it == index.end() ? nullptr : it->second;
 }
 
 // --------------------------------------------------------------------------
@@ -259,7 +265,6 @@ struct Handle {
   int kernel_id = 0;
   // resolved kernel
   std::string kernel_name;
-  std::string blob_name;
   const Blob *blob = nullptr;
   uint32_t block_size = 0, grid_size = 0;
   int num_pointers = 0;
@@ -461,7 +466,10 @@ void set_contraction_pointers(Handle *h, const RockEpilogue &e) {
 
 // Chooses the kernel, tile and grid for a GEMM whose sizes and strides are
 // already in p.  Returns false when only the element-wise kernel fits.
-bool plan_gemm_kernel(Handle *h, RockGemmParams &p, int code, int es, const OptMap &o) {
+// `k_padded`: the caller guarantees that every K-contiguous operand row is
+// zero-filled from K up to the next whole 16-byte chunk (copies made by the
+// conversion plan), so K itself need not be a whole number of chunks.
+bool plan_gemm_kernel(Handle *h, RockGemmParams &p, int code, int es, const OptMap &o, bool k_padded = false) {
   const int64_t M = p.M, N = p.N, K = p.K, G = p.G;
   // vector path: K-contiguous rows of whole 16-byte chunks, and every byte
   // offset inside one block tile (256 rows at most) below 2^31 for the buffer
@@ -470,8 +478,9 @@ bool plan_gemm_kernel(Handle *h, RockGemmParams &p, int code, int es, const OptM
   auto al16 = [&](int64_t elems) { return (elems * es) % 16 == 0; };
   // each operand either K-contiguous (rows of whole chunks) or K-major (its
   // M / N index contiguous, k-rows of whole chunks: the transposing-read path)
-  const bool a_rows = p.a_ks == 1 && al16(p.a_ms) && al16(K) && al16(p.a_gs) && 256 * p.a_ms * es + K * es < kMaxOff;
-  const bool b_rows = p.b_ks == 1 && al16(p.b_ns) && al16(K) && al16(p.b_gs) && 256 * p.b_ns * es + K * es < kMaxOff;
+  const bool k_ok = al16(K) || k_padded;
+  const bool a_rows = p.a_ks == 1 && al16(p.a_ms) && k_ok && al16(p.a_gs) && 256 * p.a_ms * es + K * es < kMaxOff;
+  const bool b_rows = p.b_ks == 1 && al16(p.b_ns) && k_ok && al16(p.b_gs) && 256 * p.b_ns * es + K * es < kMaxOff;
   const bool a_cols = p.a_ms == 1 && al16(p.a_ks) && al16(M) && al16(p.a_gs) && K * p.a_ks * es + 256 * es < kMaxOff;
   const bool b_cols = p.b_ns == 1 && al16(p.b_ks) && al16(N) && al16(p.b_gs) && K * p.b_ks * es + 256 * es < kMaxOff;
   const bool fast = a_rows && b_rows;
@@ -504,7 +513,6 @@ bool plan_gemm_kernel(Handle *h, RockGemmParams &p, int code, int es, const OptM
     h->block_size = 256;
   h->kernel_name = std::string("rock_gemm_") + operand_name(code) + tile->suffix + (storage ? storage : "") +
                    rich_suffix(p.epi, tiled, o);
-  h->blob_name = std::string("gemm_") + operand_name(code);
   set_contraction_pointers(h, p.epi);
   h->perf_config = perf_string(*tile, es, &o);
   if (split_k > 1) { // the reference's grammar has a splitK field (7th)
@@ -549,6 +557,9 @@ bool parse_attn_perf(const std::string &pc, int &dmax, int &kpack_pb, int &force
   force_unroll = f[7];
   return true;
 }
+
+bool fill_relayout_handle(Handle *h, const int64_t size[5], const int64_t src_size[5],
+                          const int64_t src_stride[5], int es, const int64_t *dst_stride = nullptr);
 
 // ---- GEMM -----------------------------------------------------------------
 Handle *make_gemm(const OptMap &o) {
@@ -605,7 +616,98 @@ Handle *make_gemm(const OptMap &o) {
   p.b_gs = K * N; p.b_ks = tB ? 1 : N; p.b_ns = tB ? K : 1;
   p.c_gs = M * N; p.c_ms = tC ? 1 : N; p.c_ns = tC ? M : 1;
 
-  const bool vector_kernel = plan_gemm_kernel(h, p, code, dtype_size(ta), o);
+  bool vector_kernel = plan_gemm_kernel(h, p, code, dtype_size(ta), o);
+  // Padded copies.  An operand whose rows are not whole, aligned 16-byte chunks
+  // (an odd K, N = 60 under the default [K, N] storage) would leave the whole
+  // problem on the element-wise kernel.  Instead each such operand is first
+  // copied K-contiguous into the workspace by one conversion kernel, its rows
+  // zero-filled up to whole chunks, and the vector kernel reads the copies; the
+  // output is written as the caller laid it out.  The reference pads to block
+  // multiples inside its generated kernel and stays on the MFMA schedule
+  // (GridwiseGemmParams.cpp:91-103); this is the same through the multi-kernel
+  // protocol the library already speaks.
+  if (!vector_kernel && bool_or(o, "layout_conversion", true)) {
+    const int es = dtype_size(ta);
+    const int64_t ce = 16 / es, Kp = (K + ce - 1) / ce * ce;
+    auto al = [&](int64_t elems) { return (elems * es) % 16 == 0; };
+    // as plan_gemm_kernel reads them, with the K tail now allowed
+    const bool a_keep = (p.a_ks == 1 && al(p.a_ms) && al(p.a_gs) && p.a_ms >= Kp) || (p.a_ms == 1 && al(p.a_ks) && al(M) && al(p.a_gs));
+    const bool b_keep = (p.b_ks == 1 && al(p.b_ns) && al(p.b_gs) && p.b_ns >= Kp) || (p.b_ns == 1 && al(p.b_ks) && al(N) && al(p.b_gs));
+    // a kept K-contiguous operand must have zeros behind an odd K as well: only copies do
+    const bool need_a = !a_keep || (p.a_ks == 1 && Kp != K), need_b = !b_keep || (p.b_ks == 1 && Kp != K);
+    const int64_t a_bytes = align256(G * M * Kp * es), b_bytes = align256(G * N * Kp * es);
+    RockGemmParams q = p;
+    if (need_a) { q.a_gs = M * Kp; q.a_ms = Kp; q.a_ks = 1; }
+    if (need_b) { q.b_gs = N * Kp; q.b_ns = Kp; q.b_ks = 1; }
+    Handle probe;
+    probe.params.assign(sizeof q, 0);
+    if ((need_a || need_b) && G * M * Kp <= INT32_MAX && G * N * Kp <= INT32_MAX &&
+        plan_gemm_kernel(&probe, q, code, es, o, true)) {
+      // one conversion kernel: of the operand that needs it, or of both in one launch
+      const int n_copy = 1;
+      const int ws = p.epi.residual_op ? 5 : 4; // A, B, C, bias, [residual,] workspace
+      const int kid = (int)int_or(o, "kernel_id", 0);
+      if (kid < 0 || kid > n_copy) {
+        set_error("gemm: kernel_id out of range");
+        delete h;
+        return nullptr;
+      }
+      const int64_t off_a = 0, off_b = need_a ? a_bytes : 0;
+      if (kid == 0) {
+        auto fill = [&](Handle *dst, bool is_a) {
+          const int64_t rows = is_a ? M : N;
+          const int64_t size[5] = {1, 1, G, rows, Kp}, src_size[5] = {1, 1, G, rows, K};
+          const int64_t stride[5] = {0, 0, is_a ? p.a_gs : p.b_gs, is_a ? p.a_ms : p.b_ns, is_a ? p.a_ks : p.b_ks};
+          return fill_relayout_handle(dst, size, src_size, stride, es);
+        };
+        if (need_a && need_b) {
+          Handle first, second;
+          if (!fill(&first, true) || !fill(&second, false)) {
+            delete h;
+            return nullptr;
+          }
+          RockRelayoutPairParams pair;
+          std::memset(&pair, 0, sizeof pair);
+          std::memcpy(&pair.first, first.params.data(), sizeof pair.first);
+          std::memcpy(&pair.second, second.params.data(), sizeof pair.second);
+          pair.first_blocks = (int32_t)first.grid_size;
+          h->op = OP_RELAYOUT;
+          h->epi = nullptr;
+          h->params.assign(sizeof pair, 0);
+          std::memcpy(h->params.data(), &pair, sizeof pair);
+          h->kernel_name = std::string("rock_relayout_pair_b") + std::to_string(es);
+          h->block_size = 256;
+          h->grid_size = first.grid_size + second.grid_size;
+          h->num_pointers = 4;
+          h->perf_config = "";
+          h->ptr_map = {{0, 0}, {ws, off_a}, {1, 0}, {ws, off_b}};
+        } else {
+          if (!fill(h, need_a)) {
+            delete h;
+            return nullptr;
+          }
+          h->ptr_map = {{need_a ? 0 : 1, 0}, {ws, need_a ? off_a : off_b}};
+        }
+      } else {
+        p = q;
+        vector_kernel = plan_gemm_kernel(h, p, code, es, o, true);
+        h->ptr_map = {{need_a ? ws : 0, need_a ? off_a : 0}, {need_b ? ws : 1, need_b ? off_b : 0}, {2, 0}, {3, 0},
+                      {p.epi.residual_op ? 4 : -1, 0}};
+      }
+      { // every handle of the problem carries the problem's key
+        std::ostringstream k;
+        k << h->arch << '\t' << int_or(o, "num_cu", kNumCU) << '\t' << "-t " << operand_name(code)
+          << " -out_datatype " << dtype_name(tc) << " -transA " << (tA ? "true" : "false")
+          << " -transB " << (tB ? "true" : "false") << " -g " << G << " -m " << M << " -n " << N
+          << " -k " << K;
+        h->problem_key = k.str();
+      }
+      h->kernel_count = n_copy + 1;
+      h->workspace_bytes = (size_t)((need_a ? a_bytes : 0) + (need_b ? b_bytes : 0));
+      h->caller_pointers = ws + 1;
+      return h;
+    }
+  }
   // problem key (RockTuningImpl.cpp:808-862)
   auto set_key = [&](Handle *hh) {
     std::ostringstream k;
@@ -673,7 +775,6 @@ Handle *make_gemm(const OptMap &o) {
         h->params.assign(sizeof r, 0);
         std::memcpy(h->params.data(), &r, sizeof r);
         h->kernel_name = "rock_reduce_splits";
-        h->blob_name = "relayout";
         h->block_size = 256;
         h->grid_size = (uint32_t)((M * N + 255) / 256);
         h->num_pointers = 2;
@@ -706,7 +807,7 @@ Handle *make_gemm(const OptMap &o) {
 // source pointer.  Returns false with the error set when the tensor is too
 // large for the kernel's 32-bit indices.
 bool fill_relayout_handle(Handle *h, const int64_t size[5], const int64_t src_size[5],
-                          const int64_t src_stride[5], int es, const int64_t *dst_stride = nullptr) {
+                          const int64_t src_stride[5], int es, const int64_t *dst_stride) {
   RockRelayoutParams r;
   std::memset(&r, 0, sizeof r);
   struct Dim { int64_t size, src_size, ss, ds; };
@@ -801,7 +902,6 @@ bool fill_relayout_handle(Handle *h, const int64_t size[5], const int64_t src_si
   h->params.assign(sizeof r, 0);
   std::memcpy(h->params.data(), &r, sizeof r);
   h->kernel_name = std::string("rock_relayout_b") + std::to_string(es);
-  h->blob_name = "relayout";
   h->block_size = 256;
   h->grid_size = (uint32_t)blocks;
   h->num_pointers = 2;
@@ -930,7 +1030,6 @@ bool select_view_conv_kernel(Handle *h, RockConvParams &p, int ti, const OptMap 
   apply_tile_grid(*tile, Mg, p.k, p.g, p.tiles_m, p.tiles_n, p.group_m, p.xcd_remap, h->block_size, h->grid_size);
   h->op = OP_CONV;
   h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + tile->suffix;
-  h->blob_name = std::string("gemm_") + dtype_name(ti);
   h->num_pointers = 5;
   h->perf_config = perf_string(*tile, es, &o);
   return true;
@@ -970,7 +1069,6 @@ Handle *utility_fill_handle(int64_t bytes) {
   h->params.assign(sizeof f, 0);
   std::memcpy(h->params.data(), &f, sizeof f);
   h->kernel_name = "rock_fill_zero";
-  h->blob_name = "relayout";
   h->block_size = 256;
   h->grid_size = (uint32_t)((bytes + 16 * 256 - 1) / (16 * 256));
   h->num_pointers = 1;
@@ -1354,7 +1452,6 @@ Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
           h->params.assign(sizeof r, 0);
           std::memcpy(h->params.data(), &r, sizeof r);
           h->kernel_name = "rock_reduce_splits";
-          h->blob_name = "relayout";
           h->block_size = 256;
           h->grid_size = (uint32_t)((dw + 255) / 256);
           h->num_pointers = 2;
@@ -1522,7 +1619,6 @@ Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
     h->params.assign(sizeof r, 0);
     std::memcpy(h->params.data(), &r, sizeof r);
     h->kernel_name = "rock_reduce_splits";
-    h->blob_name = "relayout";
     h->block_size = 256;
     h->grid_size = (uint32_t)((dw_elems + 255) / 256);
     h->num_pointers = 2;
@@ -2096,7 +2192,6 @@ Handle *make_conv(const OptMap &o) {
   apply_tile_grid(*tile, Mg, k, (int)g, p.tiles_m, p.tiles_n, p.group_m, p.xcd_remap,
                   h->block_size, h->grid_size);
   h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + tile->suffix + rich_suffix(p.epi, fast, o);
-  h->blob_name = std::string("gemm_") + dtype_name(ti);
   h->num_pointers = 5;
   if (!planned)
     set_contraction_pointers(h, p.epi);
@@ -2199,7 +2294,6 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
     h->params.assign(sizeof r, 0);
     std::memcpy(h->params.data(), &r, sizeof r);
     h->kernel_name = "rock_softmax_rows";
-    h->blob_name = "relayout";
     h->block_size = 256;
     h->grid_size = (uint32_t)(G * sq);
     h->num_pointers = 3;
@@ -2322,7 +2416,6 @@ Handle *make_attention(const OptMap &o) {
   char name[96];
   std::snprintf(name, sizeof name, "rock_attention_%s_d%dx%d_%s", dtype_name(ty), dmax, dmax, variant->kind);
   h->kernel_name = name;
-  h->blob_name = "attention";
   // kernel pointers: Q, K, V, scale tensor, bias, O; a caller passes the scale
   // tensor only when the problem names one
   h->num_pointers = 6;
@@ -2580,9 +2673,9 @@ Handle *build_handle(const OptMap &o) {
     return nullptr;
   }
   h->num_cu = (int)int_or(o, "num_cu", kNumCU);
-  h->blob = find_blob(h->blob_name);
+  h->blob = find_blob(h->kernel_name);
   if (!h->blob) {
-    set_error("no code object for " + h->blob_name);
+    set_error("no code object for " + h->kernel_name);
     delete h;
     return nullptr;
   }
@@ -2899,6 +2992,10 @@ MiirStatus rockamdSetScale(MiirHandle handle, float scale) {
       name.erase(name.size() - 5);
       h->functions.clear();
     }
+    h->blob = find_blob(name); // one code object per kernel: the handle's follows its kernel
+    if (ends_with(plain) || ends_with(scaled))
+      h->perf_config = attn_perf_string(kAttnVariants[ends_with(scaled) ? 1 : 0],
+                                        name.find("_d64x") != std::string::npos ? 64 : 128);
   } else if (h->epi)
     h->epi->scale = scale;
   else
@@ -2978,7 +3075,8 @@ int rockamdMeasureMfmaRate(int dtype, int random_data, void *stream, double *ter
     set_error("rate probe: operand type must be f32, f16, bf16, i8 or fp8");
     return (int)hipErrorInvalidValue;
   }
-  const Blob *blob = find_blob("probe");
+  const std::string kname = std::string("rock_probe_mfma_") + names[dtype];
+  const Blob *blob = find_blob(kname);
   if (!blob)
     return (int)hipErrorInvalidValue;
   int dev = 0;
@@ -3000,7 +3098,6 @@ int rockamdMeasureMfmaRate(int dtype, int random_data, void *stream, double *ter
     }
   }
   hipFunction_t fn;
-  std::string kname = std::string("rock_probe_mfma_") + names[dtype];
   e = hipModuleGetFunction(&fn, mod, kname.c_str());
   if (e != hipSuccess)
     return (int)e;

@@ -48,7 +48,37 @@ def test_miir_protocol_conv(rock):
     assert lib.miirBufferGet(h, buf, C.byref(small)) == 1  # MIIR_INVALID_PARAM: too small
     assert lib.miirBufferGet(h, buf, C.byref(n)) == 0
     assert buf.raw[:4] == b"\x7fELF"  # mlir/test/mlir-rock-lib/populate_fw.mlir checks "ELF"
+    # one kernel per code object, as the reference hands them out (rocmlir-lib.cpp:292-316):
+    # the image holds the selected kernel alone and stays small
+    from rocmlir_amd._elf import kernel_symbols
+    name_len = C.c_size_t(0)
+    assert lib.rockamdGetKernelName(h, None, C.byref(name_len)) == 0
+    name = C.create_string_buffer(name_len.value)
+    assert lib.rockamdGetKernelName(h, name, C.byref(name_len)) == 0
+    assert kernel_symbols(buf.raw[:n.value]) == [name.value.decode()]
+    assert n.value <= 512 * 1024
     assert lib.miirDestroyHandle(h) == 0
+
+
+@pytest.mark.parametrize("options", [
+    "-operation gemm -arch gfx950 -t i8 -out_datatype f16 -g 1 -m 4096 -n 4096 -k 4096 -transB true -scale 0.01",
+    "-operation gemm -arch gfx950 -t fp8 -g 1 -m 8192 -n 8192 -k 8192 -transB true -residual add -activation gelu",
+    "-operation gemm -arch gfx950 -t f16 -g 1 -m 512 -n 512 -k 512",
+    "-operation gemm -arch gfx950 -t f32 -g 1 -m 512 -n 512 -k 512 -transB true",
+    "-operation gemm -arch gfx950 -t bf16 -g 1 -m 70 -n 45 -k 97 -layout_conversion false",
+    "-operation attention -arch gfx950 -t f16 -g 128 -seq_len_q 2048 -seq_len_k 2048 -head_dim_qk 128 "
+    "-head_dim_v 128 -transK true",
+    "-operation attention -arch gfx950 -t bf16 -g 2 -seq_len_q 64 -seq_len_k 64 -head_dim_qk 64 -head_dim_v 64",
+    CONV_RESNET.replace("NHWGC", "NGCHW").replace("GNYXC", "GNCHW"),                    # relayout kernel first
+    CONV_RESNET.replace("--operation conv", "--operation conv_bwd_weight") + " --kernel_id 2",
+])
+def test_every_handle_gets_its_kernel_alone(rock, options):
+    """miirBufferGet: a gfx950 ELF whose only kernel is the one the handle names, at most 512 KiB."""
+    from rocmlir_amd._elf import kernel_symbols
+    k = rock.RockKernel(options)
+    blob = k.code_object()
+    assert kernel_symbols(blob) == [k.kernel_name]
+    assert len(blob) <= 512 * 1024
 
 
 def test_null_handle_behaviour(rock):
@@ -114,10 +144,24 @@ def test_baseline_configs_select_kernels(rock):
 
 
 def test_generic_kernels_for_unaligned_or_transposed(rock):
-    k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 3 -m 1024 -k 769 -n 1024 -transB true")
+    odd_k = "-operation gemm -arch gfx950 -t f16 -g 3 -m 1024 -k 769 -n 1024 -transB true"
+    k = rock.RockKernel(odd_k + " -layout_conversion false")
     assert k.kernel_name == "rock_gemm_f16_64x64_generic"          # odd K: no 16-byte chunks
-    k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 64 -k 64 -n 60")
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 64 -k 64 -n 60 -layout_conversion false")
     assert k.kernel_name == "rock_gemm_f16_64x64_generic"          # B is [K,N] with rows of 120 bytes
+    # by default such operands are first copied into whole, zero-padded chunks (PrGemm.toml's
+    # -k 769: the reference pads inside its kernel, GridwiseGemmParams.cpp:91-103) and the
+    # vector kernel reads the copies: one launch copying both operands + the GEMM for the odd K,
+    # a copy of B + the GEMM for N = 60
+    plan = [rock.RockKernel("%s -kernel_id %d" % (odd_k, i)) for i in range(2)]
+    assert plan[0].kernel_name == "rock_relayout_pair_b2" and plan[0].num_pointers == 4
+    assert plan[1].kernel_name.startswith("rock_gemm_f16_") and plan[1].kernel_name.endswith("_fast")
+    assert plan[0].kernel_count == 2 and plan[0].workspace_bytes == 2 * 3 * 1024 * 776 * 2
+    assert plan[1].caller_pointers == 5 and plan[1].problem_key.endswith("-g 3 -m 1024 -n 1024 -k 769")
+    n60 = [rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 64 -k 64 -n 60 -kernel_id %d" % i)
+           for i in range(2)]
+    assert n60[0].kernel_name == "rock_relayout_b2" and n60[1].kernel_name.endswith("_fast")
+    assert n60[1].kernel_count == 2
     k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 64 -k 64 -n 64 -transA false -transB true")
     assert k.kernel_name.endswith("_fast")
     # K-major operands of whole 16-byte chunks take the transposing-read kernels
@@ -328,7 +372,7 @@ def test_elementwise_epilogue_options(rock):
     assert rock.RockKernel(base + " -residual add").kernel_name == k.kernel_name + "_e"
     assert rock.RockKernel(base + " -activation clip -clip_min 0 -clip_max 6").caller_pointers == 4
     # the element-wise kernels handle every epilogue themselves
-    odd = base.replace("-k 256", "-k 255")
+    odd = base.replace("-k 256", "-k 255") + " -layout_conversion false"
     assert rock.RockKernel(odd + " -activation erf").kernel_name == rock.RockKernel(odd).kernel_name
     assert rock.RockKernel(odd).kernel_name.endswith("_generic")
     for bad in (" -activation swish", " -activation clip", " -activation clip -clip_min 2 -clip_max 1",
@@ -443,8 +487,11 @@ def test_tuning_space_lists_the_kernels_a_problem_can_run_on(rock):
     # K-major operands have the three square tiles; unaligned ones only the generic kernel
     nn = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 256 -n 256 -k 256")
     assert len(nn.tuning_space()) == 3
-    gen = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 256 -n 250 -k 256")
+    gen = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 256 -n 250 -k 256 -layout_conversion false")
     assert gen.tuning_space() == [gen.perf_config]
+    # ... unless they are copied into padded ones first: the GEMM handle of that plan has the K-contiguous tiles
+    padded = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 256 -n 250 -k 256 -kernel_id 1")
+    assert padded.kernel_count == 2 and len(padded.tuning_space()) >= 4
     # raw entry points: bad position, short buffer
     lib = rock.load_library()
     sp = lib.rockamdTuningSpaceCreate(k._h, 1)

@@ -105,7 +105,7 @@ def test_gemm_residual_and_relu_exact(rock, oracle, gpu, kernel, t, od, op):
     kw = dict(scale=0.5, relu=True) if od != "i32" else {}
     out = rock.gemm(to_gpu(rawA, t, gpu), to_gpu(rawB, t, gpu), transB=tB, out_dtype=od,
                     residual=to_gpu(raw_res, od, gpu).reshape(G, M, N), residual_op=op, perf_config=pc,
-                    info=info, **kw)
+                    info=info, layout_conversion=name != "generic", **kw)
     if name not in ("generic", "split_k", "k_major"):
         assert name.split("_")[1] in info["kernel_name"]
     else:

@@ -51,8 +51,16 @@ def _run_case(rock, oracle, gpu, t, G, M, N, K, tA, tB, tC, integer, seed, out_d
 # every transpose combination x every operand type, ragged sizes (GemmVariants.toml:5-40)
 @pytest.mark.parametrize("t", ["f32", "f16", "bf16", "i8", "fp8", "bf8", "fp8_bf8", "bf8_fp8"])
 @pytest.mark.parametrize("tA,tB,tC", list(itertools.product([False, True], repeat=3)))
-def test_gemm_transposes_exact(rock, oracle, gpu, t, tA, tB, tC):
-    out, od, ref = _run_case(rock, oracle, gpu, t, 2, 70, 45, 97, tA, tB, tC, True, 100)
+@pytest.mark.parametrize("convert", [True, False], ids=["padded-copies", "element-wise"])
+def test_gemm_transposes_exact(rock, oracle, gpu, t, tA, tB, tC, convert):
+    """Nothing here is a whole 16-byte chunk: by default the operands are
+    copied into zero-padded K-contiguous ones and a vector kernel multiplies
+    the copies; `layout_conversion=False` keeps the element-wise kernel."""
+    info = {}
+    out, od, ref = _run_case(rock, oracle, gpu, t, 2, 70, 45, 97, tA, tB, tC, True, 100,
+                             layout_conversion=convert, info=info)
+    assert ("_generic" in info["kernel_name"]) == (not convert), info
+    assert len(info["kernels"]) == (2 if convert else 1), info
     got = to_f32(out, od)
     if t == "i8":
         fails, ovf, mad = oracle.verify_int(out.cpu().numpy().ravel(), ref)
@@ -94,6 +102,41 @@ def test_gemm_k_major_real_values_with_epilogue(rock, oracle, gpu):
                              out_dtype="f32", scale=0.5, bias=bias, relu=True, info=info)
     assert info["kernel_name"].endswith("_fast_nn")
     want = np.maximum(ref.reshape(384, 320) * 0.5 + bias.cpu().numpy()[None, :], 0.0)
+    check_float(to_f32(out, od), want.ravel(), od)
+
+
+# (G, M, N, K, transA, transB): odd K (PrGemm.toml's -k 769), N = 60 under the default
+# [K, N] storage, an unaligned M of a K-major A; one or both operands need a padded copy
+RAGGED = [(3, 100, 136, 769, False, True), (1, 64, 60, 64, False, False), (2, 50, 64, 72, True, True),
+          (1, 130, 60, 300, True, False), (1, 257, 129, 1025, False, True)]
+
+
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16", "i8", "fp8", "bf8"])
+@pytest.mark.parametrize("G,M,N,K,tA,tB", RAGGED)
+def test_gemm_ragged_operands_run_on_vector_kernels(rock, oracle, gpu, t, G, M, N, K, tA, tB):
+    info = {}
+    out, od, ref = _run_case(rock, oracle, gpu, t, G, M, N, K, tA, tB, False, True, 19, info=info)
+    # a vector kernel (tiled, or the K split over a block's waves), behind as many copies as
+    # operands needed one (none where a row happens to be whole chunks for this element size)
+    assert "_generic" not in info["kernel_name"] and len(info["kernels"]) in (1, 2), info
+    if t == "i8":
+        assert oracle.verify_int(out.cpu().numpy().ravel(), ref)[0] == 0
+    else:  # exact sums; only the narrowing to the output type rounds
+        assert np.array_equal(to_f32(out, od), oracle.round_through(ref, CODE[od]))
+
+
+def test_gemm_ragged_with_bias_residual_and_real_values(rock, oracle, gpu):
+    """The padded-copy plan keeps the epilogue's pointers in place: bias
+    vector, residual tensor, ReLU; real-valued f16 data to the RMS gate."""
+    G, M, N, K = 1, 200, 60, 769
+    rng = np.random.default_rng(23)
+    bias = torch.from_numpy(rng.uniform(-1, 1, N).astype(np.float32)).to(gpu)
+    res_raw, res_q = quantise(rng.uniform(-1, 1, (G, M, N)).astype(np.float32), "f16")
+    info = {}
+    out, od, ref = _run_case(rock, oracle, gpu, "f16", G, M, N, K, False, True, False, False, 21,
+                             bias=bias, residual=to_gpu(res_raw, "f16", gpu).reshape(G, M, N), relu=True, info=info)
+    assert "_generic" not in info["kernel_name"] and len(info["kernels"]) == 2
+    want = np.maximum(ref.reshape(M, N) + bias.cpu().numpy()[None, :] + res_q.reshape(M, N), 0.0)
     check_float(to_f32(out, od), want.ravel(), od)
 
 
