@@ -122,17 +122,27 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
   using Gm = AttnTileGeom<D>;
   constexpr int KSTEPS = D / 16;  // MFMA K steps of the first GEMM
   constexpr int DTILES = D / 32;  // 32-row tiles of O^T
-  constexpr int STAGE = 2 * Gm::TILE_B;
   constexpr float kLog2e = 1.44269504088896340736f;
   // The plain kernel software-pipelines the two GEMMs (see tile_step); the
   // bias kernel needs its registers for the bias gather and keeps the simple
   // order "scores, softmax, PV" per tile.
   constexpr bool PIPE = PLAIN;
-  static_assert(2 * STAGE <= 65536, "every LDS read offset must fit the 16-bit immediate");
+  static_assert(4 * Gm::TILE_B <= 65536, "every LDS read offset must fit the 16-bit immediate");
 
-  __shared__ __attribute__((aligned(1024))) char lds_generic[2 * STAGE];
-
-  attn_lds_char_t *lds = (attn_lds_char_t *)lds_generic;
+  // Every slot is an object of its own: the compiler makes an LDS read wait for
+  // the loads into LDS still in flight unless it can tell that the two touch
+  // different objects, and each phase of a tile reads one slot while the next
+  // tiles stream into the others.
+  __shared__ __attribute__((aligned(1024))) char lds_k0_generic[Gm::TILE_B];
+  __shared__ __attribute__((aligned(1024))) char lds_k1_generic[Gm::TILE_B];
+  __shared__ __attribute__((aligned(1024))) char lds_v0_generic[Gm::TILE_B];
+  __shared__ __attribute__((aligned(1024))) char lds_v1_generic[Gm::TILE_B];
+  attn_lds_char_t *const lds_k0 = (attn_lds_char_t *)lds_k0_generic;
+  attn_lds_char_t *const lds_k1 = (attn_lds_char_t *)lds_k1_generic;
+  attn_lds_char_t *const lds_v0 = (attn_lds_char_t *)lds_v0_generic;
+  attn_lds_char_t *const lds_v1 = (attn_lds_char_t *)lds_v1_generic;
+  auto k_slot = [&](int slot) __attribute__((always_inline)) { return slot ? lds_k1 : lds_k0; };
+  auto v_slot = [&](int slot) __attribute__((always_inline)) { return slot ? lds_v1 : lds_v0; };
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -161,10 +171,10 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
   AttnTileLoader<D, true> lv;
   lk.init(K, p.k_js, p.seq_k, p.d_qk, wave, lane);
   lv.init(V, p.v_js, p.seq_k, p.d_v, wave, lane);
-  lk.issue(0, lds);
-  lv.issue(0, lds + Gm::TILE_B);
+  lk.issue(0, k_slot(0));
+  lv.issue(0, v_slot(0));
   if constexpr (PIPE)
-    lk.issue(kBKV, lds + 2 * Gm::TILE_B);
+    lk.issue(kBKV, k_slot(1));
 
   v4i qf[KSTEPS];
 #pragma unroll
@@ -174,17 +184,17 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
   // ---- per-lane LDS read offsets (bytes from the start of a K or V tile)
   // K fragment of key rows 32*st + lq at chunk 2*ks + h: the swizzle depends on
   // lq only, so "+ 32*st rows" and the stage are immediates.
-  attn_lds_char_t *const krow = lds + lq * Gm::ROWB;
+  const int krow = lq * Gm::ROWB; // byte offset inside a K tile
   const int kswz = (h ^ attn_swz<Gm::CPR, false>(lq)) * 16; // chunk 2*ks + h: ks XORs in as a constant
-  auto kptr = [&](int ks) __attribute__((always_inline)) { return krow + (kswz ^ (ks * 32)); };
+  auto koff = [&](int ks) __attribute__((always_inline)) { return krow + (kswz ^ (ks * 32)); };
   // V^T fragment through the transposing read: lane (i = lane % 16, g16) of
   // half h addresses key 4*h + i/4 (+ 32*st + 16*u, + 8) at d = 32*dt + 16*g16 + 4*(i%4).
   const int tr_i = lane & 15, tr_g = (lane >> 4) & 1;
   const int tr_key = 4 * h + (tr_i >> 2);
   const int tr_chunk = 2 * tr_g + ((tr_i & 3) >> 1);
-  attn_lds_char_t *const vrow = lds + Gm::TILE_B + tr_key * Gm::ROWB + (tr_i & 1) * 8;
+  const int vrow = tr_key * Gm::ROWB + (tr_i & 1) * 8; // byte offset inside a V tile
   const int vswz = (tr_chunk ^ attn_swz<Gm::CPR, true>(tr_key)) * 16; // chunk 4*dt + tr_chunk
-  auto vptr = [&](int dt) __attribute__((always_inline)) { return vrow + (vswz ^ (dt * 64)); };
+  auto voff = [&](int dt) __attribute__((always_inline)) { return vrow + (vswz ^ (dt * 64)); };
 
   v16f o[DTILES];
 #pragma unroll
@@ -208,7 +218,7 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
         s[st][v] = 0.0f;
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) {
-        v4i kf = *(const attn_lds_v4i_t *)(kptr(ks) + (SLOT * STAGE + st * 32 * Gm::ROWB));
+        v4i kf = *(const attn_lds_v4i_t *)(k_slot(SLOT) + koff(ks) + st * 32 * Gm::ROWB);
         s[st] = mma32<DT>(kf, qf[ks], s[st]);
       }
     }
@@ -226,17 +236,16 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
     v16f(&s)[2] = PIPE ? s_in : s_here;
     constexpr int PAR = decltype(par_const)::value;
     constexpr bool LAST = decltype(last_const)::value; // no tile t+1: nothing to issue ahead
-    constexpr int STG = PAR;
     wait_loads_and_lds_reads();       // this wave's parts of K[t+1] and V[t] have landed ...
     __builtin_amdgcn_s_barrier();     // ... everyone's have; K[t] and V[t-1] are no longer read
     if constexpr (!PIPE) {
       // plain double buffering: request tile t+1, then compute tile t's scores
-      lk.issue((t + 1) * kBKV, lds + (PAR ^ 1) * STAGE); // past the end: zeros, no traffic
-      lv.issue((t + 1) * kBKV, lds + (PAR ^ 1) * STAGE + Gm::TILE_B);
+      lk.issue((t + 1) * kBKV, k_slot(PAR ^ 1)); // past the end: zeros, no traffic
+      lv.issue((t + 1) * kBKV, v_slot(PAR ^ 1));
       scores(std::integral_constant<int, PAR>{}, s);
     } else if constexpr (!LAST) {
-      lk.issue((t + 2) * kBKV, lds + PAR * STAGE); // past the end: zeros, no traffic
-      lv.issue((t + 1) * kBKV, lds + (PAR ^ 1) * STAGE + Gm::TILE_B);
+      lk.issue((t + 2) * kBKV, k_slot(PAR)); // past the end: zeros, no traffic
+      lv.issue((t + 1) * kBKV, v_slot(PAR ^ 1));
     }
 
     // ---- online softmax on this lane's 32 scores of row q_row
@@ -328,7 +337,7 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
         constexpr int kSliceB = 16 * Gm::ROWB; // 16 keys
 #pragma unroll
         for (int dt = 0; dt < DTILES; ++dt) {
-          attn_lds_char_t *a0 = vptr(dt) + (STG * STAGE + (st * 2 + u) * kSliceB);
+          attn_lds_char_t *a0 = v_slot(PAR) + voff(dt) + (st * 2 + u) * kSliceB;
           v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((attn_lds_v4s_t *)a0);
           v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((attn_lds_v4s_t *)(a0 + 8 * Gm::ROWB));
           v2i l2 = __builtin_bit_cast(v2i, lo), h2 = __builtin_bit_cast(v2i, hi);

@@ -324,7 +324,7 @@ __device__ __forceinline__ Frag<DT> dl_read_frag_km(const char *stage, int colbl
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int row = kb + 4 * j + (l16 >> 2);
-        const char *a = stage + row * Kg::ROWB + ((((colbyte >> 4) ^ Kg::swz(row))) << 4) + (colbyte & 15);
+        const char *a = stage + (row * Kg::ROWB + ((((colbyte >> 4) ^ Kg::swz(row))) << 4) + (colbyte & 15));
         part[j] = __builtin_bit_cast(v2i, __builtin_amdgcn_ds_read_tr16_b64_v4i16((km_lds_v4s_t *)a));
       }
       f.c[c] = v4i{part[0][0], part[0][1], part[1][0], part[1][1]};
@@ -334,7 +334,7 @@ __device__ __forceinline__ Frag<DT> dl_read_frag_km(const char *stage, int colbl
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int row = kb + 8 * j + (l16 >> 1);
-        const char *a = stage + row * Kg::ROWB + ((((colbyte >> 4) ^ Kg::swz(row))) << 4) + (colbyte & 15);
+        const char *a = stage + (row * Kg::ROWB + ((((colbyte >> 4) ^ Kg::swz(row))) << 4) + (colbyte & 15));
         part[j] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((km_lds_v2i_t *)a);
       }
       f.c[c] = v4i{part[0][0], part[0][1], part[1][0], part[1][1]};
@@ -841,7 +841,18 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
   constexpr int BKE = RB / Tr::ES;
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of 32");
 
-  __shared__ __attribute__((aligned(1024))) char lds[kDlStages * STAGE];
+  // With a K-major operand the two stages are two LDS objects and the loop is
+  // unrolled over them: the compiler puts an s_waitcnt vmcnt(0) in front of every
+  // transposing LDS read that follows a load into LDS unless it can tell that
+  // the two touch different objects -- between the refill of one stage and the
+  // fragment reads of the other that wait would expose the whole load latency
+  // in every K-step of the loading waves.
+  constexpr bool KM = LDA == LD_COLS_FAST || LDB == LD_COLS_FAST;
+  static_assert(!KM || kDlStages == 2, "K-major operands: two stages, one LDS object each");
+  constexpr int WBUF = 32 * (WTN * 4 + 16); // the epilogue's staging region per wave
+  static_assert(!KM || (NW / 2) * WBUF <= STAGE, "half the waves stage their stores in each stage");
+  __shared__ __attribute__((aligned(1024))) char lds[KM ? STAGE : kDlStages * STAGE];
+  __shared__ __attribute__((aligned(1024))) char lds_hi[KM ? STAGE : 1024]; // K-major only
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -886,17 +897,16 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
     }
   }
 
-  for (int kt = 0; kt < nk; ++kt) {
+  // K-step kt: multiplies the stage at `sa`, refills the stage at `refill`
+  auto kstep = [&](int kt, const char *sa, char *refill) __attribute__((always_inline)) {
     // this wave's loads of K-step kt have landed (two younger steps may be in flight) ...
     wait_vmcnt_and_lds_reads<(kDlStages - 2) * LOADS_PER_STEP>();
     // ... and so have everyone else's; everyone is also done reading step kt-1
     __builtin_amdgcn_s_barrier();
     if (loader) {
-      char *refill = lds + ((kt + kDlStages - 1) % kDlStages) * STAGE;
       la.issue(kt + kDlStages - 1, refill);
       lb.issue(kt + kDlStages - 1, refill + A_BYTES);
     }
-    const char *sa = lds + (kt % kDlStages) * STAGE;
     const char *sb = sa + A_BYTES;
     // the fragments of MFMA step s + 1 are fetched while the MFMAs of step s run
     Frag<DT> fa[2][MI], fb[2][NI];
@@ -944,12 +954,28 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
       }
       __builtin_amdgcn_sched_group_barrier(0x008, MI * NI, 0);
     }
+  };
+  if constexpr (KM) {
+    int kt = 0;
+    for (; kt + 1 < nk; kt += 2) {
+      kstep(kt, lds, lds_hi);
+      kstep(kt + 1, lds_hi, lds);
+    }
+    if (kt < nk)
+      kstep(kt, lds, lds_hi);
+  } else {
+    for (int kt = 0; kt < nk; ++kt)
+      kstep(kt, lds + (kt % kDlStages) * STAGE, lds + ((kt + kDlStages - 1) % kDlStages) * STAGE);
   }
   // drain the out-of-range loads issued for steps >= nk before the LDS is released
   wait_vmcnt<0>();
 
-  dl_epilogue<DT, MI, NI, NW, kDlStages * STAGE, RICH>(acc, p, g, Cptr, aux, res, m0 + wm * WTM, n0 + wn * WTN, lds, wave,
-                                                 lane);
+  // the epilogue's staging region of wave w starts WBUF * w bytes behind the pointer it is given
+  char *staging = lds;
+  if constexpr (KM)
+    staging = wave < NW / 2 ? lds : lds_hi - (NW / 2) * WBUF;
+  dl_epilogue<DT, MI, NI, NW, kDlStages * STAGE, RICH>(acc, p, g, Cptr, aux, res, m0 + wm * WTM, n0 + wn * WTN, staging,
+                                                       wave, lane);
 }
 
 } // namespace rk
