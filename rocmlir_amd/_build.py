@@ -9,6 +9,7 @@ miirBufferGet returns the selected kernel alone.  This file holds the list of
 kernels; the sources under csrc/ hold the kernel bodies and the macros that
 instantiate them."""
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -33,6 +34,8 @@ DEVICE_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "--cuda-device-only", "--no-gpu-bundle-output", "-I", CSRC,
 ]
+
+SPILL_WARN = 32  # spilled vector registers above which the build prints a warning
 
 # (block tile rows, columns, waves along M, waves along N) of the tiled kernels
 TILES = {"_256x256": (256, 256, 2, 4), "_256x128": (256, 128, 4, 2),
@@ -149,9 +152,14 @@ def _compile(job):
     if text is not None:
         with open(src, "w") as f:
             f.write(text)
-    log = _run([HIPCC] + DEVICE_FLAGS + flags + ["-o", out, src])
+    log = _run([HIPCC] + DEVICE_FLAGS + flags + ["-Rpass-analysis=kernel-resource-usage", "-o", out, src])
     _check(name)
-    return log
+    # registers spilled to scratch memory: a handful outside the main loop is
+    # harmless, hundreds mean a kernel that lost its registers to a code change
+    spilled = [int(m) for m in re.findall(r"VGPRs Spill: (\d+)", log)]
+    if spilled and max(spilled) > SPILL_WARN:
+        sys.stderr.write("warning: %s spills %d vector registers\n" % (name, max(spilled)))
+    return "\n".join(l for l in log.splitlines() if ("warning:" in l or "error:" in l) and "-Rpass" not in l)
 
 
 def build(jobs=8, verbose=False, host_only=False, only=None, incremental=False):

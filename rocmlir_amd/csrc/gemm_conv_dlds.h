@@ -343,7 +343,7 @@ __device__ __forceinline__ Frag<DT> dl_read_frag_km(const char *stage, int colbl
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         const int row = kb + t;
-        f.c[c][t] = *(const int *)(stage + row * Kg::ROWB + ((((colbyte >> 4) ^ Kg::swz(row))) << 4) + (colbyte & 15));
+        f.c[c][t] = *(const int *)(stage + (row * Kg::ROWB + ((((colbyte >> 4) ^ Kg::swz(row))) << 4) + (colbyte & 15)));
       }
     }
   }
@@ -847,7 +847,9 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
   // the two touch different objects -- between the refill of one stage and the
   // fragment reads of the other that wait would expose the whole load latency
   // in every K-step of the loading waves.
-  constexpr bool KM = LDA == LD_COLS_FAST || LDB == LD_COLS_FAST;
+  // (Not for the 256x256 tile of the 8-bit float types: 128 accumulators and 96
+  // fragment registers leave the unrolled loop no room and it spills.)
+  constexpr bool KM = (LDA == LD_COLS_FAST || LDB == LD_COLS_FAST) && !(Tr::CHUNKS == 2 && BM * BN >= 256 * 256);
   static_assert(!KM || kDlStages == 2, "K-major operands: two stages, one LDS object each");
   constexpr int WBUF = 32 * (WTN * 4 + 16); // the epilogue's staging region per wave
   static_assert(!KM || (NW / 2) * WBUF <= STAGE, "half the waves stage their stores in each stage");
@@ -899,6 +901,16 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
 
   // K-step kt: multiplies the stage at `sa`, refills the stage at `refill`
   auto kstep = [&](int kt, const char *sa, char *refill) __attribute__((always_inline)) {
+    if constexpr (KM) {
+      // The unrolled loop has every fragment address of either stage as a loop
+      // invariant, and hoisting them all costs the 8-bit kernels their registers
+      // (the second stage lies beyond the reach of the reads' 16-bit offset
+      // field).  An offset of zero that the compiler cannot see through keeps
+      // the address arithmetic of a step inside the step, one add per read.
+      int zero = 0;
+      asm volatile("" : "+s"(zero));
+      sa += zero;
+    }
     // this wave's loads of K-step kt have landed (two younger steps may be in flight) ...
     wait_vmcnt_and_lds_reads<(kDlStages - 2) * LOADS_PER_STEP>();
     // ... and so have everyone else's; everyone is also done reading step kt-1
