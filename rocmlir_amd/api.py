@@ -548,7 +548,7 @@ def conv2d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize,
 
 
 def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, zero_point=0, transQ=False, transK=False,
-              transV=False, transO=False, out=None, stream=None):
+              transV=False, transO=False, out=None, stream=None, info=None):
     """O = softmax(scale * scale_tensor * Q K + bias) V (bias and scale_tensor
     optional [G,seq_q,seq_k] tensors, rocmlir-gen's -with-attn-bias /
     -with-attn-scale) with the reference's storage
@@ -556,7 +556,8 @@ def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, zero_point=0,
     transQ); k [G,d,seq_k] ([G,seq_k,d] if transK -- the usual row-major keys);
     v [G,seq_k,dv] ([G,dv,seq_k] if transV); result [G,seq_q,dv]
     ([G,dv,seq_q] if transO).  int8 q and k (with f16 v, bias, scale_tensor)
-    select the quantised first GEMM: the scores are (acc - zero_point) * scale."""
+    select the quantised first GEMM: the scores are (acc - zero_point) * scale.
+    A dict passed as `info` receives the names of the kernels that ran."""
     import torch
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     G = q.shape[0]
@@ -577,6 +578,8 @@ def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, zero_point=0,
     if zero_point:
         opts += " -zero_point %d" % zero_point
     kern = _program(opts)   # one fused kernel, or three for head dimensions above 128 and f32
+    if info is not None:
+        info["kernels"] = [k.kernel_name for k in kern.kernels]
     shape = (G, dv, sq) if transO else (G, sq, dv)
     if out is None:
         out = torch.empty(shape, dtype=v.dtype, device=q.device)

@@ -49,10 +49,11 @@ template <int D> struct AttnTileGeom {
 // from the lane), so the row index is XOR-ed into the chunk bits above them.
 // Each function spreads its access pattern over distinct bank groups for the
 // row pitch at hand (256 bytes = one full bank period for D = 128, half a
-// period for D = 64), and depends only on the row modulo 16 (K) or 8 (V).
+// period for D = 64, a quarter for int8 keys at D = 64), and depends only on
+// the row modulo 16 (K) or 8 (V).
 template <int CPR, bool IS_V> __device__ __forceinline__ int attn_swz(int row) {
-  if constexpr (!IS_V)
-    return CPR == 16 ? (row & 15) : ((row >> 1) & 7);
+  if constexpr (!IS_V) // 256 / 128 / 64 bytes per row (the last: int8 keys of a head dimension up to 64)
+    return CPR == 16 ? (row & 15) : CPR == 8 ? ((row >> 1) & 7) : ((row >> 2) & 3);
   else
     return CPR == 16 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2);
 }
@@ -115,12 +116,19 @@ template <int DT> __device__ __forceinline__ uint32_t pack2_fast(float a, float 
 
 // PLAIN: no bias and a non-negative scale, so the row maximum can be taken on
 // the raw scores and the scale folded into the exponent.
-template <int DT, int D, bool PLAIN>
+// QKI8: Q and K are int8 and the first GEMM runs on the int8 MFMA; its int32
+// sums are dequantised on the score tile in registers, (acc - zero_point) *
+// scale, before anything else touches them (the quantised first GEMM of
+// mlir/test/fusion/pr-e2e/attention/mixr-attention-first-gemm-i8-f16.mlir).
+// V, the pre-softmax tensors and O stay DT.  D counts elements, so a K row is
+// D bytes and the K tile has the geometry of a 16-bit tile of D / 2.
+template <int DT, int D, bool PLAIN, bool QKI8 = false>
 __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv, const void *Vv,
                                                   const void *scalev, const void *biasv, void *Ov,
                                                   const RockAttentionParams &p) {
-  using Gm = AttnTileGeom<D>;
-  constexpr int KSTEPS = D / 16;  // MFMA K steps of the first GEMM
+  using Gm = AttnTileGeom<D>;                  // V tile
+  using GmK = AttnTileGeom<QKI8 ? D / 2 : D>;  // K tile
+  constexpr int KSTEPS = QKI8 ? D / 32 : D / 16; // MFMA K steps of the first GEMM
   constexpr int DTILES = D / 32;  // 32-row tiles of O^T
   constexpr float kLog2e = 1.44269504088896340736f;
   // The plain kernel software-pipelines the two GEMMs (see tile_step); the
@@ -133,8 +141,8 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
   // the loads into LDS still in flight unless it can tell that the two touch
   // different objects, and each phase of a tile reads one slot while the next
   // tiles stream into the others.
-  __shared__ __attribute__((aligned(1024))) char lds_k0_generic[Gm::TILE_B];
-  __shared__ __attribute__((aligned(1024))) char lds_k1_generic[Gm::TILE_B];
+  __shared__ __attribute__((aligned(1024))) char lds_k0_generic[GmK::TILE_B];
+  __shared__ __attribute__((aligned(1024))) char lds_k1_generic[GmK::TILE_B];
   __shared__ __attribute__((aligned(1024))) char lds_v0_generic[Gm::TILE_B];
   __shared__ __attribute__((aligned(1024))) char lds_v1_generic[Gm::TILE_B];
   attn_lds_char_t *const lds_k0 = (attn_lds_char_t *)lds_k0_generic;
@@ -167,9 +175,12 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
   const uint16_t *bias = p.has_bias ? (const uint16_t *)biasv + (int64_t)g * p.bias_gs : nullptr;
   const uint16_t *scale_t = p.has_scale_tensor ? (const uint16_t *)scalev + (int64_t)g * p.bias_gs : nullptr;
 
-  AttnTileLoader<D, false> lk;
+  AttnTileLoader<QKI8 ? D / 2 : D, false> lk;
   AttnTileLoader<D, true> lv;
-  lk.init(K, p.k_js, p.seq_k, p.d_qk, wave, lane);
+  if constexpr (QKI8) // int8 rows seen as 16-bit rows of half the length (strides are even: host check)
+    lk.init((const uint16_t *)((const char *)Kv + (int64_t)g * p.k_gs), p.k_js / 2, p.seq_k, p.d_qk / 2, wave, lane);
+  else
+    lk.init(K, p.k_js, p.seq_k, p.d_qk, wave, lane);
   lv.init(V, p.v_js, p.seq_k, p.d_v, wave, lane);
   lk.issue(0, k_slot(0));
   lv.issue(0, v_slot(0));
@@ -178,14 +189,21 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
 
   v4i qf[KSTEPS];
 #pragma unroll
-  for (int ks = 0; ks < KSTEPS; ++ks)
-    qf[ks] = load8<true>(Q, p.q_is, p.q_ds, q_row, ks * 16 + h * 8, p.seq_q, p.d_qk);
+  for (int ks = 0; ks < KSTEPS; ++ks) {
+    if constexpr (QKI8) {
+      const int col = ks * 32 + h * 16; // 16 int8 values of this lane's query row
+      const char *q8 = (const char *)Qv + (int64_t)g * p.q_gs + (int64_t)q_row * p.q_is + col;
+      qf[ks] = (q_row < p.seq_q && col < p.d_qk) ? *(const v4i *)q8 : v4i{0, 0, 0, 0};
+    } else {
+      qf[ks] = load8<true>(Q, p.q_is, p.q_ds, q_row, ks * 16 + h * 8, p.seq_q, p.d_qk);
+    }
+  }
 
   // ---- per-lane LDS read offsets (bytes from the start of a K or V tile)
   // K fragment of key rows 32*st + lq at chunk 2*ks + h: the swizzle depends on
   // lq only, so "+ 32*st rows" and the stage are immediates.
-  const int krow = lq * Gm::ROWB; // byte offset inside a K tile
-  const int kswz = (h ^ attn_swz<Gm::CPR, false>(lq)) * 16; // chunk 2*ks + h: ks XORs in as a constant
+  const int krow = lq * GmK::ROWB; // byte offset inside a K tile
+  const int kswz = (h ^ attn_swz<GmK::CPR, false>(lq)) * 16; // chunk 2*ks + h: ks XORs in as a constant
   auto koff = [&](int ks) __attribute__((always_inline)) { return krow + (kswz ^ (ks * 32)); };
   // V^T fragment through the transposing read: lane (i = lane % 16, g16) of
   // half h addresses key 4*h + i/4 (+ 32*st + 16*u, + 8) at d = 32*dt + 16*g16 + 4*(i%4).
@@ -213,13 +231,26 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
     constexpr int SLOT = decltype(slot_const)::value;
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
+      if constexpr (QKI8) {
+        v16i acc;
 #pragma unroll
-      for (int v = 0; v < 16; ++v)
-        s[st][v] = 0.0f;
+        for (int v = 0; v < 16; ++v)
+          acc[v] = 0;
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        v4i kf = *(const attn_lds_v4i_t *)(k_slot(SLOT) + koff(ks) + st * 32 * Gm::ROWB);
-        s[st] = mma32<DT>(kf, qf[ks], s[st]);
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          v4i kf = *(const attn_lds_v4i_t *)(k_slot(SLOT) + koff(ks) + st * 32 * GmK::ROWB);
+          acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[ks], acc, 0, 0, 0);
+        }
+        s[st] = __builtin_bit_cast(v16f, acc); // dequantised where the tile's softmax starts
+      } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          s[st][v] = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          v4i kf = *(const attn_lds_v4i_t *)(k_slot(SLOT) + koff(ks) + st * 32 * GmK::ROWB);
+          s[st] = mma32<DT>(kf, qf[ks], s[st]);
+        }
       }
     }
   };
@@ -248,6 +279,16 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
       lv.issue((t + 1) * kBKV, v_slot(PAR ^ 1));
     }
 
+    if constexpr (QKI8) {
+      const float zp = (float)p.zero_point;
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const float raw = s[st][v]; // (a bit cast applied to a vector element directly reads element 0)
+          s[st][v] = (float)__builtin_bit_cast(int, raw) - zp;
+        }
+    }
     // ---- online softmax on this lane's 32 scores of row q_row
     const int key_base = t * kBKV + 4 * h;
     const bool tail = LAST && (t + 1) * kBKV > p.seq_k; // only the last tile can be ragged

@@ -370,6 +370,14 @@ __device__ __forceinline__ void wait_loads_and_lds_reads() {
 // The build (rocmlir_amd/_build.py holds the list) compiles every kernel into a
 // code object of its own from a small source that includes this file and
 // invokes one of the two macros.
+// int8 Q and K, f16 V / bias / O
+#define RK_ATTN_DL_I8(D, SUFFIX, PLAIN)                                                       \
+  extern "C" __global__ __launch_bounds__(rk::kAttnThreads, 2) void                           \
+      rock_attention_i8_d##D##x##D##_##SUFFIX(const void *Q, const void *K, const void *V,    \
+                                              const void *scale, const void *bias, void *O,   \
+                                              RockAttentionParams p) {                        \
+    rk::attention_body_dl<MM_F16, D, PLAIN, true>(Q, K, V, scale, bias, O, p);                \
+  }
 #define RK_ATTN_DL(DTNAME, DT, D, SUFFIX, PLAIN)                                              \
   extern "C" __global__ __launch_bounds__(rk::kAttnThreads, 2) void                           \
       rock_attention_##DTNAME##_d##D##x##D##_##SUFFIX(const void *Q, const void *K,           \

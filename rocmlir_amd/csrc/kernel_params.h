@@ -165,4 +165,6 @@ struct RockAttentionParams {
   int32_t has_bias;
   int32_t xcd_remap;
   int32_t has_scale_tensor; // scores are multiplied element-wise by the scale tensor before `scale`
+  int32_t zero_point;       // int8 Q and K: the scores are (int32 sum - zero_point) * scale
+  int32_t pad_;
 };

@@ -2362,8 +2362,18 @@ Handle *make_attention(const OptMap &o) {
   // "-with-attn-scale": a full [G, seq_q, seq_k] tensor multiplied into the
   // scores before the softmax (rocmlir-gen.cpp:2185-2196), besides the scalar "-scale"
   bool has_scale_t = bool_or(o, "with-attn-scale", false);
-  if (ty == ROCK_F32 || ty == ROCK_I8 || dqk > 128 || dv > 128)
-    return make_attention_unfused(o, ty, G, sq, sk, dqk, dv, tQ, tK, tV, tO, has_bias, has_scale_t);
+  // "-t i8": int8 Q and K (the quantised first GEMM), f16 V, pre-softmax tensors and O
+  const bool qk_i8 = ty == ROCK_I8;
+  {
+    // the fused kernels: head dimensions up to 128, tensors contiguous along the head dimension in
+    // whole 16-byte chunks; int8 Q and K only on the vector kernels
+    const bool i8_fused = qk_i8 && !tQ && tK && !tV && !tO && dqk % 16 == 0 && dv % 8 == 0 &&
+                          sk * dqk < ((int64_t)1 << 31) && sk * dv * 2 < ((int64_t)1 << 31) &&
+                          ((!has_bias && !has_scale_t) || sq * sk < ((int64_t)1 << 31)) &&
+                          bool_or(o, "fused", true);
+    if (ty == ROCK_F32 || (qk_i8 && !i8_fused) || dqk > 128 || dv > 128)
+      return make_attention_unfused(o, ty, G, sq, sk, dqk, dv, tQ, tK, tV, tO, has_bias, has_scale_t);
+  }
 
   auto *h = new Handle;
   h->op = OP_ATTENTION;
@@ -2382,6 +2392,7 @@ Handle *make_attention(const OptMap &o) {
   p.has_scale_tensor = has_scale_t ? 1 : 0;
   p.scale = 1.0f;
   get_float(o, "scale", p.scale);
+  p.zero_point = qk_i8 ? (int32_t)int_or(o, "zero_point", 0) : 0;
   p.q_blocks = ceil_div(sq, 128);
   int64_t total = G * p.q_blocks;
   if (total > INT32_MAX) {
@@ -2390,7 +2401,8 @@ Handle *make_attention(const OptMap &o) {
     return nullptr;
   }
   p.xcd_remap = total >= 2 * kNumXCD ? 1 : 0;
-  const bool fast = p.q_ds == 1 && p.k_ds == 1 && p.v_es == 1 && p.o_es == 1 && dqk % 8 == 0 &&
+  const bool fast = qk_i8 || // checked above: there is no element-wise int8 kernel to fall back to
+                    p.q_ds == 1 && p.k_ds == 1 && p.v_es == 1 && p.o_es == 1 && dqk % 8 == 0 &&
                     dv % 8 == 0 && p.o_is % 4 == 0 && p.k_js % 8 == 0 && p.v_js % 8 == 0 &&
                     p.q_is % 8 == 0 &&
                     // byte offsets inside one g slice below 2^31 (buffer descriptors)
@@ -2407,7 +2419,7 @@ Handle *make_attention(const OptMap &o) {
     if (parse_attn_perf(str_or(o, "perf_config", ""), want_d, want_kpack, want_unroll)) {
       if ((want_d == 64 || want_d == 128) && want_d >= dmax)
         dmax = want_d;
-      if (want_kpack == 1)
+      if (want_kpack == 1 && !qk_i8)
         variant = &kAttnVariants[2];
       else if (fast && want_kpack == 8)
         variant = (want_unroll != 0 && plain_ok) ? &kAttnVariants[0] : &kAttnVariants[1];

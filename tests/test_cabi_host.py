@@ -315,10 +315,21 @@ def test_attention_as_three_kernels(rock):
         assert ks[2].kernel_name.startswith("rock_gemm_%s_" % t) and ks[2].kernel_name.endswith("_fast_nn")
         assert all(k.kernel_count == 3 and k.workspace_bytes == 16384 * 16384 * 4 and k.caller_pointers == 6
                    for k in ks)
-    # int8 first GEMM: int8 contraction into f32 scores, f16 from there on
-    q8 = [rock.RockKernel("-operation attention -arch gfx950 -t i8 -g 2 -seq_len_q 128 -seq_len_k 128 -head_dim_qk 64 "
-                          "-head_dim_v 64 -transK true -zero_point 3 -scale 0.001 -kernel_id %d" % i) for i in range(3)]
-    assert q8[0].kernel_name.startswith("rock_gemm_i8_") and q8[2].kernel_name.startswith("rock_gemm_f16_")
+    # int8 first GEMM: one fused kernel where the layout allows it (its score tile is dequantised in
+    # registers); "-fused false", K stored [G, d, seq_k] or a head dimension above 128 give the three
+    # kernels: int8 contraction into f32 scores, f16 from there on
+    i8 = ("-operation attention -arch gfx950 -t i8 -g 2 -seq_len_q 128 -seq_len_k 128 -head_dim_qk 64 "
+          "-head_dim_v 64 -transK true -zero_point 3 -scale 0.001")
+    fused = rock.RockKernel(i8)
+    assert fused.kernel_name == "rock_attention_i8_d64x64_fast" and fused.kernel_count == 1
+    assert fused.workspace_bytes == 0 and fused.caller_pointers == 5
+    with pytest.raises(rock.RockError):
+        rock.RockKernel(i8 + " -kernel_id 1")
+    for three in (i8 + " -fused false", i8.replace("-transK true", "-transK false"),
+                  i8.replace("-head_dim_qk 64", "-head_dim_qk 256")):
+        q8 = [rock.RockKernel(three + " -kernel_id %d" % i) for i in range(3)]
+        assert q8[0].kernel_name.startswith("rock_gemm_i8_") and q8[2].kernel_name.startswith("rock_gemm_f16_")
+        assert q8[1].kernel_name == "rock_softmax_rows" and q8[0].kernel_count == 3
     lib = rock.load_library()
     k = rock.RockKernel((vae % "f16").replace("-g 1 ", "-g 4 "))
     assert k.workspace_bytes == 4 * 16384 * 16384 * 4 and lib.miirGetWorkspaceSize(k._h) == -1   # beyond an int

@@ -124,13 +124,43 @@ def test_attention_int8_first_gemm(rock, oracle, gpu, shape, bias):
     braw = bq = None
     if bias:
         braw, bq = quantise(rng.standard_normal((G, sq, sk)).astype(np.float32), "f16")
+    info = {}
     out = rock.attention(torch.from_numpy(Q).to(gpu), torch.from_numpy(K).to(gpu), to_gpu(rv, "f16", gpu),
-                         scale=scale, zero_point=zp, bias=to_gpu(braw, "f16", gpu) if bias else None, transK=True)
+                         scale=scale, zero_point=zp, bias=to_gpu(braw, "f16", gpu) if bias else None, transK=True,
+                         info=info)
     torch.cuda.synchronize()
+    if dqk <= 128:  # fused: the int32 score tile is dequantised in registers
+        dmax = 64 if max(dqk, dv) <= 64 else 128
+        assert info["kernels"] == ["rock_attention_i8_d%dx%d_%s" % (dmax, dmax, "fast_bias" if bias else "fast")]
+    else:
+        assert len(info["kernels"]) == 3
     shift = np.full((G, sq, sk), -zp * scale, np.float32) + (bq.reshape(G, sq, sk) if bias else 0.0)
     ref = oracle.attention(Q.astype(np.float32), K.astype(np.float32), Vq, G, sq, sk, dqk, dv, scale=scale,
                            bias_t=shift.astype(np.float32), transK=True)
     check_float(to_f32(out, "f16"), ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
+
+
+def test_attention_int8_first_gemm_fused_at_size(rock, oracle, gpu):
+    """Head dimension 128, several key tiles and query blocks, ragged in both:
+    the fused int8 kernel against the oracle, and against the three-kernel
+    form of the same problem (K stored [G, d, seq_k] takes that one)."""
+    G, sq, sk, dqk, dv = 3, 300, 333, 128, 128
+    rng = np.random.default_rng(59)
+    Q = rng.integers(-128, 128, (G, sq, dqk)).astype(np.int8)
+    K = rng.integers(-128, 128, (G, sk, dqk)).astype(np.int8)
+    rv, Vq = quantise(rng.standard_normal((G, sk, dv)).astype(np.float32), "f16")
+    zp, scale = -5, float(np.float16(2.0e-4))
+    info, info3 = {}, {}
+    q, k, v = torch.from_numpy(Q).to(gpu), torch.from_numpy(K).to(gpu), to_gpu(rv, "f16", gpu)
+    out = rock.attention(q, k, v, scale=scale, zero_point=zp, transK=True, info=info)
+    out3 = rock.attention(q, k.transpose(1, 2).contiguous(), v, scale=scale, zero_point=zp, transK=False, info=info3)
+    torch.cuda.synchronize()
+    assert info["kernels"] == ["rock_attention_i8_d128x128_fast"] and len(info3["kernels"]) == 3
+    shift = np.full((G, sq, sk), -zp * scale, np.float32)
+    ref = oracle.attention(Q.astype(np.float32), K.astype(np.float32), Vq, G, sq, sk, dqk, dv, scale=scale,
+                           bias_t=shift, transK=True)
+    check_float(to_f32(out, "f16"), ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
+    check_float(to_f32(out, "f16"), to_f32(out3, "f16"), "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
 
 
 def test_attention_rows_of_p_sum_to_one(rock, oracle, gpu):
