@@ -135,7 +135,7 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
   // bias kernel needs its registers for the bias gather and keeps the simple
   // order "scores, softmax, PV" per tile.
   constexpr bool PIPE = PLAIN;
-  static_assert(4 * Gm::TILE_B <= 65536, "every LDS read offset must fit the 16-bit immediate");
+  static_assert(D > 128 || 4 * Gm::TILE_B <= 65536, "up to D = 128 every LDS read offset fits the 16-bit immediate");
 
   // Every slot is an object of its own: the compiler makes an LDS read wait for
   // the loads into LDS still in flight unless it can tell that the two touch

@@ -370,6 +370,17 @@ __device__ __forceinline__ void wait_loads_and_lds_reads() {
 // The build (rocmlir_amd/_build.py holds the list) compiles every kernel into a
 // code object of its own from a small source that includes this file and
 // invokes one of the two macros.
+// Head dimensions above 128: one block per compute unit (its K and V slots
+// fill 128 KiB of LDS and its O accumulators half a wave's registers), simple
+// order "scores, softmax, PV" per tile, with or without the pre-softmax tensors.
+#define RK_ATTN_DL_WIDE(DTNAME, DT, D)                                                        \
+  extern "C" __global__ __launch_bounds__(rk::kAttnThreads, 1) void                           \
+      rock_attention_##DTNAME##_d##D##x##D##_fast_bias(const void *Q, const void *K,          \
+                                                       const void *V, const void *scale,      \
+                                                       const void *bias, void *O,             \
+                                                       RockAttentionParams p) {               \
+    rk::attention_body_dl<DT, D, false>(Q, K, V, scale, bias, O, p);                          \
+  }
 // int8 Q and K, f16 V / bias / O
 #define RK_ATTN_DL_I8(D, SUFFIX, PLAIN)                                                       \
   extern "C" __global__ __launch_bounds__(rk::kAttnThreads, 2) void                           \

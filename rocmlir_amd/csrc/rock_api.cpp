@@ -2371,7 +2371,10 @@ Handle *make_attention(const OptMap &o) {
                           sk * dqk < ((int64_t)1 << 31) && sk * dv * 2 < ((int64_t)1 << 31) &&
                           ((!has_bias && !has_scale_t) || sq * sk < ((int64_t)1 << 31)) &&
                           bool_or(o, "fused", true);
-    if (ty == ROCK_F32 || (qk_i8 && !i8_fused) || dqk > 128 || dv > 128)
+    // 16-bit types up to 256 on the vector kernel (head-dimension-contiguous tensors, checked below)
+    const bool wide_ok = !qk_i8 && !tQ && tK && !tV && !tO && dqk % 8 == 0 && dv % 8 == 0 && bool_or(o, "fused", true);
+    const int64_t dlimit = wide_ok ? 256 : 128;
+    if (ty == ROCK_F32 || (qk_i8 && (!i8_fused || dqk > 128 || dv > 128)) || dqk > dlimit || dv > dlimit)
       return make_attention_unfused(o, ty, G, sq, sk, dqk, dv, tQ, tK, tV, tO, has_bias, has_scale_t);
   }
 
@@ -2409,8 +2412,13 @@ Handle *make_attention(const OptMap &o) {
                     sk * p.k_js * 2 < ((int64_t)1 << 31) && sk * p.v_js * 2 < ((int64_t)1 << 31) &&
                     // the bias gather indexes one g slice with 32-bit element offsets
                     ((!has_bias && !has_scale_t) || sq * sk < ((int64_t)1 << 31));
-  int dmax = (dqk <= 64 && dv <= 64) ? 64 : 128;
-  const bool plain_ok = !p.has_bias && !has_scale_t && p.scale >= 0.0f;
+  const bool wide = dqk > 128 || dv > 128; // one kernel: vector loads, simple order per tile
+  int dmax = (dqk <= 64 && dv <= 64) ? 64 : wide ? 256 : 128;
+  const bool plain_ok = !p.has_bias && !has_scale_t && p.scale >= 0.0f && !wide;
+  if (wide && !fast) {
+    delete h;
+    return make_attention_unfused(o, ty, G, sq, sk, dqk, dv, tQ, tK, tV, tO, has_bias, has_scale_t);
+  }
   const AttnVariant *variant = !fast ? &kAttnVariants[2] : plain_ok ? &kAttnVariants[0] : &kAttnVariants[1];
   {
     // a perf_config that names a kernel this problem can run on selects it;
@@ -2419,7 +2427,9 @@ Handle *make_attention(const OptMap &o) {
     if (parse_attn_perf(str_or(o, "perf_config", ""), want_d, want_kpack, want_unroll)) {
       if ((want_d == 64 || want_d == 128) && want_d >= dmax)
         dmax = want_d;
-      if (want_kpack == 1 && !qk_i8)
+      if (wide)
+        ; // a single kernel
+      else if (want_kpack == 1 && !qk_i8)
         variant = &kAttnVariants[2];
       else if (fast && want_kpack == 8)
         variant = (want_unroll != 0 && plain_ok) ? &kAttnVariants[0] : &kAttnVariants[1];

@@ -19,7 +19,7 @@ def _store(mat, trans):
 
 
 def _run(rock, oracle, gpu, t, G, sq, sk, dqk, dv, scale, seed, tQ=False, tK=True, tV=False, tO=False,
-         bias=False, vones=False, scale_tensor=False):
+         bias=False, vones=False, scale_tensor=False, info=None):
     rng = np.random.default_rng(seed)
     Q = rng.standard_normal((G, sq, dqk)).astype(np.float32)
     K = rng.standard_normal((G, sk, dqk)).astype(np.float32)
@@ -36,7 +36,7 @@ def _run(rock, oracle, gpu, t, G, sq, sk, dqk, dv, scale, seed, tQ=False, tK=Tru
     out = rock.attention(to_gpu(rq, t, gpu), to_gpu(rk, t, gpu), to_gpu(rv, t, gpu), scale=scale,
                          bias=to_gpu(braw, t, gpu) if bias else None,
                          scale_tensor=to_gpu(sraw, t, gpu) if scale_tensor else None,
-                         transQ=tQ, transK=tK, transV=tV, transO=tO)
+                         transQ=tQ, transK=tK, transV=tV, transO=tO, info=info)
     torch.cuda.synchronize()
     ref = oracle.attention(Qq, Kq, Vq, G, sq, sk, dqk, dv, scale=scale, bias_t=bq, scale_t=sq_,
                            transQ=tQ, transK=tK, transV=tV, transO=tO)
@@ -89,17 +89,37 @@ def test_attention_with_scale_tensor(rock, oracle, gpu, shape, bias):
 @pytest.mark.parametrize("shape", [(2, 200, 333, 256, 256), (1, 130, 520, 512, 512), (3, 64, 100, 40, 72)],
                          ids=["d256", "d512", "small"])
 def test_attention_three_kernel_form(rock, oracle, gpu, t, shape):
-    """Head dimensions above 128, and every f32 problem: GEMM, row softmax, GEMM."""
+    """Head dimensions above 256, and every f32 problem: GEMM, row softmax, GEMM.
+    The 16-bit types up to head dimension 256 run on one fused kernel."""
     G, sq, sk, dqk, dv = shape
     if t != "f32" and dqk <= 128:
         pytest.skip("the fused kernel takes this one")
     gate = {"f16": GATE["f16"], "bf16": GATE["bf16"], "f32": (3e-5, 1e-4)}[t]
-    got, ref = _run(rock, oracle, gpu, t, G, sq, sk, dqk, dv, 1.0 / np.sqrt(dqk), 51)
+    info = {}
+    got, ref = _run(rock, oracle, gpu, t, G, sq, sk, dqk, dv, 1.0 / np.sqrt(dqk), 51, info=info)
+    if t != "f32" and dqk <= 256:
+        assert info["kernels"] == ["rock_attention_%s_d256x256_fast_bias" % t]
+    else:
+        assert len(info["kernels"]) == 3
     check_float(got, ref, t, rms=gate[0], max_abs=gate[1])
 
 
+@pytest.mark.parametrize("shape,bias,scale_tensor", [((2, 300, 333, 192, 256), False, False),
+                                                      ((1, 129, 64, 256, 136), True, False),
+                                                      ((2, 64, 200, 160, 160), True, True)])
+def test_attention_head_dims_up_to_256_fused(rock, oracle, gpu, shape, bias, scale_tensor):
+    """Head dimensions between 129 and 256 (ragged ones, different for QK and
+    V, with and without the pre-softmax tensors): one kernel, no score workspace."""
+    G, sq, sk, dqk, dv = shape
+    info = {}
+    got, ref = _run(rock, oracle, gpu, "f16", G, sq, sk, dqk, dv, 1.0 / np.sqrt(dqk), 61, bias=bias,
+                    scale_tensor=scale_tensor, info=info)
+    assert info["kernels"] == ["rock_attention_f16_d256x256_fast_bias"]
+    check_float(got, ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
+
+
 def test_attention_three_kernel_form_with_bias_and_scale_tensor(rock, oracle, gpu):
-    got, ref = _run(rock, oracle, gpu, "f16", 2, 100, 150, 256, 192, 0.07, 53, bias=True, scale_tensor=True)
+    got, ref = _run(rock, oracle, gpu, "f16", 2, 100, 150, 320, 192, 0.07, 53, bias=True, scale_tensor=True)
     check_float(got, ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
     got, ref = _run(rock, oracle, gpu, "f32", 2, 96, 80, 64, 64, 0.125, 55, tQ=True, tK=False, tV=True, tO=True,
                     bias=True)
