@@ -76,6 +76,9 @@ def contraction_kernels(type_code):
                             % (name, bm, bn, wm, wn, "true" if rich else "false")))
         out.append(("rock_conv_%s_64x64_generic" % t,
                     "RK_CONV(_64x64_generic, 64, 64, 2, 2, rk::LD_CONV_IN_GENERIC, rk::LD_CONV_FIL_GENERIC)"))
+        if t in ("f32", "f16", "bf16"):   # filter gradient as one K-major GEMM over the tensors as they lie
+            out.append(("rock_conv_bwd_weight_%s_128x128" % t, "RK_CONV_BWD_WEIGHT(_128x128, 128, 128, 2, 2)"))
+            out.append(("rock_conv_bwd_weight_%s_64x64" % t, "RK_CONV_BWD_WEIGHT(_64x64, 64, 64, 2, 2)"))
         out.append(("rock_conv_%s_direct224" % t, "RK_CONV_DIRECT(_direct224, false)"))
         out.append(("rock_conv_%s_direct224_e" % t, "RK_CONV_DIRECT(_direct224_e, true)"))
     return out

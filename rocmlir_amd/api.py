@@ -663,15 +663,19 @@ def conv2d_bwd_data(fil, dout, *, fil_layout, in_layout, out_layout, batchsize, 
 
 def conv2d_bwd_weight(inp, dout, *, fil_layout, in_layout, out_layout, batchsize, in_channels, out_channels, in_h,
                       in_w, fil_h, fil_w, groupsize=1, stride=(1, 1), padding=(0, 0), dilation=(1, 1), out=None,
-                      layout_conversion=True, stream=None, info=None):
+                      layout_conversion=True, stream=None, info=None, as_gemm=True):
     """Gradient of conv2d with respect to its filter (operation
-    conv_bwd_weight); returns the flat filter-shaped gradient."""
+    conv_bwd_weight); returns the flat filter-shaped gradient.  as_gemm=False
+    keeps channels-last problems off the single K-major GEMM over the tensors
+    as they lie (--bwd_weight_gemm false)."""
     import torch
     t = _dtype_name(dout.dtype)
     opts = _conv_options("conv_bwd_weight", t, fil_layout, in_layout, out_layout, batchsize, groupsize, in_channels,
                          out_channels, in_h, in_w, fil_h, fil_w, stride, padding, dilation)
     if not layout_conversion:
         opts += " --layout_conversion false"
+    if not as_gemm:
+        opts += " --bwd_weight_gemm false"
     prog = _program(opts)
     if info is not None:
         info["kernels"] = [k.kernel_name for k in prog.kernels]

@@ -303,6 +303,87 @@ template <int DT, int COLS, int NW, int RB> struct ColsDl {
   }
 };
 
+// The forward im2col matrix as a K-major operand: the reduction index is the
+// output pixel m = (n, ho, wo), a stage row holds COLS consecutive columns
+// (y, x, c) -- c fastest -- of one pixel, i.e. runs of input channels of the
+// pixel (n, ho*s + y*d - p, wo*s + x*d - p), or zeros where that lies in the
+// padding.  Which tap and channel a lane's chunk belongs to depends on the
+// column only, so it is fixed for the whole loop; the pixel walks on by KR per
+// K-step, carried through (wo, ho, n) without a division.  Same LDS placement
+// as ColsDl, so the fragments come out through the same transposing reads.
+// The reference reaches this operand through its backward-weight coordinate
+// transforms (ConvToGemm.cpp:530-768).
+template <int DT, int COLS, int NW, int RB> struct ConvColsDl {
+  using Kg = KmGeom<DT, COLS, RB>;
+  struct Sg {
+    static constexpr int SLABS = COLS * RB / 1024;
+    static constexpr int PER_WAVE = SLABS / NW;
+    static_assert(SLABS % NW == 0, "stage must split into 1 KiB slabs per wave");
+  };
+  static constexpr int ES = Kg::ES;
+  __amdgpu_buffer_rsrc_t rsrc;
+  int krow[Sg::PER_WAVE];                // k-row (pixel) of the chunk inside a stage
+  int coff[Sg::PER_WAVE];                // byte offset of the chunk's channels inside a pixel, or -1: column beyond N
+  int dy[Sg::PER_WAVE], dx[Sg::PER_WAVE]; // the tap's displacement in input rows / pixels
+  int n[Sg::PER_WAVE], ho[Sg::PER_WAVE], wo[Sg::PER_WAVE]; // the output pixel this lane loads for next
+  int s_n, s_h, s_w;                     // KR pixels as (images, rows, pixels)
+  int K, hi_, wi_, ho_, wo_, sh, sw, pix_bytes, wave;
+
+  __device__ __forceinline__ void init(const void *in, const RockConvBwdWeightParams &p, int g, int col0, int wave_,
+                                       int lane) {
+    wave = wave_;
+    K = p.K;
+    hi_ = p.hi; wi_ = p.wi; ho_ = p.ho; wo_ = p.wo;
+    sh = p.stride_h; sw = p.stride_w;
+    pix_bytes = (int)p.in_pix_stride * ES;
+    rsrc = dl_rsrc(in);
+    {
+      const int kr = Kg::KR, img = p.ho * p.wo;
+      s_n = kr / img;
+      const int rem = kr - s_n * img;
+      s_h = rem / p.wo;
+      s_w = rem - s_h * p.wo;
+    }
+#pragma unroll
+    for (int i = 0; i < Sg::PER_WAVE; ++i) {
+      const int idx = (wave * Sg::PER_WAVE + i) * 64 + lane; // physical chunk inside the stage
+      const int r = idx / Kg::CPR, pc = idx % Kg::CPR;
+      const int lc = pc ^ Kg::swz(r);                        // logical chunk this lane fetches
+      krow[i] = r;
+      const int col = col0 + lc * (kChunk / ES);             // first column of the chunk (c % 8 == 0: one tap)
+      const int tap = col / p.c, y = tap / p.x, x = tap - y * p.x;
+      coff[i] = col < p.N ? (col - tap * p.c) * ES : -1;
+      dy[i] = y * p.dil_h - p.pad_h;
+      dx[i] = x * p.dil_w - p.pad_w;
+      const int m = g * p.K + r; // batch entry g reduces the pixels [g*K, (g+1)*K)
+      const int img = p.ho * p.wo;
+      n[i] = m / img;
+      const int rem = m - n[i] * img;
+      ho[i] = rem / p.wo;
+      wo[i] = rem - ho[i] * p.wo;
+    }
+  }
+  // must be called with kt = 0, 1, 2, ... in order (the pixel state advances)
+  __device__ __forceinline__ void issue(int kt, char *stage) {
+    const int k0 = kt * Kg::KR;
+#pragma unroll
+    for (int i = 0; i < Sg::PER_WAVE; ++i) {
+      const int hi = ho[i] * sh + dy[i], wi = wo[i] * sw + dx[i];
+      const bool ok = coff[i] >= 0 && k0 + krow[i] < K && hi >= 0 && hi < hi_ && wi >= 0 && wi < wi_;
+      const unsigned voff = ok ? (unsigned)(((n[i] * hi_ + hi) * wi_ + wi) * pix_bytes + coff[i]) : kOobOffset;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrc, (lds_void_t *)(stage + (wave * Sg::PER_WAVE + i) * 1024), 16, (int)voff, 0, 0, 0);
+      wo[i] += s_w;
+      const int cw = wo[i] >= wo_ ? 1 : 0;
+      wo[i] -= cw ? wo_ : 0;
+      ho[i] += s_h + cw;
+      const int ch = ho[i] >= ho_ ? 1 : 0;
+      ho[i] -= ch ? ho_ : 0;
+      n[i] += s_n + ch;
+    }
+  }
+};
+
 typedef __attribute__((address_space(3))) v4s km_lds_v4s_t;
 typedef __attribute__((address_space(3))) v2i km_lds_v2i_t;
 
@@ -376,6 +457,14 @@ __device__ __forceinline__ auto make_dl_b(const void *B, const RockGemmParams &p
     l.init(base, p.b_ns, n0, p.N, p.K, wave, lane);
     return l;
   }
+}
+template <int DT, int ROWS, int NW, int RB, int KIND>
+__device__ __forceinline__ auto make_dl_b(const void *in, const RockConvBwdWeightParams &p, int g, int n0, int wave,
+                                          int lane) {
+  static_assert(KIND == LD_CONV_COLS, "filter gradient: the second operand is the im2col matrix");
+  ConvColsDl<DT, ROWS, NW, RB> l;
+  l.init(in, p, g, n0, wave, lane);
+  return l;
 }
 template <int DT, int ROWS, int NW, int RB, int KIND>
 __device__ __forceinline__ auto make_dl_a(const void *in, const RockConvParams &p, int g, int m0, int wave, int lane) {
@@ -849,7 +938,8 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
   // in every K-step of the loading waves.
   // (Not for the 256x256 tile of the 8-bit float types: 128 accumulators and 96
   // fragment registers leave the unrolled loop no room and it spills.)
-  constexpr bool KM = (LDA == LD_COLS_FAST || LDB == LD_COLS_FAST) && !(Tr::CHUNKS == 2 && BM * BN >= 256 * 256);
+  constexpr bool KM = (LDA == LD_COLS_FAST || LDB == LD_COLS_FAST || LDB == LD_CONV_COLS) &&
+                      !(Tr::CHUNKS == 2 && BM * BN >= 256 * 256);
   static_assert(!KM || kDlStages == 2, "K-major operands: two stages, one LDS object each");
   constexpr int WBUF = 32 * (WTN * 4 + 16); // the epilogue's staging region per wave
   static_assert(!KM || (NW / 2) * WBUF <= STAGE, "half the waves stage their stores in each stage");
@@ -925,7 +1015,7 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
     auto fetch = [&](int s, Frag<DT> *a, Frag<DT> *b) {
 #pragma unroll
       for (int j = 0; j < NI; ++j) {
-        if constexpr (LDB == LD_COLS_FAST)
+        if constexpr (LDB == LD_COLS_FAST || LDB == LD_CONV_COLS)
           b[j] = dl_read_frag_km<DT, BN, RB>(sb, wn * WTN + j * 32, s, lane);
         else
           b[j] = dl_read_frag<DT, RB>(sb, wn * WTN + j * 32 + lrow, s, lgrp);
@@ -952,7 +1042,7 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
     // Issue order for the scheduler: the first step's fragment reads, then per
     // step one LDS read of the next step's fragments after every MFMA until
     // they are all out, then the step's remaining MFMAs.
-    if constexpr (LDA != LD_COLS_FAST && LDB != LD_COLS_FAST && MI * NI >= MI + NI) {
+    if constexpr (LDA != LD_COLS_FAST && LDB != LD_COLS_FAST && LDB != LD_CONV_COLS && MI * NI >= MI + NI) {
       __builtin_amdgcn_sched_group_barrier(0x100, MI + NI, 0);
 #pragma unroll
       for (int s = 0; s + 1 < STEPS; ++s) {

@@ -61,3 +61,12 @@
       const void *fil, const void *in, void *out, const void *aux, const void *res, RockConvParams p) { \
     rk::conv_direct_body<ROCK_DT, 7, 2, RICH>(in, fil, out, aux, res, p);                             \
   }
+
+// filter gradient: A = the output gradient [k][pixel], B = the im2col matrix [(y, x, c)][pixel], both K-major
+#define RK_CONV_BWD_WEIGHT(NAME, BM, BN, WM, WN)                                                      \
+  extern "C" __global__ __launch_bounds__(WM *WN * 64) void RK_CAT(RK_CAT(rock_conv_bwd_weight_, ROCK_DTNAME), NAME)( \
+      const void *dy, const void *in, void *dw, const void *aux, const void *res,                      \
+      RockConvBwdWeightParams p) {                                                                     \
+    rk::contraction_body_dl<ROCK_DT, BM, BN, WM, WN, 128, rk::LD_COLS_FAST, rk::LD_CONV_COLS, false>(dy, in, dw, aux, \
+                                                                                                      res, p);    \
+  }

@@ -35,7 +35,8 @@ enum LoaderKind : int {
   LD_CONV_IN_FAST = 2,  // convolution input, channel-contiguous, C*ES % 16 == 0 (direct-to-LDS body)
   LD_CONV_IN_GENERIC = 3,
   LD_CONV_FIL_GENERIC = 4,
-  LD_COLS_FAST = 5      // GEMM operand stored K-major (its M or N index contiguous), 16-byte aligned chunks
+  LD_COLS_FAST = 5,     // GEMM operand stored K-major (its M or N index contiguous), 16-byte aligned chunks
+  LD_CONV_COLS = 6      // forward im2col matrix as a K-major operand (reduction over pixels): filter gradient
 };
 
 constexpr int kChunk = 16;       // bytes

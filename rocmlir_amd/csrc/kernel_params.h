@@ -91,6 +91,23 @@ struct RockConvParams {
   RockEpilogue epi;
 };
 
+// Filter gradient of a convolution as one K-major GEMM over the tensors as they
+// lie (channels-last input and output gradient, one group):
+//   dW[k, (y, x, c)] = sum over pixels m = (n, ho, wo) of dY[m, k] * X[n, ho*s + y*d - p, wo*s + x*d - p, c]
+// The GEMM part describes A = dY as [k][pixel] (K-major: a_ms = 1, a_ks = pixel
+// stride), C = the gradient (or its f32 partial sums) as [k][(y, x, c)], and
+// the batch index G = the split of the pixel range (batch entry g reduces the
+// pixels [g*K, (g+1)*K)); the second operand is the forward im2col matrix,
+// gathered by the loader from what follows (b_* are unused).
+struct RockConvBwdWeightParams : RockGemmParams {
+  int64_t in_pix_stride; // elements between neighbouring input pixels along w; rows and images follow densely
+  int32_t c;             // input channels (the columns run (y, x, c) with c fastest)
+  int32_t hi, wi, ho, wo;
+  int32_t x;             // filter width (a column's tap is (col / c) / x, (col / c) % x)
+  int32_t stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
+  int32_t pad_;
+};
+
 // Layout conversion of a 5-D tensor (the utility "converting copy" of the
 // reference's multi-kernel flows, ConvGenerator.cpp:279-344): element (i0..i4)
 // moves from src[sum i_d * src_stride[d]] to dst[sum i_d * dst_stride[d]].

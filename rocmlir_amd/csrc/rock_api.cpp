@@ -1538,6 +1538,99 @@ Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
     }
   }
 
+  // Channels-last input and output gradient, one group, a filter gradient whose
+  // (y, x, c) run is contiguous: one K-major GEMM over the tensors as they lie,
+  //   dW[k, (y, x, c)] = sum over pixels of dY[pixel, k] * im2col(X)[pixel, (y, x, c)],
+  // the second operand gathered by the kernel's loader (no copies), the pixel
+  // range cut into S batch entries whose f32 partial results the reduction
+  // kernel adds up in split order.  The reference lowers the same contraction
+  // through its backward-weight coordinate transforms with atomic adds into a
+  // zero-filled workspace (ConvToGemm.cpp:530-768).
+  if (cp.g == 1 && (cp.ti == ROCK_F32 || cp.ti == ROCK_F16 || cp.ti == ROCK_BF16) &&
+      bool_or(o, "bwd_weight_gemm", true)) {
+    auto al = [&](int64_t elems) { return (elems * es) % 16 == 0; };
+    const int64_t P = cp.n * cp.ho * cp.wo, Ng = cp.y * cp.x * cp.c;
+    const bool in_ok = cp.is[2] == 1 && cp.is[3] == cp.wi * cp.is[4] && cp.is[0] == cp.hi * cp.is[3] && al(cp.c) &&
+                       al(cp.is[4]) && cp.n * cp.hi * cp.wi * cp.is[4] * es < ((int64_t)1 << 31);
+    const bool dy_ok = cp.os[2] == 1 && cp.os[3] == cp.wo * cp.os[4] && cp.os[0] == cp.ho * cp.os[3] && al(cp.k) &&
+                       al(cp.os[4]);
+    const bool dw_ok = cp.fs[2] == 1 && cp.fs[4] == cp.c && cp.fs[3] == cp.x * cp.c && cp.fs[1] >= Ng && al(cp.fs[1]);
+    if (in_ok && dy_ok && dw_ok && P <= INT32_MAX && Ng <= INT32_MAX) {
+      const Tile &tile = cp.k <= 64 ? kFastTiles[3] : kFastTiles[2]; // 64x64 or 128x128
+      const int64_t tiles = (int64_t)ceil_div(cp.k, tile.bm) * ceil_div(Ng, tile.bn);
+      // enough batch entries to fill the chip, each a divisor's share of the pixels (at least 256 of them)
+      const int64_t want = std::max<int64_t>(1, std::min<int64_t>(tile.blocks_per_cu * kNumCU / tiles, P / 256));
+      int64_t S = 1;
+      for (int64_t d = want; d >= 1; --d)
+        if (P % d == 0) {
+          S = d;
+          break;
+        }
+      const int64_t Ks = P / S;
+      const int count = S > 1 ? 2 : 1;
+      const int64_t workspace = S > 1 ? align256(S * cp.k * Ng * 4) : 0;
+      if (Ks * cp.os[4] * es < ((int64_t)1 << 31)) {
+        if (kid < 0 || kid >= count) {
+          set_error("conv: kernel_id out of range");
+          return nullptr;
+        }
+        auto *h = new Handle;
+        if (kid == 0) {
+          RockConvBwdWeightParams bp;
+          std::memset(&bp, 0, sizeof bp);
+          bp.G = (int)S; bp.M = (int)cp.k; bp.N = (int)Ng; bp.K = (int)Ks;
+          bp.a_ms = 1; bp.a_ks = cp.os[4]; bp.a_gs = Ks * cp.os[4];
+          if (S > 1) {
+            bp.c_ms = Ng; bp.c_ns = 1; bp.c_gs = cp.k * Ng;
+            default_epilogue(bp.epi, ROCK_F32);
+          } else {
+            bp.c_ms = cp.fs[1]; bp.c_ns = 1; bp.c_gs = 0;
+            default_epilogue(bp.epi, cp.ti);
+          }
+          bp.in_pix_stride = cp.is[4];
+          bp.c = (int)cp.c; bp.hi = (int)cp.hi; bp.wi = (int)cp.wi; bp.ho = (int)cp.ho; bp.wo = (int)cp.wo;
+          bp.x = (int)cp.x;
+          bp.stride_h = (int)cp.sh; bp.stride_w = (int)cp.sw; bp.pad_h = (int)cp.ph; bp.pad_w = (int)cp.pw;
+          bp.dil_h = (int)cp.dh; bp.dil_w = (int)cp.dw;
+          apply_tile_grid(tile, cp.k, Ng, (int)S, bp.tiles_m, bp.tiles_n, bp.group_m, bp.xcd_remap, h->block_size,
+                          h->grid_size);
+          h->op = OP_GEMM;
+          h->params.assign(sizeof bp, 0);
+          std::memcpy(h->params.data(), &bp, sizeof bp);
+          h->epi = &reinterpret_cast<RockConvBwdWeightParams *>(h->params.data())->epi;
+          h->kernel_name = std::string("rock_conv_bwd_weight_") + dtype_name(cp.ti) + (tile.bm == 64 ? "_64x64" : "_128x128");
+          h->num_pointers = 5;
+          h->perf_config = perf_string(tile, es, &o);
+          h->ptr_map = {{2, 0}, {1, 0}, S > 1 ? Handle::PtrSrc{4, 0} : Handle::PtrSrc{0, 0}, {-1, 0}, {-1, 0}};
+          h->problem_key = conv_problem_key(h, o, cp, 4);
+        } else {
+          RockReduceParams r;
+          std::memset(&r, 0, sizeof r);
+          r.split_stride = cp.k * Ng;
+          r.size[0] = 1; r.size[1] = 1; r.size[2] = (int)cp.k; r.size[3] = (int)Ng;
+          r.dst_stride[2] = cp.fs[1]; r.dst_stride[3] = 1;
+          r.splits = (int)S;
+          r.out_dtype = cp.ti;
+          h->op = OP_RELAYOUT;
+          h->epi = nullptr;
+          h->params.assign(sizeof r, 0);
+          std::memcpy(h->params.data(), &r, sizeof r);
+          h->kernel_name = "rock_reduce_splits";
+          h->block_size = 256;
+          h->grid_size = (uint32_t)((cp.k * Ng + 255) / 256);
+          h->num_pointers = 2;
+          h->perf_config = "";
+          h->ptr_map = {{4, 0}, {0, 0}};
+          h->problem_key = "reduction of the split partial sums";
+        }
+        h->kernel_count = count;
+        h->workspace_bytes = (size_t)workspace;
+        h->caller_pointers = workspace ? 5 : 4;
+        return h;
+      }
+    }
+  }
+
   // split of the reduction over n (one group only: the splits take the group index)
   int64_t S = 1;
   if (cp.g == 1) {

@@ -70,7 +70,9 @@ def test_miir_protocol_conv(rock):
     "-head_dim_v 128 -transK true",
     "-operation attention -arch gfx950 -t bf16 -g 2 -seq_len_q 64 -seq_len_k 64 -head_dim_qk 64 -head_dim_v 64",
     CONV_RESNET.replace("NHWGC", "NGCHW").replace("GNYXC", "GNCHW"),                    # relayout kernel first
-    CONV_RESNET.replace("--operation conv", "--operation conv_bwd_weight") + " --kernel_id 2",
+    CONV_RESNET.replace("--operation conv", "--operation conv_bwd_weight"),               # filter gradient as one GEMM
+    CONV_RESNET.replace("--operation conv", "--operation conv_bwd_weight") + " --kernel_id 1",
+    CONV_RESNET.replace("--operation conv", "--operation conv_bwd_weight") + " --bwd_weight_gemm false --kernel_id 2",
 ])
 def test_every_handle_gets_its_kernel_alone(rock, options):
     """miirBufferGet: a gfx950 ELF whose only kernel is the one the handle names, at most 512 KiB."""
@@ -358,12 +360,24 @@ def test_backward_convolution_plans(rock):
     k = rock.RockKernel(s2 + " --layout_conversion false")
     assert (k.kernel_count, k.workspace_bytes, k.caller_pointers) == (4, 0, 4)
     assert k.kernel_name == "rock_conv_f16_64x64_generic"
+    # channels-last, one group: one K-major GEMM over the tensors as they lie (the second operand is the
+    # im2col matrix, gathered by the kernel) into f32 partial sums per pixel split, and their reduction
     bwd_w = CONV_RESNET.replace("--operation conv", "--operation conv_bwd_weight")
-    names = [rock.RockKernel(bwd_w + " --kernel_id %d" % i).kernel_name for i in range(4)]
+    ks = [rock.RockKernel(bwd_w + " --kernel_id %d" % i) for i in range(2)]
+    assert [k.kernel_name for k in ks] == ["rock_conv_bwd_weight_f16_128x128", "rock_reduce_splits"]
+    splits = ks[0].grid_size // 9                      # 128 x 1152 gradient: nine 128 x 128 tiles per split
+    assert ks[0].grid_size == 9 * splits and (256 * 28 * 28) % splits == 0 and splits >= 32
+    assert all(k.kernel_count == 2 and k.caller_pointers == 5 and k.workspace_bytes == splits * 128 * 1152 * 4
+               for k in ks)
+    assert "convfp16 -F 4 " in ks[0].problem_key
+    # the plan it replaces, still there for the other layouts: two copies, a forward kernel, the reduction
+    old = bwd_w + " --bwd_weight_gemm false"
+    names = [rock.RockKernel(old + " --kernel_id %d" % i).kernel_name for i in range(4)]
     assert names[:2] == ["rock_relayout_b2", "rock_relayout_b2"] and names[3] == "rock_reduce_splits"
     assert names[2].startswith("rock_conv_f16_") and names[2].endswith("_fast")
-    assert "convfp16 -F 4 " in rock.RockKernel(bwd_w + " --kernel_id 2").problem_key
-    k = rock.RockKernel(bwd_w + " --layout_conversion false")
+    assert "convfp16 -F 4 " in rock.RockKernel(old + " --kernel_id 2").problem_key
+    assert rock.RockKernel(bwd_w.replace("GNYXC", "GNCHW")).kernel_name == "rock_relayout_b2"
+    k = rock.RockKernel(old + " --layout_conversion false")
     assert (k.kernel_count, k.workspace_bytes, k.kernel_name) == (1, 0, "rock_conv_f16_64x64_generic")
 
 

@@ -139,8 +139,41 @@ def test_conv_bwd_weight_exact(rock, oracle, gpu, case, layouts, t, convert):
     elif (y, x, c % 64, hi % 16) == (1, 1, 0, 0) and layouts in (NHWC, NCHW) and convert:
         # strided pointwise: the pixels read are gathered first, then the same GEMM
         assert info["kernels"][0].startswith("rock_relayout") and info["kernels"][1].startswith("rock_gemm_")
+    elif info["kernels"][0].startswith("rock_conv_bwd_weight_"):
+        # channels-last, one group: one K-major GEMM whose second operand is the im2col matrix, no copies
+        assert layouts == NHWC and g == 1 and info["kernels"][1:] in ([], ["rock_reduce_splits"])
     elif not convert and not info["kernels"][0].startswith("rock_gemm_"):
         assert len(info["kernels"]) == 1
+
+
+BWD_WEIGHT_GEMM_CASES = [
+    (16, 1, 128, 128, 28, 28, 3, 3, (1, 1), (1, 1), (1, 1)),   # the ResNet 3x3 layer: 9 column tiles, split pixels
+    (4, 1, 64, 64, 14, 14, 3, 3, (1, 1), (1, 1), (1, 1)),      # 64x64 tiles
+    (3, 1, 40, 72, 9, 11, 3, 2, (1, 1), (1, 0), (1, 1)),       # ragged rows and columns, taps straddle column tiles
+    (2, 1, 16, 136, 13, 10, 5, 5, (2, 1), (2, 2), (1, 2)),     # stride, dilation, 5x5
+    (5, 1, 8, 24, 7, 7, 7, 7, (1, 1), (3, 3), (1, 1)),         # filter as large as the image
+    (1, 1, 256, 8, 6, 6, 1, 1, (1, 1), (0, 0), (1, 1)),        # 36 pixels: no split, gradient written directly
+]
+
+
+@pytest.mark.parametrize("case", BWD_WEIGHT_GEMM_CASES)
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16"])
+def test_conv_bwd_weight_as_one_gemm_exact(rock, oracle, gpu, case, t):
+    """The filter gradient of a channels-last problem as one K-major GEMM over
+    the tensors as they lie, against the oracle and against the plan it replaces."""
+    n, g, c, k, hi, wi, y, x, stride, pad, dil = case
+    _, (raw_i, iq), (raw_dy, dyq), ho, wo = _tensors(case, NHWC, t, 79)
+    info, info_old = {}, {}
+    xi, dy = to_gpu(raw_i, t, gpu), to_gpu(raw_dy, t, gpu)
+    got = rock.conv2d_bwd_weight(xi, dy, info=info, **_kw(case, NHWC))
+    old = rock.conv2d_bwd_weight(xi, dy, info=info_old, as_gemm=False, **_kw(case, NHWC))
+    torch.cuda.synchronize()
+    if (y, x) != (1, 1):
+        assert info["kernels"][0] == "rock_conv_bwd_weight_%s_%s" % (t, "64x64" if k <= 64 else "128x128")
+        assert not any(name.startswith("rock_conv_bwd_weight_") for name in info_old["kernels"])
+    ref, _, _ = oracle.conv_bwd_weight(iq, dyq, *NHWC, n, g, c, k, hi, wi, y, x, stride, pad, dil)
+    assert np.array_equal(to_f32(got, t), oracle.round_through(ref, CODE[t]))
+    assert torch.equal(got.view(torch.uint8), old.view(torch.uint8))
 
 
 @pytest.mark.parametrize("t", ["f16", "f32"])
@@ -156,6 +189,6 @@ def test_conv_backward_resnet_block_real_values(rock, oracle, gpu, t):
     ref, _, _ = oracle.conv_bwd_data(fq, dyq, *NHWC, n, g, c, k, hi, wi, y, x, stride, pad, dil)
     check_float(to_f32(dx, t), ref, t)
     dw = rock.conv2d_bwd_weight(to_gpu(raw_i, t, gpu), to_gpu(raw_dy, t, gpu), info=info, **_kw(case, NHWC))
-    assert info["kernels"][-1] == "rock_reduce_splits" and info["kernels"][-2].endswith("_fast")
+    assert info["kernels"] == ["rock_conv_bwd_weight_%s_128x128" % t, "rock_reduce_splits"]
     ref, _, _ = oracle.conv_bwd_weight(iq, dyq, *NHWC, n, g, c, k, hi, wi, y, x, stride, pad, dil)
     check_float(to_f32(dw, t), ref, t)
