@@ -1307,6 +1307,72 @@ Handle *make_conv_bwd_data(const OptMap &o, const ConvProblem &cp) {
 // groups of that convolution into f32 partial sums, added up in split order by
 // a reduction kernel (the reference's answer is atomic adds into a zero-filled
 // f32 workspace, ConvGenerator.cpp:434-480).
+// Tensors that are not channels-last are copied into that form in the
+// workspace and the filter gradient is planned again over the copies (all
+// pixels of all images then form one equally spaced run).  nullptr with no
+// error set when the copies would not help (channel runs not in whole 16-byte
+// chunks, or conversions switched off).
+Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp);
+Handle *bwd_weight_over_channels_last_copies(const OptMap &o, const ConvProblem &cp, bool &applies) {
+  const int es = dtype_size(cp.ti);
+  const int kid = (int)int_or(o, "kernel_id", 0);
+  const bool cl_in = cp.is[2] == 1, cl_out = cp.os[2] == 1;
+  applies = (!cl_in || !cl_out) && (cp.c * es) % 16 == 0 && (cp.k * es) % 16 == 0 && bool_or(o, "layout_conversion", true);
+  if (!applies)
+    return nullptr;
+  ConvProblem inner = cp;
+  const int64_t isz[5] = {cp.n, cp.g, cp.c, cp.hi, cp.wi}, osz[5] = {cp.n, cp.g, cp.k, cp.ho, cp.wo};
+  if (!cl_in) {
+    inner.il = "nhwgc";
+    layout_strides(inner.il, "ngchw", isz, inner.is);
+  }
+  if (!cl_out) {
+    inner.ol = "nhwgk";
+    layout_strides(inner.ol, "ngkhw", osz, inner.os);
+  }
+  const int64_t x_bytes = cl_in ? 0 : align256(cp.n * cp.c * cp.hi * cp.wi * es);
+  const int64_t y_bytes = cl_out ? 0 : align256(cp.n * cp.k * cp.ho * cp.wo * es);
+  const int pre = (cl_in ? 0 : 1) + (cl_out ? 0 : 1);
+  OptMap o2 = o;
+  o2["kernel_id"] = std::to_string(std::max(0, kid - pre));
+  Handle *sub = make_conv_bwd_weight(o2, inner);
+  if (!sub)
+    return nullptr;
+  const int total = sub->kernel_count + pre;
+  const size_t ws_total = (size_t)(x_bytes + y_bytes) + sub->workspace_bytes;
+  if (kid < pre) {
+    delete sub;
+    const bool input = kid == 0 && !cl_in;
+    auto *c2 = new Handle;
+    const int64_t size_x[5] = {cp.n, cp.hi, cp.wi, cp.g, cp.c}, size_y[5] = {cp.n, cp.ho, cp.wo, cp.g, cp.k};
+    const int64_t str_x[5] = {cp.is[0], cp.is[3], cp.is[4], cp.is[1], cp.is[2]};
+    const int64_t str_y[5] = {cp.os[0], cp.os[3], cp.os[4], cp.os[1], cp.os[2]};
+    if (!fill_relayout_handle(c2, input ? size_x : size_y, input ? size_x : size_y, input ? str_x : str_y, es)) {
+      delete c2;
+      return nullptr;
+    }
+    c2->ptr_map = input ? std::vector<Handle::PtrSrc>{{1, 0}, {4, 0}}
+                        : std::vector<Handle::PtrSrc>{{2, 0}, {4, x_bytes}};
+    c2->problem_key = input ? "relayout input " + cp.il : "relayout output gradient " + cp.ol;
+    sub = c2;
+  } else {
+    for (auto &src : sub->ptr_map) {
+      if (src.source == 4)
+        src.offset += x_bytes + y_bytes;
+      else if (src.source == 1 && !cl_in)
+        src = Handle::PtrSrc{4, src.offset};
+      else if (src.source == 2 && !cl_out)
+        src = Handle::PtrSrc{4, x_bytes + src.offset};
+    }
+    if (sub->op != OP_RELAYOUT)
+      sub->problem_key = conv_problem_key(sub, o, cp, 4);
+  }
+  sub->kernel_count = total;
+  sub->workspace_bytes = ws_total;
+  sub->caller_pointers = 5;
+  return sub;
+}
+
 Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
   // A strided 1x1 filter without padding touches one input pixel in
   // stride_h * stride_w.  A first kernel gathers those into the workspace
@@ -1480,60 +1546,11 @@ Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
       // while the channel runs are: the tensors that are not channels-last are
       // copied into that form in the workspace and the problem is planned
       // again over the copies (all pixels of all images then form one run).
-      const bool cl_in = cp.is[2] == 1, cl_out = cp.os[2] == 1;
-      if ((!cl_in || !cl_out) && (cp.c * es) % 16 == 0 && (cp.k * es) % 16 == 0 &&
-          bool_or(o, "layout_conversion", true)) {
-        ConvProblem inner = cp;
-        const int64_t isz[5] = {cp.n, cp.g, cp.c, cp.hi, cp.wi}, osz[5] = {cp.n, cp.g, cp.k, cp.ho, cp.wo};
-        if (!cl_in) {
-          inner.il = "nhwgc";
-          layout_strides(inner.il, "ngchw", isz, inner.is);
-        }
-        if (!cl_out) {
-          inner.ol = "nhwgk";
-          layout_strides(inner.ol, "ngkhw", osz, inner.os);
-        }
-        const int64_t x_bytes = cl_in ? 0 : align256(cp.n * cp.c * cp.hi * cp.wi * es);
-        const int64_t y_bytes = cl_out ? 0 : align256(cp.n * cp.k * cp.ho * cp.wo * es);
-        const int pre = (cl_in ? 0 : 1) + (cl_out ? 0 : 1);
-        OptMap o2 = o;
-        o2["kernel_id"] = std::to_string(std::max(0, kid - pre));
-        Handle *sub = make_conv_bwd_weight(o2, inner);
-        if (!sub)
-          return nullptr;
-        const int total = sub->kernel_count + pre;
-        const size_t ws_total = (size_t)(x_bytes + y_bytes) + sub->workspace_bytes;
-        if (kid < pre) {
-          delete sub;
-          const bool input = kid == 0 && !cl_in;
-          auto *c2 = new Handle;
-          const int64_t size_x[5] = {cp.n, cp.hi, cp.wi, cp.g, cp.c}, size_y[5] = {cp.n, cp.ho, cp.wo, cp.g, cp.k};
-          const int64_t str_x[5] = {cp.is[0], cp.is[3], cp.is[4], cp.is[1], cp.is[2]};
-          const int64_t str_y[5] = {cp.os[0], cp.os[3], cp.os[4], cp.os[1], cp.os[2]};
-          if (!fill_relayout_handle(c2, input ? size_x : size_y, input ? size_x : size_y, input ? str_x : str_y, es)) {
-            delete c2;
-            return nullptr;
-          }
-          c2->ptr_map = input ? std::vector<Handle::PtrSrc>{{1, 0}, {4, 0}}
-                              : std::vector<Handle::PtrSrc>{{2, 0}, {4, x_bytes}};
-          c2->problem_key = input ? "relayout input " + cp.il : "relayout output gradient " + cp.ol;
-          sub = c2;
-        } else {
-          for (auto &src : sub->ptr_map) {
-            if (src.source == 4)
-              src.offset += x_bytes + y_bytes;
-            else if (src.source == 1 && !cl_in)
-              src = Handle::PtrSrc{4, src.offset};
-            else if (src.source == 2 && !cl_out)
-              src = Handle::PtrSrc{4, x_bytes + src.offset};
-          }
-          if (sub->op != OP_RELAYOUT)
-            sub->problem_key = conv_problem_key(sub, o, cp, 4);
-        }
-        sub->kernel_count = total;
-        sub->workspace_bytes = ws_total;
-        sub->caller_pointers = 5;
-        return sub;
+      {
+        bool applies = false;
+        Handle *via = bwd_weight_over_channels_last_copies(o, cp, applies);
+        if (applies)
+          return via;
       }
     }
   }
@@ -1554,8 +1571,17 @@ Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
                        al(cp.is[4]) && cp.n * cp.hi * cp.wi * cp.is[4] * es < ((int64_t)1 << 31);
     const bool dy_ok = cp.os[2] == 1 && cp.os[3] == cp.wo * cp.os[4] && cp.os[0] == cp.ho * cp.os[3] && al(cp.k) &&
                        al(cp.os[4]);
-    const bool dw_ok = cp.fs[2] == 1 && cp.fs[4] == cp.c && cp.fs[3] == cp.x * cp.c && cp.fs[1] >= Ng && al(cp.fs[1]);
-    if (in_ok && dy_ok && dw_ok && P <= INT32_MAX && Ng <= INT32_MAX) {
+    // a gradient whose (y, x, c) run is contiguous can be written by the GEMM itself when the pixels are
+    // not split; any other layout is produced by the reduction kernel from the [k][y][x][c] partial sums
+    const bool dw_direct = cp.fs[2] == 1 && cp.fs[4] == cp.c && cp.fs[3] == cp.x * cp.c && cp.fs[1] >= Ng && al(cp.fs[1]);
+    if (!(in_ok && dy_ok) && cp.y * cp.x > 1 && P <= INT32_MAX && Ng <= INT32_MAX) {
+      // not channels-last: copies in that form first (the 1 x 1 case has its own plans below)
+      bool applies = false;
+      Handle *via = bwd_weight_over_channels_last_copies(o, cp, applies);
+      if (applies)
+        return via;
+    }
+    if (in_ok && dy_ok && P <= INT32_MAX && Ng <= INT32_MAX) {
       const Tile &tile = cp.k <= 64 ? kFastTiles[3] : kFastTiles[2]; // 64x64 or 128x128
       const int64_t tiles = (int64_t)ceil_div(cp.k, tile.bm) * ceil_div(Ng, tile.bn);
       // enough batch entries to fill the chip, each a divisor's share of the pixels (at least 256 of them)
@@ -1567,8 +1593,9 @@ Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
           break;
         }
       const int64_t Ks = P / S;
-      const int count = S > 1 ? 2 : 1;
-      const int64_t workspace = S > 1 ? align256(S * cp.k * Ng * 4) : 0;
+      const bool reduce = S > 1 || !dw_direct;
+      const int count = reduce ? 2 : 1;
+      const int64_t workspace = reduce ? align256(S * cp.k * Ng * 4) : 0;
       if (Ks * cp.os[4] * es < ((int64_t)1 << 31)) {
         if (kid < 0 || kid >= count) {
           set_error("conv: kernel_id out of range");
@@ -1580,7 +1607,7 @@ Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
           std::memset(&bp, 0, sizeof bp);
           bp.G = (int)S; bp.M = (int)cp.k; bp.N = (int)Ng; bp.K = (int)Ks;
           bp.a_ms = 1; bp.a_ks = cp.os[4]; bp.a_gs = Ks * cp.os[4];
-          if (S > 1) {
+          if (reduce) {
             bp.c_ms = Ng; bp.c_ns = 1; bp.c_gs = cp.k * Ng;
             default_epilogue(bp.epi, ROCK_F32);
           } else {
@@ -1601,14 +1628,14 @@ Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
           h->kernel_name = std::string("rock_conv_bwd_weight_") + dtype_name(cp.ti) + (tile.bm == 64 ? "_64x64" : "_128x128");
           h->num_pointers = 5;
           h->perf_config = perf_string(tile, es, &o);
-          h->ptr_map = {{2, 0}, {1, 0}, S > 1 ? Handle::PtrSrc{4, 0} : Handle::PtrSrc{0, 0}, {-1, 0}, {-1, 0}};
+          h->ptr_map = {{2, 0}, {1, 0}, reduce ? Handle::PtrSrc{4, 0} : Handle::PtrSrc{0, 0}, {-1, 0}, {-1, 0}};
           h->problem_key = conv_problem_key(h, o, cp, 4);
         } else {
           RockReduceParams r;
           std::memset(&r, 0, sizeof r);
           r.split_stride = cp.k * Ng;
-          r.size[0] = 1; r.size[1] = 1; r.size[2] = (int)cp.k; r.size[3] = (int)Ng;
-          r.dst_stride[2] = cp.fs[1]; r.dst_stride[3] = 1;
+          r.size[0] = (int)cp.k; r.size[1] = (int)cp.y; r.size[2] = (int)cp.x; r.size[3] = (int)cp.c;
+          r.dst_stride[0] = cp.fs[1]; r.dst_stride[1] = cp.fs[3]; r.dst_stride[2] = cp.fs[4]; r.dst_stride[3] = cp.fs[2];
           r.splits = (int)S;
           r.out_dtype = cp.ti;
           h->op = OP_RELAYOUT;

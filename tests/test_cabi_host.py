@@ -376,7 +376,14 @@ def test_backward_convolution_plans(rock):
     assert names[:2] == ["rock_relayout_b2", "rock_relayout_b2"] and names[3] == "rock_reduce_splits"
     assert names[2].startswith("rock_conv_f16_") and names[2].endswith("_fast")
     assert "convfp16 -F 4 " in rock.RockKernel(old + " --kernel_id 2").problem_key
-    assert rock.RockKernel(bwd_w.replace("GNYXC", "GNCHW")).kernel_name == "rock_relayout_b2"
+    # any other gradient layout comes out of the reduction kernel; tensors that are not channels-last are
+    # first copied into that form
+    kcyx = bwd_w.replace("GNYXC", "GNCHW")
+    assert [rock.RockKernel(kcyx + " --kernel_id %d" % i).kernel_name for i in range(2)] == \
+        ["rock_conv_bwd_weight_f16_128x128", "rock_reduce_splits"]
+    nchw = kcyx.replace("NHWGC", "NGCHW")
+    assert [rock.RockKernel(nchw + " --kernel_id %d" % i).kernel_name for i in range(4)] == \
+        ["rock_relayout_b2", "rock_relayout_b2", "rock_conv_bwd_weight_f16_128x128", "rock_reduce_splits"]
     k = rock.RockKernel(old + " --layout_conversion false")
     assert (k.kernel_count, k.workspace_bytes, k.kernel_name) == (1, 0, "rock_conv_f16_64x64_generic")
 
