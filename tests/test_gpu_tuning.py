@@ -64,3 +64,39 @@ def test_tuner_conv_includes_the_window_resident_kernel(rock, oracle, gpu):
         kern.launch(F, I, out, None)
         torch.cuda.synchronize()
         assert np.array_equal(to_f32(out, "f16"), ref), name
+
+
+def test_tuner_attention_candidates_agree_and_best_applied(rock, oracle, gpu):
+    """The attention tuning space (attn:v1 strings: head-dimension tile 64 / 128,
+    plain / bias-capable / element-wise kernel): every candidate passes the
+    attention gate against the oracle, the fastest is left applied and goes
+    into the table under the problem's key."""
+    from rocmlir_amd import tuning
+    from tests.gpu_util import check_float
+    G, sq, sk, d = 4, 200, 333, 64
+    rng = np.random.default_rng(55)
+    rq, Qq = quantise(rng.standard_normal((G, sq, d)).astype(np.float32), "f16")
+    rk, Kq = quantise(rng.standard_normal((G, sk, d)).astype(np.float32), "f16")
+    rv, Vq = quantise(rng.standard_normal((G, sk, d)).astype(np.float32), "f16")
+    scale = d ** -0.5
+    ref = oracle.attention(Qq, Kq, Vq, G, sq, sk, d, d, scale=scale, transK=True)
+    Q, K, V = to_gpu(rq, "f16", gpu), to_gpu(rk, "f16", gpu), to_gpu(rv, "f16", gpu)
+    out = torch.zeros(G * sq * d, dtype=torch.float16, device=gpu)
+    kern = rock.RockKernel("-operation attention -arch gfx950 -t f16 -g %d -seq_len_q %d -seq_len_k %d -head_dim_qk %d "
+                           "-head_dim_v %d -transK true -scale %.9g" % (G, sq, sk, d, d, scale))
+    space = kern.tuning_space()
+    assert len(space) >= 3 and all(p.startswith("attn:v1:") for p in space)
+    names = set()
+    for perf in space:
+        kern.set_perf_config(perf)
+        names.add(kern.kernel_name)
+        out.zero_()
+        kern.launch(Q, K, V, None, out)
+        torch.cuda.synchronize()
+        check_float(to_f32(out, "f16"), ref, "f16", rms=1e-3, max_abs=0.02)
+    assert len(names) == len(space) and {"rock_attention_f16_d64x64_fast", "rock_attention_f16_d128x128_fast"} <= names
+    table = tuning.TuningTable()
+    results = tuning.tune(kern, Q, K, V, None, out, table=table, warmup=3, iters=10)
+    assert kern.perf_config == results[0][0] and kern.kernel_name == results[0][1]
+    fresh = rock.RockKernel(kern.options)
+    assert table.apply(fresh) and fresh.kernel_name == results[0][1]
