@@ -735,10 +735,14 @@ Handle *make_gemm(const OptMap &o) {
     const int64_t tiles64 = (int64_t)ceil_div(M, 64) * ceil_div(N, 64);
     // ... unless that kernel's 32x32 tiles already occupy half the chip by themselves
     const bool wave_split = h->kernel_name.find(kSplitKTile.suffix) != std::string::npos;
-    const bool wave_split_fills = wave_split && (int64_t)ceil_div(M, 32) * ceil_div(N, 32) * 2 > kNumCU;
+    // (measured: with K = 1024 the second kernel costs more than the split gives back; from K = 2048 on the
+    // split over blocks wins even against the wave-split kernel with all its tiles resident -- M 640, N 768,
+    // K 8192 f16: 21 us against 36 (NT, wave split) and 58 (NN, one block per tile))
+    const bool long_k = K >= 2048;
+    const bool wave_split_fills = wave_split && !long_k && (int64_t)ceil_div(M, 32) * ceil_div(N, 32) * 2 > kNumCU;
     int64_t S = 1;
-    if (G == 1 && is_float_in(ta) && is_float_in(tb) && identity && tiled && !wave_split_fills && tiles64 * 4 <= kNumCU &&
-        forced_tile(o).empty() && bool_or(o, "split_k", true)) {
+    if (G == 1 && is_float_in(ta) && is_float_in(tb) && identity && tiled && !wave_split_fills &&
+        tiles64 * (long_k ? 2 : 4) <= kNumCU && forced_tile(o).empty() && bool_or(o, "split_k", true)) {
       const int64_t want = std::min<int64_t>(2 * kNumCU / tiles64, K / 512);
       for (int64_t d = want; d >= 2; --d)
         if (K % d == 0 && ((K / d) * es) % 64 == 0) {
