@@ -72,22 +72,33 @@ typedef void *MiirHandle;
  * head_dim_qk, head_dim_v, transQ, transK, transV, transO, with-attn-bias,
  * with-attn-scale (pointer order Q, K, V, [scale tensor], bias slot, O);
  * attention types f16, bf16, f32, and i8 = int8 Q and K with f16 V / O, the
- * scores dequantised as (acc - zero_point) * scale.  Head dimensions above
- * 128, f32 and i8 run as three kernels over a score workspace.
+ * scores dequantised as (acc - zero_point) * scale.  One fused kernel covers
+ * the 16-bit types up to head dimension 256 and i8 up to 128 (beyond 128, and
+ * for i8, over tensors contiguous along the head dimension: transK, no other
+ * transpose); f32, larger head dimensions and "-fused false" run as three
+ * kernels over a score workspace.
  * Epilogue keys (all optional): scale, zero_point, quant_scale,
  * out_zero_point, bias, relu; and the element-wise operations MIGraphX fuses
  * behind a contraction (MIGraphXToTosa.cpp:1009-1016, 1089-1100, 1283-1295):
  * activation {relu|clip|sigmoid|tanh|erf|gelu|exp} with clip_min / clip_max
  * for clip, residual {add|mul} for a second tensor of the output's type and
  * layout.  Order: scale and zero point, bias, residual, activation,
- * narrowing.  Convolution-only switches: layout_conversion {true|false},
- * pointwise_as_gemm {true|false}.  A single leading dash and "key=value" are
- * accepted as well.  Returns NULL on any parse, validation or support
+ * narrowing.  Plan switches, all {true|false}, default true:
+ * layout_conversion (conversion kernels in front of the vector contraction
+ * kernel instead of the element-wise kernel), pointwise_as_gemm (1x1
+ * convolutions as a batched GEMM over the tensors as they lie),
+ * bwd_weight_gemm (the filter gradient of a one-group convolution as one
+ * K-major GEMM plus the reduction of its pixel splits), split_k (a GEMM with
+ * few output tiles and a long reduction split over blocks, partial sums in the
+ * workspace), fused (attention, above).  A single leading dash and "key=value"
+ * are accepted as well.  Returns NULL on any parse, validation or support
  * failure, as the reference does. */
 ROCMLIR_AMD_API MiirHandle miirCreateHandle(const char *options);
 
-/* Miir.h:56 -- number of kernels the operation needs (1, or up to 3 for a
- * convolution run through the layout-conversion plan, see
+/* Miir.h:56 -- number of kernels the operation needs (1 for most problems; 2
+ * for a GEMM or filter gradient split along its reduction; up to 3 for a
+ * forward convolution behind layout conversions and for attention run
+ * unfused; more for the backward and 3-D convolution plans, see
  * rockamdGetPointerMap); -1 for a NULL handle. */
 ROCMLIR_AMD_API int miirGetKernelCount(MiirHandle handle);
 
