@@ -63,10 +63,10 @@ typedef void *MiirHandle;
  * out_layout, batchsize, groupsize, in_channels, out_channels, in_h, in_w,
  * out_h, out_w, fil_h, fil_w, dilation_{h,w}, conv_stride_{h,w},
  * padding_{h,w}.  With in_d / fil_d (and out_d, dilation_d, conv_stride_d,
- * padding_d; rocmlir-gen.cpp:171-294) the forward convolution runs over three
- * spatial dimensions and the layouts have six letters (ngc012 / gkc012 /
- * ngk012, h w d and y x z accepted for 0 1 2): several kernels over a
- * workspace, same pointer order.  `--operation gemm` and `--operation attention` take the
+ * padding_d; rocmlir-gen.cpp:171-294) the convolution, forward or either
+ * gradient, runs over three spatial dimensions and the layouts have six
+ * letters (ngc012 / gkc012 / ngk012, h w d and y x z accepted for 0 1 2):
+ * several kernels over a workspace, same pointer order.  `--operation gemm` and `--operation attention` take the
  * reference's rocmlir-gen flag names (rocmlir-gen.cpp:90-561): t,
  * out_datatype, g, m, k, n, transA, transB, transC; g, seq_len_q, seq_len_k,
  * head_dim_qk, head_dim_v, transQ, transK, transV, transO, with-attn-bias,

@@ -266,6 +266,63 @@ def conv3d(fil, inp, fil_layout, in_layout, out_layout, n, g, c, k, in_size, fil
     return flat, outs
 
 
+def _conv3d_canon(flat, layout, letters, sizes):
+    shape = [sizes[letters.index(ch)] for ch in layout]
+    arr = np.asarray(flat, np.float64).reshape(shape)
+    return arr.transpose([layout.index(ch) for ch in letters])
+
+
+def _conv3d_windows(in_size, fil_size, outs, stride, pad, dil):
+    """For every filter tap the slices of the padded input its products touch
+    (one input position per output position)."""
+    for t0 in range(fil_size[0]):
+        for t1 in range(fil_size[1]):
+            for t2 in range(fil_size[2]):
+                yield (t0, t1, t2), tuple(
+                    slice(t * dil[a], t * dil[a] + (outs[a] - 1) * stride[a] + 1, stride[a])
+                    for a, t in enumerate((t0, t1, t2)))
+
+
+def conv3d_bwd_data(fil, dout, fil_layout, in_layout, out_layout, n, g, c, k, in_size, fil_size,
+                    stride=(1, 1, 1), pad=(0, 0, 0), dil=(1, 1, 1)):
+    """Input gradient of the 3-D convolution: the reference's CPU validator
+    is one loop nest for every direction and any number of spatial dimensions
+    (createCPUConvWithMLIR, rocmlir-gen.cpp:1715-1997); for this direction the
+    result tensor is the input (:1731-1733), the output position follows from
+    out_tmp = in + pad - t*dilation, out = out_tmp / stride where that divides
+    (:1895-1904) and in[n,g,c,i] += fil[g,k,c,t] * out[n,g,k,o] (:1938-1945,
+    1951-1966).  numpy, one slice update
+    per filter tap, sums in f64.  Returns the flat input-shaped gradient."""
+    outs = tuple(conv_out_dim(in_size[a], fil_size[a], pad[a], pad[a], stride[a], dil[a]) for a in range(3))
+    f = _conv3d_canon(fil, fil_layout, "gkc012", (g, k, c) + tuple(fil_size))
+    dy = _conv3d_canon(dout, out_layout, "ngk012", (n, g, k) + outs)
+    dxp = np.zeros((n, g, c) + tuple(in_size[a] + 2 * pad[a] for a in range(3)))
+    for (t0, t1, t2), win in _conv3d_windows(in_size, fil_size, outs, stride, pad, dil):
+        dxp[(slice(None),) * 3 + win] += np.einsum("ngkabd,gkc->ngcabd", dy, f[:, :, :, t0, t1, t2])
+    dx = dxp[:, :, :, pad[0]:pad[0] + in_size[0], pad[1]:pad[1] + in_size[1], pad[2]:pad[2] + in_size[2]]
+    return dx.transpose(["ngc012".index(ch) for ch in in_layout]).astype(np.float32).ravel()
+
+
+def conv3d_bwd_weight(inp, dout, fil_layout, in_layout, out_layout, n, g, c, k, in_size, fil_size,
+                      stride=(1, 1, 1), pad=(0, 0, 0), dil=(1, 1, 1)):
+    """Filter gradient of the 3-D convolution, the same loop nest
+    (rocmlir-gen.cpp:1715-1997) with the filter as the result tensor
+    (:1734-1736): fil[g,k,c,t] += out[n,g,k,o] * in[n,g,c,i] with
+    i = o*stride + t*dilation - pad, wherever i lies inside the input
+    (:1905-1911, 1930-1937).
+    numpy, one product per filter tap, sums in f64.  Returns the flat
+    filter-shaped gradient."""
+    outs = tuple(conv_out_dim(in_size[a], fil_size[a], pad[a], pad[a], stride[a], dil[a]) for a in range(3))
+    x = _conv3d_canon(inp, in_layout, "ngc012", (n, g, c) + tuple(in_size))
+    dy = _conv3d_canon(dout, out_layout, "ngk012", (n, g, k) + outs)
+    xp = np.zeros((n, g, c) + tuple(in_size[a] + 2 * pad[a] for a in range(3)))
+    xp[:, :, :, pad[0]:pad[0] + in_size[0], pad[1]:pad[1] + in_size[1], pad[2]:pad[2] + in_size[2]] = x
+    df = np.zeros((g, k, c) + tuple(fil_size))
+    for (t0, t1, t2), win in _conv3d_windows(in_size, fil_size, outs, stride, pad, dil):
+        df[:, :, :, t0, t1, t2] = np.einsum("ngcabd,ngkabd->gkc", xp[(slice(None),) * 3 + win], dy)
+    return df.transpose(["gkc012".index(ch) for ch in fil_layout]).astype(np.float32).ravel()
+
+
 # ---- attention ------------------------------------------------------------
 def attention(Q, K, V, G, sq, sk, dqk, dv, scale=1.0, scale_t=None,
               bias_t=None, transQ=False, transK=False, transV=False,

@@ -8,8 +8,9 @@ CPU or eager fallback: if the library is missing, importing the binding
 raises.
 """
 from .api import (RockError, RockKernel, RockProgram, attention, conv2d, conv2d_bwd_data,  conv3d,  # noqa: F401
-                  conv2d_bwd_weight, gemm, library_path, load_library, mfma_rate)
+                  conv2d_bwd_weight, conv3d_bwd_data, conv3d_bwd_weight, gemm, library_path, load_library,
+                  mfma_rate)
 
-__all__ = ["RockError", "RockKernel", "RockProgram", "gemm", "conv2d", "conv3d", "conv2d_bwd_data", "conv2d_bwd_weight", "attention",
-           "library_path", "load_library", "mfma_rate"]
+__all__ = ["RockError", "RockKernel", "RockProgram", "gemm", "conv2d", "conv3d", "conv2d_bwd_data", "conv2d_bwd_weight",
+           "conv3d_bwd_data", "conv3d_bwd_weight", "attention", "library_path", "load_library", "mfma_rate"]
 # rocmlir_amd.tuning (tuning table + in-process tuner) is imported on demand

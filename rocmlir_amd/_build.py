@@ -103,7 +103,7 @@ def attention_kernels():
 # kernels of csrc/relayout_kernels.hip in file order (-DROCK_KERNEL=<position>)
 RELAYOUT_KERNELS = ["rock_relayout_b1", "rock_relayout_b2", "rock_relayout_b4", "rock_fill_zero",
                     "rock_reduce_splits", "rock_softmax_rows", "rock_relayout_pair_b1", "rock_relayout_pair_b2",
-                    "rock_relayout_pair_b4"]
+                    "rock_relayout_pair_b4", "rock_fold_depth"]
 # kernels of csrc/probe_kernels.hip by operand-type code (-DROCK_KERNEL=<code>)
 PROBE_KERNELS = {0: "rock_probe_mfma_f32", 1: "rock_probe_mfma_f16", 2: "rock_probe_mfma_bf16",
                  3: "rock_probe_mfma_i8", 4: "rock_probe_mfma_fp8"}

@@ -593,12 +593,13 @@ def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, zero_point=0,
 def conv3d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize, in_channels, out_channels, in_size,
            fil_size, groupsize=1, stride=(1, 1, 1), padding=(0, 0, 0), dilation=(1, 1, 1), out_dtype=None,
            scale=None, zero_point=0, bias=None, relu=False, quant_scale=None, out_zero_point=0,
-           activation=None, clip=None, out=None, perf_config=None, stream=None, info=None):
+           activation=None, clip=None, residual=None, residual_op="add", out=None, perf_config=None,
+           stream=None, info=None):
     """Forward convolution over three spatial dimensions.  Sizes, strides,
     padding and dilation are (h, w, d) triples; the layout strings have six
     letters ('ngc012' / 'gkc012' / 'ngk012' in rocmlir-gen's spelling, h w d
-    and y x z accepted for 0 1 2).  Epilogue arguments as for conv2d(), without
-    a residual tensor.  Returns the flat output tensor."""
+    and y x z accepted for 0 1 2).  Epilogue arguments as for conv2d(); the
+    residual is laid out like the output.  Returns the flat output tensor."""
     import torch
     t = _dtype_name(inp.dtype)
     outs = [(in_size[a] + 2 * padding[a] - (fil_size[a] - 1) * dilation[a] - 1) // stride[a] + 1 for a in range(3)]
@@ -613,7 +614,8 @@ def conv3d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize, in_channel
         opts += " --out_type %s" % out_dtype
     if perf_config:
         opts += " --perf_config %s" % perf_config
-    opts += _epilogue_flags(scale, zero_point, bias, relu, quant_scale, out_zero_point, activation, clip, None, "add")
+    opts += _epilogue_flags(scale, zero_point, bias, relu, quant_scale, out_zero_point, activation, clip, residual,
+                            residual_op)
     prog = _program(opts)
     if info is not None:
         info["kernels"] = [x.kernel_name for x in prog.kernels]
@@ -623,7 +625,64 @@ def conv3d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize, in_channel
     if out is None:
         out = torch.empty(batchsize * out_channels * outs[0] * outs[1] * outs[2], dtype=_torch_dtype(out_dtype),
                           device=inp.device)
-    prog.launch(fil.contiguous(), inp.contiguous(), out, bias, stream=stream)
+    if residual is None:
+        prog.launch(fil.contiguous(), inp.contiguous(), out, bias, stream=stream)
+    else:
+        if residual.dtype != out.dtype or residual.numel() != out.numel():
+            raise RockError("conv3d: the residual must have the output's type and size")
+        prog.launch(fil.contiguous(), inp.contiguous(), out, bias, residual.contiguous(), stream=stream)
+    return out
+
+
+def _conv3d_options(operation, t, fil_layout, in_layout, out_layout, batchsize, groupsize, in_channels,
+                    out_channels, in_size, fil_size, stride, padding, dilation):
+    opts = ("--operation %s --arch gfx950 --in_type %s --fil_type %s --out_type %s --fil_layout %s --in_layout %s"
+            " --out_layout %s --batchsize %d --groupsize %d --in_channels %d --out_channels %d"
+            % (operation, t, t, t, fil_layout, in_layout, out_layout, batchsize, groupsize, in_channels,
+               out_channels))
+    for a, s in enumerate("hwd"):
+        opts += (" --in_%s %d --fil_%s %d --dilation_%s %d --conv_stride_%s %d --padding_%s %d"
+                 % (s, in_size[a], s, fil_size[a], s, dilation[a], s, stride[a], s, padding[a]))
+    return opts
+
+
+def conv3d_bwd_data(fil, dout, *, fil_layout, in_layout, out_layout, batchsize, in_channels, out_channels, in_size,
+                    fil_size, groupsize=1, stride=(1, 1, 1), padding=(0, 0, 0), dilation=(1, 1, 1), out=None,
+                    stream=None, info=None):
+    """Gradient of conv3d with respect to its input (operation conv_bwd_data
+    with the in_d / fil_d keys): `dout` is the gradient of the output, laid
+    out as `out_layout` says; returns the flat input-shaped gradient."""
+    import torch
+    t = _dtype_name(dout.dtype)
+    prog = _program(_conv3d_options("conv_bwd_data", t, fil_layout, in_layout, out_layout, batchsize, groupsize,
+                                    in_channels, out_channels, in_size, fil_size, stride, padding, dilation))
+    if info is not None:
+        info["kernels"] = [k.kernel_name for k in prog.kernels]
+        info["workspace_bytes"] = prog.workspace_bytes
+    if out is None:
+        out = torch.empty(batchsize * in_channels * in_size[0] * in_size[1] * in_size[2], dtype=dout.dtype,
+                          device=dout.device)
+    prog.launch(fil.contiguous(), out, dout.contiguous(), None, stream=stream)
+    return out
+
+
+def conv3d_bwd_weight(inp, dout, *, fil_layout, in_layout, out_layout, batchsize, in_channels, out_channels,
+                      in_size, fil_size, groupsize=1, stride=(1, 1, 1), padding=(0, 0, 0), dilation=(1, 1, 1),
+                      out=None, stream=None, info=None):
+    """Gradient of conv3d with respect to its filter (operation
+    conv_bwd_weight with the in_d / fil_d keys); returns the flat
+    filter-shaped gradient."""
+    import torch
+    t = _dtype_name(dout.dtype)
+    prog = _program(_conv3d_options("conv_bwd_weight", t, fil_layout, in_layout, out_layout, batchsize, groupsize,
+                                    in_channels, out_channels, in_size, fil_size, stride, padding, dilation))
+    if info is not None:
+        info["kernels"] = [k.kernel_name for k in prog.kernels]
+        info["workspace_bytes"] = prog.workspace_bytes
+    if out is None:
+        out = torch.empty(out_channels * (in_channels // groupsize) * fil_size[0] * fil_size[1] * fil_size[2],
+                          dtype=dout.dtype, device=dout.device)
+    prog.launch(out, inp.contiguous(), dout.contiguous(), None, stream=stream)
     return out
 
 

@@ -153,6 +153,22 @@ struct RockReduceParams {
   int32_t out_dtype; // RockDType: f32, f16 or bf16
 };
 
+// rock_fold_depth(T, dst, p): last step of the input gradient of a convolution
+// over three spatial dimensions.  T[n, do, h, w, g, z, c] (c padded to cp,
+// t_pix = g * z * cp elements per pixel) holds the gradient with the depth
+// taps still unfolded; every input element (n, g, c, h, w, d) is the sum, in
+// ascending z, of T at the (do, z) with do * stride_d + z * dil_d - pad_d == d,
+// added in f32 and written once in the tensor's type at
+// dst[n*s0 + g*s1 + c*s2 + h*s3 + w*s4 + d*s5].
+struct RockFoldDepthParams {
+  int64_t dst_stride[6];
+  int64_t t_pix;
+  int32_t n, g, c, cp, hi, wi, di, d_out, z;
+  int32_t stride_d, dil_d, pad_d;
+  int32_t dtype; // RockDType: f32, f16 or bf16
+  int32_t pad_;
+};
+
 // rock_softmax_rows(S, scale_tensor, bias, p): the middle kernel of attention
 // run as three kernels (head dimensions beyond the fused kernel's, f32).  S
 // holds G*seq_q rows of seq_k f32 scores, `row_pitch` floats apart; row by row

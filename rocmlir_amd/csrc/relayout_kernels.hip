@@ -366,3 +366,42 @@ extern "C" __global__ __launch_bounds__(256) void rock_relayout_pair_b4(const vo
   relayout_pair_body<uint32_t>(src0, dst0, src1, dst1, p);
 }
 #endif
+
+// one input element per thread, channels fastest
+#if RK_SELECTED(9)
+extern "C" __global__ __launch_bounds__(256) void rock_fold_depth(const void *T, void *dst, RockFoldDepthParams p) {
+  const int64_t total = (int64_t)p.n * p.di * p.hi * p.wi * p.g * p.c;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total)
+    return;
+  int64_t rem = i;
+  const int c = (int)(rem % p.c); rem /= p.c;
+  const int g = (int)(rem % p.g); rem /= p.g;
+  const int w = (int)(rem % p.wi); rem /= p.wi;
+  const int h = (int)(rem % p.hi); rem /= p.hi;
+  const int d = (int)(rem % p.di);
+  const int64_t n = rem / p.di;
+  float acc = 0.0f;
+  for (int z = 0; z < p.z; ++z) {
+    const int num = d + p.pad_d - z * p.dil_d;
+    if (num < 0)
+      break;
+    if (num % p.stride_d != 0)
+      continue;
+    const int od = num / p.stride_d;
+    if (od >= p.d_out)
+      continue;
+    const int64_t pix = ((n * p.d_out + od) * p.hi + h) * p.wi + w;
+    acc = acc + load_as_f32(T, pix * p.t_pix + ((int64_t)g * p.z + z) * p.cp + c, p.dtype);
+  }
+  const int64_t off = n * p.dst_stride[0] + g * p.dst_stride[1] + c * p.dst_stride[2] + h * p.dst_stride[3] +
+                      w * p.dst_stride[4] + d * p.dst_stride[5];
+  if (p.dtype == ROCK_F32) {
+    ((float *)dst)[off] = acc;
+  } else if (p.dtype == ROCK_F16) {
+    ((_Float16 *)dst)[off] = (_Float16)acc;
+  } else {
+    ((__bf16 *)dst)[off] = (__bf16)acc;
+  }
+}
+#endif

@@ -225,6 +225,47 @@ def test_conv3d_with_depth_one_is_the_2d_oracle(oracle):
     assert outs == (ho, wo, 1) and np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("case", CONV3D_CASES)
+@pytest.mark.parametrize("layouts", CONV3D_LAYOUTS, ids=lambda l: l[1])
+def test_conv3d_gradients_vs_torch_autograd(oracle, case, layouts):
+    """Both 3-D gradients against torch's autograd of conv3d (library routines)
+    on integer-valued data in float64: every sum is exact, so a wrong index,
+    a transposed operand or a missed padding check shows."""
+    n, g, c, k, ins, fs, stride, pad, dil = case
+    rng = np.random.default_rng(4000 + 16 * CONV3D_CASES.index(case) + CONV3D_LAYOUTS.index(layouts))
+    outs = tuple(oracle.conv_out_dim(ins[a], fs[a], pad[a], pad[a], stride[a], dil[a]) for a in range(3))
+    fil = rng.integers(-3, 4, (g, k, c) + fs).astype(np.float32)
+    inp = rng.integers(-3, 4, (n, g, c) + ins).astype(np.float32)
+    dout = rng.integers(-3, 4, (n, g, k) + outs).astype(np.float32)
+    fl, il, ol = layouts
+    x = torch.from_numpy(inp.reshape((n, g * c) + ins)).double().requires_grad_()
+    w = torch.from_numpy(fil.reshape((g * k, c) + fs)).double().requires_grad_()
+    y = torch.nn.functional.conv3d(x, w, stride=stride, padding=pad, dilation=dil, groups=g)
+    y.backward(torch.from_numpy(dout.reshape((n, g * k) + outs)).double())
+    dx = oracle.conv3d_bwd_data(_to_layout(fil, "gkc012", fl), _to_layout(dout, "ngk012", ol), fl, il, ol,
+                                n, g, c, k, ins, fs, stride, pad, dil)
+    dw = oracle.conv3d_bwd_weight(_to_layout(inp, "ngc012", il), _to_layout(dout, "ngk012", ol), fl, il, ol,
+                                  n, g, c, k, ins, fs, stride, pad, dil)
+    assert np.array_equal(dx.astype(np.float64), _to_layout(x.grad.numpy().reshape((n, g, c) + ins), "ngc012", il))
+    assert np.array_equal(dw.astype(np.float64), _to_layout(w.grad.numpy().reshape((g, k, c) + fs), "gkc012", fl))
+
+
+def test_conv3d_gradients_with_depth_one_are_the_2d_oracle(oracle):
+    n, g, c, k, hi, wi, y, x = 2, 2, 3, 4, 6, 7, 3, 2
+    rng = np.random.default_rng(18)
+    ho, wo = oracle.conv_out_dim(hi, y, 1, 1, 2, 1), oracle.conv_out_dim(wi, x, 0, 0, 1, 2)
+    fil = rng.integers(-3, 4, g * k * c * y * x).astype(np.float32)
+    inp = rng.integers(-3, 4, n * g * c * hi * wi).astype(np.float32)
+    dout = rng.integers(-3, 4, n * g * k * ho * wo).astype(np.float32)
+    want_dx, _, _ = oracle.conv_bwd_data(fil, dout, "gkcyx", "ngchw", "ngkhw", n, g, c, k, hi, wi, y, x, (2, 1), (1, 0),
+                                         (1, 2))
+    want_dw, _, _ = oracle.conv_bwd_weight(inp, dout, "gkcyx", "ngchw", "ngkhw", n, g, c, k, hi, wi, y, x, (2, 1),
+                                           (1, 0), (1, 2))
+    a3 = ("gkc012", "ngc012", "ngk012", n, g, c, k, (hi, wi, 1), (y, x, 1), (2, 1, 1), (1, 0, 0), (1, 2, 1))
+    assert np.array_equal(oracle.conv3d_bwd_data(fil, dout, *a3), want_dx)
+    assert np.array_equal(oracle.conv3d_bwd_weight(inp, dout, *a3), want_dw)
+
+
 def _bwd_golden_cases():
     with open(os.path.join(HERE, "golden", "conv_bwd_kats.json")) as f:
         return json.load(f)
