@@ -328,6 +328,10 @@ class RockProgram:
     on one stream.  Single-kernel problems behave like their RockKernel."""
 
     def __init__(self, options):
+        self.options = options
+        self._build(options)
+
+    def _build(self, options):
         first = RockKernel(options)
         self.kernels = [first] + [RockKernel("%s --kernel_id %d" % (options, i))
                                   for i in range(1, first.kernel_count)]
@@ -338,6 +342,19 @@ class RockProgram:
     def main(self):
         """The contraction kernel (the last of the problem)."""
         return self.kernels[-1]
+
+    # what rocmlir_amd.tuning.tune() uses, so that problems of several kernels tune like single ones
+    kernel_name = property(lambda self: self.main.kernel_name)
+    perf_config = property(lambda self: self.main.perf_config)
+    problem_key = property(lambda self: self.main.problem_key)
+
+    def tuning_space(self, kind="full"):
+        return self.kernels[0].tuning_space(kind)
+
+    def set_perf_config(self, perf_config):
+        """Plans the problem again under `perf_config` (the kernel list can
+        change: a request may add or drop conversion kernels)."""
+        self._build(self.options + (" --perf_config %s" % perf_config if perf_config else ""))
 
     def _args(self, args):
         if self.kernels[0].caller_pointers == len(args):

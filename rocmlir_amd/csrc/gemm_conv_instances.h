@@ -55,11 +55,14 @@
     rk::gemm_body_splitk<ROCK_DT, RICH>(A, B, C, aux, res, p);                                        \
   }
 
-// input window resident in LDS: 224 output pixels x 128 channels per block
+// input window resident in LDS: 224 (types with 32-byte MFMA operands: 128) output pixels x 128 channels per
+// block, two blocks per CU;
+// `fil` is the filter as the conversion kernel in front repacked it
 #define RK_CONV_DIRECT(NAME, RICH)                                                                    \
-  extern "C" __global__ __launch_bounds__(512) void RK_CONV_NAME(NAME)(                               \
+  extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void RK_CONV_NAME(NAME)( \
       const void *fil, const void *in, void *out, const void *aux, const void *res, RockConvParams p) { \
-    rk::conv_direct_body<ROCK_DT, 7, 2, RICH>(in, fil, out, aux, res, p);                             \
+    rk::conv_direct_body<ROCK_DT, rk::kDirectPixelBlocks<ROCK_DT>, RICH, rk::kDirectPrefetch<ROCK_DT>>(in, fil, out, aux, \
+                                                                                                       res, p);        \
   }
 
 // filter gradient: A = the output gradient [k][pixel], B = the im2col matrix [(y, x, c)][pixel], both K-major

@@ -38,6 +38,7 @@ __device__ __forceinline__ void relayout_transpose(const T *src, T *dst, const R
   const int org_d = (int)(b % tiles_d) << td_shift;
   b /= tiles_d;
   int64_t so = 0, dof = 0;
+  bool outer_in = true; // the block's position in the other three dimensions lies inside the source
 #pragma unroll
   for (int d = 4; d >= 0; --d) {
     int i;
@@ -48,6 +49,7 @@ __device__ __forceinline__ void relayout_transpose(const T *src, T *dst, const R
     } else {
       i = (int)(b % (unsigned)p.size[d]);
       b /= (unsigned)p.size[d];
+      outer_in = outer_in && i < p.src_size[d];
     }
     so += (int64_t)i * p.src_stride[d];
     dof += (int64_t)i * p.dst_stride[d];
@@ -61,7 +63,7 @@ __device__ __forceinline__ void relayout_transpose(const T *src, T *dst, const R
     const int r = idx >> ts_shift, cs = idx & (ts - 1); // along dst_fast, along src_fast
     if (org_d + r < size_d && org_s + cs < size_s)
       tile[r * (ts + 1) + cs] =
-          (org_d + r < src_d && org_s + cs < src_s) ? src[so + (int64_t)r * ss_d + (int64_t)cs * ss_s] : (T)0;
+          (outer_in && org_d + r < src_d && org_s + cs < src_s) ? src[so + (int64_t)r * ss_d + (int64_t)cs * ss_s] : (T)0;
   }
   __syncthreads();
   // write: consecutive threads walk the destination's contiguous dimension
@@ -95,6 +97,7 @@ __device__ __forceinline__ void relayout_transpose_vec(const T *src, T *dst, con
   const int org_d = (int)(b % tiles_d) * TILE;
   b /= tiles_d;
   int64_t so = 0, dof = 0;
+  bool outer_in = true; // the block's position in the other three dimensions lies inside the source
 #pragma unroll
   for (int d = 4; d >= 0; --d) {
     int i;
@@ -105,6 +108,7 @@ __device__ __forceinline__ void relayout_transpose_vec(const T *src, T *dst, con
     } else {
       i = (int)(b % (unsigned)p.size[d]);
       b /= (unsigned)p.size[d];
+      outer_in = outer_in && i < p.src_size[d];
     }
     so += (int64_t)i * p.src_stride[d];
     dof += (int64_t)i * p.dst_stride[d];
@@ -123,12 +127,12 @@ __device__ __forceinline__ void relayout_transpose_vec(const T *src, T *dst, con
       continue;
     const T *g = src + so + (int64_t)r * ss_d + cs0;
     Vec u;
-    if (org_d + r < src_d && org_s + cs0 + V <= src_s && ((uintptr_t)g & 15) == 0) {
+    if (outer_in && org_d + r < src_d && org_s + cs0 + V <= src_s && ((uintptr_t)g & 15) == 0) {
       u.v = *(const uint4 *)g;
     } else {
 #pragma unroll
       for (int e = 0; e < V; ++e)
-        u.e[e] = (org_d + r < src_d && org_s + cs0 + e < src_s) ? g[e] : (T)0;
+        u.e[e] = (outer_in && org_d + r < src_d && org_s + cs0 + e < src_s) ? g[e] : (T)0;
     }
     *(uint4 *)&tile[r * PITCH + cs0] = u.v;
   }
@@ -159,7 +163,7 @@ __device__ __forceinline__ void relayout_transpose_vec(const T *src, T *dst, con
 // RELAYOUT_COPY: source and destination share their contiguous dimension
 // (index 4) but not its length or the other strides.  The destination's runs
 // along it are whole 16-byte chunks; a thread builds one chunk, reading zero
-// beyond the source's length.  blockIdx.x enumerates groups of 256 chunks over
+// beyond the source's extent.  blockIdx.x enumerates groups of 256 chunks over
 // the flattened dimensions (2, 3, chunk), then dimensions 1 and 0.
 template <typename T>
 __device__ __forceinline__ void relayout_copy(const T *src, T *dst, const RockRelayoutParams &p, unsigned block) {
@@ -180,7 +184,10 @@ __device__ __forceinline__ void relayout_copy(const T *src, T *dst, const RockRe
                      (int64_t)i2 * p.src_stride[2] + (int64_t)i3 * p.src_stride[3];
   const int64_t dof = (int64_t)i0 * p.dst_stride[0] + (int64_t)i1 * p.dst_stride[1] +
                       (int64_t)i2 * p.dst_stride[2] + (int64_t)i3 * p.dst_stride[3] + (int64_t)ch * EPC;
-  const int e0 = (int)ch * EPC, lim = p.src_size[4];
+  // zero beyond the source's extent in EVERY dimension (a filter padded with whole rows as well as channels)
+  const bool outer_in = i0 < (unsigned)p.src_size[0] && i1 < (unsigned)p.src_size[1] && i2 < (unsigned)p.src_size[2] &&
+                        i3 < (unsigned)p.src_size[3];
+  const int e0 = (int)ch * EPC, lim = outer_in ? p.src_size[4] : 0;
   const int64_t ss = p.src_stride[4];
   union {
     T e[EPC];

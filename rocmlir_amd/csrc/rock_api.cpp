@@ -208,7 +208,7 @@ const Tile kGenericTile = {"_64x64_generic", 64, 64, 2, 2, 4, 0.1f, true, true};
 const Tile kSplitKTile = {"_32x32_splitk", 32, 32, 1, 4, 2, 0.3f, true, false};
 constexpr int kNumCU = 256; // MI355X
 constexpr int kDirectTilePixels = 224;          // conv_direct.h: 7 blocks of 32 output pixels
-constexpr int64_t kDirectWindowBytes = 96 * 1024; // and its LDS window
+constexpr int64_t kDirectWindowBytes = 80 * 1024; // conv_direct.h: the window's share of LDS (two blocks per CU)
 constexpr int kNumXCD = 8;
 
 int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
@@ -2686,51 +2686,83 @@ Handle *make_conv(const OptMap &o) {
     set_contraction_pointers(h, p.epi);
   h->perf_config = perf_string(*tile, es, &o);
 
-  // Window-resident kernel (conv_direct.h), chosen by "-perf_config
-  // v2:224,128,...": stride 1, dilation 1, a filter of more than one tap,
-  // channel run a power of two of 128..1024 bytes, output width within the
-  // 224-pixel tile and a window of TH + 2(Y-1) padded rows (a tile may
-  // straddle two images) within 96 KiB of LDS.  On the ResNet 3x3 layer of
-  // the benchmark it runs within a few percent of the implicit-GEMM kernel,
-  // so the table does not pick it by itself; a request that cannot be met
-  // falls back to the table like any other perf_config.
-  {
+  // Window-resident kernel (conv_direct.h): stride 1, dilation 1, a filter of
+  // more than one tap, channel run a power of two of 128..1024 bytes, whole
+  // 32-channel blocks of output channels, output rows that fit the tile's
+  // pixels and a window of TH + Y - 1 padded rows (Y - 1 more when tiles
+  // straddle two images) within 80 KiB of LDS.  Two kernels: a conversion
+  // kernel first stores the filter fragment-major in the workspace
+  //   F'[g][32-channel block][K-step of 128 bytes][chunk 0..7][channel 0..31][16 B]
+  // (every group padded with zero rows to whole 128-channel tiles), then the
+  // contraction reads it with coalesced loads straight into registers.  Taken
+  // on request ("-perf_config v2:224,128,...") and, for the 16-bit types, by
+  // itself where its tiles fill (3x3 layers of 28- and 56-wide images: 1.2-1.3x
+  // the implicit-GEMM kernel); a request that cannot be met falls back to the
+  // table like any other perf_config.
+  if (!planned) {
     const int64_t cbytes = c * es;
-    const int64_t th = std::min<int64_t>(ho, wo > 0 ? kDirectTilePixels / wo : 0);
+    const bool wide_operands = ti == ROCK_FP8 || ti == ROCK_BF8; // conv_direct.h: 4 pixel blocks per tile, else 7
+    const int64_t tile_px = wide_operands ? 128 : kDirectTilePixels;
     const int64_t row_pitch = ((wi + 2 * pw) * cbytes + 1023) / 1024 * 1024; // whole 1 KiB load slabs
-    const int64_t window = (th + 2 * (y - 1)) * row_pitch;
+    auto window_rows = [&](int64_t rows) { return rows + (y - 1) + (ho % rows ? y - 1 : 0); };
+    const int64_t tiles_n = ceil_div(k, 128);
+    auto tiles_of = [&](int64_t rows) { return (int64_t)ceil_div(n * ho, rows) * tiles_n * g; };
+    // rows per tile: the fewest rounds of blocks (two per CU), then the most rows
+    const int64_t per_round = 2 * (int64_t)kNumCU;
+    int64_t th = 0;
+    for (int64_t rows = std::min<int64_t>(ho, wo > 0 ? tile_px / wo : 0); rows >= 1; --rows) {
+      if (window_rows(rows) * row_pitch > kDirectWindowBytes)
+        continue;
+      if (th == 0 || ceil_div(tiles_of(rows), per_round) < ceil_div(tiles_of(th), per_round))
+        th = rows;
+    }
     // the kernel sizes its window from the left / top padding alone: both sides must be equal
     const bool direct_ok = fast && sh == 1 && sw == 1 && dh == 1 && dw == 1 && y * x > 1 &&
-                           ph_r == ph && pw_r == pw &&
+                           ph_r == ph && pw_r == pw && k % 32 == 0 &&
                            cbytes >= 128 && cbytes <= 1024 && (cbytes & (cbytes - 1)) == 0 &&
-                           th >= 1 && window <= kDirectWindowBytes && row_pitch <= 32 * 1024;
+                           th >= 1 && row_pitch <= 32 * 1024 && p.fil_cs == 1 && p.fil_xs == c && p.fil_ys == x * c;
     const bool asked = requested_tile_is(o, kDirectTilePixels, 128);
-    if (direct_ok && asked) {
-      // rows per tile: the most that fit, unless a slightly shorter tile fills
-      // the last round of blocks better (cost = rounds x (rows + ~2 rows of
-      // window halo and epilogue per tile))
-      int64_t best_th = th;
-      const int64_t per_round = (int64_t)kNumCU;
-      auto cost = [&](int64_t rows) {
-        int64_t tiles = (int64_t)ceil_div(n * ho, rows) * ceil_div(k, 128) * g;
-        return ((tiles + per_round - 1) / per_round) * (rows + 2);
-      };
-      for (int64_t rows = th - 1; rows >= std::max<int64_t>(1, th / 2); --rows)
-        if (cost(rows) < cost(best_th))
-          best_th = rows;
-      const int64_t th = best_th;
+    // by itself: 16-bit types, tiles at least 85 % full, enough of them for every CU, no tile requested
+    const bool by_itself = direct_ok && (ti == ROCK_F16 || ti == ROCK_BF16) && forced_tile(o).empty() && y * x >= 4 &&
+                           th * wo * 100 >= tile_px * 85 && tiles_of(th) >= per_round;
+    if (direct_ok && (asked || by_itself)) {
+      const int64_t kbytes = Kg * es;                         // a whole number of 128-byte K-steps
+      const int64_t rows_p = tiles_n * 128;                   // channels per group in F'
+      const int64_t f_bytes = align256(g * rows_p * kbytes);
+      const int ws = p.epi.residual_op ? 5 : 4;
+      const int kid = (int)int_or(o, "kernel_id", 0);
+      h->kernel_count = 2;
+      h->workspace_bytes = (size_t)f_bytes;
+      if (kid == 0) {
+        const int64_t e = 16 / es;
+        const int64_t size[5] = {g, rows_p / 32, kbytes / 16, 32, e};
+        const int64_t src_size[5] = {g, k / 32, kbytes / 16, 32, e};
+        const int64_t stride[5] = {p.fil_gs, 32 * p.fil_ks, e, p.fil_ks, 1};
+        if (!fill_relayout_handle(h, size, src_size, stride, es)) {
+          delete h;
+          return nullptr;
+        }
+        h->kernel_count = 2;
+        h->workspace_bytes = (size_t)f_bytes;
+        h->caller_pointers = ws + 1;
+        h->ptr_map = {{0, 0}, {ws, 0}};
+        h->problem_key = "repack filter " + fl;
+        return h;
+      }
       p.rows_per_tile = (int)th;
       p.tiles_m = ceil_div(n * ho, th);
-      p.tiles_n = ceil_div(k, 128);
+      p.tiles_n = (int)tiles_n;
       p.group_m = std::min(p.tiles_m, 8);
       int64_t total = (int64_t)p.tiles_m * p.tiles_n * g;
       p.xcd_remap = total >= 2 * kNumXCD ? 1 : 0;
-      h->block_size = 512;
+      h->block_size = 256;
       h->grid_size = (uint32_t)total;
       h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + "_direct224" + rich_suffix(p.epi, true, o);
       char buf[96];
       std::snprintf(buf, sizeof buf, "v2:224,128,8,224,32,%d,1,1,1", 16 / es);
       h->perf_config = buf;
+      h->caller_pointers = ws + 1;
+      h->ptr_map = {{ws, 0}, {1, 0}, {2, 0}, {3, 0}, {p.epi.residual_op ? 4 : -1, 0}};
     }
   }
   set_problem_key();
@@ -3231,7 +3263,19 @@ std::vector<std::string> tuning_candidates(const Handle &h, int kind) {
     o.erase("perf_config");
     if (!r.empty())
       o["perf_config"] = r;
+    // the contraction kernel of the plan the request leads to (conversion kernels may run in front of it)
+    o.erase("kernel_id");
     Handle *c = build_handle(o);
+    for (int id = 1; c && c->op == OP_RELAYOUT && id < c->kernel_count; ++id) {
+      const int count = c->kernel_count;
+      delete c;
+      o["kernel_id"] = std::to_string(id);
+      c = build_handle(o);
+      if (c && c->kernel_count != count) {
+        delete c;
+        c = nullptr;
+      }
+    }
     if (!c)
       continue;
     if (std::find(seen.begin(), seen.end(), c->kernel_name) == seen.end()) {

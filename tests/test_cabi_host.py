@@ -16,6 +16,9 @@ CONV_RESNET = (
     "--groupsize 1 --in_channels 128 --out_channels 128 --in_h 28 --in_w 28 --out_h 28 --out_w 28 "
     "--fil_h 3 --fil_w 3 --dilation_h 1 --dilation_w 1 --conv_stride_h 1 --conv_stride_w 1 "
     "--padding_h 1 --padding_w 1")
+# the same problem on the implicit-GEMM kernel alone (the table's own plan puts a filter conversion in front of
+# the window-resident kernel)
+CONV_IMPLICIT = CONV_RESNET + " --perf_config v2:128,128,8,64,16,8,1,1,1"
 
 
 def test_every_declared_symbol_is_exported(rock):
@@ -29,7 +32,7 @@ def test_every_declared_symbol_is_exported(rock):
 
 def test_miir_protocol_conv(rock):
     lib = rock.load_library()
-    h = lib.miirCreateHandle(CONV_RESNET.encode())
+    h = lib.miirCreateHandle(CONV_IMPLICIT.encode())
     assert h
     assert lib.miirGetKernelCount(h) == 1
     assert lib.miirGetWorkspaceSize(h) == 0
@@ -113,7 +116,8 @@ def test_null_handle_behaviour(rock):
     "--operation attention --arch gfx950 -t f16 -g 1 -seq_len_q 8 -seq_len_k 8 -head_dim_qk 256 -head_dim_v 8 "
     "--kernel_id 3",
     "--operation transpose --arch gfx950",
-    CONV_RESNET + " --kernel_id 1",
+    CONV_IMPLICIT + " --kernel_id 1",
+    CONV_RESNET + " --kernel_id 2",
 ])
 def test_bad_problems_give_null(rock, bad):
     lib = rock.load_library()
@@ -135,8 +139,12 @@ def test_baseline_configs_select_kernels(rock):
     assert (k.block_size, k.grid_size) == (512, 256)
     assert k.execution_dims() == (512 * 256, 512)
     assert k.perf_config == "v2:256,256,8,128,16,16,1,1,1"
+    # the 3x3 ResNet layer: the filter repacked for the window-resident kernel, then that kernel, two blocks per CU
     k = rock.RockKernel(CONV_RESNET)
-    assert k.kernel_name.startswith("rock_conv_f16_") and k.kernel_name.endswith("_fast")
+    assert (k.kernel_name, k.kernel_count, k.workspace_bytes, k.caller_pointers) == ("rock_relayout_b2", 2, 128 * 1152 * 2, 5)
+    k = rock.RockKernel(CONV_RESNET + " --kernel_id 1")
+    assert (k.kernel_name, k.block_size, k.grid_size) == ("rock_conv_f16_direct224", 256, 1024)
+    assert rock.RockKernel(CONV_IMPLICIT).kernel_name == "rock_conv_f16_128x128_fast"
     k = rock.RockKernel("-operation gemm -arch gfx950 -t fp8 -g 1 -m 8192 -n 8192 -k 8192 -transB true")
     assert k.kernel_name == "rock_gemm_fp8_256x256_fast" and k.grid_size == 1024
     k = rock.RockKernel("-operation attention -arch gfx950 -t f16 -g 128 -seq_len_q 2048 -seq_len_k 2048 "
@@ -267,7 +275,7 @@ def test_layout_conversion_plan_follows_the_multi_kernel_protocol(rock):
     assert [k.kernel_name for k in ks] == ["rock_relayout_b2", "rock_conv_f16_128x128_fast"]
     assert ks[0].workspace_bytes == in_bytes
     # single-kernel problems: identity map, no workspace
-    k = rock.RockKernel(CONV_RESNET)
+    k = rock.RockKernel(CONV_IMPLICIT)
     assert (k.kernel_count, k.workspace_bytes, k.caller_pointers) == (1, 0, 4)
     # a conversion kernel has no epilogue scalars to set
     assert lib.rockamdSetScale(rock.RockKernel(nchw)._h, C.c_float(2.0)) != 0
@@ -279,9 +287,10 @@ def test_argument_info_describes_the_caller_list(rock):
     k = rock.RockKernel("-operation gemm -arch gfx950 -t i8 -out_datatype f16 -g 2 -m 64 -n 48 -k 32 -transB true "
                         "-scale 0.01 -residual add")
     assert k.arguments() == [(3, [2, 64, 32]), (3, [2, 48, 32]), (1, [2, 64, 48]), (0, [48]), (1, [2, 64, 48])]
-    k = rock.RockKernel(CONV_RESNET)
+    k = rock.RockKernel(CONV_IMPLICIT)
     assert k.arguments() == [(1, [1, 128, 3, 3, 128]), (1, [256, 28, 28, 1, 128]), (1, [256, 28, 28, 1, 128]),
                              (0, [128])]
+    assert rock.RockKernel(CONV_RESNET).arguments() == k.arguments() + [(-1, [128 * 1152 * 2])]
     nchw = CONV_RESNET.replace("NHWGC", "NGCHW").replace("GNYXC", "GNCHW")
     args = rock.RockKernel(nchw + " --kernel_id 1").arguments()     # every kernel of a plan: the same list
     assert args[1] == (1, [256, 1, 128, 28, 28]) and args[4] == (-1, [rock.RockKernel(nchw).workspace_bytes])
@@ -444,7 +453,8 @@ def test_problem_keys_follow_reference_format(rock):
     k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 1024 -n 512 -k 769 -transB true")
     assert k.problem_key.split("\t")[2] == \
         "-t f16 -out_datatype f16 -transA false -transB true -g 1 -m 1024 -n 512 -k 769"
-    k = rock.RockKernel(CONV_RESNET)
+    k = rock.RockKernel(CONV_RESNET + " --kernel_id 1")
+    assert rock.RockKernel(CONV_IMPLICIT).problem_key == k.problem_key
     assert k.problem_key.split("\t")[2] == (
         "convfp16 -F 1 -f GN01C -I N01GC -O N01GC -n 256 -c 128 -H 28 -W 28 -k 128 -y 3 -x 3 "
         "-p 1 -q 1 -u 1 -v 1 -l 1 -j 1 -g 1")
@@ -615,7 +625,7 @@ def test_window_resident_request_with_asymmetric_padding_falls_back(rock):
     asked = rock.RockKernel(asym + " --perf_config v2:224,128,8,224,32,8,1,1,1")
     assert "direct224" not in asked.kernel_name and asked.kernel_name == base.kernel_name
     assert "v2:224,128,8,224,32,8,1,1,1" not in base.tuning_space()
-    sym = rock.RockKernel(CONV_RESNET + " --perf_config v2:224,128,8,224,32,8,1,1,1")
+    sym = rock.RockKernel(CONV_RESNET + " --perf_config v2:224,128,8,224,32,8,1,1,1 --kernel_id 1")
     assert sym.kernel_name == "rock_conv_f16_direct224"
 
 

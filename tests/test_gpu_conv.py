@@ -218,26 +218,29 @@ def test_conv_every_fast_tile(rock, oracle, gpu, tile):
 # The window-resident kernel ("-perf_config v2:224,128,..."): stride 1, dilation 1.
 # (n g pixel_bytes k hi wi y x pad); the channel count follows from the element size.
 WINDOW_CASES = [
-    (3, 1, 128, 128, 28, 28, 3, 3, (1, 1)),  # 8-row tiles over 28-row images: tiles straddle images
+    (3, 1, 128, 128, 28, 28, 3, 3, (1, 1)),  # 7-row tiles: four per image
     (5, 1, 256, 96, 9, 7, 3, 3, (1, 1)),     # whole small images per tile, 96 of 128 output channels
     (4, 1, 128, 32, 30, 30, 3, 3, (0, 1)),   # 28x30 outputs, padding in one direction only
-    (3, 1, 128, 64, 10, 12, 3, 3, (1, 1)),   # 18-row tiles capped at the image height of 10
-    (7, 1, 128, 48, 6, 50, 3, 3, (1, 1)),    # 4-row tiles against 6-row images: tiles straddle images
-    (2, 2, 128, 40, 12, 20, 3, 5, (1, 2)),   # two groups, 3x5 filter
-    (2, 1, 128, 130, 10, 33, 2, 2, (0, 0)),  # even filter, no padding, two blocks of output channels
+    (3, 1, 128, 64, 10, 12, 3, 3, (1, 1)),   # tiles capped at the image height of 10
+    (7, 1, 128, 64, 6, 50, 3, 3, (1, 1)),    # 4-row tiles against 6-row images: tiles straddle images
+    (2, 2, 128, 96, 12, 20, 3, 5, (1, 2)),   # two groups, 3x5 filter, each group padded to 128 channels
+    (2, 1, 128, 160, 10, 33, 2, 2, (0, 0)),  # even filter, no padding, two tiles of output channels
     (1, 1, 512, 64, 6, 6, 5, 5, (2, 2)),     # 512-byte pixels, 5x5 filter
+    (9, 1, 256, 128, 14, 14, 3, 3, (1, 1)),  # 14-wide images: 16-row budget, window-limited
 ]
 
 
 @pytest.mark.parametrize("case", WINDOW_CASES)
-@pytest.mark.parametrize("t", ["f32", "f16", "bf16", "i8"])
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16", "i8", "fp8"])
 def test_conv_window_resident_kernel_exact(rock, oracle, gpu, case, t):
     n, g, pixel_bytes, k, hi, wi, y, x, pad = case
-    c = pixel_bytes // {"f32": 4, "f16": 2, "bf16": 2, "i8": 1}[t]
+    c = pixel_bytes // {"f32": 4, "f16": 2, "bf16": 2, "i8": 1, "fp8": 1}[t]
     info = {}
+    print("window-resident conv", case, t, flush=True)
     out, od, ref = _run(rock, oracle, gpu, t, n, g, c, k, hi, wi, y, x, (1, 1), pad, (1, 1), NHWC, True, 41,
                         perf_config="v2:224,128,8,224,32,8,1,1,1", info=info)
-    assert info["kernel_name"] == "rock_conv_%s_direct224" % t
+    assert info["kernels"] == ["rock_relayout_b%d" % {"f32": 4, "f16": 2, "bf16": 2}.get(t, 1),
+                               "rock_conv_%s_direct224" % t]
     if t == "i8":
         assert oracle.verify_int(out.cpu().numpy().ravel(), ref)[0] == 0
     else:

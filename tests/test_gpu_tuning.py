@@ -51,7 +51,7 @@ def test_tuner_conv_includes_the_window_resident_kernel(rock, oracle, gpu):
                                   (1, 1))
     F, I = to_gpu(rf, "f16", gpu), to_gpu(ri, "f16", gpu)
     out = torch.zeros(n * ho * wo * k, dtype=torch.float16, device=gpu)
-    kern = rock.RockKernel(
+    kern = rock.RockProgram(   # the window-resident kernel comes with a filter conversion in front of it
         "--operation conv --arch gfx950 --in_type fp16 --fil_type fp16 --out_type fp16 --fil_layout gkyxc "
         "--in_layout nhwgc --out_layout nhwgk --batchsize %d --groupsize 1 --in_channels %d --out_channels %d "
         "--in_h %d --in_w %d --fil_h 3 --fil_w 3 --dilation_h 1 --dilation_w 1 --conv_stride_h 1 "
