@@ -88,7 +88,9 @@ typedef void *MiirHandle;
  * kernel instead of the element-wise kernel), pointwise_as_gemm (1x1
  * convolutions as a batched GEMM over the tensors as they lie),
  * bwd_weight_gemm (the filter gradient of a one-group convolution as one
- * K-major GEMM plus the reduction of its pixel splits), split_k (a GEMM with
+ * K-major GEMM plus the reduction of its pixel splits), window_resident (a
+ * 16-bit stride-1 convolution whose tiles fill on the kernel that keeps the
+ * input window in LDS, behind a conversion of the filter), split_k (a GEMM with
  * few output tiles and a long reduction split over blocks, partial sums in the
  * workspace), fused (attention, above).  A single leading dash and "key=value"
  * are accepted as well.  Returns NULL on any parse, validation or support

@@ -2697,7 +2697,7 @@ Handle *make_conv(const OptMap &o) {
   // contraction reads it with coalesced loads straight into registers.  Taken
   // on request ("-perf_config v2:224,128,...") and, for the 16-bit types, by
   // itself where its tiles fill (3x3 layers of 28- and 56-wide images: 1.2-1.3x
-  // the implicit-GEMM kernel); a request that cannot be met falls back to the
+  // the implicit-GEMM kernel; "--window_resident false" declines); a request that cannot be met falls back to the
   // table like any other perf_config.
   if (!planned) {
     const int64_t cbytes = c * es;
@@ -2722,9 +2722,12 @@ Handle *make_conv(const OptMap &o) {
                            cbytes >= 128 && cbytes <= 1024 && (cbytes & (cbytes - 1)) == 0 &&
                            th >= 1 && row_pitch <= 32 * 1024 && p.fil_cs == 1 && p.fil_xs == c && p.fil_ys == x * c;
     const bool asked = requested_tile_is(o, kDirectTilePixels, 128);
-    // by itself: 16-bit types, tiles at least 85 % full, enough of them for every CU, no tile requested
-    const bool by_itself = direct_ok && (ti == ROCK_F16 || ti == ROCK_BF16) && forced_tile(o).empty() && y * x >= 4 &&
-                           th * wo * 100 >= tile_px * 85 && tiles_of(th) >= per_round;
+    // by itself: 16-bit types, tiles at least 85 % full in pixels and 75 % in channels, enough of them for every
+    // CU, no tile requested
+    const bool by_itself = direct_ok && bool_or(o, "window_resident", true) && (ti == ROCK_F16 || ti == ROCK_BF16) &&
+                           forced_tile(o).empty() && y * x >= 4 &&
+                           th * wo * 100 >= tile_px * 85 && tiles_of(th) >= per_round &&
+                           (k % 128 == 0 || k % 128 >= 96); // (a 64-channel layer leaves half the block's waves idle)
     if (direct_ok && (asked || by_itself)) {
       const int64_t kbytes = Kg * es;                         // a whole number of 128-byte K-steps
       const int64_t rows_p = tiles_n * 128;                   // channels per group in F'

@@ -153,6 +153,7 @@ def main(argv=None):
     ap.add_argument("--warm-ms", type=float, default=30.0,
                     help="keep the GPU busy with the problem for this long before timing it (clock ramp-up)")
     ap.add_argument("--max-bytes", type=float, default=8e9, help="skip problems whose tensors exceed this")
+    ap.add_argument("--extra-options", default="", help="appended to every problem string (plan switches, a perf_config)")
     args = ap.parse_args(argv)
 
     import torch
@@ -174,6 +175,8 @@ def main(argv=None):
                 except (KeyError, ValueError) as e:
                     print(json.dumps({"config": line, "status": "unparsed", "error": str(e)}), flush=True)
                     continue
+                if args.extra_options:
+                    opts += " " + args.extra_options
                 if opts in seen:
                     continue
                 seen.add(opts)

@@ -145,6 +145,11 @@ def test_baseline_configs_select_kernels(rock):
     k = rock.RockKernel(CONV_RESNET + " --kernel_id 1")
     assert (k.kernel_name, k.block_size, k.grid_size) == ("rock_conv_f16_direct224", 256, 1024)
     assert rock.RockKernel(CONV_IMPLICIT).kernel_name == "rock_conv_f16_128x128_fast"
+    k = rock.RockKernel(CONV_RESNET + " --window_resident false")
+    assert (k.kernel_name, k.kernel_count, k.workspace_bytes) == ("rock_conv_f16_128x128_fast", 1, 0)
+    # a 64-channel layer would leave half of the window-resident kernel's waves idle: the table keeps it off
+    k = rock.RockKernel(CONV_RESNET.replace("--out_channels 128", "--out_channels 64"))
+    assert k.kernel_count == 1 and "direct224" not in k.kernel_name
     k = rock.RockKernel("-operation gemm -arch gfx950 -t fp8 -g 1 -m 8192 -n 8192 -k 8192 -transB true")
     assert k.kernel_name == "rock_gemm_fp8_256x256_fast" and k.grid_size == 1024
     k = rock.RockKernel("-operation attention -arch gfx950 -t f16 -g 128 -seq_len_q 2048 -seq_len_k 2048 "
