@@ -1065,6 +1065,65 @@ Handle *conv_handle_from_view(const RockConvParams &q, int ti, const OptMap &o) 
   return h;
 }
 
+// The window-resident kernel (conv_direct.h) on a convolution given as a view
+// (p: sizes, strides of input and output, unit stride and dilation assumed
+// checked here).  It needs: a filter of more than one tap, equal padding on
+// both sides (the caller says so), a channel run that is a power of two of
+// 128..1024 bytes, whole 32-channel blocks of output channels, output rows
+// that fit the tile's pixels, and a window of TH + Y - 1 padded rows (Y - 1
+// more when tiles straddle two images) within 80 KiB of LDS.  The filter
+// reaches it repacked (fragment-major, every group padded to whole 128-channel
+// tiles): `filter_bytes` of workspace.
+struct WindowPlan {
+  bool ok = false, by_itself = false;
+  int64_t rows = 0, tiles_n = 0, filter_bytes = 0;
+};
+WindowPlan window_plan(const RockConvParams &p, int ti, bool equal_padding, const OptMap &o) {
+  WindowPlan w;
+  const int es = dtype_size(ti);
+  const int64_t cbytes = (int64_t)p.c * es;
+  const bool wide_operands = ti == ROCK_FP8 || ti == ROCK_BF8; // 4 pixel blocks per tile, else 7
+  const int64_t tile_px = wide_operands ? 128 : kDirectTilePixels;
+  const int64_t row_pitch = ((p.wi + 2 * p.pad_w) * cbytes + 1023) / 1024 * 1024; // whole 1 KiB load slabs
+  auto window_rows = [&](int64_t rows) { return rows + (p.y - 1) + (p.ho % rows ? p.y - 1 : 0); };
+  w.tiles_n = ceil_div(p.k, 128);
+  auto tiles_of = [&](int64_t rows) { return (int64_t)ceil_div((int64_t)p.n * p.ho, rows) * w.tiles_n * p.g; };
+  // rows per tile: the fewest rounds of blocks (two per CU), then the most rows
+  const int64_t per_round = 2 * (int64_t)kNumCU;
+  for (int64_t rows = std::min<int64_t>(p.ho, p.wo > 0 ? tile_px / p.wo : 0); rows >= 1; --rows) {
+    if (window_rows(rows) * row_pitch > kDirectWindowBytes)
+      continue;
+    if (w.rows == 0 || ceil_div(tiles_of(rows), per_round) < ceil_div(tiles_of(w.rows), per_round))
+      w.rows = rows;
+  }
+  w.ok = p.stride_h == 1 && p.stride_w == 1 && p.dil_h == 1 && p.dil_w == 1 && p.y * p.x > 1 && equal_padding &&
+         p.k % 32 == 0 && cbytes >= 128 && cbytes <= 1024 && (cbytes & (cbytes - 1)) == 0 && w.rows >= 1 &&
+         row_pitch <= 32 * 1024 && p.in_cs == 1;
+  // by itself: 16-bit types, tiles at least 85 % full in pixels and 75 % in channels, enough of them for every
+  // CU, no tile requested
+  w.by_itself = w.ok && bool_or(o, "window_resident", true) && (ti == ROCK_F16 || ti == ROCK_BF16) &&
+                forced_tile(o).empty() && p.y * p.x >= 4 && w.rows * p.wo * 100 >= tile_px * 85 &&
+                tiles_of(w.rows) >= per_round &&
+                (p.k % 128 == 0 || p.k % 128 >= 96); // (a 64-channel layer leaves half the block's waves idle)
+  w.filter_bytes = align256((int64_t)p.g * w.tiles_n * 128 * p.c * p.y * p.x * es);
+  return w;
+}
+// h becomes the window-resident kernel over p (the caller sets the pointer map)
+void apply_window_plan(Handle *h, RockConvParams &p, const WindowPlan &w, int ti, const OptMap &o) {
+  p.rows_per_tile = (int)w.rows;
+  p.tiles_m = ceil_div((int64_t)p.n * p.ho, w.rows);
+  p.tiles_n = (int)w.tiles_n;
+  p.group_m = std::min(p.tiles_m, 8);
+  const int64_t total = (int64_t)p.tiles_m * p.tiles_n * p.g;
+  p.xcd_remap = total >= 2 * kNumXCD ? 1 : 0;
+  h->block_size = 256;
+  h->grid_size = (uint32_t)total;
+  h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + "_direct224" + rich_suffix(p.epi, true, o);
+  char buf[96];
+  std::snprintf(buf, sizeof buf, "v2:224,128,8,224,32,%d,1,1,1", 16 / dtype_size(ti));
+  h->perf_config = buf;
+}
+
 Handle *utility_fill_handle(int64_t bytes) {
   auto *h = new Handle;
   RockFillParams f{bytes};
@@ -1078,6 +1137,42 @@ Handle *utility_fill_handle(int64_t bytes) {
   h->num_pointers = 1;
   h->perf_config = "";
   return h;
+}
+
+// A conversion kernel between two views of one tensor of more than five
+// dimensions, listed in the destination's order (the last one contiguous
+// there): unit dimensions go, neighbours that lie back to back on both sides
+// fold, and what is left has to fit the kernel's five.
+struct ViewDim { int64_t size, src_size, ss, ds; };
+bool relayout_handle_nd(Handle *h, std::vector<ViewDim> dims, int es, const char *what) {
+  for (size_t d = 0; d + 1 < dims.size();)
+    if (dims[d].size == 1)
+      dims.erase(dims.begin() + d);
+    else
+      ++d;
+  for (size_t d = 0; d + 1 < dims.size() && dims.size() > 5;) {
+    const ViewDim &o = dims[d], &i = dims[d + 1];
+    if (i.src_size == i.size && o.ss == i.size * i.ss && o.ds == i.size * i.ds && o.size * i.size <= INT32_MAX) {
+      dims[d] = ViewDim{o.size * i.size, o.src_size * i.size, i.ss, i.ds};
+      dims.erase(dims.begin() + d + 1);
+    } else {
+      ++d;
+    }
+  }
+  if (dims.size() > 5) {
+    set_error(std::string("conv: this 3-D ") + what + " layout needs more than five independent dimensions");
+    return false;
+  }
+  while (dims.size() < 5)
+    dims.insert(dims.begin(), ViewDim{1, 1, 0, 0});
+  int64_t size[5], src_size[5], ss[5], ds[5];
+  for (int d = 0; d < 5; ++d) {
+    size[d] = dims[d].size;
+    src_size[d] = dims[d].src_size;
+    ss[d] = dims[d].ss;
+    ds[d] = dims[d].ds;
+  }
+  return fill_relayout_handle(h, size, src_size, ss, es, ds);
 }
 
 // One spatial axis of the backward-data decomposition.  Input positions with
@@ -1233,6 +1328,42 @@ Handle *make_conv_bwd_data(const OptMap &o, const ConvProblem &cp) {
     int64_t unused;
     fast = fast && conv_view_fast(phase_fast_view(ph, unused), es);
   }
+  // Phases that the window-resident kernel takes (unit stride: the one phase there is): the conversion of the
+  // flipped sub-filter then writes it fragment-major,
+  //   F'[g][32-channel block of c][(t_h, t_w, 16-byte chunk of k)][channel][k in chunk],
+  // for that kernel instead of as K-contiguous rows.  One conversion kernel has to do (five independent
+  // dimensions: one group, taps that fold), else the phase stays on the implicit-GEMM kernel.
+  const int64_t ek = 16 / es; // elements per chunk
+  auto window_filter_dims = [&](const Phase &ph, const RockConvParams &generic, const WindowPlan &w) {
+    const int64_t chunks = kp / ek, tap = 32 * kp; // elements of one tap of one channel block in F'
+    std::vector<ViewDim> dims = {
+        {cp.g, cp.g, generic.fil_gs, w.tiles_n * 4 * ph.h.T * ph.w.T * tap},
+        {w.tiles_n * 4, cp.c / 32, 32 * generic.fil_ks, ph.h.T * ph.w.T * tap},
+        {ph.h.T, ph.h.T, generic.fil_ys, ph.w.T * tap},
+        {ph.w.T, ph.w.T, generic.fil_xs, tap},
+        {chunks, chunks, ek * generic.fil_cs, 32 * ek},
+        {32, 32, generic.fil_ks, ek},
+        {ek, ek, generic.fil_cs, 1}};
+    return dims;
+  };
+  std::vector<WindowPlan> win(phases.size());
+  if (fast && kp == cp.k) {
+    const std::string keep_error = g_last_error;
+    for (size_t i = 0; i < phases.size(); ++i) {
+      int64_t u0, u1;
+      const RockConvParams q = phase_fast_view(phases[i], u0);
+      // (the view's padding is equal on both sides when the last output row ends where the padded input does)
+      const bool equal = q.ho - 1 + q.y - 1 - q.pad_h - (q.hi - 1) == q.pad_h &&
+                         q.wo - 1 + q.x - 1 - q.pad_w - (q.wi - 1) == q.pad_w;
+      const WindowPlan w = window_plan(q, cp.ti, equal, o);
+      if (!w.by_itself)
+        continue;
+      Handle probe;
+      if (relayout_handle_nd(&probe, window_filter_dims(phases[i], phase_view(phases[i], u0, u1), w), es, "filter"))
+        win[i] = w;
+    }
+    g_last_error = keep_error;
+  }
   // kernel list
   const int first_phase = (need_fill ? 1 : 0) + (fast && !dy_as_is ? 1 : 0);
   const int per_phase = fast ? 2 : 1;
@@ -1243,7 +1374,7 @@ Handle *make_conv_bwd_data(const OptMap &o, const ConvProblem &cp) {
     workspace = dy_bytes;
     for (size_t i = 0; i < phases.size(); ++i) {
       fil_ws[i] = workspace;
-      workspace += align256(cp.g * cp.c * phases[i].h.T * phases[i].w.T * kp * es);
+      workspace += win[i].ok ? win[i].filter_bytes : align256(cp.g * cp.c * phases[i].h.T * phases[i].w.T * kp * es);
     }
   }
   if (count == 0 || kid < 0 || kid >= count) {
@@ -1272,12 +1403,14 @@ Handle *make_conv_bwd_data(const OptMap &o, const ConvProblem &cp) {
     const int64_t fil_dst = fil_ws[idx / per_phase];
     int64_t fil_off, out_off;
     const RockConvParams generic = phase_view(ph, fil_off, out_off);
+    const WindowPlan &w = win[idx / per_phase];
     if (fast && idx % 2 == 0) {
-      // flipped sub-filter -> [g][c][T_h][T_w][kp]
+      // flipped sub-filter -> [g][c][T_h][T_w][kp], or fragment-major for the window-resident kernel
       h = new Handle;
       const int64_t size[5] = {cp.g, cp.c, ph.h.T, ph.w.T, kp}, src_size[5] = {cp.g, cp.c, ph.h.T, ph.w.T, cp.k};
       const int64_t stride[5] = {generic.fil_gs, generic.fil_ks, generic.fil_ys, generic.fil_xs, generic.fil_cs};
-      if (!fill_relayout_handle(h, size, src_size, stride, es)) {
+      if (!(w.ok ? relayout_handle_nd(h, window_filter_dims(ph, generic, w), es, "filter")
+                 : fill_relayout_handle(h, size, src_size, stride, es))) {
         delete h;
         return nullptr;
       }
@@ -1288,6 +1421,8 @@ Handle *make_conv_bwd_data(const OptMap &o, const ConvProblem &cp) {
       h = conv_handle_from_view(fast ? phase_fast_view(ph, off2) : generic, cp.ti, o);
       if (!h)
         return nullptr;
+      if (w.ok)
+        apply_window_plan(h, *reinterpret_cast<RockConvParams *>(h->params.data()), w, cp.ti, o);
       h->ptr_map = {fast ? Handle::PtrSrc{ws, fil_dst} : Handle::PtrSrc{0, fil_off * es},
                     (fast && !dy_as_is) ? Handle::PtrSrc{ws, 0} : Handle::PtrSrc{2, 0},
                     {1, out_off * es}, {-1, 0}, {-1, 0}};
@@ -1789,42 +1924,6 @@ bool canon_layout3(std::string s, char channel, bool filter, std::string &out) {
     return false;
   out = r;
   return true;
-}
-
-// A conversion kernel between two views of one tensor of up to six
-// dimensions, listed in the destination's order (the last one contiguous
-// there): unit dimensions go, neighbours that lie back to back on both sides
-// fold, and what is left has to fit the kernel's five.
-struct ViewDim { int64_t size, src_size, ss, ds; };
-bool relayout_handle_nd(Handle *h, std::vector<ViewDim> dims, int es, const char *what) {
-  for (size_t d = 0; d + 1 < dims.size();)
-    if (dims[d].size == 1)
-      dims.erase(dims.begin() + d);
-    else
-      ++d;
-  for (size_t d = 0; d + 1 < dims.size() && dims.size() > 5;) {
-    const ViewDim &o = dims[d], &i = dims[d + 1];
-    if (i.src_size == i.size && o.ss == i.size * i.ss && o.ds == i.size * i.ds && o.size * i.size <= INT32_MAX) {
-      dims[d] = ViewDim{o.size * i.size, o.src_size * i.size, i.ss, i.ds};
-      dims.erase(dims.begin() + d + 1);
-    } else {
-      ++d;
-    }
-  }
-  if (dims.size() > 5) {
-    set_error(std::string("conv: this 3-D ") + what + " layout needs more than five independent dimensions");
-    return false;
-  }
-  while (dims.size() < 5)
-    dims.insert(dims.begin(), ViewDim{1, 1, 0, 0});
-  int64_t size[5], src_size[5], ss[5], ds[5];
-  for (int d = 0; d < 5; ++d) {
-    size[d] = dims[d].size;
-    src_size[d] = dims[d].src_size;
-    ss[d] = dims[d].ss;
-    ds[d] = dims[d].ds;
-  }
-  return fill_relayout_handle(h, size, src_size, ss, es, ds);
 }
 
 // What the option list says about a convolution over three spatial dimensions.
@@ -2699,46 +2798,18 @@ Handle *make_conv(const OptMap &o) {
   // itself where its tiles fill (3x3 layers of 28- and 56-wide images: 1.2-1.3x
   // the implicit-GEMM kernel; "--window_resident false" declines); a request that cannot be met falls back to the
   // table like any other perf_config.
-  if (!planned) {
-    const int64_t cbytes = c * es;
-    const bool wide_operands = ti == ROCK_FP8 || ti == ROCK_BF8; // conv_direct.h: 4 pixel blocks per tile, else 7
-    const int64_t tile_px = wide_operands ? 128 : kDirectTilePixels;
-    const int64_t row_pitch = ((wi + 2 * pw) * cbytes + 1023) / 1024 * 1024; // whole 1 KiB load slabs
-    auto window_rows = [&](int64_t rows) { return rows + (y - 1) + (ho % rows ? y - 1 : 0); };
-    const int64_t tiles_n = ceil_div(k, 128);
-    auto tiles_of = [&](int64_t rows) { return (int64_t)ceil_div(n * ho, rows) * tiles_n * g; };
-    // rows per tile: the fewest rounds of blocks (two per CU), then the most rows
-    const int64_t per_round = 2 * (int64_t)kNumCU;
-    int64_t th = 0;
-    for (int64_t rows = std::min<int64_t>(ho, wo > 0 ? tile_px / wo : 0); rows >= 1; --rows) {
-      if (window_rows(rows) * row_pitch > kDirectWindowBytes)
-        continue;
-      if (th == 0 || ceil_div(tiles_of(rows), per_round) < ceil_div(tiles_of(th), per_round))
-        th = rows;
-    }
-    // the kernel sizes its window from the left / top padding alone: both sides must be equal
-    const bool direct_ok = fast && sh == 1 && sw == 1 && dh == 1 && dw == 1 && y * x > 1 &&
-                           ph_r == ph && pw_r == pw && k % 32 == 0 &&
-                           cbytes >= 128 && cbytes <= 1024 && (cbytes & (cbytes - 1)) == 0 &&
-                           th >= 1 && row_pitch <= 32 * 1024 && p.fil_cs == 1 && p.fil_xs == c && p.fil_ys == x * c;
-    const bool asked = requested_tile_is(o, kDirectTilePixels, 128);
-    // by itself: 16-bit types, tiles at least 85 % full in pixels and 75 % in channels, enough of them for every
-    // CU, no tile requested
-    const bool by_itself = direct_ok && bool_or(o, "window_resident", true) && (ti == ROCK_F16 || ti == ROCK_BF16) &&
-                           forced_tile(o).empty() && y * x >= 4 &&
-                           th * wo * 100 >= tile_px * 85 && tiles_of(th) >= per_round &&
-                           (k % 128 == 0 || k % 128 >= 96); // (a 64-channel layer leaves half the block's waves idle)
-    if (direct_ok && (asked || by_itself)) {
-      const int64_t kbytes = Kg * es;                         // a whole number of 128-byte K-steps
-      const int64_t rows_p = tiles_n * 128;                   // channels per group in F'
-      const int64_t f_bytes = align256(g * rows_p * kbytes);
+  if (!planned && fast) {
+    const WindowPlan w = window_plan(p, ti, ph_r == ph && pw_r == pw, o);
+    const bool rows_as_they_lie = p.fil_cs == 1 && p.fil_xs == c && p.fil_ys == x * c;
+    if (w.ok && rows_as_they_lie && (requested_tile_is(o, kDirectTilePixels, 128) || w.by_itself)) {
+      const int64_t kbytes = Kg * es; // a whole number of 128-byte K-steps
       const int ws = p.epi.residual_op ? 5 : 4;
       const int kid = (int)int_or(o, "kernel_id", 0);
       h->kernel_count = 2;
-      h->workspace_bytes = (size_t)f_bytes;
+      h->workspace_bytes = (size_t)w.filter_bytes;
       if (kid == 0) {
         const int64_t e = 16 / es;
-        const int64_t size[5] = {g, rows_p / 32, kbytes / 16, 32, e};
+        const int64_t size[5] = {g, w.tiles_n * 4, kbytes / 16, 32, e};
         const int64_t src_size[5] = {g, k / 32, kbytes / 16, 32, e};
         const int64_t stride[5] = {p.fil_gs, 32 * p.fil_ks, e, p.fil_ks, 1};
         if (!fill_relayout_handle(h, size, src_size, stride, es)) {
@@ -2746,24 +2817,13 @@ Handle *make_conv(const OptMap &o) {
           return nullptr;
         }
         h->kernel_count = 2;
-        h->workspace_bytes = (size_t)f_bytes;
+        h->workspace_bytes = (size_t)w.filter_bytes;
         h->caller_pointers = ws + 1;
         h->ptr_map = {{0, 0}, {ws, 0}};
         h->problem_key = "repack filter " + fl;
         return h;
       }
-      p.rows_per_tile = (int)th;
-      p.tiles_m = ceil_div(n * ho, th);
-      p.tiles_n = (int)tiles_n;
-      p.group_m = std::min(p.tiles_m, 8);
-      int64_t total = (int64_t)p.tiles_m * p.tiles_n * g;
-      p.xcd_remap = total >= 2 * kNumXCD ? 1 : 0;
-      h->block_size = 256;
-      h->grid_size = (uint32_t)total;
-      h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + "_direct224" + rich_suffix(p.epi, true, o);
-      char buf[96];
-      std::snprintf(buf, sizeof buf, "v2:224,128,8,224,32,%d,1,1,1", 16 / es);
-      h->perf_config = buf;
+      apply_window_plan(h, p, w, ti, o);
       h->caller_pointers = ws + 1;
       h->ptr_map = {{ws, 0}, {1, 0}, {2, 0}, {3, 0}, {p.epi.residual_op ? 4 : -1, 0}};
     }

@@ -69,3 +69,32 @@ def test_window_fits_its_share_of_lds(rock, shape):
     pitch = -(-((wi + 2 * pad) * c * 2) // 1024) * 1024
     window_rows = rows + y - 1 + (y - 1 if ho % rows else 0)     # tiles that straddle two images hold the padding rows between them
     assert window_rows * pitch <= 80 * 1024
+
+
+@pytest.mark.parametrize("fil_layout", ["gkyxc", "gkcyx"])
+def test_backward_data_filter_is_flipped_and_repacked_in_one_kernel(rock, fil_layout):
+    """Unit-stride input gradient of the 3x3 ResNet layer: a stride-1 convolution
+    of dY with the flipped, k <-> c swapped filter, on the window-resident
+    kernel; ONE conversion kernel writes that filter fragment-major."""
+    n, c, k, hw, y = 256, 128, 128, 28, 3
+    opts = ("--operation conv_bwd_data --arch gfx950 -t f16 --fil_layout %s --in_layout nhwgc --out_layout nhwgk"
+            " --batchsize %d --groupsize 1 --in_channels %d --out_channels %d --in_h %d --in_w %d --fil_h %d --fil_w %d"
+            " --padding_h 1 --padding_w 1" % (fil_layout, n, c, k, hw, hw, y, y))
+    first, second = rock.RockKernel(opts), rock.RockKernel(opts + " --kernel_id 1")
+    assert (first.kernel_count, first.kernel_name, second.kernel_name) == (2, "rock_relayout_b2",
+                                                                          "rock_conv_f16_direct224")
+    K = y * y * k
+    assert first.workspace_bytes == c * K * 2
+    W = np.arange(1, k * c * y * y + 1, dtype=np.float32).reshape(k, c, y, y)          # canonical k c y x
+    fil = np.ascontiguousarray(W.transpose(0, 2, 3, 1) if fil_layout == "gkyxc" else W).ravel()
+    ws = np.full(first.workspace_bytes // 2, np.nan, np.float32)
+    (s_src, s_off), (d_src, d_off) = _pointer_map(rock, first)
+    assert (s_src, d_src, d_off) == (0, 4, 0)
+    _replay_relayout(first.params(), fil, s_off // 2, ws, 0)
+    virt = W[:, :, ::-1, ::-1].transpose(1, 2, 3, 0).reshape(c, K)                    # rows c, reduction (t_h, t_w, k)
+    want = virt.reshape(c // 32, 32, K // 64, 8, 8).transpose(0, 2, 3, 1, 4)           # blk kt chunk row e
+    assert np.array_equal(ws, want.ravel())
+    assert [src for src, _ in _pointer_map(rock, second)] == [4, 2, 1, -1, -1]
+    # off the table's choice the phase keeps the implicit-GEMM kernel and its K-contiguous filter copy
+    plain = rock.RockKernel(opts + " --window_resident false --kernel_id 1")
+    assert plain.kernel_name == "rock_conv_f16_128x128_fast" and plain.kernel_count == 2

@@ -227,6 +227,8 @@ WINDOW_CASES = [
     (2, 1, 128, 160, 10, 33, 2, 2, (0, 0)),  # even filter, no padding, two tiles of output channels
     (1, 1, 512, 64, 6, 6, 5, 5, (2, 2)),     # 512-byte pixels, 5x5 filter
     (9, 1, 256, 128, 14, 14, 3, 3, (1, 1)),  # 14-wide images: 16-row budget, window-limited
+    (2, 1, 1024, 32, 8, 8, 3, 3, (1, 1)),    # 1024-byte pixels: 64 chunks per pixel, eight K-steps per tap
+    (3, 1, 128, 64, 12, 16, 1, 3, (0, 1)),   # one filter row: the window holds exactly the tile's rows
 ]
 
 

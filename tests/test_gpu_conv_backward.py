@@ -192,3 +192,21 @@ def test_conv_backward_resnet_block_real_values(rock, oracle, gpu, t):
     assert info["kernels"] == ["rock_conv_bwd_weight_%s_128x128" % t, "rock_reduce_splits"]
     ref, _, _ = oracle.conv_bwd_weight(iq, dyq, *NHWC, n, g, c, k, hi, wi, y, x, stride, pad, dil)
     check_float(to_f32(dw, t), ref, t)
+
+
+@pytest.mark.parametrize("layouts", [NHWC, ("gkcyx", "nhwgc", "nhwgk")], ids=["gkyxc", "gkcyx"])
+def test_conv_bwd_data_on_the_window_resident_kernel_exact(rock, oracle, gpu, layouts):
+    """The unit-stride input gradient of a full-size 3x3 layer (batch 128 of
+    ResNet50's 28x28 stage): the table puts it on the window-resident kernel,
+    behind ONE conversion that flips, swaps and repacks the filter.  Integer
+    data, bit for bit against the oracle and against the implicit-GEMM plan."""
+    case = (128, 1, 128, 128, 28, 28, 3, 3, (1, 1), (1, 1), (1, 1))
+    n, g, c, k, hi, wi, y, x, stride, pad, dil = case
+    (raw_f, fq), _, (raw_dy, dyq), ho, wo = _tensors(case, layouts, "f16", 79, integer=True)
+    info = {}
+    print("bwd data, window-resident", layouts, flush=True)
+    dx = rock.conv2d_bwd_data(to_gpu(raw_f, "f16", gpu), to_gpu(raw_dy, "f16", gpu), info=info, **_kw(case, layouts))
+    torch.cuda.synchronize()
+    assert info["kernels"] == ["rock_relayout_b2", "rock_conv_f16_direct224"]
+    ref, _, _ = oracle.conv_bwd_data(fq, dyq, *layouts, n, g, c, k, hi, wi, y, x, stride, pad, dil)
+    assert np.array_equal(to_f32(dx, "f16"), oracle.round_through(ref, CODE["f16"]))
