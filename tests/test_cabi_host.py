@@ -356,10 +356,13 @@ def test_backward_convolution_plans(rock):
     (rocmlir-lib.cpp:150-199): kernel lists, workspace, problem keys with the
     reference's direction codes (RockTuningImpl.cpp:759-772)."""
     bwd_data = CONV_RESNET.replace("--operation conv", "--operation conv_bwd_data")
-    ks = [rock.RockKernel(bwd_data + " --kernel_id %d" % i) for i in range(2)]
-    assert [k.kernel_name for k in ks] == ["rock_relayout_b2", "rock_conv_f16_128x128_fast"]
-    assert all(k.kernel_count == 2 and k.workspace_bytes == 128 * 128 * 9 * 2 and k.caller_pointers == 5 for k in ks)
-    assert "convfp16 -F 2 " in ks[1].problem_key
+    # (this unit-stride layer fills the window-resident kernel's tiles: the table takes it, "--window_resident false"
+    # keeps the implicit-GEMM kernel; either way one filter conversion and one contraction)
+    for switch, name in (("", "rock_conv_f16_direct224"), (" --window_resident false", "rock_conv_f16_128x128_fast")):
+        ks = [rock.RockKernel(bwd_data + switch + " --kernel_id %d" % i) for i in range(2)]
+        assert [k.kernel_name for k in ks] == ["rock_relayout_b2", name]
+        assert all(k.kernel_count == 2 and k.workspace_bytes == 128 * 128 * 9 * 2 and k.caller_pointers == 5 for k in ks)
+        assert "convfp16 -F 2 " in ks[1].problem_key
     # stride 2: one sub-filter conversion and one convolution per phase of the input grid
     s2 = bwd_data.replace("--conv_stride_h 1 --conv_stride_w 1", "--conv_stride_h 2 --conv_stride_w 2") \
                  .replace("--out_h 28 --out_w 28", "--out_h 14 --out_w 14")
