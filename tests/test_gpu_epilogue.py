@@ -169,12 +169,15 @@ NCHW = ("gkcyx", "ngchw", "ngkhw")
 
 @pytest.mark.parametrize("layouts", [NHWC, NCHW], ids=["nhwc", "nchw"])
 @pytest.mark.parametrize("t,od", [("f16", "f16"), ("f32", "f32"), ("i8", "i32"), ("i8", "f16")])
-@pytest.mark.parametrize("shape", [(4, 64, 64, 14, 14, 3, 1), (2, 32, 48, 9, 9, 1, 0), (2, 3, 16, 12, 12, 3, 1)],
-                         ids=["3x3", "1x1", "padded-channels"])
+@pytest.mark.parametrize("shape", [(4, 64, 64, 14, 14, 3, 1), (2, 32, 48, 9, 9, 1, 0), (2, 3, 16, 12, 12, 3, 1),
+                                   (3, 128, 96, 14, 16, 3, 1, "v2:224,128,8,224,32,8,1,1,1")],
+                         ids=["3x3", "1x1", "padded-channels", "window-resident"])
 def test_conv_bias_residual_relu_exact(rock, oracle, gpu, layouts, t, od, shape):
     """The ResNet block tail relu(conv + bias + shortcut), every layout route
-    (vector kernel, conversion plan, pointwise-as-GEMM falls back because of the bias)."""
-    n, c, k, hi, wi, y, pad = shape
+    (vector kernel, conversion plan, pointwise-as-GEMM falls back because of the bias,
+    the window-resident kernel behind its filter conversion)."""
+    n, c, k, hi, wi, y, pad = shape[:7]
+    perf = shape[7] if len(shape) > 7 else None
     fl, il, ol = layouts
     rng = np.random.default_rng(67)
     lim = 128 if t == "i8" else 3
@@ -196,7 +199,9 @@ def test_conv_bias_residual_relu_exact(rock, oracle, gpu, layouts, t, od, shape)
     out = rock.conv2d(to_gpu(raw_f, t, gpu), to_gpu(raw_i, t, gpu), fil_layout=fl, in_layout=il, out_layout=ol,
                       batchsize=n, in_channels=c, out_channels=k, in_h=hi, in_w=wi, fil_h=y, fil_w=y,
                       padding=(pad, pad), out_dtype=od, bias=bias_t, residual=to_gpu(raw_res, od, gpu), info=info,
-                      **kw)
+                      perf_config=perf, **kw)
+    if perf and layouts is NHWC:
+        assert info["kernels"][-1].startswith("rock_conv_%s_direct224" % t) and len(info["kernels"]) == 2
     acc, _, _ = oracle.conv_fwd(raw_f if t == "i8" else fq, raw_i if t == "i8" else iq, fl, il, ol, n, 1, c, k, hi, wi,
                                 y, y, (1, 1), (pad, pad), (1, 1))
     acc = np.asarray(acc, np.float64)
