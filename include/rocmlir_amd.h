@@ -93,8 +93,12 @@ typedef void *MiirHandle;
  * input window in LDS, behind a conversion of the filter), split_k (a GEMM with
  * few output tiles and a long reduction split over blocks, partial sums in the
  * workspace), fused (attention, above).  A single leading dash and "key=value"
- * are accepted as well.  Returns NULL on any parse, validation or support
- * failure, as the reference does. */
+ * are accepted as well.  rocmlir-gen's scheduling and instruction-set toggles
+ * (reverse_grid, mfma, wmma, dot, x2) are accepted and ignored; flags that
+ * would change the result and have no kernel here are refused: "store-method"
+ * other than set (pass the addend as "residual add"), "force-f8-types" other
+ * than arch / ocp.  Returns NULL on any parse, validation or support failure,
+ * as the reference does. */
 ROCMLIR_AMD_API MiirHandle miirCreateHandle(const char *options);
 
 /* Miir.h:56 -- number of kernels the operation needs (1 for most problems; 2

@@ -3256,6 +3256,23 @@ Handle *build_handle(const OptMap &o) {
     set_error("only gfx950 is supported (got '" + arch + "')");
     return nullptr;
   }
+  // Flags of rocmlir-gen that change what a kernel computes and that no kernel here implements are refused
+  // rather than ignored (its scheduling and instruction-set toggles -- reverse_grid, mfma, wmma, dot, x2 -- are
+  // ignored: they leave the results alone): an accumulating store (rocmlir-gen.cpp:295-331; pass the tensor
+  // as "-residual add" instead), and the non-OCP 8-bit float encodings (rocmlir-gen.cpp:772-785; gfx950's
+  // matrix cores take e4m3fn / e5m2).
+  {
+    const std::string store = str_or(o, "store-method", str_or(o, "store_method", "set"));
+    if (store != "set") {
+      set_error("store-method '" + store + "' is not built: outputs are overwritten (an addend goes in as -residual add)");
+      return nullptr;
+    }
+    const std::string f8 = str_or(o, "force-f8-types", str_or(o, "force_f8_types", "arch"));
+    if (f8 != "arch" && f8 != "ocp") {
+      set_error("force-f8-types '" + f8 + "': only the OCP encodings (e4m3fn, e5m2) have kernels on gfx950");
+      return nullptr;
+    }
+  }
   std::string op = str_or(o, "operation", "");
   Handle *h = nullptr;
   try {

@@ -118,6 +118,8 @@ def test_null_handle_behaviour(rock):
     "--operation transpose --arch gfx950",
     CONV_IMPLICIT + " --kernel_id 1",
     CONV_RESNET + " --kernel_id 2",
+    "-operation gemm -arch gfx950 -t f16 -g 1 -m 64 -n 64 -k 64 -store-method atomic_add",   # would change the result: refused, not ignored
+    "-operation gemm -arch gfx950 -t fp8 -g 1 -m 64 -n 64 -k 64 -force-f8-types fnuz",
 ])
 def test_bad_problems_give_null(rock, bad):
     lib = rock.load_library()
