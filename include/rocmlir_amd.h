@@ -94,7 +94,9 @@ typedef void *MiirHandle;
  * few output tiles and a long reduction split over blocks, partial sums in the
  * workspace), fused (attention, above).  A single leading dash and "key=value"
  * are accepted as well.  rocmlir-gen's scheduling and instruction-set toggles
- * (reverse_grid, mfma, wmma, dot, x2) are accepted and ignored; flags that
+ * (reverse_grid, mfma, wmma, dot, x2) are accepted and ignored, and so is
+ * kernel_name: the code objects are built ahead of time and their kernel
+ * symbols are fixed (rockamdGetKernelName tells the symbol to launch); flags that
  * would change the result and have no kernel here are refused: "store-method"
  * other than set (pass the addend as "residual add"), "force-f8-types" other
  * than arch / ocp.  Returns NULL on any parse, validation or support failure,
