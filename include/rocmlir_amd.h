@@ -89,7 +89,7 @@ typedef void *MiirHandle;
  * convolutions as a batched GEMM over the tensors as they lie),
  * bwd_weight_gemm (the filter gradient of a one-group convolution as one
  * K-major GEMM plus the reduction of its pixel splits), window_resident (a
- * 16-bit stride-1 convolution whose tiles fill on the kernel that keeps the
+ * 16-bit or int8 stride-1 convolution whose tiles fill on the kernel that keeps the
  * input window in LDS, behind a conversion of the filter), split_k (a GEMM with
  * few output tiles and a long reduction split over blocks, partial sums in the
  * workspace), fused (attention, above).  A single leading dash and "key=value"

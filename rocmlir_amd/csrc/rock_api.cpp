@@ -1099,9 +1099,9 @@ WindowPlan window_plan(const RockConvParams &p, int ti, bool equal_padding, cons
   w.ok = p.stride_h == 1 && p.stride_w == 1 && p.dil_h == 1 && p.dil_w == 1 && p.y * p.x > 1 && equal_padding &&
          p.k % 32 == 0 && cbytes >= 128 && cbytes <= 1024 && (cbytes & (cbytes - 1)) == 0 && w.rows >= 1 &&
          row_pitch <= 32 * 1024 && p.in_cs == 1;
-  // by itself: 16-bit types, tiles at least 85 % full in pixels and 75 % in channels, enough of them for every
-  // CU, no tile requested
-  w.by_itself = w.ok && bool_or(o, "window_resident", true) && (ti == ROCK_F16 || ti == ROCK_BF16) &&
+  // by itself: 16-bit types and int8 (measured: 1.13-1.3x), tiles at least 85 % full in pixels and 75 % in
+  // channels, enough of them for every CU, no tile requested
+  w.by_itself = w.ok && bool_or(o, "window_resident", true) && (ti == ROCK_F16 || ti == ROCK_BF16 || ti == ROCK_I8) &&
                 forced_tile(o).empty() && p.y * p.x >= 4 && w.rows * p.wo * 100 >= tile_px * 85 &&
                 tiles_of(w.rows) >= per_round &&
                 (p.k % 128 == 0 || p.k % 128 >= 96); // (a 64-channel layer leaves half the block's waves idle)
@@ -2794,7 +2794,7 @@ Handle *make_conv(const OptMap &o) {
   //   F'[g][32-channel block][K-step of 128 bytes][chunk 0..7][channel 0..31][16 B]
   // (every group padded with zero rows to whole 128-channel tiles), then the
   // contraction reads it with coalesced loads straight into registers.  Taken
-  // on request ("-perf_config v2:224,128,...") and, for the 16-bit types, by
+  // on request ("-perf_config v2:224,128,...") and, for the 16-bit types and int8, by
   // itself where its tiles fill (3x3 layers of 28- and 56-wide images: 1.2-1.3x
   // the implicit-GEMM kernel; "--window_resident false" declines); a request that cannot be met falls back to the
   // table like any other perf_config.
