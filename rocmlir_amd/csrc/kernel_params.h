@@ -115,8 +115,14 @@ struct RockConvBwdWeightParams : RockGemmParams {
 // padding): positions at or beyond src_size read as zero.
 enum RockRelayoutMode {
   RELAYOUT_TRANSPOSE = 0, // contiguous dimensions differ: tile_d x (1024/tile_d) tiles through LDS
-  RELAYOUT_COPY = 1,      // both contiguous along dimension 4: one 16-byte destination chunk per thread
-  RELAYOUT_TRANSPOSE_VEC = 2, // as TRANSPOSE with 128-byte tile rows and 16-byte accesses
+  RELAYOUT_COPY = 1,      // one 16-byte destination chunk (along dimension 4) per thread
+  RELAYOUT_TRANSPOSE_VEC = 2, // as TRANSPOSE with 16-byte accesses: tiles of tile_d x (AREA / tile_d), relayout_body.h
+};
+// Division of a block or chunk index (below 2^31) by a divisor fixed at plan
+// time: n / d == (n * mul) >> shift in 64-bit arithmetic, with
+// mul = ceil(2^shift / d) and shift = 31 + ceil(log2 d).
+struct RockFastDiv {
+  uint32_t mul, shift;
 };
 struct RockRelayoutParams {
   int64_t src_stride[5], dst_stride[5]; // in elements
@@ -124,7 +130,20 @@ struct RockRelayoutParams {
   int32_t src_size[5];
   int32_t src_fast, dst_fast; // dimension indices
   int32_t mode;               // RockRelayoutMode
-  int32_t tile_d;             // RELAYOUT_TRANSPOSE: tile extent along dst_fast (8, 16 or 32)
+  int32_t tile_d;             // tile extent along dst_fast (TRANSPOSE: 8, 16 or 32; TRANSPOSE_VEC: a power of two)
+  // the divisors of the kernel's index decoding, in the order it divides by them.
+  // TRANSPOSE, TRANSPOSE_VEC: tiles along src_fast, tiles along dst_fast, then the sizes of the other three
+  // dimensions from the last to the first.  COPY: blocks per (i0, i1) pair, size[1], chunks per run, size[3].
+  RockFastDiv div[5];
+  // TRANSPOSE, TRANSPOSE_VEC: the same description resolved for the kernel, which then indexes nothing by
+  // src_fast / dst_fast: the tiled dimensions (s = src_fast, d = dst_fast) and the other three from the last
+  // to the first
+  int64_t ss_s, ss_d, ds_s, ds_d;       // strides of the tiled dimensions in source / destination
+  int64_t outer_ss[3], outer_ds[3];
+  int32_t size_s, size_d, src_s, src_d; // destination extents and source extents of the tiled dimensions
+  int32_t outer_size[3], outer_src[3];
+  int32_t tiles_s, tiles_d;             // tiles along each
+  int32_t ts_shift, td_shift;           // log2 of the tile extents
 };
 
 // rock_relayout_pair_b{1,2,4}(src0, dst0, src1, dst1, p): two conversions in one

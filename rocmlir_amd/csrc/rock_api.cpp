@@ -803,6 +803,16 @@ Handle *make_gemm(const OptMap &o) {
   return h;
 }
 
+// n / d for n < 2^31 as a multiplication and a shift (Granlund and Montgomery, "Division by invariant integers
+// using multiplication", 1994, theorem 4.2 with 31-bit dividends): mul = ceil(2^(31 + l) / d), l = ceil(log2 d)
+RockFastDiv fast_div_of(int64_t d) {
+  int l = 0;
+  while (((int64_t)1 << l) < d)
+    ++l;
+  const unsigned __int128 pow = (unsigned __int128)1 << (31 + l);
+  return RockFastDiv{(uint32_t)((pow + (unsigned __int128)d - 1) / (unsigned __int128)d), (uint32_t)(31 + l)};
+}
+
 // Makes h a layout-conversion kernel: a 5-D tensor, dimensions listed in the
 // destination's order (the last one contiguous there, the destination dense
 // unless dst_stride says otherwise),
@@ -872,7 +882,12 @@ bool fill_relayout_handle(Handle *h, const int64_t size[5], const int64_t src_si
         r.src_fast = d;
   }
   int64_t blocks = 1;
-  if (r.src_fast == r.dst_fast) {
+  int tile_s_of_plan = 1;
+  // a destination run of one 16-byte chunk (a 3-channel image padded to 8):
+  // one thread per chunk gathers its elements wherever the source keeps them;
+  // consecutive threads take consecutive pixels
+  const bool one_chunk = (int64_t)r.size[4] * es == 16 && r.src_fast == 3;
+  if (r.src_fast == r.dst_fast || one_chunk) {
     // whole 16-byte chunks along the contiguous dimension (by construction of cp)
     r.mode = RELAYOUT_COPY;
     const int64_t chunks = (int64_t)r.size[2] * r.size[3] * (r.size[4] * es / 16);
@@ -882,12 +897,28 @@ bool fill_relayout_handle(Handle *h, const int64_t size[5], const int64_t src_si
     }
     blocks = (chunks + 255) / 256 * r.size[1] * r.size[0];
   } else {
-    // short channel runs: narrow tiles, element-wise; otherwise 128-byte
-    // tile rows with 16-byte accesses
-    const bool vec = r.size[r.dst_fast] > 16 && r.src_stride[r.src_fast] == 1;
+    // short channel runs: narrow tiles, element-wise; otherwise tiles with
+    // 16-byte accesses (relayout_body.h): 128-byte rows on both sides, reshaped
+    // when either dimension is shorter than that
+    const bool vec = r.size[r.dst_fast] > 16;
     r.mode = vec ? RELAYOUT_TRANSPOSE_VEC : RELAYOUT_TRANSPOSE;
-    r.tile_d = vec ? 128 / es : r.size[r.dst_fast] <= 8 ? 8 : r.size[r.dst_fast] <= 16 ? 16 : 32;
-    const int tile_s = vec ? 128 / es : 1024 / r.tile_d;
+    int tile_s;
+    if (vec) {
+      const int v = 16 / es, area = 256 * (es == 1 ? 4 : 2) * v, min_side = 2 * v;
+      auto pow2_at_least = [](int64_t n) { int q = 1; while (q < n) q *= 2; return q; };
+      int td = std::min(std::max(pow2_at_least(r.size[r.dst_fast]), min_side), 8 * v);
+      int ts = area / td;
+      if (r.size[r.src_fast] < ts) {
+        ts = std::max(pow2_at_least(r.size[r.src_fast]), min_side);
+        td = area / ts;
+      }
+      r.tile_d = td;
+      tile_s = ts;
+    } else {
+      r.tile_d = r.size[r.dst_fast] <= 8 ? 8 : r.size[r.dst_fast] <= 16 ? 16 : 32;
+      tile_s = 1024 / r.tile_d;
+    }
+    tile_s_of_plan = tile_s;
     for (int d = 0; d < 5; ++d) {
       if (d == r.src_fast)
         blocks *= (r.size[d] + tile_s - 1) / tile_s;
@@ -900,6 +931,42 @@ bool fill_relayout_handle(Handle *h, const int64_t size[5], const int64_t src_si
   if (blocks > INT32_MAX) {
     set_error("conv: tensor too large for the layout-conversion kernel");
     return false;
+  }
+  {
+    // the divisors of the kernel's index decoding, in its order (kernel_params.h)
+    int64_t divisor[5] = {1, 1, 1, 1, 1};
+    if (r.mode == RELAYOUT_COPY) {
+      const int64_t chunks4 = r.size[4] * es / 16;
+      divisor[0] = ((int64_t)r.size[2] * r.size[3] * chunks4 + 255) / 256;
+      divisor[1] = r.size[1];
+      divisor[2] = chunks4;
+      divisor[3] = r.size[3];
+    } else {
+      const int sf = r.src_fast, df = r.dst_fast;
+      r.ss_s = r.src_stride[sf]; r.ss_d = r.src_stride[df];
+      r.ds_s = r.dst_stride[sf]; r.ds_d = r.dst_stride[df];
+      r.size_s = r.size[sf]; r.size_d = r.size[df];
+      r.src_s = r.src_size[sf]; r.src_d = r.src_size[df];
+      r.tiles_s = (r.size[sf] + tile_s_of_plan - 1) / tile_s_of_plan;
+      r.tiles_d = (r.size[df] + r.tile_d - 1) / r.tile_d;
+      r.ts_shift = __builtin_ctz((unsigned)tile_s_of_plan);
+      r.td_shift = __builtin_ctz((unsigned)r.tile_d);
+      divisor[0] = r.tiles_s;
+      divisor[1] = r.tiles_d;
+      int n = 0;
+      for (int d = 4; d >= 0; --d) {
+        if (d == sf || d == df)
+          continue;
+        r.outer_size[n] = r.size[d];
+        r.outer_src[n] = r.src_size[d];
+        r.outer_ss[n] = r.src_stride[d];
+        r.outer_ds[n] = r.dst_stride[d];
+        divisor[2 + n] = r.size[d];
+        ++n;
+      }
+    }
+    for (int i = 0; i < 5; ++i)
+      r.div[i] = fast_div_of(divisor[i]);
   }
   h->op = OP_RELAYOUT;
   h->epi = nullptr;
@@ -3090,7 +3157,12 @@ int get_function(Handle *h, hipFunction_t *fn) {
 
 int launch_once(Handle *h, hipFunction_t fn, void *const *pointers, hipStream_t stream) {
   // argument buffer: the pointers, then the parameter block (8-byte aligned)
-  char buf[8 * 8 + 512];
+  constexpr size_t kMaxPointers = 8, kMaxParams = 1024;
+  char buf[kMaxPointers * 8 + kMaxParams];
+  if ((size_t)h->num_pointers > kMaxPointers || h->params.size() > kMaxParams) {
+    set_error("launch: kernel argument block larger than the launch buffer");
+    return (int)hipErrorInvalidValue;
+  }
   size_t off = 0;
   for (int i = 0; i < h->num_pointers; ++i, off += 8) {
     const void *ptr = h->ptr_map.empty()           ? pointers[i]

@@ -19,6 +19,12 @@ data, and is reported with the reference's FLOP formulas
 kernel for are listed with the library's error message, not skipped silently.
 
   python -m rocmlir_amd.perf_suite --op gemm --types f16,i8 FILE
+
+With --tune quick|full|exhaustive every problem is also run under each entry of
+its tuning space (what mlir/utils/performance/tuningRunner.py does over the
+same lists with rocmlir-tuning-driver): the line then carries the fastest
+perf_config, its kernel and time next to the built-in choice, and --table PATH
+saves the winners in the reference's tab-separated ".tuning" form.
 """
 import argparse
 import json
@@ -116,7 +122,7 @@ def conv_problem(line, t, layout, direction_flag=None):
     return opts, shapes, 2.0 * n * (c // g) * k * ho * wo * y * x
 
 
-def run_problem(rock, torch, dev, opts, shapes, flops, warmup, iters, warm_ms=0.0):
+def run_problem(rock, torch, dev, opts, shapes, flops, warmup, iters, warm_ms=0.0, tune_kind=None, table=None):
     try:
         prog = rock.RockProgram(opts)  # every kernel of the problem and its workspace
     except rock.RockError as e:
@@ -136,8 +142,14 @@ def run_problem(rock, torch, dev, opts, shapes, flops, warmup, iters, warm_ms=0.
     ms = prog.benchmark(*args, warmup=warmup, iters=iters)
     contraction = [k.kernel_name for k in prog.kernels if k.kernel_name.startswith(("rock_conv", "rock_gemm",
                                                                                      "rock_attention"))]
-    return {"status": "ok", "kernel": contraction[-1], "kernels": len(prog.kernels), "ms": round(ms, 5),
-            "tflops": round(flops / (ms * 1e-3) / 1e12, 2)}
+    res = {"status": "ok", "kernel": contraction[-1], "kernels": len(prog.kernels), "ms": round(ms, 5),
+           "tflops": round(flops / (ms * 1e-3) / 1e12, 2)}
+    if tune_kind:
+        from .tuning import tune
+        best = tune(prog, *args, table=table, warmup=warmup, iters=iters, kind=tune_kind)
+        res.update({"tuned_perf_config": best[0][0], "tuned_kernel": best[0][1], "tuned_ms": round(best[0][2], 5),
+                    "tuned_tflops": round(flops / (best[0][2] * 1e-3) / 1e12, 2), "candidates": len(best)})
+    return res
 
 
 def main(argv=None):
@@ -154,11 +166,18 @@ def main(argv=None):
                     help="keep the GPU busy with the problem for this long before timing it (clock ramp-up)")
     ap.add_argument("--max-bytes", type=float, default=8e9, help="skip problems whose tensors exceed this")
     ap.add_argument("--extra-options", default="", help="appended to every problem string (plan switches, a perf_config)")
+    ap.add_argument("--tune", choices=["quick", "full", "exhaustive"], default=None,
+                    help="also time every entry of each problem's tuning space and report the fastest")
+    ap.add_argument("--table", default=None, help="with --tune: save the winners as a .tuning table here")
     args = ap.parse_args(argv)
 
     import torch
     import rocmlir_amd as rock
     rock.load_library()
+    table = None
+    if args.tune and args.table:
+        from .tuning import TuningTable
+        table = TuningTable()
     dev = torch.device("cuda:0")
     lines = [l.strip() for l in open(args.file) if l.strip() and not l.lstrip().startswith("#")]
     seen = set()
@@ -185,10 +204,13 @@ def main(argv=None):
                 if nbytes > args.max_bytes:
                     print(json.dumps({"problem": opts, "status": "skipped", "bytes": nbytes}), flush=True)
                     continue
-                res = run_problem(rock, torch, dev, opts, shapes, flops, args.warmup, args.iters, args.warm_ms)
+                res = run_problem(rock, torch, dev, opts, shapes, flops, args.warmup, args.iters, args.warm_ms,
+                                  args.tune, table)
                 res["problem"] = opts
                 print(json.dumps(res), flush=True)
                 torch.cuda.empty_cache()
+    if table is not None:
+        table.save(args.table)
     return 0
 
 

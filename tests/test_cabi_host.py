@@ -229,9 +229,9 @@ def test_layout_conversion_pads_channel_runs_to_whole_chunks(rock):
     # n, h and w fold into one dimension; one thread per 16-byte chunk, 256 chunks a block
     assert ks[1].grid_size == -(-4 * 230 * 230 // 256)
     assert " -c 3 " in ks[2].problem_key
-    # NCHW with the same channels: h and w fold; transposing tiles of 8 channels x 128 pixels
+    # NCHW with the same channels: h and w fold; again one thread per pixel (one 16-byte chunk), 256 pixels a block
     k = rock.RockKernel(first.replace("NHWGC", "NGCHW") + " --kernel_id 1")
-    assert k.kernel_name == "rock_relayout_b2" and k.grid_size == -(-230 * 230 // 128) * 4
+    assert k.kernel_name == "rock_relayout_b2" and k.grid_size == -(-4 * 230 * 230 // 256)
     # 128 channels: 64 x 64 tiles of 16-bit elements over (channel, folded pixel)
     nchw = CONV_RESNET.replace("NHWGC", "NGCHW").replace("GNYXC", "GNCHW")
     k = rock.RockKernel(nchw + " --kernel_id 1")
