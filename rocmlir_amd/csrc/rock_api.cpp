@@ -2702,6 +2702,12 @@ Handle *make_conv(const OptMap &o) {
     p.fil_gs = fs[0]; p.fil_ks = fs[1]; p.fil_cs = fs[2]; p.fil_ys = fs[3]; p.fil_xs = fs[4];
     p.in_ns = is[0]; p.in_gs = is[1]; p.in_cs = is[2]; p.in_hs = is[3]; p.in_ws = is[4];
     p.out_ns = os[0]; p.out_gs = os[1]; p.out_ks = os[2]; p.out_hs = os[3]; p.out_ws = os[4];
+    // a filter dimension of one element is described by any stride: a 1x1 filter stored gkcyx is the
+    // channels-last filter as it lies and needs no conversion
+    if (x == 1 && p.fil_cs == 1)
+      p.fil_xs = c;
+    if (y == 1 && p.fil_cs == 1 && p.fil_xs == c)
+      p.fil_ys = x * c;
   }
   const int es = dtype_size(ti);
   auto al = [&](int64_t elems) { return (elems * es) % 16 == 0; };

@@ -202,13 +202,17 @@ def test_pointwise_nchw_convolution_is_a_k_major_gemm(rock):
     assert k.kernel_name.startswith("rock_gemm_f16_") and k.kernel_name.endswith("_fast_nn")
     assert (k.kernel_count, k.workspace_bytes, k.num_pointers, k.caller_pointers) == (1, 0, 5, 4)
     assert "convfp16" in k.problem_key and " -y 1 -x 1 " in k.problem_key
-    # anything the GEMM form cannot express converts instead
+    # anything the GEMM form cannot express converts the image instead; the 1x1 filter, whose gkcyx form is
+    # the channels-last one as it lies, is read in place
     for change in (("--conv_stride_h 1", "--conv_stride_h 2"), ("--padding_w 0", "--padding_w 1"),
                    ("--in_h 56 --in_w 56", "--in_h 7 --in_w 7"), ("--out_layout NGCHW", "--out_layout NHWGC")):
         k = rock.RockKernel(pw.replace(*change))
-        assert k.kernel_count == 3, change
-    assert rock.RockKernel(pw + " --bias true").kernel_count == 3
-    assert rock.RockKernel(pw + " --pointwise_as_gemm false").kernel_count == 3
+        assert k.kernel_count == 2, change
+    assert rock.RockKernel(pw + " --bias true").kernel_count == 2
+    assert rock.RockKernel(pw + " --pointwise_as_gemm false").kernel_count == 2
+    from tests.test_conv3d_plan import _pointer_map
+    conv = rock.RockKernel(pw + " --pointwise_as_gemm false --kernel_id 1")
+    assert conv.kernel_name.startswith("rock_conv_f16_") and _pointer_map(rock, conv)[0] == (0, 0)
 
 
 def test_layout_conversion_pads_channel_runs_to_whole_chunks(rock):
