@@ -130,10 +130,12 @@ struct RockRelayoutParams {
   int32_t src_size[5];
   int32_t src_fast, dst_fast; // dimension indices
   int32_t mode;               // RockRelayoutMode
-  int32_t tile_d;             // tile extent along dst_fast (TRANSPOSE: 8, 16 or 32; TRANSPOSE_VEC: a power of two)
+  int32_t tile_d;             // tile extent along dst_fast (TRANSPOSE: 8, 16 or 32; TRANSPOSE_VEC: a power of two);
+                              // COPY: positions of dimension 3 whose runs share one chunk (1: runs of whole chunks)
   // the divisors of the kernel's index decoding, in the order it divides by them.
   // TRANSPOSE, TRANSPOSE_VEC: tiles along src_fast, tiles along dst_fast, then the sizes of the other three
-  // dimensions from the last to the first.  COPY: blocks per (i0, i1) pair, size[1], chunks per run, size[3].
+  // dimensions from the last to the first.  COPY: blocks per (i0, i1) pair, size[1], chunks per run,
+  // chunk positions along dimension 3 (size[3] / tile_d).
   RockFastDiv div[5];
   // TRANSPOSE, TRANSPOSE_VEC: the same description resolved for the kernel, which then indexes nothing by
   // src_fast / dst_fast: the tiled dimensions (s = src_fast, d = dst_fast) and the other three from the last
@@ -170,6 +172,7 @@ struct RockReduceParams {
   int32_t size[4];
   int32_t splits;
   int32_t out_dtype; // RockDType: f32, f16 or bf16
+  int32_t valid[4];  // elements at or beyond valid[d] along dimension d are padding and are not written (0: none)
 };
 
 // rock_fold_depth(T, dst, p): last step of the input gradient of a convolution

@@ -250,19 +250,24 @@ RK_DEV void transpose_vec_phase(int phase, const T *src, T *dst, const RockRelay
   }
 }
 
-// RELAYOUT_COPY: the destination's runs along dimension 4 are whole 16-byte
-// chunks; a thread builds one chunk, reading zero beyond the source's extent
-// in any dimension.  Source and destination usually share their contiguous
-// dimension; when a run is a single chunk (a 3-channel image padded to one)
-// the source may be contiguous along another dimension, and consecutive
-// threads, which take consecutive chunks, still read consecutive addresses.
-// blockIdx.x enumerates groups of 256 chunks over the flattened dimensions
-// (2, 3, chunk), then dimensions 1 and 0.
+// RELAYOUT_COPY: a thread builds one 16-byte chunk of the destination, reading
+// zero beyond the source's extent in any dimension.  Either the destination's
+// runs along dimension 4 are whole chunks (tile_d == 1), or a run is a fraction
+// of a chunk (3 channels padded to 4 of 16 bits) and a chunk holds the runs of
+// tile_d consecutive positions of dimension 3, which the destination stores
+// back to back; size[3] is then a multiple of tile_d.  Source and destination
+// usually share their contiguous dimension; when not (an NCHW image whose
+// pixels become such runs), consecutive threads, which take consecutive
+// chunks, still read consecutive addresses.  blockIdx.x enumerates groups of
+// 256 chunks over the flattened dimensions (2, 3, chunk), then dimensions 1
+// and 0.
 template <typename T>
 RK_DEV void copy_thread(const T *src, T *dst, const RockRelayoutParams &p, unsigned block, int tid) {
   constexpr int EPC = 16 / (int)sizeof(T); // elements per chunk
-  const unsigned chunks4 = (unsigned)p.size[4] / EPC;
-  const unsigned inner = (unsigned)p.size[2] * (unsigned)p.size[3] * chunks4;
+  const int ppc = p.tile_d;                // positions of dimension 3 per chunk
+  const unsigned chunks4 = ppc > 1 ? 1u : (unsigned)p.size[4] / EPC;
+  const unsigned groups3 = (unsigned)p.size[3] / (unsigned)ppc;
+  const unsigned inner = (unsigned)p.size[2] * groups3 * chunks4;
   const unsigned per = (inner + 255) / 256;
   unsigned b = fast_div(block, p.div[0]);
   unsigned q = (block - b * per) * 256 + (unsigned)tid;
@@ -271,21 +276,30 @@ RK_DEV void copy_thread(const T *src, T *dst, const RockRelayoutParams &p, unsig
     return;
   unsigned r = fast_div(q, p.div[2]);
   const unsigned ch = q - r * chunks4;
-  const unsigned i2 = fast_div(r, p.div[3]), i3 = r - i2 * (unsigned)p.size[3];
+  const unsigned i2 = fast_div(r, p.div[3]), i3 = (r - i2 * groups3) * (unsigned)ppc;
   const int64_t so = (int64_t)i0 * p.src_stride[0] + (int64_t)i1 * p.src_stride[1] +
                      (int64_t)i2 * p.src_stride[2] + (int64_t)i3 * p.src_stride[3];
   const int64_t dof = (int64_t)i0 * p.dst_stride[0] + (int64_t)i1 * p.dst_stride[1] +
                       (int64_t)i2 * p.dst_stride[2] + (int64_t)i3 * p.dst_stride[3] + (int64_t)ch * EPC;
   const bool outer_in = i0 < (unsigned)p.src_size[0] && i1 < (unsigned)p.src_size[1] &&
-                        i2 < (unsigned)p.src_size[2] && i3 < (unsigned)p.src_size[3];
-  const int e0 = (int)ch * EPC, lim = outer_in ? p.src_size[4] : 0;
-  const int64_t ss = p.src_stride[4];
+                        i2 < (unsigned)p.src_size[2];
+  const int lim4 = outer_in ? p.src_size[4] : 0;
+  const int64_t ss3 = p.src_stride[3], ss4 = p.src_stride[4];
   union {
     T e[EPC];
     Bytes16 v;
   } u;
-  for (int j = 0; j < EPC; ++j)
-    u.e[j] = e0 + j < lim ? src[so + (int64_t)(e0 + j) * ss] : (T)0;
+  if (ppc > 1) {
+    const int run_shift = __builtin_ctz((unsigned)p.size[4]); // a run is a power of two of elements
+    for (int j = 0; j < EPC; ++j) {
+      const int pos = j >> run_shift, e = j & (p.size[4] - 1);
+      u.e[j] = (e < lim4 && (int)i3 + pos < p.src_size[3]) ? src[so + (int64_t)pos * ss3 + (int64_t)e * ss4] : (T)0;
+    }
+  } else {
+    const int e0 = (int)ch * EPC, lim = (int)i3 < p.src_size[3] ? lim4 : 0;
+    for (int j = 0; j < EPC; ++j)
+      u.e[j] = e0 + j < lim ? src[so + (int64_t)(e0 + j) * ss4] : (T)0;
+  }
   *(Bytes16 *)(dst + dof) = u.v;
 }
 

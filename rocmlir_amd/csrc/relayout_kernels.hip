@@ -82,15 +82,20 @@ extern "C" __global__ __launch_bounds__(256) void rock_reduce_splits(const float
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= total)
     return;
+  int64_t rem = i, off = 0;
+  bool padding = false;
+#pragma unroll
+  for (int d = 3; d >= 0; --d) {
+    const int64_t at = rem % p.size[d];
+    padding = padding || (p.valid[d] != 0 && at >= p.valid[d]);
+    off += at * p.dst_stride[d];
+    rem /= p.size[d];
+  }
+  if (padding)
+    return;
   float acc = 0.0f;
   for (int s = 0; s < p.splits; ++s)
     acc = acc + partials[(int64_t)s * p.split_stride + i];
-  int64_t rem = i, off = 0;
-#pragma unroll
-  for (int d = 3; d >= 0; --d) {
-    off += (rem % p.size[d]) * p.dst_stride[d];
-    rem /= p.size[d];
-  }
   if (p.out_dtype == ROCK_F32) {
     ((float *)dst)[off] = acc;
   } else if (p.out_dtype == ROCK_F16) {

@@ -872,7 +872,16 @@ bool fill_relayout_handle(Handle *h, const int64_t size[5], const int64_t src_si
           std::llabs(r.src_stride[d]) < std::llabs(r.src_stride[r.src_fast]))
         r.src_fast = d;
   }
-  if (r.src_fast == r.dst_fast && ((int64_t)r.size[4] * es) % 16 != 0) {
+  // runs along the shared contiguous dimension that are a power-of-two fraction of a 16-byte chunk, stored
+  // back to back along dimension 3 (3 channels padded to 4 of 16 bits): a chunk holds several of them
+  int positions_per_chunk = 1;
+  {
+    const int64_t run_bytes = (int64_t)r.size[4] * es;
+    if (run_bytes < 16 && 16 % run_bytes == 0 && r.dst_stride[3] == r.size[4] && r.size[3] % (16 / run_bytes) == 0 &&
+        (r.src_fast == 4 || r.src_fast == 3))
+      positions_per_chunk = (int)(16 / run_bytes);
+  }
+  if (positions_per_chunk == 1 && r.src_fast == r.dst_fast && ((int64_t)r.size[4] * es) % 16 != 0) {
     // runs along the shared contiguous dimension that are not whole 16-byte
     // chunks (an output with 12 f16 channels): element-wise tiles over that
     // dimension and the longest other one
@@ -887,10 +896,12 @@ bool fill_relayout_handle(Handle *h, const int64_t size[5], const int64_t src_si
   // one thread per chunk gathers its elements wherever the source keeps them;
   // consecutive threads take consecutive pixels
   const bool one_chunk = (int64_t)r.size[4] * es == 16 && r.src_fast == 3;
-  if (r.src_fast == r.dst_fast || one_chunk) {
-    // whole 16-byte chunks along the contiguous dimension (by construction of cp)
+  if (r.src_fast == r.dst_fast || one_chunk || positions_per_chunk > 1) {
+    // whole 16-byte chunks along the contiguous dimension (by construction of cp), or several runs a chunk
     r.mode = RELAYOUT_COPY;
-    const int64_t chunks = (int64_t)r.size[2] * r.size[3] * (r.size[4] * es / 16);
+    r.tile_d = positions_per_chunk;
+    const int64_t chunks = positions_per_chunk > 1 ? (int64_t)r.size[2] * (r.size[3] / positions_per_chunk)
+                                                   : (int64_t)r.size[2] * r.size[3] * (r.size[4] * es / 16);
     if (chunks > INT32_MAX) {
       set_error("conv: tensor too large for the layout-conversion kernel");
       return false;
@@ -936,11 +947,11 @@ bool fill_relayout_handle(Handle *h, const int64_t size[5], const int64_t src_si
     // the divisors of the kernel's index decoding, in its order (kernel_params.h)
     int64_t divisor[5] = {1, 1, 1, 1, 1};
     if (r.mode == RELAYOUT_COPY) {
-      const int64_t chunks4 = r.size[4] * es / 16;
-      divisor[0] = ((int64_t)r.size[2] * r.size[3] * chunks4 + 255) / 256;
+      const int64_t chunks4 = r.tile_d > 1 ? 1 : r.size[4] * es / 16, groups3 = r.size[3] / r.tile_d;
+      divisor[0] = ((int64_t)r.size[2] * groups3 * chunks4 + 255) / 256;
       divisor[1] = r.size[1];
       divisor[2] = chunks4;
-      divisor[3] = r.size[3];
+      divisor[3] = groups3;
     } else {
       const int sf = r.src_fast, df = r.dst_fast;
       r.ss_s = r.src_stride[sf]; r.ss_d = r.src_stride[df];
@@ -1579,6 +1590,125 @@ Handle *bwd_weight_over_channels_last_copies(const OptMap &o, const ConvProblem 
   return sub;
 }
 
+// Filter gradient of a convolution over images with a few channels (the
+// 3-channel first layer of a CNN), one group, no padding or dilation along w.
+// The input is copied channels-last with the channel run padded to a power of
+// two that divides a 16-byte chunk (3 -> 4 of 16 bits); a row of x filter taps
+// then reads x neighbouring pixels, one contiguous run, which is padded to
+// whole chunks.  The K-major GEMM of the channels-last route runs over that
+// view -- "channels" = the run, a filter one tap wide:
+//   dW'[k, (y, run)] = sum over pixels of dY[pixel, k] * X4[n, ho*sh + y*dh - ph, (wo*sw)*cpad + run]
+// The columns of a run beyond x taps (the next pixels, or the neighbouring
+// row or image at the end of a row) and the padded channels are outputs of
+// their own, which the reduction kernel leaves out when it adds up the
+// partial sums and writes the caller's layout.  nullptr with `applies` false
+// when the problem is not of this kind.
+Handle *bwd_weight_narrow_channels(const OptMap &o, const ConvProblem &cp, bool &applies) {
+  applies = false;
+  const int es = dtype_size(cp.ti);
+  const int kid = (int)int_or(o, "kernel_id", 0);
+  if (!(cp.g == 1 && (cp.ti == ROCK_F32 || cp.ti == ROCK_F16 || cp.ti == ROCK_BF16) && cp.y * cp.x > 1 &&
+        bool_or(o, "bwd_weight_gemm", true) && bool_or(o, "layout_conversion", true)))
+    return nullptr;
+  int64_t cpad = 1;
+  while (cpad < cp.c)
+    cpad *= 2;
+  const int64_t pix_bytes = cpad * es;
+  if ((cp.c * es) % 16 == 0 || pix_bytes > 16 || cp.pw != 0 || cp.dw != 1 || (cp.sw * pix_bytes) % 16 != 0 ||
+      (cp.wi * pix_bytes) % 16 != 0 || (cp.k * es) % 16 != 0)
+    return nullptr;
+  const int64_t run = (cp.x * pix_bytes + 15) / 16 * 16 / es; // elements of a row of taps, in whole chunks
+  const int64_t Ng = cp.y * run, P = cp.n * cp.ho * cp.wo;
+  const int64_t x_bytes = align256(cp.n * cp.hi * cp.wi * pix_bytes + run * es); // the last run reaches past the end
+  if (P > INT32_MAX || Ng > INT32_MAX || x_bytes >= ((int64_t)1 << 31))
+    return nullptr;
+  auto al = [&](int64_t elems) { return (elems * es) % 16 == 0; };
+  const bool dy_ok = cp.os[2] == 1 && cp.os[3] == cp.wo * cp.os[4] && cp.os[0] == cp.ho * cp.os[3] && al(cp.os[4]);
+  const int64_t dy_pix = dy_ok ? cp.os[4] : cp.k; // elements between neighbouring pixels of the gradient read
+  const Tile &tile = cp.k <= 64 ? kFastTiles[3] : kFastTiles[2]; // 64x64 or 128x128
+  const int64_t tiles = (int64_t)ceil_div(cp.k, tile.bm) * ceil_div(Ng, tile.bn);
+  const int64_t want = std::max<int64_t>(1, std::min<int64_t>(tile.blocks_per_cu * kNumCU / tiles, P / 256));
+  int64_t S = 1;
+  for (int64_t d = want; d >= 1; --d)
+    if (P % d == 0) {
+      S = d;
+      break;
+    }
+  const int64_t Ks = P / S;
+  if (Ks * dy_pix * es >= ((int64_t)1 << 31))
+    return nullptr;
+  applies = true;
+  const int64_t dy_bytes = dy_ok ? 0 : align256(P * cp.k * es);
+  const int64_t part_off = x_bytes + dy_bytes, part_bytes = align256(S * cp.k * Ng * 4);
+  const int pre = dy_ok ? 1 : 2, count = pre + 2;
+  if (kid < 0 || kid >= count) {
+    set_error("conv: kernel_id out of range");
+    return nullptr;
+  }
+  auto *h = new Handle;
+  if (kid < pre) {
+    const bool input = kid == 0;
+    // dimensions in the destination's order n, h, w, g, c
+    const int64_t size[5] = {cp.n, input ? cp.hi : cp.ho, input ? cp.wi : cp.wo, 1, input ? cpad : cp.k};
+    const int64_t src_size[5] = {size[0], size[1], size[2], 1, input ? cp.c : cp.k};
+    const int64_t *st = input ? cp.is : cp.os;
+    const int64_t stride[5] = {st[0], st[3], st[4], st[1], st[2]};
+    if (!fill_relayout_handle(h, size, src_size, stride, es)) {
+      delete h;
+      return nullptr;
+    }
+    h->ptr_map = {{input ? 1 : 2, 0}, {4, input ? 0 : x_bytes}};
+    h->problem_key = input ? "relayout input: channel runs padded to a fraction of a chunk" : "relayout output gradient";
+  } else if (kid == pre) {
+    RockConvBwdWeightParams bp;
+    std::memset(&bp, 0, sizeof bp);
+    bp.G = (int)S; bp.M = (int)cp.k; bp.N = (int)Ng; bp.K = (int)Ks;
+    bp.a_ms = 1; bp.a_ks = dy_pix; bp.a_gs = Ks * dy_pix;
+    bp.c_ms = Ng; bp.c_ns = 1; bp.c_gs = cp.k * Ng;
+    default_epilogue(bp.epi, ROCK_F32);
+    bp.in_pix_stride = cpad;
+    bp.c = (int)run; bp.hi = (int)cp.hi; bp.wi = (int)cp.wi; bp.ho = (int)cp.ho; bp.wo = (int)cp.wo;
+    bp.x = 1;
+    bp.stride_h = (int)cp.sh; bp.stride_w = (int)cp.sw; bp.pad_h = (int)cp.ph; bp.pad_w = 0;
+    bp.dil_h = (int)cp.dh; bp.dil_w = 1;
+    apply_tile_grid(tile, cp.k, Ng, (int)S, bp.tiles_m, bp.tiles_n, bp.group_m, bp.xcd_remap, h->block_size,
+                    h->grid_size);
+    h->op = OP_GEMM;
+    h->params.assign(sizeof bp, 0);
+    std::memcpy(h->params.data(), &bp, sizeof bp);
+    h->epi = &reinterpret_cast<RockConvBwdWeightParams *>(h->params.data())->epi;
+    h->kernel_name = std::string("rock_conv_bwd_weight_") + dtype_name(cp.ti) + (tile.bm == 64 ? "_64x64" : "_128x128");
+    h->num_pointers = 5;
+    h->perf_config = perf_string(tile, es, &o);
+    h->ptr_map = {dy_ok ? Handle::PtrSrc{2, 0} : Handle::PtrSrc{4, x_bytes}, {4, 0}, {4, part_off}, {-1, 0}, {-1, 0}};
+    h->problem_key = conv_problem_key(h, o, cp, 4);
+  } else {
+    RockReduceParams r;
+    std::memset(&r, 0, sizeof r);
+    r.split_stride = cp.k * Ng;
+    r.size[0] = (int)cp.k; r.size[1] = (int)cp.y; r.size[2] = (int)(run / cpad); r.size[3] = (int)cpad;
+    r.valid[2] = (int)cp.x; r.valid[3] = (int)cp.c;
+    r.dst_stride[0] = cp.fs[1]; r.dst_stride[1] = cp.fs[3]; r.dst_stride[2] = cp.fs[4]; r.dst_stride[3] = cp.fs[2];
+    r.splits = (int)S;
+    r.out_dtype = cp.ti;
+    h->op = OP_RELAYOUT;
+    h->epi = nullptr;
+    h->params.assign(sizeof r, 0);
+    std::memcpy(h->params.data(), &r, sizeof r);
+    h->kernel_name = "rock_reduce_splits";
+    h->block_size = 256;
+    h->grid_size = (uint32_t)((cp.k * Ng + 255) / 256);
+    h->num_pointers = 2;
+    h->perf_config = "";
+    h->ptr_map = {{4, part_off}, {0, 0}};
+    h->problem_key = "reduction of the split partial sums";
+  }
+  h->kernel_count = count;
+  h->workspace_bytes = (size_t)(part_off + part_bytes);
+  h->caller_pointers = 5;
+  return h;
+}
+
 Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
   // A strided 1x1 filter without padding touches one input pixel in
   // stride_h * stride_w.  A first kernel gathers those into the workspace
@@ -1769,6 +1899,12 @@ Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
   // kernel adds up in split order.  The reference lowers the same contraction
   // through its backward-weight coordinate transforms with atomic adds into a
   // zero-filled workspace (ConvToGemm.cpp:530-768).
+  {
+    bool applies = false;
+    Handle *via = bwd_weight_narrow_channels(o, cp, applies);
+    if (applies)
+      return via;
+  }
   if (cp.g == 1 && (cp.ti == ROCK_F32 || cp.ti == ROCK_F16 || cp.ti == ROCK_BF16) &&
       bool_or(o, "bwd_weight_gemm", true)) {
     auto al = [&](int64_t elems) { return (elems * es) % 16 == 0; };

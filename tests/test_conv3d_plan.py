@@ -275,8 +275,8 @@ def _replay_bwd_weight_gemm(params, dy, dy_off, xin, x_off, dst, d_off, es):
         im2col = np.where(ok, xin[np.where(ok, src, 0)], 0).astype(np.float64)
         ysrc = dy_off + pix[:, None] * a_ks + np.arange(M)[None, :] * a_ms
         assert ysrc.min() >= 0 and ysrc.max() < dy.size
+        # (columns that are padding may hold anything, NaN included: the reduction leaves them out)
         part = dy[ysrc].astype(np.float64).T @ im2col
-        assert not np.isnan(part).any()
         o = d_off + wide * (sp * c_gs + np.arange(M)[:, None] * c_ms + cols[None, :] * c_ns)
         assert o.min() >= 0 and o.max() + wide - 1 < dst.size
         dst[o] = part
@@ -289,16 +289,18 @@ def _replay_reduce(params, parts, p_off, dst, d_off, es):
     ds = struct.unpack_from("<4q", params, 8)
     size = struct.unpack_from("<4i", params, 40)
     splits, _ = struct.unpack_from("<2i", params, 56)
+    valid = [v or s for v, s in zip(struct.unpack_from("<4i", params, 64), size)]  # 0: the whole dimension
     total = int(np.prod(size))
     acc = np.zeros(total, np.float64)
     wide = 4 // es
     for sp in range(splits):
         acc += parts[p_off + wide * (sp * split_stride + np.arange(total))]
-    assert not np.isnan(acc).any()
     idx = np.indices(size).reshape(4, -1)
-    o = d_off + (idx * np.array(ds)[:, None]).sum(0)
+    keep = np.all(idx < np.array(valid)[:, None], axis=0)
+    assert not np.isnan(acc[keep]).any()
+    o = d_off + (idx * np.array(ds)[:, None]).sum(0)[keep]
     assert o.min() >= 0 and o.max() < dst.size and len(np.unique(o)) == o.size
-    dst[o] = acc
+    dst[o] = acc[keep]
 
 
 BWD_CASES = [

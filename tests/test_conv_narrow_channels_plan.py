@@ -1,0 +1,65 @@
+"""Filter gradient of convolutions over images with a few channels (the
+3-channel first layer of a CNN): the plan -- a channels-last copy with the
+channel run padded to a fraction of a 16-byte chunk, the K-major GEMM over
+rows of filter taps read as one run, the reduction that leaves the padding
+columns out -- replayed kernel by kernel in numpy from the parameter blocks and
+pointer maps the C ABI hands out, against the CPU oracle.  The workspace
+starts as NaN, so a kernel that used a byte no earlier kernel wrote, outside
+the padding columns, would show."""
+import numpy as np
+import pytest
+
+from oracle import rock_oracle as orc
+from tests.test_conv3d_plan import _replay_plan
+from tests.test_relayout_host import conv
+
+# (n c k hi wi y x stride pad_h) -- no padding along w, even image width
+CASES = [
+    (2, 3, 16, 20, 20, 7, 7, 2, 0),    # the ResNet first layer in small
+    (3, 3, 64, 15, 18, 3, 3, 2, 1),    # rows padded at the top and bottom
+    (2, 4, 24, 12, 16, 5, 3, 2, 2),    # four channels: no channel padding, rows of 3 taps
+    (2, 2, 8, 9, 16, 3, 5, 4, 0),      # two channels (a quarter of a chunk), stride 4
+    (1, 1, 8, 10, 24, 3, 3, 8, 1),     # one channel
+]
+
+
+def _options(case, il, fl, t):
+    n, c, k, hi, wi, y, x, s, ph = case
+    ho = (hi + 2 * ph - y) // s + 1
+    wo = (wi - x) // s + 1
+    return (conv(t, il, fl, n, c, hi, wi, k, y, x, stride=s, op="conv_bwd_weight")
+            .replace("--padding_h 0", "--padding_h %d" % ph).replace("--out_h %d" % ((hi - y) // s + 1), "--out_h %d" % ho)), ho, wo
+
+
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("il,fl", [("nhwgc", "gkyxc"), ("ngchw", "gkcyx"), ("nhwgc", "gkcyx")])
+@pytest.mark.parametrize("t,es", [("fp16", 2), ("f32", 4)])
+def test_narrow_channel_filter_gradient_plan_replayed_on_the_cpu(rock, case, il, fl, t, es):
+    n, c, k, hi, wi, y, x, s, ph = case
+    if es == 4 and c == 4:
+        pytest.skip("four 32-bit channels are a whole chunk: the channels-last route takes it")
+    opts, ho, wo = _options(case, il, fl, t)
+    ol = il.replace("c", "k")
+    rng = np.random.default_rng(11)
+    inp = rng.integers(-3, 4, n * c * hi * wi).astype(np.float32)
+    dout = rng.integers(-3, 4, n * k * ho * wo).astype(np.float32)
+    want, _, _ = orc.conv_bwd_weight(inp, dout, fl, il, ol, n, 1, c, k, hi, wi, y, x, (s, s), (ph, 0), (1, 1))
+    first = rock.RockKernel(opts)
+    dw = np.full(want.size, np.nan, np.float32)
+    ws = np.full(first.workspace_bytes // es, np.nan, np.float32)
+    tn = {"fp16": "f16"}.get(t, t)
+    names = _replay_plan(rock, opts, [dw, inp, dout, None, ws], tn, es)
+    assert np.array_equal(dw, want.ravel())
+    copies = 1 if il == "nhwgc" else 2
+    assert names == ["rock_relayout_b%d" % es] * copies + ["rock_conv_bwd_weight_%s_64x64" % tn, "rock_reduce_splits"]
+
+
+def test_narrow_channel_route_conditions(rock):
+    """Padding or dilation along w, an odd image width, or a switch decline the route."""
+    base, _, _ = _options(CASES[0], "nhwgc", "gkyxc", "fp16")
+    names = lambda o: [rock.RockKernel(o + " --kernel_id %d" % i).kernel_name for i in range(rock.RockKernel(o).kernel_count)]
+    assert names(base)[-2:] == ["rock_conv_bwd_weight_f16_64x64", "rock_reduce_splits"]
+    for change in (("--padding_w 0", "--padding_w 1 --out_w 8"), ("--in_w 20 --out_h 7 --out_w 7", "--in_w 21 --out_h 7 --out_w 8"),
+                   ("--dilation_w 1", "--dilation_w 2 --out_w 4")):
+        assert not any(nm.startswith("rock_conv_bwd_weight_") for nm in names(base.replace(*change))), change
+    assert not any(nm.startswith("rock_conv_bwd_weight_") for nm in names(base + " --bwd_weight_gemm false"))

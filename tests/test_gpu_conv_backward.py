@@ -210,3 +210,36 @@ def test_conv_bwd_data_on_the_window_resident_kernel_exact(rock, oracle, gpu, la
     assert info["kernels"] == ["rock_relayout_b2", "rock_conv_f16_direct224"]
     ref, _, _ = oracle.conv_bwd_data(fq, dyq, *layouts, n, g, c, k, hi, wi, y, x, stride, pad, dil)
     assert np.array_equal(to_f32(dx, "f16"), oracle.round_through(ref, CODE["f16"]))
+
+
+NARROW_CASES = [
+    (8, 1, 3, 64, 38, 38, 7, 7, (2, 2), (0, 0), (1, 1)),      # the ResNet first layer in small, pixels split
+    (2, 1, 3, 16, 20, 20, 7, 7, (2, 2), (0, 0), (1, 1)),
+    (3, 1, 3, 136, 15, 18, 3, 3, (2, 2), (1, 0), (1, 1)),     # rows padded at the top and bottom, 128x128 tiles
+    (2, 1, 4, 24, 12, 16, 5, 3, (2, 2), (2, 0), (1, 1)),      # four channels
+    (2, 1, 2, 8, 9, 16, 3, 5, (3, 4), (0, 0), (2, 1)),        # two channels, stride 4 along w, dilated rows
+    (1, 1, 1, 8, 10, 24, 3, 3, (1, 8), (1, 0), (1, 1)),       # one channel
+]
+
+
+@pytest.mark.parametrize("case", NARROW_CASES)
+@pytest.mark.parametrize("layouts", [NHWC, NCHW], ids=lambda l: l[1])
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16"])
+def test_conv_bwd_weight_over_a_few_channels_exact(rock, oracle, gpu, case, layouts, t):
+    """Images with a few channels: channels-last copy with the channel run padded to a fraction of a chunk,
+    rows of filter taps read as one run by the K-major GEMM, padding columns left out by the reduction."""
+    n, g, c, k, hi, wi, y, x, stride, pad, dil = case
+    _, (raw_i, iq), (raw_dy, dyq), ho, wo = _tensors(case, layouts, t, 83)
+    info, info_old = {}, {}
+    xi, dy = to_gpu(raw_i, t, gpu), to_gpu(raw_dy, t, gpu)
+    got = rock.conv2d_bwd_weight(xi, dy, info=info, **_kw(case, layouts))
+    old = rock.conv2d_bwd_weight(xi, dy, info=info_old, as_gemm=False, **_kw(case, layouts))
+    torch.cuda.synchronize()
+    if not (t == "f32" and c == 4):
+        assert info["kernels"][-2:] == ["rock_conv_bwd_weight_%s_%s" % (t, "64x64" if k <= 64 else "128x128"),
+                                        "rock_reduce_splits"]
+        assert info["kernels"][0].startswith("rock_relayout_b")
+    assert not any(name.startswith("rock_conv_bwd_weight_") for name in info_old["kernels"])
+    ref, _, _ = oracle.conv_bwd_weight(iq, dyq, *layouts, n, g, c, k, hi, wi, y, x, stride, pad, dil)
+    assert np.array_equal(to_f32(got, t), oracle.round_through(ref, CODE[t]))
+    assert torch.equal(got.view(torch.uint8), old.view(torch.uint8))

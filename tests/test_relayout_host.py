@@ -73,6 +73,13 @@ PROBLEMS = [
     # backward weight through channels-last copies, and the filter gradient written back as gkcyx
     conv("fp16", "ngchw", "gkcyx", 4, 32, 10, 10, 32, 3, 3, pad=1, op="conv_bwd_weight"),
     conv("f32", "ngchw", "gkcyx", 4, 16, 8, 8, 32, 3, 3, pad=1, op="conv_bwd_weight"),
+    # filter gradient over a few channels: 3 -> 4 channels of 16 bits, two pixels a chunk (NHWC and NCHW sources);
+    # 2 and 1 channels; 32-bit elements
+    conv("fp16", "nhwgc", "gkyxc", 2, 3, 20, 20, 16, 7, 7, stride=2, op="conv_bwd_weight"),
+    conv("fp16", "ngchw", "gkcyx", 2, 3, 20, 20, 16, 7, 7, stride=2, op="conv_bwd_weight"),
+    conv("bf16", "nhwgc", "gkyxc", 2, 2, 9, 16, 8, 3, 5, stride=4, op="conv_bwd_weight"),
+    conv("fp16", "ngchw", "gkcyx", 1, 1, 10, 24, 8, 3, 3, stride=8, op="conv_bwd_weight"),
+    conv("f32", "ngchw", "gkcyx", 2, 2, 9, 16, 8, 3, 5, stride=4, op="conv_bwd_weight"),
     # the window-resident kernel's fragment-major filter
     conv("fp16", "nhwgc", "gkyxc", 8, 128, 28, 28, 128, 3, 3, pad=1, extra="--perf_config v2:224,128,8,224,32,8,1,1,1"),
     # ragged GEMM operands copied into padded rows (two conversions in one launch)
@@ -156,6 +163,10 @@ def test_modes_chosen(rock):
     # 14 x 14 images of 256 channels: 64 x 64 tiles
     size, (sf, df, mode, td) = params_of(conv("fp16", "ngchw", "gkcyx", 2, 256, 14, 14, 256, 3, 3, pad=1), 1)
     assert size[-2:] == (196, 256) and (mode, td) == (2, 64)
+    # 3 -> 4 channels of 16 bits: two pixels a chunk
+    size, (sf, df, mode, ppc) = params_of(conv("fp16", "ngchw", "gkcyx", 2, 3, 20, 20, 16, 7, 7, stride=2,
+                                               op="conv_bwd_weight"), 0)
+    assert size[-2:] == (400, 4) and (mode, ppc) == (1, 2)
     # every other pixel of every other row: vector tiles with element-wise reads (the 1x1 filter needs no kernel)
     size, (sf, df, mode, td) = params_of(conv("fp16", "ngchw", "gkcyx", 2, 64, 14, 14, 128, 1, 1, stride=2), 0)
     assert size[-2:] == (7, 64) and (mode, td) == (2, 256)
