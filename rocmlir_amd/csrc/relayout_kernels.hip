@@ -93,8 +93,19 @@ extern "C" __global__ __launch_bounds__(256) void rock_reduce_splits(const float
   }
   if (padding)
     return;
+  // summed in split order; sixteen loads are in flight at a time, the additions stay sequential
   float acc = 0.0f;
-  for (int s = 0; s < p.splits; ++s)
+  int s = 0;
+  for (; s + 16 <= p.splits; s += 16) {
+    float v[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+      v[j] = partials[(int64_t)(s + j) * p.split_stride + i];
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+      acc = acc + v[j];
+  }
+  for (; s < p.splits; ++s)
     acc = acc + partials[(int64_t)s * p.split_stride + i];
   if (p.out_dtype == ROCK_F32) {
     ((float *)dst)[off] = acc;
