@@ -74,6 +74,10 @@ def contraction_kernels(type_code):
                 name = tile + "_fast" + e
                 out.append(("rock_conv_%s%s" % (t, name), "RK_CONV_DL(%s, %d, %d, %d, %d, 128, %s)"
                             % (name, bm, bn, wm, wn, "true" if rich else "false")))
+        if t != "f32":   # rows of taps over narrow pixels (32-bit pixels of 4 channels are whole chunks)
+            for rich, e in ((False, ""), (True, "_e")):
+                out.append(("rock_conv_%s_64x64_fast_runs%s" % (t, e),
+                            "RK_CONV_DL_RUNS(_64x64_fast_runs%s, 64, 64, 2, 2, 128, %s)" % (e, "true" if rich else "false")))
         out.append(("rock_conv_%s_64x64_generic" % t,
                     "RK_CONV(_64x64_generic, 64, 64, 2, 2, rk::LD_CONV_IN_GENERIC, rk::LD_CONV_FIL_GENERIC)"))
         if t in ("f32", "f16", "bf16"):   # filter gradient as one K-major GEMM over the tensors as they lie

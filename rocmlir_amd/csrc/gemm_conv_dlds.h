@@ -121,7 +121,14 @@ template <int DT, int ROWS, int NW, int RB> struct RowsDl {
 // of a K-step sits in the same filter tap: the tap walk is scalar state, the
 // per-lane work of a step is one add, and the (hi, wi) bounds test runs once
 // per tap.  Otherwise each lane tracks the tap of its own chunk.
-template <int DT, int ROWS, int NW, int RB> struct ConvInDl {
+//
+// RUNS: the last chunk of a channel run holds run_valid % EPC elements of data
+// and, behind them, whatever follows in memory.  Every lane remembers, per
+// stage in flight, which of its chunks are such tails (`tails`), and clears the
+// bytes behind the data in LDS once its loads of that stage have landed
+// (zero_tails, between the wait for the stage and the barrier that hands it to
+// the readers), so that nothing but data reaches the MFMAs.
+template <int DT, int ROWS, int NW, int RB, bool RUNS = false> struct ConvInDl {
   using Sg = SlabGeom<ROWS, NW, RB>;
   using Dg = DlGeom<RB>;
   static constexpr int ES = MmaTraits<DT>::ES;
@@ -143,12 +150,17 @@ template <int DT, int ROWS, int NW, int RB> struct ConvInDl {
   int step_y, step_x, step_c;
   bool padded; // some window reaches outside the image
   int wave;
+  unsigned tails;  // RUNS: bit (stage slot * PER_WAVE + i) set: chunk i of that stage is the tail of a run
+  int run_valid;
+  static_assert(!RUNS || DlGeom<RB>::STAGES * Sg::PER_WAVE <= 32, "one bit per chunk in flight");
 
   __device__ __forceinline__ void init(const void *in, const RockConvParams &cp, int g, int row0,
                                        int wave_, int lane) {
     p = &cp;
     wave = wave_;
-    uniform = (cp.c * ES) % RB == 0;
+    uniform = !RUNS && (cp.c * ES) % RB == 0;
+    tails = 0;
+    run_valid = cp.run_valid;
     uy = ux = uc0 = 0;
     {
       const int taps = BKE / cp.c;
@@ -183,6 +195,23 @@ template <int DT, int ROWS, int NW, int RB> struct ConvInDl {
     }
   }
   // must be called with kt = 0, 1, 2, ... in order (tap state advances)
+  // RUNS: clears what lies behind the data in this lane's tail chunks of K-step kt (their loads have landed)
+  __device__ __forceinline__ void zero_tails(int kt, char *stage) {
+    if constexpr (RUNS) {
+      typedef __attribute__((address_space(3))) int lds_int_t;
+      const int valid_dwords = ((run_valid % EPC) * ES) >> 2;
+#pragma unroll
+      for (int i = 0; i < Sg::PER_WAVE; ++i) {
+        if (tails & (1u << ((kt % DlGeom<RB>::STAGES) * Sg::PER_WAVE + i))) {
+          lds_int_t *q = (lds_int_t *)(stage + (wave * Sg::PER_WAVE + i) * 1024 + (threadIdx.x & 63) * 16);
+#pragma unroll
+          for (int d = 1; d < 4; ++d)
+            if (d >= valid_dwords)
+              q[d] = 0;
+        }
+      }
+    }
+  }
   __device__ __forceinline__ void issue(int kt, char *stage) {
     (void)kt;
     if (uniform) {
@@ -221,6 +250,10 @@ template <int DT, int ROWS, int NW, int RB> struct ConvInDl {
                         : kOobOffset;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
           rsrc, (lds_void_t *)(stage + (wave * Sg::PER_WAVE + i) * 1024), 16, (int)voff, 0, 0, 0);
+      if constexpr (RUNS) {
+        const unsigned bit = 1u << ((kt % DlGeom<RB>::STAGES) * Sg::PER_WAVE + i);
+        tails = (v && cc[i] + EPC > run_valid) ? (tails | bit) : (tails & ~bit);
+      }
       cc[i] += step_c;
       const int carry = cc[i] >= p->c ? 1 : 0;
       cc[i] -= carry ? p->c : 0;
@@ -468,8 +501,9 @@ __device__ __forceinline__ auto make_dl_b(const void *in, const RockConvBwdWeigh
 }
 template <int DT, int ROWS, int NW, int RB, int KIND>
 __device__ __forceinline__ auto make_dl_a(const void *in, const RockConvParams &p, int g, int m0, int wave, int lane) {
-  static_assert(KIND == LD_CONV_IN_FAST, "convolution fast path gathers channel-contiguous input");
-  ConvInDl<DT, ROWS, NW, RB> l;
+  static_assert(KIND == LD_CONV_IN_FAST || KIND == LD_CONV_IN_RUNS,
+                "convolution fast path gathers channel-contiguous input");
+  ConvInDl<DT, ROWS, NW, RB, KIND == LD_CONV_IN_RUNS> l;
   l.init(in, p, g, m0, wave, lane);
   return l;
 }
@@ -1003,6 +1037,11 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
     }
     // this wave's loads of K-step kt have landed (two younger steps may be in flight) ...
     wait_vmcnt_and_lds_reads<(kDlStages - 2) * LOADS_PER_STEP>();
+    if constexpr (LDA == LD_CONV_IN_RUNS) {
+      if (loader)
+        la.zero_tails(kt, const_cast<char *>(sa));
+      __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): the clearing stores are in LDS before the barrier
+    }
     // ... and so have everyone else's; everyone is also done reading step kt-1
     __builtin_amdgcn_s_barrier();
     if (loader) {

@@ -48,6 +48,14 @@
         in, fil, out, aux, res, p);                                                                   \
   }
 
+// channel runs whose last chunk holds bytes that are not data (rows of filter taps over narrow pixels)
+#define RK_CONV_DL_RUNS(NAME, BM, BN, WM, WN, RB, RICH)                                               \
+  extern "C" __global__ __launch_bounds__(WM *WN * 64) void RK_CONV_NAME(NAME)(                       \
+      const void *fil, const void *in, void *out, const void *aux, const void *res, RockConvParams p) { \
+    rk::contraction_body_dl<ROCK_DT, BM, BN, WM, WN, RB, rk::LD_CONV_IN_RUNS, rk::LD_ROWS_FAST, RICH>( \
+        in, fil, out, aux, res, p);                                                                   \
+  }
+
 // small outputs: 32x32 tile per block, K split over the block's four waves
 #define RK_GEMM_SPLITK(NAME, RICH)                                                                    \
   extern "C" __global__ __launch_bounds__(256) void RK_GEMM_NAME(NAME)(                               \

@@ -36,7 +36,8 @@ enum LoaderKind : int {
   LD_CONV_IN_GENERIC = 3,
   LD_CONV_FIL_GENERIC = 4,
   LD_COLS_FAST = 5,     // GEMM operand stored K-major (its M or N index contiguous), 16-byte aligned chunks
-  LD_CONV_COLS = 6      // forward im2col matrix as a K-major operand (reduction over pixels): filter gradient
+  LD_CONV_COLS = 6,     // forward im2col matrix as a K-major operand (reduction over pixels): filter gradient
+  LD_CONV_IN_RUNS = 7   // as LD_CONV_IN_FAST over channel runs whose last chunk holds bytes that are not data
 };
 
 constexpr int kChunk = 16;       // bytes

@@ -89,6 +89,11 @@ struct RockConvParams {
   int32_t k_order_yxc; // 1: reduction index runs (y,x,c) with c fastest; 0: (c,y,x)
   int32_t rows_per_tile; // window-resident kernel: output rows (n, ho) per block; else 0
   RockEpilogue epi;
+  // Kernels named "_runs": a channel run of c elements is a row of filter taps over neighbouring narrow pixels
+  // padded to whole 16-byte chunks; its first run_valid elements are data, what the load brings along behind
+  // them (the next pixel) is cleared in LDS before it is multiplied.  0 elsewhere.
+  int32_t run_valid;
+  int32_t pad_;
 };
 
 // Filter gradient of a convolution as one K-major GEMM over the tensors as they

@@ -2896,6 +2896,67 @@ Handle *make_conv(const OptMap &o) {
     }
   }
 
+  // Narrow pixels (the 3-channel first layer of a CNN), one group, no padding or
+  // dilation along w.  Both tensors are copied channels-last with the channel
+  // run padded to a power of two that divides a 16-byte chunk (3 -> 4 of 16
+  // bits, 3 -> 8 of 8 bits); a row of x filter taps then reads x neighbouring
+  // pixels, one contiguous run, padded to whole chunks, and the contraction
+  // sees "channels" = that run under a filter one tap wide: K = y * run in
+  // place of y * x * (c padded to a whole chunk).  The last chunk of a run
+  // brings the next pixel along; the "_runs" kernels clear it in LDS (the
+  // filter holds zeros there, but zero times an Inf in that pixel would not be
+  // zero).  Every window must start on a chunk boundary: stride_w pixels and an
+  // image row are whole chunks.
+  bool runs_kernel = false;
+  if (!fast && g == 1 && pw == 0 && pw_r == 0 && dw == 1 && y * x > 1 && ti != ROCK_F32 &&
+      bool_or(o, "layout_conversion", true) && bool_or(o, "tap_rows", true)) {
+    int64_t cpad = 1;
+    while (cpad < c || cpad * es < 4)
+      cpad *= 2;
+    while ((sw * cpad * es) % 16 != 0 && cpad * es < 16)
+      cpad *= 2;
+    const int64_t pix_bytes = cpad * es;
+    const int64_t run = (x * pix_bytes + 15) / 16 * 16 / es; // elements of a row of taps, in whole chunks
+    const int64_t in_bytes = align256(n * hi * wi * pix_bytes + run * es); // the last run reaches past the end
+    const int64_t fil_bytes = align256(k * y * run * es);
+    if ((c * es) % 16 != 0 && pix_bytes < 16 && (sw * pix_bytes) % 16 == 0 && (wi * pix_bytes) % 16 == 0 &&
+        in_bytes < ((int64_t)1 << 31) && (256 * y * run + run) * es < ((int64_t)1 << 31) && y * run <= INT32_MAX) {
+      const int ws = p.epi.residual_op ? 5 : 4;
+      h->kernel_count = 3;
+      h->workspace_bytes = (size_t)(fil_bytes + in_bytes);
+      h->caller_pointers = ws + 1;
+      planned = true;
+      const int kid = (int)int_or(o, "kernel_id", 0);
+      if (kid == 0 || kid == 1) {
+        const bool is_f = kid == 0;
+        // dimensions in destination order: g k y x c ; n h w g c
+        const int64_t size_f[5] = {1, k, y, run / cpad, cpad}, from_f[5] = {1, k, y, x, c};
+        const int64_t stride_f[5] = {p.fil_gs, p.fil_ks, p.fil_ys, p.fil_xs, p.fil_cs};
+        const int64_t size_i[5] = {n, hi, wi, 1, cpad}, from_i[5] = {n, hi, wi, 1, c};
+        const int64_t stride_i[5] = {p.in_ns, p.in_hs, p.in_ws, p.in_gs, p.in_cs};
+        const int callers = h->caller_pointers;
+        if (!fill_relayout_handle(h, is_f ? size_f : size_i, is_f ? from_f : from_i, is_f ? stride_f : stride_i, es)) {
+          delete h;
+          return nullptr;
+        }
+        h->caller_pointers = callers;
+        h->ptr_map = {{is_f ? 0 : 1, 0}, {ws, is_f ? 0 : fil_bytes}};
+        h->problem_key = std::string("relayout ") + (is_f ? "filter " : "input ") + (is_f ? fl : il) + " into rows of taps";
+        return h;
+      }
+      p.c = (int)run; p.x = 1;
+      p.in_cs = 1; p.in_gs = 0; p.in_ws = cpad; p.in_hs = wi * cpad; p.in_ns = hi * wi * cpad;
+      p.fil_cs = 1; p.fil_xs = run; p.fil_ys = run; p.fil_ks = y * run; p.fil_gs = k * y * run;
+      p.run_valid = x * cpad < run ? (int)(x * cpad) : 0;
+      c = run;
+      Kg = y * run;
+      p.K = (int)Kg;
+      fast = true;
+      runs_kernel = p.run_valid != 0;
+      h->ptr_map = {{ws, 0}, {ws, fil_bytes}, {2, 0}, {3, 0}, {p.epi.residual_op ? 4 : -1, 0}};
+    }
+  }
+
   // Layout-conversion plan.  A problem whose filter or input is not
   // channel-contiguous (the reference's default gkcyx / ngchw) would run the
   // element-wise kernel; if the channel-contiguous form qualifies for the
@@ -2983,12 +3044,13 @@ Handle *make_conv(const OptMap &o) {
     }
   }
   p.k_order_yxc = (p.in_cs == 1) ? 1 : 0;
-  const Tile *tile = fast ? pick_tile(Mg, k, (int)g, true, forced_tile(o)) : nullptr;
+  const Tile *tile = runs_kernel ? &kFastTiles[3] : fast ? pick_tile(Mg, k, (int)g, true, forced_tile(o)) : nullptr;
   if (!tile)
     tile = fast ? pick_tile(Mg, k, (int)g, true, "") : &kGenericTile;
   apply_tile_grid(*tile, Mg, k, (int)g, p.tiles_m, p.tiles_n, p.group_m, p.xcd_remap,
                   h->block_size, h->grid_size);
-  h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + tile->suffix + rich_suffix(p.epi, fast, o);
+  h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + tile->suffix + (runs_kernel ? "_runs" : "") +
+                   rich_suffix(p.epi, fast, o);
   h->num_pointers = 5;
   if (!planned)
     set_contraction_pointers(h, p.epi);

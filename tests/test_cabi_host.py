@@ -224,6 +224,10 @@ def test_layout_conversion_pads_channel_runs_to_whole_chunks(rock):
              "--in_layout NHWGC --out_layout NHWGK --batchsize 4 --groupsize 1 --in_channels 3 --out_channels 64 "
              "--in_h 230 --in_w 230 --fil_h 7 --fil_w 7 --dilation_h 1 --dilation_w 1 --conv_stride_h 2 "
              "--conv_stride_w 2 --padding_h 0 --padding_w 0")
+    # (this layer has no padding along w and an even stride: by itself it takes the rows-of-taps plan,
+    # tests/test_conv_narrow_channels_plan.py; the switch keeps it on the plan for any narrow layer)
+    assert rock.RockKernel(first + " --kernel_id 2").kernel_name == "rock_conv_f16_64x64_fast_runs"
+    first += " --tap_rows false"
     ks = [rock.RockKernel(first + " --kernel_id %d" % i) for i in range(3)]
     assert [k.kernel_name for k in ks[:2]] == ["rock_relayout_b2", "rock_relayout_b2"]
     assert ks[2].kernel_name.startswith("rock_conv_f16_") and ks[2].kernel_name.endswith("_fast")

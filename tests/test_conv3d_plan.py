@@ -74,6 +74,9 @@ def _replay_conv(params, fil, fil_off, inp, in_off, out, out_off):
         return o
 
     xin = inp[gather(inp, in_off, (n, g, c, hi, wi), in_s)].reshape(n, g, c, hi, wi).astype(np.float64)
+    (run_valid,) = struct.unpack_from("<i", params, 260)
+    if run_valid:  # "_runs" kernels: what a channel run holds behind its data is cleared before it is multiplied
+        xin[:, :, run_valid:] = 0
     f = fil[gather(fil, fil_off, (g, k, c, y, x), fil_s)].reshape(g, k, c, y, x).astype(np.float64)
     if (ho, wo) == (orc.conv_out_dim(hi, y, ph, ph, sh, dh), orc.conv_out_dim(wi, x, pw, pw, sw, dw)):
         # symmetric padding: the 2-D convolution of the CPU oracle

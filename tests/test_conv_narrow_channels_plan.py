@@ -54,6 +54,43 @@ def test_narrow_channel_filter_gradient_plan_replayed_on_the_cpu(rock, case, il,
     assert names == ["rock_relayout_b%d" % es] * copies + ["rock_conv_bwd_weight_%s_64x64" % tn, "rock_reduce_splits"]
 
 
+FWD_CASES = [
+    # (type, element size, n c k hi wi y x stride pad_h): no padding along w, rows of whole chunks
+    ("fp16", 2, (2, 3, 16, 20, 20, 7, 7, 2, 0)),    # the ResNet first layer in small: 3 -> 4 channels, run of 28 in 32
+    ("fp16", 2, (2, 3, 72, 15, 18, 3, 3, 2, 1)),    # run of 12 in 16; rows padded at the top and bottom
+    ("fp16", 2, (2, 2, 8, 9, 16, 3, 5, 4, 0)),      # 2 channels: run of 10 in 16
+    ("fp16", 2, (2, 4, 24, 12, 16, 4, 4, 2, 2)),    # 4 taps of 4 channels: whole chunks, no kernel of its own needed
+    ("i8", 1, (2, 3, 16, 20, 20, 7, 7, 2, 0)),      # 8-bit: 3 -> 8 channels, run of 56 in 64
+    ("i8", 1, (1, 1, 8, 10, 24, 3, 3, 4, 1)),
+]
+
+
+@pytest.mark.parametrize("t,es,case", FWD_CASES)
+@pytest.mark.parametrize("il,fl", [("nhwgc", "gkyxc"), ("ngchw", "gkcyx")])
+def test_rows_of_taps_forward_plan_replayed_on_the_cpu(rock, t, es, case, il, fl):
+    n, c, k, hi, wi, y, x, s, ph = case
+    opts, ho, wo = _options(case, il, fl, t)
+    opts = opts.replace("--operation conv_bwd_weight", "--operation conv")
+    ol = il.replace("c", "k")
+    rng = np.random.default_rng(12)
+    fil = rng.integers(-3, 4, k * c * y * x).astype(np.float32)
+    inp = rng.integers(-3, 4, n * c * hi * wi).astype(np.float32)
+    want, _, _ = orc.conv_fwd(fil, inp, fl, il, ol, n, 1, c, k, hi, wi, y, x, (s, s), (ph, 0), (1, 1))
+    first = rock.RockKernel(opts)
+    out = np.full(want.size, np.nan, np.float32)
+    ws = np.full(first.workspace_bytes // es, np.nan, np.float32)
+    tn = {"fp16": "f16"}.get(t, t)
+    names = _replay_plan(rock, opts, [fil, inp, out, None, ws], tn, es)
+    assert np.array_equal(out, want.ravel())
+    whole = (x * max(c, 4 // es) * es) % 16 == 0 and t == "fp16"
+    assert names == ["rock_relayout_b%d" % es] * 2 + ["rock_conv_%s_64x64_fast%s" % (tn, "" if whole else "_runs")]
+    # the contraction reduces over rows of taps: K = y * run
+    import struct
+    conv_k = rock.RockKernel(opts + " --kernel_id 2")
+    cc, xx = struct.unpack_from("<i", conv_k.params(), 128)[0], struct.unpack_from("<i", conv_k.params(), 148)[0]
+    assert xx == 1 and (cc * es) % 16 == 0 and cc * es < x * 16
+
+
 def test_narrow_channel_route_conditions(rock):
     """Padding or dilation along w, an odd image width, or a switch decline the route."""
     base, _, _ = _options(CASES[0], "nhwgc", "gkyxc", "fp16")
@@ -63,3 +100,9 @@ def test_narrow_channel_route_conditions(rock):
                    ("--dilation_w 1", "--dilation_w 2 --out_w 4")):
         assert not any(nm.startswith("rock_conv_bwd_weight_") for nm in names(base.replace(*change))), change
     assert not any(nm.startswith("rock_conv_bwd_weight_") for nm in names(base + " --bwd_weight_gemm false"))
+    fwd = base.replace("--operation conv_bwd_weight", "--operation conv")
+    assert names(fwd)[-1] == "rock_conv_f16_64x64_fast_runs"
+    for change in (("--padding_w 0", "--padding_w 1 --out_w 8"), ("--in_w 20 --out_h 7 --out_w 7", "--in_w 21 --out_h 7 --out_w 8"),
+                   ("--dilation_w 1", "--dilation_w 2 --out_w 4"), ("--conv_stride_w 2", "--conv_stride_w 1 --out_w 14"),
+                   ("--padding_w 0 ", "--padding_w 0 --tap_rows false")):
+        assert not names(fwd.replace(*change))[-1].endswith("_runs"), change

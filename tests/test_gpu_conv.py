@@ -195,7 +195,7 @@ def test_conv_channel_padding_takes_the_vector_kernel(rock, oracle, gpu):
     info = {}
     out, od, ref = _run(rock, oracle, gpu, "f16", 4, 1, 3, 64, 230, 230, 7, 7, (2, 2), (0, 0), (1, 1),
                         NCHW, False, 43, info=info)
-    assert info["kernels"][:2] == ["rock_relayout_b2", "rock_relayout_b2"] and info["kernels"][2].endswith("_fast")
+    assert info["kernels"] == ["rock_relayout_b2", "rock_relayout_b2", "rock_conv_f16_64x64_fast_runs"]
     check_float(to_f32(out, od), ref, od)
 
 
@@ -301,3 +301,64 @@ def test_conv_pixel_contiguous_output_vector_store_exact(rock, oracle, gpu, t, o
                            143, out_dtype=od, scale=0.25)
         want = oracle.round_through(np.asarray(ref, np.float32) * np.float32(0.25), CODE[od])
         assert np.array_equal(to_f32(out, od), want)
+
+
+# (n g c k hi wi y x stride pad dil): narrow pixels, no padding or dilation along w, rows of whole chunks
+TAP_ROW_CASES = [
+    (4, 1, 3, 64, 38, 38, 7, 7, (2, 2), (0, 0), (1, 1)),      # the ResNet first layer in small
+    (2, 1, 3, 16, 20, 20, 7, 7, (2, 2), (0, 0), (1, 1)),
+    (3, 1, 3, 136, 15, 18, 3, 3, (2, 2), (1, 0), (1, 1)),     # rows padded at the top and bottom, three column tiles
+    (2, 1, 2, 8, 9, 16, 3, 5, (3, 4), (0, 0), (2, 1)),        # two channels, stride 4 along w, dilated rows
+    (2, 1, 4, 24, 12, 16, 4, 4, (2, 2), (2, 0), (1, 1)),      # 4 taps of 4 channels
+    (1, 1, 1, 8, 10, 24, 3, 3, (1, 8), (1, 0), (1, 1)),       # one channel
+    (2, 1, 3, 32, 70, 64, 5, 5, (1, 2), (2, 0), (1, 1)),      # many K-steps over the rows of taps
+]
+
+
+@pytest.mark.parametrize("case", TAP_ROW_CASES)
+@pytest.mark.parametrize("layouts", [NHWC, NCHW], ids=["nhwc", "nchw"])
+@pytest.mark.parametrize("t", ["f16", "bf16", "i8", "fp8"])
+def test_conv_rows_of_taps_exact(rock, oracle, gpu, case, layouts, t):
+    """Narrow pixels: both tensors copied into rows of taps, the contraction over K = y * run on the kernels
+    that clear what a run holds behind its data."""
+    info = {}
+    out, od, ref = _run(rock, oracle, gpu, t, *case, layouts, True, 47, info=info)
+    assert len(info["kernels"]) == 3 and "_64x64_fast" in info["kernels"][2]
+    c, x = case[2], case[7]
+    es = 2 if t in ("f16", "bf16") else 1
+    cpad = max(4 // es, 1 << (c - 1).bit_length())
+    while (case[8][1] * cpad * es) % 16:
+        cpad *= 2
+    assert info["kernels"][2].endswith("_runs") == ((x * cpad * es) % 16 != 0)
+    if t == "i8":
+        assert oracle.verify_int(out.cpu().numpy().ravel(), ref)[0] == 0
+    else:
+        assert np.array_equal(to_f32(out, od), ref)
+
+
+@pytest.mark.parametrize("layouts", [NHWC, NCHW], ids=["nhwc", "nchw"])
+def test_conv_rows_of_taps_keep_an_infinity_in_its_own_windows(rock, oracle, gpu, layouts):
+    """The pixel behind a row of taps comes along with the run's last chunk and meets zeros of the filter;
+    an Inf there must not reach the sum (0 * Inf is NaN): the kernel clears it first."""
+    n, g, c, k, hi, wi, y, x = 2, 1, 3, 16, 20, 20, 7, 7
+    fl, il, ol = layouts
+    rng = np.random.default_rng(53)
+    fil = rng.integers(-2, 3, (g, k, c, y, x)).astype(np.float32)
+    inp = rng.integers(-2, 3, (n, g, c, hi, wi)).astype(np.float32)
+    inp[0, 0, 1, 9, 13] = np.inf     # column 13 = 2 * 3 + 7: the pixel behind the taps of output column 3
+    inp[1, 0, 0, 4, 7] = -np.inf
+    raw_f, fq = quantise(_to_layout(fil, "gkcyx", fl), "f16")
+    raw_i, iq = quantise(_to_layout(inp, "ngchw", il), "f16")
+    info = {}
+    out = rock.conv2d(to_gpu(raw_f, "f16", gpu), to_gpu(raw_i, "f16", gpu), fil_layout=fl, in_layout=il,
+                      out_layout=ol, batchsize=n, in_channels=c, out_channels=k, in_h=hi, in_w=wi, fil_h=y, fil_w=x,
+                      groupsize=1, stride=(2, 2), padding=(0, 0), dilation=(1, 1), info=info)
+    torch.cuda.synchronize()
+    assert info["kernels"][2] == "rock_conv_f16_64x64_fast_runs"
+    with np.errstate(invalid="ignore"):
+        ref, ho, wo = oracle.conv_fwd(fq, iq, fl, il, ol, n, g, c, k, hi, wi, y, x, (2, 2), (0, 0), (1, 1))
+    got = to_f32(out, "f16")
+    assert np.isnan(ref).any() or np.isinf(ref).any()
+    finite = np.isfinite(ref)
+    assert np.array_equal(np.isfinite(got), finite) and np.array_equal(got[finite], ref[finite])
+    assert np.array_equal(np.isnan(got), np.isnan(ref))

@@ -59,8 +59,14 @@ PROBLEMS = [
     conv("i8", "ngchw", "gkcyx", 2, 64, 10, 10, 128, 1, 1, stride=2),
     conv("f32", "ngchw", "gkcyx", 2, 32, 9, 9, 64, 1, 1, stride=2),
     # three channels padded to one 16-byte chunk per pixel, NCHW and NHWC
+    conv("fp16", "ngchw", "gkcyx", 2, 3, 30, 30, 64, 7, 7, stride=2, extra="--tap_rows false"),
+    conv("i8", "ngchw", "gkcyx", 2, 3, 30, 30, 64, 7, 7, stride=2, extra="--tap_rows false"),
+    conv("fp16", "nhwgc", "gkyxc", 2, 3, 30, 30, 64, 7, 7, stride=2, extra="--tap_rows false"),
+    # ... and into rows of taps: 3 -> 4 channels of 16 bits (two pixels a chunk), 3 -> 8 of 8 bits, the filter
+    # rows padded to whole chunks
     conv("fp16", "ngchw", "gkcyx", 2, 3, 30, 30, 64, 7, 7, stride=2),
     conv("i8", "ngchw", "gkcyx", 2, 3, 30, 30, 64, 7, 7, stride=2),
+    conv("i8", "nhwgc", "gkyxc", 2, 3, 30, 30, 64, 7, 7, stride=2),
     conv("f32", "ngchw", "gkcyx", 2, 3, 18, 18, 64, 3, 3),
     conv("fp16", "nhwgc", "gkyxc", 2, 3, 30, 30, 64, 7, 7, stride=2),
     # channel counts that are not whole chunks
@@ -155,7 +161,8 @@ def test_modes_chosen(rock):
         raw = rock.RockKernel("%s --kernel_id %d" % (options, kid)).params()
         return struct.unpack_from("<5i", raw, 80), struct.unpack_from("<4i", raw, 120)
     # 3 channels -> 8: RELAYOUT_COPY for the NCHW image as well (source contiguous along the folded pixels)
-    size, (sf, df, mode, _) = params_of(conv("fp16", "ngchw", "gkcyx", 2, 3, 30, 30, 64, 7, 7, stride=2), 1)
+    size, (sf, df, mode, _) = params_of(conv("fp16", "ngchw", "gkcyx", 2, 3, 30, 30, 64, 7, 7, stride=2,
+                                             extra="--tap_rows false"), 1)
     assert size[-2:] == (900, 8) and (sf, df, mode) == (3, 4, 1)
     # a 3x3 filter gkcyx -> gkyxc: runs of 9 along the source, tiles of 256 channels x 16 taps
     size, (sf, df, mode, td) = params_of(conv("fp16", "ngchw", "gkcyx", 2, 256, 14, 14, 256, 3, 3, pad=1), 0)
