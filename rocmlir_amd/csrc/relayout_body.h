@@ -131,7 +131,8 @@ template <typename T> RK_DEV void lds_store16(T *at, const Bytes16 &v) {
 // RELAYOUT_TRANSPOSE_VEC: the same transposition with 16-byte accesses.  The
 // destination's contiguous dimension has unit stride; the source's need not
 // (every other pixel of a row, a flipped filter), and is then read element by
-// element.
+// element, or, for a stride of two over rows that start on 16-byte boundaries,
+// with aligned vectors of which every other element is kept.
 //
 // Reading (unit stride): row r of the tile starts m_r elements past a 16-byte
 // boundary.  Its lanes load the aligned vectors from that boundary on (one
@@ -184,6 +185,23 @@ RK_DEV void transpose_vec_phase(int phase, const T *src, T *dst, const RockRelay
           lds_store16(&tile[r * pitch + k * V], *(const Bytes16 *)g);
         if (k == vpr - 1 && m != 0 && ts - m < lim)
           lds_store16(&tile[r * pitch + ts], *(const Bytes16 *)(g + V));
+      }
+    } else if (ss_s == 2 && (((uintptr_t)(src + t.so) / ES) & (unsigned)(V - 1)) == 0 &&
+               ((unsigned)ss_d & (unsigned)(V - 1)) == 0) {
+      // every other element of rows that start on 16-byte boundaries (every other pixel of an image
+      // row): aligned vectors, of which every other element is kept -- V/2 tile columns per vector
+      const int lim = src_s - t.org_s < ts ? src_s - t.org_s : ts;
+      const int vpr_shift = ts_shift - __builtin_ctz((unsigned)(V / 2)), vpr = 1 << vpr_shift;
+      for (int j = 0; j < 2 * Geo::VPT; ++j) {
+        const int vi = j * 256 + tid;
+        const int r = vi >> vpr_shift, k = vi & (vpr - 1);
+        if (t.org_d + r >= src_d || k * (V / 2) >= lim)
+          continue;
+        Vec u;
+        u.v = *(const Bytes16 *)(src + t.so + (int64_t)r * ss_d + k * V);
+        T *at = &tile[r * pitch + k * (V / 2)];
+        for (int e = 0; e < V / 2; ++e)
+          at[e] = u.e[2 * e];
       }
     } else {
       for (int j = 0; j < Geo::AREA / 256; ++j) {

@@ -58,6 +58,10 @@ PROBLEMS = [
     conv("fp16", "ngchw", "gkcyx", 2, 64, 14, 14, 128, 1, 1, stride=2),
     conv("i8", "ngchw", "gkcyx", 2, 64, 10, 10, 128, 1, 1, stride=2),
     conv("f32", "ngchw", "gkcyx", 2, 32, 9, 9, 64, 1, 1, stride=2),
+    # ... of rows that start on 16-byte boundaries: aligned vectors, every other element kept
+    conv("fp16", "ngchw", "gkcyx", 2, 64, 16, 24, 128, 1, 1, stride=2),
+    conv("i8", "ngchw", "gkcyx", 2, 64, 32, 32, 128, 1, 1, stride=2),
+    conv("f32", "ngchw", "gkcyx", 2, 40, 8, 8, 64, 1, 1, stride=2),
     # three channels padded to one 16-byte chunk per pixel, NCHW and NHWC
     conv("fp16", "ngchw", "gkcyx", 2, 3, 30, 30, 64, 7, 7, stride=2, extra="--tap_rows false"),
     conv("i8", "ngchw", "gkcyx", 2, 3, 30, 30, 64, 7, 7, stride=2, extra="--tap_rows false"),
