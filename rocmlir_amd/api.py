@@ -372,8 +372,12 @@ class RockProgram:
 
     def benchmark(self, *args, warmup=3, iters=20, stream=None):
         """Sum of the kernels' average times in milliseconds."""
+        return sum(ms for _, ms in self.benchmark_each(*args, warmup=warmup, iters=iters, stream=stream))
+
+    def benchmark_each(self, *args, warmup=3, iters=20, stream=None):
+        """[(kernel name, average time in milliseconds)] in launch order."""
         full = self._args(args)
-        return sum(k.benchmark(*full, warmup=warmup, iters=iters, stream=stream) for k in self.kernels)
+        return [(k.kernel_name, k.benchmark(*full, warmup=warmup, iters=iters, stream=stream)) for k in self.kernels]
 
 
 # ---------------------------------------------------------------------------

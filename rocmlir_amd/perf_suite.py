@@ -122,7 +122,8 @@ def conv_problem(line, t, layout, direction_flag=None):
     return opts, shapes, 2.0 * n * (c // g) * k * ho * wo * y * x
 
 
-def run_problem(rock, torch, dev, opts, shapes, flops, warmup, iters, warm_ms=0.0, tune_kind=None, table=None):
+def run_problem(rock, torch, dev, opts, shapes, flops, warmup, iters, warm_ms=0.0, tune_kind=None, table=None,
+                per_kernel=False):
     try:
         prog = rock.RockProgram(opts)  # every kernel of the problem and its workspace
     except rock.RockError as e:
@@ -139,11 +140,14 @@ def run_problem(rock, torch, dev, opts, shapes, flops, warmup, iters, warm_ms=0.
         for _ in range(10):
             prog.launch(*args)
         torch.cuda.synchronize()
-    ms = prog.benchmark(*args, warmup=warmup, iters=iters)
+    each = prog.benchmark_each(*args, warmup=warmup, iters=iters)
+    ms = sum(t for _, t in each)
     contraction = [k.kernel_name for k in prog.kernels if k.kernel_name.startswith(("rock_conv", "rock_gemm",
                                                                                      "rock_attention"))]
     res = {"status": "ok", "kernel": contraction[-1], "kernels": len(prog.kernels), "ms": round(ms, 5),
            "tflops": round(flops / (ms * 1e-3) / 1e12, 2)}
+    if per_kernel:
+        res["kernel_ms"] = [[name, round(t, 5)] for name, t in each]
     if tune_kind:
         from .tuning import tune
         best = tune(prog, *args, table=table, warmup=warmup, iters=iters, kind=tune_kind)
@@ -169,6 +173,7 @@ def main(argv=None):
     ap.add_argument("--tune", choices=["quick", "full", "exhaustive"], default=None,
                     help="also time every entry of each problem's tuning space and report the fastest")
     ap.add_argument("--table", default=None, help="with --tune: save the winners as a .tuning table here")
+    ap.add_argument("--per-kernel", action="store_true", help="list every kernel of a problem with its own time")
     args = ap.parse_args(argv)
 
     import torch
@@ -205,7 +210,7 @@ def main(argv=None):
                     print(json.dumps({"problem": opts, "status": "skipped", "bytes": nbytes}), flush=True)
                     continue
                 res = run_problem(rock, torch, dev, opts, shapes, flops, args.warmup, args.iters, args.warm_ms,
-                                  args.tune, table)
+                                  args.tune, table, args.per_kernel)
                 res["problem"] = opts
                 print(json.dumps(res), flush=True)
                 torch.cuda.empty_cache()
