@@ -92,7 +92,10 @@ typedef void *MiirHandle;
  * 16-bit or int8 stride-1 convolution whose tiles fill on the kernel that keeps the
  * input window in LDS, behind a conversion of the filter), split_k (a GEMM with
  * few output tiles and a long reduction split over blocks, partial sums in the
- * workspace), fused (attention, above).  A single leading dash and "key=value"
+ * workspace), tap_rows (a convolution over pixels of a few channels, without
+ * padding or dilation along w, reads a row of filter taps as one run of
+ * neighbouring pixels: conversions of both tensors, then a "_runs" kernel),
+ * fused (attention, above).  A single leading dash and "key=value"
  * are accepted as well.  rocmlir-gen's scheduling and instruction-set toggles
  * (reverse_grid, mfma, wmma, dot, x2) are accepted and ignored, and so is
  * kernel_name: the code objects are built ahead of time and their kernel
