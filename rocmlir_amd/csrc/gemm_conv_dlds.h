@@ -161,7 +161,14 @@ template <int DT, int ROWS, int NW, int RB, bool RUNS = false> struct ConvInDl {
     uniform = !RUNS && (cp.c * ES) % RB == 0;
     tails = 0;
     run_valid = cp.run_valid;
-    uy = ux = uc0 = 0;
+    // first element of this group's share of the reduction (0 unless the reduction is split over the groups)
+    const int kstart = g * cp.k_group_stride;
+    {
+      const int tap0 = kstart / cp.c;
+      uc0 = (kstart - tap0 * cp.c) * ES;
+      uy = tap0 / cp.x;
+      ux = tap0 - uy * cp.x;
+    }
     {
       const int taps = BKE / cp.c;
       step_c = BKE - taps * cp.c;
@@ -186,15 +193,28 @@ template <int DT, int ROWS, int NW, int RB, bool RUNS = false> struct ConvInDl {
       pix[i] = (m < cp.M) ? (unsigned)(n * (int)cp.in_ns * ES) : kOobOffset;
       int lc = (lane % Dg::CHUNKS) ^ Dg::swz(r);
       kb[i] = lc * kChunk;
-      int k0 = lc * EPC;
+      int k0 = kstart + lc * EPC;
       int tap = k0 / cp.c;
       cc[i] = k0 - tap * cp.c;
       y[i] = tap / cp.x;
       x[i] = tap - y[i] * cp.x;
       tapoff[i] = kOobOffset;
     }
+    if (uniform && uc0 != 0) // a share of a split reduction that starts inside a tap
+      enter_tap();
   }
   // must be called with kt = 0, 1, 2, ... in order (tap state advances)
+  // uniform walk: the rows' offsets at channel 0 of the tap (uy, ux)
+  __device__ __forceinline__ void enter_tap() {
+    const int dh = uy * p->dil_h, dw = ux * p->dil_w;
+    const bool tap_ok = uy < p->y;
+#pragma unroll
+    for (int i = 0; i < Sg::PER_WAVE; ++i) {
+      int hi = h0[i] + dh, wi = w0[i] + dw;
+      bool v = tap_ok && pix[i] != kOobOffset && hi >= 0 && hi < p->hi && wi >= 0 && wi < p->wi;
+      tapoff[i] = v ? pix[i] + (unsigned)((hi * (int)p->in_hs + wi * (int)p->in_ws) * ES + kb[i]) : kOobOffset;
+    }
+  }
   // RUNS: clears what lies behind the data in this lane's tail chunks of K-step kt (their loads have landed)
   __device__ __forceinline__ void zero_tails(int kt, char *stage) {
     if constexpr (RUNS) {
@@ -215,17 +235,8 @@ template <int DT, int ROWS, int NW, int RB, bool RUNS = false> struct ConvInDl {
   __device__ __forceinline__ void issue(int kt, char *stage) {
     (void)kt;
     if (uniform) {
-      if (uc0 == 0) { // entering a tap: one bounds test per row
-        const int dh = uy * p->dil_h, dw = ux * p->dil_w;
-        const bool tap_ok = uy < p->y;
-#pragma unroll
-        for (int i = 0; i < Sg::PER_WAVE; ++i) {
-          int hi = h0[i] + dh, wi = w0[i] + dw;
-          bool v = tap_ok && pix[i] != kOobOffset && hi >= 0 && hi < p->hi && wi >= 0 && wi < p->wi;
-          tapoff[i] = v ? pix[i] + (unsigned)((hi * (int)p->in_hs + wi * (int)p->in_ws) * ES + kb[i])
-                        : kOobOffset;
-        }
-      }
+      if (uc0 == 0) // entering a tap: one bounds test per row
+        enter_tap();
 #pragma unroll
       for (int i = 0; i < Sg::PER_WAVE; ++i)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(

@@ -93,7 +93,10 @@ struct RockConvParams {
   // padded to whole 16-byte chunks; its first run_valid elements are data, what the load brings along behind
   // them (the next pixel) is cleared in LDS before it is multiplied.  0 elsewhere.
   int32_t run_valid;
-  int32_t pad_;
+  // Reduction split over the groups of a one-group problem (few output tiles, long reduction): group s
+  // reduces the elements [s * k_group_stride, s * k_group_stride + K) of every row of taps-and-channels,
+  // a whole number of K-steps, into an f32 partial result of its own (in_gs = 0, fil_gs = K).  0 elsewhere.
+  int32_t k_group_stride;
 };
 
 // Filter gradient of a convolution as one K-major GEMM over the tensors as they

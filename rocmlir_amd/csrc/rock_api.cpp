@@ -2857,6 +2857,35 @@ Handle *make_conv(const OptMap &o) {
   bool fast = conv_fast(p, c);
   bool planned = false; // the layout-conversion plan fixes the pointer map itself
 
+  // Reduction split over blocks: few output tiles and a long reduction (the 3x3 layers of a UNet at batch 2:
+  // 512 pixels x 1280 channels over K = 17280 is 160 tiles of 64 x 64, each with 270 K-steps in a row).  The
+  // (taps, channels) range is cut into S equal shares of whole K-steps; the contraction kernel runs them as S
+  // groups of the one-group problem (RockConvParams::k_group_stride) into f32 partial results in the
+  // workspace, which rock_reduce_splits adds in split order into the caller's layout.  Only with the
+  // identity epilogue, which commutes with the sum (as for the GEMM, and as the reference's split-K,
+  // Rock.cpp:167-198); "--split_k false" or any perf_config declines.
+  int64_t S = 1, k_part = 0, part_off = 0;
+  int conv_kid = 0;
+  {
+    const RockEpilogue &e = p.epi;
+    const bool identity = e.scale == 1.0f && !e.has_bias && e.activation == ROCK_ACT_NONE &&
+                          e.residual_op == ROCK_RES_NONE && to == ti &&
+                          (ti == ROCK_F32 || ti == ROCK_F16 || ti == ROCK_BF16);
+    const int64_t c_chunks = (c * es + 15) / 16 * 16 / es, Kfull = c_chunks * y * x, step = 128 / es;
+    const int64_t tiles64 = (int64_t)ceil_div(Mg, 64) * ceil_div(k, 64);
+    if (g == 1 && identity && tiles64 <= 2 * kNumCU && Kfull >= 2048 && !o.count("perf_config") &&
+        bool_or(o, "split_k", true)) {
+      const int64_t want = std::min<int64_t>(4 * kNumCU / tiles64, Kfull / 1024);
+      for (int64_t d = want; d >= 2; --d)
+        if (Kfull % d == 0 && (Kfull / d) % step == 0) {
+          S = d;
+          k_part = Kfull / d;
+          break;
+        }
+    }
+  }
+  const int64_t part_bytes = S > 1 ? align256(S * Mg * k * 4) : 0;
+
   auto set_problem_key = [&] {
     std::ostringstream key;
     const char *opname = ti == ROCK_F32 ? "conv" : ti == ROCK_F16 ? "convfp16"
@@ -2907,7 +2936,7 @@ Handle *make_conv(const OptMap &o) {
   // filter holds zeros there, but zero times an Inf in that pixel would not be
   // zero).  Every window must start on a chunk boundary: stride_w pixels and an
   // image row are whole chunks.
-  bool runs_kernel = false;
+  bool runs_kernel = false, rows_plan = false;
   if (!fast && g == 1 && pw == 0 && pw_r == 0 && dw == 1 && y * x > 1 && ti != ROCK_F32 &&
       bool_or(o, "layout_conversion", true) && bool_or(o, "tap_rows", true)) {
     int64_t cpad = 1;
@@ -2952,6 +2981,7 @@ Handle *make_conv(const OptMap &o) {
       Kg = y * run;
       p.K = (int)Kg;
       fast = true;
+      rows_plan = true;
       runs_kernel = p.run_valid != 0;
       h->ptr_map = {{ws, 0}, {ws, fil_bytes}, {2, 0}, {3, 0}, {p.epi.residual_op ? 4 : -1, 0}};
     }
@@ -3003,6 +3033,12 @@ Handle *make_conv(const OptMap &o) {
       const int64_t off_f = 0, off_i = need_f ? fil_bytes : 0;
       h->kernel_count = n_relayout + 1;
       h->workspace_bytes = (size_t)((need_f ? fil_bytes : 0) + (need_i ? in_bytes : 0));
+      if (S > 1) { // the partial sums behind the converted tensors, the reduction kernel behind the contraction
+        conv_kid = n_relayout;
+        part_off = (int64_t)h->workspace_bytes;
+        h->kernel_count += 1;
+        h->workspace_bytes += (size_t)part_bytes;
+      }
       // filter, input, output, bias, [residual,] workspace
       const int ws = p.epi.residual_op ? 5 : 4;
       h->caller_pointers = ws + 1;
@@ -3044,10 +3080,58 @@ Handle *make_conv(const OptMap &o) {
     }
   }
   p.k_order_yxc = (p.in_cs == 1) ? 1 : 0;
-  const Tile *tile = runs_kernel ? &kFastTiles[3] : fast ? pick_tile(Mg, k, (int)g, true, forced_tile(o)) : nullptr;
+  int64_t groups = g;
+  if (S > 1 && fast && !rows_plan) {
+    if (!planned) { // the tensors as they lie: the contraction, then the reduction
+      planned = true;
+      h->kernel_count = 2;
+      h->workspace_bytes = (size_t)part_bytes;
+      h->caller_pointers = 5;
+      h->ptr_map = {{0, 0}, {1, 0}, {2, 0}, {3, 0}, {-1, 0}};
+    }
+    const int kid = (int)int_or(o, "kernel_id", 0);
+    if (kid == conv_kid + 1) {
+      RockReduceParams r;
+      std::memset(&r, 0, sizeof r);
+      r.split_stride = Mg * k;
+      r.size[0] = (int)n; r.size[1] = (int)ho; r.size[2] = (int)wo; r.size[3] = (int)k;
+      r.dst_stride[0] = p.out_ns; r.dst_stride[1] = p.out_hs; r.dst_stride[2] = p.out_ws; r.dst_stride[3] = p.out_ks;
+      r.splits = (int)S;
+      r.out_dtype = to;
+      h->op = OP_RELAYOUT;
+      h->epi = nullptr;
+      h->params.assign(sizeof r, 0); // p is gone from here on
+      std::memcpy(h->params.data(), &r, sizeof r);
+      h->kernel_name = "rock_reduce_splits";
+      h->block_size = 256;
+      h->grid_size = (uint32_t)((Mg * k + 255) / 256);
+      h->num_pointers = 2;
+      h->perf_config = "";
+      h->ptr_map = {{4, part_off}, {2, 0}};
+      h->problem_key = "reduction of the split partial sums";
+      return h;
+    }
+    if (kid != conv_kid) {
+      set_error("conv: kernel_id out of range");
+      delete h;
+      return nullptr;
+    }
+    groups = S;
+    p.g = (int)S;
+    p.K = (int)k_part;
+    p.k_group_stride = (int)k_part;
+    p.in_gs = 0;
+    p.fil_gs = k_part;
+    p.out_ks = 1; p.out_ws = k; p.out_hs = wo * k; p.out_ns = ho * wo * k; p.out_gs = Mg * k;
+    p.epi.out_dtype = ROCK_F32;
+    h->ptr_map[2] = Handle::PtrSrc{4, part_off};
+  }
+  const Tile *tile = runs_kernel ? &kFastTiles[3]
+                     : fast      ? pick_tile(Mg, k, (int)groups, true, forced_tile(o))
+                                 : nullptr;
   if (!tile)
-    tile = fast ? pick_tile(Mg, k, (int)g, true, "") : &kGenericTile;
-  apply_tile_grid(*tile, Mg, k, (int)g, p.tiles_m, p.tiles_n, p.group_m, p.xcd_remap,
+    tile = fast ? pick_tile(Mg, k, (int)groups, true, "") : &kGenericTile;
+  apply_tile_grid(*tile, Mg, k, (int)groups, p.tiles_m, p.tiles_n, p.group_m, p.xcd_remap,
                   h->block_size, h->grid_size);
   h->kernel_name = std::string("rock_conv_") + dtype_name(ti) + tile->suffix + (runs_kernel ? "_runs" : "") +
                    rich_suffix(p.epi, fast, o);

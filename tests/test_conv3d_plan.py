@@ -62,10 +62,48 @@ def _replay_relayout(params, src, src_off, dst, dst_off):
     dst[do] = vals
 
 
-def _replay_conv(params, fil, fil_off, inp, in_off, out, out_off):
+def _replay_split_conv(params, fil, fil_off, inp, in_off, out, out_off, es):
+    """A one-group convolution whose reduction is split over its groups (k_group_stride): group s
+    reduces the elements [s * K, (s + 1) * K) of the (tap, channel) index into its own f32 result."""
+    st = struct.unpack_from("<15q", params, 0)
+    n, S, c, k, hi, wi, y, x, ho, wo, sh, sw, ph, pw, dh, dw = struct.unpack_from("<16i", params, 120)
+    (K,) = struct.unpack_from("<i", params, 192)
+    (stride,) = struct.unpack_from("<i", params, 264)
+    (out_dtype,) = struct.unpack_from("<i", params, 240)
+    in_s, fil_s, out_s = st[0:5], st[5:10], st[10:15]
+    assert stride == K and S * K == c * y * x and in_s[1] == 0 and fil_s[0] == K and out_dtype == 0
+    kk = np.arange(c * y * x)
+    tap, ch = kk // c, kk % c
+    ty, tx = tap // x, tap % x
+    pix = np.arange(n * ho * wo)
+    nn, oh, ow = pix // (ho * wo), (pix // wo) % ho, pix % wo
+    ih = oh[:, None] * sh + ty[None, :] * dh - ph
+    iw = ow[:, None] * sw + tx[None, :] * dw - pw
+    ok = (ih >= 0) & (ih < hi) & (iw >= 0) & (iw < wi)
+    src = in_off + nn[:, None] * in_s[0] + ih * in_s[3] + iw * in_s[4] + ch[None, :] * in_s[2]
+    assert src[ok].min() >= 0 and src[ok].max() < inp.size
+    a = np.where(ok, inp[np.where(ok, src, 0)], 0).astype(np.float64)
+    fsrc = fil_off + np.arange(k)[:, None] * fil_s[1] + ty[None, :] * fil_s[3] + tx[None, :] * fil_s[4] + ch[None, :] * fil_s[2]
+    assert fsrc.min() >= 0 and fsrc.max() < fil.size
+    b = fil[fsrc].astype(np.float64)
+    wide = 4 // es
+    for sp in range(S):
+        part = a[:, sp * K:(sp + 1) * K] @ b[:, sp * K:(sp + 1) * K].T
+        assert not np.isnan(part).any()
+        o = out_off + wide * (sp * out_s[1] + nn[:, None] * out_s[0] + oh[:, None] * out_s[3] + ow[:, None] * out_s[4]
+                              + np.arange(k)[None, :] * out_s[2])
+        assert o.min() >= 0 and o.max() + wide - 1 < out.size and len(np.unique(o)) == o.size
+        out[o] = part
+        if wide > 1:
+            out[o + 1] = np.nan
+
+
+def _replay_conv(params, fil, fil_off, inp, in_off, out, out_off, es=None):
     st = struct.unpack_from("<15q", params, 0)
     n, g, c, k, hi, wi, y, x, ho, wo, sh, sw, ph, pw, dh, dw = struct.unpack_from("<16i", params, 120)
     in_s, fil_s, out_s = st[0:5], st[5:10], st[10:15]   # n g c h w / g k c y x / n g k h w
+    if struct.unpack_from("<i", params, 264)[0]:
+        return _replay_split_conv(params, fil, fil_off, inp, in_off, out, out_off, es)
 
     def gather(buf, off, sizes, strides):
         idx = np.indices(sizes).reshape(len(sizes), -1)
@@ -133,7 +171,7 @@ def test_conv3d_plan_replayed_on_the_cpu(rock, case, layouts, t, es):
             (f_src, f_off), (i_src, i_off), (o_src, o_off) = pm[:3]
             assert pm[3][0] == 3 and pm[4][0] == -1
             _replay_conv(kern.params(), buffers[f_src], f_off // es, buffers[i_src], i_off // es, buffers[o_src],
-                         o_off // es)
+                         o_off // es, es)
     assert np.array_equal(out, want)
     assert sum(nm.startswith("rock_conv_") for nm in names) == 1
     with pytest.raises(rock.RockError, match="kernel_id out of range"):
@@ -218,7 +256,7 @@ def _replay_plan(rock, opts, buffers, t, es):
         elif name.startswith("rock_conv_" + t + "_"):
             (f_src, f_off), (i_src, i_off), (o_src, o_off) = pm[:3]
             _replay_conv(kern.params(), buffers[f_src], f_off // es, buffers[i_src], i_off // es, buffers[o_src],
-                         o_off // es)
+                         o_off // es, es)
         elif name.startswith("rock_conv_bwd_weight_"):
             (y_src, y_off), (x_src, x_off), (w_src, w_off) = pm[:3]
             _replay_bwd_weight_gemm(kern.params(), buffers[y_src], y_off // es, buffers[x_src], x_off // es,

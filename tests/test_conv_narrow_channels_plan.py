@@ -6,6 +6,8 @@ columns out -- replayed kernel by kernel in numpy from the parameter blocks and
 pointer maps the C ABI hands out, against the CPU oracle.  The workspace
 starts as NaN, so a kernel that used a byte no earlier kernel wrote, outside
 the padding columns, would show."""
+import struct
+
 import numpy as np
 import pytest
 
@@ -106,3 +108,47 @@ def test_narrow_channel_route_conditions(rock):
                    ("--dilation_w 1", "--dilation_w 2 --out_w 4"), ("--conv_stride_w 2", "--conv_stride_w 1 --out_w 14"),
                    ("--padding_w 0 ", "--padding_w 0 --tap_rows false")):
         assert not names(fwd.replace(*change))[-1].endswith("_runs"), change
+
+
+SPLIT_CASES = [
+    # (n c k hi wi y x stride pad): few output tiles, a long reduction
+    (2, 320, 64, 8, 8, 3, 3, 1, 1),      # K = 2880: halves of 1440 are whole K-steps of 32-bit elements only
+    (1, 256, 32, 6, 6, 3, 3, 1, 1),      # K = 2304
+    (2, 512, 40, 5, 7, 2, 2, 1, 0),      # K = 2048, ragged output channels
+    (1, 100, 16, 9, 12, 4, 8, 1, 0),     # 16-bit channels padded to 104 by the conversion: K = 3328
+    (2, 384, 24, 6, 6, 3, 3, 2, 1),      # K = 3456: three shares
+]
+
+
+@pytest.mark.parametrize("case", SPLIT_CASES)
+@pytest.mark.parametrize("il,fl", [("nhwgc", "gkyxc"), ("ngchw", "gkcyx")])
+@pytest.mark.parametrize("t,es", [("fp16", 2), ("f32", 4)])
+def test_forward_reduction_split_plan_replayed_on_the_cpu(rock, case, il, fl, t, es):
+    n, c, k, hi, wi, y, x, s, pd = case
+    opts = conv(t, il, fl, n, c, hi, wi, k, y, x, stride=s, pad=pd)
+    ol = il.replace("c", "k")
+    rng = np.random.default_rng(13)
+    fil = rng.integers(-3, 4, k * c * y * x).astype(np.float32)
+    inp = rng.integers(-3, 4, n * c * hi * wi).astype(np.float32)
+    want, ho, wo = orc.conv_fwd(fil, inp, fl, il, ol, n, 1, c, k, hi, wi, y, x, (s, s), (pd, pd), (1, 1))
+    first = rock.RockKernel(opts)
+    c_chunks = -(-c * es // 16) * 16 // es
+    kfull, tiles = c_chunks * y * x, -(-n * ho * wo // 64) * -(-k // 64)
+    most = min(1024 // tiles, kfull // 1024)
+    splits = [d for d in range(most, 1, -1) if kfull % d == 0 and (kfull // d) % (128 // es) == 0]
+    if first.kernel_count == 1:   # the tensors as they lie and no share of whole K-steps: one kernel, nothing to replay
+        assert not splits
+        return
+    out = np.full(want.size, np.nan, np.float32)
+    ws = np.full(max(first.workspace_bytes // es, 1), np.nan, np.float32)
+    tn = {"fp16": "f16"}.get(t, t)
+    names = _replay_plan(rock, opts, [fil, inp, out, None, ws], tn, es)
+    assert np.array_equal(out, want.ravel())
+    if splits:
+        assert struct.unpack_from("<i", rock.RockKernel("%s --kernel_id %d" % (opts, len(names) - 2)).params(), 124)[0] == splits[0]
+        assert names[-1] == "rock_reduce_splits" and names[-2].startswith("rock_conv_%s_" % tn)
+        # an epilogue that does not commute with the sum, or the switch, keeps the single contraction kernel
+        assert rock.RockKernel(opts + " --relu true").kernel_count == first.kernel_count - 1
+        assert rock.RockKernel(opts + " --split_k false").kernel_count == first.kernel_count - 1
+    else:
+        assert "rock_reduce_splits" not in names

@@ -362,3 +362,46 @@ def test_conv_rows_of_taps_keep_an_infinity_in_its_own_windows(rock, oracle, gpu
     finite = np.isfinite(ref)
     assert np.array_equal(np.isfinite(got), finite) and np.array_equal(got[finite], ref[finite])
     assert np.array_equal(np.isnan(got), np.isnan(ref))
+
+
+# few output tiles, a long reduction: the (taps, channels) range split over blocks
+SPLIT_CASES = [
+    (2, 1, 640, 320, 16, 16, 3, 3, (1, 1), (1, 1), (1, 1)),   # a UNet layer at batch 2 in small: 160 tiles, K 5760
+    (2, 1, 320, 64, 8, 8, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (1, 1, 256, 32, 6, 6, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (2, 1, 512, 40, 5, 7, 2, 2, (1, 1), (0, 0), (1, 1)),      # ragged output channels
+    (1, 1, 100, 16, 9, 12, 4, 8, (1, 1), (0, 0), (1, 1)),     # channels padded by the conversion kernels
+    (2, 1, 384, 24, 6, 6, 3, 3, (2, 2), (1, 1), (1, 1)),
+    (3, 1, 128, 72, 11, 9, 5, 5, (1, 2), (2, 2), (2, 1)),     # stride, dilation, 5x5
+]
+
+
+@pytest.mark.parametrize("case", SPLIT_CASES)
+@pytest.mark.parametrize("layouts", [NHWC, NCHW, ("gyxck", "hwcgn", "hwkgn")], ids=["nhwc", "nchw", "hwcgn"])
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16"])
+def test_conv_reduction_split_over_blocks_exact(rock, oracle, gpu, case, layouts, t):
+    info = {}
+    out, od, ref = _run(rock, oracle, gpu, t, *case, layouts, True, 59, info=info)
+    # integer data: every partial sum is exact in f32; only the final narrowing rounds
+    assert np.array_equal(to_f32(out, od), oracle.round_through(ref, CODE[od]))
+    n, g, c, k, hi, wi, y, x, stride, pad, dil = case
+    es = 4 if t == "f32" else 2
+    ho = (hi + 2 * pad[0] - (y - 1) * dil[0] - 1) // stride[0] + 1
+    wo = (wi + 2 * pad[1] - (x - 1) * dil[1] - 1) // stride[1] + 1
+    kfull = -(-c * es // 16) * 16 // es * y * x
+    want = min(1024 // (-(-n * ho * wo // 64) * -(-k // 64)), kfull // 1024)
+    if any(kfull % d == 0 and (kfull // d) % (128 // es) == 0 for d in range(2, want + 1)):
+        assert info["kernels"][-1] == "rock_reduce_splits" and info["kernels"][-2].startswith("rock_conv_")
+    else:
+        assert "rock_reduce_splits" not in info["kernels"]
+
+
+def test_conv_reduction_split_real_values_and_declined_with_an_epilogue(rock, oracle, gpu):
+    case = (2, 1, 640, 320, 16, 16, 3, 3, (1, 1), (1, 1), (1, 1))
+    info = {}
+    out, od, ref = _run(rock, oracle, gpu, "f16", *case, NHWC, False, 61, info=info)
+    assert info["kernels"] == ["rock_conv_f16_64x64_fast", "rock_reduce_splits"]
+    check_float(to_f32(out, od), ref, od)
+    info = {}
+    out, od, ref = _run(rock, oracle, gpu, "f16", *case, NHWC, False, 61, info=info, relu=True)
+    assert len(info["kernels"]) == 1
