@@ -181,6 +181,8 @@ struct RockReduceParams {
   int32_t splits;
   int32_t out_dtype; // RockDType: f32, f16 or bf16
   int32_t valid[4];  // elements at or beyond valid[d] along dimension d are padding and are not written (0: none)
+  int32_t int_partials; // 1: the partial sums and the result are int32 (out_dtype ROCK_I32)
+  int32_t pad_;
 };
 
 // rock_fold_depth(T, dst, p): last step of the input gradient of a convolution

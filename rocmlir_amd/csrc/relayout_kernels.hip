@@ -93,6 +93,14 @@ extern "C" __global__ __launch_bounds__(256) void rock_reduce_splits(const float
   }
   if (padding)
     return;
+  if (p.int_partials) { // integer sums: exact in any order
+    const int *ip = (const int *)partials;
+    int acc = 0;
+    for (int s = 0; s < p.splits; ++s)
+      acc += ip[(int64_t)s * p.split_stride + i];
+    ((int *)dst)[off] = acc;
+    return;
+  }
   // summed in split order; sixteen loads are in flight at a time, the additions stay sequential
   float acc = 0.0f;
   int s = 0;

@@ -2861,16 +2861,17 @@ Handle *make_conv(const OptMap &o) {
   // 512 pixels x 1280 channels over K = 17280 is 160 tiles of 64 x 64, each with 270 K-steps in a row).  The
   // (taps, channels) range is cut into S equal shares of whole K-steps; the contraction kernel runs them as S
   // groups of the one-group problem (RockConvParams::k_group_stride) into f32 partial results in the
-  // workspace, which rock_reduce_splits adds in split order into the caller's layout.  Only with the
-  // identity epilogue, which commutes with the sum (as for the GEMM, and as the reference's split-K,
+  // workspace (int32 for int8 operands), which rock_reduce_splits adds in split order into the caller's
+  // layout.  Only with the identity epilogue, which commutes with the sum (as for the GEMM, and as the reference's split-K,
   // Rock.cpp:167-198); "--split_k false" or any perf_config declines.
   int64_t S = 1, k_part = 0, part_off = 0;
   int conv_kid = 0;
   {
     const RockEpilogue &e = p.epi;
-    const bool identity = e.scale == 1.0f && !e.has_bias && e.activation == ROCK_ACT_NONE &&
-                          e.residual_op == ROCK_RES_NONE && to == ti &&
-                          (ti == ROCK_F32 || ti == ROCK_F16 || ti == ROCK_BF16);
+    const bool plain = e.scale == 1.0f && !e.has_bias && e.activation == ROCK_ACT_NONE &&
+                       e.residual_op == ROCK_RES_NONE;
+    const bool identity = plain && ((to == ti && (ti == ROCK_F32 || ti == ROCK_F16 || ti == ROCK_BF16)) ||
+                                    (ti == ROCK_I8 && to == ROCK_I32 && e.zero_point == 0));
     const int64_t c_chunks = (c * es + 15) / 16 * 16 / es, Kfull = c_chunks * y * x, step = 128 / es;
     const int64_t tiles64 = (int64_t)ceil_div(Mg, 64) * ceil_div(k, 64);
     if (g == 1 && identity && tiles64 <= 2 * kNumCU && Kfull >= 2048 && !o.count("perf_config") &&
@@ -3098,6 +3099,7 @@ Handle *make_conv(const OptMap &o) {
       r.dst_stride[0] = p.out_ns; r.dst_stride[1] = p.out_hs; r.dst_stride[2] = p.out_ws; r.dst_stride[3] = p.out_ks;
       r.splits = (int)S;
       r.out_dtype = to;
+      r.int_partials = ti == ROCK_I8 ? 1 : 0;
       h->op = OP_RELAYOUT;
       h->epi = nullptr;
       h->params.assign(sizeof r, 0); // p is gone from here on
@@ -3123,7 +3125,7 @@ Handle *make_conv(const OptMap &o) {
     p.in_gs = 0;
     p.fil_gs = k_part;
     p.out_ks = 1; p.out_ws = k; p.out_hs = wo * k; p.out_ns = ho * wo * k; p.out_gs = Mg * k;
-    p.epi.out_dtype = ROCK_F32;
+    p.epi.out_dtype = ti == ROCK_I8 ? ROCK_I32 : ROCK_F32;
     h->ptr_map[2] = Handle::PtrSrc{4, part_off};
   }
   const Tile *tile = runs_kernel ? &kFastTiles[3]

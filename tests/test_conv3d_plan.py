@@ -71,7 +71,7 @@ def _replay_split_conv(params, fil, fil_off, inp, in_off, out, out_off, es):
     (stride,) = struct.unpack_from("<i", params, 264)
     (out_dtype,) = struct.unpack_from("<i", params, 240)
     in_s, fil_s, out_s = st[0:5], st[5:10], st[10:15]
-    assert stride == K and S * K == c * y * x and in_s[1] == 0 and fil_s[0] == K and out_dtype == 0
+    assert stride == K and S * K == c * y * x and in_s[1] == 0 and fil_s[0] == K and out_dtype in (0, 6)  # f32, i32
     kk = np.arange(c * y * x)
     tap, ch = kk // c, kk % c
     ty, tx = tap // x, tap % x
@@ -94,8 +94,8 @@ def _replay_split_conv(params, fil, fil_off, inp, in_off, out, out_off, es):
                               + np.arange(k)[None, :] * out_s[2])
         assert o.min() >= 0 and o.max() + wide - 1 < out.size and len(np.unique(o)) == o.size
         out[o] = part
-        if wide > 1:
-            out[o + 1] = np.nan
+        for extra in range(1, wide):   # the value sits in the first of the elements it covers
+            out[o + extra] = np.nan
 
 
 def _replay_conv(params, fil, fil_off, inp, in_off, out, out_off, es=None):

@@ -122,7 +122,7 @@ SPLIT_CASES = [
 
 @pytest.mark.parametrize("case", SPLIT_CASES)
 @pytest.mark.parametrize("il,fl", [("nhwgc", "gkyxc"), ("ngchw", "gkcyx")])
-@pytest.mark.parametrize("t,es", [("fp16", 2), ("f32", 4)])
+@pytest.mark.parametrize("t,es", [("fp16", 2), ("f32", 4), ("i8", 1)])
 def test_forward_reduction_split_plan_replayed_on_the_cpu(rock, case, il, fl, t, es):
     n, c, k, hi, wi, y, x, s, pd = case
     opts = conv(t, il, fl, n, c, hi, wi, k, y, x, stride=s, pad=pd)
@@ -148,7 +148,8 @@ def test_forward_reduction_split_plan_replayed_on_the_cpu(rock, case, il, fl, t,
         assert struct.unpack_from("<i", rock.RockKernel("%s --kernel_id %d" % (opts, len(names) - 2)).params(), 124)[0] == splits[0]
         assert names[-1] == "rock_reduce_splits" and names[-2].startswith("rock_conv_%s_" % tn)
         # an epilogue that does not commute with the sum, or the switch, keeps the single contraction kernel
-        assert rock.RockKernel(opts + " --relu true").kernel_count == first.kernel_count - 1
+        other = " --zero_point 3" if t == "i8" else " --relu true"
+        assert rock.RockKernel(opts + other).kernel_count == first.kernel_count - 1
         assert rock.RockKernel(opts + " --split_k false").kernel_count == first.kernel_count - 1
     else:
         assert "rock_reduce_splits" not in names

@@ -378,14 +378,17 @@ SPLIT_CASES = [
 
 @pytest.mark.parametrize("case", SPLIT_CASES)
 @pytest.mark.parametrize("layouts", [NHWC, NCHW, ("gyxck", "hwcgn", "hwkgn")], ids=["nhwc", "nchw", "hwcgn"])
-@pytest.mark.parametrize("t", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16", "i8"])
 def test_conv_reduction_split_over_blocks_exact(rock, oracle, gpu, case, layouts, t):
     info = {}
     out, od, ref = _run(rock, oracle, gpu, t, *case, layouts, True, 59, info=info)
-    # integer data: every partial sum is exact in f32; only the final narrowing rounds
-    assert np.array_equal(to_f32(out, od), oracle.round_through(ref, CODE[od]))
+    if t == "i8":
+        assert oracle.verify_int(out.cpu().numpy().ravel(), ref)[0] == 0
+    else:
+        # integer data: every partial sum is exact in f32; only the final narrowing rounds
+        assert np.array_equal(to_f32(out, od), oracle.round_through(ref, CODE[od]))
     n, g, c, k, hi, wi, y, x, stride, pad, dil = case
-    es = 4 if t == "f32" else 2
+    es = {"f32": 4, "i8": 1}.get(t, 2)
     ho = (hi + 2 * pad[0] - (y - 1) * dil[0] - 1) // stride[0] + 1
     wo = (wi + 2 * pad[1] - (x - 1) * dil[1] - 1) // stride[1] + 1
     kfull = -(-c * es // 16) * 16 // es * y * x
