@@ -1079,6 +1079,9 @@ struct ConvProblem {
   std::string fl, il, ol;
   int64_t n, g, c, k, hi, wi, y, x, ho, wo, sh, sw, ph, pw, dh, dw;
   int64_t fs[5], is[5], os[5]; // element strides in letter order gkcyx / ngchw / ngkhw
+  // filter gradient only: the output gradient is a copy whose k channels were padded with zeros up to a whole
+  // 16-byte chunk; only the first k_valid rows of the gradient exist in the caller's tensor (0: all k)
+  int64_t k_valid = 0;
 };
 
 int64_t floor_div(int64_t a, int64_t b) { return a >= 0 ? a / b : -((-a + b - 1) / b); }
@@ -1687,7 +1690,7 @@ Handle *bwd_weight_narrow_channels(const OptMap &o, const ConvProblem &cp, bool 
     std::memset(&r, 0, sizeof r);
     r.split_stride = cp.k * Ng;
     r.size[0] = (int)cp.k; r.size[1] = (int)cp.y; r.size[2] = (int)(run / cpad); r.size[3] = (int)cpad;
-    r.valid[2] = (int)cp.x; r.valid[3] = (int)cp.c;
+    r.valid[0] = (int)cp.k_valid; r.valid[2] = (int)cp.x; r.valid[3] = (int)cp.c;
     r.dst_stride[0] = cp.fs[1]; r.dst_stride[1] = cp.fs[3]; r.dst_stride[2] = cp.fs[4]; r.dst_stride[3] = cp.fs[2];
     r.splits = (int)S;
     r.out_dtype = cp.ti;
@@ -1770,6 +1773,94 @@ Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
   }
   const int es = dtype_size(cp.ti);
   const int kid = (int)int_or(o, "kernel_id", 0);
+
+  // An output gradient with a few channels (k * es not a whole 16-byte chunk: a layer that ends in 4
+  // channels): a first kernel copies it channels-last with the k run padded with zeros to whole chunks,
+  // which the K-major GEMM route below reads; the rows of the gradient beyond k come out zero and the
+  // reduction kernel leaves them out (k_valid).  Only where that route is certain to take the padded
+  // problem (more than one tap, one group, channel runs of the input in whole chunks).
+  if (!cp.k_valid && cp.g == 1 && cp.y * cp.x > 1 && (cp.k * es) % 16 != 0 && (cp.c * es) % 16 == 0 &&
+      (cp.ti == ROCK_F32 || cp.ti == ROCK_F16 || cp.ti == ROCK_BF16) && bool_or(o, "bwd_weight_gemm", true) &&
+      bool_or(o, "layout_conversion", true)) {
+    const int64_t kpad = (cp.k * es + 15) / 16 * 16 / es;
+    ConvProblem inner = cp;
+    inner.k = kpad;
+    inner.k_valid = cp.k;
+    inner.ol = "nhwgk";
+    const int64_t osz[5] = {cp.n, cp.g, kpad, cp.ho, cp.wo};
+    layout_strides(inner.ol, "ngkhw", osz, inner.os);
+    const int64_t dy_bytes = align256(cp.n * cp.ho * cp.wo * kpad * es);
+    const std::string keep_error = g_last_error;
+    // the padded problem ends in rock_conv_bwd_weight_* and the reduction kernel when the GEMM route took it
+    // (decided on the plan as a whole, whatever kernel_id asks for)
+    bool took = false;
+    int inner_count = 0;
+    {
+      OptMap probe = o;
+      probe["kernel_id"] = "0";
+      Handle *first = make_conv_bwd_weight(probe, inner);
+      inner_count = first ? first->kernel_count : 0;
+      delete first;
+      if (inner_count >= 2) {
+        probe["kernel_id"] = std::to_string(inner_count - 2);
+        Handle *gemm = make_conv_bwd_weight(probe, inner);
+        probe["kernel_id"] = std::to_string(inner_count - 1);
+        Handle *last = make_conv_bwd_weight(probe, inner);
+        took = gemm && last && gemm->kernel_name.rfind("rock_conv_bwd_weight_", 0) == 0 &&
+               last->kernel_name == "rock_reduce_splits";
+        delete gemm;
+        delete last;
+      }
+    }
+    Handle *sub = nullptr;
+    if (took) {
+      if (kid < 0 || kid > inner_count) {
+        set_error("conv: kernel_id out of range");
+        return nullptr;
+      }
+      OptMap o2 = o;
+      o2["kernel_id"] = std::to_string(kid == 0 ? 0 : kid - 1);
+      sub = make_conv_bwd_weight(o2, inner);
+      if (!sub)
+        return nullptr;
+    }
+    if (took) {
+      const int count = sub->kernel_count + 1;
+      const size_t workspace = (size_t)dy_bytes + sub->workspace_bytes;
+      if (kid == 0) {
+        delete sub;
+        auto *h = new Handle;
+        // dimensions in the destination's order n, h, w, g, k
+        const int64_t size[5] = {cp.n, cp.ho, cp.wo, 1, kpad}, src_size[5] = {cp.n, cp.ho, cp.wo, 1, cp.k};
+        const int64_t stride[5] = {cp.os[0], cp.os[3], cp.os[4], cp.os[1], cp.os[2]};
+        if (!fill_relayout_handle(h, size, src_size, stride, es)) {
+          delete h;
+          return nullptr;
+        }
+        h->ptr_map = {{2, 0}, {4, 0}};
+        h->problem_key = "relayout output gradient: channel runs padded to whole chunks";
+        h->kernel_count = count;
+        h->workspace_bytes = workspace;
+        h->caller_pointers = 5;
+        return h;
+      }
+      // the inner plan reads the copy; its own workspace lies behind it
+      for (auto &src : sub->ptr_map) {
+        if (src.source == 4)
+          src.offset += dy_bytes;
+        else if (src.source == 2)
+          src = Handle::PtrSrc{4, src.offset};
+      }
+      if (sub->op != OP_RELAYOUT)
+        sub->problem_key = conv_problem_key(sub, o, cp, 4);
+      sub->kernel_count = count;
+      sub->workspace_bytes = workspace;
+      sub->caller_pointers = 5;
+      return sub;
+    }
+    delete sub;
+    g_last_error = keep_error; // not taken: the plans below see the problem as it is
+  }
   RockConvParams q;
   std::memset(&q, 0, sizeof q);
   q.n = (int)cp.c; q.g = (int)cp.g; q.c = (int)cp.n; q.k = (int)cp.k;
@@ -1915,7 +2006,8 @@ Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
                        al(cp.os[4]);
     // a gradient whose (y, x, c) run is contiguous can be written by the GEMM itself when the pixels are
     // not split; any other layout is produced by the reduction kernel from the [k][y][x][c] partial sums
-    const bool dw_direct = cp.fs[2] == 1 && cp.fs[4] == cp.c && cp.fs[3] == cp.x * cp.c && cp.fs[1] >= Ng && al(cp.fs[1]);
+    const bool dw_direct = cp.fs[2] == 1 && cp.fs[4] == cp.c && cp.fs[3] == cp.x * cp.c && cp.fs[1] >= Ng && al(cp.fs[1]) &&
+                           !cp.k_valid;
     if (!(in_ok && dy_ok) && cp.y * cp.x > 1 && P <= INT32_MAX && Ng <= INT32_MAX) {
       // not channels-last: copies in that form first (the 1 x 1 case has its own plans below)
       bool applies = false;
@@ -1977,6 +2069,7 @@ Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
           std::memset(&r, 0, sizeof r);
           r.split_stride = cp.k * Ng;
           r.size[0] = (int)cp.k; r.size[1] = (int)cp.y; r.size[2] = (int)cp.x; r.size[3] = (int)cp.c;
+          r.valid[0] = (int)cp.k_valid;
           r.dst_stride[0] = cp.fs[1]; r.dst_stride[1] = cp.fs[3]; r.dst_stride[2] = cp.fs[4]; r.dst_stride[3] = cp.fs[2];
           r.splits = (int)S;
           r.out_dtype = cp.ti;

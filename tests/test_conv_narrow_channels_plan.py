@@ -153,3 +153,38 @@ def test_forward_reduction_split_plan_replayed_on_the_cpu(rock, case, il, fl, t,
         assert rock.RockKernel(opts + " --split_k false").kernel_count == first.kernel_count - 1
     else:
         assert "rock_reduce_splits" not in names
+
+
+# (n c k hi wi y x stride pad): an output gradient with a few channels
+NARROW_K_CASES = [
+    (2, 32, 4, 12, 12, 3, 3, 1, 1),      # a layer that ends in 4 channels
+    (3, 16, 3, 9, 11, 3, 3, 2, 1),
+    (2, 64, 12, 8, 8, 5, 5, 1, 2),       # 12 channels: one and a half chunks of 16 bits
+    (1, 8, 1, 10, 10, 2, 2, 1, 0),
+]
+
+
+@pytest.mark.parametrize("case", NARROW_K_CASES)
+@pytest.mark.parametrize("il,fl", [("nhwgc", "gkyxc"), ("ngchw", "gkcyx")])
+@pytest.mark.parametrize("t,es", [("fp16", 2), ("f32", 4)])
+def test_filter_gradient_of_a_narrow_output_gradient_replayed_on_the_cpu(rock, case, il, fl, t, es):
+    n, c, k, hi, wi, y, x, s, pd = case
+    if (c * es) % 16 or (k * es) % 16 == 0:
+        pytest.skip("not this route")
+    opts = conv(t, il, fl, n, c, hi, wi, k, y, x, stride=s, pad=pd, op="conv_bwd_weight")
+    ol = il.replace("c", "k")
+    ho, wo = (hi + 2 * pd - y) // s + 1, (wi + 2 * pd - x) // s + 1
+    rng = np.random.default_rng(14)
+    inp = rng.integers(-3, 4, n * c * hi * wi).astype(np.float32)
+    dout = rng.integers(-3, 4, n * k * ho * wo).astype(np.float32)
+    want, _, _ = orc.conv_bwd_weight(inp, dout, fl, il, ol, n, 1, c, k, hi, wi, y, x, (s, s), (pd, pd), (1, 1))
+    first = rock.RockKernel(opts)
+    dw = np.full(want.size, np.nan, np.float32)
+    ws = np.full(first.workspace_bytes // es, np.nan, np.float32)
+    tn = {"fp16": "f16"}.get(t, t)
+    names = _replay_plan(rock, opts, [dw, inp, dout, None, ws], tn, es)
+    assert np.array_equal(dw, want.ravel())
+    assert names[0].startswith("rock_relayout_b") and names[-2:] == ["rock_conv_bwd_weight_%s_64x64" % tn, "rock_reduce_splits"]
+    # a kernel_id behind the plan is an error, not another plan
+    with pytest.raises(rock.RockError):
+        rock.RockKernel(opts + " --kernel_id %d" % len(names))

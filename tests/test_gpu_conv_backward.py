@@ -243,3 +243,34 @@ def test_conv_bwd_weight_over_a_few_channels_exact(rock, oracle, gpu, case, layo
     ref, _, _ = oracle.conv_bwd_weight(iq, dyq, *layouts, n, g, c, k, hi, wi, y, x, stride, pad, dil)
     assert np.array_equal(to_f32(got, t), oracle.round_through(ref, CODE[t]))
     assert torch.equal(got.view(torch.uint8), old.view(torch.uint8))
+
+
+NARROW_K_CASES = [
+    (2, 1, 320, 4, 64, 64, 3, 3, (1, 1), (1, 1), (1, 1)),     # the UNet layer that ends in 4 channels
+    (2, 1, 32, 4, 12, 12, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (3, 1, 16, 3, 9, 11, 3, 3, (2, 2), (1, 1), (1, 1)),
+    (2, 1, 64, 12, 8, 8, 5, 5, (1, 1), (2, 2), (1, 1)),
+    (1, 1, 8, 1, 10, 10, 2, 2, (1, 1), (0, 0), (1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", NARROW_K_CASES)
+@pytest.mark.parametrize("layouts", [NHWC, NCHW], ids=lambda l: l[1])
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16"])
+def test_conv_bwd_weight_of_a_narrow_output_gradient_exact(rock, oracle, gpu, case, layouts, t):
+    """k * es not a whole chunk: the output gradient is copied with its channels padded with zeros, the
+    K-major GEMM runs over the copy and the reduction leaves the padding rows out."""
+    n, g, c, k, hi, wi, y, x, stride, pad, dil = case
+    es = 4 if t == "f32" else 2
+    _, (raw_i, iq), (raw_dy, dyq), ho, wo = _tensors(case, layouts, t, 89)
+    info, info_old = {}, {}
+    xi, dy = to_gpu(raw_i, t, gpu), to_gpu(raw_dy, t, gpu)
+    got = rock.conv2d_bwd_weight(xi, dy, info=info, **_kw(case, layouts))
+    old = rock.conv2d_bwd_weight(xi, dy, info=info_old, as_gemm=False, **_kw(case, layouts))
+    torch.cuda.synchronize()
+    if (c * es) % 16 == 0 and (k * es) % 16 != 0:
+        assert info["kernels"][-2:] == ["rock_conv_bwd_weight_%s_64x64" % t, "rock_reduce_splits"]
+        assert info["kernels"][0].startswith("rock_relayout_b")
+    ref, _, _ = oracle.conv_bwd_weight(iq, dyq, *layouts, n, g, c, k, hi, wi, y, x, stride, pad, dil)
+    assert np.array_equal(to_f32(got, t), oracle.round_through(ref, CODE[t]))
+    assert torch.equal(got.view(torch.uint8), old.view(torch.uint8))
