@@ -1445,9 +1445,28 @@ Handle *make_conv_bwd_data(const OptMap &o, const ConvProblem &cp) {
     }
     g_last_error = keep_error;
   }
+  // A single phase (unit stride) with few output tiles and a long reduction: the (taps, k) range split over
+  // blocks as in the forward direction (make_conv), partial sums in the workspace, a reduction kernel
+  // behind the contraction that writes the input gradient.
+  int64_t S = 1, k_part = 0, part_off = 0, part_bytes = 0;
+  if (fast && phases.size() == 1 && !win[0].ok && cp.g == 1 && !o.count("perf_config") && bool_or(o, "split_k", true)) {
+    const Phase &ph = phases[0];
+    const int64_t Mg = cp.n * ph.h.A * ph.w.A, Kfull = kp * ph.h.T * ph.w.T, step = 128 / es;
+    const int64_t tiles64 = (int64_t)ceil_div(Mg, 64) * ceil_div(cp.c, 64);
+    if (tiles64 <= 2 * kNumCU && Kfull >= 2048 && Mg * cp.c <= INT32_MAX) {
+      const int64_t want = std::min<int64_t>(4 * kNumCU / tiles64, Kfull / 1024);
+      for (int64_t d = want; d >= 2; --d)
+        if (Kfull % d == 0 && (Kfull / d) % step == 0) {
+          S = d;
+          k_part = Kfull / d;
+          part_bytes = align256(S * Mg * cp.c * 4);
+          break;
+        }
+    }
+  }
   // kernel list
   const int first_phase = (need_fill ? 1 : 0) + (fast && !dy_as_is ? 1 : 0);
-  const int per_phase = fast ? 2 : 1;
+  const int per_phase = fast ? (S > 1 ? 3 : 2) : 1;
   const int count = first_phase + per_phase * (int)phases.size();
   int64_t workspace = 0;
   std::vector<int64_t> fil_ws(phases.size(), 0);
@@ -1457,6 +1476,8 @@ Handle *make_conv_bwd_data(const OptMap &o, const ConvProblem &cp) {
       fil_ws[i] = workspace;
       workspace += win[i].ok ? win[i].filter_bytes : align256(cp.g * cp.c * phases[i].h.T * phases[i].w.T * kp * es);
     }
+    part_off = workspace;
+    workspace += part_bytes;
   }
   if (count == 0 || kid < 0 || kid >= count) {
     set_error(count == 0 ? "conv_bwd_data: empty problem" : "conv: kernel_id out of range");
@@ -1485,7 +1506,30 @@ Handle *make_conv_bwd_data(const OptMap &o, const ConvProblem &cp) {
     int64_t fil_off, out_off;
     const RockConvParams generic = phase_view(ph, fil_off, out_off);
     const WindowPlan &w = win[idx / per_phase];
-    if (fast && idx % 2 == 0) {
+    if (fast && idx % per_phase == 2) {
+      // the split's partial sums [S][n][a_h][a_w][c] added into the phase's positions of the input gradient
+      const int64_t Mg = cp.n * ph.h.A * ph.w.A;
+      RockReduceParams r;
+      std::memset(&r, 0, sizeof r);
+      r.split_stride = Mg * cp.c;
+      r.size[0] = (int)cp.n; r.size[1] = (int)ph.h.A; r.size[2] = (int)ph.w.A; r.size[3] = (int)cp.c;
+      r.dst_stride[0] = generic.out_ns; r.dst_stride[1] = generic.out_hs; r.dst_stride[2] = generic.out_ws;
+      r.dst_stride[3] = generic.out_ks;
+      r.splits = (int)S;
+      r.out_dtype = cp.ti;
+      h = new Handle;
+      h->op = OP_RELAYOUT;
+      h->epi = nullptr;
+      h->params.assign(sizeof r, 0);
+      std::memcpy(h->params.data(), &r, sizeof r);
+      h->kernel_name = "rock_reduce_splits";
+      h->block_size = 256;
+      h->grid_size = (uint32_t)((Mg * cp.c + 255) / 256);
+      h->num_pointers = 2;
+      h->perf_config = "";
+      h->ptr_map = {{ws, part_off}, {1, out_off * es}};
+      h->problem_key = "reduction of the split partial sums";
+    } else if (fast && idx % per_phase == 0) {
       // flipped sub-filter -> [g][c][T_h][T_w][kp], or fragment-major for the window-resident kernel
       h = new Handle;
       const int64_t size[5] = {cp.g, cp.c, ph.h.T, ph.w.T, kp}, src_size[5] = {cp.g, cp.c, ph.h.T, ph.w.T, cp.k};
@@ -1499,14 +1543,26 @@ Handle *make_conv_bwd_data(const OptMap &o, const ConvProblem &cp) {
       h->problem_key = "relayout filter phase " + std::to_string(ph.rh) + "," + std::to_string(ph.rw);
     } else {
       int64_t off2;
-      h = conv_handle_from_view(fast ? phase_fast_view(ph, off2) : generic, cp.ti, o);
+      RockConvParams view = fast ? phase_fast_view(ph, off2) : generic;
+      if (S > 1) { // the shares of the reduction as groups, each into its own f32 partial result
+        view.g = (int)S;
+        view.k_group_stride = (int)k_part;
+        view.in_gs = 0;
+        view.fil_gs = k_part;
+        view.out_ks = 1; view.out_ws = cp.c; view.out_hs = ph.w.A * cp.c; view.out_ns = ph.h.A * ph.w.A * cp.c;
+        view.out_gs = cp.n * view.out_ns;
+        view.epi.out_dtype = ROCK_F32;
+      }
+      h = conv_handle_from_view(view, cp.ti, o);
       if (!h)
         return nullptr;
+      if (S > 1)
+        reinterpret_cast<RockConvParams *>(h->params.data())->K = (int)k_part;
       if (w.ok)
         apply_window_plan(h, *reinterpret_cast<RockConvParams *>(h->params.data()), w, cp.ti, o);
       h->ptr_map = {fast ? Handle::PtrSrc{ws, fil_dst} : Handle::PtrSrc{0, fil_off * es},
                     (fast && !dy_as_is) ? Handle::PtrSrc{ws, 0} : Handle::PtrSrc{2, 0},
-                    {1, out_off * es}, {-1, 0}, {-1, 0}};
+                    S > 1 ? Handle::PtrSrc{ws, part_off} : Handle::PtrSrc{1, out_off * es}, {-1, 0}, {-1, 0}};
       h->problem_key = conv_problem_key(h, o, cp, 2);
     }
   }

@@ -188,3 +188,39 @@ def test_filter_gradient_of_a_narrow_output_gradient_replayed_on_the_cpu(rock, c
     # a kernel_id behind the plan is an error, not another plan
     with pytest.raises(rock.RockError):
         rock.RockKernel(opts + " --kernel_id %d" % len(names))
+
+
+# (n c k hi wi y x pad): unit stride, few tiles, k * taps >= 2048
+BWD_DATA_SPLIT_CASES = [
+    (2, 64, 256, 8, 8, 3, 3, 1),
+    (1, 40, 512, 6, 7, 2, 2, 0),       # ragged channels of the input gradient
+    (2, 24, 100, 5, 5, 5, 5, 2),       # 16-bit k padded to 104 by the conversion of the output gradient
+    (2, 128, 384, 6, 6, 3, 3, 1),      # three shares
+]
+
+
+@pytest.mark.parametrize("case", BWD_DATA_SPLIT_CASES)
+@pytest.mark.parametrize("il,fl", [("nhwgc", "gkyxc"), ("ngchw", "gkcyx")])
+@pytest.mark.parametrize("t,es", [("fp16", 2), ("f32", 4)])
+def test_backward_data_reduction_split_plan_replayed_on_the_cpu(rock, case, il, fl, t, es):
+    n, c, k, hi, wi, y, x, pd = case
+    opts = conv(t, il, fl, n, c, hi, wi, k, y, x, stride=1, pad=pd, op="conv_bwd_data")
+    ol = il.replace("c", "k")
+    ho, wo = hi + 2 * pd - y + 1, wi + 2 * pd - x + 1
+    rng = np.random.default_rng(15)
+    fil = rng.integers(-3, 4, k * c * y * x).astype(np.float32)
+    dout = rng.integers(-3, 4, n * k * ho * wo).astype(np.float32)
+    want, _, _ = orc.conv_bwd_data(fil, dout, fl, il, ol, n, 1, c, k, hi, wi, y, x, (1, 1), (pd, pd), (1, 1))
+    first = rock.RockKernel(opts)
+    dx = np.full(want.size, np.nan, np.float32)
+    ws = np.full(first.workspace_bytes // es, np.nan, np.float32)
+    tn = {"fp16": "f16"}.get(t, t)
+    names = _replay_plan(rock, opts, [fil, dx, dout, None, ws], tn, es)
+    assert np.array_equal(dx, want.ravel())
+    kfull = -(-k * es // 16) * 16 // es * y * x
+    most = min(1024 // (-(-n * hi * wi // 64) * -(-c // 64)), kfull // 1024)
+    if any(kfull % d == 0 and (kfull // d) % (128 // es) == 0 for d in range(2, most + 1)):
+        assert names[-1] == "rock_reduce_splits" and names[-2].startswith("rock_conv_%s_" % tn)
+        assert rock.RockKernel(opts + " --split_k false").kernel_count == first.kernel_count - 1
+    else:
+        assert "rock_reduce_splits" not in names

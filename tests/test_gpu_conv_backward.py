@@ -274,3 +274,33 @@ def test_conv_bwd_weight_of_a_narrow_output_gradient_exact(rock, oracle, gpu, ca
     ref, _, _ = oracle.conv_bwd_weight(iq, dyq, *layouts, n, g, c, k, hi, wi, y, x, stride, pad, dil)
     assert np.array_equal(to_f32(got, t), oracle.round_through(ref, CODE[t]))
     assert torch.equal(got.view(torch.uint8), old.view(torch.uint8))
+
+
+BWD_DATA_SPLIT_CASES = [
+    (2, 1, 320, 640, 16, 16, 3, 3, (1, 1), (1, 1), (1, 1)),    # a UNet layer at batch 2 in small
+    (2, 1, 64, 256, 8, 8, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (1, 1, 40, 512, 6, 7, 2, 2, (1, 1), (0, 0), (1, 1)),
+    (2, 1, 24, 100, 5, 5, 5, 5, (1, 1), (2, 2), (1, 1)),
+    (2, 1, 128, 384, 6, 6, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (2, 1, 72, 256, 9, 7, 3, 3, (1, 1), (1, 1), (2, 1)),       # dilated rows
+]
+
+
+@pytest.mark.parametrize("case", BWD_DATA_SPLIT_CASES)
+@pytest.mark.parametrize("layouts", LAYOUTS, ids=lambda l: l[1])
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16"])
+def test_conv_bwd_data_reduction_split_exact(rock, oracle, gpu, case, layouts, t):
+    """Unit stride, few output tiles, a long reduction over (taps, k): shares of the reduction as groups,
+    partial sums added by the reduction kernel into the input gradient."""
+    n, g, c, k, hi, wi, y, x, stride, pad, dil = case
+    (raw_f, fq), _, (raw_dy, dyq), ho, wo = _tensors(case, layouts, t, 97)
+    info = {}
+    got = rock.conv2d_bwd_data(to_gpu(raw_f, t, gpu), to_gpu(raw_dy, t, gpu), info=info, **_kw(case, layouts))
+    torch.cuda.synchronize()
+    ref, _, _ = oracle.conv_bwd_data(fq, dyq, *layouts, n, g, c, k, hi, wi, y, x, stride, pad, dil)
+    assert np.array_equal(to_f32(got, t), oracle.round_through(ref, CODE[t]))
+    es = 4 if t == "f32" else 2
+    kfull = -(-k * es // 16) * 16 // es * y * x
+    most = min(1024 // (-(-n * hi * wi // 64) * -(-c // 64)), kfull // 1024)
+    if any(kfull % d == 0 and (kfull // d) % (128 // es) == 0 for d in range(2, most + 1)):
+        assert info["kernels"][-1] == "rock_reduce_splits"
