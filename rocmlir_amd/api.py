@@ -340,7 +340,11 @@ class RockProgram:
 
     @property
     def main(self):
-        """The contraction kernel (the last of the problem)."""
+        """The contraction kernel: the last GEMM, convolution or attention kernel of the list (conversion
+        kernels may run in front of it, the reduction of split partial sums behind it)."""
+        for k in reversed(self.kernels):
+            if k.kernel_name.startswith(("rock_gemm_", "rock_conv_", "rock_attention_")):
+                return k
         return self.kernels[-1]
 
     # what rocmlir_amd.tuning.tune() uses, so that problems of several kernels tune like single ones

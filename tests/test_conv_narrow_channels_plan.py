@@ -224,3 +224,13 @@ def test_backward_data_reduction_split_plan_replayed_on_the_cpu(rock, case, il, 
         assert rock.RockKernel(opts + " --split_k false").kernel_count == first.kernel_count - 1
     else:
         assert "rock_reduce_splits" not in names
+
+
+def test_program_reports_its_contraction_kernel(rock):
+    """A plan that ends in the reduction kernel still answers with the contraction kernel's name, perf_config
+    and problem key (what the tuner records)."""
+    opts = conv("fp16", "nhwgc", "gkyxc", 2, 640, 16, 16, 320, 3, 3, pad=1)
+    prog = rock.RockProgram(opts)
+    assert [k.kernel_name for k in prog.kernels][-1] == "rock_reduce_splits"
+    assert prog.kernel_name.startswith("rock_conv_f16_") and prog.perf_config.startswith("v2:")
+    assert "convfp16" in prog.problem_key and " -c 640 " in prog.problem_key
