@@ -163,10 +163,12 @@ template <int DT, int ROWS, int NW, int RB, bool RUNS = false> struct ConvInDl {
     run_valid = cp.run_valid;
     // first element of this group's share of the reduction (0 unless the reduction is split over the groups)
     const int kstart = g * cp.k_group_stride;
+    // n / d for 0 <= n < 2^31 with the plan's multiply-and-shift constants
+    auto div = [](int n, const RockFastDiv &d) { return (int)(((uint64_t)(unsigned)n * d.mul) >> d.shift); };
     {
-      const int tap0 = kstart / cp.c;
+      const int tap0 = div(kstart, cp.div_c);
       uc0 = (kstart - tap0 * cp.c) * ES;
-      uy = tap0 / cp.x;
+      uy = div(tap0, cp.div_x);
       ux = tap0 - uy * cp.x;
     }
     {
@@ -184,9 +186,9 @@ template <int DT, int ROWS, int NW, int RB, bool RUNS = false> struct ConvInDl {
       int r = (wave * Sg::PER_WAVE + i) * Dg::SLAB_ROWS + lane / Dg::CHUNKS;
       int m = row0 + r;
       int mm = min(m, cp.M - 1);
-      int n = mm / (cp.ho * cp.wo);
+      int n = div(mm, cp.div_image);
       int rem = mm - n * (cp.ho * cp.wo);
-      int ho = rem / cp.wo;
+      int ho = div(rem, cp.div_row);
       int wo = rem - ho * cp.wo;
       h0[i] = ho * cp.stride_h - cp.pad_h;
       w0[i] = wo * cp.stride_w - cp.pad_w;
@@ -194,9 +196,9 @@ template <int DT, int ROWS, int NW, int RB, bool RUNS = false> struct ConvInDl {
       int lc = (lane % Dg::CHUNKS) ^ Dg::swz(r);
       kb[i] = lc * kChunk;
       int k0 = kstart + lc * EPC;
-      int tap = k0 / cp.c;
+      int tap = div(k0, cp.div_c);
       cc[i] = k0 - tap * cp.c;
-      y[i] = tap / cp.x;
+      y[i] = div(tap, cp.div_x);
       x[i] = tap - y[i] * cp.x;
       tapoff[i] = kOobOffset;
     }

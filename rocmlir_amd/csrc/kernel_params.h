@@ -76,6 +76,12 @@ struct RockGemmParams {
 // Forward convolution as an implicit GEMM:
 //   M = N*Ho*Wo (output pixels), N = K_out per group, K = Y*X*C per group.
 // Strides are in elements of the respective tensor.
+// Division of a block or chunk index (below 2^31) by a divisor fixed at plan
+// time: n / d == (n * mul) >> shift in 64-bit arithmetic, with
+// mul = ceil(2^shift / d) and shift = 31 + ceil(log2 d).
+struct RockFastDiv {
+  uint32_t mul, shift;
+};
 struct RockConvParams {
   int64_t in_ns, in_gs, in_cs, in_hs, in_ws;
   int64_t fil_gs, fil_ks, fil_cs, fil_ys, fil_xs;
@@ -97,6 +103,9 @@ struct RockConvParams {
   // reduces the elements [s * k_group_stride, s * k_group_stride + K) of every row of taps-and-channels,
   // a whole number of K-steps, into an f32 partial result of its own (in_gs = 0, fil_gs = K).  0 elsewhere.
   int32_t k_group_stride;
+  // plan-time constants for the divisions of the fast loader's set-up (row -> image, output row, output
+  // pixel; reduction index -> tap, channel; tap -> filter row, filter column): by ho * wo, wo, c, x
+  RockFastDiv div_image, div_row, div_c, div_x;
 };
 
 // Filter gradient of a convolution as one K-major GEMM over the tensors as they
@@ -125,12 +134,6 @@ enum RockRelayoutMode {
   RELAYOUT_TRANSPOSE = 0, // contiguous dimensions differ: tile_d x (1024/tile_d) tiles through LDS
   RELAYOUT_COPY = 1,      // one 16-byte destination chunk (along dimension 4) per thread
   RELAYOUT_TRANSPOSE_VEC = 2, // as TRANSPOSE with 16-byte accesses: tiles of tile_d x (AREA / tile_d), relayout_body.h
-};
-// Division of a block or chunk index (below 2^31) by a divisor fixed at plan
-// time: n / d == (n * mul) >> shift in 64-bit arithmetic, with
-// mul = ceil(2^shift / d) and shift = 31 + ceil(log2 d).
-struct RockFastDiv {
-  uint32_t mul, shift;
 };
 struct RockRelayoutParams {
   int64_t src_stride[5], dst_stride[5]; // in elements

@@ -3809,6 +3809,14 @@ Handle *build_handle(const OptMap &o) {
     return nullptr;
   }
   h->num_cu = (int)int_or(o, "num_cu", kNumCU);
+  if (h->op == OP_CONV && h->params.size() == sizeof(RockConvParams)) {
+    // every plan's convolution kernels leave through here: the division constants of the loader's set-up
+    auto &cpar = *reinterpret_cast<RockConvParams *>(h->params.data());
+    cpar.div_image = fast_div_of(std::max<int64_t>(1, (int64_t)cpar.ho * cpar.wo));
+    cpar.div_row = fast_div_of(std::max<int64_t>(1, cpar.wo));
+    cpar.div_c = fast_div_of(std::max<int64_t>(1, cpar.c));
+    cpar.div_x = fast_div_of(std::max<int64_t>(1, cpar.x));
+  }
   h->blob = find_blob(h->kernel_name);
   if (!h->blob) {
     set_error("no code object for " + h->kernel_name);
