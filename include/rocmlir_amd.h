@@ -90,10 +90,11 @@ typedef void *MiirHandle;
  * bwd_weight_gemm (the filter gradient of a one-group convolution as one
  * K-major GEMM plus the reduction of its pixel splits), window_resident (a
  * 16-bit or int8 stride-1 convolution whose tiles fill on the kernel that keeps the
- * input window in LDS, behind a conversion of the filter), split_k (a GEMM or
- * forward convolution with few output tiles and a long reduction split over
- * blocks, f32 partial sums in the workspace, a reduction kernel behind the
- * contraction; identity epilogue only), tap_rows (a convolution over pixels of a few channels, without
+ * input window in LDS, behind a conversion of the filter), split_k (a GEMM,
+ * forward convolution or unit-stride input gradient with few output tiles and
+ * a long reduction split over blocks, f32 (int8 operands: int32) partial sums
+ * in the workspace, a reduction kernel behind the contraction; identity
+ * epilogue only), tap_rows (a convolution over pixels of a few channels, without
  * padding or dilation along w, reads a row of filter taps as one run of
  * neighbouring pixels: conversions of both tensors, then a "_runs" kernel),
  * fused (attention, above).  A single leading dash and "key=value"
