@@ -97,6 +97,9 @@ typedef void *MiirHandle;
  * epilogue only), tap_rows (a convolution over pixels of a few channels, without
  * padding or dilation along w, reads a row of filter taps as one run of
  * neighbouring pixels: conversions of both tensors, then a "_runs" kernel),
+ * merge_phases (the input gradient of a strided layer whose phases times
+ * channels fit 64 output columns: all phases in one convolution over the union
+ * of their windows, a conversion kernel puts the positions together),
  * fused (attention, above).  A single leading dash and "key=value"
  * are accepted as well.  rocmlir-gen's scheduling and instruction-set toggles
  * (reverse_grid, mfma, wmma, dot, x2) are accepted and ignored, and so is

@@ -884,10 +884,15 @@ bool fill_relayout_handle(Handle *h, const int64_t size[5], const int64_t src_si
   if (positions_per_chunk == 1 && r.src_fast == r.dst_fast && ((int64_t)r.size[4] * es) % 16 != 0) {
     // runs along the shared contiguous dimension that are not whole 16-byte
     // chunks (an output with 12 f16 channels): element-wise tiles over that
-    // dimension and the longest other one
+    // dimension and another one: of those long enough to fill a tile's rows
+    // the one whose runs lie closest together in the source, else the longest
     r.src_fast = 3;
     for (int d = 0; d < 4; ++d)
       if (r.size[d] > r.size[r.src_fast])
+        r.src_fast = d;
+    for (int d = 0; d < 4; ++d)
+      if (r.size[d] >= 32 && r.src_stride[d] != 0 &&
+          (r.size[r.src_fast] < 32 || std::llabs(r.src_stride[d]) < std::llabs(r.src_stride[r.src_fast])))
         r.src_fast = d;
   }
   int64_t blocks = 1;
@@ -1408,6 +1413,127 @@ Handle *make_conv_bwd_data(const OptMap &o, const ConvProblem &cp) {
   for (const Phase &ph : phases) {
     int64_t unused;
     fast = fast && conv_view_fast(phase_fast_view(ph, unused), es);
+  }
+  // A strided layer with few input channels (the 3-channel first layer): each phase alone fills 3 of the 64
+  // output columns of a tile.  The phases read the same neighbourhood of the output gradient, so they run as
+  // ONE unit-stride convolution whose output columns are (phase, channel): its window is the union of the
+  // offsets that any phase reaches, its filter [(phase, c)][u_h][u_w][k] holds every phase's flipped taps at
+  // their offsets and zeros elsewhere, and its output T[n][b_h][b_w][(j_h, j_w, c)] (in the workspace) is the
+  // input gradient with the position i = stride * b + j taken apart; a conversion kernel puts it together.
+  // Kernels: [output gradient copy], zero fill of the filter, one filter conversion per phase, the
+  // convolution, T -> channels-last gradient, [-> the caller's layout].
+  if (fast && phases.size() > 1 && (int64_t)phases.size() == cp.sh * cp.sw && !need_fill && cp.g == 1 &&
+      cp.dh == 1 && cp.dw == 1 && cp.hi % cp.sh == 0 && cp.wi % cp.sw == 0 && (int64_t)phases.size() * cp.c <= 64 &&
+      bool_or(o, "merge_phases", true)) {
+    const int64_t P = (int64_t)phases.size(), Bh = cp.hi / cp.sh, Bw = cp.wi / cp.sw, cols = P * cp.c;
+    int64_t lo_h = INT64_MAX, hi_h = INT64_MIN, lo_w = INT64_MAX, hi_w = INT64_MIN;
+    bool regular = true;
+    for (const Phase &ph : phases) {
+      const int64_t eh = ph.h.a_min + ph.h.o_first, ew = ph.w.a_min + ph.w.o_first;
+      lo_h = std::min(lo_h, eh - (ph.h.T - 1)); hi_h = std::max(hi_h, eh);
+      lo_w = std::min(lo_w, ew - (ph.w.T - 1)); hi_w = std::max(hi_w, ew);
+      regular = regular && ph.h.dd == 1 && ph.w.dd == 1 && ph.h.A == Bh && ph.w.A == Bw;
+    }
+    const int64_t Uh = hi_h - lo_h + 1, Uw = hi_w - lo_w + 1;
+    RockConvParams q;
+    std::memset(&q, 0, sizeof q);
+    q.n = (int)cp.n; q.g = 1; q.c = (int)kp; q.k = (int)cols;
+    q.hi = (int)cp.ho; q.wi = (int)cp.wo; q.y = (int)Uh; q.x = (int)Uw; q.ho = (int)Bh; q.wo = (int)Bw;
+    q.stride_h = q.stride_w = q.dil_h = q.dil_w = 1;
+    q.pad_h = (int)-lo_h; q.pad_w = (int)-lo_w;
+    if (dy_as_is) {
+      q.in_ns = cp.os[0]; q.in_gs = cp.os[1]; q.in_cs = cp.os[2]; q.in_hs = cp.os[3]; q.in_ws = cp.os[4];
+    } else {
+      q.in_cs = 1; q.in_gs = kp; q.in_ws = kp; q.in_hs = cp.wo * kp; q.in_ns = cp.ho * q.in_hs;
+    }
+    q.fil_cs = 1; q.fil_xs = kp; q.fil_ys = Uw * kp; q.fil_ks = Uh * Uw * kp; q.fil_gs = cols * q.fil_ks;
+    q.out_ks = 1; q.out_ws = cols; q.out_hs = Bw * cols; q.out_ns = Bh * Bw * cols; q.out_gs = 0;
+    default_epilogue(q.epi, cp.ti);
+    // the gradient in the caller's tensor when that is dense channels-last, else by way of such a copy
+    const bool cl = cp.is[2] == 1 && cp.is[4] == cp.c && cp.is[3] == cp.wi * cp.c && cp.is[0] == cp.hi * cp.wi * cp.c;
+    std::vector<ViewDim> to_layout = {{cp.n, cp.n, cp.hi * cp.wi * cp.c, cp.is[0]}, {cp.c, cp.c, 1, cp.is[2]},
+                                      {cp.hi, cp.hi, cp.wi * cp.c, cp.is[3]}, {cp.wi, cp.wi, cp.c, cp.is[4]}};
+    std::stable_sort(to_layout.begin(), to_layout.end(), [](const ViewDim &a, const ViewDim &b) { return a.ds > b.ds; });
+    const std::vector<ViewDim> scatter = {{cp.n, cp.n, Bh * Bw * cols, cp.hi * cp.wi * cp.c},
+                                          {Bh, Bh, Bw * cols, cp.sh * cp.wi * cp.c},
+                                          {cp.sh, cp.sh, cp.sw * cp.c, cp.wi * cp.c},
+                                          {Bw, Bw, cols, cp.sw * cp.c},
+                                          {cp.sw * cp.c, cp.sw * cp.c, 1, 1}};
+    bool take = regular && lo_h <= 0 && lo_w <= 0 && conv_view_fast(q, es) && (cl || to_layout.back().ds == 1) &&
+                cp.n * cp.hi * cp.wi * cp.c <= INT32_MAX;
+    if (take) {
+      const std::string keep_error = g_last_error;
+      Handle probe;
+      take = relayout_handle_nd(&probe, scatter, es, "input gradient") &&
+             (cl || relayout_handle_nd(&probe, to_layout, es, "input gradient"));
+      g_last_error = keep_error;
+    }
+    if (take) {
+      const int64_t fil_off_ws = dy_bytes, t_off = fil_off_ws + align256(cols * Uh * Uw * kp * es);
+      const int64_t cl_off = t_off + align256(cp.n * Bh * Bw * cols * es);
+      const int64_t total = cl_off + (cl ? 0 : align256(cp.n * cp.hi * cp.wi * cp.c * es));
+      const int pre = dy_as_is ? 0 : 1, count = pre + 1 + (int)P + 2 + (cl ? 0 : 1);
+      if (kid < 0 || kid >= count) {
+        set_error("conv: kernel_id out of range");
+        return nullptr;
+      }
+      const int ws = 4;
+      Handle *h = nullptr;
+      int idx = kid - pre;
+      if (idx < 0) {
+        h = new Handle;
+        const int64_t size[5] = {cp.n, cp.ho, cp.wo, 1, kp}, src_size[5] = {cp.n, cp.ho, cp.wo, 1, cp.k};
+        const int64_t stride[5] = {cp.os[0], cp.os[3], cp.os[4], cp.os[1], cp.os[2]};
+        if (!fill_relayout_handle(h, size, src_size, stride, es)) {
+          delete h;
+          return nullptr;
+        }
+        h->ptr_map = {{2, 0}, {ws, 0}};
+        h->problem_key = "relayout output gradient " + cp.ol;
+      } else if (idx == 0) {
+        h = utility_fill_handle(cols * Uh * Uw * kp * es);
+        h->ptr_map = {{ws, fil_off_ws}};
+        h->problem_key = "zero fill of the merged filter";
+      } else if (idx <= P) {
+        const Phase &ph = phases[idx - 1];
+        int64_t fil_off, out_off;
+        const RockConvParams generic = phase_view(ph, fil_off, out_off);
+        // the phase's columns and where its window starts inside the union
+        const int64_t jh = cp.sh * ph.h.a_min + ph.rh - cp.ph, jw = cp.sw * ph.w.a_min + ph.rw - cp.pw;
+        const int64_t uh0 = ph.h.a_min + ph.h.o_first - (ph.h.T - 1) - lo_h, uw0 = ph.w.a_min + ph.w.o_first - (ph.w.T - 1) - lo_w;
+        const int64_t size[5] = {1, cp.c, ph.h.T, ph.w.T, kp}, src_size[5] = {1, cp.c, ph.h.T, ph.w.T, cp.k};
+        const int64_t stride[5] = {generic.fil_gs, generic.fil_ks, generic.fil_ys, generic.fil_xs, generic.fil_cs};
+        const int64_t dst_stride[5] = {q.fil_gs, q.fil_ks, q.fil_ys, q.fil_xs, 1};
+        h = new Handle;
+        if (!fill_relayout_handle(h, size, src_size, stride, es, dst_stride)) {
+          delete h;
+          return nullptr;
+        }
+        const int64_t dst_off = (jh * cp.sw + jw) * cp.c * q.fil_ks + uh0 * q.fil_ys + uw0 * q.fil_xs;
+        h->ptr_map = {{0, fil_off * es}, {ws, fil_off_ws + dst_off * es}};
+        h->problem_key = "relayout filter phase " + std::to_string(ph.rh) + "," + std::to_string(ph.rw);
+      } else if (idx == P + 1) {
+        h = conv_handle_from_view(q, cp.ti, o);
+        if (!h)
+          return nullptr;
+        h->ptr_map = {{ws, fil_off_ws}, dy_as_is ? Handle::PtrSrc{2, 0} : Handle::PtrSrc{ws, 0}, {ws, t_off}, {-1, 0}, {-1, 0}};
+        h->problem_key = conv_problem_key(h, o, cp, 2);
+      } else {
+        h = new Handle;
+        const bool last = idx == P + 3;
+        if (!relayout_handle_nd(h, last ? to_layout : scatter, es, "input gradient")) {
+          delete h;
+          return nullptr;
+        }
+        h->ptr_map = last ? std::vector<Handle::PtrSrc>{{ws, cl_off}, {1, 0}}
+                          : std::vector<Handle::PtrSrc>{{ws, t_off}, cl ? Handle::PtrSrc{1, 0} : Handle::PtrSrc{ws, cl_off}};
+        h->problem_key = last ? "relayout input gradient " + cp.il : "phases of the input gradient put together";
+      }
+      h->kernel_count = count;
+      h->workspace_bytes = (size_t)total;
+      h->caller_pointers = 5;
+      return h;
+    }
   }
   // Phases that the window-resident kernel takes (unit stride: the one phase there is): the conversion of the
   // flipped sub-filter then writes it fragment-major,

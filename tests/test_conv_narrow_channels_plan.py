@@ -234,3 +234,61 @@ def test_program_reports_its_contraction_kernel(rock):
     assert [k.kernel_name for k in prog.kernels][-1] == "rock_reduce_splits"
     assert prog.kernel_name.startswith("rock_conv_f16_") and prog.perf_config.startswith("v2:")
     assert "convfp16" in prog.problem_key and " -c 640 " in prog.problem_key
+
+
+# (n, c, k, hi, wi, y, x, stride, pad)
+MERGED_PHASE_CASES = [
+    (2, 3, 8, 20, 16, 7, 7, 2, 0),    # the first layer's shape in small: windows of 4 and 3 taps
+    (2, 3, 8, 16, 16, 7, 7, 2, 3),    # padded: the phases start at different rows
+    (1, 4, 16, 12, 12, 3, 3, 2, 1),
+    (1, 2, 8, 12, 18, 5, 5, 3, 2),    # nine phases
+    (2, 16, 8, 8, 8, 3, 3, 2, 1),     # 64 merged columns
+    (1, 3, 5, 12, 12, 3, 3, 2, 1),    # k padded to whole chunks
+]
+
+
+@pytest.mark.parametrize("t,es", [("fp16", 2), ("f32", 4)])
+@pytest.mark.parametrize("il,fl", [("nhwgc", "gkyxc"), ("ngchw", "gkcyx")])
+@pytest.mark.parametrize("case", MERGED_PHASE_CASES)
+def test_backward_data_merged_phases_plan_replayed_on_the_cpu(rock, case, il, fl, t, es):
+    """A strided layer with few input channels computes all its phases in one convolution with (phase, channel)
+    output columns; a conversion kernel interleaves them into the input gradient."""
+    n, c, k, hi, wi, y, x, st, pd = case
+    ho, wo = (hi + 2 * pd - y) // st + 1, (wi + 2 * pd - x) // st + 1
+    opts = conv(t, il, fl, n, c, hi, wi, k, y, x, stride=st, pad=pd, op="conv_bwd_data")
+    ol = il.replace("c", "k")
+    rng = np.random.default_rng(16)
+    fil = rng.integers(-3, 4, k * c * y * x).astype(np.float32)
+    dout = rng.integers(-3, 4, n * k * ho * wo).astype(np.float32)
+    want, _, _ = orc.conv_bwd_data(fil, dout, fl, il, ol, n, 1, c, k, hi, wi, y, x, (st, st), (pd, pd), (1, 1))
+    first = rock.RockKernel(opts)
+    dx = np.full(want.size, np.nan, np.float32)
+    ws = np.full(first.workspace_bytes // es, np.nan, np.float32)
+    tn = {"fp16": "f16"}.get(t, t)
+    names = _replay_plan(rock, opts, [fil, dx, dout, None, ws], tn, es)
+    assert np.array_equal(dx, want.ravel())
+    assert sum(nm.startswith("rock_conv_") for nm in names) == 1 and names.count("rock_fill_zero") == 1
+    # switched off: one convolution per phase
+    off = rock.RockKernel(opts + " --merge_phases false")
+    names_off = [rock.RockKernel(opts + " --merge_phases false --kernel_id %d" % i).kernel_name
+                 for i in range(off.kernel_count)]
+    assert sum(nm.startswith("rock_conv_") for nm in names_off) == st * st
+
+
+@pytest.mark.parametrize("extra,why", [
+    (dict(c=32), "too many merged columns"),
+    (dict(hi=15), "phases of different sizes"),
+    (dict(dilation=2), "dilated"),
+])
+def test_backward_data_merged_phases_declined(rock, extra, why):
+    kw = dict(c=3, hi=16, dilation=1)
+    kw.update(extra)
+    opts = conv("fp16", "nhwgc", "gkyxc", 2, kw["c"], kw["hi"], 16, 8, 3, 3, stride=2, pad=1, op="conv_bwd_data")
+    if kw["dilation"] != 1:  # same output size: (16 + 2*2 - 5) // 2 + 1 == 8
+        opts = opts.replace("--dilation_h 1 --dilation_w 1", "--dilation_h 2 --dilation_w 2").replace(
+            "--padding_h 1 --padding_w 1", "--padding_h 2 --padding_w 2")
+    first = rock.RockKernel(opts)
+    names = [rock.RockKernel(opts + " --kernel_id %d" % i).kernel_name for i in range(first.kernel_count)]
+    off = opts + " --merge_phases false"
+    assert names == [rock.RockKernel(off + " --kernel_id %d" % i).kernel_name
+                     for i in range(rock.RockKernel(off).kernel_count)], why

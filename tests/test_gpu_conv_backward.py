@@ -304,3 +304,31 @@ def test_conv_bwd_data_reduction_split_exact(rock, oracle, gpu, case, layouts, t
     most = min(1024 // (-(-n * hi * wi // 64) * -(-c // 64)), kfull // 1024)
     if any(kfull % d == 0 and (kfull // d) % (128 // es) == 0 for d in range(2, most + 1)):
         assert info["kernels"][-1] == "rock_reduce_splits"
+
+
+MERGED_PHASE_CASES = [
+    (4, 1, 3, 64, 46, 46, 7, 7, (2, 2), (0, 0), (1, 1)),      # the first layer in small
+    (2, 1, 3, 64, 32, 32, 7, 7, (2, 2), (3, 3), (1, 1)),      # padded: the phases start at different rows
+    (3, 1, 4, 16, 12, 20, 3, 3, (2, 2), (1, 1), (1, 1)),
+    (1, 1, 2, 24, 12, 18, 5, 5, (3, 3), (2, 2), (1, 1)),      # nine phases
+    (2, 1, 16, 40, 16, 16, 3, 3, (2, 2), (1, 1), (1, 1)),     # 64 merged columns
+    (2, 1, 3, 5, 12, 12, 3, 3, (2, 2), (1, 1), (1, 1)),       # k padded to whole chunks
+    (2, 1, 1, 32, 16, 16, 4, 4, (2, 2), (1, 1), (1, 1)),      # one channel: runs of two elements
+]
+
+
+@pytest.mark.parametrize("case", MERGED_PHASE_CASES)
+@pytest.mark.parametrize("layouts", LAYOUTS, ids=lambda l: l[1])
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16"])
+def test_conv_bwd_data_merged_phases_exact(rock, oracle, gpu, case, layouts, t):
+    """A strided layer with few input channels: every phase in one convolution with (phase, channel) output
+    columns, interleaved into the input gradient by a conversion kernel."""
+    n, g, c, k, hi, wi, y, x, stride, pad, dil = case
+    (raw_f, fq), _, (raw_dy, dyq), ho, wo = _tensors(case, layouts, t, 98)
+    info = {}
+    got = rock.conv2d_bwd_data(to_gpu(raw_f, t, gpu), to_gpu(raw_dy, t, gpu), info=info, **_kw(case, layouts))
+    torch.cuda.synchronize()
+    ref, _, _ = oracle.conv_bwd_data(fq, dyq, *layouts, n, g, c, k, hi, wi, y, x, stride, pad, dil)
+    assert np.array_equal(to_f32(got, t), oracle.round_through(ref, CODE[t]))
+    names = info["kernels"]
+    assert sum(nm.startswith("rock_conv_") for nm in names) == 1 and "rock_fill_zero" in names, names
