@@ -1454,17 +1454,21 @@ Handle *make_conv_bwd_data(const OptMap &o, const ConvProblem &cp) {
     std::vector<ViewDim> to_layout = {{cp.n, cp.n, cp.hi * cp.wi * cp.c, cp.is[0]}, {cp.c, cp.c, 1, cp.is[2]},
                                       {cp.hi, cp.hi, cp.wi * cp.c, cp.is[3]}, {cp.wi, cp.wi, cp.c, cp.is[4]}};
     std::stable_sort(to_layout.begin(), to_layout.end(), [](const ViewDim &a, const ViewDim &b) { return a.ds > b.ds; });
-    const std::vector<ViewDim> scatter = {{cp.n, cp.n, Bh * Bw * cols, cp.hi * cp.wi * cp.c},
-                                          {Bh, Bh, Bw * cols, cp.sh * cp.wi * cp.c},
-                                          {cp.sh, cp.sh, cp.sw * cp.c, cp.wi * cp.c},
-                                          {Bw, Bw, cols, cp.sw * cp.c},
-                                          {cp.sw * cp.c, cp.sw * cp.c, 1, 1}};
+    // (moved as 4-byte words when the runs of s_w * c elements are whole words: every stride and offset is
+    // a multiple of such a run)
+    const int64_t wide = (es < 4 && (cp.sw * cp.c * es) % 4 == 0) ? 4 / es : 1;
+    const int es_scatter = (int)(es * wide);
+    const std::vector<ViewDim> scatter = {{cp.n, cp.n, Bh * Bw * cols / wide, cp.hi * cp.wi * cp.c / wide},
+                                          {Bh, Bh, Bw * cols / wide, cp.sh * cp.wi * cp.c / wide},
+                                          {cp.sh, cp.sh, cp.sw * cp.c / wide, cp.wi * cp.c / wide},
+                                          {Bw, Bw, cols / wide, cp.sw * cp.c / wide},
+                                          {cp.sw * cp.c / wide, cp.sw * cp.c / wide, 1, 1}};
     bool take = regular && lo_h <= 0 && lo_w <= 0 && conv_view_fast(q, es) && (cl || to_layout.back().ds == 1) &&
                 cp.n * cp.hi * cp.wi * cp.c <= INT32_MAX;
     if (take) {
       const std::string keep_error = g_last_error;
       Handle probe;
-      take = relayout_handle_nd(&probe, scatter, es, "input gradient") &&
+      take = relayout_handle_nd(&probe, scatter, es_scatter, "input gradient") &&
              (cl || relayout_handle_nd(&probe, to_layout, es, "input gradient"));
       g_last_error = keep_error;
     }
@@ -1521,7 +1525,7 @@ Handle *make_conv_bwd_data(const OptMap &o, const ConvProblem &cp) {
       } else {
         h = new Handle;
         const bool last = idx == P + 3;
-        if (!relayout_handle_nd(h, last ? to_layout : scatter, es, "input gradient")) {
+        if (!relayout_handle_nd(h, last ? to_layout : scatter, last ? es : es_scatter, "input gradient")) {
           delete h;
           return nullptr;
         }

@@ -165,7 +165,12 @@ def test_conv3d_plan_replayed_on_the_cpu(rock, case, layouts, t, es):
             buffers[src][off // es:(off + nbytes) // es] = 0
         elif kern.kernel_name.startswith("rock_relayout"):
             (s_src, s_off), (d_src, d_off) = pm
-            _replay_relayout(kern.params(), buffers[s_src], s_off // es, buffers[d_src], d_off // es)
+            # a kernel that moves words of several elements: once per element of the word
+            wide = int(kern.kernel_name[len("rock_relayout_b"):]) // es
+            assert wide >= 1 and s_off % (es * wide) == 0 and d_off % (es * wide) == 0
+            for part in range(wide):
+                _replay_relayout(kern.params(), buffers[s_src][part::wide], s_off // (es * wide),
+                                 buffers[d_src][part::wide], d_off // (es * wide))
         else:
             assert kern.kernel_name.startswith("rock_conv_" + t)
             (f_src, f_off), (i_src, i_off), (o_src, o_off) = pm[:3]
@@ -249,7 +254,12 @@ def _replay_plan(rock, opts, buffers, t, es):
             buffers[src][off // es:(off + nbytes) // es] = 0
         elif name.startswith("rock_relayout_b"):
             (s_src, s_off), (d_src, d_off) = pm
-            _replay_relayout(kern.params(), buffers[s_src], s_off // es, buffers[d_src], d_off // es)
+            # a kernel that moves words of several elements: once per element of the word
+            wide = int(kern.kernel_name[len("rock_relayout_b"):]) // es
+            assert wide >= 1 and s_off % (es * wide) == 0 and d_off % (es * wide) == 0
+            for part in range(wide):
+                _replay_relayout(kern.params(), buffers[s_src][part::wide], s_off // (es * wide),
+                                 buffers[d_src][part::wide], d_off // (es * wide))
         elif name == "rock_fold_depth":
             (s_src, s_off), (d_src, d_off) = pm
             _replay_fold(kern.params(), buffers[s_src], s_off // es, buffers[d_src], d_off // es)
