@@ -106,6 +106,7 @@ BWD_CASES = [
     (3, 1, 8, 8, (4, 4, 9), (1, 1, 5), (1, 1, 3), (0, 0, 2), (1, 1, 1)),       # taps along depth only, depth stride 3
     (1, 1, 16, 8, (5, 5, 6), (3, 3, 3), (1, 1, 1), (0, 0, 0), (1, 1, 1)),      # one image: output gradient read in place
     (2, 1, 16, 16, (4, 5, 1), (3, 3, 1), (1, 1, 1), (1, 1, 0), (1, 1, 1)),     # depth 1: a 2-D problem
+    (2, 1, 3, 8, (5, 8, 6), (3, 3, 3), (2, 2, 2), (1, 1, 1), (1, 1, 1)),       # few channels, strided: 2-D phases merged
 ]
 
 
