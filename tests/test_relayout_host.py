@@ -96,6 +96,11 @@ PROBLEMS = [
     "-operation gemm -arch gfx950 -t f16 -g 2 -m 70 -n 45 -k 97",
     "-operation gemm -arch gfx950 -t i8 -out_datatype i32 -g 1 -m 33 -n 50 -k 75 -transA true",
     "-operation gemm -arch gfx950 -t f32 -g 1 -m 30 -n 41 -k 37 -transB true",
+    # input gradients with their phases merged: filter slices, the phases put together (4-byte words), to NCHW
+    conv("fp16", "nhwgc", "gkyxc", 2, 3, 20, 16, 8, 7, 7, stride=2, op="conv_bwd_data"),
+    conv("fp16", "ngchw", "gkcyx", 2, 3, 16, 16, 8, 7, 7, stride=2, pad=3, op="conv_bwd_data"),
+    conv("f32", "nhwgc", "gkyxc", 1, 2, 12, 18, 8, 5, 5, stride=3, pad=2, op="conv_bwd_data"),
+    conv("bf16", "ngchw", "gkcyx", 2, 1, 16, 16, 5, 4, 4, stride=2, pad=1, op="conv_bwd_data"),
 ]
 
 
