@@ -272,6 +272,7 @@ struct Handle {
   std::string perf_config;
   std::string problem_key;
   bool tuned = false, lowered = false;
+  bool moved_for_scale_sign = false; // attention: rockamdSetScale took the handle off the plain fused kernel
   OptMap options; // the parsed problem, kept so that a perf_config can be applied later
   // multi-kernel problems (layout conversion + contraction): every kernel of
   // the problem is launched with the same caller pointer list, the problem's
@@ -4262,26 +4263,39 @@ MiirStatus rockamdSetScale(MiirHandle handle, float scale) {
     return MIIR_INVALID_PARAM;
   if (h->op == OP_ATTENTION) {
     auto *ap = reinterpret_cast<RockAttentionParams *>(h->params.data());
-    ap->scale = scale;
     // The plain fused kernel takes the row maximum of the raw scores and
-    // scales afterwards, which is only right for a non-negative scale: a sign
-    // change moves the handle to or from the kernel that scales first.
-    const std::string plain = "_fast", scaled = "_fast_bias";
-    std::string &name = h->kernel_name;
+    // scales afterwards, which is only right for a non-negative scale: a
+    // negative one moves such a handle to the kernel that scales first.  A
+    // handle that the caller, the table or the tuner put on the scale-first
+    // kernel is valid for either sign and stays there; one that a negative scale
+    // moved comes back when the scale turns non-negative again.
+    const std::string plain = "_fast", first = "_fast_bias";
+    const std::string &name = h->kernel_name;
     auto ends_with = [&](const std::string &suffix) {
       return name.size() >= suffix.size() && name.compare(name.size() - suffix.size(), suffix.size(), suffix) == 0;
     };
-    if (scale < 0.0f && ends_with(plain)) {
-      name += "_bias";
+    std::string target;
+    if (scale < 0.0f && ends_with(plain))
+      target = name + "_bias";
+    else if (scale >= 0.0f && h->moved_for_scale_sign && ends_with(first))
+      target = name.substr(0, name.size() - 5);
+    if (!target.empty()) {
+      const Blob *blob = find_blob(target);
+      if (!blob) { // never leave a handle without its code object
+        set_error("attention kernel " + target + " is not in this library");
+        return MIIR_INVALID_PARAM;
+      }
+      const bool to_first = scale < 0.0f;
+      h->kernel_name = target;
+      h->blob = blob; // one code object per kernel: the handle's follows its kernel
       h->functions.clear();
-    } else if (scale >= 0.0f && ends_with(scaled) && !ap->has_bias && !ap->has_scale_tensor) {
-      name.erase(name.size() - 5);
-      h->functions.clear();
+      h->moved_for_scale_sign = to_first;
+      const int dmax = target.find("_d64x") != std::string::npos    ? 64
+                       : target.find("_d256x") != std::string::npos ? 256
+                                                                     : 128;
+      h->perf_config = attn_perf_string(kAttnVariants[to_first ? 1 : 0], dmax);
     }
-    h->blob = find_blob(name); // one code object per kernel: the handle's follows its kernel
-    if (ends_with(plain) || ends_with(scaled))
-      h->perf_config = attn_perf_string(kAttnVariants[ends_with(scaled) ? 1 : 0],
-                                        name.find("_d64x") != std::string::npos ? 64 : 128);
+    ap->scale = scale;
   } else if (h->epi)
     h->epi->scale = scale;
   else

@@ -692,6 +692,29 @@ def test_attention_scale_sign_selects_the_kernel(rock):
     assert b.kernel_name == "rock_attention_f16_d64x64_fast_bias"
 
 
+def test_attention_set_scale_keeps_a_code_object(rock):
+    """Head dimension 256 exists only as the scale-first kernel: rockamdSetScale must leave the handle on it
+    (kernel name, perf_config with its 256 tile, a code object that still lowers), whatever the sign; and a
+    handle put on the scale-first kernel by its perf_config stays there when the scale is set."""
+    opts = ("-operation attention -arch gfx950 -t f16 -g 2 -seq_len_q 256 -seq_len_k 256 "
+            "-head_dim_qk 256 -head_dim_v 256 -transK true -scale 0.125")
+    k = rock.RockKernel(opts)
+    assert k.kernel_name == "rock_attention_f16_d256x256_fast_bias"
+    size = len(k.code_object())
+    for scale in (0.0625, -0.0625, 0.25):
+        k.set_scale(scale)
+        k._refresh()
+        assert k.kernel_name == "rock_attention_f16_d256x256_fast_bias"
+        assert k.perf_config.split(":")[2].split(",")[1] == "256"
+        assert len(k.code_object()) == size
+    chosen = rock.RockKernel(opts.replace("256 -head_dim_v 256", "64 -head_dim_v 64") +
+                             " -perf_config attn:v1:64,64,128,8,32,32,8,0")
+    assert chosen.kernel_name == "rock_attention_f16_d64x64_fast_bias"
+    chosen.set_scale(0.5)
+    chosen._refresh()
+    assert chosen.kernel_name == "rock_attention_f16_d64x64_fast_bias"
+
+
 def test_fusibility_and_prefill_queries(rock):
     """mlirIsModuleFusible / mlirGetNumPrefillArgs (mlir-c/Dialect/Rock.h:145-158)."""
     lib = rock.load_library()
