@@ -428,6 +428,36 @@ bool requested_tile_is(const OptMap &o, int bm, int bn) {
   return std::sscanf(pc.c_str(), "%d,%d", &a, &b) == 2 && a == bm && b == bn;
 }
 
+// A reduction split over blocks (S shares of K into f32 partial sums, added by
+// rock_reduce_splits) rides in the 7th field of the string, splitK in the
+// reference's grammar (RockAttrDefs.td:241-251), so that the perf_config a
+// split plan reports leads back to the same plan.  The 32x32 kernel that divides K
+// over the four waves of a block has always reported 4 there: its field is 4 * S.
+// -1: no perf_config given, the table decides.
+int64_t requested_block_splits(const OptMap &o) {
+  if (!o.count("perf_config"))
+    return -1;
+  const int64_t field = std::max<int64_t>(1, perf_field(o, 6, 1));
+  return requested_tile_is(o, 32, 32) ? std::max<int64_t>(1, field / 4) : field;
+}
+
+std::string with_block_splits(const std::string &pc, int64_t S) {
+  if (S <= 1 || pc.rfind("v2:", 0) != 0)
+    return pc;
+  std::vector<std::string> f;
+  std::istringstream iss(pc.substr(3));
+  for (std::string part; std::getline(iss, part, ',');)
+    f.push_back(part);
+  if (f.size() < 7)
+    return pc;
+  const bool wave_split = f[0] == "32" && f[1] == "32";
+  f[6] = std::to_string(wave_split ? 4 * S : S);
+  std::string out = "v2:";
+  for (size_t i = 0; i < f.size(); ++i)
+    out += (i ? "," : "") + f[i];
+  return out;
+}
+
 void default_epilogue(RockEpilogue &e, int out_dtype) {
   std::memset(&e, 0, sizeof e);
   e.scale = 1.0f;
@@ -742,14 +772,19 @@ Handle *make_gemm(const OptMap &o) {
     const bool long_k = K >= 2048;
     const bool wave_split_fills = wave_split && !long_k && (int64_t)ceil_div(M, 32) * ceil_div(N, 32) * 2 > kNumCU;
     int64_t S = 1;
-    if (G == 1 && is_float_in(ta) && is_float_in(tb) && identity && tiled && !wave_split_fills &&
-        tiles64 * (long_k ? 2 : 4) <= kNumCU && forced_tile(o).empty() && bool_or(o, "split_k", true)) {
-      const int64_t want = std::min<int64_t>(2 * kNumCU / tiles64, K / 512);
-      for (int64_t d = want; d >= 2; --d)
-        if (K % d == 0 && ((K / d) * es) % 64 == 0) {
-          S = d;
-          break;
-        }
+    const int64_t s_req = requested_block_splits(o); // a perf_config names the split itself
+    auto share_ok = [&](int64_t d) { return K % d == 0 && ((K / d) * es) % 64 == 0; };
+    if (G == 1 && is_float_in(ta) && is_float_in(tb) && identity && tiled && bool_or(o, "split_k", true)) {
+      if (s_req > 1 && share_ok(s_req))
+        S = s_req;
+      else if (s_req < 0 && !wave_split_fills && tiles64 * (long_k ? 2 : 4) <= kNumCU) {
+        const int64_t want = std::min<int64_t>(2 * kNumCU / tiles64, K / 512);
+        for (int64_t d = want; d >= 2; --d)
+          if (share_ok(d)) {
+            S = d;
+            break;
+          }
+      }
     }
     if (S > 1) {
       const int kid = (int)int_or(o, "kernel_id", 0);
@@ -765,6 +800,7 @@ Handle *make_gemm(const OptMap &o) {
         p.c_gs = M * N; p.c_ms = N; p.c_ns = 1;
         default_epilogue(p.epi, ROCK_F32);
         plan_gemm_kernel(h, p, code, es, o);
+        h->perf_config = with_block_splits(h->perf_config, S);
         h->ptr_map = {{0, 0}, {1, 0}, {4, 0}, {-1, 0}, {-1, 0}};
         set_key(h);
       } else {
@@ -1580,19 +1616,27 @@ Handle *make_conv_bwd_data(const OptMap &o, const ConvProblem &cp) {
   // blocks as in the forward direction (make_conv), partial sums in the workspace, a reduction kernel
   // behind the contraction that writes the input gradient.
   int64_t S = 1, k_part = 0, part_off = 0, part_bytes = 0;
-  if (fast && phases.size() == 1 && !win[0].ok && cp.g == 1 && !o.count("perf_config") && bool_or(o, "split_k", true)) {
+  if (fast && phases.size() == 1 && !win[0].ok && cp.g == 1 && bool_or(o, "split_k", true)) {
     const Phase &ph = phases[0];
     const int64_t Mg = cp.n * ph.h.A * ph.w.A, Kfull = kp * ph.h.T * ph.w.T, step = 128 / es;
     const int64_t tiles64 = (int64_t)ceil_div(Mg, 64) * ceil_div(cp.c, 64);
-    if (tiles64 <= 2 * kNumCU && Kfull >= 2048 && Mg * cp.c <= INT32_MAX) {
-      const int64_t want = std::min<int64_t>(4 * kNumCU / tiles64, Kfull / 1024);
-      for (int64_t d = want; d >= 2; --d)
-        if (Kfull % d == 0 && (Kfull / d) % step == 0) {
-          S = d;
-          k_part = Kfull / d;
-          part_bytes = align256(S * Mg * cp.c * 4);
-          break;
-        }
+    const int64_t s_req = requested_block_splits(o); // a perf_config names the split itself
+    auto share_ok = [&](int64_t d) { return Kfull % d == 0 && (Kfull / d) % step == 0; };
+    if (Mg * cp.c <= INT32_MAX) {
+      if (s_req > 1 && share_ok(s_req))
+        S = s_req;
+      else if (s_req < 0 && tiles64 <= 2 * kNumCU && Kfull >= 2048) {
+        const int64_t want = std::min<int64_t>(4 * kNumCU / tiles64, Kfull / 1024);
+        for (int64_t d = want; d >= 2; --d)
+          if (share_ok(d)) {
+            S = d;
+            break;
+          }
+      }
+      if (S > 1) {
+        k_part = Kfull / S;
+        part_bytes = align256(S * Mg * cp.c * 4);
+      }
     }
   }
   // kernel list
@@ -1687,8 +1731,10 @@ Handle *make_conv_bwd_data(const OptMap &o, const ConvProblem &cp) {
       h = conv_handle_from_view(view, cp.ti, o);
       if (!h)
         return nullptr;
-      if (S > 1)
+      if (S > 1) {
         reinterpret_cast<RockConvParams *>(h->params.data())->K = (int)k_part;
+        h->perf_config = with_block_splits(h->perf_config, S);
+      }
       if (w.ok)
         apply_window_plan(h, *reinterpret_cast<RockConvParams *>(h->params.data()), w, cp.ti, o);
       h->ptr_map = {fast ? Handle::PtrSrc{ws, fil_dst} : Handle::PtrSrc{0, fil_off * es},
@@ -3143,7 +3189,8 @@ Handle *make_conv(const OptMap &o) {
   // groups of the one-group problem (RockConvParams::k_group_stride) into f32 partial results in the
   // workspace (int32 for int8 operands), which rock_reduce_splits adds in split order into the caller's
   // layout.  Only with the identity epilogue, which commutes with the sum (as for the GEMM, and as the reference's split-K,
-  // Rock.cpp:167-198); "--split_k false" or any perf_config declines.
+  // Rock.cpp:167-198); "--split_k false" declines, and a perf_config names the split itself in its splitK field
+  // (1 = none), so that the string a split plan reports leads back to it.
   int64_t S = 1, k_part = 0, part_off = 0;
   int conv_kid = 0;
   {
@@ -3154,15 +3201,21 @@ Handle *make_conv(const OptMap &o) {
                                     (ti == ROCK_I8 && to == ROCK_I32 && e.zero_point == 0));
     const int64_t c_chunks = (c * es + 15) / 16 * 16 / es, Kfull = c_chunks * y * x, step = 128 / es;
     const int64_t tiles64 = (int64_t)ceil_div(Mg, 64) * ceil_div(k, 64);
-    if (g == 1 && identity && tiles64 <= 2 * kNumCU && Kfull >= 2048 && !o.count("perf_config") &&
-        bool_or(o, "split_k", true)) {
-      const int64_t want = std::min<int64_t>(4 * kNumCU / tiles64, Kfull / 1024);
-      for (int64_t d = want; d >= 2; --d)
-        if (Kfull % d == 0 && (Kfull / d) % step == 0) {
-          S = d;
-          k_part = Kfull / d;
-          break;
-        }
+    const int64_t s_req = requested_block_splits(o); // a perf_config names the split itself
+    auto share_ok = [&](int64_t d) { return Kfull % d == 0 && (Kfull / d) % step == 0; };
+    if (g == 1 && identity && Mg * k <= INT32_MAX && bool_or(o, "split_k", true)) {
+      if (s_req > 1 && share_ok(s_req))
+        S = s_req;
+      else if (s_req < 0 && tiles64 <= 2 * kNumCU && Kfull >= 2048) {
+        const int64_t want = std::min<int64_t>(4 * kNumCU / tiles64, Kfull / 1024);
+        for (int64_t d = want; d >= 2; --d)
+          if (share_ok(d)) {
+            S = d;
+            break;
+          }
+      }
+      if (S > 1)
+        k_part = Kfull / S;
     }
   }
   const int64_t part_bytes = S > 1 ? align256(S * Mg * k * 4) : 0;
@@ -3420,7 +3473,7 @@ Handle *make_conv(const OptMap &o) {
   h->num_pointers = 5;
   if (!planned)
     set_contraction_pointers(h, p.epi);
-  h->perf_config = perf_string(*tile, es, &o);
+  h->perf_config = with_block_splits(perf_string(*tile, es, &o), S);
 
   // Window-resident kernel (conv_direct.h): stride 1, dilation 1, a filter of
   // more than one tap, channel run a power of two of 128..1024 bytes, whole
@@ -4008,8 +4061,10 @@ std::vector<std::string> tuning_candidates(const Handle &h, int kind) {
     }
     if (!c)
       continue;
-    if (std::find(seen.begin(), seen.end(), c->kernel_name) == seen.end()) {
-      seen.push_back(c->kernel_name);
+    // one entry per distinct plan: a reduction split over blocks runs the same kernel as the unsplit plan
+    const std::string plan = c->kernel_name + "/" + std::to_string(c->kernel_count);
+    if (std::find(seen.begin(), seen.end(), plan) == seen.end()) {
+      seen.push_back(plan);
       out.push_back(c->perf_config);
     }
     delete c;

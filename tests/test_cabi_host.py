@@ -793,3 +793,41 @@ def test_tuning_table_shared_by_threads(rock):
         t.join()
     assert lib.rockamdTuningUpdateTable(table._t, key, b"v2:64,64,8,32,16,8,1,1,1", C.c_float(1.0)) == 0
     assert lib.rockamdTuningUpdateTable(table._t, key, b"v2:64,64,8,32,16,8,1,1,1", C.c_float(0.5)) == 1
+
+
+def test_split_plans_round_trip_through_their_perf_config(rock):
+    """A plan whose reduction is split over blocks reports the split in the splitK field of its perf_config
+    (RockAttrDefs.td:241-251), and applying that string again leads back to the same plan: same kernels, same
+    workspace, for every kernel_id; splitK 1 names the unsplit plan; the tuning space lists both."""
+    conv = ("--operation conv --arch gfx950 --in_type fp16 --fil_type fp16 --out_type fp16 --fil_layout gkyxc "
+            "--in_layout nhwgc --out_layout nhwgk --batchsize 2 --groupsize 1 --in_channels 1920 --out_channels 1280 "
+            "--in_h 16 --in_w 16 --fil_h 3 --fil_w 3 --dilation_h 1 --dilation_w 1 --conv_stride_h 1 "
+            "--conv_stride_w 1 --padding_h 1 --padding_w 1")
+    problems = [conv, conv.replace("--operation conv", "--operation conv_bwd_data"),
+                "-operation gemm -arch gfx950 -t f16 -g 1 -m 128 -n 1280 -k 5120",
+                "-operation gemm -arch gfx950 -t f16 -g 1 -m 128 -n 128 -k 16384 -transB true"]
+    for opts in problems:
+        flag = "--" if opts.startswith("--") else "-"
+        first = rock.RockKernel(opts)
+        assert first.kernel_count >= 2 and first.workspace_bytes > 0
+        # the contraction kernel of the plan carries the string
+        plan = [rock.RockKernel("%s %skernel_id %d" % (opts, flag, i)) for i in range(first.kernel_count)]
+        strings = [k.perf_config for k in plan if k.perf_config]
+        assert len(strings) == 1
+        pc = strings[0]
+        assert int(pc.split(":")[1].split(",")[6]) > 1
+        for i, k in enumerate(plan):
+            again = rock.RockKernel("%s %skernel_id %d %sperf_config %s" % (opts, flag, i, flag, pc))
+            assert (again.kernel_name, again.kernel_count, again.workspace_bytes, again.grid_size) == \
+                   (k.kernel_name, k.kernel_count, k.workspace_bytes, k.grid_size)
+            k.set_perf_config(pc)       # rockamdTuningSetFromStr on a separately held handle
+            assert (k.kernel_name, k.kernel_count, k.workspace_bytes) == \
+                   (again.kernel_name, again.kernel_count, again.workspace_bytes)
+        # splitK = 1: the same tile without the split
+        fields = pc.split(":")[1].split(",")
+        fields[6] = "4" if fields[:2] == ["32", "32"] else "1"
+        single = rock.RockKernel("%s %sperf_config v2:%s" % (opts, flag, ",".join(fields)))
+        assert single.kernel_count < first.kernel_count
+        space = plan[[bool(k.perf_config) for k in plan].index(True)].tuning_space("full")
+        assert space[0] == pc
+        assert any(int(t.split(":")[1].split(",")[6]) in (1, 4) and t.split(",")[:2] == pc.split(",")[:2] for t in space[1:])
