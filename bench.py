@@ -151,6 +151,42 @@ def cpu_baseline(name, budget_s, threads):
     raise KeyError(name)
 
 
+def vendor_gemms(torch, rock, dev, n):
+    """Same shapes, same tensors: the vendor library's GEMM and this library's, n launches each."""
+    torch.manual_seed(1)
+
+    def ours(t, od, m, k, a, b):
+        kern = rock.RockKernel("-operation gemm -arch gfx950 -t %s -g 1 -m %d -n %d -k %d -transB true "
+                               "-out_datatype %s" % (t, m, m, k, od))
+        out = torch.empty((m, m), dtype=rock.api._torch_dtype(od), device=dev)
+        for _ in range(n):
+            kern.launch(a, b, out, None)
+        torch.cuda.synchronize()
+
+    for m in (8192, 4096):
+        a = torch.randn(m, m, device=dev, dtype=torch.float16)
+        b = torch.randn(m, m, device=dev, dtype=torch.float16)
+        for _ in range(n):
+            torch.matmul(a, b.t())
+        torch.cuda.synchronize()
+        ours("f16", "f16", m, m, a, b)
+    a = torch.randn(8192, 8192, device=dev).to(torch.float8_e4m3fn)
+    b = torch.randn(8192, 8192, device=dev).to(torch.float8_e4m3fn)
+    one = torch.ones((), device=dev)
+    for od, name in ((torch.bfloat16, "bf16"), (torch.float32, "f32")):
+        for _ in range(n):
+            torch._scaled_mm(a, b.t(), scale_a=one, scale_b=one, out_dtype=od)
+        torch.cuda.synchronize()
+        ours("fp8", name, 8192, 8192, a, b)
+    a = torch.randint(-128, 128, (4096, 4096), dtype=torch.int8, device=dev)
+    b = torch.randint(-128, 128, (4096, 4096), dtype=torch.int8, device=dev)
+    for _ in range(n):
+        torch._int_mm(a, b.t())
+    torch.cuda.synchronize()
+    ours("i8", "i32", 4096, 4096, a, b)
+    print(json.dumps({"vendor_gemms": n}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -172,6 +208,11 @@ def main():
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="only run a plain device-to-device copy of MIB MiB five times (the known-size "
                          "kernel that FETCH_SIZE / WRITE_SIZE readings are scaled by) and exit")
+    ap.add_argument("--vendor-gemms", type=int, default=0, metavar="N",
+                    help="only launch, N times each, the GEMMs of the vendor libraries shipped with torch "
+                         "(torch.matmul f16, torch._scaled_mm fp8, torch._int_mm int8) and this library's "
+                         "kernels on the same shapes and data, and exit: the command that rocprofv3 traces "
+                         "for the side-by-side table of kernel geometry and counters under profiles/")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (every box has one); --gpus %d is not "
@@ -193,6 +234,9 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes": src.numel(), "launches": 5}))
+        return
+    if args.vendor_gemms:
+        vendor_gemms(torch, rock, dev, args.vendor_gemms)
         return
     cfgs = make_configs(torch, rock, dev)
     head_name = "c2_gemm_i8_4096_f16out"
