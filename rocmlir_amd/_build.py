@@ -95,9 +95,14 @@ def attention_kernels():
             out.append(("rock_attention_%s_d%dx%d_fast" % (t, d, d), "RK_ATTN_DL(%s, %s, %d, fast, true)" % (t, code, d)))
             out.append(("rock_attention_%s_d%dx%d_fast_bias" % (t, d, d),
                         "RK_ATTN_DL(%s, %s, %d, fast_bias, false)" % (t, code, d)))
+            # K stored [d][seq_k]
+            out.append(("rock_attention_%s_d%dx%d_fast_kt" % (t, d, d), "RK_ATTN_DL_KT(%s, %s, %d, fast_kt, true, 2)" % (t, code, d)))
+            out.append(("rock_attention_%s_d%dx%d_fast_bias_kt" % (t, d, d),
+                        "RK_ATTN_DL_KT(%s, %s, %d, fast_bias_kt, false, 2)" % (t, code, d)))
             out.append(("rock_attention_%s_d%dx%d_generic" % (t, d, d),
                         "RK_ATTN(%s, %s, %d, %d, generic, false)" % (t, code, d, d)))
         out.append(("rock_attention_%s_d256x256_fast_bias" % t, "RK_ATTN_DL_WIDE(%s, %s, 256)" % (t, code)))
+        out.append(("rock_attention_%s_d256x256_fast_bias_kt" % t, "RK_ATTN_DL_KT(%s, %s, 256, fast_bias_kt, false, 1)" % (t, code)))
     for d in (128, 64):   # int8 Q and K, f16 V and output
         out.append(("rock_attention_i8_d%dx%d_fast" % (d, d), "RK_ATTN_DL_I8(%d, fast, true)" % d))
         out.append(("rock_attention_i8_d%dx%d_fast_bias" % (d, d), "RK_ATTN_DL_I8(%d, fast_bias, false)" % d))

@@ -98,6 +98,53 @@ template <int D, bool IS_V> struct AttnTileLoader {
   }
 };
 
+// K stored [d][seq_k] (the reference's default, rocmlir-gen.cpp:2164-2165): a
+// tile holds D rows of d, each the 64 keys of the tile (128 bytes, 8 chunks),
+// in the geometry of a V tile of head dimension 64 with D rows; the S^T row
+// operand then comes out of it through the transposing read, exactly as V^T
+// does out of a V tile (rows = the reduction index, columns = the MFMA row index).
+template <int D> struct AttnKtLoader {
+  static constexpr int CPR = 8;                 // 16-byte chunks per row of 64 keys
+  static constexpr int ROWB = 128;
+  static constexpr int TILE_B = D * ROWB;
+  static constexpr int SLABS = TILE_B / 1024;
+  static constexpr int PER_WAVE = SLABS / 4;
+  static_assert(SLABS % 4 == 0, "tile must split over 4 waves");
+  __amdgpu_buffer_rsrc_t rsrc;
+  unsigned off[PER_WAVE]; // byte offset of the chunk at key tile 0, or kAttnOob for rows of d beyond the head dimension
+  int key_of_chunk;       // first key (inside a tile) of this lane's chunks: the same for all of them
+  int seq_k, wave;
+
+  __device__ __forceinline__ void init(const uint16_t *base, int64_t d_stride, int seq_k_, int d, int wave_, int lane) {
+    wave = wave_;
+    seq_k = seq_k_;
+    rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(base), 0, (int)kAttnOob, 0x00020000);
+    const int pitch_b = (int)d_stride * 2;
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; ++i) {
+      const int c = (wave * PER_WAVE + i) * 64 + lane; // physical chunk inside the tile
+      const int r = c / CPR, pc = c - r * CPR;
+      const int lc = pc ^ attn_swz<CPR, true>(r);
+      // (64 lanes = 8 rows of 8 chunks, and the swizzle only flips chunk bit 2 by row bit 1: the chunk a lane fills
+      // differs from slab to slab by that bit only when the slab's first row does, which it does not: slabs start
+      // at multiples of 8 rows)
+      if (i == 0)
+        key_of_chunk = lc * 8;
+      off[i] = r < d ? (unsigned)(r * pitch_b + lc * 16) : kAttnOob;
+    }
+  }
+  // keys [key0, key0 + 64); chunks that start at or beyond seq_k read as zeros
+  __device__ __forceinline__ void issue(int key0, attn_lds_char_t *tile) {
+    const bool in_range = key0 + key_of_chunk < seq_k;
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; ++i) {
+      const unsigned voff = in_range ? off[i] : kAttnOob;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrc, (attn_lds_void_t *)(tile + (wave * PER_WAVE + i) * 1024), 16, (int)voff, key0 * 2, 0, 0);
+    }
+  }
+};
+
 template <int DT> __device__ __forceinline__ uint32_t pack2_fast(float a, float b) {
   if constexpr (DT == MM_F16) {
     typedef float v2f_t __attribute__((ext_vector_type(2)));
@@ -122,12 +169,14 @@ template <int DT> __device__ __forceinline__ uint32_t pack2_fast(float a, float 
 // mlir/test/fusion/pr-e2e/attention/mixr-attention-first-gemm-i8-f16.mlir).
 // V, the pre-softmax tensors and O stay DT.  D counts elements, so a K row is
 // D bytes and the K tile has the geometry of a 16-bit tile of D / 2.
-template <int DT, int D, bool PLAIN, bool QKI8 = false>
+// KT: K is stored [d][seq_k] instead of [seq_k][d] (16-bit types).
+template <int DT, int D, bool PLAIN, bool QKI8 = false, bool KT = false>
 __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv, const void *Vv,
                                                   const void *scalev, const void *biasv, void *Ov,
                                                   const RockAttentionParams &p) {
   using Gm = AttnTileGeom<D>;                  // V tile
-  using GmK = AttnTileGeom<QKI8 ? D / 2 : D>;  // K tile
+  using GmK = AttnTileGeom<QKI8 ? D / 2 : D>;  // K tile (KT: the same bytes as D rows of 64 keys)
+  static_assert(!(KT && QKI8), "int8 keys stored [d][seq_k] are not built");
   constexpr int KSTEPS = QKI8 ? D / 32 : D / 16; // MFMA K steps of the first GEMM
   constexpr int DTILES = D / 32;  // 32-row tiles of O^T
   constexpr float kLog2e = 1.44269504088896340736f;
@@ -175,9 +224,11 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
   const uint16_t *bias = p.has_bias ? (const uint16_t *)biasv + (int64_t)g * p.bias_gs : nullptr;
   const uint16_t *scale_t = p.has_scale_tensor ? (const uint16_t *)scalev + (int64_t)g * p.bias_gs : nullptr;
 
-  AttnTileLoader<QKI8 ? D / 2 : D, false> lk;
+  std::conditional_t<KT, AttnKtLoader<D>, AttnTileLoader<QKI8 ? D / 2 : D, false>> lk;
   AttnTileLoader<D, true> lv;
-  if constexpr (QKI8) // int8 rows seen as 16-bit rows of half the length (strides are even: host check)
+  if constexpr (KT)
+    lk.init(K, p.k_ds, p.seq_k, p.d_qk, wave, lane);
+  else if constexpr (QKI8) // int8 rows seen as 16-bit rows of half the length (strides are even: host check)
     lk.init((const uint16_t *)((const char *)Kv + (int64_t)g * p.k_gs), p.k_js / 2, p.seq_k, p.d_qk / 2, wave, lane);
   else
     lk.init(K, p.k_js, p.seq_k, p.d_qk, wave, lane);
@@ -213,6 +264,12 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
   const int vrow = tr_key * Gm::ROWB + (tr_i & 1) * 8; // byte offset inside a V tile
   const int vswz = (tr_chunk ^ attn_swz<Gm::CPR, true>(tr_key)) * 16; // chunk 4*dt + tr_chunk
   auto voff = [&](int dt) __attribute__((always_inline)) { return vrow + (vswz ^ (dt * 64)); };
+  // KT: S^T row operand through the same read.  Lane (i, g16) of half h addresses row d = 16*ks + 8*h + i/4
+  // (+ 4 for the second read) at keys 32*st + 16*g16 + 4*(i%4), and receives key 32*st + lq for four
+  // consecutive d: two reads give the 8 consecutive d that the lane's Q fragment holds.
+  const int ktrow = (8 * h + (tr_i >> 2)) * 128 + (tr_i & 1) * 8;
+  const int ktswz = (tr_chunk ^ attn_swz<8, true>(tr_i >> 2)) * 16; // chunk 4*st + tr_chunk; row bit 1 comes from i/4
+  auto ktoff = [&](int ks, int st) __attribute__((always_inline)) { return ktrow + ks * 16 * 128 + (ktswz ^ (st * 64)); };
 
   v16f o[DTILES];
 #pragma unroll
@@ -248,7 +305,16 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
           s[st][v] = 0.0f;
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
-          v4i kf = *(const attn_lds_v4i_t *)(k_slot(SLOT) + koff(ks) + st * 32 * GmK::ROWB);
+          v4i kf;
+          if constexpr (KT) {
+            attn_lds_char_t *a0 = k_slot(SLOT) + ktoff(ks, st);
+            v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((attn_lds_v4s_t *)a0);
+            v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((attn_lds_v4s_t *)(a0 + 4 * 128));
+            v2i l2 = __builtin_bit_cast(v2i, lo), h2 = __builtin_bit_cast(v2i, hi);
+            kf = v4i{l2[0], l2[1], h2[0], h2[1]};
+          } else {
+            kf = *(const attn_lds_v4i_t *)(k_slot(SLOT) + koff(ks) + st * 32 * GmK::ROWB);
+          }
           s[st] = mma32<DT>(kf, qf[ks], s[st]);
         }
       }

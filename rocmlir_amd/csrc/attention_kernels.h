@@ -389,6 +389,15 @@ __device__ __forceinline__ void wait_loads_and_lds_reads() {
                                               RockAttentionParams p) {                        \
     rk::attention_body_dl<MM_F16, D, PLAIN, true>(Q, K, V, scale, bias, O, p);                \
   }
+// K stored [d][seq_k] (the reference's default layout)
+#define RK_ATTN_DL_KT(DTNAME, DT, D, SUFFIX, PLAIN, OCC)                                      \
+  extern "C" __global__ __launch_bounds__(rk::kAttnThreads, OCC) void                         \
+      rock_attention_##DTNAME##_d##D##x##D##_##SUFFIX(const void *Q, const void *K,           \
+                                                      const void *V, const void *scale,       \
+                                                      const void *bias, void *O,              \
+                                                      RockAttentionParams p) {                \
+    rk::attention_body_dl<DT, D, PLAIN, false, true>(Q, K, V, scale, bias, O, p);             \
+  }
 #define RK_ATTN_DL(DTNAME, DT, D, SUFFIX, PLAIN)                                              \
   extern "C" __global__ __launch_bounds__(rk::kAttnThreads, 2) void                           \
       rock_attention_##DTNAME##_d##D##x##D##_##SUFFIX(const void *Q, const void *K,           \

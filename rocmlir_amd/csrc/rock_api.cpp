@@ -3638,6 +3638,99 @@ Handle *make_attention(const OptMap &o) {
   bool has_scale_t = bool_or(o, "with-attn-scale", false);
   // "-t i8": int8 Q and K (the quantised first GEMM), f16 V, pre-softmax tensors and O
   const bool qk_i8 = ty == ROCK_I8;
+  // Transposed Q, V or O ([G, d, seq_q], [G, dv, seq_k], [G, dv, seq_q]): the fused vector kernels want the
+  // head dimension contiguous.  Conversion kernels in front copy Q and V into that layout, one behind writes
+  // the result as the caller laid it out, and the fused kernel in between runs on the copies -- the
+  // multi-kernel protocol of the convolution plans (rocmlir-lib.cpp:150-199).  The reference reaches every
+  // storage through its coordinate transforms (rocmlir-gen.cpp:2149-2200).  "-layout_conversion false", or a
+  // problem whose untransposed twin has no fused vector kernel, leaves the tensors to the kernels that read
+  // them as they lie (element-wise gathers, or the GEMMs of the three-kernel form).
+  // K stored [G, d, seq_k] is read as it lies by the "_kt" kernels when its rows of keys are whole 16-byte
+  // chunks; otherwise (seq_k = 27; int8 keys) it is copied to [G, seq_k, d] the same way.
+  const bool copy_k = !tK && (qk_i8 || sk % 8 != 0);
+  if ((tQ || tV || tO || copy_k) && ty != ROCK_F32 && bool_or(o, "layout_conversion", true)) {
+    OptMap inner = o;
+    inner["transQ"] = inner["transV"] = inner["transO"] = "false";
+    if (copy_k)
+      inner["transK"] = "true";
+    inner.erase("kernel_id");
+    const std::string keep_error = g_last_error;
+    Handle *core = make_attention(inner);
+    const bool usable = core && core->op == OP_ATTENTION && core->kernel_count == 1 &&
+                        core->kernel_name.find("_generic") == std::string::npos;
+    if (!usable) {
+      delete core;
+      g_last_error = keep_error;
+    } else {
+      const int es_q = qk_i8 ? 1 : 2;
+      const int64_t q_bytes = tQ ? align256(G * sq * dqk * es_q) : 0, v_bytes = tV ? align256(G * sk * dv * 2) : 0,
+                    o_bytes = tO ? align256(G * sq * dv * 2) : 0, k_bytes = copy_k ? align256(G * sk * dqk * es_q) : 0;
+      const int64_t q_off = 0, v_off = q_bytes, o_off = q_bytes + v_bytes, k_off = o_off + o_bytes;
+      // caller pointers: Q, K, V, [scale tensor,] bias, O, workspace
+      const int i_scale = has_scale_t ? 3 : -1, i_bias = has_scale_t ? 4 : 3, i_out = i_bias + 1, i_ws = i_out + 1;
+      std::vector<int> kinds; // 0 = Q copy, 1 = V copy, 4 = K copy, 2 = the fused kernel, 3 = O written in the caller's layout
+      if (tQ) kinds.push_back(0);
+      if (tV) kinds.push_back(1);
+      if (copy_k) kinds.push_back(4);
+      kinds.push_back(2);
+      if (tO) kinds.push_back(3);
+      const int kid = (int)int_or(o, "kernel_id", 0);
+      if (kid < 0 || kid >= (int)kinds.size()) {
+        set_error("attention: kernel_id out of range");
+        delete core;
+        return nullptr;
+      }
+      Handle *h = core;
+      const std::string problem_key = core->problem_key;
+      if (kinds[kid] != 2) {
+        h = new Handle;
+        h->arch = core->arch;
+        bool ok;
+        if (kinds[kid] == 0) { // [G, d, seq_q] -> [G, seq_q, d]
+          const int64_t size[5] = {1, 1, G, sq, dqk}, stride[5] = {0, 0, sq * dqk, 1, sq};
+          ok = fill_relayout_handle(h, size, size, stride, es_q);
+          h->ptr_map = {{0, 0}, {i_ws, q_off}};
+          h->problem_key = "relayout attention Q";
+        } else if (kinds[kid] == 1) { // [G, dv, seq_k] -> [G, seq_k, dv]
+          const int64_t size[5] = {1, 1, G, sk, dv}, stride[5] = {0, 0, sk * dv, 1, sk};
+          ok = fill_relayout_handle(h, size, size, stride, 2);
+          h->ptr_map = {{2, 0}, {i_ws, v_off}};
+          h->problem_key = "relayout attention V";
+        } else if (kinds[kid] == 4) { // [G, d, seq_k] -> [G, seq_k, d]
+          const int64_t size[5] = {1, 1, G, sk, dqk}, stride[5] = {0, 0, sk * dqk, 1, sk};
+          ok = fill_relayout_handle(h, size, size, stride, es_q);
+          h->ptr_map = {{1, 0}, {i_ws, k_off}};
+          h->problem_key = "relayout attention K";
+        } else { // [G, seq_q, dv] -> [G, dv, seq_q]
+          const int64_t size[5] = {1, 1, G, dv, sq}, stride[5] = {0, 0, sq * dv, 1, dv};
+          ok = fill_relayout_handle(h, size, size, stride, 2);
+          h->ptr_map = {{i_ws, o_off}, {i_out, 0}};
+          h->problem_key = "relayout attention O";
+        }
+        delete core;
+        if (!ok) {
+          delete h;
+          return nullptr;
+        }
+      } else {
+        h->ptr_map = {tQ ? Handle::PtrSrc{i_ws, q_off} : Handle::PtrSrc{0, 0},
+                      copy_k ? Handle::PtrSrc{i_ws, k_off} : Handle::PtrSrc{1, 0},
+                      tV ? Handle::PtrSrc{i_ws, v_off} : Handle::PtrSrc{2, 0}, {i_scale, 0}, {i_bias, 0},
+                      tO ? Handle::PtrSrc{i_ws, o_off} : Handle::PtrSrc{i_out, 0}};
+        // the key names the problem as the caller posed it
+        auto tf = [](bool b) { return b ? "true" : "false"; };
+        std::ostringstream key;
+        key << h->arch << '\t' << int_or(o, "num_cu", kNumCU) << '\t' << "-t " << dtype_name(ty) << " -transQ " << tf(tQ)
+            << " -transK " << tf(tK) << " -transV " << tf(tV) << " -transO " << tf(tO) << " -g " << G << " -seq_len_q "
+            << sq << " -seq_len_k " << sk << " -head_dim_qk " << dqk << " -head_dim_v " << dv;
+        h->problem_key = key.str();
+      }
+      h->kernel_count = (int)kinds.size();
+      h->workspace_bytes = (size_t)(q_bytes + v_bytes + o_bytes + k_bytes);
+      h->caller_pointers = i_ws + 1;
+      return h;
+    }
+  }
   {
     // the fused kernels: head dimensions up to 128, tensors contiguous along the head dimension in
     // whole 16-byte chunks; int8 Q and K only on the vector kernels
@@ -3646,7 +3739,9 @@ Handle *make_attention(const OptMap &o) {
                           ((!has_bias && !has_scale_t) || sq * sk < ((int64_t)1 << 31)) &&
                           bool_or(o, "fused", true);
     // 16-bit types up to 256 on the vector kernel (head-dimension-contiguous tensors, checked below)
-    const bool wide_ok = !qk_i8 && !tQ && tK && !tV && !tO && dqk % 8 == 0 && dv % 8 == 0 && bool_or(o, "fused", true);
+    // (K either way: [seq_k, d], or the reference's default [d, seq_k] with whole 16-byte rows of keys)
+    const bool wide_ok = !qk_i8 && !tQ && (tK || sk % 8 == 0) && !tV && !tO && dqk % 8 == 0 && dv % 8 == 0 &&
+                         bool_or(o, "fused", true);
     const int64_t dlimit = wide_ok ? 256 : 128;
     if (ty == ROCK_F32 || (qk_i8 && (!i8_fused || dqk > 128 || dv > 128)) || dqk > dlimit || dv > dlimit)
       return make_attention_unfused(o, ty, G, sq, sk, dqk, dv, tQ, tK, tV, tO, has_bias, has_scale_t);
@@ -3678,12 +3773,17 @@ Handle *make_attention(const OptMap &o) {
     return nullptr;
   }
   p.xcd_remap = total >= 2 * kNumXCD ? 1 : 0;
+  // K stored [d, seq_k] (no -transK: the reference's default) goes to the "_kt" twins of the vector kernels,
+  // which take the S^T row operand out of a [d][64 keys] tile through the transposing LDS read
+  const bool kt = !qk_i8 && !tK;
+  const bool k_fast = kt ? (p.k_js == 1 && p.k_ds % 8 == 0 && dqk * p.k_ds * 2 < ((int64_t)1 << 31))
+                         : (p.k_ds == 1 && p.k_js % 8 == 0 && sk * p.k_js * 2 < ((int64_t)1 << 31));
   const bool fast = qk_i8 || // checked above: there is no element-wise int8 kernel to fall back to
-                    p.q_ds == 1 && p.k_ds == 1 && p.v_es == 1 && p.o_es == 1 && dqk % 8 == 0 &&
-                    dv % 8 == 0 && p.o_is % 4 == 0 && p.k_js % 8 == 0 && p.v_js % 8 == 0 &&
+                    p.q_ds == 1 && k_fast && p.v_es == 1 && p.o_es == 1 && dqk % 8 == 0 &&
+                    dv % 8 == 0 && p.o_is % 4 == 0 && p.v_js % 8 == 0 &&
                     p.q_is % 8 == 0 &&
                     // byte offsets inside one g slice below 2^31 (buffer descriptors)
-                    sk * p.k_js * 2 < ((int64_t)1 << 31) && sk * p.v_js * 2 < ((int64_t)1 << 31) &&
+                    sk * p.v_js * 2 < ((int64_t)1 << 31) &&
                     // the bias gather indexes one g slice with 32-bit element offsets
                     ((!has_bias && !has_scale_t) || sq * sk < ((int64_t)1 << 31));
   const bool wide = dqk > 128 || dv > 128; // one kernel: vector loads, simple order per tile
@@ -3710,7 +3810,8 @@ Handle *make_attention(const OptMap &o) {
     }
   }
   char name[96];
-  std::snprintf(name, sizeof name, "rock_attention_%s_d%dx%d_%s", dtype_name(ty), dmax, dmax, variant->kind);
+  std::snprintf(name, sizeof name, "rock_attention_%s_d%dx%d_%s%s", dtype_name(ty), dmax, dmax, variant->kind,
+                (kt && variant != &kAttnVariants[2]) ? "_kt" : "");
   h->kernel_name = name;
   // kernel pointers: Q, K, V, scale tensor, bias, O; a caller passes the scale
   // tensor only when the problem names one
@@ -4325,15 +4426,20 @@ MiirStatus rockamdSetScale(MiirHandle handle, float scale) {
     // kernel is valid for either sign and stays there; one that a negative scale
     // moved comes back when the scale turns non-negative again.
     const std::string plain = "_fast", first = "_fast_bias";
-    const std::string &name = h->kernel_name;
+    // (the kernels for K stored [d, seq_k] carry "_kt" behind the variant)
+    std::string name = h->kernel_name, layout;
+    if (name.size() > 3 && name.compare(name.size() - 3, 3, "_kt") == 0) {
+      layout = "_kt";
+      name.erase(name.size() - 3);
+    }
     auto ends_with = [&](const std::string &suffix) {
       return name.size() >= suffix.size() && name.compare(name.size() - suffix.size(), suffix.size(), suffix) == 0;
     };
     std::string target;
     if (scale < 0.0f && ends_with(plain))
-      target = name + "_bias";
+      target = name + "_bias" + layout;
     else if (scale >= 0.0f && h->moved_for_scale_sign && ends_with(first))
-      target = name.substr(0, name.size() - 5);
+      target = name.substr(0, name.size() - 5) + layout;
     if (!target.empty()) {
       const Blob *blob = find_blob(target);
       if (!blob) { // never leave a handle without its code object

@@ -351,7 +351,12 @@ def test_attention_as_three_kernels(rock):
     assert fused.workspace_bytes == 0 and fused.caller_pointers == 5
     with pytest.raises(rock.RockError):
         rock.RockKernel(i8 + " -kernel_id 1")
-    for three in (i8 + " -fused false", i8.replace("-transK true", "-transK false"),
+    # K stored [G, d, seq_k]: a copy to [G, seq_k, d] in front of the fused kernel
+    copied = i8.replace("-transK true", "-transK false")
+    plan = [rock.RockKernel(copied + " -kernel_id %d" % i) for i in range(2)]
+    assert [k.kernel_name for k in plan] == ["rock_relayout_b1", "rock_attention_i8_d64x64_fast"]
+    assert all(k.kernel_count == 2 and k.workspace_bytes == 2 * 128 * 64 and k.caller_pointers == 6 for k in plan)
+    for three in (i8 + " -fused false", copied + " -layout_conversion false",
                   i8.replace("-head_dim_qk 64", "-head_dim_qk 256")):
         q8 = [rock.RockKernel(three + " -kernel_id %d" % i) for i in range(3)]
         assert q8[0].kernel_name.startswith("rock_gemm_i8_") and q8[2].kernel_name.startswith("rock_gemm_f16_")
@@ -831,3 +836,31 @@ def test_split_plans_round_trip_through_their_perf_config(rock):
         space = plan[[bool(k.perf_config) for k in plan].index(True)].tuning_space("full")
         assert space[0] == pc
         assert any(int(t.split(":")[1].split(",")[6]) in (1, 4) and t.split(",")[:2] == pc.split(",")[:2] for t in space[1:])
+
+
+def test_reference_attention_list_resolves_to_fused_vector_kernels(rock):
+    """Every case of mlir/test/e2e/PrAttentionF16.toml:20-67, with -transK true and false (its axis, :10-13), and
+    the int8 shape of mixr-attention-first-gemm-i8.mlir:6-10 (K stored [G, d, seq_k]) end on a fused vector
+    kernel, conversion kernels around it where a tensor is not laid out for it."""
+    cases = ["-seq_len_q 384 -seq_len_k 384 -head_dim_qk 64 -head_dim_v 64",
+             "-seq_len_q 64 -seq_len_k 64 -head_dim_qk 64 -head_dim_v 64 -perf_config attn:v1:32,32,64,32,32,32,4,1",
+             "-seq_len_q 256 -seq_len_k 256 -head_dim_qk 128 -head_dim_v 128 -perf_config attn:v1:128,128,128,32,64,64,4,1",
+             "-seq_len_q 64 -seq_len_k 64 -head_dim_qk 64 -head_dim_v 64",
+             "-seq_len_q 64 -seq_len_k 64 -head_dim_qk 64 -head_dim_v 64 -perf_config attn:v1:64,64,256,4,64,64,8,1",
+             "-seq_len_q 256 -seq_len_k 256 -head_dim_qk 128 -head_dim_v 128 -perf_config attn:v1:128,128,128,32,128,32,4,1",
+             "-seq_len_q 384 -seq_len_k 384 -head_dim_qk 64 -head_dim_v 64 -perf_config attn:v1:32,32,64,8,32,32,8,1",
+             "-seq_len_q 384 -seq_len_k 384 -head_dim_qk 64 -head_dim_v 64 -perf_config attn:v1:32,32,64,8,16,16,8,1",
+             "-seq_len_q 384 -seq_len_k 384 -head_dim_qk 64 -head_dim_v 64 -with-attn-scale true",
+             "-seq_len_q 384 -seq_len_k 384 -head_dim_qk 64 -head_dim_v 64 -with-attn-bias true",
+             "-seq_len_q 384 -seq_len_k 384 -head_dim_qk 64 -head_dim_v 64 -with-attn-scale true -with-attn-bias true",
+             "-seq_len_q 128 -seq_len_k 27 -head_dim_qk 64 -head_dim_v 32 -with-attn-scale true -with-attn-bias true"]
+    problems = ["-operation attention -arch gfx950 -t f16 -g 1 %s -transK %s" % (c, tk) for c in cases
+                for tk in ("true", "false")]
+    problems.append("-operation attention -arch gfx950 -t i8 -g 1 -seq_len_q 64 -seq_len_k 64 -head_dim_qk 32 "
+                    "-head_dim_v 32 -with-attn-bias true")
+    for opts in problems:
+        first = rock.RockKernel(opts)
+        names = [rock.RockKernel("%s -kernel_id %d" % (opts, i)).kernel_name for i in range(first.kernel_count)]
+        fused = [n for n in names if n.startswith("rock_attention")]
+        assert len(fused) == 1 and "_fast" in fused[0], (opts, names)
+        assert all(n.startswith("rock_relayout_b") for n in names if n not in fused), (opts, names)

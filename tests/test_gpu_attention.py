@@ -57,9 +57,43 @@ def test_attention_shapes(rock, oracle, gpu, t, G, sq, sk, dqk, dv):
     check_float(got, ref, t, rms=GATE[t][0], max_abs=GATE[t][1])
 
 
-@pytest.mark.parametrize("tQ,tK,tV,tO", [(0, 0, 0, 0), (1, 1, 0, 0), (0, 1, 1, 0), (0, 1, 0, 1), (1, 0, 1, 1)])
+@pytest.mark.parametrize("tQ,tK,tV,tO", [(0, 0, 0, 0), (1, 1, 0, 0), (0, 1, 1, 0), (0, 1, 0, 1), (1, 0, 1, 1),
+                                         (1, 1, 1, 1), (0, 0, 1, 0), (1, 0, 0, 0)])
 def test_attention_transposed_operands(rock, oracle, gpu, tQ, tK, tV, tO):
-    got, ref = _run(rock, oracle, gpu, "f16", 2, 72, 96, 64, 64, 0.125, 43, bool(tQ), bool(tK), bool(tV), bool(tO))
+    """Every storage of rocmlir-gen.cpp:2149-2200 ends on a fused vector kernel: K [G, d, seq_k] on the
+    "_kt" kernels, transposed Q / V / O through conversion kernels around the fused one."""
+    info = {}
+    got, ref = _run(rock, oracle, gpu, "f16", 2, 72, 96, 64, 64, 0.125, 43, bool(tQ), bool(tK), bool(tV), bool(tO),
+                    info=info)
+    fused = "rock_attention_f16_d64x64_fast" + ("" if tK else "_kt")
+    assert info["kernels"] == ["rock_relayout_b2"] * (tQ + tV) + [fused] + ["rock_relayout_b2"] * tO
+    check_float(got, ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
+
+
+@pytest.mark.parametrize("t", ["f16", "bf16"])
+@pytest.mark.parametrize("G,sq,sk,dqk,dv,bias", [
+    (1, 384, 384, 64, 64, False), (2, 64, 64, 64, 64, False), (1, 256, 256, 128, 128, False),
+    (2, 100, 328, 40, 72, False), (1, 300, 72, 128, 64, True), (2, 33, 136, 16, 128, False),
+    (1, 1, 8, 8, 8, False), (2, 130, 200, 192, 256, False), (1, 129, 64, 256, 136, True),
+    (1, 384, 384, 64, 64, True)])
+def test_attention_default_key_layout(rock, oracle, gpu, t, G, sq, sk, dqk, dv, bias):
+    """K stored [G, d, seq_k], the reference's default (rocmlir-gen.cpp:2164-2165; PrAttentionF16.toml:10-13
+    runs every case both ways): one fused kernel that takes its K fragments through the transposing LDS
+    read; ragged tiles, head-dimension padding, head dimensions up to 256, with and without bias."""
+    info = {}
+    got, ref = _run(rock, oracle, gpu, t, G, sq, sk, dqk, dv, 1.0 / np.sqrt(dqk), 47, tK=False, bias=bias, info=info)
+    dmax = 64 if max(dqk, dv) <= 64 else 128 if max(dqk, dv) <= 128 else 256
+    assert info["kernels"] == ["rock_attention_%s_d%dx%d_fast%s_kt" % (t, dmax, dmax, "_bias" if bias or dmax == 256 else "")]
+    check_float(got, ref, t, rms=GATE[t][0], max_abs=GATE[t][1])
+
+
+def test_attention_default_key_layout_unaligned_rows(rock, oracle, gpu):
+    """seq_k = 27 under the default storage: rows of keys are not whole 16-byte chunks, K is copied to
+    [G, seq_k, d] in front of the fused kernel (cross attention case of PrAttentionF16.toml:64-67)."""
+    info = {}
+    got, ref = _run(rock, oracle, gpu, "f16", 2, 128, 27, 64, 32, 0.125, 48, tK=False, bias=True, scale_tensor=True,
+                    info=info)
+    assert info["kernels"] == ["rock_relayout_b2", "rock_attention_f16_d64x64_fast_bias"]
     check_float(got, ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
 
 
@@ -162,8 +196,8 @@ def test_attention_int8_first_gemm(rock, oracle, gpu, shape, bias):
 
 def test_attention_int8_first_gemm_fused_at_size(rock, oracle, gpu):
     """Head dimension 128, several key tiles and query blocks, ragged in both:
-    the fused int8 kernel against the oracle, and against the three-kernel
-    form of the same problem (K stored [G, d, seq_k] takes that one)."""
+    the fused int8 kernel against the oracle, and on K stored the other way
+    round."""
     G, sq, sk, dqk, dv = 3, 300, 333, 128, 128
     rng = np.random.default_rng(59)
     Q = rng.integers(-128, 128, (G, sq, dqk)).astype(np.int8)
@@ -173,9 +207,12 @@ def test_attention_int8_first_gemm_fused_at_size(rock, oracle, gpu):
     info, info3 = {}, {}
     q, k, v = torch.from_numpy(Q).to(gpu), torch.from_numpy(K).to(gpu), to_gpu(rv, "f16", gpu)
     out = rock.attention(q, k, v, scale=scale, zero_point=zp, transK=True, info=info)
+    # K stored [G, d, seq_k] (as mixr-attention-first-gemm-i8.mlir:7 holds it): copied in front of the same kernel
     out3 = rock.attention(q, k.transpose(1, 2).contiguous(), v, scale=scale, zero_point=zp, transK=False, info=info3)
     torch.cuda.synchronize()
-    assert info["kernels"] == ["rock_attention_i8_d128x128_fast"] and len(info3["kernels"]) == 3
+    assert info["kernels"] == ["rock_attention_i8_d128x128_fast"]
+    assert info3["kernels"] == ["rock_relayout_b1", "rock_attention_i8_d128x128_fast"]
+    assert torch.equal(out, out3)
     shift = np.full((G, sq, sk), -zp * scale, np.float32)
     ref = oracle.attention(Q.astype(np.float32), K.astype(np.float32), Vq, G, sq, sk, dqk, dv, scale=scale,
                            bias_t=shift, transK=True)
