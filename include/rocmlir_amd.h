@@ -213,6 +213,22 @@ ROCMLIR_AMD_API size_t rockamdGetProblemKey(MiirHandle handle, char *buffer, siz
 ROCMLIR_AMD_API MiirStatus rockamdGetPointerMap(MiirHandle handle, int *caller_pointers, int *kernel_pointers,
                                                 int32_t *source, int64_t *offset);
 
+/* Per-channel (broadcast-vector) quantisation, the form the reference lowers when the scale and zero point
+ * of migraphx.dequantizelinear / quantizelinear are tensors with one value per output channel
+ * (MIGraphXToTosa.cpp:874-982; mlir/test/fusion/resnet50-e2e/mixr-resnet-fusion-case-1-quantization.mlir:8-9).
+ * GEMM and forward 2-D convolution take the options "--scale_vector true", "--zero_point_vector i32|i8",
+ * "--quant_scale_vector true", "--out_zero_point_vector i32|i8": element n of the vector replaces the scalar
+ * of the same name for output channel n (GEMM: column n of C; convolution: channel g * K + k).  The vectors
+ * are further tensors of the CALLER list, in the order above, behind the problem's own pointers (A, B, C,
+ * aux[, residual]) and in front of the workspace.  They are not kernel pointers: the contraction kernel reads
+ * their addresses from pointer fields of its parameter block.  For a client that launches the code object
+ * itself this call lists, for the handle's kernel, the byte offset inside the parameter block
+ * (rockamdGetKernelArgs) at which caller pointer source[i] has to be written before the launch; *count is 0
+ * for kernels that read no vector (the other kernels of a plan, every problem without vectors).  Either
+ * array may be NULL; at most four entries. */
+ROCMLIR_AMD_API MiirStatus rockamdGetParamPointers(MiirHandle handle, int *count, int32_t *param_offset,
+                                                   int32_t *source);
+
 /* Epilogue scalars can be changed after creation (they live in the by-value
  * parameter block; fetch it again after a change).  Formulas:
  * MIGraphXToTosa.cpp:874-982.  No counterpart entry point in the reference,

@@ -612,13 +612,13 @@ ORC_EXPORT int orc_conv_bwd_weight_f32(float *fil, const float *in, const float 
  * in the reference's MIGraphX tests); pass 1.0f for none.
  * All arithmetic in f32 (deviation noted in the file header).
  * q_begin/q_end restrict the computed query rows per g. */
-ORC_EXPORT void orc_attention_f32(const float *Q, const float *K,
-                                  const float *V, const float *scale_t,
-                                  const float *bias_t, float scale, float *O,
-                                  int64_t G, int64_t sq, int64_t sk,
-                                  int64_t dqk, int64_t dv, int transQ,
-                                  int transK, int transV, int transO,
-                                  int64_t q_begin, int64_t q_end, int threads) {
+static void attention_f32(const float *Q, const float *K,
+                          const float *V, const float *scale_t,
+                          const float *bias_t, const int8_t *mask, const float *other, float scale, float *O,
+                          int64_t G, int64_t sq, int64_t sk,
+                          int64_t dqk, int64_t dv, int transQ,
+                          int transK, int transV, int transO,
+                          int64_t q_begin, int64_t q_end, int threads) {
   int64_t q_rs = transQ ? 1 : dqk, q_ds = transQ ? sq : 1;
   int64_t k_ds = transK ? 1 : sk, k_js = transK ? dqk : 1;
   int64_t v_js = transV ? 1 : dv, v_es = transV ? sk : 1;
@@ -649,6 +649,10 @@ ORC_EXPORT void orc_attention_f32(const float *Q, const float *K,
             acc = acc * scale;
           if (bias_t)
             acc = acc + bias_t[(g * sq + i) * sk + j];
+          /* migraphx.where(mask, scores, other) in front of the softmax
+           * (mlir/test/fusion/pr-e2e/attention/mixr-attn-where.mlir:11): a select, not an addition */
+          if (mask && !mask[(g * sq + i) * sk + j])
+            acc = other[(g * sq + i) * sk + j];
           s[j] = acc;
         }
         float m = s[0];
@@ -674,6 +678,28 @@ ORC_EXPORT void orc_attention_f32(const float *Q, const float *K,
     }
     free(s);
   }
+}
+
+ORC_EXPORT void orc_attention_f32(const float *Q, const float *K,
+                                  const float *V, const float *scale_t,
+                                  const float *bias_t, float scale, float *O,
+                                  int64_t G, int64_t sq, int64_t sk,
+                                  int64_t dqk, int64_t dv, int transQ,
+                                  int transK, int transV, int transO,
+                                  int64_t q_begin, int64_t q_end, int threads) {
+  attention_f32(Q, K, V, scale_t, bias_t, NULL, NULL, scale, O, G, sq, sk, dqk, dv, transQ, transK, transV, transO,
+                q_begin, q_end, threads);
+}
+
+/* The same with a pre-softmax select: where mask[g,i,j] is zero the score is
+ * replaced by other[g,i,j] (after the scale tensor, the scale and the bias). */
+ORC_EXPORT void orc_attention_where_f32(const float *Q, const float *K, const float *V, const float *scale_t,
+                                        const float *bias_t, const int8_t *mask, const float *other, float scale,
+                                        float *O, int64_t G, int64_t sq, int64_t sk, int64_t dqk, int64_t dv,
+                                        int transQ, int transK, int transV, int transO, int64_t q_begin,
+                                        int64_t q_end, int threads) {
+  attention_f32(Q, K, V, scale_t, bias_t, mask, other, scale, O, G, sq, sk, dqk, dv, transQ, transK, transV, transO,
+                q_begin, q_end, threads);
 }
 
 /* softmax over the last axis, the decomposition of
@@ -724,6 +750,39 @@ ORC_EXPORT void orc_quantize_i8(const float *x, int64_t n, float scale,
     if (r > 127)
       r = 127;
     q[i] = (int8_t)r;
+  }
+}
+
+/* The same two with one scale and one zero point per output channel: the
+ * reference broadcasts scale and zero-point tensors shaped like one value per
+ * channel through the same element-wise chain (MIGraphXToTosa.cpp:874-982;
+ * mlir/test/fusion/resnet50-e2e/mixr-resnet-fusion-case-1-quantization.mlir:8-9
+ * passes a <1x128x1x1xf32> scale to both).  x is [rows][channels]; a NULL
+ * zero-point vector means zero. */
+ORC_EXPORT void orc_dequantize_i64_per_channel(const int64_t *acc, int64_t rows, int64_t channels,
+                                               const float *scale, const int32_t *zero_point, float *y) {
+  for (int64_t r = 0; r < rows; ++r)
+    for (int64_t c = 0; c < channels; ++c) {
+      float a = (float)(int32_t)acc[r * channels + c];
+      float z = (float)(zero_point ? zero_point[c] : 0);
+      y[r * channels + c] = (a - z) * scale[c];
+    }
+}
+
+ORC_EXPORT void orc_quantize_i8_per_channel(const float *x, int64_t rows, int64_t channels, const float *scale,
+                                            const int32_t *zero_point, int8_t *q) {
+  for (int64_t c = 0; c < channels; ++c) {
+    float inv = 1.0f / scale[c]; /* tosa.reciprocal, then the multiplication */
+    for (int64_t r = 0; r < rows; ++r) {
+      float scaled = x[r * channels + c] * inv;
+      int64_t v = round_even_sat(scaled, INT32_MIN, INT32_MAX);
+      v += zero_point ? zero_point[c] : 0;
+      if (v < -128)
+        v = -128;
+      if (v > 127)
+        v = 127;
+      q[r * channels + c] = (int8_t)v;
+    }
   }
 }
 

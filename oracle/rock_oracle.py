@@ -90,9 +90,14 @@ def lib():
         L.orc_attention_f32.argtypes = [vp, vp, vp, vp, vp, f32, vp, i64, i64,
                                         i64, i64, i64, C.c_int, C.c_int,
                                         C.c_int, C.c_int, i64, i64, C.c_int]
+        L.orc_attention_where_f32.argtypes = [vp, vp, vp, vp, vp, vp, vp, f32, vp, i64, i64,
+                                              i64, i64, i64, C.c_int, C.c_int,
+                                              C.c_int, C.c_int, i64, i64, C.c_int]
         L.orc_softmax_f32.argtypes = [vp, vp, i64, i64]
         L.orc_dequantize_i64.argtypes = [vp, i64, f32, i32, vp]
         L.orc_quantize_i8.argtypes = [vp, i64, f32, i32, vp]
+        L.orc_dequantize_i64_per_channel.argtypes = [vp, i64, i64, vp, vp, vp]
+        L.orc_quantize_i8_per_channel.argtypes = [vp, i64, i64, vp, vp, vp]
         L.orc_scale_bias_f32.argtypes = [vp, i64, i64, f32, vp]
         L.orc_verify_float.argtypes = [vp, vp, i64, f32, f32, f32,
                                        C.POINTER(VerifyResult)]
@@ -326,7 +331,9 @@ def conv3d_bwd_weight(inp, dout, fil_layout, in_layout, out_layout, n, g, c, k, 
 # ---- attention ------------------------------------------------------------
 def attention(Q, K, V, G, sq, sk, dqk, dv, scale=1.0, scale_t=None,
               bias_t=None, transQ=False, transK=False, transV=False,
-              transO=False, q_rows=None, threads=0):
+              transO=False, q_rows=None, threads=0, mask=None, other=None):
+    """mask (int8 [G,sq,sk]) and other (f32 [G,sq,sk]): where mask is zero the
+    score is replaced by other before the softmax (migraphx.where)."""
     Q, K, V = _c(Q, np.float32), _c(K, np.float32), _c(V, np.float32)
     assert Q.size == G * sq * dqk and K.size == G * sk * dqk
     assert V.size == G * sk * dv
@@ -334,6 +341,14 @@ def attention(Q, K, V, G, sq, sk, dqk, dv, scale=1.0, scale_t=None,
     bt = _c(bias_t, np.float32) if bias_t is not None else None
     O = np.zeros(G * sq * dv, np.float32)
     q0, q1 = q_rows if q_rows is not None else (0, sq)
+    if mask is not None:
+        mk, ot = _c(mask, np.int8), _c(other, np.float32)
+        assert mk.size == G * sq * sk and ot.size == G * sq * sk
+        lib().orc_attention_where_f32(_p(Q), _p(K), _p(V), _p(st), _p(bt), _p(mk), _p(ot),
+                                      np.float32(scale), _p(O), G, sq, sk, dqk, dv,
+                                      int(transQ), int(transK), int(transV), int(transO),
+                                      q0, q1, threads)
+        return O
     lib().orc_attention_f32(_p(Q), _p(K), _p(V), _p(st), _p(bt),
                             np.float32(scale), _p(O), G, sq, sk, dqk, dv,
                             int(transQ), int(transK), int(transV), int(transO),
@@ -361,6 +376,30 @@ def quantize_i8(x, scale, zero_point=0):
     x = _c(x, np.float32)
     q = np.empty(x.shape, np.int8)
     lib().orc_quantize_i8(_p(x), x.size, np.float32(scale), zero_point, _p(q))
+    return q
+
+
+def dequantize_per_channel(acc_i64, scale, zero_point=None):
+    """acc [..., channels]; scale f32[channels], zero_point int32[channels] or None."""
+    acc = _c(acc_i64, np.int64)
+    ch = acc.shape[-1]
+    sc = _c(scale, np.float32)
+    zp = _c(zero_point, np.int32) if zero_point is not None else None
+    assert sc.size == ch and (zp is None or zp.size == ch)
+    y = np.empty(acc.shape, np.float32)
+    lib().orc_dequantize_i64_per_channel(_p(acc), acc.size // ch, ch, _p(sc), _p(zp), _p(y))
+    return y
+
+
+def quantize_i8_per_channel(x, scale, zero_point=None):
+    """x [..., channels]; scale f32[channels], zero_point int32[channels] or None."""
+    x = _c(x, np.float32)
+    ch = x.shape[-1]
+    sc = _c(scale, np.float32)
+    zp = _c(zero_point, np.int32) if zero_point is not None else None
+    assert sc.size == ch and (zp is None or zp.size == ch)
+    q = np.empty(x.shape, np.int8)
+    lib().orc_quantize_i8_per_channel(_p(x), x.size // ch, ch, _p(sc), _p(zp), _p(q))
     return q
 
 

@@ -107,6 +107,8 @@ def load_library():
                                            C.POINTER(C.c_int),
                                            C.POINTER(C.c_int32),
                                            C.POINTER(C.c_int64)]
+        L.rockamdGetParamPointers.restype = C.c_int
+        L.rockamdGetParamPointers.argtypes = [vp, C.POINTER(C.c_int), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
         L.rockamdIsFusible.restype = C.c_int
         L.rockamdIsFusible.argtypes = [vp, C.c_char_p]
         L.rockamdGetNumPrefillArgs.restype = sz
@@ -427,17 +429,46 @@ def _torch_dtype(name):
             "fp8": torch.float8_e4m3fn, "bf8": torch.float8_e5m2}[name]
 
 
+def _is_tensor(x):
+    return hasattr(x, "data_ptr")
+
+
+def _channel_vectors(scale, zero_point, quant_scale, out_zero_point):
+    """The per-channel quantisation vectors among the four epilogue values, in
+    the order the library takes them behind the problem's own tensors, and the
+    flags that announce them (a torch tensor instead of a number means one
+    value per output channel: f32 scales, int32 or int8 zero points)."""
+    import torch
+    flags, vectors = "", []
+    for name, val, is_zp in (("scale_vector", scale, False), ("zero_point_vector", zero_point, True),
+                             ("quant_scale_vector", quant_scale, False),
+                             ("out_zero_point_vector", out_zero_point, True)):
+        if not _is_tensor(val):
+            continue
+        if is_zp:
+            if val.dtype not in (torch.int8, torch.int32):
+                raise RockError("%s: int32 or int8 elements" % name)
+            flags += " -%s %s" % (name, "i8" if val.dtype == torch.int8 else "i32")
+        else:
+            if val.dtype != torch.float32:
+                raise RockError("%s: f32 elements" % name)
+            flags += " -%s true" % name
+        vectors.append(val.contiguous())
+    return flags, vectors
+
+
 def _epilogue_flags(scale, zero_point, bias, relu, quant_scale, out_zero_point,
                     activation=None, clip=None, residual=None, residual_op="add"):
     s = ""
-    if scale is not None:
+    if scale is not None and not _is_tensor(scale):
         s += " -scale %.9g" % scale
-    if zero_point:
+    if not _is_tensor(zero_point) and zero_point:
         s += " -zero_point %d" % zero_point
-    if quant_scale is not None:
+    if quant_scale is not None and not _is_tensor(quant_scale):
         s += " -quant_scale %.9g" % quant_scale
-    if out_zero_point:
+    if not _is_tensor(out_zero_point) and out_zero_point:
         s += " -out_zero_point %d" % out_zero_point
+    s += _channel_vectors(scale, zero_point, quant_scale, out_zero_point)[0]
     if bias is not None:
         s += " -bias true"
     if relu:
@@ -459,7 +490,10 @@ def gemm(a, b, *, transA=False, transB=False, transC=False, out_dtype=None,
     """C = epilogue(A x B) with the reference's storage conventions
     (rocmlir-gen.cpp:2058-2080): a is [G,M,K] ([G,K,M] if transA), b is
     [G,K,N] ([G,N,K] if transB), result [G,M,N] ([G,N,M] if transC).
-    2-D inputs mean G = 1.  The epilogue runs scale / zero point, per-column
+    2-D inputs mean G = 1.  `scale`, `zero_point`, `quant_scale` and
+    `out_zero_point` are numbers (per tensor) or torch tensors with one element
+    per column of the result (per channel: f32 scales, int32 / int8 zero
+    points).  The epilogue runs scale / zero point, per-column
     `bias`, `residual` (a tensor shaped and typed like the result, combined by
     `residual_op` "add" or "mul"), then `activation` ("relu", "sigmoid",
     "tanh", "erf", "gelu", "exp") or `clip=(lo, hi)`, then the narrowing to
@@ -505,12 +539,15 @@ def gemm(a, b, *, transA=False, transB=False, transC=False, out_dtype=None,
     shape = (G, N, M) if transC else (G, M, N)
     if out is None:
         out = torch.empty(shape, dtype=_torch_dtype(out_dtype), device=a.device)
+    vectors = _channel_vectors(scale, zero_point, quant_scale, out_zero_point)[1]
+    if any(v.numel() != N for v in vectors):
+        raise RockError("gemm: a per-channel vector holds one element per column of the result")
     if residual is None:
-        prog.launch(a3, b3, out, bias, stream=stream)
+        prog.launch(a3, b3, out, bias, *vectors, stream=stream)
     else:
         if residual.dtype != out.dtype or residual.numel() != out.numel():
             raise RockError("gemm: the residual must have the result's type and size")
-        prog.launch(a3, b3, out, bias, residual.contiguous(), stream=stream)
+        prog.launch(a3, b3, out, bias, residual.contiguous(), *vectors, stream=stream)
     return out if a.dim() == 3 else out.squeeze(0)
 
 
@@ -520,14 +557,16 @@ def conv2d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize,
            scale=None, zero_point=0, bias=None, relu=False, quant_scale=None,
            out_zero_point=0, activation=None, clip=None, residual=None,
            residual_op="add", out=None, perf_config=None, stream=None,
-           info=None, padding_r=None):
+           info=None, padding_r=None, layout_conversion=True):
     """Forward convolution; tensors are flat device buffers laid out as the
     layout strings say (Miir / rocmlir-gen spelling, e.g. 'gkyxc', 'nhwgc',
     'NGCHW').  Epilogue arguments as for gemm(); the residual is laid out
     like the output.  `padding` is the top / left padding and, unless
     `padding_r` gives the bottom / right one (--padding_h_r / --padding_w_r),
     that one too.  Returns the flat output tensor.  A dict passed as `info`
-    receives the name and perf_config of the kernel that ran."""
+    receives the name and perf_config of the kernel that ran.
+    `layout_conversion=False` keeps the tensors where they lie (no conversion
+    kernels in front; the element-wise kernel where the vector ones cannot read them)."""
     import torch
     t = _dtype_name(inp.dtype)
     pr = padding if padding_r is None else padding_r
@@ -549,6 +588,8 @@ def conv2d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize,
         opts += " --out_type %s" % out_dtype
     if perf_config:
         opts += " --perf_config %s" % perf_config
+    if not layout_conversion:
+        opts += " --layout_conversion false"
     opts += _epilogue_flags(scale, zero_point, bias, relu, quant_scale,
                             out_zero_point, activation, clip, residual,
                             residual_op)
@@ -563,26 +604,35 @@ def conv2d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize,
     if out is None:
         out = torch.empty(batchsize * out_channels * ho * wo,
                           dtype=_torch_dtype(out_dtype), device=inp.device)
+    vectors = _channel_vectors(scale, zero_point, quant_scale, out_zero_point)[1]
+    if any(v.numel() != out_channels for v in vectors):
+        raise RockError("conv2d: a per-channel vector holds one element per output channel")
     if residual is None:
-        prog.launch(fil.contiguous(), inp.contiguous(), out, bias, stream=stream)
+        prog.launch(fil.contiguous(), inp.contiguous(), out, bias, *vectors, stream=stream)
     else:
         if residual.dtype != out.dtype or residual.numel() != out.numel():
             raise RockError("conv2d: the residual must have the output's type and size")
-        prog.launch(fil.contiguous(), inp.contiguous(), out, bias, residual.contiguous(), stream=stream)
+        prog.launch(fil.contiguous(), inp.contiguous(), out, bias, residual.contiguous(), *vectors, stream=stream)
     return out
 
 
-def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, zero_point=0, transQ=False, transK=False,
-              transV=False, transO=False, out=None, stream=None, info=None):
+def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, mask=None, other=None, zero_point=0,
+              transQ=False, transK=False, transV=False, transO=False, out=None, stream=None, info=None,
+              score_workspace_limit=None):
     """O = softmax(scale * scale_tensor * Q K + bias) V (bias and scale_tensor
     optional [G,seq_q,seq_k] tensors, rocmlir-gen's -with-attn-bias /
-    -with-attn-scale) with the reference's storage
+    -with-attn-scale).  `mask` (int8 or bool, [G,seq_q,seq_k]) with `other`
+    (same shape, v's type) puts migraphx.where(mask, scores, other) in front of
+    the softmax (mixr-attn-where.mlir:11): a zero in the mask replaces the score
+    by other's element.  Storage follows the reference's
     conventions (rocmlir-gen.cpp:2149-2200): q [G,seq_q,d] ([G,d,seq_q] if
     transQ); k [G,d,seq_k] ([G,seq_k,d] if transK -- the usual row-major keys);
     v [G,seq_k,dv] ([G,dv,seq_k] if transV); result [G,seq_q,dv]
     ([G,dv,seq_q] if transO).  int8 q and k (with f16 v, bias, scale_tensor)
     select the quantised first GEMM: the scores are (acc - zero_point) * scale.
-    A dict passed as `info` receives the names of the kernels that ran."""
+    A dict passed as `info` receives the names of the kernels that ran.
+    `score_workspace_limit` (bytes) bounds the score chunk of the three-kernel
+    form (f32, head dimensions above 256); the default is 32 MiB."""
     import torch
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     G = q.shape[0]
@@ -602,16 +652,25 @@ def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, zero_point=0,
         opts += " -with-attn-scale true"
     if zero_point:
         opts += " -zero_point %d" % zero_point
+    if (mask is None) != (other is None):
+        raise RockError("attention: mask and other come together")
+    if mask is not None:
+        opts += " -with-attn-mask true"
+        if tuple(mask.shape) != (G, sq, sk) or tuple(other.shape) != (G, sq, sk) or other.dtype != v.dtype:
+            raise RockError("attention: mask and other are [G, seq_q, seq_k]; other has v's type")
+        mask = mask.to(torch.int8).contiguous()
+    if score_workspace_limit is not None:
+        opts += " -score_workspace_limit %d" % score_workspace_limit
     kern = _program(opts)   # one fused kernel, or three for head dimensions above 128 and f32
     if info is not None:
         info["kernels"] = [k.kernel_name for k in kern.kernels]
     shape = (G, dv, sq) if transO else (G, sq, dv)
     if out is None:
         out = torch.empty(shape, dtype=v.dtype, device=q.device)
-    if scale_tensor is None:
-        kern.launch(q, k, v, bias, out, stream=stream)
-    else:
-        kern.launch(q, k, v, scale_tensor.contiguous(), bias, out, stream=stream)
+    pre = ([] if scale_tensor is None else [scale_tensor.contiguous()]) + [bias]
+    if mask is not None:
+        pre += [mask, other.contiguous()]
+    kern.launch(q, k, v, *pre, out, stream=stream)
     return out
 
 

@@ -172,8 +172,8 @@ template <int DT> __device__ __forceinline__ uint32_t pack2_fast(float a, float 
 // KT: K is stored [d][seq_k] instead of [seq_k][d] (16-bit types).
 template <int DT, int D, bool PLAIN, bool QKI8 = false, bool KT = false>
 __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv, const void *Vv,
-                                                  const void *scalev, const void *biasv, void *Ov,
-                                                  const RockAttentionParams &p) {
+                                                  const void *scalev, const void *biasv, const void *maskv,
+                                                  const void *otherv, void *Ov, const RockAttentionParams &p) {
   using Gm = AttnTileGeom<D>;                  // V tile
   using GmK = AttnTileGeom<QKI8 ? D / 2 : D>;  // K tile (KT: the same bytes as D rows of 64 keys)
   static_assert(!(KT && QKI8), "int8 keys stored [d][seq_k] are not built");
@@ -223,6 +223,8 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
   uint16_t *O = (uint16_t *)Ov + (int64_t)g * p.o_gs;
   const uint16_t *bias = p.has_bias ? (const uint16_t *)biasv + (int64_t)g * p.bias_gs : nullptr;
   const uint16_t *scale_t = p.has_scale_tensor ? (const uint16_t *)scalev + (int64_t)g * p.bias_gs : nullptr;
+  const int8_t *mask = p.has_mask ? (const int8_t *)maskv + (int64_t)g * p.bias_gs : nullptr;
+  const uint16_t *other = p.has_mask ? (const uint16_t *)otherv + (int64_t)g * p.bias_gs : nullptr;
 
   std::conditional_t<KT, AttnKtLoader<D>, AttnTileLoader<QKI8 ? D / 2 : D, false>> lk;
   AttnTileLoader<D, true> lv;
@@ -374,6 +376,9 @@ __device__ __forceinline__ void attention_body_dl(const void *Qv, const void *Kv
           x = x * c_scale;
           if (bias != nullptr && in_range)
             x = x + elem_to_f32<DT>(bias[boff + (unsigned)kofs * bias_js]) * kLog2e;
+          // where(mask, x, other): a select behind the element-wise chain (mixr-attn-where.mlir:11)
+          if (mask != nullptr && in_range && mask[boff + (unsigned)kofs * bias_js] == 0)
+            x = elem_to_f32<DT>(other[boff + (unsigned)kofs * bias_js]) * kLog2e;
           s[st][v] = x;
         }
     }

@@ -115,8 +115,8 @@ __device__ __forceinline__ v4i load8(const uint16_t *base, int64_t rs, int64_t c
 
 template <int DT, int DQK, int DV, bool FAST>
 __device__ __forceinline__ void attention_body(const void *Qv, const void *Kv, const void *Vv,
-                                               const void *scalev, const void *biasv, void *Ov,
-                                               const RockAttentionParams &p) {
+                                               const void *scalev, const void *biasv, const void *maskv,
+                                               const void *otherv, void *Ov, const RockAttentionParams &p) {
   constexpr int KCH = DQK / 8;              // 16-byte chunks per K row
   constexpr int KPITCH = DQK * 2 + 16;      // bytes
   constexpr int K_BYTES = kBKV * KPITCH;
@@ -154,6 +154,8 @@ __device__ __forceinline__ void attention_body(const void *Qv, const void *Kv, c
   uint16_t *O = (uint16_t *)Ov + (int64_t)g * p.o_gs;
   const uint16_t *bias = p.has_bias ? (const uint16_t *)biasv + (int64_t)g * p.bias_gs : nullptr;
   const uint16_t *scale_t = p.has_scale_tensor ? (const uint16_t *)scalev + (int64_t)g * p.bias_gs : nullptr;
+  const int8_t *mask = p.has_mask ? (const int8_t *)maskv + (int64_t)g * p.bias_gs : nullptr;
+  const uint16_t *other = p.has_mask ? (const uint16_t *)otherv + (int64_t)g * p.bias_gs : nullptr;
 
   // ---- Q^T fragments: column operand, lane = query row, 8 d per K step
   v4i qf[KSTEPS];
@@ -267,6 +269,10 @@ __device__ __forceinline__ void attention_body(const void *Qv, const void *Kv, c
         if (bias != nullptr && key < p.seq_k && q_row < p.seq_q)
           x = x + elem_to_f32<DT>(bias[(int64_t)q_row * p.bias_is + (int64_t)key * p.bias_js]) *
                       1.44269504088896340736f;
+        // where(mask, x, other): a select behind the element-wise chain (mixr-attn-where.mlir:11)
+        if (mask != nullptr && key < p.seq_k && q_row < p.seq_q &&
+            mask[(int64_t)q_row * p.bias_is + (int64_t)key * p.bias_js] == 0)
+          x = elem_to_f32<DT>(other[(int64_t)q_row * p.bias_is + (int64_t)key * p.bias_js]) * 1.44269504088896340736f;
         x = key < p.seq_k ? x : -INFINITY;
         s[st][v] = x;
         mloc = fmaxf(mloc, x);
@@ -356,14 +362,15 @@ __device__ __forceinline__ void wait_loads_and_lds_reads() {
 
 #include "attention_dlds.h"
 
-// pointer order follows the reference: Q, K, V, [pre-softmax scale tensor], [pre-softmax bias], O
+// pointer order follows the reference: Q, K, V, the pre-softmax inputs (scale tensor, bias, where-mask and its
+// "other" tensor; NULL when the problem has none), O
 #define RK_ATTN(DTNAME, DT, DQK, DV, FASTNAME, FAST)                                          \
   extern "C" __global__ __launch_bounds__(rk::kAttnThreads) void                              \
-      rock_attention_##DTNAME##_d##DQK##x##DV##_##FASTNAME(const void *Q, const void *K,     \
-                                                           const void *V, const void *scale, \
-                                                           const void *bias, void *O,        \
-                                                           RockAttentionParams p) {          \
-    rk::attention_body<DT, DQK, DV, FAST>(Q, K, V, scale, bias, O, p);                        \
+      rock_attention_##DTNAME##_d##DQK##x##DV##_##FASTNAME(const void *Q, const void *K,      \
+                                                           const void *V, const void *scale,  \
+                                                           const void *bias, const void *mask, const void *other, void *O, \
+                                                           RockAttentionParams p) {           \
+    rk::attention_body<DT, DQK, DV, FAST>(Q, K, V, scale, bias, mask, other, O, p);           \
   }
 
 // fast variants: two blocks per compute unit (register budget 256 per lane).
@@ -377,32 +384,32 @@ __device__ __forceinline__ void wait_loads_and_lds_reads() {
   extern "C" __global__ __launch_bounds__(rk::kAttnThreads, 1) void                           \
       rock_attention_##DTNAME##_d##D##x##D##_fast_bias(const void *Q, const void *K,          \
                                                        const void *V, const void *scale,      \
-                                                       const void *bias, void *O,             \
+                                                       const void *bias, const void *mask, const void *other, void *O, \
                                                        RockAttentionParams p) {               \
-    rk::attention_body_dl<DT, D, false>(Q, K, V, scale, bias, O, p);                          \
+    rk::attention_body_dl<DT, D, false>(Q, K, V, scale, bias, mask, other, O, p);             \
   }
 // int8 Q and K, f16 V / bias / O
 #define RK_ATTN_DL_I8(D, SUFFIX, PLAIN)                                                       \
   extern "C" __global__ __launch_bounds__(rk::kAttnThreads, 2) void                           \
       rock_attention_i8_d##D##x##D##_##SUFFIX(const void *Q, const void *K, const void *V,    \
-                                              const void *scale, const void *bias, void *O,   \
+                                              const void *scale, const void *bias, const void *mask, const void *other, void *O, \
                                               RockAttentionParams p) {                        \
-    rk::attention_body_dl<MM_F16, D, PLAIN, true>(Q, K, V, scale, bias, O, p);                \
+    rk::attention_body_dl<MM_F16, D, PLAIN, true>(Q, K, V, scale, bias, mask, other, O, p);   \
   }
 // K stored [d][seq_k] (the reference's default layout)
 #define RK_ATTN_DL_KT(DTNAME, DT, D, SUFFIX, PLAIN, OCC)                                      \
   extern "C" __global__ __launch_bounds__(rk::kAttnThreads, OCC) void                         \
       rock_attention_##DTNAME##_d##D##x##D##_##SUFFIX(const void *Q, const void *K,           \
                                                       const void *V, const void *scale,       \
-                                                      const void *bias, void *O,              \
+                                                      const void *bias, const void *mask, const void *other, void *O, \
                                                       RockAttentionParams p) {                \
-    rk::attention_body_dl<DT, D, PLAIN, false, true>(Q, K, V, scale, bias, O, p);             \
+    rk::attention_body_dl<DT, D, PLAIN, false, true>(Q, K, V, scale, bias, mask, other, O, p); \
   }
 #define RK_ATTN_DL(DTNAME, DT, D, SUFFIX, PLAIN)                                              \
   extern "C" __global__ __launch_bounds__(rk::kAttnThreads, 2) void                           \
       rock_attention_##DTNAME##_d##D##x##D##_##SUFFIX(const void *Q, const void *K,           \
                                                       const void *V, const void *scale,       \
-                                                      const void *bias, void *O,              \
+                                                      const void *bias, const void *mask, const void *other, void *O, \
                                                       RockAttentionParams p) {                \
-    rk::attention_body_dl<DT, D, PLAIN>(Q, K, V, scale, bias, O, p);                          \
+    rk::attention_body_dl<DT, D, PLAIN>(Q, K, V, scale, bias, mask, other, O, p);             \
   }

@@ -747,7 +747,7 @@ __device__ __forceinline__ void dl_epilogue_rich(typename MmaTraits<DT>::Acc (&a
           }
         } else {
           float v[4];
-          epilogue_affine4<Tr::INT_ACC, ROCK_DTYPE_COUNT>(a4, e, aux, n, p.N, nullptr, 0, 1, v);
+          epilogue_affine4<Tr::INT_ACC, ROCK_DTYPE_COUNT, true>(a4, e, aux, n, p.N, nullptr, 0, 1, v);
           if (res_vec) {
             float rf[4];
             unpack4_rt(rr[t], od, rf);
@@ -763,7 +763,7 @@ __device__ __forceinline__ void dl_epilogue_rich(typename MmaTraits<DT>::Acc (&a
               for (int k = 0; k < 4; ++k)
                 v[k] = activation_fast(v[k], e);
             }
-            dl_rich_emit<NI>(p, Cptr, wbuf, epilogue_pack4_rt(v, od, e), t, es, row, n_wave, lane, staged_ok);
+            dl_rich_emit<NI>(p, Cptr, wbuf, epilogue_pack4_rt(v, od, e, n, p.N), t, es, row, n_wave, lane, staged_ok);
           }
         }
       }
@@ -809,7 +809,7 @@ __device__ __forceinline__ void dl_epilogue_rich(typename MmaTraits<DT>::Acc (&a
             for (int r = 0; r < 4; ++r)
               v[r] = activation_fast(v[r], e);
           }
-          *(v4i *)slot = epilogue_pack4_rt(v, od, e);
+          *(v4i *)slot = epilogue_pack4_rt(v, od, e, n_wave + (t >> 2) * 32 + (t & 3) * 8 + lgrp * 4, p.N);
         }
       }
       // results back into registers, then to their store positions: every lane
@@ -837,10 +837,12 @@ __device__ __forceinline__ void dl_epilogue_rich(typename MmaTraits<DT>::Acc (&a
 // RICH kernels are separate instantiations (kernel name suffix "_e") so that
 // the plain kernels' register allocation is untouched by the rich path.
 template <int DT, int MI, int NI, int NWAVES, int LDS_BYTES, bool RICH = false, typename Params>
-__device__ __forceinline__ void dl_epilogue(typename MmaTraits<DT>::Acc (&acc)[MI][NI], const Params &p, int g,
+__device__ __forceinline__ void dl_epilogue(typename MmaTraits<DT>::Acc (&acc)[MI][NI], const Params &p_in, int g,
                                             void *Cptr, const void *aux, const void *res, int m_wave, int n_wave, char *lds,
                                             int wave, int lane) {
   using Tr = MmaTraits<DT>;
+  Params p = p_in; // a convolution's per-channel pointers moved on to this block's group
+  group_channel_pointers(p, aux, g);
   constexpr int WTN = NI * 32;
   const int lrow = lane & 31, lgrp = lane >> 5;
   const RockEpilogue &e = p.epi;

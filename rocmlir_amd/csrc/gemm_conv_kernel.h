@@ -338,7 +338,15 @@ template <int N, typename F> __device__ __forceinline__ void static_for(F &&f) {
 // acc[r] belongs to channel n0 + r.  `res` is the residual tensor and res_off
 // the element offset of (row, n0) in it, channels res_ns apart; null when the
 // epilogue names no residual operation or the row is out of range.
-template <bool INT_ACC, int OD, typename Acc4>
+// element n of a per-channel zero-point vector of int32 or int8 elements
+__device__ __forceinline__ float chan_zero_point(const void *vec, int n, bool is_i8) {
+  return is_i8 ? (float)((const int8_t *)vec)[n] : (float)((const int *)vec)[n];
+}
+
+// CHAN: the per-channel vectors of RockEpilogue::chan_flags are honoured (the
+// kernels with the rolled epilogue and the element-wise kernels); the plain
+// tiled kernels are compiled without them.
+template <bool INT_ACC, int OD, bool CHAN = false, typename Acc4>
 __device__ __forceinline__ void epilogue_affine4(const Acc4 &acc, const RockEpilogue &e, const void *aux,
                                                  int n0, int n_limit, const void *res, int64_t res_off,
                                                  int64_t res_ns, float (&v)[4]) {
@@ -356,13 +364,27 @@ __device__ __forceinline__ void epilogue_affine4(const Acc4 &acc, const RockEpil
           b4[r] = ((const float *)aux)[n0 + r];
     }
   }
+  float s4[4] = {e.scale, e.scale, e.scale, e.scale};
+  float z4[4] = {(float)e.zero_point, (float)e.zero_point, (float)e.zero_point, (float)e.zero_point};
+  if constexpr (CHAN) {
+    if (e.chan_flags & (ROCK_CHAN_SCALE | ROCK_CHAN_ZP)) { // uniform
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n0 + r < n_limit) {
+          if (e.chan_flags & ROCK_CHAN_SCALE)
+            s4[r] = e.scale_vec[n0 + r];
+          if (e.chan_flags & ROCK_CHAN_ZP)
+            z4[r] = chan_zero_point(e.zero_point_vec, n0 + r, (e.chan_flags & ROCK_CHAN_ZP_I8) != 0);
+        }
+    }
+  }
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     float f;
     if constexpr (INT_ACC)
-      f = ((float)(int)acc[r] - (float)e.zero_point) * e.scale;
+      f = ((float)(int)acc[r] - z4[r]) * s4[r];
     else
-      f = (float)acc[r] * e.scale;
+      f = (float)acc[r] * s4[r];
     if (e.has_bias)
       f = f + b4[r];
     if (res && n0 + r < n_limit) {
@@ -375,7 +397,10 @@ __device__ __forceinline__ void epilogue_affine4(const Acc4 &acc, const RockEpil
 
 // Step 5: 4 values narrowed to the output type and packed back to back in the
 // low 4*elem_size bytes.
-template <int OD> __device__ __forceinline__ v4i epilogue_pack4(const float (&v)[4], const RockEpilogue &e) {
+// n0 / n_limit: the channels the four values belong to (read only for a
+// per-channel requantisation, CHAN)
+template <int OD, bool CHAN = false>
+__device__ __forceinline__ v4i epilogue_pack4(const float (&v)[4], const RockEpilogue &e, int n0 = 0, int n_limit = 0) {
   v4i out = {0, 0, 0, 0};
   if constexpr (OD == ROCK_F32 || OD == ROCK_I32) {
 #pragma unroll
@@ -396,7 +421,16 @@ template <int OD> __device__ __forceinline__ v4i epilogue_pack4(const float (&v)
   } else if constexpr (OD == ROCK_I8) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      float q = __builtin_rintf(v[r] * e.inv_quant_scale) + (float)e.out_zero_point;
+      float inv = e.inv_quant_scale, zp = (float)e.out_zero_point;
+      if constexpr (CHAN) {
+        if ((e.chan_flags & (ROCK_CHAN_QUANT_SCALE | ROCK_CHAN_OUT_ZP)) && n0 + r < n_limit) { // uniform flags
+          if (e.chan_flags & ROCK_CHAN_QUANT_SCALE)
+            inv = 1.0f / e.quant_scale_vec[n0 + r]; // tosa.reciprocal, then the multiplication (MIGraphXToTosa.cpp:917-921)
+          if (e.chan_flags & ROCK_CHAN_OUT_ZP)
+            zp = chan_zero_point(e.out_zero_point_vec, n0 + r, (e.chan_flags & ROCK_CHAN_OUT_ZP_I8) != 0);
+        }
+      }
+      float q = __builtin_rintf(v[r] * inv) + zp;
       out[0] |= ((int)f32_to_i8_sat(q) & 0xff) << (8 * r);
     }
   } else if constexpr (OD == ROCK_FP8) {
@@ -411,12 +445,12 @@ template <int OD> __device__ __forceinline__ v4i epilogue_pack4(const float (&v)
   return out;
 }
 
-__device__ __forceinline__ v4i epilogue_pack4_rt(const float (&v)[4], int od, const RockEpilogue &e) {
+__device__ __forceinline__ v4i epilogue_pack4_rt(const float (&v)[4], int od, const RockEpilogue &e, int n0, int n_limit) {
   switch (od) {
   case ROCK_F32: return epilogue_pack4<ROCK_F32>(v, e);
   case ROCK_F16: return epilogue_pack4<ROCK_F16>(v, e);
   case ROCK_BF16: return epilogue_pack4<ROCK_BF16>(v, e);
-  case ROCK_I8: return epilogue_pack4<ROCK_I8>(v, e);
+  case ROCK_I8: return epilogue_pack4<ROCK_I8, true>(v, e, n0, n_limit);
   case ROCK_FP8: return epilogue_pack4<ROCK_FP8>(v, e);
   default: return epilogue_pack4<ROCK_BF8>(v, e);
   }
@@ -426,7 +460,7 @@ __device__ __forceinline__ v4i epilogue_pack4_rt(const float (&v)[4], int od, co
 // constant so that the unrolled epilogue is straight-line code.  SLOW_CALL:
 // transcendental activations are applied here through an out-of-line call
 // (element-wise kernels); otherwise the caller has dealt with them.
-template <bool INT_ACC, int OD, bool SLOW_CALL = false, typename Acc4>
+template <bool INT_ACC, int OD, bool SLOW_CALL = false, bool CHAN = false, typename Acc4>
 __device__ __forceinline__ v4i epilogue_convert4(const Acc4 &acc, const RockEpilogue &e,
                                                  const void *aux, int n0, int n_limit,
                                                  const void *res = nullptr, int64_t res_off = 0,
@@ -446,7 +480,7 @@ __device__ __forceinline__ v4i epilogue_convert4(const Acc4 &acc, const RockEpil
     return v;
   } else {
     float v[4];
-    epilogue_affine4<INT_ACC, OD>(acc, e, aux, n0, n_limit, res, res_off, res_ns, v);
+    epilogue_affine4<INT_ACC, OD, CHAN>(acc, e, aux, n0, n_limit, res, res_off, res_ns, v);
     if (SLOW_CALL && activation_is_slow(e)) {
 #pragma unroll
       for (int r = 0; r < 4; ++r)
@@ -456,7 +490,7 @@ __device__ __forceinline__ v4i epilogue_convert4(const Acc4 &acc, const RockEpil
       for (int r = 0; r < 4; ++r)
         v[r] = activation_fast(v[r], e);
     }
-    return epilogue_pack4<OD>(v, e);
+    return epilogue_pack4<OD, CHAN>(v, e, n0, n_limit);
   }
 }
 
@@ -511,6 +545,30 @@ __device__ __forceinline__ void store_packed4(const v4i &raw, int es, void *out_
 // ---- parameter-block adapters ------------------------------------------------
 __device__ __forceinline__ int p_batch(const RockGemmParams &p) { return p.G; }
 __device__ __forceinline__ int p_batch(const RockConvParams &p) { return p.g; }
+
+// The per-channel values of the epilogue (bias, quantisation vectors) belong to
+// output channel g * K + k of a convolution, to column n of a GEMM whatever the
+// batch entry: a convolution block of group g moves the pointers on by g * K
+// channels before its epilogue indexes them with the channel inside the group.
+// (The shares of a split reduction, which run as groups, take no such values.)
+__device__ __forceinline__ void group_channel_pointers(RockGemmParams &, const void *&, int) {}
+__device__ __forceinline__ void group_channel_pointers(RockConvParams &p, const void *&aux, int g) {
+  const int base = g * p.N;
+  if (base == 0)
+    return;
+  RockEpilogue &e = p.epi;
+  if (e.has_bias)
+    aux = (const char *)aux + (int64_t)base * 4; // f32, or int32 beside int32 results
+  if (e.chan_flags & ROCK_CHAN_SCALE)
+    e.scale_vec += base;
+  if (e.chan_flags & ROCK_CHAN_ZP)
+    e.zero_point_vec = (const char *)e.zero_point_vec + (int64_t)base * ((e.chan_flags & ROCK_CHAN_ZP_I8) ? 1 : 4);
+  if (e.chan_flags & ROCK_CHAN_QUANT_SCALE)
+    e.quant_scale_vec += base;
+  if (e.chan_flags & ROCK_CHAN_OUT_ZP)
+    e.out_zero_point_vec =
+        (const char *)e.out_zero_point_vec + (int64_t)base * ((e.chan_flags & ROCK_CHAN_OUT_ZP_I8) ? 1 : 4);
+}
 
 __device__ __forceinline__ bool aligned_for_vec(const void *base, int64_t row_off, int out_dtype) {
   // 4 consecutive outputs stored as one 4/8/16-byte access need that alignment
@@ -632,7 +690,8 @@ __device__ __forceinline__ void direct_epilogue(const AccArr &acc, const Params 
           continue;
         Acc4 a4 = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
                    acc[i][j][4 * q + 3]};
-        v4i raw = epilogue_convert4<INT_ACC, OD, SLOW_CALL>(a4, p.epi, aux, n, p.N, p.epi.residual_op ? res : nullptr,
+        // (the callers that take every epilogue -- SLOW_CALL -- also take the per-channel vectors)
+        v4i raw = epilogue_convert4<INT_ACC, OD, SLOW_CALL, SLOW_CALL>(a4, p.epi, aux, n, p.N, p.epi.residual_op ? res : nullptr,
                                                  row_off + (int64_t)n * n_stride, n_stride);
         store_packed4(raw, ES, Cptr, row_off + (int64_t)n * n_stride, n_stride, n, p.N, vec_ok);
       }
@@ -723,11 +782,14 @@ __device__ __forceinline__ void contraction_body(const void *Aptr, const void *B
   }
 
   // ---- epilogue: lane holds m = .. + lrow, n = .. + 8*q + 4*lgrp + {0..3}
-  const RockEpilogue &e = p.epi;
+  Params pg = p;
+  const void *aux_g = aux;
+  group_channel_pointers(pg, aux_g, g);
+  const RockEpilogue &e = pg.epi;
   using Acc4 = decltype(__builtin_shufflevector(acc[0][0], acc[0][0], 0, 1, 2, 3));
   dispatch_out_dtype<Tr::INT_ACC>(e.out_dtype, [&](auto od_const) __attribute__((always_inline)) {
     constexpr int OD = decltype(od_const)::value;
-    direct_epilogue<Tr::INT_ACC, OD, MI, NI, Acc4>(acc, p, g, Cptr, aux, res, m0 + wm * WTM + lrow,
+    direct_epilogue<Tr::INT_ACC, OD, MI, NI, Acc4>(acc, pg, g, Cptr, aux_g, res, m0 + wm * WTM + lrow,
                                                   n0 + wn * WTN + lgrp * 4);
   });
 }

@@ -59,6 +59,25 @@ struct RockEpilogue {
   int32_t activation;   // RockActivation
   int32_t residual_op;  // RockResidualOp; the residual pointer follows the bias pointer
   float act_lo, act_hi; // clamp applied for relu [0, +inf) and clip [lo, hi]; (-inf, +inf) otherwise
+  // Per-channel (broadcast-vector) quantisation, the form the reference lowers for scale and zero-point tensors
+  // shaped like one value per output channel (MIGraphXToTosa.cpp:874-982; mixr-resnet-fusion-case-1-
+  // quantization.mlir:8-9 dequantises and re-quantises with a <1x128x1x1xf32> scale): a set bit replaces
+  // the scalar above by element n of the vector.  Only the kernels with the rolled epilogue ("_e") and the
+  // element-wise kernels read them.
+  int32_t chan_flags;            // RockChannelVector bits
+  int32_t pad_;
+  const float *scale_vec;        // step 1: scale[n]
+  const void *zero_point_vec;    // step 1: zero_point[n], int32 or int8 (ROCK_CHAN_ZP_I8)
+  const float *quant_scale_vec;  // step 5: the quantisation scale[n] (the kernel multiplies by its reciprocal)
+  const void *out_zero_point_vec; // step 5: out_zero_point[n], int32 or int8 (ROCK_CHAN_OUT_ZP_I8)
+};
+enum RockChannelVector : int32_t {
+  ROCK_CHAN_SCALE = 1,
+  ROCK_CHAN_ZP = 2,
+  ROCK_CHAN_QUANT_SCALE = 4,
+  ROCK_CHAN_OUT_ZP = 8,
+  ROCK_CHAN_ZP_I8 = 16,     // the zero-point vector holds int8 elements
+  ROCK_CHAN_OUT_ZP_I8 = 32, // the output zero-point vector holds int8 elements
 };
 
 struct RockGemmParams {
@@ -217,7 +236,7 @@ struct RockSoftmaxParams {
   float scale;
   int32_t has_bias, has_scale_tensor;
   int32_t dtype; // RockDType of P, the scale tensor and the bias: f32, f16 or bf16
-  int32_t pad_;
+  int32_t has_mask; // where(mask, score, other): an int8 mask and a tensor of `dtype`, both [g, i, j] like the bias
 };
 
 struct RockAttentionParams {
@@ -234,5 +253,7 @@ struct RockAttentionParams {
   int32_t xcd_remap;
   int32_t has_scale_tensor; // scores are multiplied element-wise by the scale tensor before `scale`
   int32_t zero_point;       // int8 Q and K: the scores are (int32 sum - zero_point) * scale
-  int32_t pad_;
+  // migraphx.where(mask, scores, other) in front of the softmax (mixr-attn-where.mlir:11): where the int8 mask
+  // [g,i,j] is zero, the score (after scale tensor, scale and bias) is REPLACED by other[g,i,j]
+  int32_t has_mask;
 };

@@ -157,6 +157,7 @@ __device__ __forceinline__ float block_reduce(float v, bool take_max, float *scr
 // narrower results over them.
 #if RK_SELECTED(5)
 extern "C" __global__ __launch_bounds__(256) void rock_softmax_rows(float *S, const void *scale_t, const void *bias,
+                                                                    const void *mask, const void *other,
                                                                     RockSoftmaxParams p) {
   __shared__ float scratch[4];
   const int64_t row = blockIdx.x;
@@ -170,6 +171,8 @@ extern "C" __global__ __launch_bounds__(256) void rock_softmax_rows(float *S, co
     x = x * p.scale;
     if (p.has_bias)
       x = x + load_as_f32(bias, t_off + (int64_t)j * p.t_js, p.dtype);
+    if (p.has_mask && ((const int8_t *)mask)[t_off + (int64_t)j * p.t_js] == 0) // where(mask, x, other)
+      x = load_as_f32(other, t_off + (int64_t)j * p.t_js, p.dtype);
     return x;
   };
   float m = -INFINITY;

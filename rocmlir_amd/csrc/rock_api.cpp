@@ -293,6 +293,12 @@ struct Handle {
     std::vector<int64_t> dims;
   };
   std::vector<ArgInfo> args;
+  // Pointers that ride INSIDE the parameter block (the per-channel quantisation vectors of RockEpilogue):
+  // at launch the caller pointer `source` is written at byte `offset` of the block
+  struct ParamPtr {
+    int offset, source;
+  };
+  std::vector<ParamPtr> param_ptrs;
   // typed views of `params`
   RockEpilogue *epi = nullptr;
   // launch cache: device -> function
@@ -350,6 +356,36 @@ bool parse_epilogue(const OptMap &o, int in_a, int out_dtype, RockEpilogue &e) {
   }
   e.zero_point = (int32_t)int_or(o, "zero_point", 0);
   e.out_zero_point = (int32_t)int_or(o, "out_zero_point", 0);
+  // Per-channel vectors in place of the four scalars above: "-scale_vector true", "-zero_point_vector i32|i8",
+  // "-quant_scale_vector true", "-out_zero_point_vector i32|i8" (one element per output channel, passed as
+  // further tensors behind the problem's own; MIGraphXToTosa.cpp:874-982 broadcasts such tensors)
+  e.chan_flags = 0;
+  {
+    auto vec = [&](const char *key, int bit, int i8_bit) {
+      const std::string v = str_or(o, key, "false");
+      if (v == "false" || v == "0")
+        return true;
+      if (v == "i8" && i8_bit)
+        e.chan_flags |= bit | i8_bit;
+      else if (v == "true" || v == "1" || v == "i32" || (v == "f32" && !i8_bit))
+        e.chan_flags |= bit;
+      else
+        return false;
+      return true;
+    };
+    if (!vec("scale_vector", ROCK_CHAN_SCALE, 0) || !vec("zero_point_vector", ROCK_CHAN_ZP, ROCK_CHAN_ZP_I8) ||
+        !vec("quant_scale_vector", ROCK_CHAN_QUANT_SCALE, 0) ||
+        !vec("out_zero_point_vector", ROCK_CHAN_OUT_ZP, ROCK_CHAN_OUT_ZP_I8))
+      return false;
+    // the dequantisation vectors need the float step, a zero point an integer accumulator, the
+    // quantisation vectors an int8 result
+    if ((e.chan_flags & (ROCK_CHAN_SCALE | ROCK_CHAN_ZP)) && out_dtype == ROCK_I32)
+      return false;
+    if ((e.chan_flags & ROCK_CHAN_ZP) && is_float_in(in_a))
+      return false;
+    if ((e.chan_flags & (ROCK_CHAN_QUANT_SCALE | ROCK_CHAN_OUT_ZP)) && out_dtype != ROCK_I8)
+      return false;
+  }
   // legality (RockDialect.cpp:539-568): float in -> float out, int in -> int
   // out; the fused quantisation epilogue additionally lets an int8 problem
   // leave as a float (dequantizelinear) and a float problem leave as int8
@@ -357,6 +393,21 @@ bool parse_epilogue(const OptMap &o, int in_a, int out_dtype, RockEpilogue &e) {
   if (is_float_in(in_a) && out_dtype == ROCK_I32)
     return false;
   return true;
+}
+
+// RockChannelVector bits of the per-channel quantisation vectors a problem asks for (the keys parse_epilogue reads)
+int channel_vector_flags(const OptMap &o) {
+  int flags = 0;
+  auto vec = [&](const char *key, int bit, int i8_bit) {
+    const std::string v = str_or(o, key, "false");
+    if (v != "false" && v != "0")
+      flags |= bit | (v == "i8" ? i8_bit : 0);
+  };
+  vec("scale_vector", ROCK_CHAN_SCALE, 0);
+  vec("zero_point_vector", ROCK_CHAN_ZP, ROCK_CHAN_ZP_I8);
+  vec("quant_scale_vector", ROCK_CHAN_QUANT_SCALE, 0);
+  vec("out_zero_point_vector", ROCK_CHAN_OUT_ZP, ROCK_CHAN_OUT_ZP_I8);
+  return flags;
 }
 
 void apply_tile_grid(const Tile &t, int64_t M, int64_t N, int G, int &tiles_m, int &tiles_n,
@@ -476,7 +527,8 @@ int64_t align256(int64_t bytes) { return (bytes + 255) / 256 * 256; }
 const char *rich_suffix(const RockEpilogue &e, bool tiled_kernel, const OptMap &o) {
   // "-rolled_epilogue true", or a perf_config whose eighth field (forceUnroll)
   // is 0, asks for the twin regardless (it handles every epilogue)
-  return tiled_kernel && (e.residual_op != ROCK_RES_NONE || e.activation > ROCK_ACT_CLIP ||
+  // (so do the per-channel quantisation vectors: the plain kernels are compiled without them)
+  return tiled_kernel && (e.residual_op != ROCK_RES_NONE || e.activation > ROCK_ACT_CLIP || e.chan_flags != 0 ||
                           bool_or(o, "rolled_epilogue", false) || perf_field(o, 7, 1) == 0) ? "_e" : "";
 }
 
@@ -757,7 +809,7 @@ Handle *make_gemm(const OptMap &o) {
   {
     const int es = dtype_size(ta);
     const RockEpilogue &e = p.epi;
-    const bool identity = e.scale == 1.0f && !e.has_bias && e.activation == ROCK_ACT_NONE &&
+    const bool identity = e.scale == 1.0f && !e.has_bias && e.activation == ROCK_ACT_NONE && !e.chan_flags &&
                           e.residual_op == ROCK_RES_NONE && (tc == ROCK_F32 || tc == ROCK_F16 || tc == ROCK_BF16);
     // any vector storage, including the K-contiguous one for which the planner
     // has just chosen the split over the waves of a block: the sub-problems
@@ -3195,7 +3247,7 @@ Handle *make_conv(const OptMap &o) {
   int conv_kid = 0;
   {
     const RockEpilogue &e = p.epi;
-    const bool plain = e.scale == 1.0f && !e.has_bias && e.activation == ROCK_ACT_NONE &&
+    const bool plain = e.scale == 1.0f && !e.has_bias && e.activation == ROCK_ACT_NONE && !e.chan_flags &&
                        e.residual_op == ROCK_RES_NONE;
     const bool identity = plain && ((to == ti && (ti == ROCK_F32 || ti == ROCK_F16 || ti == ROCK_BF16)) ||
                                     (ti == ROCK_I8 && to == ROCK_I32 && e.zero_point == 0));
@@ -3240,7 +3292,7 @@ Handle *make_conv(const OptMap &o) {
   // as it lies: no conversion, no workspace.  (A per-channel bias would run
   // along GEMM rows, which the epilogue does not do; such problems convert.)
   if (!fast && y == 1 && x == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && g == 1 && !p.epi.has_bias &&
-      p.in_ws == 1 && p.in_hs == wi && p.out_ws == 1 && p.out_hs == wo && hi * wi <= INT32_MAX &&
+      !p.epi.chan_flags && p.in_ws == 1 && p.in_hs == wi && p.out_ws == 1 && p.out_hs == wo && hi * wi <= INT32_MAX &&
       bool_or(o, "pointwise_as_gemm", true)) {
     RockGemmParams gp;
     std::memset(&gp, 0, sizeof gp);
@@ -3522,14 +3574,21 @@ Handle *make_conv(const OptMap &o) {
   return h;
 }
 
-// Attention outside the fused kernel's reach (head dimensions above 128, f32):
-// three kernels over a workspace of G * seq_q * seq_k f32 scores -- the GEMM
-// Q K^T, a row softmax that applies scale tensor, scale and bias and narrows
-// the probabilities in place, and the GEMM P V.  The reference fuses every
-// shape (GridwiseGemmToBlockwise.cpp:1607-2403); its validator computes these
-// same three steps (rocmlir-gen.cpp:2565-2620).
+// Attention outside the fused kernel's reach (head dimensions above 256, f32):
+// three kernels over a workspace of f32 scores -- the GEMM Q K^T, a row softmax
+// that applies scale tensor, scale, bias and mask and narrows the probabilities
+// in place, and the GEMM P V.  The reference fuses every shape
+// (GridwiseGemmToBlockwise.cpp:1607-2403); its validator computes these same
+// three steps (rocmlir-gen.cpp:2565-2620).
+// A score matrix above kScoreChunkBytes is worked off in chunks of whole
+// groups, or of query rows of one group, each with its own three kernels in
+// the list (kernel_id = 3 * chunk + step): the workspace holds one chunk --
+// small enough for the array of rockamdLaunchStaticWorkspace and for the
+// scores to stay in the memory-side cache between the three kernels -- instead
+// of G * seq_q * seq_k * 4 bytes.
+constexpr int64_t kScoreChunkBytes = (int64_t)32 << 20;
 Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, int64_t sk, int64_t dqk, int64_t dv,
-                               bool tQ, bool tK, bool tV, bool tO, bool has_bias, bool has_scale_t) {
+                               bool tQ, bool tK, bool tV, bool tO, bool has_bias, bool has_scale_t, bool has_mask) {
   // "-t i8": Q and K are int8, their product is dequantised before the softmax
   // ((acc - zero_point) * scale, the scalars rocmlir-gen passes as [1,1,1]
   // tensors, rocmlir-gen.cpp:2173-2184, 2353-2367); V, the pre-softmax tensors
@@ -3538,19 +3597,37 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
   if (ty == ROCK_I8)
     ty = ROCK_F16;
   const int es = dtype_size(ty);
-  const int kid = (int)int_or(o, "kernel_id", 0);
-  if (kid < 0 || kid > 2) {
-    set_error("attention: kernel_id out of range");
-    return nullptr;
+  // chunk = gc groups x rc query rows
+  // ("-score_workspace_limit BYTES" moves the bound, e.g. to keep one chunk inside a smaller cache share)
+  const int64_t limit = std::max<int64_t>(int_or(o, "score_workspace_limit", kScoreChunkBytes), sk * 4);
+  int64_t gc = G, rc = sq;
+  if (G * sq * sk * 4 > limit) {
+    if (sq * sk * 4 <= limit) {
+      gc = limit / (sq * sk * 4);
+    } else {
+      gc = 1;
+      rc = std::max<int64_t>(1, limit / (sk * 4));
+      rc = rc >= 128 ? rc / 128 * 128 : rc >= 8 ? rc / 8 * 8 : rc; // chunk boundaries on whole tiles / 16-byte columns
+    }
   }
-  if (sq * sk > INT32_MAX * (int64_t)4 || G * sq > INT32_MAX) {
+  const int64_t row_chunks = ceil_div(sq, rc), chunks = ceil_div(G, gc) * row_chunks;
+  const int64_t kid_all = int_or(o, "kernel_id", 0);
+  if (chunks * 3 > INT32_MAX || gc * rc > INT32_MAX) {
     set_error("attention: score matrix too large for the three-kernel form");
     return nullptr;
   }
+  if (kid_all < 0 || kid_all >= 3 * chunks) {
+    set_error("attention: kernel_id out of range");
+    return nullptr;
+  }
+  const int kid = (int)(kid_all % 3);
+  const int64_t g0 = kid_all / 3 / row_chunks * gc, r0 = kid_all / 3 % row_chunks * rc;
+  const int64_t gn = std::min(gc, G - g0), rn = std::min(rc, sq - r0); // this chunk
   float scale = 1.0f;
   get_float(o, "scale", scale);
-  // caller list: Q, K, V, [scale tensor], bias slot, O, workspace
-  const int i_bias = has_scale_t ? 4 : 3, i_out = i_bias + 1, i_ws = i_out + 1;
+  // caller list: Q, K, V, [scale tensor], bias slot, [mask, other], O, workspace
+  const int i_bias = has_scale_t ? 4 : 3, i_mask = has_mask ? i_bias + 1 : -1, i_other = has_mask ? i_bias + 2 : -1,
+            i_out = i_bias + 1 + (has_mask ? 2 : 0), i_ws = i_out + 1;
   const int64_t pitch_p = 4 / es; // elements of P per f32 score: P lies in place, rows sk * 4 bytes apart
   auto *h = new Handle;
   if (kid == 1) {
@@ -3558,10 +3635,11 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
     std::memset(&r, 0, sizeof r);
     r.row_pitch = sk;
     r.t_gs = sq * sk; r.t_is = sk; r.t_js = 1;
-    r.G = (int)G; r.seq_q = (int)sq; r.seq_k = (int)sk;
+    r.G = (int)gn; r.seq_q = (int)rn; r.seq_k = (int)sk;
     r.scale = scale;
     r.has_bias = has_bias ? 1 : 0;
     r.has_scale_tensor = has_scale_t ? 1 : 0;
+    r.has_mask = has_mask ? 1 : 0;
     r.dtype = ty;
     h->op = OP_RELAYOUT;
     h->epi = nullptr;
@@ -3569,35 +3647,44 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
     std::memcpy(h->params.data(), &r, sizeof r);
     h->kernel_name = "rock_softmax_rows";
     h->block_size = 256;
-    h->grid_size = (uint32_t)(G * sq);
-    h->num_pointers = 3;
+    h->grid_size = (uint32_t)(gn * rn);
+    h->num_pointers = 5;
     h->perf_config = "";
-    h->ptr_map = {{i_ws, 0}, {has_scale_t ? 3 : -1, 0}, {has_bias ? i_bias : -1, 0}};
+    const int64_t t_off = (g0 * sq * sk + r0 * sk) * es; // the chunk's first row in the [G, seq_q, seq_k] tensors
+    h->ptr_map = {{i_ws, 0}, {has_scale_t ? 3 : -1, t_off}, {has_bias ? i_bias : -1, t_off}, {i_mask, t_off / es},
+                  {i_other, t_off}};
     h->problem_key = "row softmax of the attention scores";
   } else {
     RockGemmParams gp;
     std::memset(&gp, 0, sizeof gp);
-    gp.G = (int)G;
+    gp.G = (int)gn;
+    int64_t a_off, b_off, c_off; // bytes from the tensors' starts to the chunk
     if (kid == 0) { // S[g,i,j] = sum_d Q[g,i,d] K[g,j,d], f32
-      gp.M = (int)sq; gp.N = (int)sk; gp.K = (int)dqk;
+      gp.M = (int)rn; gp.N = (int)sk; gp.K = (int)dqk;
       gp.a_gs = sq * dqk; gp.a_ms = tQ ? 1 : dqk; gp.a_ks = tQ ? sq : 1;
       gp.b_gs = sk * dqk; gp.b_ns = tK ? dqk : 1; gp.b_ks = tK ? 1 : sk;
-      gp.c_gs = sq * sk; gp.c_ms = sk; gp.c_ns = 1;
+      gp.c_gs = rn * sk; gp.c_ms = sk; gp.c_ns = 1;
+      a_off = (g0 * gp.a_gs + r0 * gp.a_ms) * dtype_size(tq);
+      b_off = g0 * gp.b_gs * dtype_size(tq);
+      c_off = 0;
       default_epilogue(gp.epi, ROCK_F32);
       gp.epi.zero_point = (int32_t)int_or(o, "zero_point", 0); // i8: scores leave as float(acc) - zero_point
     } else { // O[g,i,e] = sum_j P[g,i,j] V[g,j,e]
-      gp.M = (int)sq; gp.N = (int)dv; gp.K = (int)sk;
-      gp.a_gs = sq * sk * pitch_p; gp.a_ms = sk * pitch_p; gp.a_ks = 1;
+      gp.M = (int)rn; gp.N = (int)dv; gp.K = (int)sk;
+      gp.a_gs = rn * sk * pitch_p; gp.a_ms = sk * pitch_p; gp.a_ks = 1;
       gp.b_gs = sk * dv; gp.b_ns = tV ? sk : 1; gp.b_ks = tV ? 1 : dv;
       gp.c_gs = sq * dv; gp.c_ms = tO ? 1 : dv; gp.c_ns = tO ? sq : 1;
       default_epilogue(gp.epi, ty);
+      a_off = 0;
+      b_off = g0 * gp.b_gs * es;
+      c_off = (g0 * gp.c_gs + r0 * gp.c_ms) * es;
     }
     const int tg = kid == 0 ? tq : ty;
     plan_gemm_kernel(h, gp, operand_code(tg, tg), dtype_size(tg), o);
     if (kid == 0)
-      h->ptr_map = {{0, 0}, {1, 0}, {i_ws, 0}, {-1, 0}, {-1, 0}};
+      h->ptr_map = {{0, a_off}, {1, b_off}, {i_ws, c_off}, {-1, 0}, {-1, 0}};
     else
-      h->ptr_map = {{i_ws, 0}, {2, 0}, {i_out, 0}, {-1, 0}, {-1, 0}};
+      h->ptr_map = {{i_ws, a_off}, {2, b_off}, {i_out, c_off}, {-1, 0}, {-1, 0}};
     h->op = OP_GEMM;
     h->params.assign(sizeof gp, 0);
     std::memcpy(h->params.data(), &gp, sizeof gp);
@@ -3609,8 +3696,8 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
         << sq << " -seq_len_k " << sk << " -head_dim_qk " << dqk << " -head_dim_v " << dv;
     h->problem_key = key.str();
   }
-  h->kernel_count = 3;
-  h->workspace_bytes = (size_t)(G * sq * sk * 4);
+  h->kernel_count = (int)(3 * chunks);
+  h->workspace_bytes = (size_t)(gc * rc * sk * 4);
   h->caller_pointers = i_ws + 1;
   return h;
 }
@@ -3636,6 +3723,10 @@ Handle *make_attention(const OptMap &o) {
   // "-with-attn-scale": a full [G, seq_q, seq_k] tensor multiplied into the
   // scores before the softmax (rocmlir-gen.cpp:2185-2196), besides the scalar "-scale"
   bool has_scale_t = bool_or(o, "with-attn-scale", false);
+  // "-with-attn-mask": migraphx.where(mask, scores, other) in front of the softmax (mixr-attn-where.mlir:11) --
+  // an int8 mask and a tensor of replacement scores, both [G, seq_q, seq_k], behind the bias in the caller's list.
+  // Where the mask is zero the score (after scale tensor, scale and bias) is replaced, not added to.
+  const bool has_mask = bool_or(o, "with-attn-mask", false);
   // "-t i8": int8 Q and K (the quantised first GEMM), f16 V, pre-softmax tensors and O
   const bool qk_i8 = ty == ROCK_I8;
   // Transposed Q, V or O ([G, d, seq_q], [G, dv, seq_k], [G, dv, seq_q]): the fused vector kernels want the
@@ -3666,8 +3757,9 @@ Handle *make_attention(const OptMap &o) {
       const int64_t q_bytes = tQ ? align256(G * sq * dqk * es_q) : 0, v_bytes = tV ? align256(G * sk * dv * 2) : 0,
                     o_bytes = tO ? align256(G * sq * dv * 2) : 0, k_bytes = copy_k ? align256(G * sk * dqk * es_q) : 0;
       const int64_t q_off = 0, v_off = q_bytes, o_off = q_bytes + v_bytes, k_off = o_off + o_bytes;
-      // caller pointers: Q, K, V, [scale tensor,] bias, O, workspace
-      const int i_scale = has_scale_t ? 3 : -1, i_bias = has_scale_t ? 4 : 3, i_out = i_bias + 1, i_ws = i_out + 1;
+      // caller pointers: Q, K, V, [scale tensor,] bias, [mask, other,] O, workspace
+      const int i_scale = has_scale_t ? 3 : -1, i_bias = has_scale_t ? 4 : 3, i_mask = has_mask ? i_bias + 1 : -1,
+                i_other = has_mask ? i_bias + 2 : -1, i_out = i_bias + 1 + (has_mask ? 2 : 0), i_ws = i_out + 1;
       std::vector<int> kinds; // 0 = Q copy, 1 = V copy, 4 = K copy, 2 = the fused kernel, 3 = O written in the caller's layout
       if (tQ) kinds.push_back(0);
       if (tV) kinds.push_back(1);
@@ -3716,6 +3808,7 @@ Handle *make_attention(const OptMap &o) {
         h->ptr_map = {tQ ? Handle::PtrSrc{i_ws, q_off} : Handle::PtrSrc{0, 0},
                       copy_k ? Handle::PtrSrc{i_ws, k_off} : Handle::PtrSrc{1, 0},
                       tV ? Handle::PtrSrc{i_ws, v_off} : Handle::PtrSrc{2, 0}, {i_scale, 0}, {i_bias, 0},
+                      {i_mask, 0}, {i_other, 0},
                       tO ? Handle::PtrSrc{i_ws, o_off} : Handle::PtrSrc{i_out, 0}};
         // the key names the problem as the caller posed it
         auto tf = [](bool b) { return b ? "true" : "false"; };
@@ -3736,7 +3829,7 @@ Handle *make_attention(const OptMap &o) {
     // whole 16-byte chunks; int8 Q and K only on the vector kernels
     const bool i8_fused = qk_i8 && !tQ && tK && !tV && !tO && dqk % 16 == 0 && dv % 8 == 0 &&
                           sk * dqk < ((int64_t)1 << 31) && sk * dv * 2 < ((int64_t)1 << 31) &&
-                          ((!has_bias && !has_scale_t) || sq * sk < ((int64_t)1 << 31)) &&
+                          ((!has_bias && !has_scale_t && !has_mask) || sq * sk < ((int64_t)1 << 31)) &&
                           bool_or(o, "fused", true);
     // 16-bit types up to 256 on the vector kernel (head-dimension-contiguous tensors, checked below)
     // (K either way: [seq_k, d], or the reference's default [d, seq_k] with whole 16-byte rows of keys)
@@ -3744,7 +3837,7 @@ Handle *make_attention(const OptMap &o) {
                          bool_or(o, "fused", true);
     const int64_t dlimit = wide_ok ? 256 : 128;
     if (ty == ROCK_F32 || (qk_i8 && (!i8_fused || dqk > 128 || dv > 128)) || dqk > dlimit || dv > dlimit)
-      return make_attention_unfused(o, ty, G, sq, sk, dqk, dv, tQ, tK, tV, tO, has_bias, has_scale_t);
+      return make_attention_unfused(o, ty, G, sq, sk, dqk, dv, tQ, tK, tV, tO, has_bias, has_scale_t, has_mask);
   }
 
   auto *h = new Handle;
@@ -3762,6 +3855,7 @@ Handle *make_attention(const OptMap &o) {
   p.bias_gs = sq * sk; p.bias_is = sk; p.bias_js = 1;
   p.has_bias = has_bias ? 1 : 0;
   p.has_scale_tensor = has_scale_t ? 1 : 0;
+  p.has_mask = has_mask ? 1 : 0;
   p.scale = 1.0f;
   get_float(o, "scale", p.scale);
   p.zero_point = qk_i8 ? (int32_t)int_or(o, "zero_point", 0) : 0;
@@ -3785,13 +3879,13 @@ Handle *make_attention(const OptMap &o) {
                     // byte offsets inside one g slice below 2^31 (buffer descriptors)
                     sk * p.v_js * 2 < ((int64_t)1 << 31) &&
                     // the bias gather indexes one g slice with 32-bit element offsets
-                    ((!has_bias && !has_scale_t) || sq * sk < ((int64_t)1 << 31));
+                    ((!has_bias && !has_scale_t && !has_mask) || sq * sk < ((int64_t)1 << 31));
   const bool wide = dqk > 128 || dv > 128; // one kernel: vector loads, simple order per tile
   int dmax = (dqk <= 64 && dv <= 64) ? 64 : wide ? 256 : 128;
-  const bool plain_ok = !p.has_bias && !has_scale_t && p.scale >= 0.0f && !wide;
+  const bool plain_ok = !p.has_bias && !has_scale_t && !has_mask && p.scale >= 0.0f && !wide;
   if (wide && !fast) {
     delete h;
-    return make_attention_unfused(o, ty, G, sq, sk, dqk, dv, tQ, tK, tV, tO, has_bias, has_scale_t);
+    return make_attention_unfused(o, ty, G, sq, sk, dqk, dv, tQ, tK, tV, tO, has_bias, has_scale_t, has_mask);
   }
   const AttnVariant *variant = !fast ? &kAttnVariants[2] : plain_ok ? &kAttnVariants[0] : &kAttnVariants[1];
   {
@@ -3813,14 +3907,14 @@ Handle *make_attention(const OptMap &o) {
   std::snprintf(name, sizeof name, "rock_attention_%s_d%dx%d_%s%s", dtype_name(ty), dmax, dmax, variant->kind,
                 (kt && variant != &kAttnVariants[2]) ? "_kt" : "");
   h->kernel_name = name;
-  // kernel pointers: Q, K, V, scale tensor, bias, O; a caller passes the scale
-  // tensor only when the problem names one
-  h->num_pointers = 6;
-  if (has_scale_t) {
-    h->caller_pointers = 0;
-  } else {
-    h->caller_pointers = 5;
-    h->ptr_map = {{0, 0}, {1, 0}, {2, 0}, {-1, 0}, {3, 0}, {4, 0}};
+  // kernel pointers: Q, K, V, scale tensor, bias, mask, other, O; a caller passes the scale tensor and the
+  // mask with its replacement scores only when the problem names them, the bias slot always
+  h->num_pointers = 8;
+  {
+    const int i_bias = has_scale_t ? 4 : 3, i_out = i_bias + 1 + (has_mask ? 2 : 0);
+    h->caller_pointers = i_out + 1;
+    h->ptr_map = {{0, 0}, {1, 0}, {2, 0}, {has_scale_t ? 3 : -1, 0}, {i_bias, 0}, {has_mask ? i_bias + 1 : -1, 0},
+                  {has_mask ? i_bias + 2 : -1, 0}, {i_out, 0}};
   }
   h->block_size = 256;
   h->grid_size = (uint32_t)total;
@@ -3895,6 +3989,8 @@ int launch_once(Handle *h, hipFunction_t fn, void *const *pointers, hipStream_t 
     std::memcpy(buf + off, &ptr, 8);
   }
   std::memcpy(buf + off, h->params.data(), h->params.size());
+  for (const Handle::ParamPtr &pp : h->param_ptrs) // tensors whose pointers ride inside the block
+    std::memcpy(buf + off + pp.offset, &pointers[pp.source], 8);
   size_t size = off + h->params.size();
   void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, buf, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
                     HIP_LAUNCH_PARAM_END};
@@ -3939,7 +4035,17 @@ bool check_launch_args(Handle *h, void *const *pointers, int num_pointers) {
 void describe_arguments(const OptMap &o, Handle *h) {
   using A = Handle::ArgInfo;
   const std::string op = str_or(o, "operation", "");
-  auto with_workspace = [&] {
+  // the per-channel quantisation vectors follow the problem's own tensors, the workspace closes the list
+  auto with_workspace = [&](int64_t channels = 0) {
+    const int flags = channel_vector_flags(o);
+    if (flags & ROCK_CHAN_SCALE)
+      h->args.push_back(A{ROCK_F32, {channels}});
+    if (flags & ROCK_CHAN_ZP)
+      h->args.push_back(A{(flags & ROCK_CHAN_ZP_I8) ? ROCK_I8 : ROCK_I32, {channels}});
+    if (flags & ROCK_CHAN_QUANT_SCALE)
+      h->args.push_back(A{ROCK_F32, {channels}});
+    if (flags & ROCK_CHAN_OUT_ZP)
+      h->args.push_back(A{(flags & ROCK_CHAN_OUT_ZP_I8) ? ROCK_I8 : ROCK_I32, {channels}});
     if (h->workspace_bytes)
       h->args.push_back(A{-1, {(int64_t)h->workspace_bytes}});
   };
@@ -3961,7 +4067,7 @@ void describe_arguments(const OptMap &o, Handle *h) {
                A{out_t == ROCK_I32 ? ROCK_I32 : ROCK_F32, {N}}};
     if (str_or(o, "residual", "none") != "none")
       h->args.push_back(A{out_t, h->args[2].dims});
-    with_workspace();
+    with_workspace(N);
   } else if (op == "attention") {
     const int t = parse_dtype(str_or(o, "t", "f16"));
     const int tv = t == ROCK_I8 ? ROCK_F16 : t;
@@ -3973,6 +4079,10 @@ void describe_arguments(const OptMap &o, Handle *h) {
     if (bool_or(o, "with-attn-scale", false))
       h->args.push_back(A{tv, {G, sq, sk}});
     h->args.push_back(A{tv, {G, sq, sk}}); // bias slot
+    if (bool_or(o, "with-attn-mask", false)) {
+      h->args.push_back(A{ROCK_I8, {G, sq, sk}});
+      h->args.push_back(A{tv, {G, sq, sk}});
+    }
     h->args.push_back(A{tv, mat(bool_or(o, "transO", false), sq, dv)});
     with_workspace();
   } else if (o.count("in_d") || o.count("fil_d")) { // three spatial dimensions: six-dimensional tensors
@@ -4039,7 +4149,7 @@ void describe_arguments(const OptMap &o, Handle *h) {
                A{to == ROCK_I32 ? ROCK_I32 : ROCK_F32, {g * k}}};
     if (str_or(o, "residual", "none") != "none")
       h->args.push_back(A{to, h->args[2].dims});
-    with_workspace();
+    with_workspace(g * k);
   }
 }
 
@@ -4070,6 +4180,11 @@ Handle *build_handle(const OptMap &o) {
     }
   }
   std::string op = str_or(o, "operation", "");
+  const int chan = channel_vector_flags(o);
+  if (chan && !(op == "gemm" || ((op == "conv" || op == "conv2d") && !o.count("in_d") && !o.count("fil_d")))) {
+    set_error("per-channel quantisation vectors: GEMM and forward 2-D convolution only");
+    return nullptr;
+  }
   Handle *h = nullptr;
   try {
     if (op == "gemm")
@@ -4094,6 +4209,35 @@ Handle *build_handle(const OptMap &o) {
     return nullptr;
   }
   h->num_cu = (int)int_or(o, "num_cu", kNumCU);
+  if (chan) {
+    // The vectors are further caller tensors between the problem's own and the workspace (which closes
+    // every multi-kernel problem's list): every kernel of the plan sees the longer list, and the
+    // contraction kernel finds the vectors through pointer fields of its parameter block.
+    int nvec = 0;
+    for (int bit : {ROCK_CHAN_SCALE, ROCK_CHAN_ZP, ROCK_CHAN_QUANT_SCALE, ROCK_CHAN_OUT_ZP})
+      nvec += (chan & bit) ? 1 : 0;
+    const int base = h->caller_pointers ? h->caller_pointers : h->num_pointers;
+    const int first = h->workspace_bytes ? base - 1 : base;
+    if (h->ptr_map.empty())
+      for (int i = 0; i < h->num_pointers; ++i)
+        h->ptr_map.push_back(Handle::PtrSrc{i, 0});
+    for (Handle::PtrSrc &m : h->ptr_map)
+      if (m.source >= first)
+        m.source += nvec;
+    h->caller_pointers = base + nvec;
+    if (h->epi && h->epi->chan_flags) {
+      const int at = (int)((const char *)h->epi - h->params.data());
+      int next = first;
+      if (chan & ROCK_CHAN_SCALE)
+        h->param_ptrs.push_back({at + (int)offsetof(RockEpilogue, scale_vec), next++});
+      if (chan & ROCK_CHAN_ZP)
+        h->param_ptrs.push_back({at + (int)offsetof(RockEpilogue, zero_point_vec), next++});
+      if (chan & ROCK_CHAN_QUANT_SCALE)
+        h->param_ptrs.push_back({at + (int)offsetof(RockEpilogue, quant_scale_vec), next++});
+      if (chan & ROCK_CHAN_OUT_ZP)
+        h->param_ptrs.push_back({at + (int)offsetof(RockEpilogue, out_zero_point_vec), next++});
+    }
+  }
   if (h->op == OP_CONV && h->params.size() == sizeof(RockConvParams)) {
     // every plan's convolution kernels leave through here: the division constants of the loader's set-up
     auto &cpar = *reinterpret_cast<RockConvParams *>(h->params.data());
@@ -4409,6 +4553,20 @@ MiirStatus rockamdGetPointerMap(MiirHandle handle, int *caller_pointers, int *ke
       source[i] = h->ptr_map.empty() ? i : h->ptr_map[i].source;
     if (offset)
       offset[i] = h->ptr_map.empty() ? 0 : h->ptr_map[i].offset;
+  }
+  return MIIR_SUCCESS;
+}
+
+MiirStatus rockamdGetParamPointers(MiirHandle handle, int *count, int32_t *param_offset, int32_t *source) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h || !count)
+    return MIIR_INVALID_PARAM;
+  *count = (int)h->param_ptrs.size();
+  for (size_t i = 0; i < h->param_ptrs.size(); ++i) {
+    if (param_offset)
+      param_offset[i] = h->param_ptrs[i].offset;
+    if (source)
+      source[i] = h->param_ptrs[i].source;
   }
   return MIIR_SUCCESS;
 }

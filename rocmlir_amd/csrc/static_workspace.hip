@@ -8,8 +8,12 @@
 // The array exists once per GPU (every device that loads the library's device
 // image holds its own copy until the process ends) and keeps the last call's
 // contents.  Nothing has to be cleared between problems: every kernel list of
-// this library writes each workspace byte before a later kernel of the same
-// list reads it.  All calls on one GPU share the array, so two problems whose
+// this library writes each workspace byte whose value reaches a result before
+// a later kernel of the same list reads it.  The one exception reads stale
+// bytes without using them: the rows-of-taps copies of an input are sized one
+// run of taps past their last row, the contraction loads that slack (left over
+// from an earlier problem) and discards it -- the forward kernel zeroes the
+// row tails, the filter gradient drops those columns.  All calls on one GPU share the array, so two problems whose
 // kernel lists overlap in time on the same GPU (different streams or threads)
 // race on it; serialise them or use rockamdLaunch with separate workspaces.
 #include <hip/hip_runtime.h>

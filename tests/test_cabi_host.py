@@ -157,7 +157,7 @@ def test_baseline_configs_select_kernels(rock):
     k = rock.RockKernel("-operation attention -arch gfx950 -t f16 -g 128 -seq_len_q 2048 -seq_len_k 2048 "
                         "-head_dim_qk 128 -head_dim_v 128 -transK true -scale 0.08838834764831845")
     assert k.kernel_name == "rock_attention_f16_d128x128_fast"
-    assert (k.block_size, k.grid_size, k.num_pointers, k.caller_pointers) == (256, 128 * 16, 6, 5)
+    assert (k.block_size, k.grid_size, k.num_pointers, k.caller_pointers) == (256, 128 * 16, 8, 5)
 
 
 def test_generic_kernels_for_unaligned_or_transposed(rock):
@@ -326,7 +326,7 @@ def test_attention_pre_softmax_tensors(rock):
     k = rock.RockKernel(base + " -with-attn-bias true")
     assert (k.kernel_name, k.caller_pointers) == ("rock_attention_f16_d64x64_fast_bias", 5)
     k = rock.RockKernel(base + " -with-attn-scale true")
-    assert (k.kernel_name, k.caller_pointers, k.num_pointers) == ("rock_attention_f16_d64x64_fast_bias", 6, 6)
+    assert (k.kernel_name, k.caller_pointers, k.num_pointers) == ("rock_attention_f16_d64x64_fast_bias", 6, 8)
 
 
 def test_attention_as_three_kernels(rock):
@@ -334,13 +334,25 @@ def test_attention_as_three_kernels(rock):
     GEMM, row softmax in place over an f32 score workspace, GEMM."""
     vae = ("-operation attention -arch gfx950 -t %s -g 1 -seq_len_q 16384 -seq_len_k 16384 -head_dim_qk 512 "
            "-head_dim_v 512 -transK true")
+    whole = " -score_workspace_limit %d" % (1 << 40)      # the whole score matrix in one piece
     for t in ("f16", "f32"):
-        ks = [rock.RockKernel(vae % t + " -kernel_id %d" % i) for i in range(3)]
+        ks = [rock.RockKernel(vae % t + whole + " -kernel_id %d" % i) for i in range(3)]
         assert ks[0].kernel_name.startswith("rock_gemm_%s_" % t) and ks[0].kernel_name.endswith("_fast")
         assert ks[1].kernel_name == "rock_softmax_rows" and ks[1].grid_size == 16384
         assert ks[2].kernel_name.startswith("rock_gemm_%s_" % t) and ks[2].kernel_name.endswith("_fast_nn")
         assert all(k.kernel_count == 3 and k.workspace_bytes == 16384 * 16384 * 4 and k.caller_pointers == 6
                    for k in ks)
+        # by default in chunks of at most 32 MiB of scores: 512 query rows x 16384 keys, 32 chunks of three kernels
+        ks = [rock.RockKernel(vae % t + " -kernel_id %d" % i) for i in (0, 1, 2, 94, 95)]
+        assert all(k.kernel_count == 96 and k.workspace_bytes == 32 << 20 and k.caller_pointers == 6 for k in ks)
+        assert ks[1].kernel_name == "rock_softmax_rows" and ks[1].grid_size == 512
+        assert ks[3].kernel_name == "rock_softmax_rows" and ks[4].kernel_name == ks[2].kernel_name
+        with pytest.raises(rock.RockError):
+            rock.RockKernel(vae % t + " -kernel_id 96")
+    # many small groups: whole groups per chunk (8 x 2048 x 2048 f32 scores = 128 MiB -> 2 groups a chunk)
+    k = rock.RockKernel("-operation attention -arch gfx950 -t f32 -g 7 -seq_len_q 2048 -seq_len_k 2048 "
+                        "-head_dim_qk 64 -head_dim_v 64 -transK true -kernel_id 9")
+    assert k.kernel_count == 12 and k.workspace_bytes == 32 << 20 and k.grid_size > 0
     # int8 first GEMM: one fused kernel where the layout allows it (its score tile is dequantised in
     # registers); "-fused false", K stored [G, d, seq_k] or a head dimension above 128 give the three
     # kernels: int8 contraction into f32 scores, f16 from there on
@@ -362,7 +374,7 @@ def test_attention_as_three_kernels(rock):
         assert q8[0].kernel_name.startswith("rock_gemm_i8_") and q8[2].kernel_name.startswith("rock_gemm_f16_")
         assert q8[1].kernel_name == "rock_softmax_rows" and q8[0].kernel_count == 3
     lib = rock.load_library()
-    k = rock.RockKernel((vae % "f16").replace("-g 1 ", "-g 4 "))
+    k = rock.RockKernel((vae % "f16").replace("-g 1 ", "-g 4 ") + whole)
     assert k.workspace_bytes == 4 * 16384 * 16384 * 4 and lib.miirGetWorkspaceSize(k._h) == -1   # beyond an int
 
 
@@ -488,7 +500,9 @@ def test_param_block_and_setters(rock):
                         "-transB true -scale 0.5 -zero_point 3")
     import struct
     blob = k.params()
-    assert len(blob) == k.params_size == 9 * 8 + 8 * 4 + 10 * 4   # strides, sizes/tiling, epilogue
+    # strides, sizes / tiling, epilogue scalars, per-channel vector flags + padding + four pointer fields
+    assert len(blob) == k.params_size == 9 * 8 + 8 * 4 + 10 * 4 + 2 * 4 + 4 * 8
+    assert struct.unpack_from("i", blob, 72 + 32 + 40) == (0,) and not any(blob[72 + 32 + 48:])   # no vectors
     G, M, N, K = struct.unpack_from("4i", blob, 72)
     assert (G, M, N, K) == (1, 64, 64, 64)
     scale, inv_q, zp = struct.unpack_from("ffi", blob, 72 + 32)
@@ -864,3 +878,80 @@ def test_reference_attention_list_resolves_to_fused_vector_kernels(rock):
         fused = [n for n in names if n.startswith("rock_attention")]
         assert len(fused) == 1 and "_fast" in fused[0], (opts, names)
         assert all(n.startswith("rock_relayout_b") for n in names if n not in fused), (opts, names)
+
+
+def test_per_channel_quantisation_vectors_in_the_caller_list(rock):
+    """--scale_vector / --zero_point_vector / --quant_scale_vector / --out_zero_point_vector: the kernel with the
+    rolled epilogue, the vectors as further caller tensors behind the problem's own and in front of the
+    workspace, their addresses written into pointer fields of the parameter block (rockamdGetParamPointers)."""
+    lib = rock.load_library()
+
+    def param_ptrs(k):
+        n = C.c_int(0)
+        off = (C.c_int32 * 4)()
+        src = (C.c_int32 * 4)()
+        assert lib.rockamdGetParamPointers(k._h, C.byref(n), off, src) == 0
+        return [(off[i], src[i]) for i in range(n.value)]
+
+    gemm = "-operation gemm -arch gfx950 -t i8 -g 1 -m 512 -n 384 -k 256 -transB true -out_datatype i8"
+    plain = rock.RockKernel(gemm + " -scale 0.01 -quant_scale 0.5")
+    assert plain.kernel_name == "rock_gemm_i8_64x64_fast" and plain.caller_pointers == 4 and param_ptrs(plain) == []
+    k = rock.RockKernel(gemm + " -scale_vector true -zero_point_vector i8 -quant_scale_vector true -out_zero_point_vector i32")
+    assert k.kernel_name == "rock_gemm_i8_64x64_fast_e" and k.caller_pointers == 8
+    ptrs = param_ptrs(k)
+    assert [s for _, s in ptrs] == [4, 5, 6, 7]
+    assert all(0 < o < k.params_size and o % 8 == 0 for o, _ in ptrs) and len({o for o, _ in ptrs}) == 4
+    args = k.arguments()
+    assert args[4:] == [(0, [384]), (3, [384]), (0, [384]), (6, [384])]   # f32, i8, f32, i32
+    # with a residual the vectors follow it; a plan with a workspace keeps it last
+    r = rock.RockKernel(gemm + " -residual add -scale_vector true")
+    assert r.caller_pointers == 6 and [s for _, s in param_ptrs(r)] == [5]
+    nchw = ("--operation conv --arch gfx950 --in_type i8 --fil_type i8 --out_type i8 --fil_layout gkcyx --in_layout ngchw "
+            "--out_layout ngkhw --batchsize 1 --groupsize 1 --in_channels 128 --out_channels 128 --in_h 56 --in_w 56 "
+            "--fil_h 3 --fil_w 3 --dilation_h 1 --dilation_w 1 --conv_stride_h 2 --conv_stride_w 2 --padding_h 1 "
+            "--padding_w 1 --scale_vector true --quant_scale_vector true")
+    first = rock.RockKernel(nchw)
+    plan = [rock.RockKernel("%s --kernel_id %d" % (nchw, i)) for i in range(first.kernel_count)]
+    assert first.kernel_count == 3 and first.workspace_bytes > 0
+    assert all(p.caller_pointers == 7 for p in plan)          # filter, input, output, bias, 2 vectors, workspace
+    assert [param_ptrs(p) != [] for p in plan] == [False, False, True]
+    assert [s for _, s in param_ptrs(plan[2])] == [4, 5] and plan[2].kernel_name.endswith("_e")
+    ncall = C.c_int(0)
+    nk = C.c_int(0)
+    src = (C.c_int32 * 8)()
+    off = (C.c_int64 * 8)()
+    for p in plan:   # the conversion kernels write into, the contraction reads from, the LAST caller pointer
+        assert lib.rockamdGetPointerMap(p._h, C.byref(ncall), C.byref(nk), src, off) == 0
+        assert ncall.value == 7 and max(src[i] for i in range(nk.value)) == 6
+    assert plan[2].arguments()[-1][0] == -1 and plan[2].arguments()[4] == (0, [128])   # bytes of workspace last
+    # what the vectors need: the float step, an integer accumulator for zero points, an int8 result to quantise
+    for bad in (gemm.replace("-out_datatype i8", "-out_datatype i32") + " -scale_vector true",
+                gemm.replace("-out_datatype i8", "-out_datatype f16") + " -quant_scale_vector true",
+                gemm.replace("-t i8", "-t f16") + " -zero_point_vector i32",
+                "-operation attention -arch gfx950 -t f16 -g 1 -seq_len_q 64 -seq_len_k 64 -head_dim_qk 64 "
+                "-head_dim_v 64 -scale_vector true",
+                nchw.replace("--operation conv ", "--operation conv_bwd_data ").replace("i8", "f16")):
+        with pytest.raises(rock.RockError):
+            rock.RockKernel(bad)
+
+
+def test_attention_where_mask_in_the_caller_list(rock):
+    """-with-attn-mask: the int8 mask and the tensor of replacement scores (migraphx.where in front of the softmax,
+    mixr-attn-where.mlir:4-13) follow the bias slot in the caller's list; the plain fused kernel, which scales
+    after the row maximum, is never chosen for such a problem."""
+    base = "-operation attention -arch gfx950 -t f16 -g 12 -seq_len_q 256 -seq_len_k 256 -transK true "
+    k = rock.RockKernel(base + "-head_dim_qk 256 -head_dim_v 256 -with-attn-mask true")
+    assert k.kernel_name == "rock_attention_f16_d256x256_fast_bias" and k.kernel_count == 1
+    assert k.caller_pointers == 7          # Q, K, V, bias slot, mask, other, O
+    args = k.arguments()
+    assert [a[0] for a in args] == [1, 1, 1, 1, 3, 1, 1]   # f16 tensors and the int8 mask
+    assert args[4][1] == [12, 256, 256] and args[5][1] == [12, 256, 256]
+    k = rock.RockKernel(base + "-head_dim_qk 64 -head_dim_v 64 -with-attn-mask true")
+    assert k.kernel_name == "rock_attention_f16_d64x64_fast_bias"
+    k = rock.RockKernel(base + "-head_dim_qk 64 -head_dim_v 64 -with-attn-mask true -perf_config attn:v1:64,64,128,8,64,32,8,1")
+    assert k.kernel_name.endswith("_fast_bias")
+    k = rock.RockKernel(base + "-head_dim_qk 64 -head_dim_v 64 -with-attn-scale true -with-attn-mask true")
+    assert k.caller_pointers == 8
+    # three-kernel form: the row softmax takes them, the workspace still closes the list
+    k = rock.RockKernel(base.replace("f16", "f32") + "-head_dim_qk 64 -head_dim_v 64 -with-attn-mask true -kernel_id 1")
+    assert k.kernel_name == "rock_softmax_rows" and k.kernel_count == 3 and k.caller_pointers == 8

@@ -68,8 +68,8 @@ def _replay_split_conv(params, fil, fil_off, inp, in_off, out, out_off, es):
     st = struct.unpack_from("<15q", params, 0)
     n, S, c, k, hi, wi, y, x, ho, wo, sh, sw, ph, pw, dh, dw = struct.unpack_from("<16i", params, 120)
     (K,) = struct.unpack_from("<i", params, 192)
-    (stride,) = struct.unpack_from("<i", params, 264)
-    (out_dtype,) = struct.unpack_from("<i", params, 240)
+    (stride,) = struct.unpack_from("<i", params, 308)
+    (out_dtype,) = struct.unpack_from("<i", params, 244)
     in_s, fil_s, out_s = st[0:5], st[5:10], st[10:15]
     assert stride == K and S * K == c * y * x and in_s[1] == 0 and fil_s[0] == K and out_dtype in (0, 6)  # f32, i32
     kk = np.arange(c * y * x)
@@ -102,7 +102,7 @@ def _replay_conv(params, fil, fil_off, inp, in_off, out, out_off, es=None):
     st = struct.unpack_from("<15q", params, 0)
     n, g, c, k, hi, wi, y, x, ho, wo, sh, sw, ph, pw, dh, dw = struct.unpack_from("<16i", params, 120)
     in_s, fil_s, out_s = st[0:5], st[5:10], st[10:15]   # n g c h w / g k c y x / n g k h w
-    if struct.unpack_from("<i", params, 264)[0]:
+    if struct.unpack_from("<i", params, 308)[0]:
         return _replay_split_conv(params, fil, fil_off, inp, in_off, out, out_off, es)
 
     def gather(buf, off, sizes, strides):
@@ -112,7 +112,7 @@ def _replay_conv(params, fil, fil_off, inp, in_off, out, out_off, es=None):
         return o
 
     xin = inp[gather(inp, in_off, (n, g, c, hi, wi), in_s)].reshape(n, g, c, hi, wi).astype(np.float64)
-    (run_valid,) = struct.unpack_from("<i", params, 260)
+    (run_valid,) = struct.unpack_from("<i", params, 304)
     if run_valid:  # "_runs" kernels: what a channel run holds behind its data is cleared before it is multiplied
         xin[:, :, run_valid:] = 0
     f = fil[gather(fil, fil_off, (g, k, c, y, x), fil_s)].reshape(g, k, c, y, x).astype(np.float64)
@@ -310,8 +310,8 @@ def _replay_bwd_weight_gemm(params, dy, dy_off, xin, x_off, dst, d_off, es):
     wide = 4 // es if out_dtype == 0 else 1
     a_gs, a_ms, a_ks, _, _, _, c_gs, c_ms, c_ns = struct.unpack_from("<9q", params, 0)
     S, M, N, K = struct.unpack_from("<4i", params, 72)
-    (pix_stride,) = struct.unpack_from("<q", params, 144)
-    c, hi, wi, ho, wo, X, sh, sw, ph, pw, dh, dw = struct.unpack_from("<12i", params, 152)
+    (pix_stride,) = struct.unpack_from("<q", params, 184)
+    c, hi, wi, ho, wo, X, sh, sw, ph, pw, dh, dw = struct.unpack_from("<12i", params, 192)
     cols = np.arange(N)
     tap, cc = cols // c, cols % c
     ty, tx = tap // X, tap % X

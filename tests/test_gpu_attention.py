@@ -19,7 +19,7 @@ def _store(mat, trans):
 
 
 def _run(rock, oracle, gpu, t, G, sq, sk, dqk, dv, scale, seed, tQ=False, tK=True, tV=False, tO=False,
-         bias=False, vones=False, scale_tensor=False, info=None):
+         bias=False, vones=False, scale_tensor=False, info=None, mask=False, limit=None):
     rng = np.random.default_rng(seed)
     Q = rng.standard_normal((G, sq, dqk)).astype(np.float32)
     K = rng.standard_normal((G, sk, dqk)).astype(np.float32)
@@ -33,14 +33,45 @@ def _run(rock, oracle, gpu, t, G, sq, sk, dqk, dv, scale, seed, tQ=False, tK=Tru
     sq_ = sraw = None
     if scale_tensor:
         sraw, sq_ = quantise(rng.uniform(-1.5, 1.5, (G, sq, sk)).astype(np.float32), t)
+    mk = oraw = oq = None
+    if mask:  # about a third of the scores replaced; some rows wholly (row 0 of every g), some not at all (row 1)
+        mk = (rng.uniform(0, 1, (G, sq, sk)) > 0.35).astype(np.int8)
+        mk[:, 0, :] = 0
+        if sq > 1:
+            mk[:, 1, :] = 1
+        oraw, oq = quantise(rng.uniform(-6.0, 1.0, (G, sq, sk)).astype(np.float32), t)
     out = rock.attention(to_gpu(rq, t, gpu), to_gpu(rk, t, gpu), to_gpu(rv, t, gpu), scale=scale,
                          bias=to_gpu(braw, t, gpu) if bias else None,
                          scale_tensor=to_gpu(sraw, t, gpu) if scale_tensor else None,
-                         transQ=tQ, transK=tK, transV=tV, transO=tO, info=info)
+                         mask=torch.from_numpy(mk).to(gpu) if mask else None,
+                         other=to_gpu(oraw, t, gpu) if mask else None,
+                         transQ=tQ, transK=tK, transV=tV, transO=tO, info=info, score_workspace_limit=limit)
     torch.cuda.synchronize()
     ref = oracle.attention(Qq, Kq, Vq, G, sq, sk, dqk, dv, scale=scale, bias_t=bq, scale_t=sq_,
-                           transQ=tQ, transK=tK, transV=tV, transO=tO)
+                           transQ=tQ, transK=tK, transV=tV, transO=tO, mask=mk, other=oq)
     return to_f32(out, t), ref
+
+
+def _run_i8(rock, oracle, gpu, G, sq, sk, dqk, dv, bias=False, info=None, limit=None):
+    """int8 Q and K, f16 V: the GPU result and the oracle's, which gets the same scores through a bias that
+    carries -zero_point * scale."""
+    rng = np.random.default_rng(57)
+    Q = rng.integers(-128, 128, (G, sq, dqk)).astype(np.int8)
+    K = rng.integers(-128, 128, (G, sk, dqk)).astype(np.int8)
+    V = rng.standard_normal((G, sk, dv)).astype(np.float32)
+    rv, Vq = quantise(V, "f16")
+    zp, scale = 37, float(np.float16(3.0e-4))
+    braw = bq = None
+    if bias:
+        braw, bq = quantise(rng.standard_normal((G, sq, sk)).astype(np.float32), "f16")
+    out = rock.attention(torch.from_numpy(Q).to(gpu), torch.from_numpy(K).to(gpu), to_gpu(rv, "f16", gpu),
+                         scale=scale, zero_point=zp, bias=to_gpu(braw, "f16", gpu) if bias else None, transK=True,
+                         info=info, score_workspace_limit=limit)
+    torch.cuda.synchronize()
+    shift = np.full((G, sq, sk), -zp * scale, np.float32) + (bq.reshape(G, sq, sk) if bias else 0.0)
+    ref = oracle.attention(Q.astype(np.float32), K.astype(np.float32), Vq, G, sq, sk, dqk, dv, scale=scale,
+                           bias_t=shift.astype(np.float32), transK=True)
+    return to_f32(out, "f16"), ref
 
 
 # PrAttentionF16.toml:20-67 shapes (+ ragged ones)
@@ -119,6 +150,36 @@ def test_attention_with_scale_tensor(rock, oracle, gpu, shape, bias):
     check_float(got, ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
 
 
+@pytest.mark.parametrize("case", [
+    # the reference's own case: 12 heads, 256 x 256 scores, head dimension 256, scale 0.125 (mixr-attn-where.mlir:4-13)
+    dict(id="mixr-attn-where", t="f16", shape=(12, 256, 256, 256, 256), kernels=["rock_attention_f16_d256x256_fast_bias"]),
+    dict(id="d128-ragged-bias", t="f16", shape=(2, 300, 200, 128, 128), bias=True, kernels=["rock_attention_f16_d128x128_fast_bias"]),
+    dict(id="d64-scale-tensor-bf16", t="bf16", shape=(3, 128, 27, 64, 32), scale_tensor=True,
+         kernels=["rock_attention_bf16_d64x64_fast_bias"]),
+    dict(id="default-key-layout", t="f16", shape=(2, 130, 136, 64, 64), tK=False, kernels=["rock_attention_f16_d64x64_fast_bias_kt"]),
+    dict(id="generic", t="f16", shape=(2, 50, 70, 20, 12), kernels=["rock_attention_f16_d64x64_generic"]),
+    dict(id="transposed-q-o", t="f16", shape=(2, 96, 80, 64, 64), tQ=True, tO=True, count=3),
+    dict(id="three-kernels-d320", t="f16", shape=(2, 100, 150, 320, 192), bias=True, count=3),
+    dict(id="three-kernels-f32", t="f32", shape=(2, 96, 80, 64, 64), bias=True, scale_tensor=True, count=3),
+], ids=lambda c: c["id"])
+def test_attention_where_mask(rock, oracle, gpu, case):
+    """migraphx.where(mask, scores, other) in front of the softmax (mixr-attn-where.mlir:11): a zero in the int8
+    mask replaces the score -- after scale tensor, scale and bias -- by other's element.  Every kernel family that
+    takes pre-softmax tensors, rows masked wholly and not at all."""
+    t = case["t"]
+    G, sq, sk, dqk, dv = case["shape"]
+    info = {}
+    got, ref = _run(rock, oracle, gpu, t, G, sq, sk, dqk, dv, 0.125, 71, tQ=case.get("tQ", False),
+                    tK=case.get("tK", True), tO=case.get("tO", False), bias=case.get("bias", False),
+                    scale_tensor=case.get("scale_tensor", False), mask=True, info=info)
+    if "kernels" in case:
+        assert info["kernels"] == case["kernels"]
+    else:
+        assert len(info["kernels"]) == case["count"]
+    gate = {"f16": GATE["f16"], "bf16": GATE["bf16"], "f32": (3e-5, 1e-4)}[t]
+    check_float(got, ref, t, rms=gate[0], max_abs=gate[1])
+
+
 @pytest.mark.parametrize("t", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("shape", [(2, 200, 333, 256, 256), (1, 130, 520, 512, 512), (3, 64, 100, 40, 72)],
                          ids=["d256", "d512", "small"])
@@ -152,6 +213,31 @@ def test_attention_head_dims_up_to_256_fused(rock, oracle, gpu, shape, bias, sca
     check_float(got, ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
 
 
+@pytest.mark.parametrize("case", [
+    dict(id="row-chunks", t="f16", shape=(3, 200, 333, 320, 192), limit=200 << 10, kernels=18),   # 128 + 72 rows per group
+    dict(id="group-chunks", t="f16", shape=(3, 200, 333, 320, 192), limit=600 << 10, kernels=6),  # 2 groups + 1
+    dict(id="f32-transposed", t="f32", shape=(2, 150, 96, 64, 64), limit=40 << 10, kernels=12, tQ=True, tK=False,
+         tV=True, tO=True),
+    dict(id="i8-rows", t="i8", shape=(2, 300, 136, 320, 64), limit=100 << 10, kernels=18),
+], ids=lambda c: c["id"])
+def test_attention_three_kernel_form_in_chunks(rock, oracle, gpu, case):
+    """A score matrix above the workspace bound is worked off chunk by chunk (whole groups, or query rows of one
+    group), three kernels each; pre-softmax tensors and the result are addressed at the chunk's rows."""
+    t = case["t"]
+    G, sq, sk, dqk, dv = case["shape"]
+    info = {}
+    if t == "i8":
+        got, ref = _run_i8(rock, oracle, gpu, G, sq, sk, dqk, dv, info=info, limit=case["limit"])
+        t = "f16"
+    else:
+        got, ref = _run(rock, oracle, gpu, t, G, sq, sk, dqk, dv, 0.1, 57, tQ=case.get("tQ", False),
+                        tK=case.get("tK", True), tV=case.get("tV", False), tO=case.get("tO", False), bias=True,
+                        scale_tensor=True, mask=True, info=info, limit=case["limit"])
+    assert len(info["kernels"]) == case["kernels"], info["kernels"]
+    gate = {"f16": GATE["f16"], "f32": (3e-5, 1e-4)}[t]
+    check_float(got, ref, t, rms=gate[0], max_abs=gate[1])
+
+
 def test_attention_three_kernel_form_with_bias_and_scale_tensor(rock, oracle, gpu):
     got, ref = _run(rock, oracle, gpu, "f16", 2, 100, 150, 320, 192, 0.07, 53, bias=True, scale_tensor=True)
     check_float(got, ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
@@ -169,29 +255,14 @@ def test_attention_int8_first_gemm(rock, oracle, gpu, shape, bias):
     f16 V and output.  The oracle gets the same scores through a bias that
     carries -zero_point * scale."""
     G, sq, sk, dqk, dv = shape
-    rng = np.random.default_rng(57)
-    Q = rng.integers(-128, 128, (G, sq, dqk)).astype(np.int8)
-    K = rng.integers(-128, 128, (G, sk, dqk)).astype(np.int8)
-    V = rng.standard_normal((G, sk, dv)).astype(np.float32)
-    rv, Vq = quantise(V, "f16")
-    zp, scale = 37, float(np.float16(3.0e-4))
-    braw = bq = None
-    if bias:
-        braw, bq = quantise(rng.standard_normal((G, sq, sk)).astype(np.float32), "f16")
     info = {}
-    out = rock.attention(torch.from_numpy(Q).to(gpu), torch.from_numpy(K).to(gpu), to_gpu(rv, "f16", gpu),
-                         scale=scale, zero_point=zp, bias=to_gpu(braw, "f16", gpu) if bias else None, transK=True,
-                         info=info)
-    torch.cuda.synchronize()
+    got, ref = _run_i8(rock, oracle, gpu, G, sq, sk, dqk, dv, bias=bias, info=info)
     if dqk <= 128:  # fused: the int32 score tile is dequantised in registers
         dmax = 64 if max(dqk, dv) <= 64 else 128
         assert info["kernels"] == ["rock_attention_i8_d%dx%d_%s" % (dmax, dmax, "fast_bias" if bias else "fast")]
     else:
         assert len(info["kernels"]) == 3
-    shift = np.full((G, sq, sk), -zp * scale, np.float32) + (bq.reshape(G, sq, sk) if bias else 0.0)
-    ref = oracle.attention(Q.astype(np.float32), K.astype(np.float32), Vq, G, sq, sk, dqk, dv, scale=scale,
-                           bias_t=shift.astype(np.float32), transK=True)
-    check_float(to_f32(out, "f16"), ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
+    check_float(got, ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
 
 
 def test_attention_int8_first_gemm_fused_at_size(rock, oracle, gpu):

@@ -162,10 +162,13 @@ def test_conv3d_bwd_weight_exact(rock, oracle, gpu, case, layouts, t):
         assert any(name.startswith("rock_conv_bwd_weight_") for name in info["kernels"])
 
 
-@pytest.mark.parametrize("t", ["f32", "f16"])
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16"])
 def test_conv3d_gradients_real_values_unet_block(rock, oracle, gpu, t):
     """A 3-D UNet block (32 -> 64 channels at 16^3, batch 2, 3x3x3, padding 1)
-    on real-valued data against the oracle under the reference's RMS gates."""
+    on real-valued data against the oracle under the reference's RMS gates.
+    The 16-bit input gradient is rounded twice (each depth tap's 2-D gradient in
+    the tensor type, then their f32 sum) where the reference rounds once: the
+    gate is the measure of that, bf16 included."""
     n, g, c, k, ins, fs, stride, pad, dil = 2, 1, 32, 64, (16, 16, 16), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)
     rng = np.random.default_rng(99)
     raw_f, fq = quantise(rng.standard_normal(g * k * c * 27).astype(np.float32) * 0.1, t)

@@ -373,6 +373,34 @@ def test_attention_vs_float64_all_layouts(oracle, tQ, tK, tV, tO):
     assert np.allclose(got, want, rtol=0, atol=3e-6)
 
 
+def test_attention_where_mask_vs_float64(oracle):
+    """migraphx.where(mask, scale * Q K^T [+ bias], other) in front of the softmax (mixr-attn-where.mlir:11):
+    against torch.where + softmax in float64; an all-ones mask changes nothing, an all-zero mask makes the
+    weights softmax(other) whatever Q and K hold (an additive mask, or a select on the wrong side, fails both)."""
+    rng = np.random.default_rng(33)
+    G, sq, sk, d, dv = 2, 7, 19, 8, 5
+    Q = rng.standard_normal((G, sq, d)).astype(np.float32)
+    K = rng.standard_normal((G, sk, d)).astype(np.float32)
+    V = rng.standard_normal((G, sk, dv)).astype(np.float32)
+    bias = rng.standard_normal((G, sq, sk)).astype(np.float32)
+    other = rng.standard_normal((G, sq, sk)).astype(np.float32) * 3
+    mask = (rng.random((G, sq, sk)) < 0.6).astype(np.int8)
+    mask[0, 0, :] = 0          # a fully masked row
+    mask[1, 2, :] = 1          # an untouched row
+    att = lambda **kw: oracle.attention(Q, K, V, G, sq, sk, d, dv, transK=True, **kw).reshape(G, sq, dv)
+    for b in (None, bias):
+        S = np.einsum("gid,gjd->gij", Q.astype(np.float64), K.astype(np.float64)) * 0.3
+        if b is not None:
+            S = S + b
+        S = torch.where(torch.from_numpy(mask != 0), torch.from_numpy(S), torch.from_numpy(other.astype(np.float64)))
+        want = np.einsum("gij,gje->gie", torch.softmax(S, dim=-1).numpy(), V.astype(np.float64))
+        assert np.allclose(att(scale=0.3, bias_t=b, mask=mask, other=other), want, rtol=0, atol=3e-6)
+    assert np.array_equal(att(scale=0.3, mask=np.ones_like(mask), other=other), att(scale=0.3))
+    only_other = np.einsum("gij,gje->gie", torch.softmax(torch.from_numpy(other.astype(np.float64)), dim=-1).numpy(),
+                           V.astype(np.float64))
+    assert np.allclose(att(scale=0.3, mask=np.zeros_like(mask), other=other), only_other, rtol=0, atol=3e-6)
+
+
 def test_attention_invariants(oracle):
     rng = np.random.default_rng(21)
     G, sq, sk, d, dv = 1, 4, 16, 8, 6
@@ -414,6 +442,39 @@ def test_quantize_formula(oracle):
     assert got.tolist() == [1, 1, 3, 3, 1, -1, 127, -128, 127]
     assert oracle.quantize_i8(np.array([63.4], np.float32), 0.5, 0)[0] == 127
     assert oracle.quantize_i8(np.array([63.2], np.float32), 0.5, 0)[0] == 126
+
+
+def test_per_channel_quantisation_formulas(oracle):
+    """One scale and zero point per output channel (MIGraphXToTosa.cpp:874-982 with broadcast tensors, as in
+    mixr-resnet-fusion-case-1-quantization.mlir:8-9): hand-computed values, channel c must see only element c
+    of each vector (a transposed or shifted index fails), and constant vectors reduce to the per-tensor routines."""
+    acc = np.array([[10, -20, 7], [3, 4, -5]], np.int64)
+    scale = np.array([0.5, 0.25, 2.0], np.float32)
+    zp = np.array([2, 0, -1], np.int32)
+    got = oracle.dequantize_per_channel(acc, scale, zp)
+    assert got.tolist() == [[4.0, -5.0, 16.0], [0.5, 1.0, -8.0]]
+    assert oracle.dequantize_per_channel(acc, scale).tolist() == [[5.0, -5.0, 14.0], [1.5, 1.0, -10.0]]
+    x = np.array([[1.0, 1.0, 1.0], [-3.3, 0.3, 300.0]], np.float32)
+    qs = np.array([0.5, 0.25, 2.0], np.float32)
+    qz = np.array([0, 10, -100], np.int32)
+    # 1/0.5 = 2, 1/0.25 = 4, 1/2 = 0.5: round_even(x * inv) + zp, clamped
+    assert oracle.quantize_i8_per_channel(x, qs, qz).tolist() == [[2, 14, -100], [-7, 11, 50]]
+    assert oracle.quantize_i8_per_channel(x, qs).tolist() == [[2, 4, 0], [-7, 1, 127]]
+    rng = np.random.default_rng(5)
+    big = rng.integers(-2 ** 20, 2 ** 20, (37, 11)).astype(np.int64)
+    assert np.array_equal(oracle.dequantize_per_channel(big, np.full(11, 0.013, np.float32), np.full(11, -4, np.int32)),
+                          oracle.dequantize(big, 0.013, -4))
+    xf = rng.standard_normal((37, 11)).astype(np.float32) * 50
+    assert np.array_equal(oracle.quantize_i8_per_channel(xf, np.full(11, 0.37, np.float32), np.full(11, 5, np.int32)),
+                          oracle.quantize_i8(xf, 0.37, 5))
+    # column by column against the per-tensor routine with that column's values
+    sc = rng.uniform(0.01, 2.0, 11).astype(np.float32)
+    zz = rng.integers(-9, 9, 11).astype(np.int32)
+    d = oracle.dequantize_per_channel(big, sc, zz)
+    q = oracle.quantize_i8_per_channel(xf, sc, zz)
+    for c in range(11):
+        assert np.array_equal(d[:, c], oracle.dequantize(big[:, c].copy(), sc[c], int(zz[c])))
+        assert np.array_equal(q[:, c], oracle.quantize_i8(xf[:, c].copy(), sc[c], int(zz[c])))
 
 
 def test_scale_bias(oracle):
