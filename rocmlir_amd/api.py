@@ -380,6 +380,23 @@ class RockProgram:
         """Sum of the kernels' average times in milliseconds."""
         return sum(ms for _, ms in self.benchmark_each(*args, warmup=warmup, iters=iters, stream=stream))
 
+    def benchmark_sequence(self, *args, warmup=2, iters=5):
+        """Average milliseconds for the whole list launched in order, back to back (events on torch's current
+        stream, where launch() puts the kernels): what a caller of a many-kernel problem waits for, gaps between
+        the kernels and the state of the caches they leave each other included."""
+        import torch
+        full = self._args(args)
+        for _ in range(warmup):
+            self.launch(*args)
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(iters):
+            for k in self.kernels:
+                k.launch(*full)
+        stop.record()
+        stop.synchronize()
+        return start.elapsed_time(stop) / iters
+
     def benchmark_each(self, *args, warmup=3, iters=20, stream=None):
         """[(kernel name, average time in milliseconds)] in launch order."""
         full = self._args(args)

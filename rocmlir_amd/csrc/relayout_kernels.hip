@@ -134,6 +134,7 @@ __device__ __forceinline__ float load_as_f32(const void *base, int64_t idx, int 
   return __builtin_bit_cast(float, (uint32_t)((const uint16_t *)base)[idx] << 16);
 }
 
+// over the block's waves (at most 16); scratch holds one float per wave
 __device__ __forceinline__ float block_reduce(float v, bool take_max, float *scratch) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
@@ -144,27 +145,28 @@ __device__ __forceinline__ float block_reduce(float v, bool take_max, float *scr
   if ((threadIdx.x & 63) == 0)
     scratch[threadIdx.x >> 6] = v;
   __syncthreads();
+  const int waves = (int)blockDim.x >> 6;
   float r = scratch[0];
-#pragma unroll
-  for (int w = 1; w < 4; ++w)
+  for (int w = 1; w < waves; ++w)
     r = take_max ? fmaxf(r, scratch[w]) : r + scratch[w];
   return r;
 }
 } // namespace
 
-// One block per row, three passes over it (maximum, sum, normalise); the last
-// pass loads a chunk of scores into registers before any thread overwrites the
-// narrower results over them.
-#if RK_SELECTED(5)
-extern "C" __global__ __launch_bounds__(256) void rock_softmax_rows(float *S, const void *scale_t, const void *bias,
-                                                                    const void *mask, const void *other,
-                                                                    RockSoftmaxParams p) {
-  __shared__ float scratch[4];
-  const int64_t row = blockIdx.x;
-  const int g = (int)(row / p.seq_q), i = (int)(row - (int64_t)g * p.seq_q);
-  float *s = S + row * p.row_pitch;
-  const int64_t t_off = (int64_t)g * p.t_gs + (int64_t)i * p.t_is;
-  auto score = [&](int j) {
+// One block per row: 256 threads, or 1024 for rows above 4096 scores (the
+// host picks).  A row of up to 16 scores per thread is read once into
+// registers (the pre-softmax tensors applied on the way), reduced twice and
+// written once -- 4 bytes read and one result written per score; longer rows
+// take three passes over memory (maximum, sum, normalise).  Either way every
+// score of a stretch is in a register before any thread writes the narrower
+// results over the row.
+namespace {
+struct SoftmaxRow {
+  float *s;
+  const void *scale_t, *bias, *mask, *other;
+  int64_t t_off;
+  const RockSoftmaxParams &p;
+  __device__ __forceinline__ float score(int j) const {
     float x = s[j];
     if (p.has_scale_tensor)
       x = x * load_as_f32(scale_t, t_off + (int64_t)j * p.t_js, p.dtype);
@@ -174,30 +176,129 @@ extern "C" __global__ __launch_bounds__(256) void rock_softmax_rows(float *S, co
     if (p.has_mask && ((const int8_t *)mask)[t_off + (int64_t)j * p.t_js] == 0) // where(mask, x, other)
       x = load_as_f32(other, t_off + (int64_t)j * p.t_js, p.dtype);
     return x;
-  };
+  }
+  __device__ __forceinline__ void store(int j, float e) const {
+    if (p.dtype == ROCK_F32)
+      s[j] = e;
+    else if (p.dtype == ROCK_F16)
+      ((_Float16 *)s)[j] = (_Float16)e;
+    else
+      ((__bf16 *)s)[j] = (__bf16)e;
+  }
+};
+
+__device__ __forceinline__ float widen(float x) { return x; }
+__device__ __forceinline__ float widen(_Float16 x) { return (float)x; }
+__device__ __forceinline__ float widen(__bf16 x) { return (float)x; }
+
+// Rows of at most EPT * NT scores, NT threads; T is the type of P and of the
+// pre-softmax tensors.  Loads are unconditional (columns beyond the row read its last
+// score and are set to -inf afterwards) and each tensor has a loop of its
+// own, so that a thread's loads are all in flight together.
+template <int EPT, int NT, typename T>
+__device__ __forceinline__ void softmax_row_in_registers(const SoftmaxRow &row, float *scratch) {
+  const RockSoftmaxParams &p = row.p;
+  const int n = p.seq_k, tid = (int)threadIdx.x;
+  float v[EPT];
+#pragma unroll
+  for (int c = 0; c < EPT; ++c)
+    v[c] = row.s[min(c * NT + tid, n - 1)];
+  if (p.has_scale_tensor) {
+    const T *t = (const T *)row.scale_t + row.t_off;
+#pragma unroll
+    for (int c = 0; c < EPT; ++c)
+      v[c] = v[c] * widen(t[(int64_t)min(c * NT + tid, n - 1) * p.t_js]);
+  }
+#pragma unroll
+  for (int c = 0; c < EPT; ++c)
+    v[c] = v[c] * p.scale;
+  if (p.has_bias) {
+    const T *t = (const T *)row.bias + row.t_off;
+#pragma unroll
+    for (int c = 0; c < EPT; ++c)
+      v[c] = v[c] + widen(t[(int64_t)min(c * NT + tid, n - 1) * p.t_js]);
+  }
+  if (p.has_mask) { // where(mask, x, other)
+    const int8_t *mk = (const int8_t *)row.mask + row.t_off;
+    const T *t = (const T *)row.other + row.t_off;
+#pragma unroll
+    for (int c = 0; c < EPT; ++c) {
+      const int64_t at = (int64_t)min(c * NT + tid, n - 1) * p.t_js;
+      const float o = widen(t[at]);
+      v[c] = mk[at] == 0 ? o : v[c];
+    }
+  }
   float m = -INFINITY;
-  for (int j = threadIdx.x; j < p.seq_k; j += 256)
-    m = fmaxf(m, score(j));
+#pragma unroll
+  for (int c = 0; c < EPT; ++c) {
+    v[c] = c * NT + tid < n ? v[c] : -INFINITY;
+    m = fmaxf(m, v[c]);
+  }
   m = block_reduce(m, true, scratch);
   float l = 0.0f;
-  for (int j = threadIdx.x; j < p.seq_k; j += 256)
-    l = l + expf(score(j) - m);
+#pragma unroll
+  for (int c = 0; c < EPT; ++c) {
+    v[c] = expf(v[c] - m); // (columns beyond the row: exp(-inf) = 0)
+    l = l + v[c];
+  }
+  l = block_reduce(l, false, scratch); // its barriers also separate the reads above from the stores below
+  const float inv = 1.0f / l;
+  T *out = (T *)row.s;
+#pragma unroll
+  for (int c = 0; c < EPT; ++c) {
+    const int j = c * NT + tid;
+    if (j < n)
+      out[j] = (T)(v[c] * inv);
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ bool softmax_short_row(const SoftmaxRow &row, float *scratch) {
+  const int n = row.p.seq_k;
+  if (blockDim.x == 1024) {
+    if (n > 16 * 1024)
+      return false;
+    softmax_row_in_registers<16, 1024, T>(row, scratch);
+  } else if (n <= 4 * 256) {
+    softmax_row_in_registers<4, 256, T>(row, scratch);
+  } else if (n <= 16 * 256) {
+    softmax_row_in_registers<16, 256, T>(row, scratch);
+  } else {
+    return false;
+  }
+  return true;
+}
+} // namespace
+#if RK_SELECTED(5)
+extern "C" __global__ __launch_bounds__(1024) void rock_softmax_rows(float *S, const void *scale_t, const void *bias,
+                                                                     const void *mask, const void *other,
+                                                                     RockSoftmaxParams p) {
+  __shared__ float scratch[16];
+  const int64_t r = blockIdx.x;
+  const int g = (int)(r / p.seq_q), i = (int)(r - (int64_t)g * p.seq_q);
+  const SoftmaxRow row{S + r * p.row_pitch, scale_t, bias, mask, other, (int64_t)g * p.t_gs + (int64_t)i * p.t_is, p};
+  if (p.dtype == ROCK_F32 ? softmax_short_row<float>(row, scratch)
+      : p.dtype == ROCK_F16 ? softmax_short_row<_Float16>(row, scratch)
+                            : softmax_short_row<__bf16>(row, scratch))
+    return;
+  const int nt = (int)blockDim.x, tid = (int)threadIdx.x;
+  float m = -INFINITY;
+  for (int j = tid; j < p.seq_k; j += nt)
+    m = fmaxf(m, row.score(j));
+  m = block_reduce(m, true, scratch);
+  float l = 0.0f;
+  for (int j = tid; j < p.seq_k; j += nt)
+    l = l + expf(row.score(j) - m);
   l = block_reduce(l, false, scratch);
   const float inv = 1.0f / l;
-  for (int j0 = 0; j0 < p.seq_k; j0 += 256) {
-    const int j = j0 + (int)threadIdx.x;
+  for (int j0 = 0; j0 < p.seq_k; j0 += nt) {
+    const int j = j0 + tid;
     float e = 0.0f;
     if (j < p.seq_k)
-      e = expf(score(j) - m) * inv;
-    __syncthreads(); // every score of this chunk is in a register
-    if (j < p.seq_k) {
-      if (p.dtype == ROCK_F32)
-        s[j] = e;
-      else if (p.dtype == ROCK_F16)
-        ((_Float16 *)s)[j] = (_Float16)e;
-      else
-        ((__bf16 *)s)[j] = (__bf16)e;
-    }
+      e = expf(row.score(j) - m) * inv;
+    __syncthreads(); // every score of this stretch is in a register
+    if (j < p.seq_k)
+      row.store(j, e);
   }
 }
 #endif

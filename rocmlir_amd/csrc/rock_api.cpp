@@ -3580,12 +3580,16 @@ Handle *make_conv(const OptMap &o) {
 // in place, and the GEMM P V.  The reference fuses every shape
 // (GridwiseGemmToBlockwise.cpp:1607-2403); its validator computes these same
 // three steps (rocmlir-gen.cpp:2565-2620).
-// A score matrix above kScoreChunkBytes is worked off in chunks of whole
-// groups, or of query rows of one group, each with its own three kernels in
-// the list (kernel_id = 3 * chunk + step): the workspace holds one chunk --
-// small enough for the array of rockamdLaunchStaticWorkspace and for the
-// scores to stay in the memory-side cache between the three kernels -- instead
-// of G * seq_q * seq_k * 4 bytes.
+// A score matrix that fits the array of rockamdLaunchStaticWorkspace is worked
+// on in one piece.  A larger one is worked off in chunks of kScoreChunkBytes --
+// whole groups, or query rows of one group -- each with its own kernels in the
+// list (kernel_id = kernels per chunk * chunk + step): the workspace holds one
+// chunk, small enough for that array and for the scores to stay in the
+// memory-side cache between the kernels, instead of G * seq_q * seq_k * 4
+// bytes.  A chunk of one group's rows leaves the second GEMM few output tiles
+// and a long reduction; that one is split over blocks as a GEMM of its own
+// would be (f32 partial sums behind the scores, a fourth kernel adds them up).
+constexpr int64_t kScoreWholeBytes = ROCKAMD_STATIC_WORKSPACE_BYTES - ((int64_t)16 << 20); // room for the partial sums
 constexpr int64_t kScoreChunkBytes = (int64_t)32 << 20;
 Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, int64_t sk, int64_t dqk, int64_t dv,
                                bool tQ, bool tK, bool tV, bool tO, bool has_bias, bool has_scale_t, bool has_mask) {
@@ -3599,7 +3603,10 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
   const int es = dtype_size(ty);
   // chunk = gc groups x rc query rows
   // ("-score_workspace_limit BYTES" moves the bound, e.g. to keep one chunk inside a smaller cache share)
-  const int64_t limit = std::max<int64_t>(int_or(o, "score_workspace_limit", kScoreChunkBytes), sk * 4);
+  const int64_t limit =
+      std::max<int64_t>(int_or(o, "score_workspace_limit", G * sq * sk * 4 <= kScoreWholeBytes ? kScoreWholeBytes
+                                                                                                : kScoreChunkBytes),
+                        sk * 4);
   int64_t gc = G, rc = sq;
   if (G * sq * sk * 4 > limit) {
     if (sq * sk * 4 <= limit) {
@@ -3611,17 +3618,28 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
     }
   }
   const int64_t row_chunks = ceil_div(sq, rc), chunks = ceil_div(G, gc) * row_chunks;
+  // the second GEMM of a one-group chunk: its reduction over the keys in S shares (as make_gemm splits a GEMM)
+  int64_t S = 1;
+  if (gc == 1 && bool_or(o, "split_k", true)) {
+    const int64_t tiles64 = (int64_t)ceil_div(rc, 64) * ceil_div(dv, 64);
+    if (sk >= 2048 && tiles64 * 2 <= kNumCU)
+      for (int64_t d = std::min<int64_t>(2 * kNumCU / tiles64, sk / 512); d >= 2 && S == 1; --d)
+        if (sk % d == 0 && (sk / d * es) % 64 == 0)
+          S = d;
+  }
+  const int per_chunk = S > 1 ? 4 : 3;
+  const int64_t score_bytes = align256(gc * rc * sk * 4), partial_bytes = S > 1 ? align256(S * rc * dv * 4) : 0;
   const int64_t kid_all = int_or(o, "kernel_id", 0);
-  if (chunks * 3 > INT32_MAX || gc * rc > INT32_MAX) {
+  if (chunks * per_chunk > INT32_MAX || gc * rc > INT32_MAX) {
     set_error("attention: score matrix too large for the three-kernel form");
     return nullptr;
   }
-  if (kid_all < 0 || kid_all >= 3 * chunks) {
+  if (kid_all < 0 || kid_all >= per_chunk * chunks) {
     set_error("attention: kernel_id out of range");
     return nullptr;
   }
-  const int kid = (int)(kid_all % 3);
-  const int64_t g0 = kid_all / 3 / row_chunks * gc, r0 = kid_all / 3 % row_chunks * rc;
+  const int kid = (int)(kid_all % per_chunk);
+  const int64_t g0 = kid_all / per_chunk / row_chunks * gc, r0 = kid_all / per_chunk % row_chunks * rc;
   const int64_t gn = std::min(gc, G - g0), rn = std::min(rc, sq - r0); // this chunk
   float scale = 1.0f;
   get_float(o, "scale", scale);
@@ -3646,7 +3664,7 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
     h->params.assign(sizeof r, 0);
     std::memcpy(h->params.data(), &r, sizeof r);
     h->kernel_name = "rock_softmax_rows";
-    h->block_size = 256;
+    h->block_size = sk > 4096 ? 1024 : 256; // rows up to 16 scores per thread stay in registers
     h->grid_size = (uint32_t)(gn * rn);
     h->num_pointers = 5;
     h->perf_config = "";
@@ -3654,6 +3672,25 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
     h->ptr_map = {{i_ws, 0}, {has_scale_t ? 3 : -1, t_off}, {has_bias ? i_bias : -1, t_off}, {i_mask, t_off / es},
                   {i_other, t_off}};
     h->problem_key = "row softmax of the attention scores";
+  } else if (kid == 3) { // O = the sum of the shares' partial results
+    RockReduceParams r;
+    std::memset(&r, 0, sizeof r);
+    r.split_stride = rn * dv;
+    r.size[0] = 1; r.size[1] = 1; r.size[2] = (int)rn; r.size[3] = (int)dv;
+    r.dst_stride[2] = tO ? 1 : dv; r.dst_stride[3] = tO ? sq : 1;
+    r.splits = (int)S;
+    r.out_dtype = ty;
+    h->op = OP_RELAYOUT;
+    h->epi = nullptr;
+    h->params.assign(sizeof r, 0);
+    std::memcpy(h->params.data(), &r, sizeof r);
+    h->kernel_name = "rock_reduce_splits";
+    h->block_size = 256;
+    h->grid_size = (uint32_t)((rn * dv + 255) / 256);
+    h->num_pointers = 2;
+    h->perf_config = "";
+    h->ptr_map = {{i_ws, score_bytes}, {i_out, (g0 * sq * dv + r0 * (tO ? 1 : dv)) * es}};
+    h->problem_key = "reduction of the split partial sums";
   } else {
     RockGemmParams gp;
     std::memset(&gp, 0, sizeof gp);
@@ -3678,13 +3715,21 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
       a_off = 0;
       b_off = g0 * gp.b_gs * es;
       c_off = (g0 * gp.c_gs + r0 * gp.c_ms) * es;
+      if (S > 1) { // share s: keys s * sk / S onwards, f32 partial result s behind the scores
+        const int64_t ks = sk / S;
+        gp.G = (int)S; gp.K = (int)ks;
+        gp.a_gs = ks; gp.b_gs = ks * gp.b_ks;
+        gp.c_gs = rn * dv; gp.c_ms = dv; gp.c_ns = 1;
+        default_epilogue(gp.epi, ROCK_F32);
+        c_off = score_bytes;
+      }
     }
     const int tg = kid == 0 ? tq : ty;
     plan_gemm_kernel(h, gp, operand_code(tg, tg), dtype_size(tg), o);
     if (kid == 0)
       h->ptr_map = {{0, a_off}, {1, b_off}, {i_ws, c_off}, {-1, 0}, {-1, 0}};
     else
-      h->ptr_map = {{i_ws, a_off}, {2, b_off}, {i_out, c_off}, {-1, 0}, {-1, 0}};
+      h->ptr_map = {{i_ws, a_off}, {2, b_off}, {S > 1 ? i_ws : i_out, c_off}, {-1, 0}, {-1, 0}};
     h->op = OP_GEMM;
     h->params.assign(sizeof gp, 0);
     std::memcpy(h->params.data(), &gp, sizeof gp);
@@ -3696,8 +3741,8 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
         << sq << " -seq_len_k " << sk << " -head_dim_qk " << dqk << " -head_dim_v " << dv;
     h->problem_key = key.str();
   }
-  h->kernel_count = (int)(3 * chunks);
-  h->workspace_bytes = (size_t)(gc * rc * sk * 4);
+  h->kernel_count = (int)(per_chunk * chunks);
+  h->workspace_bytes = (size_t)(partial_bytes ? score_bytes + partial_bytes : gc * rc * sk * 4);
   h->caller_pointers = i_ws + 1;
   return h;
 }

@@ -146,6 +146,8 @@ def run_problem(rock, torch, dev, opts, shapes, flops, warmup, iters, warm_ms=0.
                                                                                      "rock_attention"))]
     res = {"status": "ok", "kernel": contraction[-1], "kernels": len(prog.kernels), "ms": round(ms, 5),
            "tflops": round(flops / (ms * 1e-3) / 1e12, 2)}
+    if len(prog.kernels) > 1:  # the list launched back to back, beside the sum of the kernels timed one by one
+        res["sequence_ms"] = round(prog.benchmark_sequence(*args), 5)
     if per_kernel:
         res["kernel_ms"] = [[name, round(t, 5)] for name, t in each]
     if tune_kind:

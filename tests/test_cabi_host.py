@@ -5,6 +5,7 @@ perf-config / problem-key strings in the reference's grammar."""
 import ctypes as C
 import os
 import re
+import struct
 
 import pytest
 
@@ -342,13 +343,19 @@ def test_attention_as_three_kernels(rock):
         assert ks[2].kernel_name.startswith("rock_gemm_%s_" % t) and ks[2].kernel_name.endswith("_fast_nn")
         assert all(k.kernel_count == 3 and k.workspace_bytes == 16384 * 16384 * 4 and k.caller_pointers == 6
                    for k in ks)
-        # by default in chunks of at most 32 MiB of scores: 512 query rows x 16384 keys, 32 chunks of three kernels
-        ks = [rock.RockKernel(vae % t + " -kernel_id %d" % i) for i in (0, 1, 2, 94, 95)]
-        assert all(k.kernel_count == 96 and k.workspace_bytes == 32 << 20 and k.caller_pointers == 6 for k in ks)
+        # by default in chunks of at most 32 MiB of scores: 512 query rows x 16384 keys, 32 chunks of four kernels
+        # (the second GEMM's 512 x 512 result in 8 shares of the keys, f32 partial sums behind the scores)
+        ks = [rock.RockKernel(vae % t + " -kernel_id %d" % i) for i in (0, 1, 2, 3, 125, 126, 127)]
+        assert all(k.kernel_count == 128 and k.workspace_bytes == (32 << 20) + 8 * 512 * 512 * 4 and
+                   k.caller_pointers == 6 for k in ks)
         assert ks[1].kernel_name == "rock_softmax_rows" and ks[1].grid_size == 512
-        assert ks[3].kernel_name == "rock_softmax_rows" and ks[4].kernel_name == ks[2].kernel_name
+        assert ks[2].kernel_name.startswith("rock_gemm_%s_" % t) and struct.unpack_from("<4i", ks[2].params(), 72) == (8, 512, 512, 2048)   # G M N K
+        assert ks[3].kernel_name == "rock_reduce_splits" and ks[6].kernel_name == "rock_reduce_splits"
+        assert ks[4].kernel_name == "rock_softmax_rows" and ks[5].kernel_name == ks[2].kernel_name
         with pytest.raises(rock.RockError):
-            rock.RockKernel(vae % t + " -kernel_id 96")
+            rock.RockKernel(vae % t + " -kernel_id 128")
+        three = [rock.RockKernel(vae % t + " -split_k false -kernel_id %d" % i) for i in (0, 95)]
+        assert all(k.kernel_count == 96 and k.workspace_bytes == 32 << 20 for k in three)
     # many small groups: whole groups per chunk (8 x 2048 x 2048 f32 scores = 128 MiB -> 2 groups a chunk)
     k = rock.RockKernel("-operation attention -arch gfx950 -t f32 -g 7 -seq_len_q 2048 -seq_len_k 2048 "
                         "-head_dim_qk 64 -head_dim_v 64 -transK true -kernel_id 9")

@@ -219,6 +219,9 @@ def test_attention_head_dims_up_to_256_fused(rock, oracle, gpu, shape, bias, sca
     dict(id="f32-transposed", t="f32", shape=(2, 150, 96, 64, 64), limit=40 << 10, kernels=12, tQ=True, tK=False,
          tV=True, tO=True),
     dict(id="i8-rows", t="i8", shape=(2, 300, 136, 320, 64), limit=100 << 10, kernels=18),
+    # chunks of one group's rows with many keys: the second GEMM's reduction in 4 shares, a fourth kernel per chunk
+    dict(id="row-chunks-split-keys", t="f16", shape=(2, 200, 2048, 320, 192), limit=1 << 20, kernels=16, tO=True),
+    dict(id="whole-f32-split-keys", t="f32", shape=(1, 130, 4096, 64, 72), limit=None, kernels=4),
 ], ids=lambda c: c["id"])
 def test_attention_three_kernel_form_in_chunks(rock, oracle, gpu, case):
     """A score matrix above the workspace bound is worked off chunk by chunk (whole groups, or query rows of one
