@@ -345,22 +345,7 @@ ROCMLIR_AMD_API int rockamdLaunch(MiirHandle handle, void *const *pointers, int 
 ROCMLIR_AMD_API int rockamdLaunchStaticWorkspace(MiirHandle handle, void *const *pointers, int num_pointers,
                                                  void *stream);
 
-/* Timed loop with HIP events on `stream`: `warmup` untimed launches, then
- * `iters` launches between one start/stop event pair; writes the average
- * milliseconds per launch.  Synchronises the stream. */
-ROCMLIR_AMD_API int rockamdBenchmark(MiirHandle handle, void *const *pointers, int num_pointers,
-                     void *stream, int warmup, int iters, float *avg_ms);
-
-/* Matrix-core issue-rate probe on the current device: runs a register-only
- * chain of 32x32 MFMAs of the given operand type (a RockDType value: f32, f16,
- * bf16, i8 or fp8) and writes the sustained rate in tera-operations per
- * second.  `random_data` != 0 gives the operands hashed bit patterns instead
- * of constants; the gap between the two is the clock the part gives up to
- * power on real data.  The reference has no counterpart (its perf scripts
- * compare against rocBLAS instead, mlir/utils/performance/perfRunner.py);
- * the benchmark reports it next to every roofline fraction. */
-ROCMLIR_AMD_API int rockamdMeasureMfmaRate(int dtype, int random_data, void *stream,
-                                           double *tera_ops);
+/* (The measurement helpers -- rockamdBenchmark, rockamdMeasureMfmaRate -- are declared in rocmlir_amd_bench.h.) */
 
 /* Text of the last failure on the calling thread ("" if none). */
 ROCMLIR_AMD_API const char *rockamdGetLastError(void);

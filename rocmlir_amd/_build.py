@@ -109,6 +109,10 @@ def attention_kernels():
     return out
 
 
+# translation units of the host side (csrc/<unit>.cpp)
+HOST_UNITS = ["rock_options", "plan_gemm", "plan_relayout", "plan_conv", "plan_conv_bwd_data", "plan_conv_bwd_weight",
+              "plan_conv3d", "plan_attention", "rock_handle", "rock_launch", "miir_api", "bench_api"]
+
 # kernels of csrc/relayout_kernels.hip in file order (-DROCK_KERNEL=<position>)
 RELAYOUT_KERNELS = ["rock_relayout_b1", "rock_relayout_b2", "rock_relayout_b4", "rock_fill_zero",
                     "rock_reduce_splits", "rock_softmax_rows", "rock_relayout_pair_b1", "rock_relayout_pair_b2",
@@ -179,7 +183,7 @@ def _compile(job):
 
 
 def build(jobs=8, verbose=False, host_only=False, only=None, incremental=False):
-    """host_only: relink rock_api.cpp against the code objects already built;
+    """host_only: recompile the host units and relink against the code objects already built;
     only: rebuild just the code objects whose kernel name contains this string;
     incremental: skip code objects newer than every file under csrc/."""
     os.makedirs(GEN, exist_ok=True)
@@ -200,7 +204,7 @@ def build(jobs=8, verbose=False, host_only=False, only=None, incremental=False):
         raise RuntimeError("code objects missing (build without host_only / only first): %s" % missing[:5])
     for n in names:
         _check(n)
-    # table of the embedded code objects for rock_api.cpp, and the assembly that places them
+    # table of the embedded code objects for rock_options.cpp, and the assembly that places them
     with open(os.path.join(BUILD, "blobs.inc"), "w") as f:
         f.write("// generated by rocmlir_amd/_build.py: one gfx950 code object per kernel\n")
         f.writelines("ROCK_BLOB(%s)\n" % n for n in names)
@@ -214,10 +218,18 @@ def build(jobs=8, verbose=False, host_only=False, only=None, incremental=False):
     _run([HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden",
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
           "-c", os.path.join(CSRC, "static_workspace.hip"), "-o", static_o])
-    _run([HIPCC, "-O2", "-std=c++17", "-fPIC", "-shared", "-x", "c++",
-          "-D__HIP_PLATFORM_AMD__", "-fvisibility=hidden",
-          "-I", os.path.join(ROCM, "include"), "-I", BUILD,
-          os.path.join(CSRC, "rock_api.cpp"), "-x", "none", blobs_o, static_o,
+    # the host side: one object per translation unit, compiled as plain C++ against the HIP runtime API
+    host_objects = []
+
+    def host_compile(unit):
+        obj = os.path.join(BUILD, unit + ".o")
+        _run([HIPCC, "-O2", "-std=c++17", "-fPIC", "-x", "c++", "-D__HIP_PLATFORM_AMD__", "-fvisibility=hidden",
+              "-I", os.path.join(ROCM, "include"), "-I", BUILD, "-c", os.path.join(CSRC, unit + ".cpp"), "-o", obj])
+        return obj
+
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        host_objects = list(pool.map(host_compile, HOST_UNITS))
+    _run([HIPCC, "-fPIC", "-shared", *host_objects, blobs_o, static_o,
           "-L", os.path.join(ROCM, "lib"), "-lamdhip64",
           "-Wl,-rpath," + os.path.join(ROCM, "lib"),
           "-o", LIB])
