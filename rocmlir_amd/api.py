@@ -503,7 +503,7 @@ def gemm(a, b, *, transA=False, transB=False, transC=False, out_dtype=None,
          scale=None, zero_point=0, bias=None, relu=False, quant_scale=None,
          out_zero_point=0, activation=None, clip=None, residual=None,
          residual_op="add", out=None, perf_config=None, stream=None,
-         info=None, split_k=True, layout_conversion=True):
+         info=None, split_k=True, layout_conversion=True, accumulate=False):
     """C = epilogue(A x B) with the reference's storage conventions
     (rocmlir-gen.cpp:2058-2080): a is [G,M,K] ([G,K,M] if transA), b is
     [G,K,N] ([G,N,K] if transB), result [G,M,N] ([G,N,M] if transC).
@@ -518,8 +518,12 @@ def gemm(a, b, *, transA=False, transB=False, transC=False, out_dtype=None,
     perf_config of the GEMM kernel that ran and the names of all kernels of
     the problem (operands that are not whole 16-byte chunks are first copied
     into padded ones unless `layout_conversion` is False; a long reduction
-    over few output tiles is split over blocks unless `split_k` is False)."""
+    over few output tiles is split over blocks unless `split_k` is False).
+    `accumulate=True` (rocmlir-gen's -store-method atomic_add) adds the
+    result into `out` instead of overwriting it."""
     import torch
+    if accumulate and (out is None or residual is not None):
+        raise RockError("gemm: accumulate=True adds into `out` and takes no residual")
     a3 = a if a.dim() == 3 else a.unsqueeze(0)
     b3 = b if b.dim() == 3 else b.unsqueeze(0)
     a3, b3 = a3.contiguous(), b3.contiguous()
@@ -542,6 +546,8 @@ def gemm(a, b, *, transA=False, transB=False, transC=False, out_dtype=None,
         opts += " -split_k false"
     if not layout_conversion:
         opts += " -layout_conversion false"
+    if accumulate:
+        opts += " -store-method atomic_add"
     opts += _epilogue_flags(scale, zero_point, bias, relu, quant_scale,
                             out_zero_point, activation, clip, residual,
                             residual_op)

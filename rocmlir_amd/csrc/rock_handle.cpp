@@ -129,7 +129,9 @@ void describe_arguments(const OptMap &o, Handle *h) {
 }
 
 // problem description -> resolved kernel; NULL with the error set on failure
-Handle *build_handle(const OptMap &o) {
+Handle *build_handle(const OptMap &given) {
+  OptMap planned = given;
+  const OptMap &o = planned;
   // arch: "[triple:]gfxNNN[:features]" (ConvGenerator.cpp:538-552); only
   // gfx950 has kernels here
   std::string arch = str_or(o, "arch", "gfx950");
@@ -139,13 +141,26 @@ Handle *build_handle(const OptMap &o) {
   }
   // Flags of rocmlir-gen that change what a kernel computes and that no kernel here implements are refused
   // rather than ignored (its scheduling and instruction-set toggles -- reverse_grid, mfma, wmma, dot, x2 -- are
-  // ignored: they leave the results alone): an accumulating store (rocmlir-gen.cpp:295-331; pass the tensor
-  // as "-residual add" instead), and the non-OCP 8-bit float encodings (rocmlir-gen.cpp:772-785; gfx950's
-  // matrix cores take e4m3fn / e5m2).
+  // ignored: they leave the results alone): the non-OCP 8-bit float encodings (rocmlir-gen.cpp:772-785;
+  // gfx950's matrix cores take e4m3fn / e5m2).
+  // "-store-method atomic_add" (rocmlir-gen.cpp:295-331: C += A B, what the reference's split-K kernels do to a
+  // pre-filled C, RockOps.td:136-181) is the residual epilogue with C itself as the addend: the problem is
+  // planned with "-residual add" and the residual's place in every kernel's pointer map is then given to the
+  // output, so the caller's list stays A, B, C, bias.  Every element is read by the thread (direct stores) or
+  // the wave (staged stores) that afterwards writes it, so reading and writing one tensor is safe; the sum is
+  // formed in f32 and rounded once, where an atomic add of a 16-bit partial result rounds twice.
+  bool accumulate = false;
   {
     const std::string store = str_or(o, "store-method", str_or(o, "store_method", "set"));
-    if (store != "set") {
-      set_error("store-method '" + store + "' is not built: outputs are overwritten (an addend goes in as -residual add)");
+    if (store == "atomic_add") {
+      if (str_or(o, "operation", "") != "gemm" || str_or(o, "residual", "none") != "none") {
+        set_error("store-method atomic_add: GEMM problems without a residual tensor (C itself is the addend)");
+        return nullptr;
+      }
+      accumulate = true;
+      planned["residual"] = "add";
+    } else if (store != "set") {
+      set_error("store-method '" + store + "': set and atomic_add are the two there are");
       return nullptr;
     }
     const std::string f8 = str_or(o, "force-f8-types", str_or(o, "force_f8_types", "arch"));
@@ -184,6 +199,16 @@ Handle *build_handle(const OptMap &o) {
     return nullptr;
   }
   h->num_cu = (int)int_or(o, "num_cu", kNumCU);
+  if (accumulate) {
+    // caller list as planned: A, B, C, bias, residual, [workspace]; the residual goes, C stands in for it
+    const int base = h->caller_pointers ? h->caller_pointers : h->num_pointers;
+    if (h->ptr_map.empty())
+      for (int i = 0; i < h->num_pointers; ++i)
+        h->ptr_map.push_back(Handle::PtrSrc{i, 0});
+    for (Handle::PtrSrc &m : h->ptr_map)
+      m.source = m.source == 4 ? 2 : m.source > 4 ? m.source - 1 : m.source;
+    h->caller_pointers = base - 1;
+  }
   if (chan) {
     // The vectors are further caller tensors between the problem's own and the workspace (which closes
     // every multi-kernel problem's list): every kernel of the plan sees the longer list, and the
@@ -227,8 +252,8 @@ Handle *build_handle(const OptMap &o) {
     delete h;
     return nullptr;
   }
-  h->options = o;
-  describe_arguments(o, h);
+  h->options = given;
+  describe_arguments(given, h);
   return h;
 }
 

@@ -119,7 +119,7 @@ def test_null_handle_behaviour(rock):
     "--operation transpose --arch gfx950",
     CONV_IMPLICIT + " --kernel_id 1",
     CONV_RESNET + " --kernel_id 2",
-    "-operation gemm -arch gfx950 -t f16 -g 1 -m 64 -n 64 -k 64 -store-method atomic_add",   # would change the result: refused, not ignored
+    "-operation gemm -arch gfx950 -t f16 -g 1 -m 64 -n 64 -k 64 -store-method atomic_max",   # would change the result: refused, not ignored
     "-operation gemm -arch gfx950 -t fp8 -g 1 -m 64 -n 64 -k 64 -force-f8-types fnuz",
 ])
 def test_bad_problems_give_null(rock, bad):
@@ -962,3 +962,35 @@ def test_attention_where_mask_in_the_caller_list(rock):
     # three-kernel form: the row softmax takes them, the workspace still closes the list
     k = rock.RockKernel(base.replace("f16", "f32") + "-head_dim_qk 64 -head_dim_v 64 -with-attn-mask true -kernel_id 1")
     assert k.kernel_name == "rock_softmax_rows" and k.kernel_count == 3 and k.caller_pointers == 8
+
+
+def test_accumulating_store_is_the_residual_epilogue_on_the_output(rock):
+    """-store-method atomic_add (rocmlir-gen.cpp:295-331): the caller's list stays A, B, C, bias; the kernel's
+    residual pointer is fed from C; plans with a workspace keep it last."""
+    lib = rock.load_library()
+
+    def pointer_map(k):
+        nc, nk = C.c_int(0), C.c_int(0)
+        src, off = (C.c_int32 * 8)(), (C.c_int64 * 8)()
+        assert lib.rockamdGetPointerMap(k._h, C.byref(nc), C.byref(nk), src, off) == 0
+        return nc.value, [src[i] for i in range(nk.value)]
+
+    g = "-operation gemm -arch gfx950 -t f16 -g 1 -m 1024 -n 1024 -k 512 -transB true"
+    k = rock.RockKernel(g + " -store-method atomic_add")
+    assert k.kernel_name == "rock_gemm_f16_64x64_fast_e" and k.kernel_count == 1
+    assert pointer_map(k) == (4, [0, 1, 2, 3, 2]) and len(k.arguments()) == 4
+    assert rock.RockKernel(g + " -store-method set").kernel_name == "rock_gemm_f16_64x64_fast"
+    # few tiles and a long reduction: no split (the sum does not commute with a split's reduction kernel)
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 1 -m 128 -n 1280 -k 5120 -store-method atomic_add")
+    assert k.kernel_count == 1
+    # ragged operands: the copy kernel in front, workspace as the fifth caller pointer
+    ragged = "-operation gemm -arch gfx950 -t f16 -g 1 -m 130 -n 60 -k 77 -store-method atomic_add"
+    plan = [rock.RockKernel(ragged + " -kernel_id %d" % i) for i in range(2)]
+    assert plan[0].kernel_name == "rock_relayout_pair_b2" and pointer_map(plan[0]) == (5, [0, 4, 1, 4])
+    assert pointer_map(plan[1]) == (5, [4, 4, 2, 3, 2])
+    for bad in (g + " -store-method atomic_add -residual add", g + " -store-method atomic_max",
+                "--operation conv --arch gfx950 --in_type fp16 --fil_type fp16 --out_type fp16 --fil_layout gkyxc "
+                "--in_layout nhwgc --out_layout nhwgk --batchsize 1 --in_channels 8 --out_channels 8 --in_h 4 "
+                "--in_w 4 --fil_h 1 --fil_w 1 --store-method atomic_add"):
+        with pytest.raises(rock.RockError):
+            rock.RockKernel(bad)

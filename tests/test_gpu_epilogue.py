@@ -123,6 +123,41 @@ def test_gemm_residual_and_relu_exact(rock, oracle, gpu, kernel, t, od, op):
     assert np.array_equal(to_f32(out, od), oracle.round_through(want.ravel(), CODE[od]))
 
 
+@pytest.mark.parametrize("kernel", KERNELS, ids=lambda k: k[0])
+@pytest.mark.parametrize("t,od", [("f32", "f32"), ("f16", "f16"), ("bf16", "f32"), ("i8", "i32"), ("fp8", "f32")])
+@pytest.mark.parametrize("transC", [False, True], ids=["c", "ct"])
+def test_gemm_accumulating_store_exact(rock, oracle, gpu, kernel, t, od, transC):
+    """-store-method atomic_add (rocmlir-gen.cpp:295-331): C += A B, twice in a row into the same tensor, on
+    every kernel family; integer data keeps every sum exact."""
+    name, (G, M, N, K), tB, pc = kernel
+    rng = np.random.default_rng(65)
+    A, B = _gemm_inputs(rng, t, G, M, N, K, True)
+    rawA, Aq = quantise(A, t)
+    rawB, Bq = quantise(B if tB else np.ascontiguousarray(B.transpose(0, 2, 1)), t)
+    c0 = rng.integers(-5, 6, (G, N, M) if transC else (G, M, N)).astype(np.float32)
+    raw_c, c0q = quantise(c0, od) if od != "i32" else (c0.astype(np.int32), c0)
+    out = to_gpu(raw_c, od, gpu).reshape(c0.shape).clone()
+    info = {}
+    for _ in range(2):
+        got = rock.gemm(to_gpu(rawA, t, gpu), to_gpu(rawB, t, gpu), transB=tB, transC=transC, out_dtype=od, out=out,
+                        accumulate=True, perf_config=pc, info=info, layout_conversion=name != "generic")
+        assert got.data_ptr() == out.data_ptr()
+    torch.cuda.synchronize()
+    assert info["kernel_name"].endswith("_e") or "generic" in info["kernel_name"]
+    acc = oracle.gemm(rawA, rawB, G, M, N, K, False, tB, False) if t == "i8" else \
+        oracle.gemm(Aq, Bq, G, M, N, K, False, tB, False)
+    acc = np.asarray(acc, np.float64).reshape(G, M, N)
+    if transC:
+        acc = acc.transpose(0, 2, 1)
+    if od == "i32":
+        assert np.array_equal(out.cpu().numpy().astype(np.float64), c0.astype(np.float64) + 2.0 * acc)
+        return
+    want = c0q.reshape(c0.shape).astype(np.float32)
+    for _ in range(2):   # each pass: f32 sum of the accumulator and the stored value, rounded to the output type
+        want = oracle.round_through((acc.astype(np.float32) + want).ravel(), CODE[od]).reshape(c0.shape)
+    assert np.array_equal(to_f32(out, od), want.ravel())
+
+
 def test_gemm_clip_exact(rock, oracle, gpu):
     rng = np.random.default_rng(63)
     A, B = _gemm_inputs(rng, "f16", 1, 128, 128, 64, True)
