@@ -3,7 +3,10 @@
 The CPU oracle checks bounded samples (whole rows / output ranges, always
 including tile-boundary rows); size-independent properties check the rest:
 row sums of the full int8 product in exact integer arithmetic, row sums of the
-fp8 product in float64, rows of the softmax summing to one."""
+fp8 product in float64, rows of the softmax summing to one.  The two large
+floating-point configurations are, besides, compared element by element with
+torch's own f32 computation on the same inputs -- a second opinion over the
+rows the oracle's samples do not reach, under the same gates."""
 import numpy as np
 import pytest
 import torch
@@ -13,9 +16,11 @@ from tests.gpu_util import CODE, check_float, quantise, to_f32, to_gpu
 pytestmark = pytest.mark.gpu
 
 
-def _row_ranges(M, tile=256, width=4):
-    """a few whole rows at the start, around tile boundaries and at the end"""
+def _row_ranges(M, tile=256, width=4, extra=0, seed=0):
+    """a few whole rows at the start, around tile boundaries and at the end, and `extra` more ranges drawn at
+    random (seeded) over the whole matrix"""
     picks = [0, tile - width // 2, M // 2 - width // 2, M - tile - width // 2, M - width]
+    picks += [int(p) for p in np.random.default_rng(seed).integers(0, M - width, extra)]
     return [(max(0, p), min(M, max(0, p) + width)) for p in picks]
 
 
@@ -100,9 +105,18 @@ def test_c4_fp8_gemm_8192(rock, oracle, gpu):
     s = float(np.float32(sa * sb))
     out = rock.gemm(to_gpu(rawA, "fp8", gpu), to_gpu(rawB, "fp8", gpu), transB=True, scale=s)
     got = to_f32(out, "f32").reshape(M, N)
-    for r0, r1 in _row_ranges(M, 256, 4):
+    for r0, r1 in _row_ranges(M, 256, 4, extra=27, seed=40):      # 128 of the 8192 rows
         ref = oracle.gemm(Aq, Bq, 1, M, N, K, transB=True, rows=(r0, r1)).reshape(M, N)[r0:r1]
         check_float(got[r0:r1], oracle.scale_bias(ref, r1 - r0, N, s), "f32", rms=3e-5)
+    # every element against torch's f32 product of the same quantised values (in two halves: 2 x 128 MiB)
+    dAq, dBq = torch.from_numpy(Aq).to(gpu), torch.from_numpy(Bq).to(gpu)
+    for half in range(2):
+        rows = slice(half * M // 2, (half + 1) * M // 2)
+        second = (dAq[rows] @ dBq.T) * s
+        diff = (out.reshape(M, N)[rows] - second).double()
+        rms = float(diff.pow(2).mean().sqrt() / (second.abs().max() * 1.0))
+        assert rms <= 3e-5, rms
+        del second, diff
     # every element: row sums in float64 (sum_n C[m,n] = s * A[m,:] . sum_n B[n,:])
     want = (Aq.astype(np.float64) @ Bq.astype(np.float64).sum(axis=0)) * s
     rows = got.astype(np.float64).sum(axis=1)
@@ -120,11 +134,21 @@ def test_c5_f16_attention_2048(rock, oracle, gpu):
     dQ, dK, dV = (to_gpu(x, "f16", gpu) for x in (rq, rk, rv))
     out = rock.attention(dQ, dK, dV, scale=scale, transK=True)
     got = to_f32(out, "f16").reshape(G, S, D)
-    for q0 in (0, 126, 1023, 2044):                 # block starts, boundaries, the tail
+    # block starts, boundaries, the tail, and a dozen seeded positions: 64 of the 2048 query rows of every head
+    starts = [0, 126, 1023, 2044] + [int(x) for x in np.random.default_rng(50).integers(0, S - 4, 12)]
+    for q0 in starts:
         ref = oracle.attention(Qq, Kq, Vq, G, S, S, D, D, scale=scale, transK=True,
                                q_rows=(q0, q0 + 4)).reshape(G, S, D)[:, q0:q0 + 4]
         check_float(got[:, q0:q0 + 4].ravel(), ref.ravel(), "f16", rms=1e-3, max_abs=0.02)
     assert np.isfinite(got).all()
+    # every element against torch's f32 softmax attention on the same f16 values, sixteen heads at a time
+    for g0 in range(0, G, 16):
+        q32, k32, v32 = (x[g0:g0 + 16].float() for x in (dQ, dK, dV))
+        second = torch.softmax((q32 @ k32.transpose(1, 2)) * scale, dim=-1) @ v32
+        diff = (out.reshape(G, S, D)[g0:g0 + 16].float() - second.half().float())
+        assert float(diff.abs().max()) <= 0.02
+        assert float(diff.double().pow(2).mean().sqrt() / second.abs().max()) <= 1e-3
+        del second, diff
     # rows of P sum to one: V = ones gives ones everywhere
     ones = torch.ones_like(dV)
     got1 = to_f32(rock.attention(dQ, dK, ones, scale=scale, transK=True), "f16")
