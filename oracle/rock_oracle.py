@@ -356,6 +356,56 @@ def attention(Q, K, V, G, sq, sk, dqk, dv, scale=1.0, scale_t=None,
     return O
 
 
+def run_attention_program(program, x, inputs):
+    """The pre-softmax region of rock.attention (RockOps.td:208-254) as postfix
+    code over float32 arrays: x = the scores, t<i> = inputs[i], c:<number>,
+    add sub mul div max min, exp neg tanh sigmoid relu abs erf, where
+    (c a b -> c != 0 ? a : b).  Plain numpy, one float32 operation per token."""
+    import math
+    f32 = np.float32
+    stack = []
+    binary = {"add": np.add, "sub": np.subtract, "mul": np.multiply, "div": np.divide,
+              "max": np.maximum, "min": np.minimum}
+    unary = {"exp": np.exp, "neg": np.negative, "tanh": np.tanh,
+             "sigmoid": lambda a: (f32(1) / (f32(1) + np.exp(-a))).astype(f32),
+             "relu": lambda a: np.maximum(a, f32(0)), "abs": np.abs,
+             "erf": lambda a: np.vectorize(math.erf)(a.astype(np.float64)).astype(f32)}
+    for tok in program.replace(" ", "").split(","):
+        if tok == "x":
+            stack.append(np.asarray(x, f32))
+        elif tok[0] == "t" and tok[1:].isdigit():
+            stack.append(np.asarray(inputs[int(tok[1:])], f32).reshape(np.shape(x)))
+        elif tok.startswith("c:"):
+            stack.append(np.full(np.shape(x), f32(float(tok[2:])), f32))
+        elif tok in binary:
+            b, a = stack.pop(), stack.pop()
+            stack.append(binary[tok](a, b).astype(f32))
+        elif tok in unary:
+            stack.append(np.asarray(unary[tok](stack.pop()), f32))
+        elif tok == "where":
+            b, a, c = stack.pop(), stack.pop(), stack.pop()
+            stack.append(np.where(c != 0, a, b).astype(f32))
+        else:
+            raise ValueError("unknown token %r" % tok)
+    assert len(stack) == 1
+    return stack[0]
+
+
+def attention_program(Q, K, V, G, sq, sk, dqk, dv, program, inputs=(), transK=False):
+    """Attention with a pre-softmax program: O = softmax(program(Q K, inputs)) V,
+    float32 throughout in the validator's order of steps (rocmlir-gen.cpp:
+    2565-2620: the first GEMM, the element-wise region, softmax over the keys,
+    the second GEMM); numpy, for sizes a test finishes in seconds.  Q [G,sq,d],
+    K [G,d,sk] ([G,sk,d] with transK), V [G,sk,dv]."""
+    Q = _c(Q, np.float32).reshape(G, sq, dqk)
+    K = _c(K, np.float32).reshape((G, sk, dqk) if transK else (G, dqk, sk))
+    V = _c(V, np.float32).reshape(G, sk, dv)
+    Kt = K.transpose(0, 2, 1) if transK else K
+    S = np.matmul(Q, Kt).astype(np.float32)
+    X = run_attention_program(program, S, inputs)
+    return np.matmul(softmax(X).reshape(G, sq, sk), V).astype(np.float32).ravel()
+
+
 def softmax(x):
     x = _c(x, np.float32)
     y = np.empty_like(x)

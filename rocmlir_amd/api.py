@@ -641,7 +641,7 @@ def conv2d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize,
 
 def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, mask=None, other=None, zero_point=0,
               transQ=False, transK=False, transV=False, transO=False, out=None, stream=None, info=None,
-              score_workspace_limit=None):
+              score_workspace_limit=None, program=None, inputs=()):
     """O = softmax(scale * scale_tensor * Q K + bias) V (bias and scale_tensor
     optional [G,seq_q,seq_k] tensors, rocmlir-gen's -with-attn-bias /
     -with-attn-scale).  `mask` (int8 or bool, [G,seq_q,seq_k]) with `other`
@@ -655,7 +655,12 @@ def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, mask=None, ot
     select the quantised first GEMM: the scores are (acc - zero_point) * scale.
     A dict passed as `info` receives the names of the kernels that ran.
     `score_workspace_limit` (bytes) bounds the score chunk of the three-kernel
-    form (f32, head dimensions above 256); the default is 32 MiB."""
+    form (f32, head dimensions above 256); the default is 32 MiB.
+    `program` is a pre-softmax element-wise tree in postfix form over the score
+    `x`, the tensors `inputs` (`t0`, `t1`, ...; each [G,seq_q,seq_k], any of
+    f32 / f16 / bf16 / int8) and constants `c:<number>`, e.g.
+    "x,t0,mul,exp,t1,add" (the region of rock.attention, RockOps.td:208-254);
+    it replaces scale, bias, scale_tensor and mask."""
     import torch
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     G = q.shape[0]
@@ -684,6 +689,12 @@ def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, mask=None, ot
         mask = mask.to(torch.int8).contiguous()
     if score_workspace_limit is not None:
         opts += " -score_workspace_limit %d" % score_workspace_limit
+    if program:
+        if bias is not None or scale_tensor is not None or mask is not None or scale != 1.0:
+            raise RockError("attention: a program replaces scale, bias, scale_tensor and mask")
+        opts += " -attn_elementwise %s" % program.replace(" ", "")
+        if inputs:
+            opts += " -attn_inputs %s" % ",".join(_dtype_name(t.dtype) for t in inputs)
     kern = _program(opts)   # one fused kernel, or three for head dimensions above 128 and f32
     if info is not None:
         info["kernels"] = [k.kernel_name for k in kern.kernels]
@@ -693,6 +704,8 @@ def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, mask=None, ot
     pre = ([] if scale_tensor is None else [scale_tensor.contiguous()]) + [bias]
     if mask is not None:
         pre += [mask, other.contiguous()]
+    if program:
+        pre = [t.contiguous() for t in inputs]
     kern.launch(q, k, v, *pre, out, stream=stream)
     return out
 

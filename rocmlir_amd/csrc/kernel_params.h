@@ -223,6 +223,17 @@ struct RockFoldDepthParams {
   int32_t pad_;
 };
 
+#define ROCK_ATTN_PROGRAM_MAX 24
+#define ROCK_ATTN_PROGRAM_INPUTS 8
+enum RockAttnOp : int32_t {
+  ROCK_AOP_SCORE = 1,  // push the score
+  ROCK_AOP_TENSOR = 2, // push element [g, i, j] of input tensor `argument`
+  ROCK_AOP_CONST = 3,  // push consts[argument]
+  ROCK_AOP_ADD = 10, ROCK_AOP_SUB, ROCK_AOP_MUL, ROCK_AOP_DIV, ROCK_AOP_MAX, ROCK_AOP_MIN, // a b -> a op b
+  ROCK_AOP_EXP = 20, ROCK_AOP_NEG, ROCK_AOP_TANH, ROCK_AOP_SIGMOID, ROCK_AOP_RELU, ROCK_AOP_ABS, ROCK_AOP_ERF,
+  ROCK_AOP_WHERE = 30, // c a b -> c != 0 ? a : b
+};
+
 // rock_softmax_rows(S, scale_tensor, bias, p): the middle kernel of attention
 // run as three kernels (head dimensions beyond the fused kernel's, f32).  S
 // holds G*seq_q rows of seq_k f32 scores, `row_pitch` floats apart; row by row
@@ -237,6 +248,16 @@ struct RockSoftmaxParams {
   int32_t has_bias, has_scale_tensor;
   int32_t dtype; // RockDType of P, the scale tensor and the bias: f32, f16 or bf16
   int32_t has_mask; // where(mask, score, other): an int8 mask and a tensor of `dtype`, both [g, i, j] like the bias
+  // A pre-softmax element-wise program (the body of rock.attention's preSoftmaxBody region, RockOps.td:208-254,
+  // which may hold any element-wise tree over the scores and further [g, i, j] tensors): postfix code for a
+  // four-deep stack machine, run per score in f32.  prog_len = 0: the fixed chain above.
+  int32_t prog_len;
+  int32_t pad_;
+  int32_t prog[ROCK_ATTN_PROGRAM_MAX]; // RockAttnOp | argument << 8
+  float consts[ROCK_ATTN_PROGRAM_INPUTS];
+  int32_t tensor_dtype[ROCK_ATTN_PROGRAM_INPUTS];      // RockDType of each input tensor (f32, f16, bf16, i8)
+  const void *tensors[ROCK_ATTN_PROGRAM_INPUTS];       // written at launch from the caller's pointer list
+  int64_t t_base;                                      // elements from the tensors' starts to this launch's first row
 };
 
 struct RockAttentionParams {

@@ -24,6 +24,119 @@ bool parse_attn_perf(const std::string &pc, int &dmax, int &kpack_pb, int &force
   return true;
 }
 
+// "-attn_elementwise x,t0,mul,exp,t1,add" with "-attn_inputs f32,f32": the pre-softmax region of rock.attention
+// as postfix code (RockOps.td:208-254: any element-wise tree over the scores and further [G, seq_q, seq_k]
+// tensors; mixr-attention-padded-scale-bias-exp.mlir and ...-complex-tree-elemwise.mlir are two).  Tokens: x (the
+// score), t<i> (input tensor i), c:<number>, add sub mul div max min (a b -> a op b), exp neg tanh sigmoid relu
+// abs erf, where (c a b -> c != 0 ? a : b).  Such a problem runs as GEMM, row softmax (which interprets the
+// program), GEMM; the fixed chain -with-attn-scale / -scale / -with-attn-bias / -with-attn-mask stays on the
+// fused kernels.
+struct AttnProgram {
+  std::vector<int32_t> code;
+  std::vector<float> consts;
+  std::vector<int> input_types; // RockDType per input tensor
+};
+
+bool parse_attention_program(const OptMap &o, int default_type, AttnProgram &prog) {
+  const std::string text = str_or(o, "attn_elementwise", "");
+  if (text.empty())
+    return true;
+  auto split = [](const std::string &t) {
+    std::vector<std::string> out;
+    std::string cur;
+    for (char ch : t) {
+      if (ch == ',') {
+        out.push_back(cur);
+        cur.clear();
+      } else {
+        cur += ch;
+      }
+    }
+    out.push_back(cur);
+    return out;
+  };
+  static const std::pair<const char *, int> kOps[] = {
+      {"add", ROCK_AOP_ADD}, {"sub", ROCK_AOP_SUB}, {"mul", ROCK_AOP_MUL}, {"div", ROCK_AOP_DIV},
+      {"max", ROCK_AOP_MAX}, {"min", ROCK_AOP_MIN}, {"exp", ROCK_AOP_EXP}, {"neg", ROCK_AOP_NEG},
+      {"tanh", ROCK_AOP_TANH}, {"sigmoid", ROCK_AOP_SIGMOID}, {"relu", ROCK_AOP_RELU}, {"abs", ROCK_AOP_ABS},
+      {"erf", ROCK_AOP_ERF}, {"where", ROCK_AOP_WHERE}};
+  int depth = 0, inputs_used = 0;
+  for (const std::string &tok : split(text)) {
+    int op = 0, arg = 0;
+    if (tok == "x") {
+      op = ROCK_AOP_SCORE;
+    } else if (tok.size() >= 2 && tok[0] == 't' && std::isdigit((unsigned char)tok[1])) {
+      op = ROCK_AOP_TENSOR;
+      arg = std::atoi(tok.c_str() + 1);
+      if (arg >= ROCK_ATTN_PROGRAM_INPUTS) {
+        set_error("attention: at most 8 pre-softmax input tensors");
+        return false;
+      }
+      inputs_used = std::max(inputs_used, arg + 1);
+    } else if (tok.rfind("c:", 0) == 0) {
+      char *end = nullptr;
+      const float v = std::strtof(tok.c_str() + 2, &end);
+      if (end == tok.c_str() + 2 || *end || prog.consts.size() == ROCK_ATTN_PROGRAM_INPUTS) {
+        set_error("attention: bad or too many constants in the pre-softmax program ('" + tok + "')");
+        return false;
+      }
+      op = ROCK_AOP_CONST;
+      arg = (int)prog.consts.size();
+      prog.consts.push_back(v);
+    } else {
+      for (const auto &k : kOps)
+        if (tok == k.first)
+          op = k.second;
+      if (!op) {
+        set_error("attention: unknown token '" + tok + "' in the pre-softmax program");
+        return false;
+      }
+    }
+    const int pops = op <= ROCK_AOP_CONST ? 0 : op < ROCK_AOP_EXP ? 2 : op < ROCK_AOP_WHERE ? 1 : 3;
+    if (depth < pops) {
+      set_error("attention: the pre-softmax program pops an empty stack at '" + tok + "'");
+      return false;
+    }
+    depth += 1 - pops;
+    if (depth > 4 || prog.code.size() == ROCK_ATTN_PROGRAM_MAX) {
+      set_error("attention: the pre-softmax program is longer than 24 steps or deeper than 4 values");
+      return false;
+    }
+    prog.code.push_back(op | (arg << 8));
+  }
+  if (depth != 1) {
+    set_error("attention: the pre-softmax program must leave exactly one value");
+    return false;
+  }
+  const std::string types = str_or(o, "attn_inputs", "");
+  if (!types.empty())
+    for (const std::string &t : split(types)) {
+      const int ty = parse_dtype(t);
+      if (ty != ROCK_F32 && ty != ROCK_F16 && ty != ROCK_BF16 && ty != ROCK_I8) {
+        set_error("attention: pre-softmax input tensors are f32, f16, bf16 or i8 ('" + t + "')");
+        return false;
+      }
+      prog.input_types.push_back(ty);
+    }
+  if ((int)prog.input_types.size() < inputs_used) {
+    if (!types.empty()) {
+      set_error("attention: the pre-softmax program reads more tensors than -attn_inputs lists");
+      return false;
+    }
+    prog.input_types.assign(inputs_used, default_type);
+  }
+  if (bool_or(o, "with-attn-scale", false) || bool_or(o, "with-attn-bias", false) || bool_or(o, "with-attn-mask", false)) {
+    set_error("attention: -attn_elementwise replaces -with-attn-scale / -with-attn-bias / -with-attn-mask");
+    return false;
+  }
+  float scale = 1.0f;
+  if (get_float(o, "scale", scale) && scale != 1.0f) {
+    set_error("attention: with -attn_elementwise the scale is a constant of the program (c:<value>), not -scale");
+    return false;
+  }
+  return true;
+}
+
 // Attention outside the fused kernel's reach (head dimensions above 256, f32):
 // three kernels over a workspace of f32 scores -- the GEMM Q K^T, a row softmax
 // that applies scale tensor, scale, bias and mask and narrows the probabilities
@@ -42,7 +155,8 @@ bool parse_attn_perf(const std::string &pc, int &dmax, int &kpack_pb, int &force
 constexpr int64_t kScoreWholeBytes = ROCKAMD_STATIC_WORKSPACE_BYTES - ((int64_t)16 << 20); // room for the partial sums
 constexpr int64_t kScoreChunkBytes = (int64_t)32 << 20;
 Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, int64_t sk, int64_t dqk, int64_t dv,
-                               bool tQ, bool tK, bool tV, bool tO, bool has_bias, bool has_scale_t, bool has_mask) {
+                               bool tQ, bool tK, bool tV, bool tO, bool has_bias, bool has_scale_t, bool has_mask,
+                               const AttnProgram &prog = AttnProgram()) {
   // "-t i8": Q and K are int8, their product is dequantised before the softmax
   // ((acc - zero_point) * scale, the scalars rocmlir-gen passes as [1,1,1]
   // tensors, rocmlir-gen.cpp:2173-2184, 2353-2367); V, the pre-softmax tensors
@@ -92,9 +206,12 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
   const int64_t gn = std::min(gc, G - g0), rn = std::min(rc, sq - r0); // this chunk
   float scale = 1.0f;
   get_float(o, "scale", scale);
-  // caller list: Q, K, V, [scale tensor], bias slot, [mask, other], O, workspace
+  // caller list: Q, K, V, [scale tensor], bias slot, [mask, other], O, workspace;
+  // with a pre-softmax program: Q, K, V, the program's input tensors, O, workspace
+  const bool programmed = !prog.code.empty();
+  const int n_in = (int)prog.input_types.size();
   const int i_bias = has_scale_t ? 4 : 3, i_mask = has_mask ? i_bias + 1 : -1, i_other = has_mask ? i_bias + 2 : -1,
-            i_out = i_bias + 1 + (has_mask ? 2 : 0), i_ws = i_out + 1;
+            i_out = programmed ? 3 + n_in : i_bias + 1 + (has_mask ? 2 : 0), i_ws = i_out + 1;
   const int64_t pitch_p = 4 / es; // elements of P per f32 score: P lies in place, rows sk * 4 bytes apart
   auto *h = new Handle;
   if (kid == 1) {
@@ -108,6 +225,11 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
     r.has_scale_tensor = has_scale_t ? 1 : 0;
     r.has_mask = has_mask ? 1 : 0;
     r.dtype = ty;
+    r.prog_len = (int)prog.code.size();
+    std::copy(prog.code.begin(), prog.code.end(), r.prog);
+    std::copy(prog.consts.begin(), prog.consts.end(), r.consts);
+    std::copy(prog.input_types.begin(), prog.input_types.end(), r.tensor_dtype);
+    r.t_base = g0 * sq * sk + r0 * sk; // the chunk's first row in the program's [G, seq_q, seq_k] tensors
     h->op = OP_RELAYOUT;
     h->epi = nullptr;
     h->params.assign(sizeof r, 0);
@@ -118,8 +240,14 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
     h->num_pointers = 5;
     h->perf_config = "";
     const int64_t t_off = (g0 * sq * sk + r0 * sk) * es; // the chunk's first row in the [G, seq_q, seq_k] tensors
-    h->ptr_map = {{i_ws, 0}, {has_scale_t ? 3 : -1, t_off}, {has_bias ? i_bias : -1, t_off}, {i_mask, t_off / es},
-                  {i_other, t_off}};
+    if (programmed) {
+      h->ptr_map = {{i_ws, 0}, {-1, 0}, {-1, 0}, {-1, 0}, {-1, 0}};
+      for (int i = 0; i < n_in; ++i) // their pointers ride in the parameter block
+        h->param_ptrs.push_back({(int)(offsetof(RockSoftmaxParams, tensors) + i * sizeof(void *)), 3 + i});
+    } else {
+      h->ptr_map = {{i_ws, 0}, {has_scale_t ? 3 : -1, t_off}, {has_bias ? i_bias : -1, t_off}, {i_mask, t_off / es},
+                    {i_other, t_off}};
+    }
     h->problem_key = "row softmax of the attention scores";
   } else if (kid == 3) { // O = the sum of the shares' partial results
     RockReduceParams r;
@@ -221,6 +349,11 @@ Handle *make_attention(const OptMap &o) {
   // an int8 mask and a tensor of replacement scores, both [G, seq_q, seq_k], behind the bias in the caller's list.
   // Where the mask is zero the score (after scale tensor, scale and bias) is replaced, not added to.
   const bool has_mask = bool_or(o, "with-attn-mask", false);
+  AttnProgram prog;
+  if (!parse_attention_program(o, ty == ROCK_I8 ? ROCK_F16 : ty, prog))
+    return nullptr;
+  if (!prog.code.empty())
+    return make_attention_unfused(o, ty, G, sq, sk, dqk, dv, tQ, tK, tV, tO, false, false, false, prog);
   // "-t i8": int8 Q and K (the quantised first GEMM), f16 V, pre-softmax tensors and O
   const bool qk_i8 = ty == ROCK_I8;
   // Transposed Q, V or O ([G, d, seq_q], [G, dv, seq_k], [G, dv, seq_q]): the fused vector kernels want the

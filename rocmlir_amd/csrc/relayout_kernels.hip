@@ -131,7 +131,46 @@ __device__ __forceinline__ float load_as_f32(const void *base, int64_t idx, int 
     return ((const float *)base)[idx];
   if (dtype == ROCK_F16)
     return (float)((const _Float16 *)base)[idx];
+  if (dtype == ROCK_I8)
+    return (float)((const int8_t *)base)[idx];
   return __builtin_bit_cast(float, (uint32_t)((const uint16_t *)base)[idx] << 16);
+}
+
+// The pre-softmax program of a score: postfix code over a stack of four floats whose top is always s0 (pushes
+// and pops shift the other three, so no stack slot is ever addressed with a run-time index).
+__device__ __forceinline__ float run_attention_program(const RockSoftmaxParams &p, float x, int64_t at) {
+  float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+  for (int i = 0; i < p.prog_len; ++i) {
+    const int op = p.prog[i] & 255, arg = p.prog[i] >> 8;
+    if (op <= ROCK_AOP_CONST) {
+      const float v = op == ROCK_AOP_SCORE    ? x
+                      : op == ROCK_AOP_TENSOR ? load_as_f32(p.tensors[arg], p.t_base + at, p.tensor_dtype[arg])
+                                              : p.consts[arg];
+      s3 = s2; s2 = s1; s1 = s0; s0 = v;
+    } else if (op < ROCK_AOP_EXP) {
+      const float a = s1, b = s0;
+      const float r = op == ROCK_AOP_ADD   ? a + b
+                      : op == ROCK_AOP_SUB ? a - b
+                      : op == ROCK_AOP_MUL ? a * b
+                      : op == ROCK_AOP_DIV ? a / b
+                      : op == ROCK_AOP_MAX ? fmaxf(a, b)
+                                           : fminf(a, b);
+      s0 = r; s1 = s2; s2 = s3;
+    } else if (op < ROCK_AOP_WHERE) {
+      const float a = s0;
+      s0 = op == ROCK_AOP_EXP       ? expf(a)
+           : op == ROCK_AOP_NEG     ? -a
+           : op == ROCK_AOP_TANH    ? tanhf(a)
+           : op == ROCK_AOP_SIGMOID ? 1.0f / (1.0f + expf(-a))
+           : op == ROCK_AOP_RELU    ? fmaxf(a, 0.0f)
+           : op == ROCK_AOP_ABS     ? fabsf(a)
+                                    : erff(a);
+    } else {
+      s0 = s2 != 0.0f ? s1 : s0;
+      s1 = s3;
+    }
+  }
+  return s0;
 }
 
 // over the block's waves (at most 16); scratch holds one float per wave
@@ -168,6 +207,8 @@ struct SoftmaxRow {
   const RockSoftmaxParams &p;
   __device__ __forceinline__ float score(int j) const {
     float x = s[j];
+    if (p.prog_len)
+      return run_attention_program(p, x, t_off + (int64_t)j * p.t_js);
     if (p.has_scale_tensor)
       x = x * load_as_f32(scale_t, t_off + (int64_t)j * p.t_js, p.dtype);
     x = x * p.scale;
@@ -277,9 +318,10 @@ extern "C" __global__ __launch_bounds__(1024) void rock_softmax_rows(float *S, c
   const int64_t r = blockIdx.x;
   const int g = (int)(r / p.seq_q), i = (int)(r - (int64_t)g * p.seq_q);
   const SoftmaxRow row{S + r * p.row_pitch, scale_t, bias, mask, other, (int64_t)g * p.t_gs + (int64_t)i * p.t_is, p};
-  if (p.dtype == ROCK_F32 ? softmax_short_row<float>(row, scratch)
-      : p.dtype == ROCK_F16 ? softmax_short_row<_Float16>(row, scratch)
-                            : softmax_short_row<__bf16>(row, scratch))
+  // (a program runs on the three-pass path below: its loads and branches do not fit the register-resident form)
+  if (p.prog_len == 0 && (p.dtype == ROCK_F32   ? softmax_short_row<float>(row, scratch)
+                          : p.dtype == ROCK_F16 ? softmax_short_row<_Float16>(row, scratch)
+                                                : softmax_short_row<__bf16>(row, scratch)))
     return;
   const int nt = (int)blockDim.x, tid = (int)threadIdx.x;
   float m = -INFINITY;

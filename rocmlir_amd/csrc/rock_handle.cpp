@@ -51,12 +51,31 @@ void describe_arguments(const OptMap &o, Handle *h) {
     auto mat = [&](bool tr, int64_t r, int64_t c) { return tr ? std::vector<int64_t>{G, c, r} : std::vector<int64_t>{G, r, c}; };
     h->args = {A{t, mat(bool_or(o, "transQ", false), sq, dqk)}, A{t, mat(!bool_or(o, "transK", false), sk, dqk)},
                A{tv, mat(bool_or(o, "transV", false), sk, dv)}};
-    if (bool_or(o, "with-attn-scale", false))
-      h->args.push_back(A{tv, {G, sq, sk}});
-    h->args.push_back(A{tv, {G, sq, sk}}); // bias slot
-    if (bool_or(o, "with-attn-mask", false)) {
-      h->args.push_back(A{ROCK_I8, {G, sq, sk}});
-      h->args.push_back(A{tv, {G, sq, sk}});
+    if (!str_or(o, "attn_elementwise", "").empty()) {
+      // the program's input tensors (their number: what the plan put into the caller's list between V and O)
+      const int total = h->caller_pointers ? h->caller_pointers : h->num_pointers;
+      const int n_in = total - 5; // Q, K, V, O, workspace
+      std::vector<int> types;
+      std::string cur;
+      for (char ch : str_or(o, "attn_inputs", "") + ",") {
+        if (ch == ',') {
+          if (!cur.empty())
+            types.push_back(parse_dtype(cur));
+          cur.clear();
+        } else {
+          cur += ch;
+        }
+      }
+      for (int i = 0; i < n_in; ++i)
+        h->args.push_back(A{i < (int)types.size() ? types[i] : tv, {G, sq, sk}});
+    } else {
+      if (bool_or(o, "with-attn-scale", false))
+        h->args.push_back(A{tv, {G, sq, sk}});
+      h->args.push_back(A{tv, {G, sq, sk}}); // bias slot
+      if (bool_or(o, "with-attn-mask", false)) {
+        h->args.push_back(A{ROCK_I8, {G, sq, sk}});
+        h->args.push_back(A{tv, {G, sq, sk}});
+      }
     }
     h->args.push_back(A{tv, mat(bool_or(o, "transO", false), sq, dv)});
     with_workspace();

@@ -19,6 +19,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
+#include <cctype>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>

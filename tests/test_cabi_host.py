@@ -994,3 +994,31 @@ def test_accumulating_store_is_the_residual_epilogue_on_the_output(rock):
                 "--in_w 4 --fil_h 1 --fil_w 1 --store-method atomic_add"):
         with pytest.raises(rock.RockError):
             rock.RockKernel(bad)
+
+
+def test_attention_pre_softmax_program(rock):
+    """-attn_elementwise: the pre-softmax region of rock.attention as postfix code (RockOps.td:208-254; the trees
+    of mixr-attention-padded-scale-bias-exp.mlir and ...-complex-tree-elemwise.mlir).  Such a problem runs as GEMM,
+    row softmax, GEMM; the program's tensors stand between V and O in the caller's list and reach the softmax
+    kernel through pointer fields of its parameter block."""
+    lib = rock.load_library()
+    base = "-operation attention -arch gfx950 -t f32 -g 1 -seq_len_q 7 -seq_len_k 7 -head_dim_qk 3 -head_dim_v 3 "
+    ks = [rock.RockKernel(base + "-attn_elementwise x,t0,mul,exp,t1,add -kernel_id %d" % i) for i in range(3)]
+    assert [k.kernel_name.split("_")[1] for k in ks] == ["gemm", "softmax", "gemm"]
+    assert all(k.kernel_count == 3 and k.caller_pointers == 7 for k in ks)      # Q K V t0 t1 O workspace
+    assert [a[1] for a in ks[0].arguments()[3:5]] == [[1, 7, 7], [1, 7, 7]]
+    n, off, src = C.c_int(0), (C.c_int32 * 8)(), (C.c_int32 * 8)()
+    assert lib.rockamdGetParamPointers(ks[1]._h, C.byref(n), off, src) == 0
+    assert n.value == 2 and [src[i] for i in range(2)] == [3, 4] and off[1] - off[0] == 8
+    assert lib.rockamdGetParamPointers(ks[0]._h, C.byref(n), off, src) == 0 and n.value == 0
+    # f16 problems with a program leave the fused kernels; input types as listed, an int8 mask among them
+    f16 = base.replace("-t f32", "-t f16").replace("-seq_len_q 7 -seq_len_k 7 -head_dim_qk 3 -head_dim_v 3",
+                                                   "-seq_len_q 256 -seq_len_k 256 -head_dim_qk 64 -head_dim_v 64 -transK true")
+    k = rock.RockKernel(f16 + "-attn_elementwise t0,x,c:0.125,mul,t1,where -attn_inputs i8,f16")
+    assert k.kernel_count == 3 and [a[0] for a in k.arguments()[3:5]] == [3, 1]
+    assert rock.RockKernel(f16).kernel_name == "rock_attention_f16_d64x64_fast"
+    for bad in ("x,add", "x,x", "x,t9,add", "x,frobnicate", "x,c:abc,mul", "x,t0,t1,t2,t3,add,add,add,add,t4",
+                "x,t0,mul -attn_inputs f16,fp8", "x,t0,t1,add,mul -attn_inputs f16", "x,t0,mul -with-attn-bias true",
+                "x,t0,mul -scale 0.5"):
+        with pytest.raises(rock.RockError):
+            rock.RockKernel(f16 + "-attn_elementwise " + bad)

@@ -241,6 +241,47 @@ def test_attention_three_kernel_form_in_chunks(rock, oracle, gpu, case):
     check_float(got, ref, t, rms=gate[0], max_abs=gate[1])
 
 
+@pytest.mark.parametrize("case", [
+    # the reference's two trees at their own shape (mixr-attention-padded-scale-bias-exp.mlir:5-16,
+    # mixr-attention-padded-complex-tree-elemwise.mlir:5-24: f32, 7 x 7 scores, head dimension 3, K [G, d, seq_k])
+    dict(id="exp-tree-7x7", t="f32", shape=(1, 7, 7, 3, 3), program="x,t0,mul,exp,t1,add", n_in=2),
+    dict(id="complex-tree-7x7", t="f32", shape=(1, 7, 7, 3, 3), program="x,t0,t1,sub,mul,t2,t3,add,add", n_in=4),
+    dict(id="exp-tree-f16", t="f16", shape=(3, 130, 200, 64, 72), program="x,t0,mul,exp,t1,add", n_in=2),
+    dict(id="complex-tree-bf16", t="bf16", shape=(2, 100, 333, 40, 128), program="x,t0,t1,sub,mul,t2,t3,add,add", n_in=4),
+    dict(id="mask-tanh-chunks", t="f16", shape=(2, 200, 136, 64, 64), program="t0,x,c:0.125,mul,tanh,c:5,mul,t1,where",
+         n_in=2, mask_first=True, limit=60 << 10, kernels=12),
+    dict(id="long-rows-f32", t="f32", shape=(1, 40, 4500, 32, 32), program="x,c:0.2,mul,t0,max,sigmoid,neg", n_in=1),
+], ids=lambda c: c["id"])
+def test_attention_pre_softmax_program(rock, oracle, gpu, case):
+    """-attn_elementwise: an element-wise tree over the scores and further [G, seq_q, seq_k] tensors in front of
+    the softmax (the region of rock.attention, RockOps.td:208-254), interpreted by the row softmax of the
+    three-kernel form; against the numpy restatement, itself pinned by torch in float64."""
+    t = case["t"]
+    G, sq, sk, dqk, dv = case["shape"]
+    rng = np.random.default_rng(73)
+    rq, Qq = quantise(rng.standard_normal((G, sq, dqk)).astype(np.float32), t)
+    rk, Kq = quantise(rng.standard_normal((G, dqk, sk)).astype(np.float32), t)      # the default storage of K
+    rv, Vq = quantise(rng.standard_normal((G, sk, dv)).astype(np.float32), t)
+    dev_in, ref_in = [], []
+    for i in range(case["n_in"]):
+        if i == 0 and case.get("mask_first"):
+            m = (rng.random((G, sq, sk)) < 0.7).astype(np.int8)
+            dev_in.append(torch.from_numpy(m).to(gpu))
+            ref_in.append(m)
+        else:
+            raw, val = quantise((rng.standard_normal((G, sq, sk)) * 0.4).astype(np.float32), t)
+            dev_in.append(to_gpu(raw, t, gpu).reshape(G, sq, sk))
+            ref_in.append(val)
+    info = {}
+    out = rock.attention(to_gpu(rq, t, gpu), to_gpu(rk, t, gpu), to_gpu(rv, t, gpu), program=case["program"],
+                         inputs=dev_in, info=info, score_workspace_limit=case.get("limit"))
+    torch.cuda.synchronize()
+    assert len(info["kernels"]) == case.get("kernels", 3) and "rock_softmax_rows" in info["kernels"]
+    ref = oracle.attention_program(Qq, Kq, Vq, G, sq, sk, dqk, dv, case["program"], ref_in)
+    gate = {"f16": GATE["f16"], "bf16": GATE["bf16"], "f32": (3e-5, 1e-4)}[t]
+    check_float(to_f32(out, t), ref, t, rms=gate[0], max_abs=gate[1])
+
+
 def test_attention_three_kernel_form_with_bias_and_scale_tensor(rock, oracle, gpu):
     got, ref = _run(rock, oracle, gpu, "f16", 2, 100, 150, 320, 192, 0.07, 53, bias=True, scale_tensor=True)
     check_float(got, ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])

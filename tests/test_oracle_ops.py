@@ -401,6 +401,49 @@ def test_attention_where_mask_vs_float64(oracle):
     assert np.allclose(att(scale=0.3, mask=np.zeros_like(mask), other=other), only_other, rtol=0, atol=3e-6)
 
 
+def test_attention_program_vs_float64_and_the_fixed_chain(oracle):
+    """The pre-softmax region as postfix code (RockOps.td:208-254).  The reference's two trees -- (x * t0) -> exp
+    -> + t1 (mixr-attention-padded-scale-bias-exp.mlir:12-15) and x * (t0 - t1) + (t2 + t3)
+    (...-complex-tree-elemwise.mlir:17-23), at their 7 x 7 x 3 shape and a larger one -- against torch in float64
+    written out operation by operation; the programs that spell the fixed chain (scale tensor, scale, bias, where)
+    against the C oracle, which takes those as arguments; operand order of the non-commutative tokens by hand."""
+    rng = np.random.default_rng(35)
+    for G, sq, sk, d, dv in ((1, 7, 7, 3, 3), (2, 9, 21, 8, 5)):
+        Q = rng.standard_normal((G, sq, d)).astype(np.float32)
+        K = rng.standard_normal((G, d, sk)).astype(np.float32)
+        V = rng.standard_normal((G, sk, dv)).astype(np.float32)
+        t = [rng.standard_normal((G, sq, sk)).astype(np.float32) * 0.5 for _ in range(4)]
+        q64, k64, v64 = (torch.from_numpy(a.astype(np.float64)) for a in (Q, K, V))
+        t64 = [torch.from_numpy(a.astype(np.float64)) for a in t]
+        s64 = q64 @ k64
+        want = torch.softmax(torch.exp(s64 * t64[0]) + t64[1], dim=-1) @ v64
+        got = oracle.attention_program(Q, K, V, G, sq, sk, d, dv, "x,t0,mul,exp,t1,add", t[:2])
+        assert np.allclose(got.reshape(G, sq, dv), want.numpy(), rtol=0, atol=5e-6)
+        want = torch.softmax(s64 * (t64[0] - t64[1]) + (t64[2] + t64[3]), dim=-1) @ v64
+        got = oracle.attention_program(Q, K, V, G, sq, sk, d, dv, "x,t0,t1,sub,mul,t2,t3,add,add", t)
+        assert np.allclose(got.reshape(G, sq, dv), want.numpy(), rtol=0, atol=5e-6)
+        # the fixed chain, spelt as programs, against the C oracle's arguments (K stored [G, sk, d] there)
+        Kt = np.ascontiguousarray(K.transpose(0, 2, 1))
+        mask = (rng.random((G, sq, sk)) < 0.5).astype(np.int8)
+        ref = oracle.attention(Q, Kt, V, G, sq, sk, d, dv, scale=0.3, scale_t=t[0], bias_t=t[1], transK=True)
+        got = oracle.attention_program(Q, K, V, G, sq, sk, d, dv, "x,t0,mul,c:0.3,mul,t1,add", t[:2])
+        assert np.allclose(got, ref, rtol=0, atol=2e-6)
+        ref = oracle.attention(Q, Kt, V, G, sq, sk, d, dv, scale=0.3, mask=mask, other=t[2], transK=True)
+        got = oracle.attention_program(Q, K, V, G, sq, sk, d, dv, "t0,x,c:0.3,mul,t1,where", [mask, t[2]])
+        assert np.allclose(got, ref, rtol=0, atol=2e-6)
+    # operand order: a b sub = a - b, a b div = a / b, c a b where = c ? a : b; unary tokens by their values
+    x = np.array([[4.0, -2.0]], np.float32)
+    run = lambda prog, *ins: oracle.run_attention_program(prog, x, ins).tolist()
+    assert run("x,c:1,sub") == [[3.0, -3.0]] and run("c:1,x,sub") == [[-3.0, 3.0]]
+    assert run("x,c:2,div") == [[2.0, -1.0]] and run("c:8,x,div") == [[2.0, -4.0]]
+    assert run("x,c:10,c:20,where") == [[10.0, 10.0]] and run("t0,c:10,c:20,where", np.array([[0, 1]], np.int8)) == [[20.0, 10.0]]
+    assert run("x,relu") == [[4.0, 0.0]] and run("x,neg,abs") == [[4.0, 2.0]]
+    assert run("x,c:0,max,x,c:0,min,add") == [[4.0, -2.0]]
+    assert np.allclose(run("x,sigmoid"), [[1 / (1 + np.exp(-4.0)), 1 / (1 + np.exp(2.0))]], atol=1e-7)
+    assert np.allclose(run("x,c:4,div,tanh"), np.tanh([[1.0, -0.5]]), atol=1e-7)
+    assert np.allclose(run("x,c:4,div,erf"), [[0.8427007929, -0.5204998778]], atol=1e-7)
+
+
 def test_attention_invariants(oracle):
     rng = np.random.default_rng(21)
     G, sq, sk, d, dv = 1, 4, 16, 8, 6
