@@ -204,10 +204,11 @@ def conv_fwd(fil, inp, fil_layout, in_layout, out_layout, n, g, c, k, hi, wi,
 
 
 def conv_bwd_data(fil, out, fil_layout, in_layout, out_layout, n, g, c, k, hi,
-                  wi, y, x, stride=(1, 1), pad=(0, 0), dil=(1, 1), threads=0):
+                  wi, y, x, stride=(1, 1), pad=(0, 0), dil=(1, 1), threads=0, pad_r=None):
     """Gradient with respect to the input: (flat input-shaped array, ho, wo)."""
-    ho = conv_out_dim(hi, y, pad[0], pad[0], stride[0], dil[0])
-    wo = conv_out_dim(wi, x, pad[1], pad[1], stride[1], dil[1])
+    pad_r = pad if pad_r is None else pad_r   # bottom / right padding: it only sets the output's extent
+    ho = conv_out_dim(hi, y, pad[0], pad_r[0], stride[0], dil[0])
+    wo = conv_out_dim(wi, x, pad[1], pad_r[1], stride[1], dil[1])
     d = ConvDims(n, g, c, k, hi, wi, y, x, ho, wo, stride[0], stride[1],
                  pad[0], pad[1], dil[0], dil[1])
     fil, out = _c(fil, np.float32), _c(out, np.float32)
@@ -221,10 +222,11 @@ def conv_bwd_data(fil, out, fil_layout, in_layout, out_layout, n, g, c, k, hi,
 
 
 def conv_bwd_weight(inp, out, fil_layout, in_layout, out_layout, n, g, c, k, hi,
-                    wi, y, x, stride=(1, 1), pad=(0, 0), dil=(1, 1), threads=0):
+                    wi, y, x, stride=(1, 1), pad=(0, 0), dil=(1, 1), threads=0, pad_r=None):
     """Gradient with respect to the filter: (flat filter-shaped array, ho, wo)."""
-    ho = conv_out_dim(hi, y, pad[0], pad[0], stride[0], dil[0])
-    wo = conv_out_dim(wi, x, pad[1], pad[1], stride[1], dil[1])
+    pad_r = pad if pad_r is None else pad_r
+    ho = conv_out_dim(hi, y, pad[0], pad_r[0], stride[0], dil[0])
+    wo = conv_out_dim(wi, x, pad[1], pad_r[1], stride[1], dil[1])
     d = ConvDims(n, g, c, k, hi, wi, y, x, ho, wo, stride[0], stride[1],
                  pad[0], pad[1], dil[0], dil[1])
     inp, out = _c(inp, np.float32), _c(out, np.float32)

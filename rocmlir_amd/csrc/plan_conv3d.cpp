@@ -117,7 +117,7 @@ bool parse_conv3d(const OptMap &o, Conv3dProblem &P, bool backward) {
       set_error("conv: out_h/out_w/out_d do not match the value computed from the other parameters");
       return false;
     }
-    if (backward && P.pl[a] != P.pr[a]) {
+    if (backward && P.pl[a] != P.pr[a]) { // (see make_conv: refused until the 2-D case has been cleared on a GPU)
       set_error("conv: the backward kernels take symmetric padding only");
       return false;
     }
@@ -413,6 +413,7 @@ Handle *make_conv3d_backward(const OptMap &o, const Conv3dProblem &P, bool data)
   inner.n = n * Do; inner.g = g; inner.c = Z * cp; inner.k = k; inner.hi = Hi; inner.wi = Wi; inner.y = Y; inner.x = X;
   inner.ho = Ho; inner.wo = Wo; inner.sh = P.str[0]; inner.sw = P.str[1]; inner.ph = P.pl[0]; inner.pw = P.pl[1];
   inner.dh = P.dil[0]; inner.dw = P.dil[1];
+  inner.ph_r = P.pr[0]; inner.pw_r = P.pr[1];
   {
     const int64_t zc = Z * cp;
     const int64_t f2[5] = {k * Y * X * zc, Y * X * zc, 1, X * zc, zc};

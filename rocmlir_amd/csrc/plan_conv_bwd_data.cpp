@@ -57,7 +57,7 @@ Handle *make_conv_bwd_data(const OptMap &o, const ConvProblem &cp) {
   // K-major; with contiguous channels (NHWC) as dY x W with the filter
   // K-major, over all images at once when their pixels are equally spaced.
   // One kernel, no workspace.
-  if (cp.y == 1 && cp.x == 1 && cp.sh == 1 && cp.sw == 1 && cp.ph == 0 && cp.pw == 0 && cp.g == 1 &&
+  if (cp.y == 1 && cp.x == 1 && cp.sh == 1 && cp.sw == 1 && cp.unpadded() && cp.g == 1 &&
       cp.hi * cp.wi <= INT32_MAX && cp.n * cp.hi * cp.wi <= INT32_MAX && RoutePolicy(o).pointwise_as_gemm &&
       RoutePolicy(o).layout_conversion) {
     const int64_t P = cp.hi * cp.wi;

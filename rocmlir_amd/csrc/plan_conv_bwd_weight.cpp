@@ -104,7 +104,7 @@ Handle *bwd_weight_narrow_channels(const OptMap &o, const ConvProblem &cp, bool 
   while (cpad < cp.c)
     cpad *= 2;
   const int64_t pix_bytes = cpad * es;
-  if ((cp.c * es) % 16 == 0 || pix_bytes > 16 || cp.pw != 0 || cp.dw != 1 || (cp.sw * pix_bytes) % 16 != 0 ||
+  if ((cp.c * es) % 16 == 0 || pix_bytes > 16 || cp.pw != 0 || cp.pw_r != 0 || cp.dw != 1 || (cp.sw * pix_bytes) % 16 != 0 ||
       (cp.wi * pix_bytes) % 16 != 0 || (cp.k * es) % 16 != 0)
     return nullptr;
   const int64_t run = (cp.x * pix_bytes + 15) / 16 * 16 / es; // elements of a row of taps, in whole chunks
@@ -206,7 +206,7 @@ Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
   // chunks, else in the caller's letter order); what remains is the
   // unit-stride problem over the gathered tensor, planned as such (a split GEMM
   // over the tensors as they lie when the runs are whole 16-byte chunks).
-  if (cp.y == 1 && cp.x == 1 && cp.ph == 0 && cp.pw == 0 && (cp.sh > 1 || cp.sw > 1) &&
+  if (cp.y == 1 && cp.x == 1 && cp.unpadded() && (cp.sh > 1 || cp.sw > 1) &&
       RoutePolicy(o).layout_conversion && RoutePolicy(o).pointwise_as_gemm) {
     const int es = dtype_size(cp.ti);
     const int kid = (int)int_or(o, "kernel_id", 0);
@@ -368,7 +368,7 @@ Handle *make_conv_bwd_weight(const OptMap &o, const ConvProblem &cp) {
   {
     const bool lin_x = cp.is[3] == cp.wi * cp.is[4], lin_y = cp.os[3] == cp.wo * cp.os[4];
     const bool all_x = lin_x && cp.is[0] == cp.hi * cp.is[3], all_y = lin_y && cp.os[0] == cp.ho * cp.os[3];
-    if (cp.y == 1 && cp.x == 1 && cp.sh == 1 && cp.sw == 1 && cp.ph == 0 && cp.pw == 0 && cp.g == 1 && lin_x && lin_y &&
+    if (cp.y == 1 && cp.x == 1 && cp.sh == 1 && cp.sw == 1 && cp.unpadded() && cp.g == 1 && lin_x && lin_y &&
         RoutePolicy(o).pointwise_as_gemm) {
       const int64_t P = cp.hi * cp.wi;
       const bool whole = all_x && all_y; // pixels of all images form one equally spaced run

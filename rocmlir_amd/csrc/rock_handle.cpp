@@ -121,8 +121,13 @@ void describe_arguments(const OptMap &o, Handle *h) {
     const int dflt = ti == ROCK_I8 ? ROCK_I32 : (ti == ROCK_FP8 || ti == ROCK_BF8) ? ROCK_F32 : ti;
     const int to = out_t.empty() ? dflt : parse_dtype(out_t);
     std::string fl, il, ol;
-    if (!canon_layout(str_or(o, "fil_layout", ""), 'k', "gkcyx", fl) || !canon_layout(str_or(o, "in_layout", ""), 'c', "ngchw", il) ||
-        !canon_layout(str_or(o, "out_layout", ""), 'k', "ngkhw", ol))
+    auto without_depth = [&](const char *key) { // a third spatial letter of extent one (make_conv)
+      std::string s = str_or(o, key, "");
+      s.erase(std::remove(s.begin(), s.end(), '2'), s.end());
+      return s;
+    };
+    if (!canon_layout(without_depth("fil_layout"), 'k', "gkcyx", fl) || !canon_layout(without_depth("in_layout"), 'c', "ngchw", il) ||
+        !canon_layout(without_depth("out_layout"), 'k', "ngkhw", ol))
       return;
     const int64_t n = int_or(o, "batchsize", 0), g = int_or(o, "groupsize", 1), c = int_or(o, "in_channels", 0) / g,
                   k = int_or(o, "out_channels", 0) / g, hi = int_or(o, "in_h", 0), wi = int_or(o, "in_w", 0),
@@ -151,6 +156,29 @@ void describe_arguments(const OptMap &o, Handle *h) {
 Handle *build_handle(const OptMap &given) {
   OptMap planned = given;
   const OptMap &o = planned;
+  // "-p": rocmlir-gen's default problem of each operation, assigned over whatever the string gave for these keys
+  // (populateDefaults, rocmlir-gen.cpp:996-1069; its regression lists name most problems "-p" and nothing else)
+  if (bool_or(given, "p", false)) {
+    const std::string op = str_or(given, "operation", "");
+    auto set = [&](std::initializer_list<std::pair<const char *, int>> values) {
+      for (const auto &kv : values)
+        planned[kv.first] = std::to_string(kv.second);
+    };
+    if (op == "gemm") {
+      set({{"g", 1}, {"m", 1024}, {"k", 769}, {"n", 512}});
+    } else if (op == "attention") {
+      set({{"g", 1}, {"seq_len_q", 1024}, {"seq_len_k", 1024}, {"head_dim_qk", 32}, {"head_dim_v", 32}});
+    } else {
+      const bool big = str_or(given, "mfma", "infer") == "on"; // the 1x1 problem rocmlir-gen takes when MFMA is forced on
+      set({{"groupsize", 1}, {"batchsize", 128}, {"in_channels", big ? 1024 : 8}, {"out_channels", big ? 1024 : 128},
+           {"in_h", big ? 14 : 32}, {"in_w", big ? 14 : 32}, {"fil_h", big ? 1 : 3}, {"fil_w", big ? 1 : 3},
+           {"dilation_h", 1}, {"dilation_w", 1}, {"conv_stride_h", 1}, {"conv_stride_w", 1}, {"padding_h", 0},
+           {"padding_w", 0}});
+      for (const char *k : {"padding_h_l", "padding_h_r", "padding_w_l", "padding_w_r", "out_h", "out_w", "in_d", "fil_d",
+                            "out_d", "padding_d", "padding_d_l", "padding_d_r", "dilation_d", "conv_stride_d"})
+        planned.erase(k);
+    }
+  }
   // arch: "[triple:]gfxNNN[:features]" (ConvGenerator.cpp:538-552); only
   // gfx950 has kernels here
   std::string arch = str_or(o, "arch", "gfx950");
@@ -272,7 +300,9 @@ Handle *build_handle(const OptMap &given) {
     return nullptr;
   }
   h->options = given;
-  describe_arguments(given, h);
+  if (accumulate)
+    planned.erase("residual"); // C stands in for it: no such tensor in the caller's list
+  describe_arguments(planned, h);
   return h;
 }
 

@@ -200,7 +200,11 @@ std::string key_layout(const std::string &layout, bool filter);
 struct ConvProblem {
   int ti; // element type of all three tensors
   std::string fl, il, ol;
-  int64_t n, g, c, k, hi, wi, y, x, ho, wo, sh, sw, ph, pw, dh, dw;
+  int64_t n, g, c, k, hi, wi, y, x, ho, wo, sh, sw, ph, pw, dh, dw; // ph, pw: the top / left padding
+  // bottom / right padding: it only enters through ho and wo (the kernels treat every read outside the tensor as
+  // zero), but the routes that read the tensors "as they lie" need both sides to be zero
+  int64_t ph_r = 0, pw_r = 0;
+  bool unpadded() const { return ph == 0 && pw == 0 && ph_r == 0 && pw_r == 0; }
   int64_t fs[5], is[5], os[5]; // element strides in letter order gkcyx / ngchw / ngkhw
   // filter gradient only: the output gradient is a copy whose k channels were padded with zeros up to a whole
   // 16-byte chunk; only the first k_valid rows of the gradient exist in the caller's tensor (0: all k)

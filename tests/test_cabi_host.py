@@ -1022,3 +1022,44 @@ def test_attention_pre_softmax_program(rock):
                 "x,t0,mul -scale 0.5"):
         with pytest.raises(rock.RockError):
             rock.RockKernel(f16 + "-attn_elementwise " + bad)
+
+
+def test_every_problem_of_the_reference_e2e_lists_resolves(rock):
+    """mlir/test/e2e/*.toml, expanded as mlir/test/e2e/generateE2ETest.py expands them (tests/e2e_lists.py): each of
+    the 2278 option strings -- "-p" default problems, layouts without g or with a third spatial letter of extent
+    one, left / right padding given apart, --reverse_grid, split-K perf_configs, --store-method=atomic_add --
+    gives a handle whose every kernel has a code object, and the handle describes tensors of the sizes the
+    option string implies.  The one exception is refused with a message: the twelve gradient problems with
+    unequal left and right padding (conv_regression_bwd.toml's 4x4 / 2x2 / stride 2 / padding 2,1 and 2,0 case)."""
+    import numpy as np
+    from tests.e2e_lists import problems
+    from tests.test_gpu_e2e_lists import parse_options
+    lists, kernels, refused = set(), 0, []
+    for name, opts in problems():
+        try:
+            first = rock.RockKernel(opts)
+        except rock.RockError as e:
+            refused.append((name, opts, str(e)))
+            continue
+        lists.add(name)
+        kernels += first.kernel_count
+        if first.kernel_count > 1:    # the last kernel of a plan too (conversions first, reductions last)
+            rock.RockKernel("%s --kernel_id %d" % (opts, first.kernel_count - 1))
+        o = parse_options(opts)
+        if o["operation"] in ("gemm", "attention"):
+            continue
+        g = int(o.get("groupsize", 1))
+        n, c, k = int(o["batchsize"]), int(o["in_channels"]) // g, int(o["out_channels"]) // g
+        hi, wi, y, x = int(o["in_h"]), int(o["in_w"]), int(o["fil_h"]), int(o["fil_w"])
+        sh, sw = int(o.get("conv_stride_h", 1)), int(o.get("conv_stride_w", 1))
+        dh, dw = int(o.get("dilation_h", 1)), int(o.get("dilation_w", 1))
+        p_h, p_w = int(o.get("padding_h", 0)), int(o.get("padding_w", 0))
+        pl = (int(o.get("padding_h_l", p_h)), int(o.get("padding_w_l", p_w)))
+        pr = (int(o.get("padding_h_r", p_h)), int(o.get("padding_w_r", p_w)))
+        ho = (hi + pl[0] + pr[0] - (y - 1) * dh - 1) // sh + 1
+        wo = (wi + pl[1] + pr[1] - (x - 1) * dw - 1) // sw + 1
+        sizes = [int(np.prod(dims)) for _, dims in first.arguments()[:3]]
+        assert sizes == [g * k * c * y * x, n * g * c * hi * wi, n * g * k * ho * wo], opts
+    assert len(lists) == 19 and kernels > 2278
+    assert len(refused) == 12 and all(name == "conv_regression_bwd.toml" and "symmetric padding" in msg and
+                                      "-padding_h_l=2 -padding_h_r=1" in opts for name, opts, msg in refused)
