@@ -58,6 +58,16 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t dl_rsrc(const void *base) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)kOobOffset, 0x00020000);
 }
 
+// a zero the compiler cannot see through (the host build of the body, which the tests step through on the CPU,
+// has no scalar registers to pin it to and needs no such barrier)
+__device__ __forceinline__ int opaque_zero() {
+  int zero = 0;
+#ifdef __AMDGCN__
+  asm volatile("" : "+s"(zero));
+#endif
+  return zero;
+}
+
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
   // gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
@@ -854,7 +864,12 @@ __device__ __forceinline__ void dl_epilogue(typename MmaTraits<DT>::Acc (&acc)[M
                                                     staged_ok);
     return;
   }
-  const bool cols_ok = !staged_ok && out_cols_chunk_aligned(p, Cptr, out_elem_size(e.out_dtype));
+  // (the 16-byte vectors of consecutive rows start at multiples of 16 bytes from the wave's first row and must
+  // neither straddle an image nor run past the last row: the implicit-GEMM tiles start at multiples of 32 rows,
+  // the window-resident kernel's at any multiple of the output width and end with their last output row)
+  const int out_es = out_elem_size(e.out_dtype);
+  const bool cols_ok = !staged_ok && out_cols_chunk_aligned(p, Cptr, out_es) &&
+                       (((int64_t)m_wave * out_es | (int64_t)p.M * out_es) & 15) == 0;
   if (staged_ok || cols_ok)
     __builtin_amdgcn_s_barrier(); // every wave is done reading the operand stages
 
@@ -1046,9 +1061,7 @@ __device__ __forceinline__ void contraction_body_dl(const void *Aptr, const void
       // (the second stage lies beyond the reach of the reads' 16-bit offset
       // field).  An offset of zero that the compiler cannot see through keeps
       // the address arithmetic of a step inside the step, one add per read.
-      int zero = 0;
-      asm volatile("" : "+s"(zero));
-      sa += zero;
+      sa += opaque_zero();
     }
     // this wave's loads of K-step kt have landed (two younger steps may be in flight) ...
     wait_vmcnt_and_lds_reads<(kDlStages - 2) * LOADS_PER_STEP>();

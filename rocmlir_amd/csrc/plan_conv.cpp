@@ -148,12 +148,20 @@ WindowPlan window_plan(const RockConvParams &p, int ti, bool equal_padding, cons
   auto tiles_of = [&](int64_t rows) { return (int64_t)ceil_div((int64_t)p.n * p.ho, rows) * w.tiles_n * p.g; };
   // rows per tile: the fewest rounds of blocks (two per CU), then the most rows
   const int64_t per_round = 2 * (int64_t)kNumCU;
-  for (int64_t rows = std::min<int64_t>(p.ho, p.wo > 0 ? tile_px / p.wo : 0); rows >= 1; --rows) {
-    if (window_rows(rows) * row_pitch > kDirectWindowBytes)
-      continue;
-    if (w.rows == 0 || ceil_div(tiles_of(rows), per_round) < ceil_div(tiles_of(w.rows), per_round))
-      w.rows = rows;
-  }
+  // An output whose pixels are contiguous per channel (NCHW style) leaves the kernel as 16-byte vectors of
+  // consecutive pixels only when every tile starts on such a vector, element by element otherwise: tiles of whole
+  // vectors first, any tile if there is none.
+  const int64_t out_es = std::max(1, dtype_size(p.epi.out_dtype));
+  const bool pixels_contiguous = p.out_ws == 1 && p.out_ks != 1;
+  for (int pass = 0; pass < 2 && w.rows == 0; ++pass)
+    for (int64_t rows = std::min<int64_t>(p.ho, p.wo > 0 ? tile_px / p.wo : 0); rows >= 1; --rows) {
+      if (window_rows(rows) * row_pitch > kDirectWindowBytes)
+        continue;
+      if (pass == 0 && pixels_contiguous && (rows * p.wo * out_es) % 16 != 0)
+        continue;
+      if (w.rows == 0 || ceil_div(tiles_of(rows), per_round) < ceil_div(tiles_of(w.rows), per_round))
+        w.rows = rows;
+    }
   w.ok = p.stride_h == 1 && p.stride_w == 1 && p.dil_h == 1 && p.dil_w == 1 && p.y * p.x > 1 && equal_padding &&
          p.k % 32 == 0 && cbytes >= 128 && cbytes <= 1024 && (cbytes & (cbytes - 1)) == 0 && w.rows >= 1 &&
          row_pitch <= 32 * 1024 && p.in_cs == 1;

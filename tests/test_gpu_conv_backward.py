@@ -212,6 +212,26 @@ def test_conv_bwd_data_on_the_window_resident_kernel_exact(rock, oracle, gpu, la
     assert np.array_equal(to_f32(dx, "f16"), oracle.round_through(ref, CODE["f16"]))
 
 
+@pytest.mark.parametrize("case,last", [
+    ((128, 1, 256, 128, 28, 28, 3, 3, (1, 1), (1, 1), (1, 1)), "rock_conv_f16_128x128_fast"),
+    ((64, 1, 256, 64, 56, 56, 3, 3, (1, 1), (1, 1), (1, 1)), "rock_conv_f16_direct224"),
+], ids=["28x28", "56x56"])
+def test_conv_bwd_data_channel_major_gradient_exact(rock, oracle, gpu, case, last):
+    """The same gradients written channel-major (NCHW), as 16-byte vectors of consecutive pixels: the reference's
+    backward regression list holds both layers.  Four rows of 56 pixels are whole vectors, so that layer stays on
+    the window-resident kernel; seven rows of 28 pixels are not (tiles would start in the middle of a vector), and
+    the table keeps the layer on the implicit-GEMM kernel, whose tiles start at multiples of 32 pixels."""
+    n, g, c, k, hi, wi, y, x, stride, pad, dil = case
+    (raw_f, fq), _, (raw_dy, dyq), ho, wo = _tensors(case, NCHW, "f16", 83, integer=True)
+    info = {}
+    print("bwd data, channel-major gradient", case, flush=True)
+    dx = rock.conv2d_bwd_data(to_gpu(raw_f, "f16", gpu), to_gpu(raw_dy, "f16", gpu), info=info, **_kw(case, NCHW))
+    torch.cuda.synchronize()
+    assert info["kernels"][-1] == last
+    ref, _, _ = oracle.conv_bwd_data(fq, dyq, *NCHW, n, g, c, k, hi, wi, y, x, stride, pad, dil)
+    assert np.array_equal(to_f32(dx, "f16"), oracle.round_through(ref, CODE["f16"]))
+
+
 NARROW_CASES = [
     (8, 1, 3, 64, 38, 38, 7, 7, (2, 2), (0, 0), (1, 1)),      # the ResNet first layer in small, pixels split
     (2, 1, 3, 16, 20, 20, 7, 7, (2, 2), (0, 0), (1, 1)),
