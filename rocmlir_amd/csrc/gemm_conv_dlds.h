@@ -829,17 +829,20 @@ __device__ __forceinline__ void dl_epilogue_rich(typename MmaTraits<DT>::Acc (&a
 #pragma unroll
       for (int t = 0; t < NI * 4; ++t)
         raw[t] = *(const v4i *)(wbuf + (t * 64 + lane) * 16);
+      RK_WAVE_LDS_ORDER();
 #pragma unroll
       for (int t = 0; t < NI * 4; ++t)
         dl_rich_emit<NI>(p, Cptr, wbuf, raw[t], t, es, row, n_wave, lane, staged_ok);
     }
     if (staged_ok) {
+      RK_WAVE_LDS_ORDER();
       if (es == 4)
         dl_rich_flush<4, NI>(p, g, Cptr, wbuf, m_wave + i * 32, n_wave, lane);
       else if (es == 2)
         dl_rich_flush<2, NI>(p, g, Cptr, wbuf, m_wave + i * 32, n_wave, lane);
       else
         dl_rich_flush<1, NI>(p, g, Cptr, wbuf, m_wave + i * 32, n_wave, lane);
+      RK_WAVE_LDS_ORDER();
     }
   });
 }
@@ -908,6 +911,7 @@ __device__ __forceinline__ void dl_epilogue(typename MmaTraits<DT>::Acc (&acc)[M
             }
           }
         }
+        RK_WAVE_LDS_ORDER();
 #pragma unroll
         for (int it = 0; it < WTN * VPR / 64; ++it) {
           const int v = it * 64 + lane;
@@ -920,6 +924,7 @@ __device__ __forceinline__ void dl_epilogue(typename MmaTraits<DT>::Acc (&acc)[M
             *(v4i *)((char *)Cptr + (off + (int64_t)n * n_stride) * ES) = d;
           }
         }
+        RK_WAVE_LDS_ORDER();
       }
       return;
     }
@@ -958,6 +963,7 @@ __device__ __forceinline__ void dl_epilogue(typename MmaTraits<DT>::Acc (&acc)[M
             *(int *)dst = raw[0];
         }
       }
+      RK_WAVE_LDS_ORDER();
 #pragma unroll
       for (int r0 = 0; r0 < 32; r0 += RPI) {
         const int row = r0 + rd_row;
@@ -973,6 +979,7 @@ __device__ __forceinline__ void dl_epilogue(typename MmaTraits<DT>::Acc (&acc)[M
           __builtin_nontemporal_store(d, (v4i *)((char *)Cptr + (row_off + n) * ES));
         }
       }
+      RK_WAVE_LDS_ORDER();
     }
   });
 }

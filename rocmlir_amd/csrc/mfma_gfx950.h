@@ -20,6 +20,13 @@
 #include <hip/hip_runtime.h>
 #include "kernel_params.h"
 
+// Where lanes of a wave hand data to each other through LDS with no instruction between the store and the load
+// (a wave's LDS operations complete in order).  Nothing on the GPU; the CPU build of the kernels that the tests
+// step through runs the lanes one after the other and makes them meet at these points.
+#ifndef RK_WAVE_LDS_ORDER
+#define RK_WAVE_LDS_ORDER() ((void)0)
+#endif
+
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v2i __attribute__((ext_vector_type(2)));

@@ -1,6 +1,7 @@
-// Runner of the host build of the contraction kernels (see hip/hip_runtime.h in
-// this directory): tensors between canary pages and inaccessible guard regions,
-// one child process per launch so that a trap ends the child and not the test.
+// Runner of the host build of the kernels (see hip/hip_runtime.h in this
+// directory): tensors between canary pages and inaccessible guard regions, one
+// child process per launch so that a trap ends the child and not the test, and
+// inside it one cooperative fiber per thread of the block that is running.
 // Test infrastructure only.
 #include "hip/hip_runtime.h"
 #include "kernel_table.h"
@@ -8,6 +9,7 @@
 #include <string>
 #include <sys/mman.h>
 #include <sys/wait.h>
+#include <ucontext.h>
 #include <unistd.h>
 #include <vector>
 
@@ -59,7 +61,99 @@ void on_trap(int sig, siginfo_t *si, void *) {
   (void)sig;
   _exit(0);
 }
+
+// ---- one block as cooperative fibers ---------------------------------------------
+enum State { kRun, kWaitWave, kWaitBlock, kDone };
+struct Fiber {
+  ucontext_t ctx;
+  State state;
+  unsigned ops; // cross-lane operations begun: picks the half of the exchange area
+};
+constexpr size_t kStack = 512 * 1024;
+constexpr unsigned kMaxThreads = 1024;
+Fiber *fibers = nullptr;
+char *stacks = nullptr;
+char (*slots)[2][64][128] = nullptr; // per wave: two halves, used in turn
+ucontext_t scheduler;
+unsigned current = 0, threads = 0;
+void (*kernel_fn)(void **, const void *) = nullptr;
+void **kernel_pointers = nullptr;
+const void *kernel_params = nullptr;
+
+void fiber_main() {
+  kernel_fn(kernel_pointers, kernel_params);
+  fibers[current].state = kDone;
+}
+void wait_as(State s) {
+  fibers[current].state = s;
+  swapcontext(&fibers[current].ctx, &scheduler);
+}
+void run_block() {
+  if (!fibers) {
+    fibers = new Fiber[kMaxThreads];
+    stacks = (char *)mmap(nullptr, kStack * kMaxThreads, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE,
+                          -1, 0);
+    slots = (char(*)[2][64][128])calloc(kMaxThreads / 64, sizeof *slots);
+    for (unsigned t = 0; t < kMaxThreads; ++t) // a stack that overflows traps instead of running into its neighbour
+      mprotect(stacks + (size_t)t * kStack, kPage, PROT_NONE);
+  }
+  for (unsigned t = 0; t < threads; ++t) {
+    getcontext(&fibers[t].ctx);
+    fibers[t].ctx.uc_stack.ss_sp = stacks + (size_t)t * kStack;
+    fibers[t].ctx.uc_stack.ss_size = kStack;
+    fibers[t].ctx.uc_link = &scheduler;
+    makecontext(&fibers[t].ctx, fiber_main, 0);
+    fibers[t].state = kRun;
+    fibers[t].ops = 0;
+  }
+  for (;;) {
+    bool ran = false;
+    for (unsigned t = 0; t < threads; ++t)
+      if (fibers[t].state == kRun) {
+        current = t;
+        threadIdx = {t, 0, 0};
+        swapcontext(&scheduler, &fibers[t].ctx);
+        ran = true;
+      }
+    // a wave goes on when all its live lanes wait for each other, the block when all its live threads do
+    bool released = false;
+    unsigned done = 0, at_barrier = 0;
+    for (unsigned w = 0; w * 64 < threads; ++w) {
+      unsigned waiting = 0, live = 0;
+      for (unsigned t = w * 64; t < std::min(threads, w * 64 + 64); ++t) {
+        waiting += fibers[t].state == kWaitWave;
+        live += fibers[t].state != kDone;
+        done += fibers[t].state == kDone;
+        at_barrier += fibers[t].state == kWaitBlock;
+      }
+      if (waiting && waiting == live) {
+        for (unsigned t = w * 64; t < std::min(threads, w * 64 + 64); ++t)
+          if (fibers[t].state == kWaitWave)
+            fibers[t].state = kRun;
+        released = true;
+      }
+    }
+    if (done == threads)
+      return;
+    if (at_barrier && at_barrier + done == threads) {
+      for (unsigned t = 0; t < threads; ++t)
+        if (fibers[t].state == kWaitBlock)
+          fibers[t].state = kRun;
+      released = true;
+    }
+    if (!ran && !released) {
+      char text[200];
+      snprintf(text, sizeof text, "%s, block %u: the threads wait for each other at different places (%u of %u at "
+               "the barrier, %u done)", cur_kernel, blockIdx.x, at_barrier, threads, done);
+      note(text);
+      _exit(0);
+    }
+  }
+}
 } // namespace
+
+void hm_wave_sync() { wait_as(kWaitWave); }
+void hm_block_sync() { wait_as(kWaitBlock); }
 
 void hm_check_global(const void *p, size_t n, const char *what) {
   const char *c = (const char *)p;
@@ -71,6 +165,162 @@ void hm_check_global(const void *p, size_t n, const char *what) {
   snprintf(text, sizeof text, "%s outside the tensors in %s, block %u thread %u: %zu bytes at %s", what, cur_kernel,
            blockIdx.x, threadIdx.x, n, at);
   note(text);
+}
+
+// ---- cross-lane operations: every lane puts its operands into its slot of the wave's exchange area, the wave
+// meets, every lane computes its result from the slots.  The area has two halves used in turn, so that a lane
+// that has gone on to the next operation does not overwrite what a slower lane still reads.
+namespace {
+inline int lane_id() { return (int)(current & 63); }
+char *my_slot() {
+  Fiber &f = fibers[current];
+  ++f.ops;
+  return slots[current / 64][f.ops & 1][current & 63];
+}
+const char *slot_of(int lane) { return slots[current / 64][fibers[current].ops & 1][lane & 63]; }
+double widen(int type, const char *p, int k) {
+  switch (type) {
+  case HM_F32: {
+    float f;
+    std::memcpy(&f, p + 4 * k, 4);
+    return f;
+  }
+  case HM_F16: {
+    _Float16 h;
+    std::memcpy(&h, p + 2 * k, 2);
+    return (double)(float)h;
+  }
+  case HM_BF16: {
+    uint16_t h;
+    std::memcpy(&h, p + 2 * k, 2);
+    const uint32_t w = (uint32_t)h << 16;
+    float f;
+    std::memcpy(&f, &w, 4);
+    return f;
+  }
+  case HM_I8: return (double)(int8_t)p[k];
+  case HM_E4M3: return hm_f8_to_f32((unsigned char)p[k], 4);
+  default: return hm_f8_to_f32((unsigned char)p[k], 5);
+  }
+}
+int elem_bytes(int type) { return type == HM_F32 ? 4 : (type == HM_F16 || type == HM_BF16) ? 2 : 1; }
+} // namespace
+
+void hm_load_lds(HmRsrc r, void *lds, int size, int voff, int soff, int ioff, int) {
+  char *dst = (char *)lds + lane_id() * size; // the wave's lanes land back to back
+  const uint64_t off = (uint64_t)(unsigned)voff + (unsigned)ioff;
+  if (off >= r.num_records || off + (unsigned)soff >= r.num_records) {
+    std::memset(dst, 0, size);
+    return;
+  }
+  const char *src = r.base + off + (unsigned)soff;
+  hm_check_global(src, size, "buffer load into LDS");
+  std::memcpy(dst, src, size);
+}
+hm_v4i hm_load_b128(HmRsrc r, int voff, int soff, int) {
+  hm_v4i v = {0, 0, 0, 0};
+  const uint64_t off = (uint64_t)(unsigned)voff;
+  if (off >= r.num_records || off + (unsigned)soff >= r.num_records)
+    return v;
+  const char *src = r.base + off + (unsigned)soff;
+  hm_check_global(src, 16, "buffer load");
+  std::memcpy(&v, src, 16);
+  return v;
+}
+void hm_first_lane(void *value, size_t bytes) {
+  std::memcpy(my_slot(), value, bytes);
+  wait_as(kWaitWave);
+  std::memcpy(value, slot_of(0), bytes);
+}
+uint64_t hm_ballot(bool p) {
+  *my_slot() = p ? 1 : 0;
+  wait_as(kWaitWave);
+  uint64_t m = 0;
+  for (int l = 0; l < 64; ++l)
+    m |= (uint64_t)(*slot_of(l) & 1) << l;
+  return m;
+}
+int hm_bpermute(int byte_index, int v) {
+  std::memcpy(my_slot(), &v, 4);
+  wait_as(kWaitWave);
+  int out;
+  std::memcpy(&out, slot_of((byte_index >> 2) & 63), 4);
+  return out;
+}
+void hm_shuffle_xor(void *value, size_t bytes, int mask, int width) {
+  std::memcpy(my_slot(), value, bytes);
+  wait_as(kWaitWave);
+  const int l = lane_id(), from = (l & ~(width - 1)) | ((l ^ mask) & (width - 1));
+  std::memcpy(value, slot_of(from), bytes);
+}
+void hm_read_transposed(const void *p, int eb, void *out8) {
+  std::memcpy(my_slot(), p, 8);
+  wait_as(kWaitWave);
+  const int l = lane_id(), group = l & ~15, i = l & 15;
+  const int per_row = 8 / eb; // elements a lane names, and rows of the block: 4 of 16-bit, 8 of 8-bit elements
+  char *out = (char *)out8;
+  const int lanes_per_row = 16 / per_row; // lanes that together name one row of 16 elements
+  for (int e = 0; e < per_row; ++e)       // column i of rows 0 .. per_row - 1
+    std::memcpy(out + e * eb, slot_of(group + lanes_per_row * e + i / per_row) + (i % per_row) * eb, eb);
+}
+float hm_f8_to_f32(unsigned code, int ebits) {
+  const int mbits = 7 - ebits, bias = (1 << (ebits - 1)) - 1;
+  const int s = (code >> 7) & 1, e = (code >> mbits) & ((1 << ebits) - 1), m = code & ((1 << mbits) - 1);
+  float v;
+  if (ebits == 5 && e == 31)
+    v = m ? NAN : INFINITY;
+  else if (ebits == 4 && e == 15 && m == 7)
+    v = NAN;
+  else if (e == 0)
+    v = std::ldexp((float)m, 1 - bias - mbits);
+  else
+    v = std::ldexp((float)((1 << mbits) + m), e - bias - mbits);
+  return s ? -v : v;
+}
+static unsigned f32_to_f8(float f, int ebits) {
+  if (f != f)
+    return ebits == 4 ? 0x7f : 0x7e;
+  unsigned best = 0;
+  double best_err = INFINITY;
+  const double a = std::fabs((double)f);
+  for (unsigned c = 0; c < 128; ++c) {
+    const float v = hm_f8_to_f32(c, ebits);
+    if (v != v || std::isinf(v))
+      continue;
+    const double err = std::fabs((double)v - a);
+    if (err < best_err || (err == best_err && (c & 1) == 0 && (best & 1) == 1)) {
+      best = c;
+      best_err = err;
+    }
+  }
+  return best | (std::signbit(f) ? 0x80u : 0u);
+}
+int hm_cvt_pk_f8(float a, float b, int old, bool hi, int ebits) {
+  const unsigned pair = f32_to_f8(a, ebits) | (f32_to_f8(b, ebits) << 8);
+  return hi ? (int)(((unsigned)old & 0xffffu) | (pair << 16)) : (int)(((unsigned)old & 0xffff0000u) | pair);
+}
+// The products are formed in double precision and added to the accumulator once per instruction: exact, like
+// the hardware's result, on the integer-valued data the tests use.
+void hm_mfma_32x32(int type_a, int type_b, const void *a, const void *b, int lane_bytes, void *acc16) {
+  char *mine = my_slot();
+  std::memcpy(mine, a, lane_bytes);
+  std::memcpy(mine + 64, b, lane_bytes);
+  wait_as(kWaitWave);
+  const int l = lane_id(), j = l & 31, per_lane = lane_bytes / elem_bytes(type_a);
+  const bool int_acc = type_a == HM_I8;
+  for (int v = 0; v < 16; ++v) {
+    const int i = 8 * (v / 4) + 4 * (l / 32) + v % 4;
+    double sum = 0.0;
+    for (int half = 0; half < 2; ++half) {
+      const char *ra = slot_of(i + 32 * half), *cb = slot_of(j + 32 * half) + 64;
+      for (int k = 0; k < per_lane; ++k)
+        sum += widen(type_a, ra, k) * widen(type_b, cb, k);
+    }
+    if (int_acc)
+      ((int *)acc16)[v] = (int)((double)((int *)acc16)[v] + sum);
+    else
+      ((float *)acc16)[v] = (float)((double)((float *)acc16)[v] + sum);
+  }
 }
 
 extern "C" {
@@ -112,7 +362,7 @@ int hm_knows(const char *name) {
       return 1;
   return 0;
 }
-// Runs every block and thread of the launch.  Returns the number of accesses outside the tensors (-1: no such
+// Runs every block of the launch, one after the other.  Returns the number of accesses outside the tensors (-1: no such
 // kernel in this build, -2: the child could not be started); `first` receives a description of the first one.
 long hm_run(const char *name, const void *params, void **pointers, unsigned grid, unsigned block, char *first,
             size_t first_bytes) {
@@ -130,21 +380,28 @@ long hm_run(const char *name, const void *params, void **pointers, unsigned grid
   if (child < 0)
     return -2;
   if (child == 0) {
+    static char trap_stack[64 * 1024];
+    stack_t alt;
+    alt.ss_sp = trap_stack;
+    alt.ss_size = sizeof trap_stack;
+    alt.ss_flags = 0;
+    sigaltstack(&alt, nullptr);
     struct sigaction sa;
     std::memset(&sa, 0, sizeof sa);
     sa.sa_sigaction = on_trap;
-    sa.sa_flags = SA_SIGINFO;
+    sa.sa_flags = SA_SIGINFO | SA_ONSTACK;
     sigaction(SIGSEGV, &sa, nullptr);
     sigaction(SIGBUS, &sa, nullptr);
     cur_kernel = name;
     gridDim = {grid, 1, 1};
     blockDim = {block, 1, 1};
+    kernel_fn = fn;
+    kernel_pointers = pointers;
+    kernel_params = params;
+    threads = block;
     for (unsigned b = 0; b < grid; ++b) {
       blockIdx = {b, 0, 0};
-      for (unsigned t = 0; t < block; ++t) {
-        threadIdx = {t, 0, 0};
-        fn(pointers, params);
-      }
+      run_block();
     }
     _exit(0);
   }

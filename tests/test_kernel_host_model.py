@@ -1,10 +1,14 @@
-"""The contraction kernels compiled for the CPU and stepped through whole plans, every block and thread, with
-every address checked (tests/kernel_host/: the stand-in for the device environment and the runner).
+"""The kernels compiled for the CPU and run through whole plans, block by block, against the oracle
+(tests/kernel_host/: the stand-in for the device environment and the runner).
 
-What the model does and does not show: a thread forms the same addresses as on the GPU (they never depend on data
-in these kernels), buffer loads are range-checked like the hardware's, every tensor lies between canary pages and
-inaccessible regions, and a 16-byte access that is not 16-byte aligned traps.  The values are not computed (the
-matrix instructions do nothing and threads do not run in step), so results are the GPU tests' business.
+What the model is: the kernels' own sources (csrc/gemm_conv_dlds.h and what it includes, relayout_kernels.hip)
+built for x86, each thread of a block a cooperative fiber that runs until it meets an operation involving other
+threads -- a barrier, a matrix instruction, a cross-lane or transposing read -- where the wave or the block
+gathers and the operation is computed from every lane's operands.  LDS then holds what the GPU's LDS holds, every
+address is the one the GPU thread forms, and on integer-valued data the results must equal the oracle's bit for
+bit.  Buffer loads are range-checked like the hardware's, every tensor lies between canary pages and inaccessible
+regions, and a 16-byte access that is not 16-byte aligned traps.  What it is not: timing, the memory model
+(loads into LDS land when issued), or the accumulation order inside a matrix instruction (exact data only).
 
 The plans come from the C ABI exactly as a caller gets them: kernel name, grid, block, parameter block and
 pointer map per kernel id, tensor sizes from rockamdGetArgumentInfo.
@@ -42,34 +46,63 @@ def _params_type(macro):
     return "RockConvBwdWeightParams" if "BWD_WEIGHT" in macro else "RockConvParams"
 
 
-def _model_source(code):
+def _model_sources(code, parts=3):
+    """The contraction kernels of one operand type as `parts` translation units (they compile side by side)."""
     t = _TYPES[code]
     kernels = [(n, m) for n, m in _build.contraction_kernels(code) if not n.endswith(_LEFT_OUT)]
-    lines = ["#define ROCK_DT %d" % code, "#define ROCK_DTNAME %s" % t, '#include "gemm_conv_instances.h"',
-             '#include "kernel_table.h"']
-    lines += [m for _, m in kernels]
-    for n, m in kernels:
+    units = {}
+    for part in range(parts):
+        mine = kernels[part::parts]
+        lines = ["#define ROCK_DT %d" % code, "#define ROCK_DTNAME %s" % t, '#include "gemm_conv_instances.h"',
+                 '#include "kernel_table.h"']
+        lines += [m for _, m in mine]
+        for n, m in mine:
+            lines.append("static void call_%s(void **q, const void *params) { %s p; std::memcpy(&p, params, sizeof p); "
+                         "%s(q[0], q[1], q[2], q[3], q[4], p); }" % (n, _params_type(m), n))
+        lines.append("static const HmEntry table[] = {")
+        lines += ['  {"%s", call_%s},' % (n, n) for n, _ in mine]
+        lines += ["  {nullptr, nullptr}};", "const HmEntry *hm_table_%s_%d() { return table; }" % (t, part)]
+        units["model_%s_%d" % (t, part)] = "\n".join(lines) + "\n"
+    return units
+
+
+# the kernels of csrc/relayout_kernels.hip: name -> (parameter block, pointers)
+_UTILITY = {"rock_relayout_b1": ("RockRelayoutParams", 2), "rock_relayout_b2": ("RockRelayoutParams", 2),
+            "rock_relayout_b4": ("RockRelayoutParams", 2), "rock_fill_zero": ("RockFillParams", 1),
+            "rock_reduce_splits": ("RockReduceParams", 2), "rock_softmax_rows": ("RockSoftmaxParams", 5),
+            "rock_relayout_pair_b1": ("RockRelayoutPairParams", 4), "rock_relayout_pair_b2": ("RockRelayoutPairParams", 4),
+            "rock_relayout_pair_b4": ("RockRelayoutPairParams", 4), "rock_fold_depth": ("RockFoldDepthParams", 2)}
+_CASTS = {"rock_reduce_splits": ["(const float *)", ""], "rock_softmax_rows": ["(float *)", "", "", "", ""]}
+
+
+def _utility_source():
+    lines = ['#include "relayout_kernels.hip"', '#include "kernel_table.h"', "#include <cstring>"]
+    for n, (ptype, count) in _UTILITY.items():
+        casts = _CASTS.get(n, [""] * count)
+        args = ", ".join("%sq[%d]" % (casts[i], i) for i in range(count))
         lines.append("static void call_%s(void **q, const void *params) { %s p; std::memcpy(&p, params, sizeof p); "
-                     "%s(q[0], q[1], q[2], q[3], q[4], p); }" % (n, _params_type(m), n))
+                     "%s(%s, p); }" % (n, ptype, n, args))
     lines.append("static const HmEntry table[] = {")
-    lines += ['  {"%s", call_%s},' % (n, n) for n, _ in kernels]
-    lines += ["  {nullptr, nullptr}};", "const HmEntry *hm_table_%s() { return table; }" % t]
+    lines += ['  {"%s", call_%s},' % (n, n) for n in _UTILITY]
+    lines += ["  {nullptr, nullptr}};", "const HmEntry *hm_table_utility() { return table; }"]
     return "\n".join(lines) + "\n"
 
 
-def _table_source():
+def _table_source(tables):
     lines = ['#include "kernel_table.h"', "#include <vector>"]
-    lines += ["const HmEntry *hm_table_%s();" % t for t in _TYPES.values()]
+    lines += ["const HmEntry *%s();" % t for t in tables]
     lines += ["const HmEntry *hm_kernel_table() {", "  static std::vector<HmEntry> all;", "  if (all.empty()) {"]
-    lines += ["    for (const HmEntry *e = hm_table_%s(); e->name; ++e) all.push_back(*e);" % t for t in _TYPES.values()]
+    lines += ["    for (const HmEntry *e = %s(); e->name; ++e) all.push_back(*e);" % t for t in tables]
     lines += ["    all.push_back({nullptr, nullptr});", "  }", "  return all.data();", "}"]
     return "\n".join(lines) + "\n"
 
 
 def build_model(d):
     """Compiles the model into directory d and returns the loaded library."""
-    units = {"kernel_table": _table_source()}
-    units.update({"model_%s" % t: _model_source(code) for code, t in _TYPES.items()})
+    units = {"model_utility": _utility_source()}
+    for code in _TYPES:
+        units.update(_model_sources(code))
+    units["kernel_table"] = _table_source(["hm_table_" + n[len("model_"):] for n in units])
     for name, text in units.items():
         with open(os.path.join(d, name + ".cpp"), "w") as f:
             f.write(text)
@@ -115,9 +148,11 @@ def _pointer_map(rock, k):
     return [(src[i], off[i]) for i in range(nk.value)]
 
 
-def run_plan(model, rock, opts, shrink=None):
-    """Steps every kernel of the plan that the model holds.  shrink = (caller index, bytes): that tensor is
-    allocated short by so many bytes (to show that the model notices).  Returns (kernel names stepped, problems)."""
+def run_plan(model, rock, opts, inputs=None, shrink=None):
+    """Runs every kernel of the plan in order.  inputs = {caller index: numpy array}, copied into that tensor as
+    it lies (the other tensors start as 0xEE bytes); shrink = (caller index, bytes): that tensor is allocated
+    short by so many bytes (to show that the model notices).  Returns (kernel names, problems, tensors) with the
+    tensors as uint8 views of the model's memory."""
     first = rock.RockKernel(opts)
     model.hm_clear()
     tensors = []
@@ -126,80 +161,162 @@ def run_plan(model, rock, opts, shrink=None):
         if shrink and shrink[0] == i:
             nbytes -= shrink[1]
         nbytes = max(nbytes, 16)
-        tensors.append((model.hm_alloc(nbytes, b"argument %d" % i), nbytes))
-    stepped, problems = [], []
+        at = model.hm_alloc(nbytes, b"argument %d" % i)
+        view = np.ctypeslib.as_array((C.c_uint8 * nbytes).from_address(at))
+        view[:] = 0xEE
+        if inputs and i in inputs:
+            raw = np.ascontiguousarray(inputs[i]).view(np.uint8).ravel()
+            view[:raw.size] = raw
+        tensors.append((at, nbytes, view))
+    names, problems = [], []
     for kid in range(first.kernel_count):
         k = first if kid == 0 else rock.RockKernel(opts + " --kernel_id %d" % kid)
         name = k.kernel_name.encode()
-        if not model.hm_knows(name):
-            continue
+        assert model.hm_knows(name), "the model does not hold " + k.kernel_name
         ptrs = (C.c_void_p * 8)()
         for j, (src, off) in enumerate(_pointer_map(rock, k)):
             ptrs[j] = None if src < 0 else tensors[src][0] + off
         text = C.create_string_buffer(512)
         bad = model.hm_run(name, k.params(), ptrs, k.grid_size, k.block_size, text, 512)
         assert bad >= 0, "the model could not run " + k.kernel_name
-        stepped.append(k.kernel_name)
+        names.append(k.kernel_name)
         if bad:
             problems.append("%s: %d, first: %s" % (k.kernel_name, bad, text.value.decode()))
-        for i, (p, n) in enumerate(tensors):
-            changed = model.hm_canaries(p, n)
+        for i, (at, n, _) in enumerate(tensors):
+            changed = model.hm_canaries(at, n)
             if changed:
                 problems.append("%s wrote %d bytes beside argument %d" % (k.kernel_name, changed, i))
-    return stepped, problems
+    return names, problems, [v for _, _, v in tensors]
 
 
-def _conv(op, t, n, c, k, hw, f, pad, layouts="kcyx nchw nkhw", stride=1, extra=""):
+_NUMPY = {"f32": np.float32, "f16": np.float16}
+
+
+def _conv_problem(op, t, n, c, k, hi, wi, f, pad, layouts, stride=1, extra=""):
     fl, il, ol = layouts.split()
     return ("-operation %s -arch gfx950 -t %s -groupsize 1 -batchsize %d -in_channels %d -out_channels %d -in_h %d "
             "-in_w %d -fil_h %d -fil_w %d -padding_h %d -padding_w %d -conv_stride_h %d -conv_stride_w %d "
-            "-fil_layout %s -in_layout %s -out_layout %s %s" % (op, t, n, c, k, hw, hw, f, f, pad, pad, stride, stride,
+            "-fil_layout %s -in_layout %s -out_layout %s %s" % (op, t, n, c, k, hi, wi, f, f, pad, pad, stride, stride,
                                                                fl, il, ol, extra))
+
+
+def run_conv(model, rock, oracle, op, t, n, c, k, hi, wi, f, pad, layouts, stride=1, extra="", seed=0):
+    """One convolution on integer-valued data through the model; returns (kernel names, problems, result equals
+    the oracle's)."""
+    dt = _NUMPY[t]
+    rng = np.random.default_rng(seed)
+    ho, wo = (hi + 2 * pad - f) // stride + 1, (wi + 2 * pad - f) // stride + 1
+    W = rng.integers(-2, 3, k * c * f * f).astype(dt)
+    X = rng.integers(-2, 3, n * c * hi * wi).astype(dt)
+    Y = rng.integers(-2, 3, n * k * ho * wo).astype(dt)
+    opts = _conv_problem(op, t, n, c, k, hi, wi, f, pad, layouts, stride, extra)
+    fl, il, ol = layouts.split()
+    five = [fl.replace("k", "gk"), il.replace("c", "gc"), ol.replace("k", "gk")]
+    args = five + [n, 1, c, k, hi, wi, f, f]
+    kw = dict(stride=(stride, stride), pad=(pad, pad), dil=(1, 1))
+    f32 = lambda a: a.astype(np.float32)
+    if op == "conv":
+        names, problems, out = run_plan(model, rock, opts, {0: W, 1: X})
+        got, ref = out[2][:Y.nbytes], oracle.conv_fwd(f32(W), f32(X), *args, **kw)[0]
+    elif op == "conv_bwd_data":
+        names, problems, out = run_plan(model, rock, opts, {0: W, 2: Y})
+        got, ref = out[1][:X.nbytes], oracle.conv_bwd_data(f32(W), f32(Y), *args, **kw)[0]
+    else:
+        names, problems, out = run_plan(model, rock, opts, {1: X, 2: Y})
+        got, ref = out[0][:W.nbytes], oracle.conv_bwd_weight(f32(X), f32(Y), *args, **kw)[0]
+    want = np.asarray(ref).ravel().astype(dt)
+    return names, problems, np.array_equal(got.view(dt).astype(np.float64), want.astype(np.float64))
+
+
+@pytest.fixture(scope="module")
+def oracle():
+    from oracle import rock_oracle
+    return rock_oracle
 
 
 def test_the_model_notices_a_short_tensor(model, rock):
     """The input gradient of a 1x1 convolution written 16 bytes short: the last store lands on the canary."""
-    opts = _conv("conv_bwd_data", "f32", 16, 32, 32, 14, 1, 1)
-    stepped, problems = run_plan(model, rock, opts)
-    assert stepped == ["rock_conv_f32_64x64_fast"] and not problems, problems
-    stepped, problems = run_plan(model, rock, opts, shrink=(1, 16))
-    assert problems and "beside argument 1" in problems[0], problems
+    opts = _conv_problem("conv_bwd_data", "f32", 16, 32, 32, 14, 14, 1, 1, "kcyx nchw nkhw")
+    names, problems, _ = run_plan(model, rock, opts)
+    assert names[-1] == "rock_conv_f32_64x64_fast" and not problems, problems
+    names, problems, _ = run_plan(model, rock, opts, shrink=(1, 16))
+    assert problems and "beside argument 1" in problems[-1], problems
 
 
 def test_the_model_notices_a_short_operand(model, rock):
     """A GEMM operand allocated one chunk short: the direct-to-LDS load of its last chunk is out of the tensor."""
     opts = "-operation gemm -arch gfx950 -t f16 -g 1 -m 128 -n 128 -k 256"
-    stepped, problems = run_plan(model, rock, opts)
-    assert stepped and not problems, (stepped, problems)
-    stepped, problems = run_plan(model, rock, opts, shrink=(0, 16))
+    names, problems, _ = run_plan(model, rock, opts)
+    assert names and not problems, (names, problems)
+    names, problems, _ = run_plan(model, rock, opts, shrink=(0, 16))
     assert problems and "buffer load into LDS outside the tensors" in problems[0], problems
 
 
-# (operation, type, batch, c, k, image, filter, padding, layouts, stride): what the reference's backward regression
-# list runs, at batches the CPU steps through in seconds, plus forward layers over the same kernels
+@pytest.mark.parametrize("t", ["f16", "f32"])
+@pytest.mark.parametrize("shape", [(128, 128, 256, False, False), (70, 45, 100, False, True), (96, 200, 64, True, False),
+                                   (33, 17, 40, True, True), (300, 260, 72, False, True)],
+                         ids=lambda s: "%dx%dx%d%s%s" % (s[0], s[1], s[2], "-tA" if s[3] else "", "-tB" if s[4] else ""))
+def test_gemm_through_the_model_equals_numpy(model, rock, t, shape):
+    """K-contiguous and K-major operands (the transposing LDS reads), ragged tiles, operands copied into padded
+    rows first: integer-valued data, every element equal to numpy's float64 product."""
+    m, n, k, ta, tb = shape
+    dt = _NUMPY[t]
+    rng = np.random.default_rng(m + n)
+    A = rng.integers(-3, 4, (k, m) if ta else (m, k)).astype(dt)
+    B = rng.integers(-3, 4, (n, k) if tb else (k, n)).astype(dt)
+    opts = "-operation gemm -arch gfx950 -t %s -g 1 -m %d -n %d -k %d -transA %s -transB %s" % (
+        t, m, n, k, str(ta).lower(), str(tb).lower())
+    names, problems, out = run_plan(model, rock, opts, {0: A, 1: B})
+    assert not problems, (names, problems)
+    got = out[2][:m * n * np.dtype(dt).itemsize].view(dt).reshape(m, n).astype(np.float64)
+    want = (A.T if ta else A).astype(np.float64) @ (B.T if tb else B).astype(np.float64)
+    assert np.array_equal(got, want), names
+
+
+# (operation, type, batch, c, k, image, filter, padding, layouts, stride, last kernel): the kinds of plan the
+# reference's regression lists hold, at sizes the CPU runs in seconds
 _PLANS = [
-    # input gradient written channel-major by the window-resident kernel: tiles of 7 rows of 28 pixels start on
-    # odd multiples of 8 bytes in f16, so the vectors of 8 pixels would straddle images and tiles
-    ("conv_bwd_data", "f16", 4, 256, 128, 28, 3, 1, "kcyx nchw nkhw", 1),
-    ("conv_bwd_data", "f16", 4, 256, 64, 56, 3, 1, "kcyx nchw nkhw", 1),
-    ("conv_bwd_data", "f16", 4, 256, 128, 28, 3, 1, "kyxc nhwc nhwk", 1),
-    ("conv", "f16", 4, 128, 128, 28, 3, 1, "kyxc nhwc nhwk", 1),
-    ("conv", "f16", 4, 128, 128, 28, 3, 1, "kcyx nchw nkhw", 1),
-    ("conv_bwd_data", "f32", 16, 32, 32, 14, 1, 1, "kcyx nchw nkhw", 1),
-    ("conv_bwd_data", "f16", 16, 32, 32, 14, 1, 1, "kyxc nhwc nhwk", 1),
-    ("conv_bwd_weight", "f32", 16, 32, 32, 14, 1, 1, "kcyx nchw nkhw", 1),
-    ("conv_bwd_weight", "f16", 8, 64, 64, 14, 3, 1, "kyxc nhwc nhwk", 1),
-    ("conv_bwd_weight", "f16", 2, 256, 256, 56, 1, 0, "kcyx nchw nkhw", 1),
-    ("conv_bwd_data", "f16", 4, 64, 64, 56, 1, 0, "kyxc nhwc nhwk", 2),
-    ("conv_bwd_data", "f32", 4, 64, 128, 17, 3, 1, "kcyx nchw nkhw", 2),
-    ("conv_bwd_weight", "f32", 4, 64, 128, 17, 3, 1, "kyxc nhwc nhwk", 2),
-    ("conv", "f32", 4, 64, 64, 15, 3, 0, "kyxc nhwc nhwk", 1),
+    ("conv_bwd_data", "f16", 1, 128, 64, 28, 3, 1, "kcyx nchw nkhw", 1, "rock_conv_f16_64x64_fast"),
+    ("conv_bwd_data", "f16", 1, 64, 64, 28, 3, 1, "kyxc nhwc nhwk", 1, "rock_conv_f16_64x64_fast"),
+    ("conv", "f16", 1, 64, 128, 28, 3, 1, "kcyx nchw nkhw", 1, "rock_conv_f16_64x64_fast"),
+    ("conv", "f32", 2, 64, 64, 15, 3, 0, "kyxc nhwc nhwk", 1, "rock_conv_f32_64x64_fast"),
+    ("conv", "f16", 2, 24, 40, 13, 3, 1, "kcyx nhwc nkhw", 2, None),   # channel runs that are not whole chunks
+    ("conv_bwd_data", "f32", 2, 32, 32, 14, 1, 1, "kcyx nchw nkhw", 1, "rock_conv_f32_64x64_fast"),
+    ("conv_bwd_data", "f16", 2, 64, 64, 56, 1, 0, "kyxc nhwc nhwk", 2, "rock_conv_f16_64x64_fast"),   # zero fill + one phase
+    ("conv_bwd_data", "f32", 2, 64, 128, 17, 3, 1, "kcyx nchw nkhw", 2, "rock_conv_f32_64x64_fast"),  # four phases
+    ("conv_bwd_weight", "f32", 2, 32, 32, 14, 1, 1, "kcyx nchw nkhw", 1, None),
+    ("conv_bwd_weight", "f16", 2, 64, 64, 14, 3, 1, "kyxc nhwc nhwk", 1, "rock_conv_bwd_weight_f16_64x64"),
+    ("conv_bwd_weight", "f32", 2, 64, 128, 17, 3, 1, "kyxc nhwc nhwk", 2, "rock_conv_bwd_weight_f32_128x128"),
+    ("conv_bwd_weight", "f16", 2, 128, 128, 28, 1, 0, "kcyx nchw nkhw", 1, "rock_reduce_splits"),    # as a split GEMM
 ]
 
 
 @pytest.mark.parametrize("plan", _PLANS, ids=lambda p: "%s-%s-%dx%d-%d-%s" % (p[0], p[1], p[5], p[5], p[6], p[8].split()[1]))
-def test_every_address_of_the_plan_lies_in_its_tensors(model, rock, plan):
-    op, t, n, c, k, hw, f, pad, layouts, stride = plan
-    stepped, problems = run_plan(model, rock, _conv(op, t, n, c, k, hw, f, pad, layouts, stride))
-    assert stepped, "no kernel of this plan is in the model"
+def test_convolution_plans_through_the_model_equal_the_oracle(model, rock, oracle, plan):
+    op, t, n, c, k, hw, f, pad, layouts, stride, last = plan
+    names, problems, equal = run_conv(model, rock, oracle, op, t, n, c, k, hw, hw, f, pad, layouts, stride)
+    assert not problems, (names, problems)
+    assert last is None or names[-1] == last, names
+    assert equal, names
+
+
+_WINDOW = "-perf_config v2:224,128,8,224,32,8,1,1,1"
+
+
+@pytest.mark.parametrize("case", [
+    # pixels-last output: whole rows of channels
+    (2, 128, 128, 28, 28, "kyxc nhwc nhwk"),
+    # channel-major output, 7 x 28-pixel tiles would start inside a 16-byte vector of pixels: the planner takes
+    # four rows per tile, whole vectors
+    (2, 128, 128, 28, 28, "kyxc nhwc nkhw"),
+    # no tile height gives whole vectors (windows of at most three rows of 14 pixels x 512 channels): the kernel
+    # stores element by element
+    (2, 512, 128, 16, 14, "kyxc nhwc nkhw"),
+], ids=["rows", "pixel-vectors", "pixel-vectors-misaligned"])
+def test_window_resident_kernel_through_the_model(model, rock, oracle, case):
+    """The window-resident kernel on request, its three ways of storing a tile."""
+    n, c, k, hi, wi, layouts = case
+    names, problems, equal = run_conv(model, rock, oracle, "conv", "f16", n, c, k, hi, wi, 3, 1, layouts, extra=_WINDOW)
+    assert names == ["rock_relayout_b2", "rock_conv_f16_direct224"], names
     assert not problems, problems
+    assert equal
