@@ -52,10 +52,16 @@ __device__ __forceinline__ float other_half(float x) {
 // write of its operands and before a VALU read of its results, which the
 // compiler's hazard pass cannot see inside an asm block.
 __device__ __forceinline__ void both_halves(float x, float &lo, float &hi) {
+#ifdef __AMDGCN__
   float a = x, b = x;
   asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
   lo = a;
   hi = b;
+#else // (the CPU build of the kernels that the tests run: the same two values through the cross-lane read)
+  const int lane = (int)(threadIdx.x & 63);
+  lo = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane & 31) << 2, __builtin_bit_cast(int, x)));
+  hi = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane | 32) << 2, __builtin_bit_cast(int, x)));
+#endif
 }
 __device__ __forceinline__ float half_swap_max_fast(float x) {
   float lo, hi;

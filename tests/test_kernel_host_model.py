@@ -37,6 +37,7 @@ pytestmark = pytest.mark.skipif(CLANG is None, reason="the host build uses clang
 _TYPES = {0: "f32", 1: "f16"}
 # every kernel but the twins with the rolled epilogue ("_e": same loads, same tiles, their own store code)
 _LEFT_OUT = ("_e",)
+_ATTENTION = True   # the fused attention kernels too
 _DTYPE_BYTES = {0: 4, 1: 2, 2: 2, 3: 1, 4: 1, 5: 1, 6: 4}
 
 
@@ -88,6 +89,25 @@ def _utility_source():
     return "\n".join(lines) + "\n"
 
 
+def _attention_sources(parts=4):
+    """The fused attention kernels (csrc/attention_kernels.h): Q, K, V, scale tensor, bias, mask, other, O."""
+    kernels = _build.attention_kernels()
+    units = {}
+    for part in range(parts):
+        mine = kernels[part::parts]
+        lines = ['#include "attention_kernels.h"', '#include "kernel_table.h"', "#include <cstring>"]
+        lines += [m for _, m in mine]
+        for n, _ in mine:
+            lines.append("static void call_%s(void **q, const void *params) { RockAttentionParams p; "
+                         "std::memcpy(&p, params, sizeof p); %s(q[0], q[1], q[2], q[3], q[4], q[5], q[6], q[7], p); }"
+                         % (n, n))
+        lines.append("static const HmEntry table[] = {")
+        lines += ['  {"%s", call_%s},' % (n, n) for n, _ in mine]
+        lines += ["  {nullptr, nullptr}};", "const HmEntry *hm_table_attention_%d() { return table; }" % part]
+        units["model_attention_%d" % part] = "\n".join(lines) + "\n"
+    return units
+
+
 def _table_source(tables):
     lines = ['#include "kernel_table.h"', "#include <vector>"]
     lines += ["const HmEntry *%s();" % t for t in tables]
@@ -102,6 +122,8 @@ def build_model(d):
     units = {"model_utility": _utility_source()}
     for code in _TYPES:
         units.update(_model_sources(code))
+    if _ATTENTION:
+        units.update(_attention_sources())
     units["kernel_table"] = _table_source(["hm_table_" + n[len("model_"):] for n in units])
     for name, text in units.items():
         with open(os.path.join(d, name + ".cpp"), "w") as f:
@@ -320,3 +342,51 @@ def test_window_resident_kernel_through_the_model(model, rock, oracle, case):
     assert names == ["rock_relayout_b2", "rock_conv_f16_direct224"], names
     assert not problems, problems
     assert equal
+
+
+def _attention_problem(t, G, sq, sk, dqk, dv, trans_k, scale, extra=""):
+    return ("-operation attention -arch gfx950 -t %s -g %d -seq_len_q %d -seq_len_k %d -head_dim_qk %d -head_dim_v %d "
+            "-transQ false -transK %s -transV false -transO false -scale %.9g %s"
+            % (t, G, sq, sk, dqk, dv, "true" if trans_k else "false", scale, extra))
+
+
+@pytest.mark.parametrize("case", [
+    # (type, heads, seq_q, seq_k, d_qk, d_v, K stored [seq_k][d], scale tensor, bias, last kernel)
+    ("f16", 2, 128, 96, 64, 64, True, False, False, "rock_attention_f16_d64x64_fast"),
+    ("f16", 1, 160, 200, 128, 128, False, False, False, "rock_attention_f16_d128x128_fast_kt"),
+    ("f16", 2, 128, 27, 64, 32, True, True, True, "rock_attention_f16_d64x64_fast_bias"),
+    ("f16", 1, 64, 128, 256, 256, True, False, False, "rock_attention_f16_d256x256_fast_bias"),
+    ("f32", 2, 70, 45, 64, 64, True, False, True, "rock_gemm_f32_64x64_generic"),   # three kernels around the row softmax
+], ids=["d64", "d128-keys-as-stored", "scale-tensor-bias-cross", "d256", "f32-three-kernels"])
+def test_attention_through_the_model_passes_the_gates(model, rock, oracle, case):
+    """The fused kernels (and the three-kernel form) on real-valued data through the model, under the gates of the
+    GPU tests: RMS 1e-3 and maximum difference 0.02 for f16, 3e-5 and 1e-4 for f32."""
+    from tests.gpu_util import check_float
+    t, G, sq, sk, dqk, dv, trans_k, with_scale, with_bias, last = case
+    dt = _NUMPY[t]
+    rng = np.random.default_rng(sq + sk)
+    Q = (rng.standard_normal((G, sq, dqk)) * 0.5).astype(dt)
+    K = (rng.standard_normal((G, sk, dqk) if trans_k else (G, dqk, sk)) * 0.5).astype(dt)
+    V = rng.standard_normal((G, sk, dv)).astype(dt)
+    St = (rng.random((G, sq, sk)) * 0.5 + 0.75).astype(dt) if with_scale else None
+    Bt = (rng.standard_normal((G, sq, sk)) * 0.5).astype(dt) if with_bias else None
+    scale = 1.0 / np.sqrt(dqk)
+    opts = _attention_problem(t, G, sq, sk, dqk, dv, trans_k, scale,
+                              ("-with-attn-scale true " if with_scale else "") + ("-with-attn-bias true" if with_bias else ""))
+    # caller list: Q, K, V, [scale tensor], bias, O, [workspace]
+    inputs = {0: Q, 1: K, 2: V}
+    at = 3
+    if with_scale:
+        inputs[at] = St
+        at += 1
+    if with_bias:
+        inputs[at] = Bt
+    names, problems, out = run_plan(model, rock, opts, inputs)
+    assert not problems, (names, problems)
+    assert names[-1] == last, names
+    got = out[at + 1][:G * sq * dv * np.dtype(dt).itemsize].view(dt).astype(np.float32)
+    f32 = lambda a: None if a is None else a.astype(np.float32)
+    ref = oracle.attention(f32(Q), f32(K), f32(V), G, sq, sk, dqk, dv, scale=scale, scale_t=f32(St), bias_t=f32(Bt),
+                           transK=trans_k)
+    gate = {"f16": (1e-3, 0.02), "f32": (3e-5, 1e-4)}[t]
+    check_float(got, ref, t, rms=gate[0], max_abs=gate[1])
