@@ -11,6 +11,10 @@
 // operations by itself) meet at RK_WAVE_LDS_ORDER(), which the kernels' sources
 // place there and which is empty on the GPU.
 //
+// A load into LDS lands either when it is issued or, with hm_set_late_loads(1), not before the wait that covers
+// it (vmcnt): the two extremes of what the hardware may do.  A kernel that reads a stage too early fails under the
+// second, one that refills a stage too early under the first.
+//
 // Buffer loads are checked against the registered tensors (the runner's
 // hm_alloc) the way the hardware checks them against the descriptor's range;
 // plain loads and stores run into canary and guard pages around the tensors,
@@ -53,9 +57,10 @@ void hm_block_sync(); // returns when every live thread of the block has called 
 #define RK_WAVE_LDS_ORDER() hm_wave_sync()
 #define __builtin_amdgcn_s_barrier() hm_block_sync()
 #define __syncthreads() hm_block_sync()
-// (loads into LDS complete when issued here, so there is nothing to count; the wave meets where it would wait
-// for its loads, so that behind a wait every lane's loads have been issued)
-#define __builtin_amdgcn_s_waitcnt(x) hm_wave_sync()
+// A wait for loads: the lane's loads into LDS beyond the count the instruction allows to stay in flight land (see
+// hm_set_late_loads in runner.cpp), then the wave meets, so that behind a wait every lane's loads are in LDS.
+void hm_waitcnt(int immediate);
+#define __builtin_amdgcn_s_waitcnt(x) hm_waitcnt(x)
 #define __builtin_amdgcn_sched_group_barrier(a, b, c) ((void)0)
 
 // ---- buffer descriptors: base and range (raw buffers, no stride, no swizzle) -----

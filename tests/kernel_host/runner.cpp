@@ -64,11 +64,18 @@ void on_trap(int sig, siginfo_t *si, void *) {
 
 // ---- one block as cooperative fibers ---------------------------------------------
 enum State { kRun, kWaitWave, kWaitBlock, kDone };
+struct PendingLoad { // a load into LDS that has been issued and has not landed
+  char *dst;
+  int size;
+  char data[16];
+};
 struct Fiber {
   ucontext_t ctx;
   State state;
   unsigned ops; // cross-lane operations begun: picks the half of the exchange area
+  std::vector<PendingLoad> pending;
 };
+bool late_loads = false;
 constexpr size_t kStack = 512 * 1024;
 constexpr unsigned kMaxThreads = 1024;
 Fiber *fibers = nullptr;
@@ -105,6 +112,7 @@ void run_block() {
     makecontext(&fibers[t].ctx, fiber_main, 0);
     fibers[t].state = kRun;
     fibers[t].ops = 0;
+    fibers[t].pending.clear();
   }
   for (;;) {
     bool ran = false;
@@ -207,15 +215,30 @@ int elem_bytes(int type) { return type == HM_F32 ? 4 : (type == HM_F16 || type =
 } // namespace
 
 void hm_load_lds(HmRsrc r, void *lds, int size, int voff, int soff, int ioff, int) {
-  char *dst = (char *)lds + lane_id() * size; // the wave's lanes land back to back
+  PendingLoad load;
+  load.dst = (char *)lds + lane_id() * size; // the wave's lanes land back to back
+  load.size = size;
+  std::memset(load.data, 0, sizeof load.data);
   const uint64_t off = (uint64_t)(unsigned)voff + (unsigned)ioff;
-  if (off >= r.num_records || off + (unsigned)soff >= r.num_records) {
-    std::memset(dst, 0, size);
-    return;
+  if (off < r.num_records && off + (unsigned)soff < r.num_records) {
+    const char *src = r.base + off + (unsigned)soff;
+    hm_check_global(src, size, "buffer load into LDS");
+    std::memcpy(load.data, src, size);
   }
-  const char *src = r.base + off + (unsigned)soff;
-  hm_check_global(src, size, "buffer load into LDS");
-  std::memcpy(dst, src, size);
+  if (late_loads)
+    fibers[current].pending.push_back(load);
+  else
+    std::memcpy(load.dst, load.data, size);
+}
+void hm_waitcnt(int immediate) {
+  // gfx9 encoding: vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits 15:14
+  const size_t allowed = (size_t)((immediate & 0xF) | (((immediate >> 14) & 3) << 4));
+  auto &q = fibers[current].pending;
+  size_t land = q.size() > allowed ? q.size() - allowed : 0;
+  for (size_t i = 0; i < land; ++i)
+    std::memcpy(q[i].dst, q[i].data, q[i].size);
+  q.erase(q.begin(), q.begin() + land);
+  wait_as(kWaitWave);
 }
 hm_v4i hm_load_b128(HmRsrc r, int voff, int soff, int) {
   hm_v4i v = {0, 0, 0, 0};
@@ -324,6 +347,8 @@ void hm_mfma_32x32(int type_a, int type_b, const void *a, const void *b, int lan
 }
 
 extern "C" {
+// 0: loads into LDS land when issued; 1: not before the wait that covers them
+void hm_set_late_loads(int on) { late_loads = on != 0; }
 void hm_clear() {
   for (auto &r : ranges) {
     const size_t body = ((size_t)(r.hi - r.lo) + kPage - 1) / kPage * kPage + 2 * kPage;

@@ -148,12 +148,22 @@ def build_model(d):
     lib.hm_knows.argtypes = [C.c_char_p]
     lib.hm_run.restype = C.c_long
     lib.hm_run.argtypes = [C.c_char_p, C.c_char_p, C.POINTER(C.c_void_p), C.c_uint, C.c_uint, C.c_char_p, C.c_size_t]
+    lib.hm_set_late_loads.argtypes = [C.c_int]
     return lib
 
 
 @pytest.fixture(scope="module")
 def model(tmp_path_factory):
     return build_model(str(tmp_path_factory.mktemp("kernel_host")))
+
+
+@pytest.fixture(params=["loads-land-at-issue", "loads-land-at-the-wait"])
+def loads(request, model):
+    """The two extremes of when a load into LDS may land: a kernel that reads a stage before its wait fails
+    under the second, one that refills a stage that is still being read under the first."""
+    model.hm_set_late_loads(1 if request.param == "loads-land-at-the-wait" else 0)
+    yield request.param
+    model.hm_set_late_loads(0)
 
 
 @pytest.fixture(scope="module")
@@ -278,7 +288,7 @@ def test_the_model_notices_a_short_operand(model, rock):
 @pytest.mark.parametrize("shape", [(128, 128, 256, False, False), (70, 45, 100, False, True), (96, 200, 64, True, False),
                                    (33, 17, 40, True, True), (300, 260, 72, False, True)],
                          ids=lambda s: "%dx%dx%d%s%s" % (s[0], s[1], s[2], "-tA" if s[3] else "", "-tB" if s[4] else ""))
-def test_gemm_through_the_model_equals_numpy(model, rock, t, shape):
+def test_gemm_through_the_model_equals_numpy(model, rock, loads, t, shape):
     """K-contiguous and K-major operands (the transposing LDS reads), ragged tiles, operands copied into padded
     rows first: integer-valued data, every element equal to numpy's float64 product."""
     m, n, k, ta, tb = shape
@@ -314,7 +324,7 @@ _PLANS = [
 
 
 @pytest.mark.parametrize("plan", _PLANS, ids=lambda p: "%s-%s-%dx%d-%d-%s" % (p[0], p[1], p[5], p[5], p[6], p[8].split()[1]))
-def test_convolution_plans_through_the_model_equal_the_oracle(model, rock, oracle, plan):
+def test_convolution_plans_through_the_model_equal_the_oracle(model, rock, oracle, loads, plan):
     op, t, n, c, k, hw, f, pad, layouts, stride, last = plan
     names, problems, equal = run_conv(model, rock, oracle, op, t, n, c, k, hw, hw, f, pad, layouts, stride)
     assert not problems, (names, problems)
@@ -335,7 +345,7 @@ _WINDOW = "-perf_config v2:224,128,8,224,32,8,1,1,1"
     # stores element by element
     (2, 512, 128, 16, 14, "kyxc nhwc nkhw"),
 ], ids=["rows", "pixel-vectors", "pixel-vectors-misaligned"])
-def test_window_resident_kernel_through_the_model(model, rock, oracle, case):
+def test_window_resident_kernel_through_the_model(model, rock, oracle, loads, case):
     """The window-resident kernel on request, its three ways of storing a tile."""
     n, c, k, hi, wi, layouts = case
     names, problems, equal = run_conv(model, rock, oracle, "conv", "f16", n, c, k, hi, wi, 3, 1, layouts, extra=_WINDOW)
@@ -358,7 +368,7 @@ def _attention_problem(t, G, sq, sk, dqk, dv, trans_k, scale, extra=""):
     ("f16", 1, 64, 128, 256, 256, True, False, False, "rock_attention_f16_d256x256_fast_bias"),
     ("f32", 2, 70, 45, 64, 64, True, False, True, "rock_gemm_f32_64x64_generic"),   # three kernels around the row softmax
 ], ids=["d64", "d128-keys-as-stored", "scale-tensor-bias-cross", "d256", "f32-three-kernels"])
-def test_attention_through_the_model_passes_the_gates(model, rock, oracle, case):
+def test_attention_through_the_model_passes_the_gates(model, rock, oracle, loads, case):
     """The fused kernels (and the three-kernel form) on real-valued data through the model, under the gates of the
     GPU tests: RMS 1e-3 and maximum difference 0.02 for f16, 3e-5 and 1e-4 for f32."""
     from tests.gpu_util import check_float
