@@ -76,6 +76,8 @@ struct Fiber {
   std::vector<PendingLoad> pending;
 };
 bool late_loads = false;
+int thread_order = 0;
+unsigned pass_seed = 12345;
 constexpr size_t kStack = 512 * 1024;
 constexpr unsigned kMaxThreads = 1024;
 Fiber *fibers = nullptr;
@@ -116,13 +118,23 @@ void run_block() {
   }
   for (;;) {
     bool ran = false;
-    for (unsigned t = 0; t < threads; ++t)
+    const unsigned waves = (threads + 63) / 64;
+    const unsigned shift = thread_order == 2 ? (pass_seed = pass_seed * 1664525u + 1013904223u) >> 16 : 0;
+    for (unsigned i = 0; i < threads; ++i) {
+      // the order in which the threads get their turn: ascending, descending, or the waves rotated by a
+      // different amount in every pass (no result may depend on it)
+      unsigned t = thread_order == 1 ? threads - 1 - i : i;
+      if (thread_order == 2)
+        t = ((i / 64 + shift) % waves) * 64 + i % 64;
+      if (t >= threads)
+        continue;
       if (fibers[t].state == kRun) {
         current = t;
         threadIdx = {t, 0, 0};
         swapcontext(&scheduler, &fibers[t].ctx);
         ran = true;
       }
+    }
     // a wave goes on when all its live lanes wait for each other, the block when all its live threads do
     bool released = false;
     unsigned done = 0, at_barrier = 0;
@@ -349,6 +361,8 @@ void hm_mfma_32x32(int type_a, int type_b, const void *a, const void *b, int lan
 extern "C" {
 // 0: loads into LDS land when issued; 1: not before the wait that covers them
 void hm_set_late_loads(int on) { late_loads = on != 0; }
+// the order in which a block's threads take their turns: 0 ascending, 1 descending, 2 waves rotated per pass
+void hm_set_thread_order(int order) { thread_order = order; }
 void hm_clear() {
   for (auto &r : ranges) {
     const size_t body = ((size_t)(r.hi - r.lo) + kPage - 1) / kPage * kPage + 2 * kPage;

@@ -149,6 +149,7 @@ def build_model(d):
     lib.hm_run.restype = C.c_long
     lib.hm_run.argtypes = [C.c_char_p, C.c_char_p, C.POINTER(C.c_void_p), C.c_uint, C.c_uint, C.c_char_p, C.c_size_t]
     lib.hm_set_late_loads.argtypes = [C.c_int]
+    lib.hm_set_thread_order.argtypes = [C.c_int]
     return lib
 
 
@@ -160,10 +161,15 @@ def model(tmp_path_factory):
 @pytest.fixture(params=["loads-land-at-issue", "loads-land-at-the-wait"])
 def loads(request, model):
     """The two extremes of when a load into LDS may land: a kernel that reads a stage before its wait fails
-    under the second, one that refills a stage that is still being read under the first."""
-    model.hm_set_late_loads(1 if request.param == "loads-land-at-the-wait" else 0)
+    under the second, one that refills a stage that is still being read under the first.  The threads of a
+    block take their turns in ascending order under the first and with the waves rotated from pass to pass
+    under the second: no result may depend on which wave runs first."""
+    late = request.param == "loads-land-at-the-wait"
+    model.hm_set_late_loads(1 if late else 0)
+    model.hm_set_thread_order(2 if late else 0)
     yield request.param
     model.hm_set_late_loads(0)
+    model.hm_set_thread_order(0)
 
 
 @pytest.fixture(scope="module")
