@@ -406,3 +406,74 @@ def test_attention_through_the_model_passes_the_gates(model, rock, oracle, loads
                            transK=trans_k)
     gate = {"f16": (1e-3, 0.02), "f32": (3e-5, 1e-4)}[t]
     check_float(got, ref, t, rms=gate[0], max_abs=gate[1])
+
+
+# ---- the reference's end-to-end lists, by the harness of tests/test_gpu_e2e_lists.py with the model as the device ---
+def _conv_macs(o):
+    g = int(o.get("groupsize", 1))
+    n, c, k = int(o["batchsize"]), int(o["in_channels"]) // g, int(o["out_channels"]) // g
+    y, x = int(o["fil_h"]), int(o["fil_w"])
+    ph, pw = int(o.get("padding_h", 0)), int(o.get("padding_w", 0))
+    ho = (int(o["in_h"]) + int(o.get("padding_h_l", ph)) + int(o.get("padding_h_r", ph))
+          - (y - 1) * int(o.get("dilation_h", 1)) - 1) // int(o.get("conv_stride_h", 1)) + 1
+    wo = (int(o["in_w"]) + int(o.get("padding_w_l", pw)) + int(o.get("padding_w_r", pw))
+          - (x - 1) * int(o.get("dilation_w", 1)) - 1) // int(o.get("conv_stride_w", 1)) + 1
+    return n * g * c * k * ho * wo * y * x
+
+
+def _listed(name, every, macs=1.5e7):
+    """Every `every`-th problem of a list, batches capped at 2, convolutions within `macs` multiply-adds."""
+    import re
+    import tests.test_gpu_e2e_lists as lists
+    out = []
+    for i, opts in enumerate(lists._BY_LIST[name]):
+        if i % every:
+            continue
+        opts = re.sub(r"-batchsize[= ](\d+)", lambda m: "-batchsize=%d" % min(int(m.group(1)), 2), opts)
+        o = lists.parse_options(opts)
+        if "conv" in o.get("operation", "") and _conv_macs(o) > macs:
+            continue
+        out.append((i, opts, o))
+    return out
+
+
+@pytest.mark.parametrize("name,every", [("conv_regression_bwd.toml", 6), ("conv_regression_fwd.toml", 15),
+                                        ("PrAttentionF16.toml", 1), ("PrAttentionI8.toml", 2), ("PrAttentionF32.toml", 2),
+                                        ("gemm_split_k_f16.toml", 3), ("gemm_split_k_f32.toml", 3)])
+def test_reference_lists_through_the_model(model, rock, oracle, name, every):
+    """Lists that have not run on a GPU (or not since the harness changed), through the same harness: its
+    RockProgram is one that runs the plan on the model, its tensors live on the CPU."""
+    import torch
+    import tests.test_gpu_e2e_lists as lists
+
+    class Program:
+        def __init__(self, opts):
+            self.opts = opts
+            first = rock.RockKernel(opts)
+            self.kernels = [first] + [rock.RockKernel("%s --kernel_id %d" % (opts, i)) for i in range(1, first.kernel_count)]
+
+        def launch(self, *args):
+            inputs = {i: a.contiguous().view(torch.uint8).numpy() for i, a in enumerate(args) if a is not None}
+            names, problems, out = run_plan(model, rock, self.opts, inputs)
+            assert not problems, (self.opts, names, problems)
+            for i, a in enumerate(args):
+                if a is not None:
+                    flat = a.view(torch.uint8).view(-1)
+                    flat.copy_(torch.from_numpy(out[i][:flat.numel()].copy()))
+
+    class Device:
+        RockProgram = Program
+
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(1234)
+    ran = 0
+    for i, opts, o in _listed(name, every):
+        try:
+            rock.RockKernel(opts)
+        except rock.RockError:
+            continue   # (the twelve stated refusals: backward convolutions with unequal padding)
+        op = o.get("operation", "")
+        run = lists.run_gemm if op == "gemm" else lists.run_attention if op == "attention" else lists.run_conv
+        run(Device, oracle, "cpu", gen, opts, o)
+        ran += 1
+    assert ran >= 2, ran
