@@ -232,9 +232,11 @@ def run_attention(rock, oracle, gpu, gen, opts, o):
 
 
 # Lists that are held back, with the reason.  The nine others ran and passed (1849 problems).
-_NOT_RUN = "not yet run on a GPU: the only run that reached it came after that run's GPU fault"
+_NOT_RUN = ("not yet run on a GPU: the only run that reached it came after that run's GPU fault (on the CPU build of the "
+            "kernels, tests/test_kernel_host_model.py, the whole list passes this harness)")
 _ATTN_FIXED = ("its first run stopped at this harness's own assertion that the lists hold no -with-attn-scale problem (they "
-               "do); the harness now passes the scale tensor and the bias, and the list has not run on a GPU since")
+               "do); the harness now passes the scale tensor and the bias, and the list has not run on a GPU since (on the "
+               "CPU build of the kernels, tests/test_kernel_host_model.py, every problem passes)")
 _HELD_BACK = {
     "conv_regression_bwd.toml": (
         "its first run ended in a GPU memory fault about 0.26 s into the list (illegal memory access, reported at "
@@ -243,7 +245,7 @@ _HELD_BACK = {
         "step through their host-compiled body against guard pages, and so do the contraction kernels "
         "(tests/test_kernel_host_model.py) -- which found one defect in this list, misplaced 16-byte stores of the "
         "window-resident kernel into channel-major outputs 28 pixels wide (wrong values inside the tensor, fixed), "
-        "but no access outside a tensor.  What the list has that no passing list has is backward convolutions with "
+        "but no access outside a tensor, and with the kernels computing there the whole list passes this harness.  What the list has that no passing list has is backward convolutions with "
         "unequal left and right padding, which the planner refuses again.  Not to be run on a GPU before the cause "
         "is shown."),
     "PrAttentionF16.toml": _ATTN_FIXED,
