@@ -6,6 +6,7 @@
 #include "hip/hip_runtime.h"
 #include "kernel_table.h"
 #include <csignal>
+#include <ctime>
 #include <string>
 #include <sys/mman.h>
 #include <sys/wait.h>
@@ -176,6 +177,8 @@ void hm_wave_sync() { wait_as(kWaitWave); }
 void hm_block_sync() { wait_as(kWaitBlock); }
 
 void hm_check_global(const void *p, size_t n, const char *what) {
+  if (ranges.empty()) // (a caller that runs in its own memory: hm_run_direct)
+    return;
   const char *c = (const char *)p;
   for (auto &r : ranges)
     if (c >= r.lo && c + n <= r.hi)
@@ -400,6 +403,35 @@ int hm_knows(const char *name) {
     if (!std::strcmp(e->name, name))
       return 1;
   return 0;
+}
+// The same in the calling process, for a caller whose tensors are its own memory (nothing is registered then, and
+// buffer loads are not range-checked; a trap ends the caller).  Returns -3 when the launch has not finished
+// after `seconds` of wall time (0: no limit).
+long hm_run_direct(const char *name, const void *params, void **pointers, unsigned grid, unsigned block, int seconds) {
+  void (*fn)(void **, const void *) = nullptr;
+  for (const HmEntry *e = hm_kernel_table(); e->name; ++e)
+    if (!std::strcmp(e->name, name))
+      fn = e->fn;
+  if (!fn)
+    return -1;
+  static Report local;
+  report = &local;
+  std::memset(report, 0, sizeof *report);
+  cur_kernel = name;
+  gridDim = {grid, 1, 1};
+  blockDim = {block, 1, 1};
+  kernel_fn = fn;
+  kernel_pointers = pointers;
+  kernel_params = params;
+  threads = block;
+  const time_t start = time(nullptr);
+  for (unsigned b = 0; b < grid; ++b) {
+    blockIdx = {b, 0, 0};
+    run_block();
+    if (seconds > 0 && time(nullptr) - start > seconds)
+      return -3;
+  }
+  return report->violations;
 }
 // Runs every block of the launch, one after the other.  Returns the number of accesses outside the tensors (-1: no such
 // kernel in this build, -2: the child could not be started); `first` receives a description of the first one.
