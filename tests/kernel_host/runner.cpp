@@ -78,6 +78,7 @@ struct Fiber {
 };
 bool late_loads = false;
 int thread_order = 0;
+unsigned first_block = 0, block_limit = ~0u; // the blocks of a launch that run
 unsigned pass_seed = 12345;
 constexpr size_t kStack = 512 * 1024;
 constexpr unsigned kMaxThreads = 1024;
@@ -367,6 +368,11 @@ extern "C" {
 void hm_set_late_loads(int on) { late_loads = on != 0; }
 // the order in which a block's threads take their turns: 0 ascending, 1 descending, 2 waves rotated per pass
 void hm_set_thread_order(int order) { thread_order = order; }
+// only blocks [first, first + count) of every launch run (a problem too large to run whole: its last tiles)
+void hm_set_blocks(unsigned first, unsigned count) {
+  first_block = first;
+  block_limit = count;
+}
 void hm_clear() {
   for (auto &r : ranges) {
     const size_t body = ((size_t)(r.hi - r.lo) + kPage - 1) / kPage * kPage + 2 * kPage;
@@ -426,7 +432,7 @@ long hm_run_direct(const char *name, const void *params, void **pointers, unsign
   kernel_params = params;
   threads = block;
   const time_t start = time(nullptr);
-  for (unsigned b = 0; b < grid; ++b) {
+  for (unsigned b = first_block; b < grid && b - first_block < block_limit; ++b) {
     blockIdx = {b, 0, 0};
     if (!run_block())
       break;
@@ -472,7 +478,7 @@ long hm_run(const char *name, const void *params, void **pointers, unsigned grid
     kernel_pointers = pointers;
     kernel_params = params;
     threads = block;
-    for (unsigned b = 0; b < grid; ++b) {
+    for (unsigned b = first_block; b < grid && b - first_block < block_limit; ++b) {
       blockIdx = {b, 0, 0};
       if (!run_block())
         break;

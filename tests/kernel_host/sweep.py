@@ -7,6 +7,7 @@ oracle (tests/test_gpu_e2e_lists.py with the model as its device).  Run from the
   ... --types all --rolled    every operand type and the rolled-epilogue kernels (ten minutes of compilation,
                               kept in --build-dir and used again while the sources are unchanged)
   ... --late --order 2        loads land at the wait that covers them, waves take their turns rotated
+  python -m tests.kernel_host.sweep --boundary                  # tensors just below and at 2 GiB, their last tiles only
 
 One line per problem: ok / FAIL / refused, the kernels that ran, the options string to run it again."""
 import argparse
@@ -144,6 +145,88 @@ def check(device, opts, gen, have):
         return "FAIL %r" % (e,)
 
 
+def _last_tiles(model, opts, fill, blocks, order_at):
+    """Runs the last `blocks` blocks of every kernel of the plan, the tiles taken in plain order (order_at: byte
+    offset of group_m in the contraction kernel's parameter block, checked against the sizes in front of it)."""
+    import ctypes as C
+    import struct
+    import numpy as np
+    first = rock.RockKernel(opts)
+    kernels = [first] + [rock.RockKernel("%s --kernel_id %d" % (opts, i)) for i in range(1, first.kernel_count)]
+    model.hm_clear()
+    tensors = []
+    for i, (dt, dims) in enumerate(first.arguments()):
+        nbytes = max(int(np.prod(dims, dtype=np.int64)) * (1 if dt < 0 else km._DTYPE_BYTES[dt]), 16)
+        at = model.hm_alloc(nbytes, b"argument %d" % i)
+        tensors.append((at, nbytes, np.ctypeslib.as_array((C.c_uint8 * nbytes).from_address(at))))
+    fill([v for _, _, v in tensors])
+    problems = []
+    for k in kernels:
+        params = bytearray(k.params())
+        if k.kernel_name.startswith(("rock_conv_", "rock_gemm_")):
+            tiles_m, tiles_n = struct.unpack_from("<2i", params, order_at - 8)
+            assert tiles_m * tiles_n in (k.grid_size, k.grid_size // max(1, struct.unpack_from("<i", params, 72)[0])), \
+                "the parameter block is not laid out as this probe assumes"
+            struct.pack_into("<2i", params, order_at, 1, 0)   # group_m = 1, xcd_remap = 0
+        ptrs = (C.c_void_p * 8)()
+        for j, (src, off) in enumerate(km.pointer_map(rock, k)):
+            ptrs[j] = None if src < 0 else tensors[src][0] + off
+        model.hm_set_blocks(max(0, k.grid_size - blocks), blocks)
+        text = C.create_string_buffer(512)
+        bad = model.hm_run(k.kernel_name.encode(), bytes(params), ptrs, k.grid_size, k.block_size, text, 512)
+        model.hm_set_blocks(0, 0xFFFFFFFF)
+        if bad:
+            problems.append("%s: %s" % (k.kernel_name, text.value.decode()))
+        problems += ["%s wrote beside argument %d" % (k.kernel_name, i) for i, (at, n, _) in enumerate(tensors)
+                     if model.hm_canaries(at, n)]
+    return [k.kernel_name for k in kernels], problems, [v for _, _, v in tensors]
+
+
+def boundary(model):
+    """The direct-to-LDS loads address a 2 GiB window behind a base pointer, and the planners send a tensor that
+    does not fit to the kernels with 64-bit addressing: a convolution input and a K-major GEMM operand of just
+    under and of exactly 2 GiB, the last tiles of each (highest offsets), results against the oracle / numpy."""
+    import numpy as np
+    bad = 0
+    rng = np.random.default_rng(0)
+    c = k = 64
+    hw, f = 16, 3
+    img = hw * hw * c
+    W = rng.integers(-2, 3, k * c * f * f).astype(np.float16)
+    X3 = rng.integers(-2, 3, 3 * img).astype(np.float16)   # the last three images hold data, the rest zeros
+    ref = rock_oracle.conv_fwd(W.astype(np.float32), X3.astype(np.float32), "gkyxc", "nhwgc", "nhwgk", 3, 1, c, k, hw, hw,
+                               f, f, stride=(1, 1), pad=(1, 1), dil=(1, 1))[0]
+    ref = np.asarray(ref).reshape(3, hw * hw * k)[2].astype(np.float16)
+    for n, expect in ((65534, "rock_conv_f16_64x64_fast"), (65536, "rock_conv_f16_64x64_generic")):
+        opts = CONV % (1, n, c, k, hw, hw, f, f, 1, 1, 1, 1, 1, 1, 1, 1, "conv", "kyxc", "nhwc", "nhwk", "f16")
+
+        def fill(t):
+            t[0][:W.nbytes] = W.view(np.uint8)
+            t[1][:] = 0
+            t[1][(n - 3) * img * 2:n * img * 2] = X3.view(np.uint8)
+        names, problems, out = _last_tiles(model, opts, fill, 8, 204)
+        got = out[2][(n - 1) * hw * hw * k * 2:n * hw * hw * k * 2].view(np.float16)
+        ok = names[-1] == expect and not problems and np.array_equal(got.astype(np.float32), ref.astype(np.float32))
+        bad += not ok
+        print("convolution input of %d bytes:" % (n * img * 2), "ok" if ok else "FAIL", names, problems, flush=True)
+    M, K = 64, 32768
+    A = rng.integers(-2, 3, (M, K)).astype(np.float16)
+    for N, expect in ((32760, "rock_gemm_f16_64x64_fast_nn"), (32768, "rock_gemm_f16_64x64_generic")):
+        B = rng.integers(-2, 3, (K, N), dtype=np.int8).astype(np.float16)
+        opts = "-operation gemm -arch gfx950 -t f16 -g 1 -m %d -n %d -k %d -transA false -transB false" % (M, N, K)
+
+        def fill(t):
+            t[0][:A.nbytes] = A.view(np.uint8).ravel()
+            t[1][:B.nbytes] = B.view(np.uint8).ravel()
+        names, problems, out = _last_tiles(model, opts, fill, 2, 96)
+        got = out[2][:M * N * 2].view(np.float16).reshape(M, N)[:, -64:].astype(np.float64)
+        want = A.astype(np.float64) @ B[:, -64:].astype(np.float64)
+        ok = names[-1] == expect and not problems and np.array_equal(got, want)
+        bad += not ok
+        print("GEMM operand of %d bytes:" % B.nbytes, "ok" if ok else "FAIL", names, problems, flush=True)
+    return bad
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--lists", default="", help="comma-separated list names of tests/golden/e2e_problems.json, or all")
@@ -156,6 +239,7 @@ def main():
     ap.add_argument("--rolled", action="store_true", help="build the rolled-epilogue kernels too")
     ap.add_argument("--late", action="store_true", help="loads into LDS land at the wait that covers them")
     ap.add_argument("--order", type=int, default=0, help="0 ascending, 1 descending, 2 waves rotated per pass")
+    ap.add_argument("--boundary", action="store_true", help="tensors just below and at 2 GiB (needs about 10 GB of memory)")
     ap.add_argument("--build-dir", default=os.path.join(os.environ.get("TMPDIR", "/tmp"), "rock_kernel_host"))
     a = ap.parse_args()
     names = {v: k for k, v in km._build.GEMM_TYPES.items()}
@@ -174,7 +258,7 @@ def main():
     for t in types:
         have |= set(km._build.GEMM_TYPES[t].split("_"))
     device = km.harness_device(model, rock)
-    bad = 0
+    bad = boundary(model) if a.boundary else 0
     wanted = sorted(lists._BY_LIST) if a.lists == "all" else [n for n in a.lists.split(",") if n]
     for name in wanted:
         gen = torch.Generator(device="cpu")
