@@ -252,7 +252,8 @@ struct RockSoftmaxParams {
   // which may hold any element-wise tree over the scores and further [g, i, j] tensors): postfix code for a
   // four-deep stack machine, run per score in f32.  prog_len = 0: the fixed chain above.
   int32_t prog_len;
-  int32_t pad_;
+  // P[i, seq_k .. seq_k_padded) is written as zeros (0: nothing): the second GEMM then reads rows of whole 16-byte chunks
+  int32_t seq_k_padded;
   int32_t prog[ROCK_ATTN_PROGRAM_MAX]; // RockAttnOp | argument << 8
   float consts[ROCK_ATTN_PROGRAM_INPUTS];
   int32_t tensor_dtype[ROCK_ATTN_PROGRAM_INPUTS];      // RockDType of each input tensor (f32, f16, bf16, i8)

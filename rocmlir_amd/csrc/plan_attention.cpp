@@ -165,18 +165,22 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
   if (ty == ROCK_I8)
     ty = ROCK_F16;
   const int es = dtype_size(ty);
+  // A row of scores is sk f32 values in a pitch of whole 16-byte chunks; P replaces it in place, its tail up to
+  // the next chunk written as zeros by the softmax kernel, so that the second GEMM reads P on its vector path
+  // whatever sk is.
+  const int64_t skp = (sk + 3) / 4 * 4;
   // chunk = gc groups x rc query rows
   // ("-score_workspace_limit BYTES" moves the bound, e.g. to keep one chunk inside a smaller cache share)
   const RoutePolicy route(o);
-  const int64_t dflt = G * sq * sk * 4 <= kScoreWholeBytes ? kScoreWholeBytes : kScoreChunkBytes;
-  const int64_t limit = std::max<int64_t>(route.score_workspace_limit > 0 ? route.score_workspace_limit : dflt, sk * 4);
+  const int64_t dflt = G * sq * skp * 4 <= kScoreWholeBytes ? kScoreWholeBytes : kScoreChunkBytes;
+  const int64_t limit = std::max<int64_t>(route.score_workspace_limit > 0 ? route.score_workspace_limit : dflt, skp * 4);
   int64_t gc = G, rc = sq;
-  if (G * sq * sk * 4 > limit) {
-    if (sq * sk * 4 <= limit) {
-      gc = limit / (sq * sk * 4);
+  if (G * sq * skp * 4 > limit) {
+    if (sq * skp * 4 <= limit) {
+      gc = limit / (sq * skp * 4);
     } else {
       gc = 1;
-      rc = std::max<int64_t>(1, limit / (sk * 4));
+      rc = std::max<int64_t>(1, limit / (skp * 4));
       rc = rc >= 128 ? rc / 128 * 128 : rc >= 8 ? rc / 8 * 8 : rc; // chunk boundaries on whole tiles / 16-byte columns
     }
   }
@@ -191,7 +195,7 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
           S = d;
   }
   const int per_chunk = S > 1 ? 4 : 3;
-  const int64_t score_bytes = align256(gc * rc * sk * 4), partial_bytes = S > 1 ? align256(S * rc * dv * 4) : 0;
+  const int64_t score_bytes = align256(gc * rc * skp * 4), partial_bytes = S > 1 ? align256(S * rc * dv * 4) : 0;
   const int64_t kid_all = int_or(o, "kernel_id", 0);
   if (chunks * per_chunk > INT32_MAX || gc * rc > INT32_MAX) {
     set_error("attention: score matrix too large for the three-kernel form");
@@ -212,12 +216,13 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
   const int n_in = (int)prog.input_types.size();
   const int i_bias = has_scale_t ? 4 : 3, i_mask = has_mask ? i_bias + 1 : -1, i_other = has_mask ? i_bias + 2 : -1,
             i_out = programmed ? 3 + n_in : i_bias + 1 + (has_mask ? 2 : 0), i_ws = i_out + 1;
-  const int64_t pitch_p = 4 / es; // elements of P per f32 score: P lies in place, rows sk * 4 bytes apart
+  const int64_t pitch_p = 4 / es; // elements of P per f32 score: P lies in place, rows skp * 4 bytes apart
   auto *h = new Handle;
   if (kid == 1) {
     RockSoftmaxParams r;
     std::memset(&r, 0, sizeof r);
-    r.row_pitch = sk;
+    r.row_pitch = skp;
+    r.seq_k_padded = (int)((sk * es + 15) / 16 * 16 / es);
     r.t_gs = sq * sk; r.t_is = sk; r.t_js = 1;
     r.G = (int)gn; r.seq_q = (int)rn; r.seq_k = (int)sk;
     r.scale = scale;
@@ -277,7 +282,7 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
       gp.M = (int)rn; gp.N = (int)sk; gp.K = (int)dqk;
       gp.a_gs = sq * dqk; gp.a_ms = tQ ? 1 : dqk; gp.a_ks = tQ ? sq : 1;
       gp.b_gs = sk * dqk; gp.b_ns = tK ? dqk : 1; gp.b_ks = tK ? 1 : sk;
-      gp.c_gs = rn * sk; gp.c_ms = sk; gp.c_ns = 1;
+      gp.c_gs = rn * skp; gp.c_ms = skp; gp.c_ns = 1;
       a_off = (g0 * gp.a_gs + r0 * gp.a_ms) * dtype_size(tq);
       b_off = g0 * gp.b_gs * dtype_size(tq);
       c_off = 0;
@@ -285,7 +290,7 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
       gp.epi.zero_point = (int32_t)int_or(o, "zero_point", 0); // i8: scores leave as float(acc) - zero_point
     } else { // O[g,i,e] = sum_j P[g,i,j] V[g,j,e]
       gp.M = (int)rn; gp.N = (int)dv; gp.K = (int)sk;
-      gp.a_gs = rn * sk * pitch_p; gp.a_ms = sk * pitch_p; gp.a_ks = 1;
+      gp.a_gs = rn * skp * pitch_p; gp.a_ms = skp * pitch_p; gp.a_ks = 1;
       gp.b_gs = sk * dv; gp.b_ns = tV ? sk : 1; gp.b_ks = tV ? 1 : dv;
       gp.c_gs = sq * dv; gp.c_ms = tO ? 1 : dv; gp.c_ns = tO ? sq : 1;
       default_epilogue(gp.epi, ty);
@@ -302,7 +307,7 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
       }
     }
     const int tg = kid == 0 ? tq : ty;
-    plan_gemm_kernel(h, gp, operand_code(tg, tg), dtype_size(tg), o);
+    plan_gemm_kernel(h, gp, operand_code(tg, tg), dtype_size(tg), o, /*k_padded=*/kid == 2);
     if (kid == 0)
       h->ptr_map = {{0, a_off}, {1, b_off}, {i_ws, c_off}, {-1, 0}, {-1, 0}};
     else
@@ -319,7 +324,7 @@ Handle *make_attention_unfused(const OptMap &o, int ty, int64_t G, int64_t sq, i
     h->problem_key = key.str();
   }
   h->kernel_count = (int)(per_chunk * chunks);
-  h->workspace_bytes = (size_t)(partial_bytes ? score_bytes + partial_bytes : gc * rc * sk * 4);
+  h->workspace_bytes = (size_t)(partial_bytes ? score_bytes + partial_bytes : gc * rc * skp * 4);
   h->caller_pointers = i_ws + 1;
   return h;
 }

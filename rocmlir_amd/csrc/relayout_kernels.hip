@@ -319,11 +319,19 @@ extern "C" __global__ __launch_bounds__(1024) void rock_softmax_rows(float *S, c
   const int g = (int)(r / p.seq_q), i = (int)(r - (int64_t)g * p.seq_q);
   const SoftmaxRow row{S + r * p.row_pitch, scale_t, bias, mask, other, (int64_t)g * p.t_gs + (int64_t)i * p.t_is, p};
   // (a program runs on the three-pass path below: its loads and branches do not fit the register-resident form)
+  const int nt = (int)blockDim.x, tid = (int)threadIdx.x;
+  // (every path has read all scores of the row before its last stores, so the bytes behind P's last element,
+  // which may be a score's, are free by now)
+  auto zero_padding = [&]() {
+    for (int j = p.seq_k + tid; j < p.seq_k_padded; j += nt)
+      row.store(j, 0.0f);
+  };
   if (p.prog_len == 0 && (p.dtype == ROCK_F32   ? softmax_short_row<float>(row, scratch)
                           : p.dtype == ROCK_F16 ? softmax_short_row<_Float16>(row, scratch)
-                                                : softmax_short_row<__bf16>(row, scratch)))
+                                                : softmax_short_row<__bf16>(row, scratch))) {
+    zero_padding();
     return;
-  const int nt = (int)blockDim.x, tid = (int)threadIdx.x;
+  }
   float m = -INFINITY;
   for (int j = tid; j < p.seq_k; j += nt)
     m = fmaxf(m, row.score(j));
@@ -342,6 +350,7 @@ extern "C" __global__ __launch_bounds__(1024) void rock_softmax_rows(float *S, c
     if (j < p.seq_k)
       row.store(j, e);
   }
+  zero_padding();
 }
 #endif
 #if RK_SELECTED(6)

@@ -4,7 +4,9 @@
 
 The binding's launch is replaced by one that runs the kernel on the model in this process, on the tensors' own
 memory (torch tensors on the CPU: the `gpu` fixture hands out the CPU device); a launch that has not finished
-after ROCK_HOST_LAUNCH_SECONDS (150) is skipped, and so is everything that measures time.  The model is built for
+after ROCK_HOST_LAUNCH_SECONDS (150) is skipped, and so is everything that measures time.  ROCK_HOST_LATE_LOADS=1
+makes loads into LDS land at the wait that covers them, ROCK_HOST_THREAD_ORDER=1|2 changes the order in which a
+block's threads take their turns (descending, waves rotated).  The model is built for
 every operand type with the rolled-epilogue kernels into ROCK_HOST_BUILD_DIR (ten minutes the first time, kept
 while the sources are unchanged).  Not for the full-size configurations, and not for the entry point that takes
 its workspace from the library's device image."""
@@ -33,6 +35,8 @@ def _the_model():
             os.makedirs(d, exist_ok=True)
             km.build_model(d, types=km.ALL_TYPES, rolled=True)
         _model = km.load_model(so)
+        _model.hm_set_late_loads(int(os.environ.get("ROCK_HOST_LATE_LOADS", "0")))
+        _model.hm_set_thread_order(int(os.environ.get("ROCK_HOST_THREAD_ORDER", "0")))
     return _model
 
 
@@ -65,13 +69,16 @@ def _launch(self, *args, stream=None):
         raise api.RockError("%d accesses outside the tensors in %s" % (bad, self.kernel_name))
 
 
-def _no_timing(self, *args, **kwargs):
+def _no_timing(*args, **kwargs):
     pytest.skip("timing is not the model's business")
 
 
 api.RockKernel.launch = _launch
 api.RockKernel._pointer_array = _pointer_array
 api.RockKernel.benchmark = _no_timing
+api.mfma_rate = _no_timing
+import rocmlir_amd  # noqa: E402
+rocmlir_amd.mfma_rate = _no_timing
 torch.cuda.synchronize = lambda *args, **kwargs: None
 
 
