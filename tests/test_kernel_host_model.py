@@ -7,8 +7,9 @@ threads -- a barrier, a matrix instruction, a cross-lane or transposing read -- 
 gathers and the operation is computed from every lane's operands.  LDS then holds what the GPU's LDS holds, every
 address is the one the GPU thread forms, and on integer-valued data the results must equal the oracle's bit for
 bit.  Buffer loads are range-checked like the hardware's, every tensor lies between canary pages and inaccessible
-regions, and a 16-byte access that is not 16-byte aligned traps.  What it is not: timing, the memory model
-(loads into LDS land when issued), or the accumulation order inside a matrix instruction (exact data only).
+regions, and a 16-byte access that is not 16-byte aligned traps.  A load into LDS lands when it is issued or at
+the wait that covers it, and the tests run under both.  What it is not: timing, caches, or the accumulation
+order inside a matrix instruction (exact data only).
 
 The plans come from the C ABI exactly as a caller gets them: kernel name, grid, block, parameter block and
 pointer map per kernel id, tensor sizes from rockamdGetArgumentInfo.
