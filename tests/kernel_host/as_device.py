@@ -43,6 +43,7 @@ def _the_model():
 def _pointer_array(self, args):
     if len(args) != self.caller_pointers:
         raise api.RockError("kernel %s takes %d pointer arguments, got %d" % (self.kernel_name, self.caller_pointers, len(args)))
+    self._check_sizes(args)
     return [None if a is None else a if isinstance(a, int) else a.data_ptr() for a in args]
 
 

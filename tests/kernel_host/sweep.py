@@ -115,7 +115,7 @@ def source_stamp():
     for d in (km.CSRC, km.HOST):
         for root, _, files in sorted(os.walk(d)):
             for f in sorted(files):
-                if f.endswith((".h", ".hip", ".cpp", ".py")):
+                if f.endswith((".h", ".hip", ".cpp")) or f == "model.py":
                     h.update(open(os.path.join(root, f), "rb").read())
     return h.hexdigest()[:16]
 

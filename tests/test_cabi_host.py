@@ -1063,3 +1063,25 @@ def test_every_problem_of_the_reference_e2e_lists_resolves(rock):
     assert len(lists) == 19 and kernels > 2278
     assert len(refused) == 12 and all(name == "conv_regression_bwd.toml" and "symmetric padding" in msg and
                                       "-padding_h_l=2 -padding_h_r=1" in opts for name, opts, msg in refused)
+
+
+def test_binding_refuses_a_tensor_shorter_than_the_plan_addresses(rock):
+    """The binding compares every tensor argument with the bytes rockamdGetArgumentInfo reports for it before
+    anything is launched: a short tensor is an error on the host, not a fault on the device."""
+    import torch
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 2 -m 100 -n 60 -k 72")
+    a, b, c = (torch.empty(n, dtype=torch.float16) for n in (2 * 100 * 72, 2 * 72 * 60, 2 * 100 * 60))
+    k._check_sizes((a, b, c, None))
+    with pytest.raises(rock.RockError, match="argument 1 .* holds 17278 bytes, the kernel list addresses 17280"):
+        k._check_sizes((a, b[:-1], c, None))
+    conv = rock.RockKernel("-operation conv_bwd_data -arch gfx950 -t f32 -groupsize 1 -batchsize 4 -in_channels 8 "
+                           "-out_channels 16 -in_h 9 -in_w 9 -fil_h 3 -fil_w 3 -padding_h 1 -padding_w 1 "
+                           "-fil_layout kcyx -in_layout nchw -out_layout nkhw")
+    sizes = [16 * 8 * 9, 4 * 8 * 81, 4 * 16 * 81]
+    tensors = [torch.empty(n, dtype=torch.float32) for n in sizes] + [None]
+    if conv.caller_pointers == 5:
+        tensors.append(torch.empty(max(conv.workspace_bytes, 16), dtype=torch.uint8))
+    conv._check_sizes(tuple(tensors))
+    tensors[1] = torch.empty(sizes[1] - 1, dtype=torch.float32)
+    with pytest.raises(rock.RockError, match="argument 1"):
+        conv._check_sizes(tuple(tensors))
