@@ -181,6 +181,15 @@ ROCMLIR_AMD_API MiirStatus rockamdGetKernelArgs(MiirHandle handle, int *num_poin
 ROCMLIR_AMD_API MiirStatus rockamdGetArgumentInfo(MiirHandle handle, int index, int *dtype, int *rank,
                                                   int64_t *dims);
 
+/* The same as one question: bytes[i] is what the caller holds behind pointer i
+ * of the list it is about to pass to rockamdLaunch (0 for a pointer it passes
+ * as NULL).  MIIR_SUCCESS when every non-empty one is at least as large as the
+ * kernel list addresses; otherwise MIIR_INVALID_PARAM with the argument and
+ * the two sizes in rockamdGetLastError().  The kernels take bare pointers and
+ * cannot check this themselves.  No counterpart in the reference, whose
+ * clients pass memrefs that carry their sizes. */
+ROCMLIR_AMD_API MiirStatus rockamdCheckArgumentSizes(MiirHandle handle, const size_t *bytes, int num_pointers);
+
 /* perf-config string of the selected kernel in the reference's grammar
  * ("v2:MPB,NPB,KpackPB,MPW,MnPerXdl,Kpack,splitK,forceUnroll,1" or
  * "attn:v1:...", RockAttrDefs.td:241-329).  Copies what fits, always

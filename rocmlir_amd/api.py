@@ -107,6 +107,8 @@ def load_library():
                                            C.POINTER(C.c_int),
                                            C.POINTER(C.c_int32),
                                            C.POINTER(C.c_int64)]
+        L.rockamdCheckArgumentSizes.restype = C.c_int
+        L.rockamdCheckArgumentSizes.argtypes = [vp, C.POINTER(sz), C.c_int]
         L.rockamdGetParamPointers.restype = C.c_int
         L.rockamdGetParamPointers.argtypes = [vp, C.POINTER(C.c_int), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
         L.rockamdIsFusible.restype = C.c_int
@@ -183,7 +185,6 @@ class RockKernel:
         ncall = C.c_int(0)
         L.rockamdGetPointerMap(self._h, C.byref(ncall), None, None, None)
         self.caller_pointers = ncall.value
-        self._argument_bytes = None
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
@@ -281,27 +282,14 @@ class RockKernel:
         load_library().rockamdSetZeroPoint(self._h, int(zp))
 
     # ---- launch --------------------------------------------------------------
-    _ELEMENT_BYTES = {0: 4, 1: 2, 2: 2, 3: 1, 4: 1, 5: 1, 6: 4}
-
     def _check_sizes(self, args):
         """Every tensor argument must hold at least the bytes the kernel list addresses in it
-        (rockamdGetArgumentInfo): a short one is an error here, not a fault on the device."""
-        need = getattr(self, "_argument_bytes", None)
-        if need is None:
-            need = []
-            for dt, dims in self.arguments():
-                count = 1
-                for d in dims:
-                    count *= int(d)
-                need.append(count * (1 if dt < 0 else self._ELEMENT_BYTES[dt]))
-            self._argument_bytes = need
+        (rockamdCheckArgumentSizes): a short one is an error here, not a fault on the device."""
+        sizes = (C.c_size_t * len(args))()
         for i, a in enumerate(args):
-            if a is None or isinstance(a, int):
-                continue
-            have = a.numel() * a.element_size()
-            if have < need[i]:
-                raise RockError("argument %d of %s holds %d bytes, the kernel list addresses %d"
-                                % (i, self.kernel_name, have, need[i]))
+            sizes[i] = 0 if a is None or isinstance(a, int) else a.numel() * a.element_size()
+        if load_library().rockamdCheckArgumentSizes(self._h, sizes, len(args)) != MIIR_SUCCESS:
+            raise RockError("%s: %s" % (self.kernel_name, last_error()))
 
     def _pointer_array(self, args):
         if len(args) != self.caller_pointers:

@@ -142,6 +142,26 @@ MiirStatus rockamdGetArgumentInfo(MiirHandle handle, int index, int *dtype, int 
   return MIIR_SUCCESS;
 }
 
+MiirStatus rockamdCheckArgumentSizes(MiirHandle handle, const size_t *bytes, int num_pointers) {
+  auto *h = static_cast<Handle *>(handle);
+  if (!h || !bytes || num_pointers != (int)h->args.size()) {
+    set_error("argument sizes: one size per pointer of the caller's list");
+    return MIIR_INVALID_PARAM;
+  }
+  for (int i = 0; i < num_pointers; ++i) {
+    const auto &a = h->args[i];
+    uint64_t need = a.dtype < 0 ? 1 : (uint64_t)dtype_size(a.dtype);
+    for (int64_t d : a.dims)
+      need *= (uint64_t)d;
+    if (bytes[i] != 0 && bytes[i] < need) {
+      set_error("argument " + std::to_string(i) + " holds " + std::to_string(bytes[i]) + " bytes, the kernel list addresses " +
+                std::to_string(need));
+      return MIIR_INVALID_PARAM;
+    }
+  }
+  return MIIR_SUCCESS;
+}
+
 // Copies as much of s as fits and ALWAYS terminates it; returns the full
 // length, so a result >= buffer_size tells the caller the text was cut.  (The
 // reference's strncpy, mlir/lib/CAPI/Dialect/Rock.cpp:86,142, leaves a short

@@ -112,10 +112,10 @@ KINDS = {"conv": conv_problem, "gemm": gemm_problem, "attention": attention_prob
 
 def source_stamp():
     h = hashlib.sha1()
-    for d in (km.CSRC, km.HOST):
+    for d in (km.CSRC, km.HOST):   # the kernels' sources (not the host library's), the stand-in, the runner
         for root, _, files in sorted(os.walk(d)):
             for f in sorted(files):
-                if f.endswith((".h", ".hip", ".cpp")) or f == "model.py":
+                if f.endswith((".h", ".hip")) or (d == km.HOST and (f.endswith(".cpp") or f == "model.py")):
                     h.update(open(os.path.join(root, f), "rb").read())
     return h.hexdigest()[:16]
 

@@ -1066,14 +1066,17 @@ def test_every_problem_of_the_reference_e2e_lists_resolves(rock):
 
 
 def test_binding_refuses_a_tensor_shorter_than_the_plan_addresses(rock):
-    """The binding compares every tensor argument with the bytes rockamdGetArgumentInfo reports for it before
-    anything is launched: a short tensor is an error on the host, not a fault on the device."""
+    """rockamdCheckArgumentSizes, which the binding asks before anything is launched: a tensor shorter than the
+    kernel list addresses is an error on the host, not a fault on the device."""
     import torch
     k = rock.RockKernel("-operation gemm -arch gfx950 -t f16 -g 2 -m 100 -n 60 -k 72")
     a, b, c = (torch.empty(n, dtype=torch.float16) for n in (2 * 100 * 72, 2 * 72 * 60, 2 * 100 * 60))
-    k._check_sizes((a, b, c, None))
-    with pytest.raises(rock.RockError, match="argument 1 .* holds 17278 bytes, the kernel list addresses 17280"):
-        k._check_sizes((a, b[:-1], c, None))
+    rest = (None,) if k.caller_pointers == 4 else (None, torch.empty(max(k.workspace_bytes, 16), dtype=torch.uint8))
+    k._check_sizes((a, b, c) + rest)
+    with pytest.raises(rock.RockError, match="argument 1 holds 17278 bytes, the kernel list addresses 17280"):
+        k._check_sizes((a, b[:-1], c) + rest)
+    with pytest.raises(rock.RockError, match="one size per pointer"):
+        k._check_sizes((a, b))
     conv = rock.RockKernel("-operation conv_bwd_data -arch gfx950 -t f32 -groupsize 1 -batchsize 4 -in_channels 8 "
                            "-out_channels 16 -in_h 9 -in_w 9 -fil_h 3 -fil_w 3 -padding_h 1 -padding_w 1 "
                            "-fil_layout kcyx -in_layout nchw -out_layout nkhw")
