@@ -145,6 +145,7 @@ def load_model(so):
     lib.hm_set_late_loads.argtypes = [C.c_int]
     lib.hm_set_thread_order.argtypes = [C.c_int]
     lib.hm_set_blocks.argtypes = [C.c_uint, C.c_uint]
+    lib.hm_set_owner_check.argtypes = [C.c_int]
     lib.hm_run_direct.restype = C.c_long
     lib.hm_run_direct.argtypes = [C.c_char_p, C.c_char_p, C.POINTER(C.c_void_p), C.c_uint, C.c_uint, C.c_int]
     return lib

@@ -63,6 +63,41 @@ void on_trap(int sig, siginfo_t *si, void *) {
   _exit(0);
 }
 
+// ---- who wrote what: no byte of a tensor may be changed by two blocks of one launch ------------
+bool check_owners = false;
+struct Shadow {
+  std::vector<char> before;          // the tensor as the last block left it
+  std::vector<unsigned char> owned;  // 1: some block of this launch has changed the byte
+};
+std::vector<Shadow> shadows;
+void owners_begin() {
+  shadows.assign(ranges.size(), Shadow());
+  for (size_t i = 0; i < ranges.size(); ++i) {
+    shadows[i].before.assign(ranges[i].lo, ranges[i].hi);
+    shadows[i].owned.assign(ranges[i].hi - ranges[i].lo, 0);
+  }
+}
+void owners_after_block() {
+  for (size_t i = 0; i < ranges.size(); ++i) {
+    Shadow &sh = shadows[i];
+    const char *now = ranges[i].lo;
+    const size_t n = sh.before.size();
+    if (!std::memcmp(now, sh.before.data(), n))
+      continue;
+    for (size_t b = 0; b < n; ++b)
+      if (now[b] != sh.before[b]) {
+        if (sh.owned[b]) {
+          char text[300];
+          snprintf(text, sizeof text, "%s, block %u changed byte %zu of %s, which an earlier block of the launch had written",
+                   cur_kernel, blockIdx.x, b, ranges[i].name.c_str());
+          note(text);
+        }
+        sh.owned[b] = 1;
+        sh.before[b] = now[b];
+      }
+  }
+}
+
 // ---- one block as cooperative fibers ---------------------------------------------
 enum State { kRun, kWaitWave, kWaitBlock, kDone };
 struct PendingLoad { // a load into LDS that has been issued and has not landed
@@ -368,6 +403,9 @@ extern "C" {
 void hm_set_late_loads(int on) { late_loads = on != 0; }
 // the order in which a block's threads take their turns: 0 ascending, 1 descending, 2 waves rotated per pass
 void hm_set_thread_order(int order) { thread_order = order; }
+// 1: after every block the tensors are compared with what they were before it, and a byte that two blocks of one
+// launch change is reported (every output element belongs to one block; costs a pass over the tensors per block)
+void hm_set_owner_check(int on) { check_owners = on != 0; }
 // only blocks [first, first + count) of every launch run (a problem too large to run whole: its last tiles)
 void hm_set_blocks(unsigned first, unsigned count) {
   first_block = first;
@@ -478,10 +516,14 @@ long hm_run(const char *name, const void *params, void **pointers, unsigned grid
     kernel_pointers = pointers;
     kernel_params = params;
     threads = block;
+    if (check_owners)
+      owners_begin();
     for (unsigned b = first_block; b < grid && b - first_block < block_limit; ++b) {
       blockIdx = {b, 0, 0};
       if (!run_block())
         break;
+      if (check_owners)
+        owners_after_block();
     }
     _exit(0);
   }

@@ -7,6 +7,7 @@ oracle (tests/test_gpu_e2e_lists.py with the model as its device).  Run from the
   ... --types all --rolled    every operand type and the rolled-epilogue kernels (ten minutes of compilation,
                               kept in --build-dir and used again while the sources are unchanged)
   ... --late --order 2        loads land at the wait that covers them, waves take their turns rotated
+  ... --owners                every launch is checked for bytes that two of its blocks change
   python -m tests.kernel_host.sweep --boundary                  # tensors just below and at 2 GiB, their last tiles only
 
 One line per problem: ok / FAIL / refused, the kernels that ran, the options string to run it again."""
@@ -239,6 +240,7 @@ def main():
     ap.add_argument("--rolled", action="store_true", help="build the rolled-epilogue kernels too")
     ap.add_argument("--late", action="store_true", help="loads into LDS land at the wait that covers them")
     ap.add_argument("--order", type=int, default=0, help="0 ascending, 1 descending, 2 waves rotated per pass")
+    ap.add_argument("--owners", action="store_true", help="report a byte that two blocks of one launch change")
     ap.add_argument("--boundary", action="store_true", help="tensors just below and at 2 GiB (needs about 10 GB of memory)")
     ap.add_argument("--build-dir", default=os.path.join(os.environ.get("TMPDIR", "/tmp"), "rock_kernel_host"))
     a = ap.parse_args()
@@ -254,6 +256,7 @@ def main():
         model = km.build_model(d, types=types, rolled=a.rolled)
     model.hm_set_late_loads(1 if a.late else 0)
     model.hm_set_thread_order(a.order)
+    model.hm_set_owner_check(1 if a.owners else 0)
     have = set()
     for t in types:
         have |= set(km._build.GEMM_TYPES[t].split("_"))

@@ -28,8 +28,11 @@ pytestmark = pytest.mark.skipif(CLANG is None, reason="the host build uses clang
 
 @pytest.fixture(scope="module")
 def model(tmp_path_factory):
-    """The f32 and f16 kernel families and the attention kernels (about a minute of compilation)."""
-    return build_model(str(tmp_path_factory.mktemp("kernel_host")))
+    """The f32 and f16 kernel families and the attention kernels (about a minute of compilation).  Every launch
+    is also checked for bytes that two of its blocks change."""
+    lib = build_model(str(tmp_path_factory.mktemp("kernel_host")))
+    lib.hm_set_owner_check(1)
+    return lib
 
 
 @pytest.fixture(params=["loads-land-at-issue", "loads-land-at-the-wait"])
@@ -114,6 +117,33 @@ def test_the_model_notices_a_short_operand(model, rock):
     assert names and not problems, (names, problems)
     names, problems, _ = run_plan(model, rock, opts, shrink=(0, 16))
     assert problems and "buffer load into LDS outside the tensors" in problems[0], problems
+
+
+def test_the_model_notices_two_blocks_writing_one_byte(model, rock):
+    """A GEMM whose result rows are given half their pitch in the parameter block: the right half of every row
+    then lies on the left half of the next, which another block writes."""
+    import ctypes as C
+    import struct
+    from tests.kernel_host.model import pointer_map
+    k = rock.RockKernel("-operation gemm -arch gfx950 -t f32 -g 1 -m 128 -n 128 -k 64 -transA false -transB true")
+    assert k.kernel_name == "rock_gemm_f32_64x64_fast" and k.grid_size == 4
+    model.hm_clear()
+    rng = np.random.default_rng(0)
+    tensors = []
+    for i, nbytes in enumerate((128 * 64 * 4, 128 * 64 * 4, 128 * 128 * 4, 16)):
+        at = model.hm_alloc(nbytes, b"argument %d" % i)
+        np.ctypeslib.as_array((C.c_uint8 * nbytes).from_address(at))[:] = rng.integers(0, 256, nbytes, dtype=np.uint8) & 0x3F
+        tensors.append(at)
+    ptrs = (C.c_void_p * 8)()
+    for j, (src, off) in enumerate(pointer_map(rock, k)):
+        ptrs[j] = None if src < 0 else tensors[src] + off
+    text = C.create_string_buffer(512)
+    params = bytearray(k.params())
+    assert model.hm_run(k.kernel_name.encode(), bytes(params), ptrs, 4, k.block_size, text, 512) == 0, text.value
+    assert struct.unpack_from("<q", params, 56)[0] == 128   # the stride between rows of C
+    struct.pack_into("<q", params, 56, 64)
+    assert model.hm_run(k.kernel_name.encode(), bytes(params), ptrs, 4, k.block_size, text, 512) > 0
+    assert b"which an earlier block of the launch had written" in text.value, text.value
 
 
 @pytest.mark.parametrize("t", ["f16", "f32"])
