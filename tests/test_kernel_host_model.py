@@ -28,9 +28,9 @@ pytestmark = pytest.mark.skipif(CLANG is None, reason="the host build uses clang
 
 @pytest.fixture(scope="module")
 def model(tmp_path_factory):
-    """The f32 and f16 kernel families and the attention kernels (about a minute of compilation).  Every launch
+    """The f32, f16 and int8 kernel families and the attention kernels (a minute or two of compilation).  Every launch
     is also checked for bytes that two of its blocks change."""
-    lib = build_model(str(tmp_path_factory.mktemp("kernel_host")))
+    lib = build_model(str(tmp_path_factory.mktemp("kernel_host")), types=(0, 1, 3))
     lib.hm_set_owner_check(1)
     return lib
 
@@ -165,6 +165,28 @@ def test_gemm_through_the_model_equals_numpy(model, rock, loads, t, shape):
     got = out[2][:m * n * np.dtype(dt).itemsize].view(dt).reshape(m, n).astype(np.float64)
     want = (A.T if ta else A).astype(np.float64) @ (B.T if tb else B).astype(np.float64)
     assert np.array_equal(got, want), names
+
+
+@pytest.mark.parametrize("tile", ["v2:256,256,8,128,16,16,1,1,1", ""], ids=["256x256", "table"])
+def test_quantised_int8_gemm_through_the_model_equals_the_oracle(model, rock, oracle, loads, tile):
+    """The headline configuration in small: int8 operands, int32 accumulators, f16(float(acc) * 0.01), on the
+    256 x 256 tile it runs on at full size and on the tile the table picks for this size; every step is a single
+    IEEE operation, so the result must equal the oracle's bit for bit."""
+    from tests.gpu_util import CODE
+    M, N, K = 512, 384, 256
+    rng = np.random.default_rng(7)
+    A = rng.integers(-128, 128, (M, K)).astype(np.int8)
+    B = rng.integers(-128, 128, (N, K)).astype(np.int8)
+    opts = ("-operation gemm -arch gfx950 -t i8 -out_datatype f16 -g 1 -m %d -n %d -k %d -transA false -transB true "
+            "-scale 0.01" % (M, N, K)) + (" -perf_config " + tile if tile else "")
+    names, problems, out = run_plan(model, rock, opts, {0: A, 1: B})
+    assert not problems, (names, problems)
+    if tile:
+        assert names == ["rock_gemm_i8_256x256_fast"], names
+    acc = A.astype(np.int64) @ B.astype(np.int64).T
+    want = oracle.round_through(oracle.dequantize(acc, 0.01, 0), CODE["f16"]).reshape(M, N)
+    got = out[2][:M * N * 2].view(np.float16).reshape(M, N).astype(np.float32)
+    assert np.array_equal(got, want.astype(np.float32)), names
 
 
 # (operation, type, batch, c, k, image, filter, padding, layouts, stride, last kernel): the kinds of plan the
