@@ -653,7 +653,7 @@ def conv2d(fil, inp, *, fil_layout, in_layout, out_layout, batchsize,
 
 def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, mask=None, other=None, zero_point=0,
               transQ=False, transK=False, transV=False, transO=False, out=None, stream=None, info=None,
-              score_workspace_limit=None, program=None, inputs=()):
+              score_workspace_limit=None, program=None, inputs=(), layout_conversion=True):
     """O = softmax(scale * scale_tensor * Q K + bias) V (bias and scale_tensor
     optional [G,seq_q,seq_k] tensors, rocmlir-gen's -with-attn-bias /
     -with-attn-scale).  `mask` (int8 or bool, [G,seq_q,seq_k]) with `other`
@@ -699,6 +699,8 @@ def attention(q, k, v, *, scale=1.0, bias=None, scale_tensor=None, mask=None, ot
         if tuple(mask.shape) != (G, sq, sk) or tuple(other.shape) != (G, sq, sk) or other.dtype != v.dtype:
             raise RockError("attention: mask and other are [G, seq_q, seq_k]; other has v's type")
         mask = mask.to(torch.int8).contiguous()
+    if not layout_conversion:   # no copies in front of or behind the kernel: tensors are read as they lie
+        opts += " -layout_conversion false"
     if score_workspace_limit is not None:
         opts += " -score_workspace_limit %d" % score_workspace_limit
     if program:

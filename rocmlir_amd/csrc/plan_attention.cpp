@@ -370,12 +370,23 @@ Handle *make_attention(const OptMap &o) {
   // them as they lie (element-wise gathers, or the GEMMs of the three-kernel form).
   // K stored [G, d, seq_k] is read as it lies by the "_kt" kernels when its rows of keys are whole 16-byte
   // chunks; otherwise (seq_k = 27; int8 keys) it is copied to [G, seq_k, d] the same way.
-  const bool copy_k = !tK && (qk_i8 || sk % 8 != 0);
-  if ((tQ || tV || tO || copy_k) && ty != ROCK_F32 && RoutePolicy(o).layout_conversion) {
+  // Head dimensions that are not whole 16-byte chunks (d = 20, 36): the same copies pad every row of Q and K to
+  // dqp and of V to dvp elements with zeros, which add nothing to a score; the fused kernel works on the padded
+  // problem and the last conversion keeps the dv columns of its result that exist.
+  const int64_t unit_qk = qk_i8 ? 16 : 8;
+  const int64_t dqp = (dqk + unit_qk - 1) / unit_qk * unit_qk, dvp = (dv + 7) / 8 * 8;
+  const bool pad_qk = dqp != dqk, pad_v = dvp != dv;
+  const bool copy_k = (!tK && (qk_i8 || sk % 8 != 0)) || pad_qk;
+  const bool copy_q = tQ || pad_qk, copy_v = tV || pad_v, copy_o = tO || pad_v;
+  if ((copy_q || copy_v || copy_o || copy_k) && ty != ROCK_F32 && RoutePolicy(o).layout_conversion) {
     OptMap inner = o;
     inner["transQ"] = inner["transV"] = inner["transO"] = "false";
     if (copy_k)
       inner["transK"] = "true";
+    if (pad_qk)
+      inner["head_dim_qk"] = std::to_string(dqp);
+    if (pad_v)
+      inner["head_dim_v"] = std::to_string(dvp);
     inner.erase("kernel_id");
     const std::string keep_error = g_last_error;
     Handle *core = make_attention(inner);
@@ -386,18 +397,18 @@ Handle *make_attention(const OptMap &o) {
       g_last_error = keep_error;
     } else {
       const int es_q = qk_i8 ? 1 : 2;
-      const int64_t q_bytes = tQ ? align256(G * sq * dqk * es_q) : 0, v_bytes = tV ? align256(G * sk * dv * 2) : 0,
-                    o_bytes = tO ? align256(G * sq * dv * 2) : 0, k_bytes = copy_k ? align256(G * sk * dqk * es_q) : 0;
+      const int64_t q_bytes = copy_q ? align256(G * sq * dqp * es_q) : 0, v_bytes = copy_v ? align256(G * sk * dvp * 2) : 0,
+                    o_bytes = copy_o ? align256(G * sq * dvp * 2) : 0, k_bytes = copy_k ? align256(G * sk * dqp * es_q) : 0;
       const int64_t q_off = 0, v_off = q_bytes, o_off = q_bytes + v_bytes, k_off = o_off + o_bytes;
       // caller pointers: Q, K, V, [scale tensor,] bias, [mask, other,] O, workspace
       const int i_scale = has_scale_t ? 3 : -1, i_bias = has_scale_t ? 4 : 3, i_mask = has_mask ? i_bias + 1 : -1,
                 i_other = has_mask ? i_bias + 2 : -1, i_out = i_bias + 1 + (has_mask ? 2 : 0), i_ws = i_out + 1;
       std::vector<int> kinds; // 0 = Q copy, 1 = V copy, 4 = K copy, 2 = the fused kernel, 3 = O written in the caller's layout
-      if (tQ) kinds.push_back(0);
-      if (tV) kinds.push_back(1);
+      if (copy_q) kinds.push_back(0);
+      if (copy_v) kinds.push_back(1);
       if (copy_k) kinds.push_back(4);
       kinds.push_back(2);
-      if (tO) kinds.push_back(3);
+      if (copy_o) kinds.push_back(3);
       const int kid = (int)int_or(o, "kernel_id", 0);
       if (kid < 0 || kid >= (int)kinds.size()) {
         set_error("attention: kernel_id out of range");
@@ -410,23 +421,32 @@ Handle *make_attention(const OptMap &o) {
         h = new Handle;
         h->arch = core->arch;
         bool ok;
-        if (kinds[kid] == 0) { // [G, d, seq_q] -> [G, seq_q, d]
-          const int64_t size[5] = {1, 1, G, sq, dqk}, stride[5] = {0, 0, sq * dqk, 1, sq};
-          ok = fill_relayout_handle(h, size, size, stride, es_q);
+        // (source strides in the order of the destination's dimensions; rows padded with zeros up to dqp / dvp)
+        if (kinds[kid] == 0) { // [G, d, seq_q] or [G, seq_q, d] -> [G, seq_q, dqp]
+          const int64_t size[5] = {1, 1, G, sq, dqp}, src_size[5] = {1, 1, G, sq, dqk};
+          const int64_t stride[5] = {0, 0, sq * dqk, tQ ? 1 : dqk, tQ ? sq : 1};
+          ok = fill_relayout_handle(h, size, src_size, stride, es_q);
           h->ptr_map = {{0, 0}, {i_ws, q_off}};
           h->problem_key = "relayout attention Q";
-        } else if (kinds[kid] == 1) { // [G, dv, seq_k] -> [G, seq_k, dv]
-          const int64_t size[5] = {1, 1, G, sk, dv}, stride[5] = {0, 0, sk * dv, 1, sk};
-          ok = fill_relayout_handle(h, size, size, stride, 2);
+        } else if (kinds[kid] == 1) { // [G, dv, seq_k] or [G, seq_k, dv] -> [G, seq_k, dvp]
+          const int64_t size[5] = {1, 1, G, sk, dvp}, src_size[5] = {1, 1, G, sk, dv};
+          const int64_t stride[5] = {0, 0, sk * dv, tV ? 1 : dv, tV ? sk : 1};
+          ok = fill_relayout_handle(h, size, src_size, stride, 2);
           h->ptr_map = {{2, 0}, {i_ws, v_off}};
           h->problem_key = "relayout attention V";
-        } else if (kinds[kid] == 4) { // [G, d, seq_k] -> [G, seq_k, d]
-          const int64_t size[5] = {1, 1, G, sk, dqk}, stride[5] = {0, 0, sk * dqk, 1, sk};
-          ok = fill_relayout_handle(h, size, size, stride, es_q);
+        } else if (kinds[kid] == 4) { // [G, d, seq_k] or [G, seq_k, d] -> [G, seq_k, dqp]
+          const int64_t size[5] = {1, 1, G, sk, dqp}, src_size[5] = {1, 1, G, sk, dqk};
+          const int64_t stride[5] = {0, 0, sk * dqk, tK ? dqk : 1, tK ? 1 : sk};
+          ok = fill_relayout_handle(h, size, src_size, stride, es_q);
           h->ptr_map = {{1, 0}, {i_ws, k_off}};
           h->problem_key = "relayout attention K";
-        } else { // [G, seq_q, dv] -> [G, dv, seq_q]
-          const int64_t size[5] = {1, 1, G, dv, sq}, stride[5] = {0, 0, sq * dv, 1, dv};
+        } else if (tO) { // [G, seq_q, dvp] -> [G, dv, seq_q]
+          const int64_t size[5] = {1, 1, G, dv, sq}, stride[5] = {0, 0, sq * dvp, 1, dvp};
+          ok = fill_relayout_handle(h, size, size, stride, 2);
+          h->ptr_map = {{i_ws, o_off}, {i_out, 0}};
+          h->problem_key = "relayout attention O";
+        } else { // [G, seq_q, dvp] -> [G, seq_q, dv]
+          const int64_t size[5] = {1, 1, G, sq, dv}, stride[5] = {0, 0, sq * dvp, dvp, 1};
           ok = fill_relayout_handle(h, size, size, stride, 2);
           h->ptr_map = {{i_ws, o_off}, {i_out, 0}};
           h->problem_key = "relayout attention O";
@@ -437,11 +457,11 @@ Handle *make_attention(const OptMap &o) {
           return nullptr;
         }
       } else {
-        h->ptr_map = {tQ ? Handle::PtrSrc{i_ws, q_off} : Handle::PtrSrc{0, 0},
+        h->ptr_map = {copy_q ? Handle::PtrSrc{i_ws, q_off} : Handle::PtrSrc{0, 0},
                       copy_k ? Handle::PtrSrc{i_ws, k_off} : Handle::PtrSrc{1, 0},
-                      tV ? Handle::PtrSrc{i_ws, v_off} : Handle::PtrSrc{2, 0}, {i_scale, 0}, {i_bias, 0},
+                      copy_v ? Handle::PtrSrc{i_ws, v_off} : Handle::PtrSrc{2, 0}, {i_scale, 0}, {i_bias, 0},
                       {i_mask, 0}, {i_other, 0},
-                      tO ? Handle::PtrSrc{i_ws, o_off} : Handle::PtrSrc{i_out, 0}};
+                      copy_o ? Handle::PtrSrc{i_ws, o_off} : Handle::PtrSrc{i_out, 0}};
         // the key names the problem as the caller posed it
         auto tf = [](bool b) { return b ? "true" : "false"; };
         std::ostringstream key;

@@ -19,7 +19,7 @@ def _store(mat, trans):
 
 
 def _run(rock, oracle, gpu, t, G, sq, sk, dqk, dv, scale, seed, tQ=False, tK=True, tV=False, tO=False,
-         bias=False, vones=False, scale_tensor=False, info=None, mask=False, limit=None):
+         bias=False, vones=False, scale_tensor=False, info=None, mask=False, limit=None, conversion=True):
     rng = np.random.default_rng(seed)
     Q = rng.standard_normal((G, sq, dqk)).astype(np.float32)
     K = rng.standard_normal((G, sk, dqk)).astype(np.float32)
@@ -45,7 +45,8 @@ def _run(rock, oracle, gpu, t, G, sq, sk, dqk, dv, scale, seed, tQ=False, tK=Tru
                          scale_tensor=to_gpu(sraw, t, gpu) if scale_tensor else None,
                          mask=torch.from_numpy(mk).to(gpu) if mask else None,
                          other=to_gpu(oraw, t, gpu) if mask else None,
-                         transQ=tQ, transK=tK, transV=tV, transO=tO, info=info, score_workspace_limit=limit)
+                         transQ=tQ, transK=tK, transV=tV, transO=tO, info=info, score_workspace_limit=limit,
+                         layout_conversion=conversion)
     torch.cuda.synchronize()
     ref = oracle.attention(Qq, Kq, Vq, G, sq, sk, dqk, dv, scale=scale, bias_t=bq, scale_t=sq_,
                            transQ=tQ, transK=tK, transV=tV, transO=tO, mask=mk, other=oq)
@@ -128,9 +129,16 @@ def test_attention_default_key_layout_unaligned_rows(rock, oracle, gpu):
     check_float(got, ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
 
 
-def test_attention_odd_head_dims_take_generic_kernel(rock, oracle, gpu):
-    got, ref = _run(rock, oracle, gpu, "f16", 2, 50, 70, 20, 12, 0.3, 44)
+@pytest.mark.parametrize("conversion", [True, False], ids=["padded-copies", "as-they-lie"])
+def test_attention_odd_head_dims(rock, oracle, gpu, conversion):
+    """Head dimensions that are not whole 16-byte chunks (20 and 12): Q, K and V are copied into rows padded with
+    zeros, the fused kernel runs on the padded problem and a last copy keeps the columns of O that exist; without
+    conversions the element-wise kernel reads the tensors as they lie."""
+    info = {}
+    got, ref = _run(rock, oracle, gpu, "f16", 2, 50, 70, 20, 12, 0.3, 44, info=info, conversion=conversion)
     check_float(got, ref, "f16", rms=GATE["f16"][0], max_abs=GATE["f16"][1])
+    assert info["kernels"] == (["rock_relayout_b2"] * 3 + ["rock_attention_f16_d64x64_fast", "rock_relayout_b2"]
+                               if conversion else ["rock_attention_f16_d64x64_generic"])
 
 
 def test_attention_with_bias(rock, oracle, gpu):
@@ -141,7 +149,7 @@ def test_attention_with_bias(rock, oracle, gpu):
 
 @pytest.mark.parametrize("bias", [False, True])
 @pytest.mark.parametrize("shape", [(2, 128, 27, 64, 32), (1, 300, 200, 128, 128), (2, 50, 70, 20, 12)],
-                         ids=["cross", "d128", "generic"])
+                         ids=["cross", "d128", "odd-head-dims"])
 def test_attention_with_scale_tensor(rock, oracle, gpu, shape, bias):
     """-with-attn-scale: a [G,seq_q,seq_k] tensor multiplied into the scores
     before the softmax (rocmlir-gen.cpp:2185-2196, 2368-2382), alone and with a bias."""
@@ -157,7 +165,8 @@ def test_attention_with_scale_tensor(rock, oracle, gpu, shape, bias):
     dict(id="d64-scale-tensor-bf16", t="bf16", shape=(3, 128, 27, 64, 32), scale_tensor=True,
          kernels=["rock_attention_bf16_d64x64_fast_bias"]),
     dict(id="default-key-layout", t="f16", shape=(2, 130, 136, 64, 64), tK=False, kernels=["rock_attention_f16_d64x64_fast_bias_kt"]),
-    dict(id="generic", t="f16", shape=(2, 50, 70, 20, 12), kernels=["rock_attention_f16_d64x64_generic"]),
+    dict(id="generic", t="f16", shape=(2, 50, 70, 20, 12), conversion=False, kernels=["rock_attention_f16_d64x64_generic"]),
+    dict(id="odd-head-dims", t="f16", shape=(2, 50, 70, 20, 12), count=5),
     dict(id="transposed-q-o", t="f16", shape=(2, 96, 80, 64, 64), tQ=True, tO=True, count=3),
     dict(id="three-kernels-d320", t="f16", shape=(2, 100, 150, 320, 192), bias=True, count=3),
     dict(id="three-kernels-f32", t="f32", shape=(2, 96, 80, 64, 64), bias=True, scale_tensor=True, count=3),
@@ -171,7 +180,8 @@ def test_attention_where_mask(rock, oracle, gpu, case):
     info = {}
     got, ref = _run(rock, oracle, gpu, t, G, sq, sk, dqk, dv, 0.125, 71, tQ=case.get("tQ", False),
                     tK=case.get("tK", True), tO=case.get("tO", False), bias=case.get("bias", False),
-                    scale_tensor=case.get("scale_tensor", False), mask=True, info=info)
+                    scale_tensor=case.get("scale_tensor", False), mask=True, info=info,
+                    conversion=case.get("conversion", True))
     if "kernels" in case:
         assert info["kernels"] == case["kernels"]
     else:

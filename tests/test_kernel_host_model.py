@@ -254,7 +254,10 @@ def _attention_problem(t, G, sq, sk, dqk, dv, trans_k, scale, extra=""):
     # rows and P's tail is written as zeros, which keeps the second GEMM on its vector path
     ("f32", 2, 70, 45, 64, 64, True, False, True, "rock_gemm_f32_64x64_fast_nn"),
     ("f16", 1, 40, 77, 320, 320, True, False, False, "rock_gemm_f16_64x64_fast_nn"),
-], ids=["d64", "d128-keys-as-stored", "scale-tensor-bias-cross", "d256", "f32-three-kernels", "d320-three-kernels"])
+    # head dimensions 20 and 12: copies padded with zeros around the fused kernel, the last one drops O's padding
+    ("f16", 2, 50, 70, 20, 12, False, False, True, "rock_relayout_b2"),
+], ids=["d64", "d128-keys-as-stored", "scale-tensor-bias-cross", "d256", "f32-three-kernels", "d320-three-kernels",
+        "odd-head-dims"])
 def test_attention_through_the_model_passes_the_gates(model, rock, oracle, loads, case):
     """The fused kernels (and the three-kernel form) on real-valued data through the model, under the gates of the
     GPU tests: RMS 1e-3 and maximum difference 0.02 for f16, 3e-5 and 1e-4 for f32."""
